@@ -1,0 +1,655 @@
+// Elementwise and strided-copy kernels (HBM bound).
+//
+// One loop-nest engine serves every all-parallel linalg.generic of the
+// reference (src/structure/kernel/kernel/{add,sub,mul,div,pow,erf,relu,clip,
+// tanh,sqrt,neg,not,cast,equal,dropout,where,transpose,squeeze,unsqueeze,
+// slice,concat,pad,add_div_erf_add_mul_mul,unsqueeze_sub_mul}.cpp): the host
+// wrapper turns the kernel's affine maps into per-operand strides, the nest is
+// canonicalised in the output's physical order, and the device walks it with
+// 128-bit accesses when the innermost dimension is contiguous for every
+// operand (or broadcast), falling back to scalar accesses otherwise.
+#include "fl_common.h"
+
+namespace fl {
+namespace {
+
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Vec {
+  T v[N];
+};
+
+struct Empty {};
+
+constexpr int kBlock = 256;
+constexpr int kVec = 4;
+
+// NIN inputs, operand 0 of the nest is the output.  `bcast` bit i set = input
+// i is broadcast along the innermost dimension (scalar load, replicated).
+template <int NIN, int VEC, typename TO, typename T0, typename T1, typename T2, typename Op>
+__global__ __launch_bounds__(kBlock) void EwKernel(NestArgs<NIN + 1> a, uint32_t n_items, uint32_t bcast,
+                                                   TO *__restrict__ out, const T0 *__restrict__ in0,
+                                                   const T1 *__restrict__ in1, const T2 *__restrict__ in2, Op op) {
+  const uint32_t stride = gridDim.x * kBlock;
+  for (uint32_t item = blockIdx.x * kBlock + threadIdx.x; item < n_items; item += stride) {
+    uint32_t rem = item;
+    int32_t off[NIN + 1];
+#pragma unroll
+    for (int o = 0; o <= NIN; ++o) off[o] = 0;
+    for (int d = a.rank - 1; d > 0; --d) {
+      uint32_t q, r;
+      a.div[d].DivMod(rem, q, r);
+      rem = q;
+#pragma unroll
+      for (int o = 0; o <= NIN; ++o) off[o] += static_cast<int32_t>(r) * a.strides[o][d];
+    }
+#pragma unroll
+    for (int o = 0; o <= NIN; ++o) off[o] += static_cast<int32_t>(rem) * a.strides[o][0];
+
+    if constexpr (VEC == 1) {
+      T0 x0 = in0[off[1]];
+      T1 x1{};
+      T2 x2{};
+      if constexpr (NIN >= 2) x1 = in1[off[2]];
+      if constexpr (NIN >= 3) x2 = in2[off[3]];
+      out[off[0]] = op(x0, x1, x2);
+    } else {
+      Vec<T0, VEC> v0;
+      Vec<T1, VEC> v1;
+      Vec<T2, VEC> v2;
+      if (bcast & 1u) {
+        const T0 s = in0[off[1]];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v0.v[i] = s;
+      } else {
+        v0 = *reinterpret_cast<const Vec<T0, VEC> *>(in0 + off[1]);
+      }
+      if constexpr (NIN >= 2) {
+        if (bcast & 2u) {
+          const T1 s = in1[off[2]];
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) v1.v[i] = s;
+        } else {
+          v1 = *reinterpret_cast<const Vec<T1, VEC> *>(in1 + off[2]);
+        }
+      }
+      if constexpr (NIN >= 3) {
+        if (bcast & 4u) {
+          const T2 s = in2[off[3]];
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) v2.v[i] = s;
+        } else {
+          v2 = *reinterpret_cast<const Vec<T2, VEC> *>(in2 + off[3]);
+        }
+      }
+      Vec<TO, VEC> r;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        T1 x1{};
+        T2 x2{};
+        if constexpr (NIN >= 2) x1 = v1.v[i];
+        if constexpr (NIN >= 3) x2 = v2.v[i];
+        r.v[i] = op(v0.v[i], x1, x2);
+      }
+      *reinterpret_cast<Vec<TO, VEC> *>(out + off[0]) = r;
+    }
+  }
+}
+
+// Decide vector width, build device args, launch.
+template <int NIN, typename TO, typename T0, typename T1, typename T2, typename Op>
+int LaunchNest(LoopNest nest, void *out, const void *in0, const void *in1, const void *in2, Op op, hipStream_t stream) {
+  nest.Canonicalise();
+  int64_t total = 1;
+  for (int i = 0; i < nest.rank; ++i) total *= nest.shape[i];
+  if (total > INT32_MAX) return FL_ERR_TOO_LARGE;
+
+  const void *ptrs[4] = {out, in0, in1, in2};
+  const size_t sizes[4] = {sizeof(TO), sizeof(T0), sizeof(T1), sizeof(T2)};
+  const int inner = nest.rank - 1;
+  bool vec_ok = nest.shape[inner] % kVec == 0 && nest.strides[0][inner] == 1;
+  uint32_t bcast = 0;
+  for (int o = 0; o <= NIN && vec_ok; ++o) {
+    const int64_t s = nest.strides[o][inner];
+    if (s == 0 && o > 0) {
+      bcast |= 1u << (o - 1);
+    } else if (s != 1) {
+      vec_ok = false;
+      break;
+    }
+    if (!IsAligned(ptrs[o], sizes[o] * kVec) && s == 1) vec_ok = false;
+    for (int d = 0; d < inner && vec_ok; ++d) {
+      if (s == 1 && nest.strides[o][d] % kVec != 0) vec_ok = false;
+    }
+  }
+  if (!vec_ok) bcast = 0;
+
+  if (vec_ok) {
+    nest.shape[inner] /= kVec;
+    for (int o = 0; o <= NIN; ++o) nest.strides[o][inner] *= kVec;
+  }
+  const int64_t n_items = vec_ok ? total / kVec : total;
+  NestArgs<NIN + 1> args = MakeNestArgs<NIN + 1>(nest);
+  const int64_t blocks_needed = (n_items + kBlock - 1) / kBlock;
+  const uint32_t grid = static_cast<uint32_t>(std::min<int64_t>(blocks_needed, 256 * 32));
+  if (vec_ok) {
+    hipLaunchKernelGGL((EwKernel<NIN, kVec, TO, T0, T1, T2, Op>), dim3(grid), dim3(kBlock), 0, stream, args,
+                       static_cast<uint32_t>(n_items), bcast, static_cast<TO *>(out), static_cast<const T0 *>(in0),
+                       static_cast<const T1 *>(in1), static_cast<const T2 *>(in2), op);
+  } else {
+    hipLaunchKernelGGL((EwKernel<NIN, 1, TO, T0, T1, T2, Op>), dim3(grid), dim3(kBlock), 0, stream, args,
+                       static_cast<uint32_t>(n_items), 0u, static_cast<TO *>(out), static_cast<const T0 *>(in0),
+                       static_cast<const T1 *>(in1), static_cast<const T2 *>(in2), op);
+  }
+  return LaunchStatus();
+}
+
+// ---- functors ---------------------------------------------------------------
+
+template <typename T>
+struct AddC {
+  T c;
+  __device__ T operator()(T x, Empty, Empty) const { return x + c; }
+};
+template <typename T>
+struct RSubC {
+  T c;
+  __device__ T operator()(T x, Empty, Empty) const { return c - x; }
+};
+template <typename T>
+struct MulC {
+  T c;
+  __device__ T operator()(T x, Empty, Empty) const { return x * c; }
+};
+struct DivC {
+  float c;
+  __device__ float operator()(float x, Empty, Empty) const { return x / c; }
+};
+struct PowC {
+  float c;
+  __device__ float operator()(float x, Empty, Empty) const { return powf(x, c); }
+};
+struct Erf {
+  __device__ float operator()(float x, Empty, Empty) const { return erff(x); }
+};
+struct Relu {
+  // arith.maximumf against 0 propagates NaN (reference relu.cpp:12-46)
+  __device__ float operator()(float x, Empty, Empty) const { return x != x ? x : fmaxf(x, 0.0f); }
+};
+struct Clip {
+  float lo, hi;
+  __device__ float operator()(float x, Empty, Empty) const {
+    return x != x ? x : fminf(fmaxf(x, lo), hi);
+  }
+};
+struct Tanh {
+  __device__ float operator()(float x, Empty, Empty) const { return tanhf(x); }
+};
+struct Sqrt {
+  __device__ float operator()(float x, Empty, Empty) const { return sqrtf(x); }
+};
+struct Neg {
+  __device__ float operator()(float x, Empty, Empty) const { return -x; }
+};
+struct Not {
+  __device__ uint8_t operator()(uint8_t x, Empty, Empty) const { return x ^ 1u; }
+};
+template <typename TO, typename TI>
+struct Copy {
+  __device__ TO operator()(TI x, Empty, Empty) const { return static_cast<TO>(x); }
+};
+struct EqC {
+  int64_t c;
+  __device__ uint8_t operator()(int64_t x, Empty, Empty) const { return x == c ? 1 : 0; }
+};
+template <typename T>
+struct Add2 {
+  __device__ T operator()(T a, T b, Empty) const { return a + b; }
+};
+template <typename T>
+struct Sub2 {
+  __device__ T operator()(T a, T b, Empty) const { return a - b; }
+};
+template <typename T>
+struct Mul2 {
+  __device__ T operator()(T a, T b, Empty) const { return a * b; }
+};
+struct Div2 {
+  __device__ float operator()(float a, float b, Empty) const { return a / b; }
+};
+struct WhereScalarY {
+  float y;
+  __device__ float operator()(uint8_t c, float x, Empty) const { return c ? x : y; }
+};
+struct WhereTensorY {
+  __device__ float operator()(uint8_t c, float x, float y) const { return c ? x : y; }
+};
+struct Gelu {
+  // t = x + b; t * (erf(t / c_div) + c_add) * c_mul, evaluated in the order of
+  // reference add_div_erf_add_mul_mul.cpp:29-132: mul0 = t * (erf + c_add); out = mul0 * c_mul
+  float c_div, c_add, c_mul;
+  __device__ float operator()(float x, float b, Empty) const {
+    const float t = x + b;
+    return (t * (erff(t / c_div) + c_add)) * c_mul;
+  }
+};
+struct SubMul {
+  float c_sub, c_mul;
+  __device__ float operator()(float x, Empty, Empty) const { return (c_sub - x) * c_mul; }
+};
+
+// ---- nest builders ----------------------------------------------------------
+
+int IdentityNest(const fl_tensor *in, const fl_tensor *out, LoopNest *nest) {
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (!SameShape(in, out)) return FL_ERR_SHAPE;
+  nest->rank = out->rank;
+  nest->n_operands = 2;
+  for (int i = 0; i < out->rank; ++i) {
+    nest->shape[i] = out->shape[i];
+    nest->strides[0][i] = out->strides[i];
+    nest->strides[1][i] = in->strides[i];
+  }
+  return FL_OK;
+}
+
+int BroadcastNest(const fl_tensor *const *ins, int n_in, const fl_tensor *out, LoopNest *nest) {
+  FL_CHECK(CheckView(out));
+  nest->rank = out->rank;
+  nest->n_operands = n_in + 1;
+  for (int i = 0; i < out->rank; ++i) {
+    nest->shape[i] = out->shape[i];
+    nest->strides[0][i] = out->strides[i];
+  }
+  for (int k = 0; k < n_in; ++k) {
+    FL_CHECK(CheckView(ins[k]));
+    FL_CHECK(BroadcastStrides(ins[k], out->rank, out->shape, nest->strides[k + 1]));
+  }
+  return FL_OK;
+}
+
+template <typename TO, typename TI, typename Op>
+int Unary(const LoopNest &nest, const fl_tensor *in, const fl_tensor *out, Op op, void *stream) {
+  return LaunchNest<1, TO, TI, Empty, Empty>(nest, out->base, in->base, nullptr, nullptr, op, AsStream(stream));
+}
+
+template <typename Op>
+int UnaryF32(const fl_tensor *in, const fl_tensor *out, Op op, void *stream) {
+  LoopNest nest;
+  FL_CHECK(IdentityNest(in, out, &nest));
+  if (in->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  return Unary<float, float>(nest, in, out, op, stream);
+}
+
+template <typename T, typename Op>
+int Binary(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, Op op, void *stream) {
+  const fl_tensor *ins[2] = {lhs, rhs};
+  LoopNest nest;
+  FL_CHECK(BroadcastNest(ins, 2, out, &nest));
+  return LaunchNest<2, T, T, T, Empty>(nest, out->base, lhs->base, rhs->base, nullptr, op, AsStream(stream));
+}
+
+// Copy `in` (already re-strided to the output's index space) into `out`,
+// whatever the (equal) element type is.
+int CopyNest(const LoopNest &nest, const fl_tensor *in, const fl_tensor *out, void *stream) {
+  if (in->dtype != out->dtype) return FL_ERR_DTYPE;
+  switch (DtypeSize(out->dtype)) {
+    case 1: return Unary<uint8_t, uint8_t>(nest, in, out, Copy<uint8_t, uint8_t>{}, stream);
+    case 2: return Unary<uint16_t, uint16_t>(nest, in, out, Copy<uint16_t, uint16_t>{}, stream);
+    case 4: return Unary<uint32_t, uint32_t>(nest, in, out, Copy<uint32_t, uint32_t>{}, stream);
+    case 8: return Unary<uint64_t, uint64_t>(nest, in, out, Copy<uint64_t, uint64_t>{}, stream);
+    default: return FL_ERR_DTYPE;
+  }
+}
+
+}  // namespace
+
+// Shared with other translation units: strided copy of `in` viewed with
+// `in_strides`/`in_offset` over the index space `shape` of the output view.
+int StridedCopy(const fl_tensor *in, int64_t in_offset, const int64_t *in_strides, const fl_tensor *out,
+                int64_t out_offset, int rank, const int64_t *shape, const int64_t *out_strides, void *stream) {
+  LoopNest nest;
+  nest.rank = rank;
+  nest.n_operands = 2;
+  for (int i = 0; i < rank; ++i) {
+    nest.shape[i] = shape[i];
+    nest.strides[0][i] = out_strides[i];
+    nest.strides[1][i] = in_strides[i];
+  }
+  fl_tensor i2 = *in, o2 = *out;
+  const size_t esz = DtypeSize(in->dtype);
+  i2.base = static_cast<char *>(in->base) + in_offset * static_cast<int64_t>(esz);
+  o2.base = static_cast<char *>(out->base) + out_offset * static_cast<int64_t>(esz);
+  return CopyNest(nest, &i2, &o2, stream);
+}
+
+}  // namespace fl
+
+using namespace fl;
+
+extern "C" {
+
+int fluidml_hip_add_constant(const fl_tensor *in, const fl_tensor *out, double value, void *stream) {
+  LoopNest nest;
+  FL_CHECK(IdentityNest(in, out, &nest));
+  if (in->dtype != out->dtype) return FL_ERR_DTYPE;
+  switch (in->dtype) {
+    case FL_FLOAT32: return Unary<float, float>(nest, in, out, AddC<float>{static_cast<float>(value)}, stream);
+    case FL_INT32: return Unary<int32_t, int32_t>(nest, in, out, AddC<int32_t>{static_cast<int32_t>(value)}, stream);
+    case FL_INT64: return Unary<int64_t, int64_t>(nest, in, out, AddC<int64_t>{static_cast<int64_t>(value)}, stream);
+    default: return FL_ERR_DTYPE;
+  }
+}
+
+int fluidml_hip_add_common(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
+  if (!lhs || !rhs || !out) return FL_ERR_NULL;
+  if (lhs->dtype != FL_FLOAT32 || rhs->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  return Binary<float>(lhs, rhs, out, Add2<float>{}, stream);
+}
+
+int fluidml_hip_sub_constant_lhs(const fl_tensor *in, const fl_tensor *out, double value, void *stream) {
+  return UnaryF32(in, out, RSubC<float>{static_cast<float>(value)}, stream);
+}
+
+int fluidml_hip_sub_common(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
+  if (!lhs || !rhs || !out) return FL_ERR_NULL;
+  if (lhs->dtype != FL_FLOAT32 || rhs->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  return Binary<float>(lhs, rhs, out, Sub2<float>{}, stream);
+}
+
+int fluidml_hip_mul_constant(const fl_tensor *in, const fl_tensor *out, double value, void *stream) {
+  return UnaryF32(in, out, MulC<float>{static_cast<float>(value)}, stream);
+}
+
+int fluidml_hip_mul_common(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
+  if (!lhs || !rhs || !out) return FL_ERR_NULL;
+  if (lhs->dtype != rhs->dtype || lhs->dtype != out->dtype) return FL_ERR_DTYPE;
+  switch (out->dtype) {
+    case FL_FLOAT32: return Binary<float>(lhs, rhs, out, Mul2<float>{}, stream);
+    case FL_INT32: return Binary<int32_t>(lhs, rhs, out, Mul2<int32_t>{}, stream);
+    case FL_INT64: return Binary<int64_t>(lhs, rhs, out, Mul2<int64_t>{}, stream);
+    default: return FL_ERR_DTYPE;
+  }
+}
+
+int fluidml_hip_div_constant_rhs(const fl_tensor *in, const fl_tensor *out, double value, void *stream) {
+  return UnaryF32(in, out, DivC{static_cast<float>(value)}, stream);
+}
+
+int fluidml_hip_div_common(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
+  if (!lhs || !rhs || !out) return FL_ERR_NULL;
+  if (lhs->dtype != FL_FLOAT32 || rhs->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  return Binary<float>(lhs, rhs, out, Div2{}, stream);
+}
+
+int fluidml_hip_pow(const fl_tensor *in, const fl_tensor *out, double exponent, void *stream) {
+  return UnaryF32(in, out, PowC{static_cast<float>(exponent)}, stream);
+}
+
+int fluidml_hip_erf(const fl_tensor *in, const fl_tensor *out, void *stream) { return UnaryF32(in, out, Erf{}, stream); }
+
+int fluidml_hip_relu(const fl_tensor *in, const fl_tensor *out, void *stream) { return UnaryF32(in, out, Relu{}, stream); }
+
+int fluidml_hip_clip(const fl_tensor *in, const fl_tensor *out, float lo, float hi, void *stream) {
+  return UnaryF32(in, out, Clip{lo, hi}, stream);
+}
+
+int fluidml_hip_tanh(const fl_tensor *in, const fl_tensor *out, void *stream) { return UnaryF32(in, out, Tanh{}, stream); }
+
+int fluidml_hip_sqrt(const fl_tensor *in, const fl_tensor *out, void *stream) { return UnaryF32(in, out, Sqrt{}, stream); }
+
+int fluidml_hip_neg(const fl_tensor *in, const fl_tensor *out, void *stream) { return UnaryF32(in, out, Neg{}, stream); }
+
+int fluidml_hip_not(const fl_tensor *in, const fl_tensor *out, void *stream) {
+  LoopNest nest;
+  FL_CHECK(IdentityNest(in, out, &nest));
+  if (in->dtype != FL_BOOL || out->dtype != FL_BOOL) return FL_ERR_DTYPE;
+  return Unary<uint8_t, uint8_t>(nest, in, out, Not{}, stream);
+}
+
+int fluidml_hip_cast(const fl_tensor *in, const fl_tensor *out, void *stream) {
+  LoopNest nest;
+  FL_CHECK(IdentityNest(in, out, &nest));
+#define FL_CAST_CASE(TI_E, TI, TO_E, TO) \
+  if (in->dtype == TI_E && out->dtype == TO_E) return Unary<TO, TI>(nest, in, out, Copy<TO, TI>{}, stream)
+  FL_CAST_CASE(FL_BOOL, uint8_t, FL_BOOL, uint8_t);
+  FL_CAST_CASE(FL_BOOL, uint8_t, FL_INT32, int32_t);
+  FL_CAST_CASE(FL_BOOL, uint8_t, FL_INT64, int64_t);
+  FL_CAST_CASE(FL_INT32, int32_t, FL_INT32, int32_t);
+  FL_CAST_CASE(FL_INT32, int32_t, FL_INT64, int64_t);
+  FL_CAST_CASE(FL_INT64, int64_t, FL_INT32, int32_t);
+  FL_CAST_CASE(FL_INT64, int64_t, FL_INT64, int64_t);
+#undef FL_CAST_CASE
+  return FL_ERR_DTYPE;
+}
+
+int fluidml_hip_equal(const fl_tensor *in, const fl_tensor *out, double value, void *stream) {
+  LoopNest nest;
+  FL_CHECK(IdentityNest(in, out, &nest));
+  if (in->dtype != FL_INT64 || out->dtype != FL_BOOL) return FL_ERR_DTYPE;
+  return Unary<uint8_t, int64_t>(nest, in, out, EqC{static_cast<int64_t>(value)}, stream);
+}
+
+int fluidml_hip_dropout(const fl_tensor *in, const fl_tensor *out, void *stream) {
+  LoopNest nest;
+  FL_CHECK(IdentityNest(in, out, &nest));
+  return CopyNest(nest, in, out, stream);
+}
+
+int fluidml_hip_where_constant_cond_constant_scalar_y(const fl_tensor *cond, const fl_tensor *x, const fl_tensor *out,
+                                                      double y, void *stream) {
+  if (!cond || !x || !out) return FL_ERR_NULL;
+  if (cond->dtype != FL_BOOL || x->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  const fl_tensor *ins[2] = {cond, x};
+  LoopNest nest;
+  FL_CHECK(BroadcastNest(ins, 2, out, &nest));
+  return LaunchNest<2, float, uint8_t, float, Empty>(nest, out->base, cond->base, x->base, nullptr,
+                                                     WhereScalarY{static_cast<float>(y)}, AsStream(stream));
+}
+
+int fluidml_hip_where_constant_cond_constant_tensor_y(const fl_tensor *cond, const fl_tensor *x, const fl_tensor *y,
+                                                      const fl_tensor *out, void *stream) {
+  if (!cond || !x || !y || !out) return FL_ERR_NULL;
+  if (cond->dtype != FL_BOOL || x->dtype != FL_FLOAT32 || y->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32)
+    return FL_ERR_DTYPE;
+  const fl_tensor *ins[3] = {cond, x, y};
+  LoopNest nest;
+  FL_CHECK(BroadcastNest(ins, 3, out, &nest));
+  return LaunchNest<3, float, uint8_t, float, float>(nest, out->base, cond->base, x->base, y->base, WhereTensorY{},
+                                                     AsStream(stream));
+}
+
+int fluidml_hip_add_div_erf_add_mul_mul(const fl_tensor *in, const fl_tensor *add0, const fl_tensor *out, double div,
+                                        double add1, double mul1, void *stream) {
+  if (!in || !add0 || !out) return FL_ERR_NULL;
+  if (in->dtype != FL_FLOAT32 || add0->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  const fl_tensor *ins[2] = {in, add0};
+  LoopNest nest;
+  FL_CHECK(BroadcastNest(ins, 2, out, &nest));
+  return LaunchNest<2, float, float, float, Empty>(
+      nest, out->base, in->base, add0->base, nullptr,
+      Gelu{static_cast<float>(div), static_cast<float>(add1), static_cast<float>(mul1)}, AsStream(stream));
+}
+
+// Strides of `in` in the index space of an output that has extra unit dims at
+// `axes` (negative axes count from the output rank).
+static int UnsqueezedStrides(const fl_tensor *in, const fl_tensor *out, const int64_t *axes, int32_t n_axes,
+                             int64_t *strides) {
+  if (n_axes < 0 || (n_axes > 0 && axes == nullptr)) return FL_ERR_ATTR;
+  if (in->rank + n_axes != out->rank) return FL_ERR_RANK;
+  int j = 0;
+  for (int i = 0; i < out->rank; ++i) {
+    bool is_axis = false;
+    for (int k = 0; k < n_axes; ++k) {
+      const int64_t ax = axes[k] < 0 ? axes[k] + out->rank : axes[k];
+      if (ax < 0 || ax >= out->rank) return FL_ERR_ATTR;
+      if (ax == i) is_axis = true;
+    }
+    if (is_axis) {
+      if (out->shape[i] != 1) return FL_ERR_SHAPE;
+      strides[i] = 0;
+    } else {
+      if (j >= in->rank || in->shape[j] != out->shape[i]) return FL_ERR_SHAPE;
+      strides[i] = in->strides[j++];
+    }
+  }
+  return j == in->rank ? FL_OK : FL_ERR_SHAPE;
+}
+
+int fluidml_hip_unsqueeze_sub_lhs_scalar_mul_rhs_scalar(const fl_tensor *in, const fl_tensor *out, const int64_t *axes,
+                                                        int32_t n_axes, double sub, double mul, void *stream) {
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (in->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  LoopNest nest;
+  nest.rank = out->rank;
+  nest.n_operands = 2;
+  FL_CHECK(UnsqueezedStrides(in, out, axes, n_axes, nest.strides[1]));
+  for (int i = 0; i < out->rank; ++i) {
+    nest.shape[i] = out->shape[i];
+    nest.strides[0][i] = out->strides[i];
+  }
+  return Unary<float, float>(nest, in, out, SubMul{static_cast<float>(sub), static_cast<float>(mul)}, stream);
+}
+
+int fluidml_hip_unsqueeze(const fl_tensor *in, const fl_tensor *out, const int64_t *axes, int32_t n_axes, void *stream) {
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  LoopNest nest;
+  nest.rank = out->rank;
+  nest.n_operands = 2;
+  FL_CHECK(UnsqueezedStrides(in, out, axes, n_axes, nest.strides[1]));
+  for (int i = 0; i < out->rank; ++i) {
+    nest.shape[i] = out->shape[i];
+    nest.strides[0][i] = out->strides[i];
+  }
+  return CopyNest(nest, in, out, stream);
+}
+
+int fluidml_hip_squeeze(const fl_tensor *in, const fl_tensor *out, const int64_t *axes, int32_t n_axes, void *stream) {
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (n_axes < 0 || (n_axes > 0 && axes == nullptr)) return FL_ERR_ATTR;
+  if (in->rank != out->rank + n_axes) return FL_ERR_RANK;
+  // reference squeeze.cpp:17-54 matches axes against the raw input index
+  LoopNest nest;
+  nest.rank = out->rank;
+  nest.n_operands = 2;
+  int j = 0;
+  for (int i = 0; i < in->rank; ++i) {
+    bool squeezed = false;
+    for (int k = 0; k < n_axes; ++k) {
+      const int64_t ax = axes[k] < 0 ? axes[k] + in->rank : axes[k];
+      if (ax == i) squeezed = true;
+    }
+    if (squeezed) {
+      if (in->shape[i] != 1) return FL_ERR_SHAPE;
+    } else {
+      if (j >= out->rank || out->shape[j] != in->shape[i]) return FL_ERR_SHAPE;
+      nest.shape[j] = out->shape[j];
+      nest.strides[0][j] = out->strides[j];
+      nest.strides[1][j] = in->strides[i];
+      ++j;
+    }
+  }
+  if (j != out->rank) return FL_ERR_SHAPE;
+  return CopyNest(nest, in, out, stream);
+}
+
+int fluidml_hip_transpose(const fl_tensor *in, const fl_tensor *out, const int64_t *perm, int32_t n_perm, void *stream) {
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (perm == nullptr) return FL_ERR_NULL;
+  if (n_perm != in->rank || in->rank != out->rank) return FL_ERR_RANK;
+  LoopNest nest;
+  nest.rank = out->rank;
+  nest.n_operands = 2;
+  bool seen[kMaxRank] = {};
+  for (int i = 0; i < out->rank; ++i) {
+    const int64_t p = perm[i];
+    if (p < 0 || p >= in->rank || seen[p]) return FL_ERR_ATTR;
+    seen[p] = true;
+    if (out->shape[i] != in->shape[p]) return FL_ERR_SHAPE;
+    nest.shape[i] = out->shape[i];
+    nest.strides[0][i] = out->strides[i];
+    nest.strides[1][i] = in->strides[p];
+  }
+  return CopyNest(nest, in, out, stream);
+}
+
+int fluidml_hip_slice(const fl_tensor *in, const fl_tensor *out, const int64_t *starts, const int64_t *axes,
+                      const int64_t *steps, int32_t n, void *stream) {
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (in->rank != out->rank) return FL_ERR_RANK;
+  if (n < 0 || (n > 0 && (!starts || !axes || !steps))) return FL_ERR_ATTR;
+  int64_t offs[kMaxRank] = {}, step[kMaxRank];
+  for (int i = 0; i < in->rank; ++i) step[i] = 1;
+  for (int k = 0; k < n; ++k) {
+    const int64_t ax = axes[k];
+    if (ax < 0 || ax >= in->rank || steps[k] <= 0 || starts[k] < 0) return FL_ERR_ATTR;
+    offs[ax] = starts[k];
+    step[ax] = steps[k];
+  }
+  int64_t in_offset = 0, in_strides[kMaxRank];
+  for (int i = 0; i < in->rank; ++i) {
+    if (offs[i] + (out->shape[i] - 1) * step[i] >= in->shape[i]) return FL_ERR_SHAPE;
+    in_offset += offs[i] * in->strides[i];
+    in_strides[i] = in->strides[i] * step[i];
+  }
+  return StridedCopy(in, in_offset, in_strides, out, 0, out->rank, out->shape, out->strides, stream);
+}
+
+int fluidml_hip_concat2(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, int64_t axis, void *stream) {
+  FL_CHECK(CheckView(lhs));
+  FL_CHECK(CheckView(rhs));
+  FL_CHECK(CheckView(out));
+  if (lhs->rank != out->rank || rhs->rank != out->rank) return FL_ERR_RANK;
+  if (axis < 0 || axis >= out->rank) return FL_ERR_ATTR;
+  if (lhs->dtype != out->dtype || rhs->dtype != out->dtype) return FL_ERR_DTYPE;
+  for (int i = 0; i < out->rank; ++i) {
+    if (i == axis) {
+      if (lhs->shape[i] + rhs->shape[i] != out->shape[i]) return FL_ERR_SHAPE;
+    } else if (lhs->shape[i] != out->shape[i] || rhs->shape[i] != out->shape[i]) {
+      return FL_ERR_SHAPE;
+    }
+  }
+  FL_CHECK(StridedCopy(lhs, 0, lhs->strides, out, 0, out->rank, lhs->shape, out->strides, stream));
+  return StridedCopy(rhs, 0, rhs->strides, out, lhs->shape[axis] * out->strides[axis], out->rank, rhs->shape,
+                     out->strides, stream);
+}
+
+int fluidml_hip_pad(const fl_tensor *in, const fl_tensor *out, const int64_t *pads_before, int32_t n, void *stream) {
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (in->rank != out->rank || n != in->rank) return FL_ERR_RANK;
+  if (pads_before == nullptr && n > 0) return FL_ERR_NULL;
+  int64_t out_offset = 0;
+  for (int i = 0; i < in->rank; ++i) {
+    if (pads_before[i] < 0 || pads_before[i] + in->shape[i] > out->shape[i]) return FL_ERR_SHAPE;
+    out_offset += pads_before[i] * out->strides[i];
+  }
+  return StridedCopy(in, 0, in->strides, out, out_offset, in->rank, in->shape, out->strides, stream);
+}
+
+int fluidml_hip_gather_constant_index_scalar(const fl_tensor *in, const fl_tensor *out, int64_t axis, int64_t index,
+                                             uint32_t flags, void *stream) {
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (in->rank != out->rank + 1) return FL_ERR_RANK;
+  // The reference normalises `axis` into a local it never uses and compares
+  // loop positions with the raw attribute (gather.cpp:113-124).
+  int64_t ax = axis;
+  if (!(flags & FL_REF_GATHER_RAW_AXIS) && ax < 0) ax += in->rank;
+  if (ax < 0 || ax >= in->rank) return (flags & FL_REF_GATHER_RAW_AXIS) ? FL_ERR_UNSUPPORTED : FL_ERR_ATTR;
+  if (index < 0 || index >= in->shape[ax]) return FL_ERR_ATTR;
+  int64_t in_strides[kMaxRank];
+  for (int i = 0, j = 0; i < in->rank; ++i) {
+    if (i == ax) continue;
+    if (in->shape[i] != out->shape[j]) return FL_ERR_SHAPE;
+    in_strides[j++] = in->strides[i];
+  }
+  return StridedCopy(in, index * in->strides[ax], in_strides, out, 0, out->rank, out->shape, out->strides, stream);
+}
+
+}  // extern "C"

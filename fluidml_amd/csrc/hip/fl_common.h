@@ -1,0 +1,266 @@
+// Shared host/device helpers for the gfx950 kernels behind include/fluidml_hip.h.
+//
+// Every kernel in this backend takes strided views (reference kernels read
+// shape and strides from the memref type, src/worker/builder.cpp:234-270), so
+// the common work is: validate views on the host, put the loop nest in the
+// output's physical order, merge dimensions that are contiguous for every
+// operand, and hand the device a small by-value descriptor with 32-bit
+// division constants.
+#ifndef FLUIDML_AMD_CSRC_HIP_FL_COMMON_H_
+#define FLUIDML_AMD_CSRC_HIP_FL_COMMON_H_
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstring>
+
+#include "fluidml_hip.h"
+
+namespace fl {
+
+constexpr int kMaxRank = FL_MAX_RANK;
+constexpr int kWave = 64;  // CDNA wavefront
+
+#define FL_HIP_CHECK(expr)                      \
+  do {                                          \
+    hipError_t fl_err__ = (expr);               \
+    if (fl_err__ != hipSuccess) {               \
+      return static_cast<int>(fl_err__);        \
+    }                                           \
+  } while (0)
+
+#define FL_CHECK(expr)            \
+  do {                            \
+    int fl_rc__ = (expr);         \
+    if (fl_rc__ != FL_OK) {       \
+      return fl_rc__;             \
+    }                             \
+  } while (0)
+
+inline hipStream_t AsStream(void *stream) { return static_cast<hipStream_t>(stream); }
+
+inline int LaunchStatus() {
+  hipError_t err = hipGetLastError();
+  return err == hipSuccess ? FL_OK : static_cast<int>(err);
+}
+
+inline size_t DtypeSize(int32_t dtype) {
+  switch (dtype) {
+    case FL_BOOL: return 1;
+    case FL_INT32: return 4;
+    case FL_INT64: return 8;
+    case FL_FLOAT16: return 2;
+    case FL_FLOAT32: return 4;
+    case FL_FLOAT64: return 8;
+    default: return 0;
+  }
+}
+
+// Division by a run-time constant for dividends below 2^31: one mul-hi and a
+// shift on the device instead of a ~40 instruction udiv sequence.
+struct FastDiv {
+  uint32_t divisor;
+  uint32_t multiplier;
+  uint32_t shift;
+
+  FastDiv() : divisor(1), multiplier(0), shift(0) {}
+  explicit FastDiv(uint32_t d) : divisor(d), multiplier(0), shift(0) {
+    if (d > 1) {
+      uint32_t log2_ceil = 0;
+      while ((1ull << log2_ceil) < d) ++log2_ceil;
+      const uint32_t p = 31 + log2_ceil;
+      multiplier = static_cast<uint32_t>(((1ull << p) + d - 1) / d);
+      shift = p - 32;
+    }
+  }
+  __host__ __device__ __forceinline__ uint32_t Div(uint32_t n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return divisor == 1 ? n : (__umulhi(n, multiplier) >> shift);
+#else
+    return n / divisor;
+#endif
+  }
+  __host__ __device__ __forceinline__ void DivMod(uint32_t n, uint32_t &q, uint32_t &r) const {
+    q = Div(n);
+    r = n - q * divisor;
+  }
+};
+
+// ---- host-side view checks ------------------------------------------------
+
+inline int CheckView(const fl_tensor *t) {
+  if (t == nullptr || t->base == nullptr) return FL_ERR_NULL;
+  if (t->rank < 0 || t->rank > kMaxRank) return FL_ERR_RANK;
+  if (DtypeSize(t->dtype) == 0) return FL_ERR_DTYPE;
+  int64_t numel = 1, span = 0;
+  for (int i = 0; i < t->rank; ++i) {
+    if (t->shape[i] <= 0) return FL_ERR_SHAPE;
+    if (t->strides[i] < 0) return FL_ERR_SHAPE;
+    numel *= t->shape[i];
+    span += (t->shape[i] - 1) * t->strides[i];
+    if (numel > INT32_MAX || span > INT32_MAX) return FL_ERR_TOO_LARGE;
+  }
+  return FL_OK;
+}
+
+inline int64_t Numel(const fl_tensor *t) {
+  int64_t n = 1;
+  for (int i = 0; i < t->rank; ++i) n *= t->shape[i];
+  return n;
+}
+
+inline bool SameShape(const fl_tensor *a, const fl_tensor *b) {
+  if (a->rank != b->rank) return false;
+  for (int i = 0; i < a->rank; ++i) {
+    if (a->shape[i] != b->shape[i]) return false;
+  }
+  return true;
+}
+
+inline bool IsAligned(const void *p, size_t bytes) {
+  return (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
+}
+
+// A loop nest over up to kMaxRank dimensions and up to kMaxOperands strided
+// operands; operand 0 is the output.  Built in logical order, then
+// canonicalised: unit dims dropped, dims ordered by descending output stride
+// (so the innermost loop walks the output's fastest physical dimension), and
+// neighbours merged when every operand agrees they are contiguous.
+constexpr int kMaxOperands = 5;
+
+struct LoopNest {
+  int rank = 0;
+  int n_operands = 0;
+  int64_t shape[kMaxRank] = {};
+  int64_t strides[kMaxOperands][kMaxRank] = {};
+
+  void Canonicalise() {
+    // drop unit dims
+    int w = 0;
+    for (int i = 0; i < rank; ++i) {
+      if (shape[i] != 1) {
+        shape[w] = shape[i];
+        for (int o = 0; o < n_operands; ++o) strides[o][w] = strides[o][i];
+        ++w;
+      }
+    }
+    rank = w;
+    // stable insertion sort by descending output stride; ties keep logical order
+    for (int i = 1; i < rank; ++i) {
+      for (int j = i; j > 0 && strides[0][j - 1] < strides[0][j]; --j) {
+        std::swap(shape[j - 1], shape[j]);
+        for (int o = 0; o < n_operands; ++o) std::swap(strides[o][j - 1], strides[o][j]);
+      }
+    }
+    // merge dim i into i-1 when stride[i-1] == stride[i] * shape[i] for all operands
+    w = 0;
+    for (int i = 0; i < rank; ++i) {
+      bool merge = w > 0;
+      if (merge) {
+        for (int o = 0; o < n_operands; ++o) {
+          if (strides[o][w - 1] != strides[o][i] * shape[i]) {
+            merge = false;
+            break;
+          }
+        }
+      }
+      if (merge) {
+        shape[w - 1] *= shape[i];
+        for (int o = 0; o < n_operands; ++o) strides[o][w - 1] = strides[o][i];
+      } else {
+        shape[w] = shape[i];
+        for (int o = 0; o < n_operands; ++o) strides[o][w] = strides[o][i];
+        ++w;
+      }
+    }
+    rank = w;
+    if (rank == 0) {
+      rank = 1;
+      shape[0] = 1;
+      for (int o = 0; o < n_operands; ++o) strides[o][0] = 0;
+    }
+  }
+};
+
+// Strides of `t` broadcast against an output of rank `out_rank`/`out_shape`
+// with trailing alignment: equal dim -> its stride, dim 1 -> 0 (reference
+// GetBroadcastAffineMaps, src/structure/kernel/kernel/utils.cpp:16-52).
+inline int BroadcastStrides(const fl_tensor *t, int out_rank, const int64_t *out_shape, int64_t *strides) {
+  if (t->rank > out_rank) return FL_ERR_RANK;
+  for (int i = 0; i < out_rank; ++i) {
+    const int j = t->rank - out_rank + i;
+    if (j < 0) {
+      strides[i] = 0;
+    } else if (t->shape[j] == out_shape[i]) {
+      strides[i] = t->strides[j];
+    } else if (t->shape[j] == 1) {
+      strides[i] = 0;
+    } else {
+      return FL_ERR_SHAPE;
+    }
+  }
+  return FL_OK;
+}
+
+// Device-side descriptor of a canonical loop nest.
+template <int NOPS>
+struct NestArgs {
+  int32_t rank;
+  uint32_t shape[kMaxRank];
+  FastDiv div[kMaxRank];
+  int32_t strides[NOPS][kMaxRank];
+};
+
+template <int NOPS>
+inline NestArgs<NOPS> MakeNestArgs(const LoopNest &nest) {
+  NestArgs<NOPS> a;
+  std::memset(&a, 0, sizeof(a));
+  a.rank = nest.rank;
+  for (int i = 0; i < nest.rank; ++i) {
+    a.shape[i] = static_cast<uint32_t>(nest.shape[i]);
+    a.div[i] = FastDiv(static_cast<uint32_t>(nest.shape[i]));
+    for (int o = 0; o < NOPS; ++o) a.strides[o][i] = static_cast<int32_t>(nest.strides[o][i]);
+  }
+  return a;
+}
+
+// ---- device-side reductions -------------------------------------------------
+
+#if defined(__HIPCC__)
+template <typename T, typename F>
+__device__ __forceinline__ T WaveReduce(T v, F f) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    v = f(v, __shfl_xor(v, off, kWave));
+  }
+  return v;
+}
+
+struct SumOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+struct MaxOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+
+// Reduce across a block of NWAVES waves; `smem` needs NWAVES floats. All
+// threads get the result.
+template <int NWAVES, typename F>
+__device__ __forceinline__ float BlockReduce(float v, F f, float *smem) {
+  v = WaveReduce(v, f);
+  if (NWAVES == 1) return v;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  __syncthreads();  // protect smem from a previous use
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  float r = smem[0];
+#pragma unroll
+  for (int w = 1; w < NWAVES; ++w) r = f(r, smem[w]);
+  return r;
+}
+#endif  // __HIPCC__
+
+}  // namespace fl
+
+#endif  // FLUIDML_AMD_CSRC_HIP_FL_COMMON_H_

@@ -1,0 +1,455 @@
+// fp32 contractions on the CDNA4 matrix cores: MatMul (NumPy batch broadcast)
+// and Gemm (rank-2 with alpha/beta/bias epilogue).
+// Reference: src/structure/kernel/kernel/matmul.cpp:28-59, gemm.cpp:39-182,
+// utils.cpp:64-147 (broadcast maps).
+//
+// C[b..., m, n] = sum_k A[b..., m, k] * B[b..., k, n] over arbitrary element
+// strides: the layout the planner picked only decides which of (m,k) resp.
+// (k,n) is walked by the 128-bit global loads and how the tile sits in LDS.
+//
+//   * v_mfma_f32_32x32x2_f32 (64 lanes x 1 A value, 1 B value -> 32x32 fp32
+//     accumulators, 16 per lane); a wave owns TM x TN such tiles;
+//   * tiles are staged global -> registers -> LDS with double buffering, one
+//     barrier per K chunk; an operand that is k-contiguous in memory is kept
+//     [x][k] (+4 pad, 128-bit LDS reads), otherwise [k][x] (32-bit reads);
+//   * each lane half handles 4 consecutive k per group of 8 (the k order inside
+//     a sum is free), so the [x][k] layout needs one ds_read_b128 per 4 MFMAs;
+//   * small problems split each K chunk over the waves of a workgroup and
+//     combine the partial tiles through LDS, so M=128-row problems still put
+//     4 waves on every tile;
+//   * workgroup ids are folded so that consecutive tiles land on one XCD and
+//     share its L2.
+//
+// A second, opt-in path rounds operands to bf16 (v_mfma_f32_32x32x8_bf16 would
+// be its instruction); it is not built yet and reports FL_ERR_UNSUPPORTED.
+#include <type_traits>
+
+#include "fl_common.h"
+
+namespace fl {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+struct MatmulArgs {
+  int32_t M, N, K;
+  int32_t sAm, sAk, sBk, sBn, sCm, sCn;
+  NestArgs<3> batch;  // operand 0 = C, 1 = A, 2 = B
+  uint32_t tiles_m, tiles_n;
+  // epilogue: C = ca * acc + cb * bias[m * sDm + n * sDn]   (bias may be null)
+  float ca, cb;
+  const float *bias;
+  int32_t sDm, sDn;
+};
+
+template <int VEC>
+struct VecF {
+  float v[VEC];
+};
+
+template <int VEC>
+__device__ __forceinline__ VecF<VEC> LoadVec(const float *p) {
+  VecF<VEC> r;
+  if constexpr (VEC == 4) {
+    const floatx4 t = *reinterpret_cast<const floatx4 *>(p);
+    r.v[0] = t.x;
+    r.v[1] = t.y;
+    r.v[2] = t.z;
+    r.v[3] = t.w;
+  } else {
+    r.v[0] = *p;
+  }
+  return r;
+}
+
+// Cooperative load of a ROWS x COLS tile whose COLS run along the operand's
+// fast dimension. Out-of-range parts read as 0.
+template <int ROWS, int COLS, int VEC, int NT>
+struct TileLoader {
+  static constexpr int kVecsPerRow = COLS / VEC;
+  static constexpr int kItems = ROWS * kVecsPerRow;
+  static constexpr int kPerThread = (kItems + NT - 1) / NT;
+
+  __device__ __forceinline__ static void Load(const float *g, int row_stride, int col_stride, int rows_valid,
+                                              int cols_valid, VecF<VEC> (&regs)[kPerThread]) {
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+      const int item = threadIdx.x + j * NT;
+      const int row = item / kVecsPerRow, col = (item % kVecsPerRow) * VEC;
+      if (item < kItems && row < rows_valid && col < cols_valid) {
+        regs[j] = LoadVec<VEC>(g + row * row_stride + col * col_stride);
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) regs[j].v[i] = 0.0f;
+      }
+    }
+  }
+
+  __device__ __forceinline__ static void Store(float *lds, int ld, const VecF<VEC> (&regs)[kPerThread]) {
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+      const int item = threadIdx.x + j * NT;
+      const int row = item / kVecsPerRow, col = (item % kVecsPerRow) * VEC;
+      if (item < kItems) {
+        if constexpr (VEC == 4) {
+          floatx4 t = {regs[j].v[0], regs[j].v[1], regs[j].v[2], regs[j].v[3]};
+          *reinterpret_cast<floatx4 *>(lds + row * ld + col) = t;
+        } else {
+          lds[row * ld + col] = regs[j].v[0];
+        }
+      }
+    }
+  }
+};
+
+// LA: 0 = A tile kept [m][k] (A is k-contiguous), 1 = kept [k][m].
+// LB: 0 = B tile kept [k][n] (B is n-contiguous), 1 = kept [n][k].
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC>
+__global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, float *__restrict__ C,
+                                                                const float *__restrict__ A,
+                                                                const float *__restrict__ B) {
+  constexpr int NT = 64 * WM * WN * KS;
+  constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);
+  constexpr int KW = BK / KS;  // k extent one wave covers per chunk
+  static_assert(KW % 8 == 0, "a wave consumes k in groups of 8");
+  constexpr int LDA = LA == 0 ? BK + 4 : BM;
+  constexpr int LDB = LB == 0 ? BN : BK + 4;
+  constexpr int A_ELEMS = LA == 0 ? BM * LDA : BK * LDA;
+  constexpr int B_ELEMS = LB == 0 ? BK * LDB : BN * LDB;
+  constexpr int RED_ELEMS = KS > 1 ? (KS - 1) * BM * BN : 0;
+  constexpr int STAGE_ELEMS = 2 * (A_ELEMS + B_ELEMS);
+  constexpr int LDS_ELEMS = STAGE_ELEMS > RED_ELEMS ? STAGE_ELEMS : RED_ELEMS;
+  __shared__ __attribute__((aligned(16))) float lds[LDS_ELEMS];
+
+  using LoaderA = typename std::conditional<LA == 0, TileLoader<BM, BK, VEC, NT>, TileLoader<BK, BM, VEC, NT>>::type;
+  using LoaderB = typename std::conditional<LB == 0, TileLoader<BK, BN, VEC, NT>, TileLoader<BN, BK, VEC, NT>>::type;
+
+  // ---- which tile -----------------------------------------------------------
+  uint32_t bid = blockIdx.x;
+  const uint32_t n_tiles = p.tiles_m * p.tiles_n;
+  if (n_tiles % 8 == 0) {
+    // ids are dealt round-robin to the 8 XCDs: give each XCD a contiguous run
+    bid = (bid % 8) * (n_tiles / 8) + bid / 8;
+  }
+  const int tile_m = bid % p.tiles_m, tile_n = bid / p.tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  int32_t boff[3] = {0, 0, 0};
+  {
+    uint32_t rem = blockIdx.y;
+    for (int d = p.batch.rank - 1; d > 0; --d) {
+      uint32_t q, r;
+      p.batch.div[d].DivMod(rem, q, r);
+      rem = q;
+#pragma unroll
+      for (int o = 0; o < 3; ++o) boff[o] += static_cast<int32_t>(r) * p.batch.strides[o][d];
+    }
+#pragma unroll
+    for (int o = 0; o < 3; ++o) boff[o] += static_cast<int32_t>(rem) * p.batch.strides[o][0];
+  }
+  const float *Ab = A + boff[1] + static_cast<int64_t>(m0) * p.sAm;
+  const float *Bb = B + boff[2] + static_cast<int64_t>(n0) * p.sBn;
+  float *Cb = C + boff[0];
+
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int ks = wave % KS, wn = (wave / KS) % WN, wm = wave / (KS * WN);
+  const int lrow = lane % 32, half = lane / 32;
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  VecF<VEC> ra[LoaderA::kPerThread], rb[LoaderB::kPerThread];
+  const int rows_m = p.M - m0, cols_n = p.N - n0;
+  const int n_chunks = (p.K + BK - 1) / BK;
+
+  auto load_chunk = [&](int c) {
+    const int k0 = c * BK, k_valid = p.K - k0;
+    if constexpr (LA == 0) {
+      LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAm, p.sAk, rows_m, k_valid, ra);
+    } else {
+      LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAk, p.sAm, k_valid, rows_m, ra);
+    }
+    if constexpr (LB == 0) {
+      LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBk, p.sBn, k_valid, cols_n, rb);
+    } else {
+      LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBn, p.sBk, cols_n, k_valid, rb);
+    }
+  };
+  auto store_chunk = [&](int buf) {
+    float *as = lds + buf * (A_ELEMS + B_ELEMS);
+    float *bs = as + A_ELEMS;
+    LoaderA::Store(as, LDA, ra);
+    LoaderB::Store(bs, LDB, rb);
+  };
+
+  load_chunk(0);
+  store_chunk(0);
+  __syncthreads();
+
+  for (int c = 0; c < n_chunks; ++c) {
+    const bool more = c + 1 < n_chunks;
+    if (more) load_chunk(c + 1);
+    const float *as = lds + (c & 1) * (A_ELEMS + B_ELEMS);
+    const float *bs = as + A_ELEMS;
+#pragma unroll
+    for (int kk = 0; kk < KW; kk += 8) {
+      const int kbase = ks * KW + kk + 4 * half;
+      float a[TM][4], b[TN][4];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = (wm * TM + i) * 32 + lrow;
+        if constexpr (LA == 0) {
+          const floatx4 t = *reinterpret_cast<const floatx4 *>(as + m * LDA + kbase);
+          a[i][0] = t.x;
+          a[i][1] = t.y;
+          a[i][2] = t.z;
+          a[i][3] = t.w;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a[i][e] = as[(kbase + e) * LDA + m];
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int n = (wn * TN + j) * 32 + lrow;
+        if constexpr (LB == 0) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) b[j][e] = bs[(kbase + e) * LDB + n];
+        } else {
+          const floatx4 t = *reinterpret_cast<const floatx4 *>(bs + n * LDB + kbase);
+          b[j][0] = t.x;
+          b[j][1] = t.y;
+          b[j][2] = t.z;
+          b[j][3] = t.w;
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][e], b[j][e], acc[i][j], 0, 0, 0);
+    }
+    if (more) store_chunk((c + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- combine the K slices of a workgroup through LDS ------------------------
+  if constexpr (KS > 1) {
+    // the final barrier of the loop above makes the staging area free
+    if (ks > 0) {
+      float *red = lds + (ks - 1) * BM * BN;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int m = (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
+            const int n = (wn * TN + j) * 32 + lrow;
+            red[m * BN + n] = acc[i][j][e];
+          }
+    }
+    __syncthreads();
+    if (ks > 0) return;
+#pragma unroll
+    for (int s = 1; s < KS; ++s) {
+      const float *red = lds + (s - 1) * BM * BN;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int m = (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
+            const int n = (wn * TN + j) * 32 + lrow;
+            acc[i][j][e] += red[m * BN + n];
+          }
+    }
+  }
+
+  // ---- epilogue ---------------------------------------------------------------
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + (wn * TN + j) * 32 + lrow;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
+        if (m < p.M && n < p.N) {
+          float v = acc[i][j][e];
+          if (p.bias != nullptr) {
+            v = p.ca * v + p.cb * p.bias[m * p.sDm + n * p.sDn];
+          }
+          Cb[static_cast<int64_t>(m) * p.sCm + static_cast<int64_t>(n) * p.sCn] = v;
+        }
+      }
+    }
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC>
+void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
+  MatmulArgs q = p;
+  q.tiles_m = (p.M + BM - 1) / BM;
+  q.tiles_n = (p.N + BN - 1) / BN;
+  hipLaunchKernelGGL((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC>), dim3(q.tiles_m * q.tiles_n, n_batch),
+                     dim3(64 * WM * WN * KS), 0, s, q, C, A, B);
+}
+
+template <int LA, int LB, int VEC>
+void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
+  const int64_t tiles_l = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * n_batch;
+  const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
+  if (tiles_l >= 192) {
+    LaunchConfig<128, 128, 16, 2, 2, 1, LA, LB, VEC>(p, n_batch, C, A, B, s);
+  } else if (tiles_m >= 192) {
+    LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC>(p, n_batch, C, A, B, s);
+  } else {
+    LaunchConfig<32, 32, 32, 1, 1, 4, LA, LB, VEC>(p, n_batch, C, A, B, s);
+  }
+}
+
+int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, bool trans_a, bool trans_b, float ca,
+             float cb, const fl_tensor *bias, void *stream) {
+  FL_CHECK(CheckView(lhs));
+  FL_CHECK(CheckView(rhs));
+  FL_CHECK(CheckView(out));
+  if (lhs->dtype != FL_FLOAT32 || rhs->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  if (lhs->rank < 2 || rhs->rank < 2 || out->rank < 2) return FL_ERR_RANK;
+  if (lhs->rank > out->rank || rhs->rank > out->rank) return FL_ERR_RANK;
+  const int lr = lhs->rank, rr = rhs->rank, orank = out->rank;
+  MatmulArgs p;
+  std::memset(&p, 0, sizeof(p));
+  const int am = trans_a ? lr - 1 : lr - 2, ak = trans_a ? lr - 2 : lr - 1;
+  const int bk = trans_b ? rr - 1 : rr - 2, bn = trans_b ? rr - 2 : rr - 1;
+  p.M = static_cast<int32_t>(out->shape[orank - 2]);
+  p.N = static_cast<int32_t>(out->shape[orank - 1]);
+  p.K = static_cast<int32_t>(lhs->shape[ak]);
+  if (lhs->shape[am] != p.M || rhs->shape[bn] != p.N || rhs->shape[bk] != p.K) return FL_ERR_SHAPE;
+  p.sAm = static_cast<int32_t>(lhs->strides[am]);
+  p.sAk = static_cast<int32_t>(lhs->strides[ak]);
+  p.sBk = static_cast<int32_t>(rhs->strides[bk]);
+  p.sBn = static_cast<int32_t>(rhs->strides[bn]);
+  p.sCm = static_cast<int32_t>(out->strides[orank - 2]);
+  p.sCn = static_cast<int32_t>(out->strides[orank - 1]);
+  // batch dims: trailing alignment, size 1 -> stride 0, missing -> stride 0
+  LoopNest nest;
+  nest.n_operands = 3;
+  nest.rank = orank - 2;
+  for (int i = 0; i < orank - 2; ++i) {
+    nest.shape[i] = out->shape[i];
+    nest.strides[0][i] = out->strides[i];
+    const int li = lr - orank + i, ri = rr - orank + i;
+    if (li < 0) {
+      nest.strides[1][i] = 0;
+    } else if (lhs->shape[li] == out->shape[i]) {
+      nest.strides[1][i] = lhs->strides[li];
+    } else if (lhs->shape[li] == 1) {
+      nest.strides[1][i] = 0;
+    } else {
+      return FL_ERR_SHAPE;
+    }
+    if (ri < 0) {
+      nest.strides[2][i] = 0;
+    } else if (rhs->shape[ri] == out->shape[i]) {
+      nest.strides[2][i] = rhs->strides[ri];
+    } else if (rhs->shape[ri] == 1) {
+      nest.strides[2][i] = 0;
+    } else {
+      return FL_ERR_SHAPE;
+    }
+  }
+  nest.Canonicalise();
+  int64_t n_batch = 1;
+  for (int i = 0; i < nest.rank; ++i) n_batch *= nest.shape[i];
+  if (n_batch > 65535) return FL_ERR_TOO_LARGE;
+  p.batch = MakeNestArgs<3>(nest);
+  p.ca = ca;
+  p.cb = cb;
+  if (bias != nullptr) {
+    FL_CHECK(CheckView(bias));
+    if (bias->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+    if (bias->rank == 1) {
+      if (bias->shape[0] != p.N) return FL_ERR_SHAPE;
+      p.sDm = 0;
+      p.sDn = static_cast<int32_t>(bias->strides[0]);
+    } else if (bias->rank == 2) {
+      if (bias->shape[0] != p.M || bias->shape[1] != p.N) return FL_ERR_SHAPE;
+      p.sDm = static_cast<int32_t>(bias->strides[0]);
+      p.sDn = static_cast<int32_t>(bias->strides[1]);
+    } else {
+      return FL_ERR_RANK;
+    }
+    p.bias = static_cast<const float *>(bias->base);
+  }
+
+  float *C = static_cast<float *>(out->base);
+  const float *A = static_cast<const float *>(lhs->base);
+  const float *B = static_cast<const float *>(rhs->base);
+  hipStream_t s = AsStream(stream);
+
+  // Layout of each staged tile follows the operand's fast dimension; 128-bit
+  // loads need that dimension to have unit stride and everything else to keep
+  // 16-byte alignment.
+  const int la = (p.sAk <= p.sAm || p.M == 1) ? 0 : 1;
+  const int lb = (p.sBn <= p.sBk || p.K == 1) ? 0 : 1;
+  bool vec = IsAligned(A, 16) && IsAligned(B, 16);
+  if (la == 0) vec = vec && (p.sAk == 1 || p.K == 1) && p.K % 4 == 0 && p.sAm % 4 == 0;
+  else vec = vec && p.sAm == 1 && p.M % 4 == 0 && p.sAk % 4 == 0;
+  if (lb == 0) vec = vec && (p.sBn == 1 || p.N == 1) && p.N % 4 == 0 && p.sBk % 4 == 0;
+  else vec = vec && p.sBk == 1 && p.K % 4 == 0 && p.sBn % 4 == 0;
+  for (int i = 0; i < nest.rank && vec; ++i) {
+    if (nest.strides[1][i] % 4 != 0 || nest.strides[2][i] % 4 != 0) vec = false;
+  }
+  const uint32_t nb = static_cast<uint32_t>(n_batch);
+#define FL_MM_DISPATCH(LA_, LB_)                              \
+  if (la == LA_ && lb == LB_) {                               \
+    if (vec) LaunchBySize<LA_, LB_, 4>(p, nb, C, A, B, s);    \
+    else LaunchBySize<LA_, LB_, 1>(p, nb, C, A, B, s);        \
+  }
+  FL_MM_DISPATCH(0, 0)
+  FL_MM_DISPATCH(0, 1)
+  FL_MM_DISPATCH(1, 0)
+  FL_MM_DISPATCH(1, 1)
+#undef FL_MM_DISPATCH
+  return LaunchStatus();
+}
+
+}  // namespace
+}  // namespace fl
+
+extern "C" {
+
+int fluidml_hip_matmul(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
+  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 0.0f, nullptr, stream);
+}
+
+int fluidml_hip_matmul_bf16(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
+  (void)lhs;
+  (void)rhs;
+  (void)out;
+  (void)stream;
+  return FL_ERR_UNSUPPORTED;
+}
+
+int fluidml_hip_gemm_constant_weights_bias(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias,
+                                           const fl_tensor *out, double alpha, double beta, int32_t trans_a,
+                                           int32_t trans_b, uint32_t flags, void *stream) {
+  if (!lhs || !rhs || !bias || !out) return FL_ERR_NULL;
+  if (lhs->rank != 2 || rhs->rank != 2 || out->rank != 2) return FL_ERR_RANK;  // reference gemm.cpp:57-61
+  // acc = A.B; reference: alpha * bias + beta * acc (gemm.cpp:176-179); ONNX: alpha * acc + beta * bias
+  const bool swapped = (flags & FL_REF_GEMM_SWAPPED_SCALARS) != 0;
+  const float ca = static_cast<float>(swapped ? beta : alpha);
+  const float cb = static_cast<float>(swapped ? alpha : beta);
+  return fl::Contract(lhs, rhs, out, trans_a != 0, trans_b != 0, ca, cb, bias, stream);
+}
+
+}  // extern "C"

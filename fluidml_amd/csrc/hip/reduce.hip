@@ -1,0 +1,467 @@
+// Row-reduction kernels (HBM bound): Softmax, LayerNormalization, ReduceMean.
+//
+// The reference runs these as chains of linalg.generic passes over a scratch
+// tensor (softmax.cpp:22-139 six passes, layer_normalization.cpp:33-220 seven,
+// reduce_mean.cpp:16-98 three).  Here a row is read once, reduced in
+// registers with wave64 shuffles (LDS only to combine waves) and written once.
+//
+// Two traversal shapes cover every layout the planner can pick:
+//   * "row"    - the reduced axis is contiguous for input and output: one wave
+//                (or one block) per row, lanes stride the row;
+//   * "column" - the axis is strided: one lane per row, rows enumerated in the
+//                output's physical order so neighbouring lanes touch
+//                neighbouring addresses while each walks its axis.
+#include "fl_common.h"
+
+namespace fl {
+namespace {
+
+constexpr int kBlock = 256;
+
+template <int NOPS>
+struct RowArgs {
+  NestArgs<NOPS> outer;  // non-axis dims, canonical order (operand 0 = output)
+  uint32_t n_rows;
+  uint32_t len;
+  int32_t axis_stride[NOPS];
+};
+
+template <int NOPS>
+__device__ __forceinline__ void RowOffsets(const NestArgs<NOPS> &a, uint32_t row, int32_t *off) {
+#pragma unroll
+  for (int o = 0; o < NOPS; ++o) off[o] = 0;
+  uint32_t rem = row;
+  for (int d = a.rank - 1; d > 0; --d) {
+    uint32_t q, r;
+    a.div[d].DivMod(rem, q, r);
+    rem = q;
+#pragma unroll
+    for (int o = 0; o < NOPS; ++o) off[o] += static_cast<int32_t>(r) * a.strides[o][d];
+  }
+#pragma unroll
+  for (int o = 0; o < NOPS; ++o) off[o] += static_cast<int32_t>(rem) * a.strides[o][0];
+}
+
+// Build the outer nest (all dims but `axis`) for the given operands' strides.
+template <int NOPS>
+RowArgs<NOPS> MakeRowArgs(int rank, const int64_t *shape, int axis, const int64_t (*strides)[kMaxRank]) {
+  LoopNest nest;
+  nest.n_operands = NOPS;
+  nest.rank = 0;
+  for (int i = 0; i < rank; ++i) {
+    if (i == axis) continue;
+    nest.shape[nest.rank] = shape[i];
+    for (int o = 0; o < NOPS; ++o) nest.strides[o][nest.rank] = strides[o][i];
+    ++nest.rank;
+  }
+  nest.Canonicalise();
+  RowArgs<NOPS> args;
+  args.outer = MakeNestArgs<NOPS>(nest);
+  int64_t rows = 1;
+  for (int i = 0; i < nest.rank; ++i) rows *= nest.shape[i];
+  args.n_rows = static_cast<uint32_t>(rows);
+  args.len = static_cast<uint32_t>(shape[axis]);
+  for (int o = 0; o < NOPS; ++o) args.axis_stride[o] = static_cast<int32_t>(strides[o][axis]);
+  return args;
+}
+
+// ---- Softmax ----------------------------------------------------------------
+
+// One wave per row, row cached in registers: len <= 64 * ITEMS.
+template <int ITEMS>
+__global__ __launch_bounds__(kBlock) void SoftmaxRowWave(RowArgs<2> a, float *__restrict__ out,
+                                                         const float *__restrict__ in) {
+  const uint32_t lane = threadIdx.x % kWave;
+  const uint32_t row = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  if (row >= a.n_rows) return;
+  int32_t off[2];
+  RowOffsets<2>(a.outer, row, off);
+  const float *src = in + off[1];
+  float *dst = out + off[0];
+  float x[ITEMS];
+  float m = -__FLT_MAX__;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = lane + i * kWave;
+    x[i] = j < a.len ? src[j] : -__FLT_MAX__;
+    m = fmaxf(m, x[i]);
+  }
+  m = WaveReduce(m, MaxOp{});
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = lane + i * kWave;
+    x[i] = j < a.len ? expf(x[i] - m) : 0.0f;
+    s += x[i];
+  }
+  s = WaveReduce(s, SumOp{});
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = lane + i * kWave;
+    if (j < a.len) dst[j] = x[i] / s;
+  }
+}
+
+// One block per row, any length, three passes over the (cache-resident) row.
+__global__ __launch_bounds__(kBlock) void SoftmaxRowBlock(RowArgs<2> a, float *__restrict__ out,
+                                                          const float *__restrict__ in) {
+  __shared__ float smem[kBlock / kWave];
+  int32_t off[2];
+  RowOffsets<2>(a.outer, blockIdx.x, off);
+  const float *src = in + off[1];
+  float *dst = out + off[0];
+  float m = -__FLT_MAX__;
+  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) m = fmaxf(m, src[j]);
+  m = BlockReduce<kBlock / kWave>(m, MaxOp{}, smem);
+  float s = 0.0f;
+  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) s += expf(src[j] - m);
+  s = BlockReduce<kBlock / kWave>(s, SumOp{}, smem);
+  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) dst[j] = expf(src[j] - m) / s;
+}
+
+// One lane per row; the axis is walked with its stride.
+__global__ __launch_bounds__(kBlock) void SoftmaxColumn(RowArgs<2> a, float *__restrict__ out,
+                                                        const float *__restrict__ in) {
+  const uint32_t row = blockIdx.x * kBlock + threadIdx.x;
+  if (row >= a.n_rows) return;
+  int32_t off[2];
+  RowOffsets<2>(a.outer, row, off);
+  const float *src = in + off[1];
+  float *dst = out + off[0];
+  const int32_t si = a.axis_stride[1], so = a.axis_stride[0];
+  float m = -__FLT_MAX__;
+  for (uint32_t j = 0; j < a.len; ++j) m = fmaxf(m, src[static_cast<int32_t>(j) * si]);
+  float s = 0.0f;
+  for (uint32_t j = 0; j < a.len; ++j) s += expf(src[static_cast<int32_t>(j) * si] - m);
+  for (uint32_t j = 0; j < a.len; ++j) dst[static_cast<int32_t>(j) * so] = expf(src[static_cast<int32_t>(j) * si] - m) / s;
+}
+
+// ---- LayerNormalization -------------------------------------------------------
+
+// operands: 0 out, 1 in, 2 scale, 3 bias, 4 scratch (one float per row)
+template <int ITEMS>
+__global__ __launch_bounds__(kBlock) void LayerNormRowBlock(RowArgs<5> a, float *__restrict__ out,
+                                                            const float *__restrict__ in,
+                                                            const float *__restrict__ scale,
+                                                            const float *__restrict__ bias,
+                                                            const float *__restrict__ scratch, float eps,
+                                                            int stale_scratch) {
+  __shared__ float smem[kBlock / kWave];
+  int32_t off[5];
+  RowOffsets<5>(a.outer, blockIdx.x, off);
+  const float *src = in + off[1];
+  const float n = static_cast<float>(a.len);
+  float x[ITEMS];
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = threadIdx.x + i * kBlock;
+    x[i] = j < a.len ? src[j] : 0.0f;
+    s += x[i];
+  }
+  s = BlockReduce<kBlock / kWave>(s, SumOp{}, smem);
+  if (stale_scratch) s += scratch[off[4]];
+  const float mean = s / n;
+  float v = 0.0f;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = threadIdx.x + i * kBlock;
+    x[i] = j < a.len ? x[i] - mean : 0.0f;
+    v += x[i] * x[i];
+  }
+  v = BlockReduce<kBlock / kWave>(v, SumOp{}, smem);
+  const float inv = 1.0f / sqrtf(v / n + eps);
+  float *dst = out + off[0];
+  const float *g = scale + off[2];
+  const float *b = bias + off[3];
+  const int32_t sg = a.axis_stride[2], sb = a.axis_stride[3];
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = threadIdx.x + i * kBlock;
+    if (j < a.len) dst[j] = (x[i] * inv) * g[static_cast<int32_t>(j) * sg] + b[static_cast<int32_t>(j) * sb];
+  }
+}
+
+// Any length / any axis stride: lanes of a block stride the row three times.
+__global__ __launch_bounds__(kBlock) void LayerNormRowLoop(RowArgs<5> a, float *__restrict__ out,
+                                                           const float *__restrict__ in,
+                                                           const float *__restrict__ scale,
+                                                           const float *__restrict__ bias,
+                                                           const float *__restrict__ scratch, float eps,
+                                                           int stale_scratch) {
+  __shared__ float smem[kBlock / kWave];
+  int32_t off[5];
+  RowOffsets<5>(a.outer, blockIdx.x, off);
+  const float *src = in + off[1];
+  const int32_t si = a.axis_stride[1], so = a.axis_stride[0], sg = a.axis_stride[2], sb = a.axis_stride[3];
+  const float n = static_cast<float>(a.len);
+  float s = 0.0f;
+  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) s += src[static_cast<int32_t>(j) * si];
+  s = BlockReduce<kBlock / kWave>(s, SumOp{}, smem);
+  if (stale_scratch) s += scratch[off[4]];
+  const float mean = s / n;
+  float v = 0.0f;
+  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) {
+    const float d = src[static_cast<int32_t>(j) * si] - mean;
+    v += d * d;
+  }
+  v = BlockReduce<kBlock / kWave>(v, SumOp{}, smem);
+  const float inv = 1.0f / sqrtf(v / n + eps);
+  float *dst = out + off[0];
+  const float *g = scale + off[2];
+  const float *b = bias + off[3];
+  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) {
+    const int32_t jj = static_cast<int32_t>(j);
+    dst[jj * so] = ((src[jj * si] - mean) * inv) * g[jj * sg] + b[jj * sb];
+  }
+}
+
+// One lane per row (strided axis, many rows).
+__global__ __launch_bounds__(kBlock) void LayerNormColumn(RowArgs<5> a, float *__restrict__ out,
+                                                          const float *__restrict__ in,
+                                                          const float *__restrict__ scale,
+                                                          const float *__restrict__ bias,
+                                                          const float *__restrict__ scratch, float eps,
+                                                          int stale_scratch) {
+  const uint32_t row = blockIdx.x * kBlock + threadIdx.x;
+  if (row >= a.n_rows) return;
+  int32_t off[5];
+  RowOffsets<5>(a.outer, row, off);
+  const float *src = in + off[1];
+  const int32_t si = a.axis_stride[1], so = a.axis_stride[0], sg = a.axis_stride[2], sb = a.axis_stride[3];
+  const float n = static_cast<float>(a.len);
+  float s = stale_scratch ? scratch[off[4]] : 0.0f;
+  for (uint32_t j = 0; j < a.len; ++j) s += src[static_cast<int32_t>(j) * si];
+  const float mean = s / n;
+  float v = 0.0f;
+  for (uint32_t j = 0; j < a.len; ++j) {
+    const float d = src[static_cast<int32_t>(j) * si] - mean;
+    v += d * d;
+  }
+  const float inv = 1.0f / sqrtf(v / n + eps);
+  float *dst = out + off[0];
+  const float *g = scale + off[2];
+  const float *b = bias + off[3];
+  for (uint32_t j = 0; j < a.len; ++j) {
+    const int32_t jj = static_cast<int32_t>(j);
+    dst[jj * so] = ((src[jj * si] - mean) * inv) * g[jj * sg] + b[jj * sb];
+  }
+}
+
+// ---- ReduceMean ---------------------------------------------------------------
+
+struct ReduceArgs {
+  NestArgs<2> outer;   // kept dims: operand 0 = output, 1 = input
+  NestArgs<1> inner;   // reduced dims of the input
+  uint32_t n_out;
+  uint32_t n_red;
+  float divisor;
+};
+
+__device__ __forceinline__ int32_t InnerOffset(const NestArgs<1> &a, uint32_t idx) {
+  int32_t off = 0;
+  uint32_t rem = idx;
+  for (int d = a.rank - 1; d > 0; --d) {
+    uint32_t q, r;
+    a.div[d].DivMod(rem, q, r);
+    rem = q;
+    off += static_cast<int32_t>(r) * a.strides[0][d];
+  }
+  return off + static_cast<int32_t>(rem) * a.strides[0][0];
+}
+
+// One wave per output element.
+__global__ __launch_bounds__(kBlock) void ReduceMeanWave(ReduceArgs a, float *__restrict__ out,
+                                                         const float *__restrict__ in) {
+  const uint32_t lane = threadIdx.x % kWave;
+  const uint32_t o = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  if (o >= a.n_out) return;
+  int32_t off[2];
+  RowOffsets<2>(a.outer, o, off);
+  const float *src = in + off[1];
+  float s = 0.0f;
+  for (uint32_t j = lane; j < a.n_red; j += kWave) s += src[InnerOffset(a.inner, j)];
+  s = WaveReduce(s, SumOp{});
+  if (lane == 0) out[off[0]] = s / a.divisor;
+}
+
+// One lane per output element.
+__global__ __launch_bounds__(kBlock) void ReduceMeanThread(ReduceArgs a, float *__restrict__ out,
+                                                           const float *__restrict__ in) {
+  const uint32_t o = blockIdx.x * kBlock + threadIdx.x;
+  if (o >= a.n_out) return;
+  int32_t off[2];
+  RowOffsets<2>(a.outer, o, off);
+  const float *src = in + off[1];
+  float s = 0.0f;
+  for (uint32_t j = 0; j < a.n_red; ++j) s += src[InnerOffset(a.inner, j)];
+  out[off[0]] = s / a.divisor;
+}
+
+}  // namespace
+}  // namespace fl
+
+using namespace fl;
+
+extern "C" {
+
+int fluidml_hip_softmax(const fl_tensor *in, const fl_tensor *out, void *scratch, size_t scratch_bytes, int64_t axis,
+                        void *stream) {
+  (void)scratch;
+  (void)scratch_bytes;
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (in->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  if (!SameShape(in, out)) return FL_ERR_SHAPE;
+  if (axis < 0 || axis >= in->rank) return FL_ERR_ATTR;  // reference normalises before the kernel
+  int64_t strides[2][kMaxRank];
+  for (int i = 0; i < in->rank; ++i) {
+    strides[0][i] = out->strides[i];
+    strides[1][i] = in->strides[i];
+  }
+  RowArgs<2> a = MakeRowArgs<2>(in->rank, in->shape, static_cast<int>(axis), strides);
+  float *o = static_cast<float *>(out->base);
+  const float *x = static_cast<const float *>(in->base);
+  hipStream_t s = AsStream(stream);
+  const bool row_contig = (a.axis_stride[0] == 1 && a.axis_stride[1] == 1) || a.len == 1;
+  if (row_contig && a.len > 16) {
+    const uint32_t wave_blocks = (a.n_rows + kBlock / kWave - 1) / (kBlock / kWave);
+    if (a.len <= 64) {
+      hipLaunchKernelGGL(SoftmaxRowWave<1>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x);
+    } else if (a.len <= 128) {
+      hipLaunchKernelGGL(SoftmaxRowWave<2>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x);
+    } else if (a.len <= 256) {
+      hipLaunchKernelGGL(SoftmaxRowWave<4>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x);
+    } else if (a.len <= 512) {
+      hipLaunchKernelGGL(SoftmaxRowWave<8>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x);
+    } else if (a.len <= 1024) {
+      hipLaunchKernelGGL(SoftmaxRowWave<16>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x);
+    } else {
+      hipLaunchKernelGGL(SoftmaxRowBlock, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x);
+    }
+  } else {
+    hipLaunchKernelGGL(SoftmaxColumn, dim3((a.n_rows + kBlock - 1) / kBlock), dim3(kBlock), 0, s, a, o, x);
+  }
+  return LaunchStatus();
+}
+
+int fluidml_hip_layer_normalization_constant_scale_bias(const fl_tensor *in, const fl_tensor *scale,
+                                                        const fl_tensor *bias, const fl_tensor *out, void *scratch,
+                                                        size_t scratch_bytes, int64_t axis, double epsilon,
+                                                        uint32_t flags, void *stream) {
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(scale));
+  FL_CHECK(CheckView(bias));
+  FL_CHECK(CheckView(out));
+  if (in->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32 || scale->dtype != FL_FLOAT32 || bias->dtype != FL_FLOAT32)
+    return FL_ERR_DTYPE;
+  if (!SameShape(in, out)) return FL_ERR_SHAPE;
+  if (axis < 0) axis += in->rank;  // reference flow/node.cpp:931-933
+  if (axis < 0 || axis >= in->rank) return FL_ERR_ATTR;
+  const int stale = (flags & FL_REF_LN_STALE_SCRATCH) ? 1 : 0;
+  int64_t strides[5][kMaxRank];
+  FL_CHECK(BroadcastStrides(scale, in->rank, in->shape, strides[2]));
+  FL_CHECK(BroadcastStrides(bias, in->rank, in->shape, strides[3]));
+  // scratch: dense row-major tensor of the input shape with axis -> 1
+  int64_t acc = 1, rows = 1;
+  for (int i = in->rank - 1; i >= 0; --i) {
+    strides[0][i] = out->strides[i];
+    strides[1][i] = in->strides[i];
+    if (i == axis) {
+      strides[4][i] = 0;
+    } else {
+      strides[4][i] = acc;
+      acc *= in->shape[i];
+      rows *= in->shape[i];
+    }
+  }
+  if (stale) {
+    if (scratch == nullptr) return FL_ERR_NULL;
+    if (scratch_bytes < static_cast<size_t>(rows) * sizeof(float)) return FL_ERR_SCRATCH;
+  }
+  RowArgs<5> a = MakeRowArgs<5>(in->rank, in->shape, static_cast<int>(axis), strides);
+  float *o = static_cast<float *>(out->base);
+  const float *x = static_cast<const float *>(in->base);
+  const float *g = static_cast<const float *>(scale->base);
+  const float *b = static_cast<const float *>(bias->base);
+  const float *sc = static_cast<const float *>(scratch);
+  const float eps = static_cast<float>(epsilon);
+  hipStream_t s = AsStream(stream);
+  const bool row_contig = a.axis_stride[0] == 1 && a.axis_stride[1] == 1;
+  if (row_contig && a.len > 64) {
+    if (a.len <= kBlock) {
+      hipLaunchKernelGGL(LayerNormRowBlock<1>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+    } else if (a.len <= 2 * kBlock) {
+      hipLaunchKernelGGL(LayerNormRowBlock<2>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+    } else if (a.len <= 4 * kBlock) {
+      hipLaunchKernelGGL(LayerNormRowBlock<4>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+    } else if (a.len <= 8 * kBlock) {
+      hipLaunchKernelGGL(LayerNormRowBlock<8>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+    } else {
+      hipLaunchKernelGGL(LayerNormRowLoop, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+    }
+  } else if (a.n_rows >= 4096 || a.len <= 64) {
+    hipLaunchKernelGGL(LayerNormColumn, dim3((a.n_rows + kBlock - 1) / kBlock), dim3(kBlock), 0, s, a, o, x, g, b, sc,
+                       eps, stale);
+  } else {
+    hipLaunchKernelGGL(LayerNormRowLoop, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+  }
+  return LaunchStatus();
+}
+
+int fluidml_hip_reduce_mean(const fl_tensor *in, const fl_tensor *out, const int64_t *axes, int32_t n_axes,
+                            void *stream) {
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (in->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  if (in->rank != out->rank) return FL_ERR_UNSUPPORTED;  // keepdims=0: unreachable in reference reduce_mean.cpp:56-62
+  if (n_axes < 0 || (n_axes > 0 && axes == nullptr)) return FL_ERR_ATTR;
+  bool reduced[kMaxRank] = {};
+  for (int k = 0; k < n_axes; ++k) {
+    if (axes[k] < 0 || axes[k] >= in->rank) return FL_ERR_ATTR;
+    reduced[axes[k]] = true;
+  }
+  LoopNest outer, inner;
+  outer.n_operands = 2;
+  inner.n_operands = 1;
+  int64_t divisor = 1;
+  for (int i = 0; i < in->rank; ++i) {
+    if (reduced[i]) {
+      if (out->shape[i] != 1) return FL_ERR_SHAPE;
+      divisor *= in->shape[i];
+      inner.shape[inner.rank] = in->shape[i];
+      inner.strides[0][inner.rank] = in->strides[i];
+      ++inner.rank;
+    } else {
+      if (out->shape[i] != in->shape[i]) return FL_ERR_SHAPE;
+      outer.shape[outer.rank] = in->shape[i];
+      outer.strides[0][outer.rank] = out->strides[i];
+      outer.strides[1][outer.rank] = in->strides[i];
+      ++outer.rank;
+    }
+  }
+  outer.Canonicalise();
+  inner.Canonicalise();
+  ReduceArgs a;
+  a.outer = MakeNestArgs<2>(outer);
+  a.inner = MakeNestArgs<1>(inner);
+  int64_t n_out = 1, n_red = 1;
+  for (int i = 0; i < outer.rank; ++i) n_out *= outer.shape[i];
+  for (int i = 0; i < inner.rank; ++i) n_red *= inner.shape[i];
+  a.n_out = static_cast<uint32_t>(n_out);
+  a.n_red = static_cast<uint32_t>(n_red);
+  a.divisor = static_cast<float>(divisor);
+  float *o = static_cast<float *>(out->base);
+  const float *x = static_cast<const float *>(in->base);
+  hipStream_t s = AsStream(stream);
+  const bool inner_contig = inner.strides[0][inner.rank - 1] == 1;
+  if ((inner_contig && n_red >= 32) || n_out < 1024) {
+    hipLaunchKernelGGL(ReduceMeanWave, dim3((a.n_out + kBlock / kWave - 1) / (kBlock / kWave)), dim3(kBlock), 0, s, a, o,
+                       x);
+  } else {
+    hipLaunchKernelGGL(ReduceMeanThread, dim3((a.n_out + kBlock - 1) / kBlock), dim3(kBlock), 0, s, a, o, x);
+  }
+  return LaunchStatus();
+}
+
+}  // extern "C"

@@ -1,0 +1,222 @@
+// Device plumbing behind the C ABI: arena, constants, copies, streams, events
+// and launch-plan capture.  It replaces what the reference gets from
+// mlir::ExecutionEngine and a per-call host vector (src/worker/runner.cpp:56-120,
+// src/structure/context/context.cpp:152-166).
+#include "fl_common.h"
+
+using namespace fl;
+
+namespace {
+
+// hipMemsetAsync nodes inside captured graphs have replayed wrongly on some
+// ROCm stacks; zeroing is therefore a plain fill kernel, safe to capture.
+__global__ __launch_bounds__(256) void FillZero(uint32_t *p, size_t n_words, uint8_t *tail, size_t n_tail) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < n_words; i += stride) p[i] = 0u;
+  if (blockIdx.x == 0 && threadIdx.x < n_tail) tail[threadIdx.x] = 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fluidml_hip_abi_version(void) { return 1; }
+
+const char *fluidml_hip_error_string(int code) {
+  switch (code) {
+    case FL_OK: return "ok";
+    case FL_ERR_NULL: return "null pointer argument";
+    case FL_ERR_RANK: return "rank out of range or ranks inconsistent";
+    case FL_ERR_SHAPE: return "shapes do not satisfy the kernel's contract";
+    case FL_ERR_DTYPE: return "unsupported element type combination";
+    case FL_ERR_ATTR: return "attribute out of range";
+    case FL_ERR_TOO_LARGE: return "view larger than 2^31-1 elements";
+    case FL_ERR_SCRATCH: return "scratch buffer too small";
+    case FL_ERR_UNSUPPORTED: return "not supported by this backend";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+  return "unknown error";
+}
+
+int fluidml_hip_device_count(void) {
+  int n = 0;
+  hipError_t err = hipGetDeviceCount(&n);
+  if (err != hipSuccess) return -static_cast<int>(err) - 1000;
+  return n;
+}
+
+int fluidml_hip_device_info(int dev, char *name, size_t name_len, char *arch, size_t arch_len, int *compute_units,
+                            size_t *total_mem) {
+  hipDeviceProp_t prop;
+  FL_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+  if (name && name_len) {
+    std::strncpy(name, prop.name, name_len - 1);
+    name[name_len - 1] = '\0';
+  }
+  if (arch && arch_len) {
+    std::strncpy(arch, prop.gcnArchName, arch_len - 1);
+    arch[arch_len - 1] = '\0';
+  }
+  if (compute_units) *compute_units = prop.multiProcessorCount;
+  if (total_mem) *total_mem = prop.totalGlobalMem;
+  return FL_OK;
+}
+
+int fluidml_hip_arena_create(size_t bytes, void **arena) {
+  if (arena == nullptr) return FL_ERR_NULL;
+  *arena = nullptr;
+  // keep a valid pointer for an empty plan; round up so 128-bit accesses near
+  // the end of the last tensor stay inside the allocation
+  const size_t alloc = ((bytes + 255) / 256 + 1) * 256;
+  void *p = nullptr;
+  FL_HIP_CHECK(hipMalloc(&p, alloc));
+  hipError_t err = hipMemset(p, 0, alloc);
+  if (err != hipSuccess) {
+    (void)hipFree(p);
+    return static_cast<int>(err);
+  }
+  *arena = p;
+  return FL_OK;
+}
+
+int fluidml_hip_arena_destroy(void *arena) {
+  if (arena == nullptr) return FL_OK;
+  FL_HIP_CHECK(hipFree(arena));
+  return FL_OK;
+}
+
+int fluidml_hip_arena_zero(void *arena, size_t bytes, void *stream) {
+  if (arena == nullptr) return FL_ERR_NULL;
+  if (bytes == 0) return FL_OK;
+  const size_t n_words = bytes / 4, n_tail = bytes % 4;
+  const size_t blocks = std::min<size_t>((n_words + 255) / 256 + 1, 4096);
+  hipLaunchKernelGGL(FillZero, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, AsStream(stream),
+                     static_cast<uint32_t *>(arena), n_words, static_cast<uint8_t *>(arena) + n_words * 4, n_tail);
+  return LaunchStatus();
+}
+
+int fluidml_hip_upload_constant(const void *host, size_t bytes, void **device) {
+  if (device == nullptr || (host == nullptr && bytes > 0)) return FL_ERR_NULL;
+  *device = nullptr;
+  const size_t alloc = ((bytes + 255) / 256 + 1) * 256;
+  void *p = nullptr;
+  FL_HIP_CHECK(hipMalloc(&p, alloc));
+  if (bytes > 0) {
+    hipError_t err = hipMemcpy(p, host, bytes, hipMemcpyHostToDevice);
+    if (err != hipSuccess) {
+      (void)hipFree(p);
+      return static_cast<int>(err);
+    }
+  }
+  *device = p;
+  return FL_OK;
+}
+
+int fluidml_hip_free(void *device) {
+  if (device == nullptr) return FL_OK;
+  FL_HIP_CHECK(hipFree(device));
+  return FL_OK;
+}
+
+int fluidml_hip_memcpy_h2d(void *device, const void *host, size_t bytes, void *stream) {
+  if (bytes == 0) return FL_OK;
+  if (device == nullptr || host == nullptr) return FL_ERR_NULL;
+  FL_HIP_CHECK(hipMemcpyAsync(device, host, bytes, hipMemcpyHostToDevice, AsStream(stream)));
+  return FL_OK;
+}
+
+int fluidml_hip_memcpy_d2h(void *host, const void *device, size_t bytes, void *stream) {
+  if (bytes == 0) return FL_OK;
+  if (device == nullptr || host == nullptr) return FL_ERR_NULL;
+  FL_HIP_CHECK(hipMemcpyAsync(host, device, bytes, hipMemcpyDeviceToHost, AsStream(stream)));
+  return FL_OK;
+}
+
+int fluidml_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes == 0) return FL_OK;
+  if (dst == nullptr || src == nullptr) return FL_ERR_NULL;
+  FL_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, AsStream(stream)));
+  return FL_OK;
+}
+
+int fluidml_hip_stream_create(void **stream) {
+  if (stream == nullptr) return FL_ERR_NULL;
+  hipStream_t s = nullptr;
+  FL_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream = s;
+  return FL_OK;
+}
+
+int fluidml_hip_stream_destroy(void *stream) {
+  if (stream == nullptr) return FL_OK;
+  FL_HIP_CHECK(hipStreamDestroy(AsStream(stream)));
+  return FL_OK;
+}
+
+int fluidml_hip_stream_synchronize(void *stream) {
+  FL_HIP_CHECK(hipStreamSynchronize(AsStream(stream)));
+  return FL_OK;
+}
+
+int fluidml_hip_event_create(void **event) {
+  if (event == nullptr) return FL_ERR_NULL;
+  hipEvent_t e = nullptr;
+  FL_HIP_CHECK(hipEventCreate(&e));
+  *event = e;
+  return FL_OK;
+}
+
+int fluidml_hip_event_destroy(void *event) {
+  if (event == nullptr) return FL_OK;
+  FL_HIP_CHECK(hipEventDestroy(static_cast<hipEvent_t>(event)));
+  return FL_OK;
+}
+
+int fluidml_hip_event_record(void *event, void *stream) {
+  if (event == nullptr) return FL_ERR_NULL;
+  FL_HIP_CHECK(hipEventRecord(static_cast<hipEvent_t>(event), AsStream(stream)));
+  return FL_OK;
+}
+
+int fluidml_hip_event_elapsed_ns(void *start, void *stop, double *ns) {
+  if (start == nullptr || stop == nullptr || ns == nullptr) return FL_ERR_NULL;
+  FL_HIP_CHECK(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+  float ms = 0.0f;
+  FL_HIP_CHECK(hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  *ns = static_cast<double>(ms) * 1.0e6;
+  return FL_OK;
+}
+
+int fluidml_hip_graph_begin_capture(void *stream) {
+  if (stream == nullptr) return FL_ERR_NULL;  // the null stream cannot be captured
+  FL_HIP_CHECK(hipStreamBeginCapture(AsStream(stream), hipStreamCaptureModeThreadLocal));
+  return FL_OK;
+}
+
+int fluidml_hip_graph_end_capture(void *stream, void **graph_exec) {
+  if (stream == nullptr || graph_exec == nullptr) return FL_ERR_NULL;
+  *graph_exec = nullptr;
+  hipGraph_t graph = nullptr;
+  FL_HIP_CHECK(hipStreamEndCapture(AsStream(stream), &graph));
+  hipGraphExec_t exec = nullptr;
+  hipError_t err = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (err != hipSuccess) return static_cast<int>(err);
+  *graph_exec = exec;
+  return FL_OK;
+}
+
+int fluidml_hip_graph_launch(void *graph_exec, void *stream) {
+  if (graph_exec == nullptr) return FL_ERR_NULL;
+  FL_HIP_CHECK(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), AsStream(stream)));
+  return FL_OK;
+}
+
+int fluidml_hip_graph_destroy(void *graph_exec) {
+  if (graph_exec == nullptr) return FL_OK;
+  FL_HIP_CHECK(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
+  return FL_OK;
+}
+
+}  // extern "C"

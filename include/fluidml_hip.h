@@ -1,0 +1,277 @@
+/*
+ * fluidml_hip.h -- C ABI of the MI355X (gfx950) execution backend for FluidML.
+ *
+ * One entry point per FluidML kernel class (the strings returned by
+ * `GetKernelName()`, reference include/structure/kernel/kernel/ *.h).  Where the
+ * reference kernel's `Run(mlir::OpBuilder&, mlir::Value&...)` *emits* a
+ * linalg.generic over strided memrefs, the entry point here *launches* a HIP
+ * kernel over strided device views.  An `fl_tensor` carries exactly what the
+ * reference kernels read from a `mlir::MemRefType`: element type, shape and
+ * element strides (reference src/worker/builder.cpp:234-270 builds those
+ * memrefs from the region's layout).
+ *
+ * Conventions
+ *   - every pointer inside an fl_tensor is a DEVICE pointer to logical element
+ *     (0,...,0); strides are in elements and may describe any permutation
+ *     layout produced by utils::GenStrides (reference src/utils/utils.cpp:85-102);
+ *   - `stream` is a hipStream_t passed as void*; NULL = the null stream;
+ *   - every call is asynchronous on `stream` and returns 0 on success, a
+ *     negative FL_ERR_* code for a rejected argument (nothing is launched) or a
+ *     positive hipError_t from the runtime;
+ *   - `scratch` is the node's buffer of the memory plan (reference
+ *     flow::Node::GetBufferSize, src/structure/flow/node.cpp:500-519, 972-985,
+ *     1355-1368).  The plan keeps those bytes so offsets stay identical to the
+ *     reference; kernels that do not need them ignore the pointer;
+ *   - `flags` selects literal reproduction of reference behaviours that differ
+ *     from ONNX semantics (FL_REF_* below). 0 = ONNX semantics.
+ *
+ * No torch types, no C++ types: this header compiles as C.
+ */
+#ifndef FLUIDML_HIP_H_
+#define FLUIDML_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FL_MAX_RANK 8
+
+/* Element types; numbering follows `enum class Type` (reference
+ * include/utils/type.h:11-19) so a host `Type` casts straight through. */
+enum fl_dtype {
+  FL_UNKNOWN = 0,
+  FL_BOOL = 1, /* 1 byte, values 0/1 (sizeof(bool), reference src/utils/type.cpp:45) */
+  FL_INT32 = 2,
+  FL_INT64 = 3,
+  FL_FLOAT16 = 4, /* carried, never computed on */
+  FL_FLOAT32 = 5,
+  FL_FLOAT64 = 6
+};
+
+enum fl_error {
+  FL_OK = 0,
+  FL_ERR_NULL = -1,        /* a required pointer is NULL */
+  FL_ERR_RANK = -2,        /* rank outside [0, FL_MAX_RANK] or ranks inconsistent */
+  FL_ERR_SHAPE = -3,       /* shapes do not satisfy the kernel's contract */
+  FL_ERR_DTYPE = -4,       /* element type combination the reference leaves unreachable */
+  FL_ERR_ATTR = -5,        /* attribute out of range (axis, pads, strides, ...) */
+  FL_ERR_TOO_LARGE = -6,   /* more than 2^31-1 elements or offsets in one view */
+  FL_ERR_SCRATCH = -7,     /* scratch smaller than the kernel needs */
+  FL_ERR_UNSUPPORTED = -8  /* legal in ONNX, unreachable in the reference, not built */
+};
+
+/* Literal-reference switches (each cites the reference lines it reproduces). */
+enum fl_ref_flags {
+  /* Conv reads input at o+k: `strides`/`dilations` never applied
+   * (reference src/structure/kernel/kernel/conv.cpp:71,118). */
+  FL_REF_CONV_UNIT_STRIDE = 1 << 0,
+  /* Conv adds bias[1] to every output element (affine map is the constant 1,
+   * reference conv.cpp:181-182). */
+  FL_REF_CONV_BIAS_INDEX1 = 1 << 1,
+  /* LayerNormalization accumulates the row sum on top of whatever the scratch
+   * holds (first FillOp comes after the mean pass, reference
+   * layer_normalization.cpp:126 vs :165). */
+  FL_REF_LN_STALE_SCRATCH = 1 << 2,
+  /* Gemm computes alpha*bias + beta*(A.B) (reference gemm.cpp:176-179);
+   * without the flag: alpha*(A.B) + beta*bias as ONNX defines it. */
+  FL_REF_GEMM_SWAPPED_SCALARS = 1 << 3,
+  /* GatherConstantIndexScalar compares against the un-normalised axis
+   * (reference gather.cpp:116). */
+  FL_REF_GATHER_RAW_AXIS = 1 << 4
+};
+
+typedef struct fl_tensor {
+  void *base;
+  int32_t dtype; /* enum fl_dtype */
+  int32_t rank;
+  int64_t shape[FL_MAX_RANK];
+  int64_t strides[FL_MAX_RANK]; /* in elements */
+} fl_tensor;
+
+/* ------------------------------------------------------------------------- */
+/* Library / device plumbing (replaces the MLIR ExecutionEngine + the per-call
+ * host arena of reference src/worker/runner.cpp:56-120).                     */
+
+/* Version of this ABI; bumped on any signature change. */
+int fluidml_hip_abi_version(void);
+/* Human-readable text for a return code of this library (static storage). */
+const char *fluidml_hip_error_string(int code);
+/* Number of visible devices, or a negative/positive error code. */
+int fluidml_hip_device_count(void);
+/* Name and arch of device `dev` into caller buffers (NUL-terminated). */
+int fluidml_hip_device_info(int dev, char *name, size_t name_len, char *arch,
+                            size_t arch_len, int *compute_units,
+                            size_t *total_mem);
+
+/* One HBM arena of `bytes` bytes (reference runner.cpp:87-96 allocates
+ * `FuncAttr::GetBuffer()` zeroed host bytes per Invoke; here it is allocated
+ * once, zero-filled once, and lives until destroy). */
+int fluidml_hip_arena_create(size_t bytes, void **arena);
+int fluidml_hip_arena_destroy(void *arena);
+int fluidml_hip_arena_zero(void *arena, size_t bytes, void *stream);
+/* Constants (reference builder.cpp:273-361 embeds them as memref.global):
+ * allocate device memory and copy `bytes` host bytes into it. */
+int fluidml_hip_upload_constant(const void *host, size_t bytes, void **device);
+int fluidml_hip_free(void *device);
+int fluidml_hip_memcpy_h2d(void *device, const void *host, size_t bytes, void *stream);
+int fluidml_hip_memcpy_d2h(void *host, const void *device, size_t bytes, void *stream);
+int fluidml_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
+int fluidml_hip_stream_create(void **stream);
+int fluidml_hip_stream_destroy(void *stream);
+int fluidml_hip_stream_synchronize(void *stream);
+/* Event pair timing used by KernelEval::GetTimeCost (reference
+ * src/evaluation/eval.cpp:64-100 times one JIT run with the host clock). */
+int fluidml_hip_event_create(void **event);
+int fluidml_hip_event_destroy(void *event);
+int fluidml_hip_event_record(void *event, void *stream);
+int fluidml_hip_event_elapsed_ns(void *start, void *stop, double *ns);
+/* Launch-plan capture: the node sequence of one Invoke recorded once and
+ * replayed (the counterpart of re-running `_mlir_ciface_<name>`,
+ * reference runner.cpp:101-109). */
+int fluidml_hip_graph_begin_capture(void *stream);
+int fluidml_hip_graph_end_capture(void *stream, void **graph_exec);
+int fluidml_hip_graph_launch(void *graph_exec, void *stream);
+int fluidml_hip_graph_destroy(void *graph_exec);
+
+/* ------------------------------------------------------------------------- */
+/* a.3 Elementwise kernels (HBM bound).                                       */
+/* Scalar operands arrive as double, as the reference stores them
+ * (`float64_t value_`, include/structure/flow/node.h:147-165), and are cast to
+ * the tensor's element type inside the call.                                 */
+
+/* AddConstantKernel: out = in + value; int32/int64/float32
+ * (reference add.cpp:22-79). */
+int fluidml_hip_add_constant(const fl_tensor *in, const fl_tensor *out, double value, void *stream);
+/* AddCommonKernel: out = lhs + rhs with trailing-aligned broadcast
+ * (reference add.cpp:83-125, utils.cpp:16-52). */
+int fluidml_hip_add_common(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream);
+/* SubConstantLhsKernel: out = value - in (reference sub.cpp:16-67). */
+int fluidml_hip_sub_constant_lhs(const fl_tensor *in, const fl_tensor *out, double value, void *stream);
+/* SubCommonKernel (reference sub.cpp:71-99). */
+int fluidml_hip_sub_common(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream);
+/* MulConstantKernel: out = in * value, float32 (reference mul.cpp:19-54). */
+int fluidml_hip_mul_constant(const fl_tensor *in, const fl_tensor *out, double value, void *stream);
+/* MulCommonKernel: integer or float (reference mul.cpp:56-99). */
+int fluidml_hip_mul_common(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream);
+/* DivConstantRhsKernel: out = in / value, true division (reference div.cpp:18-66). */
+int fluidml_hip_div_constant_rhs(const fl_tensor *in, const fl_tensor *out, double value, void *stream);
+/* DivCommonKernel (reference div.cpp:70-105). */
+int fluidml_hip_div_common(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream);
+/* PowKernel: out = powf(in, exponent) (reference pow.cpp:15-61). */
+int fluidml_hip_pow(const fl_tensor *in, const fl_tensor *out, double exponent, void *stream);
+/* ErfKernel (reference erf.cpp:18-45). */
+int fluidml_hip_erf(const fl_tensor *in, const fl_tensor *out, void *stream);
+/* ReluKernel (reference relu.cpp:12-46). */
+int fluidml_hip_relu(const fl_tensor *in, const fl_tensor *out, void *stream);
+/* ClipKernel: min(max(x, lo), hi) (reference clip.cpp:13-48). */
+int fluidml_hip_clip(const fl_tensor *in, const fl_tensor *out, float lo, float hi, void *stream);
+/* TanhKernel (reference tanh.cpp:12-40). */
+int fluidml_hip_tanh(const fl_tensor *in, const fl_tensor *out, void *stream);
+/* SqrtKernel (reference sqrt.cpp:13-36). */
+int fluidml_hip_sqrt(const fl_tensor *in, const fl_tensor *out, void *stream);
+/* NegKernel (reference neg.cpp:17-40). */
+int fluidml_hip_neg(const fl_tensor *in, const fl_tensor *out, void *stream);
+/* NotKernel: bool xor 1 (reference not.cpp:11-41). */
+int fluidml_hip_not(const fl_tensor *in, const fl_tensor *out, void *stream);
+/* CastKernel: integer<->integer; bool zero-extends (reference cast.cpp:12-63). */
+int fluidml_hip_cast(const fl_tensor *in, const fl_tensor *out, void *stream);
+/* EqualKernel: int64 == value -> bool (reference equal.cpp:14-51). */
+int fluidml_hip_equal(const fl_tensor *in, const fl_tensor *out, double value, void *stream);
+/* DropoutKernel: identity copy (reference dropout.cpp:13-33). */
+int fluidml_hip_dropout(const fl_tensor *in, const fl_tensor *out, void *stream);
+/* WhereConstantCondConstantScalarYKernel: out = cond ? x : y
+ * (reference where.cpp:30-80); cond is a bool tensor broadcast to out. */
+int fluidml_hip_where_constant_cond_constant_scalar_y(const fl_tensor *cond, const fl_tensor *x, const fl_tensor *out, double y, void *stream);
+/* WhereConstantCondConstantTensorYKernel (reference where.cpp:90-150). */
+int fluidml_hip_where_constant_cond_constant_tensor_y(const fl_tensor *cond, const fl_tensor *x, const fl_tensor *y, const fl_tensor *out, void *stream);
+/* AddDivErfAddMulMulKernel: t = x + b; out = t * (erf(t / div) + add1) * mul1
+ * (reference add_div_erf_add_mul_mul.cpp:29-132). */
+int fluidml_hip_add_div_erf_add_mul_mul(const fl_tensor *in, const fl_tensor *add0, const fl_tensor *out, double div, double add1, double mul1, void *stream);
+/* UnsqueezeSubLhsScalarMulRhsScalarKernel: out = (sub - unsqueeze(x)) * mul
+ * (reference unsqueeze_sub_mul.cpp:19-69). */
+int fluidml_hip_unsqueeze_sub_lhs_scalar_mul_rhs_scalar(const fl_tensor *in, const fl_tensor *out, const int64_t *axes, int32_t n_axes, double sub, double mul, void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* a.4 Data-movement kernels (HBM bound).                                     */
+
+/* TransposeKernel: out[d[perm[0]],...] = in[d0,...] (reference transpose.cpp:19-48). */
+int fluidml_hip_transpose(const fl_tensor *in, const fl_tensor *out, const int64_t *perm, int32_t n_perm, void *stream);
+/* ReshapeKernel: logical row-major reshape through both layouts
+ * (reference reshape.cpp:18-64). */
+int fluidml_hip_reshape(const fl_tensor *in, const fl_tensor *out, void *stream);
+/* FlattenKernel (reference flatten.cpp:15-63). */
+int fluidml_hip_flatten(const fl_tensor *in, const fl_tensor *out, int64_t axis, void *stream);
+/* SqueezeKernel / UnsqueezeKernel (reference squeeze.cpp:17-54, unsqueeze.cpp:20-63). */
+int fluidml_hip_squeeze(const fl_tensor *in, const fl_tensor *out, const int64_t *axes, int32_t n_axes, void *stream);
+int fluidml_hip_unsqueeze(const fl_tensor *in, const fl_tensor *out, const int64_t *axes, int32_t n_axes, void *stream);
+/* SliceKernel: per sliced axis (start, axis, step); extent = out shape
+ * (reference slice.cpp:17-55). */
+int fluidml_hip_slice(const fl_tensor *in, const fl_tensor *out, const int64_t *starts, const int64_t *axes, const int64_t *steps, int32_t n, void *stream);
+/* Concat2Kernel (reference concat.cpp:18-68). */
+int fluidml_hip_concat2(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, int64_t axis, void *stream);
+/* PadKernel: copies the input into the interior; the border is not written
+ * (reference pad.cpp:15-51). `pads_before[i]` per dimension. */
+int fluidml_hip_pad(const fl_tensor *in, const fl_tensor *out, const int64_t *pads_before, int32_t n, void *stream);
+/* GatherConstantIndexScalarKernel (reference gather.cpp:100-139). */
+int fluidml_hip_gather_constant_index_scalar(const fl_tensor *in, const fl_tensor *out, int64_t axis, int64_t index, uint32_t flags, void *stream);
+/* GatherConstantIndicesTensorKernel: data is the runtime input, `indices` a
+ * constant int64 tensor (reference gather.cpp:149-186, 24-86). */
+int fluidml_hip_gather_constant_indices_tensor(const fl_tensor *in, const fl_tensor *indices, const fl_tensor *out, int64_t axis, void *stream);
+/* GatherConstantDataTensorKernel: `data` is a constant float32 table, the
+ * runtime input holds int64 indices, axis 0 (reference gather.cpp:195-272). */
+int fluidml_hip_gather_constant_data_tensor(const fl_tensor *indices, const fl_tensor *data, const fl_tensor *out, void *stream);
+/* GatherConstantDataTensorAddTensorLhsAddTensorLhsKernel: data[ids] + add0 + add1
+ * (reference gather_add_add.cpp:25-163). */
+int fluidml_hip_gather_constant_data_tensor_add_tensor_lhs_add_tensor_lhs(const fl_tensor *indices, const fl_tensor *data, const fl_tensor *add0, const fl_tensor *add1, const fl_tensor *out, void *stream);
+/* CumSumKernel: integer inclusive forward scan (reference cum_sum.cpp:53-87). */
+int fluidml_hip_cum_sum(const fl_tensor *in, const fl_tensor *out, int64_t axis, void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* a.2 Row-reduction kernels (HBM bound).                                     */
+
+/* SoftmaxKernel along `axis` (>= 0) (reference softmax.cpp:22-139).  The
+ * reference makes six passes through a scratch of shape[axis->1]; here the
+ * row is reduced in registers/LDS and `scratch` is not touched. */
+int fluidml_hip_softmax(const fl_tensor *in, const fl_tensor *out, void *scratch, size_t scratch_bytes, int64_t axis, void *stream);
+/* LayerNormalizationConstantScaleBiasKernel: biased variance over the single
+ * `axis`; scale/bias broadcast from the trailing dims (reference
+ * layer_normalization.cpp:33-220).  With FL_REF_LN_STALE_SCRATCH the row sum
+ * starts from the float the scratch holds for that row. */
+int fluidml_hip_layer_normalization_constant_scale_bias(const fl_tensor *in, const fl_tensor *scale, const fl_tensor *bias, const fl_tensor *out, void *scratch, size_t scratch_bytes, int64_t axis, double epsilon, uint32_t flags, void *stream);
+/* ReduceMeanKernel, keepdims=1 only (reference reduce_mean.cpp:16-98). */
+int fluidml_hip_reduce_mean(const fl_tensor *in, const fl_tensor *out, const int64_t *axes, int32_t n_axes, void *stream);
+/* MaxPoolWithoutPaddingKernel: trailing `n` dims pooled (reference maxpool.cpp:17-82). */
+int fluidml_hip_max_pool_without_padding(const fl_tensor *in, const fl_tensor *out, const int64_t *kernel_shape, const int64_t *strides, int32_t n, void *stream);
+/* AveragePoolWithoutPaddingKernel (reference averagepool.cpp:19-87). */
+int fluidml_hip_average_pool_without_padding(const fl_tensor *in, const fl_tensor *out, const int64_t *kernel_shape, const int64_t *strides, int32_t n, void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* a.1 Contraction kernels (MFMA bound).                                      */
+
+/* MatMulKernel: NumPy batch-broadcast matmul, fp32 MFMA
+ * (reference matmul.cpp:28-59, utils.cpp:64-147). */
+int fluidml_hip_matmul(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream);
+/* Same contraction with operands rounded to bf16 and fp32 accumulation
+ * (opt-in; no counterpart in the reference, error is reported separately). */
+int fluidml_hip_matmul_bf16(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream);
+/* GemmConstantBiasKernel (kernel name "GemmConstantWeightsBiasKernel"):
+ * rank-2, bias rank 1 or 2 (reference gemm.cpp:39-182). */
+int fluidml_hip_gemm_constant_weights_bias(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double alpha, double beta, int32_t trans_a, int32_t trans_b, uint32_t flags, void *stream);
+/* ConvWithoutPaddingKernel: NCHW-logical, N-d spatial, group==1 or depthwise
+ * (reference conv.cpp:27-201, 214-218). bias may be NULL. `strides` and
+ * `dilations` have rank-2 entries. */
+int fluidml_hip_conv_without_padding(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *strides, const int64_t *dilations, int64_t group, uint32_t flags, void *stream);
+/* ConvWithPaddingKernel (reference conv.cpp:230-280). `pads` has 2*(rank-2)
+ * entries, begins then ends.  The reference materialises the zero-padded
+ * input in `scratch`; here padding is applied on the fly and scratch is
+ * untouched. */
+int fluidml_hip_conv_with_padding(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, void *scratch, size_t scratch_bytes, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, uint32_t flags, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FLUIDML_HIP_H_ */

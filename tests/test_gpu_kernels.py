@@ -1,0 +1,613 @@
+"""Parity of every HIP kernel (through the C ABI) against the C oracle on the
+same seeded inputs and the same layout permutations.
+
+Shapes follow the reference's per-operator tests (test/python/node/*.py) where
+the oracle finishes in seconds, plus ragged / unaligned cases.  Bit-exact for
+integer, copy and single-operation fp32 kernels; rel 1e-4 / abs 1e-5 (the
+tolerance BASELINE.json states) where device libm or summation order differ.
+"""
+import ctypes
+import sys
+import zlib
+
+import numpy as np
+import pytest
+
+from oracle import kernels as ok
+from tests.util import DeviceView, all_layouts, assert_close, some_layouts
+
+pytestmark = pytest.mark.gpu
+
+
+def _cabi():
+    from fluidml_amd import cabi
+
+    return cabi
+
+
+def announce(*what):
+    print("[case]", *what, flush=True)
+    sys.stdout.flush()
+
+
+def seed_of(*what):
+    return zlib.crc32(repr(what).encode())
+
+
+def rand(rng, shape, lo=-2.0, hi=2.0):
+    return rng.uniform(lo, hi, size=shape).astype(np.float32)
+
+
+# --------------------------------------------------------------------------- unary f32
+
+UNARY = [
+    # name, oracle op, c0, c1, exact, input range
+    ("add_constant", ok.OP_ADD_C, 1.5, 0, True, (-2, 2)),
+    ("sub_constant_lhs", ok.OP_RSUB_C, 1.0, 0, True, (-2, 2)),
+    ("mul_constant", ok.OP_MUL_C, -10000.0, 0, True, (-2, 2)),
+    ("div_constant_rhs", ok.OP_DIV_C, 8.0, 0, True, (-2, 2)),
+    ("pow", ok.OP_POW_C, 2.0, 0, False, (0.1, 3)),
+    ("erf", ok.OP_ERF, 0, 0, False, (-3, 3)),
+    ("relu", ok.OP_RELU, 0, 0, True, (-2, 2)),
+    ("clip", ok.OP_CLIP, 0.0, 6.0, True, (-8, 8)),
+    ("tanh", ok.OP_TANH, 0, 0, False, (-3, 3)),
+    ("sqrt", ok.OP_SQRT, 0, 0, True, (0, 4)),
+    ("neg", ok.OP_NEG, 0, 0, True, (-2, 2)),
+    ("dropout", ok.OP_COPY, 0, 0, True, (-2, 2)),
+]
+
+
+@pytest.mark.parametrize("name,op,c0,c1,exact,rng_range", UNARY, ids=[u[0] for u in UNARY])
+@pytest.mark.parametrize("shape", [(1, 128, 768), (3, 5, 7), (2, 3, 4, 6)], ids=str)
+def test_unary_f32(device, name, op, c0, c1, exact, rng_range, shape):
+    cabi = _cabi()
+    rng = np.random.default_rng(seed_of(name, shape))
+    x = rand(rng, shape, *rng_range)
+    for lin in some_layouts(len(shape), rng, 3):
+        for lout in some_layouts(len(shape), rng, 3):
+            announce(name, shape, lin, lout)
+            hx, ho = ok.View(x, lin), ok.View.empty(shape, np.float32, lout)
+            ok.unary_f32(op, hx, ho, c0, c1)
+            dx, do = DeviceView(hx, device), DeviceView(ok.View.empty(shape, np.float32, lout), device)
+            if name in ("add_constant", "sub_constant_lhs", "mul_constant", "div_constant_rhs", "pow"):
+                cabi.call(name, dx.ref(), do.ref(), ctypes.c_double(c0), None)
+            elif name == "clip":
+                cabi.call(name, dx.ref(), do.ref(), ctypes.c_float(c0), ctypes.c_float(c1), None)
+            else:
+                cabi.call(name, dx.ref(), do.ref(), None)
+            assert_close(do.logical(), ho.logical(), exact=exact, what=f"{name} {shape} {lin}->{lout}")
+
+
+def test_unary_unaligned_base(device):
+    """Arena offsets are only 4-byte aligned in general: the 128-bit path must not be taken."""
+    cabi = _cabi()
+    rng = np.random.default_rng(7)
+    x = rand(rng, (4, 64))
+    hx, ho = ok.View(x), ok.View.empty((4, 64))
+    ok.unary_f32(ok.OP_ADD_C, hx, ho, 2.0)
+    for mis_in, mis_out in [(1, 0), (0, 3), (1, 2)]:
+        announce("add_constant unaligned", mis_in, mis_out)
+        dx = DeviceView(hx, device, misalign_elems=mis_in)
+        do = DeviceView(ok.View.empty((4, 64)), device, misalign_elems=mis_out)
+        cabi.call("add_constant", dx.ref(), do.ref(), ctypes.c_double(2.0), None)
+        assert_close(do.logical(), ho.logical(), exact=True, what="unaligned add")
+
+
+def test_integer_and_bool_kernels(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(11)
+    shape = (2, 128)
+    ids = rng.integers(0, 5, size=shape).astype(np.int64)
+    for lin in all_layouts(2):
+        announce("int kernels", lin)
+        hx = ok.View(ids, lin)
+        # add constant int64
+        ho = ok.View.empty(shape, np.int64)
+        ok.unary_int(ok.IOP_ADD_C, hx, ho, 2)
+        dx, do = DeviceView(hx, device), DeviceView(ok.View.empty(shape, np.int64), device)
+        cabi.call("add_constant", dx.ref(), do.ref(), ctypes.c_double(2), None)
+        assert_close(do.logical(), ho.logical(), exact=True, what="add_constant i64")
+        # equal -> bool
+        hb = ok.View.empty(shape, np.bool_)
+        ok.unary_int(ok.IOP_EQ_C, hx, hb, 1)
+        db = DeviceView(ok.View.empty(shape, np.bool_), device)
+        cabi.call("equal", dx.ref(), db.ref(), ctypes.c_double(1), None)
+        assert_close(db.logical(), hb.logical(), exact=True, what="equal")
+        # not
+        hn = ok.View.empty(shape, np.bool_)
+        ok.unary_int(ok.IOP_NOT, hb, hn)
+        dn = DeviceView(ok.View.empty(shape, np.bool_), device)
+        dbin = DeviceView(hb, device)
+        cabi.call("not", dbin.ref(), dn.ref(), None)
+        assert_close(dn.logical(), hn.logical(), exact=True, what="not")
+        # cast bool -> int64, int64 -> int32
+        for src, dst_np in [(hb, np.int64), (hx, np.int32), (hb, np.int32)]:
+            hc = ok.View.empty(shape, dst_np)
+            ok.unary_int(ok.IOP_CAST, src, hc)
+            dc = DeviceView(ok.View.empty(shape, dst_np), device)
+            ds = DeviceView(src, device)
+            cabi.call("cast", ds.ref(), dc.ref(), None)
+            assert_close(dc.logical(), hc.logical(), exact=True, what=f"cast ->{dst_np}")
+        # cumsum along both axes
+        for axis in (0, 1):
+            hs = ok.View.empty(shape, np.int64)
+            ok.cum_sum(hx, hs, axis)
+            assert (hs.logical() == np.cumsum(ids, axis=axis)).all()
+            dsum = DeviceView(ok.View.empty(shape, np.int64), device)
+            cabi.call("cum_sum", dx.ref(), dsum.ref(), ctypes.c_int64(axis), None)
+            assert_close(dsum.logical(), hs.logical(), exact=True, what=f"cum_sum axis {axis}")
+
+
+# --------------------------------------------------------------------------- binary
+
+BINARY = [("add_common", ok.BOP_ADD), ("sub_common", ok.BOP_SUB), ("mul_common", ok.BOP_MUL), ("div_common", ok.BOP_DIV)]
+BINARY_SHAPES = [
+    ((1, 128, 768), (1, 128, 768)),  # reference add0.py / mul0.py / sub1.py / div1.py
+    ((1, 128, 768), (768,)),  # bias
+    ((1, 12, 128, 128), (1, 1, 1, 128)),  # additive attention mask
+    ((2, 5, 7), (5, 1)),
+    ((3, 1, 6), (3, 4, 6)),
+]
+
+
+@pytest.mark.parametrize("name,op", BINARY, ids=[b[0] for b in BINARY])
+@pytest.mark.parametrize("lshape,rshape", BINARY_SHAPES, ids=str)
+def test_binary_f32(device, name, op, lshape, rshape):
+    cabi = _cabi()
+    rng = np.random.default_rng(seed_of(name, lshape, rshape))
+    a, b = rand(rng, lshape), rand(rng, rshape, 0.5, 2.0)
+    oshape = np.broadcast_shapes(lshape, rshape)
+    for la in some_layouts(len(lshape), rng, 3):
+        for lb in some_layouts(len(rshape), rng, 2):
+            for lo in some_layouts(len(oshape), rng, 2):
+                announce(name, lshape, rshape, la, lb, lo)
+                ha, hb, ho = ok.View(a, la), ok.View(b, lb), ok.View.empty(oshape, np.float32, lo)
+                ok.binary_f32(op, ha, hb, ho)
+                da, db = DeviceView(ha, device), DeviceView(hb, device)
+                do = DeviceView(ok.View.empty(oshape, np.float32, lo), device)
+                cabi.call(name, da.ref(), db.ref(), do.ref(), None)
+                assert_close(do.logical(), ho.logical(), exact=True, what=f"{name} {la} {lb} {lo}")
+
+
+def test_mul_common_int(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(5)
+    a = rng.integers(-9, 9, size=(2, 16)).astype(np.int64)
+    b = rng.integers(-9, 9, size=(16,)).astype(np.int64)
+    ha, hb, ho = ok.View(a), ok.View(b), ok.View.empty((2, 16), np.int64)
+    ok.mul_int(ha, hb, ho)
+    da, db, do = DeviceView(ha, device), DeviceView(hb, device), DeviceView(ok.View.empty((2, 16), np.int64), device)
+    announce("mul_common int64")
+    cabi.call("mul_common", da.ref(), db.ref(), do.ref(), None)
+    assert_close(do.logical(), ho.logical(), exact=True, what="mul int")
+
+
+def test_where(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(3)
+    S = 64
+    cond = np.tril(np.ones((1, 1, S, S), dtype=np.bool_))
+    x = rand(rng, (1, 8, S, S))
+    y = rand(rng, (1,))
+    for lx in some_layouts(4, rng, 3):
+        announce("where", lx)
+        hc, hx, hy = ok.View(cond), ok.View(x, lx), ok.View(y)
+        ho = ok.View.empty(x.shape, np.float32, lx)
+        ok.where(hc, hx, None, -3.4e38, ho)
+        dc, dx = DeviceView(hc, device), DeviceView(hx, device)
+        do = DeviceView(ok.View.empty(x.shape, np.float32, lx), device)
+        cabi.call("where_constant_cond_constant_scalar_y", dc.ref(), dx.ref(), do.ref(), ctypes.c_double(-3.4e38), None)
+        assert_close(do.logical(), ho.logical(), exact=True, what="where scalar y")
+        ho2 = ok.View.empty(x.shape, np.float32, lx)
+        ok.where(hc, hx, hy, 0.0, ho2)
+        dy = DeviceView(hy, device)
+        do2 = DeviceView(ok.View.empty(x.shape, np.float32, lx), device)
+        cabi.call("where_constant_cond_constant_tensor_y", dc.ref(), dx.ref(), dy.ref(), do2.ref(), None)
+        assert_close(do2.logical(), ho2.logical(), exact=True, what="where tensor y")
+
+
+def test_fused_elementwise(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(21)
+    x, b = rand(rng, (1, 128, 3072)), rand(rng, (3072,))
+    for lx in some_layouts(3, rng, 3):
+        announce("add_div_erf_add_mul_mul", lx)
+        hx, hb, ho = ok.View(x, lx), ok.View(b), ok.View.empty(x.shape, np.float32, lx)
+        ok.add_div_erf_add_mul_mul(hx, hb, ho, 1.4142135381698608, 1.0, 0.5)
+        dx, db = DeviceView(hx, device), DeviceView(hb, device)
+        do = DeviceView(ok.View.empty(x.shape, np.float32, lx), device)
+        cabi.call("add_div_erf_add_mul_mul", dx.ref(), db.ref(), do.ref(), ctypes.c_double(1.4142135381698608),
+                  ctypes.c_double(1.0), ctypes.c_double(0.5), None)
+        assert_close(do.logical(), ho.logical(), what="gelu chain")
+    m = rand(rng, (1, 128), 0, 1)
+    hm, ho = ok.View(m), ok.View.empty((1, 1, 1, 128))
+    ok.unsqueeze_sub_mul(hm, ho, [1, 2], 1.0, -10000.0)
+    dm, do = DeviceView(hm, device), DeviceView(ok.View.empty((1, 1, 1, 128)), device)
+    announce("unsqueeze_sub_mul")
+    cabi.call("unsqueeze_sub_lhs_scalar_mul_rhs_scalar", dm.ref(), do.ref(), cabi.i64_array([1, 2]), 2,
+              ctypes.c_double(1.0), ctypes.c_double(-10000.0), None)
+    assert_close(do.logical(), ho.logical(), exact=True, what="unsqueeze_sub_mul")
+
+
+# --------------------------------------------------------------------------- data movement
+
+
+def test_transpose(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(31)
+    for shape, perm in [((1, 128, 12, 64), (0, 2, 1, 3)), ((1, 12, 128, 64), (0, 1, 3, 2)), ((3, 5, 7), (2, 0, 1)),
+                        ((33, 65), (1, 0))]:
+        x = rand(rng, shape)
+        oshape = tuple(shape[p] for p in perm)
+        for lin in some_layouts(len(shape), rng, 3):
+            for lout in some_layouts(len(shape), rng, 3):
+                announce("transpose", shape, perm, lin, lout)
+                hx, ho = ok.View(x, lin), ok.View.empty(oshape, np.float32, lout)
+                ok.transpose(hx, ho, perm)
+                assert (ho.logical() == np.transpose(x, perm)).all()
+                dx, do = DeviceView(hx, device), DeviceView(ok.View.empty(oshape, np.float32, lout), device)
+                cabi.call("transpose", dx.ref(), do.ref(), cabi.i64_array(perm), len(perm), None)
+                assert_close(do.logical(), ho.logical(), exact=True, what="transpose")
+
+
+def test_reshape_flatten(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(32)
+    cases = [((1, 128, 768), (1, 128, 12, 64)), ((1, 12, 128, 64), (12, 128, 64)), ((2, 3, 4), (4, 6)), ((6,), (2, 3))]
+    for ishape, oshape in cases:
+        x = rand(rng, ishape)
+        for lin in some_layouts(len(ishape), rng, 3):
+            for lout in some_layouts(len(oshape), rng, 3):
+                announce("reshape", ishape, oshape, lin, lout)
+                hx, ho = ok.View(x, lin), ok.View.empty(oshape, np.float32, lout)
+                ok.reshape(hx, ho)
+                assert (ho.logical() == x.reshape(oshape)).all()
+                dx, do = DeviceView(hx, device), DeviceView(ok.View.empty(oshape, np.float32, lout), device)
+                cabi.call("reshape", dx.ref(), do.ref(), None)
+                assert_close(do.logical(), ho.logical(), exact=True, what="reshape")
+    x = rand(rng, (2, 3, 4, 5))
+    for axis in (0, 1, 2, -1):
+        ax = axis % 4
+        oshape = (int(np.prod(x.shape[:ax])), int(np.prod(x.shape[ax:])))
+        for lin in some_layouts(4, rng, 3):
+            announce("flatten", axis, lin)
+            hx, ho = ok.View(x, lin), ok.View.empty(oshape, np.float32, [1, 0])
+            ok.reshape(hx, ho)
+            dx, do = DeviceView(hx, device), DeviceView(ok.View.empty(oshape, np.float32, [1, 0]), device)
+            cabi.call("flatten", dx.ref(), do.ref(), ctypes.c_int64(axis), None)
+            assert_close(do.logical(), ho.logical(), exact=True, what="flatten")
+
+
+def test_squeeze_unsqueeze_slice_concat_pad(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(33)
+    x = rand(rng, (1, 128, 1, 64))
+    for lin in some_layouts(4, rng, 3):
+        announce("squeeze", lin)
+        hx, ho = ok.View(x, lin), ok.View.empty((128, 64), np.float32, [1, 0])
+        ok.squeeze(hx, ho, [0, 2])
+        assert (ho.logical() == x.reshape(128, 64)).all()
+        dx, do = DeviceView(hx, device), DeviceView(ok.View.empty((128, 64), np.float32, [1, 0]), device)
+        cabi.call("squeeze", dx.ref(), do.ref(), cabi.i64_array([0, 2]), 2, None)
+        assert_close(do.logical(), ho.logical(), exact=True, what="squeeze")
+    y = rand(rng, (128, 64))
+    for lout in some_layouts(4, rng, 3):
+        announce("unsqueeze", lout)
+        hy, ho = ok.View(y, [1, 0]), ok.View.empty((1, 128, 1, 64), np.float32, lout)
+        ok.unsqueeze(hy, ho, [0, 2])
+        assert (ho.logical() == y.reshape(1, 128, 1, 64)).all()
+        dy, do = DeviceView(hy, device), DeviceView(ok.View.empty((1, 128, 1, 64), np.float32, lout), device)
+        cabi.call("unsqueeze", dy.ref(), do.ref(), cabi.i64_array([0, 2]), 2, None)
+        assert_close(do.logical(), ho.logical(), exact=True, what="unsqueeze")
+    z = rand(rng, (1, 8, 256, 64))
+    for lin in some_layouts(4, rng, 3):
+        announce("slice/concat", lin)
+        # rotary halves: z[..., :8], z[..., 8:16], and a strided slice
+        for starts, axes, steps, oshape in [([0], [3], [1], (1, 8, 256, 8)), ([8], [3], [1], (1, 8, 256, 8)),
+                                            ([1, 2], [2, 3], [2, 3], (1, 8, 100, 20))]:
+            hz, ho = ok.View(z, lin), ok.View.empty(oshape, np.float32, lin)
+            ok.slice_(hz, ho, starts, axes, steps)
+            dz, do = DeviceView(hz, device), DeviceView(ok.View.empty(oshape, np.float32, lin), device)
+            cabi.call("slice", dz.ref(), do.ref(), cabi.i64_array(starts), cabi.i64_array(axes), cabi.i64_array(steps),
+                      len(axes), None)
+            assert_close(do.logical(), ho.logical(), exact=True, what="slice")
+        a, b = rand(rng, (1, 8, 256, 8)), rand(rng, (1, 8, 256, 24))
+        ha, hb, ho = ok.View(a, lin), ok.View(b), ok.View.empty((1, 8, 256, 32), np.float32, lin)
+        ok.concat2(ha, hb, ho, 3)
+        assert (ho.logical() == np.concatenate([a, b], axis=3)).all()
+        da, db = DeviceView(ha, device), DeviceView(hb, device)
+        do = DeviceView(ok.View.empty((1, 8, 256, 32), np.float32, lin), device)
+        cabi.call("concat2", da.ref(), db.ref(), do.ref(), ctypes.c_int64(3), None)
+        assert_close(do.logical(), ho.logical(), exact=True, what="concat2")
+    p = rand(rng, (2, 3, 5))
+    hp, ho = ok.View(p), ok.View.empty((2, 4, 8), np.float32, [2, 0, 1], fill=7)
+    ok.pad(hp, ho, [0, 1, 2])
+    dp = DeviceView(hp, device)
+    do = DeviceView(ok.View.empty((2, 4, 8), np.float32, [2, 0, 1], fill=7), device)
+    announce("pad")
+    cabi.call("pad", dp.ref(), do.ref(), cabi.i64_array([0, 1, 2]), 3, None)
+    assert_close(do.logical(), ho.logical(), exact=True, what="pad (border untouched)")
+
+
+def test_gathers(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(34)
+    table = rand(rng, (1000, 768))
+    ids = rng.integers(0, 1000, size=(1, 128)).astype(np.int64)
+    pos, typ = rand(rng, (128, 768)), rand(rng, (768,))
+    for lout in some_layouts(3, rng, 3):
+        announce("gather_constant_data_tensor", lout)
+        hi, ht, ho = ok.View(ids), ok.View(table), ok.View.empty((1, 128, 768), np.float32, lout)
+        ok.gather_data_tensor(hi, ht, ho)
+        assert (ho.logical() == table[ids]).all()
+        di, dt = DeviceView(hi, device), DeviceView(ht, device)
+        do = DeviceView(ok.View.empty((1, 128, 768), np.float32, lout), device)
+        cabi.call("gather_constant_data_tensor", di.ref(), dt.ref(), do.ref(), None)
+        assert_close(do.logical(), ho.logical(), exact=True, what="gather data tensor")
+        hp, hy = ok.View(pos), ok.View(typ)
+        ho2 = ok.View.empty((1, 128, 768), np.float32, lout)
+        ok.gather_data_tensor(hi, ht, ho2, hp, hy)
+        dp, dy = DeviceView(hp, device), DeviceView(hy, device)
+        do2 = DeviceView(ok.View.empty((1, 128, 768), np.float32, lout), device)
+        cabi.call("gather_constant_data_tensor_add_tensor_lhs_add_tensor_lhs", di.ref(), dt.ref(), dp.ref(), dy.ref(),
+                  do2.ref(), None)
+        assert_close(do2.logical(), ho2.logical(), exact=True, what="gather+add+add")
+    x = rand(rng, (4, 9, 6))
+    for lin in some_layouts(3, rng, 3):
+        for axis, index in [(0, 3), (1, 0), (2, 5), (-1, 2)]:
+            announce("gather_constant_index_scalar", lin, axis, index)
+            ax = axis % 3
+            oshape = tuple(s for i, s in enumerate(x.shape) if i != ax)
+            hx, ho = ok.View(x, lin), ok.View.empty(oshape)
+            ok.gather_index_scalar(hx, ho, axis, index)
+            assert (ho.logical() == np.take(x, index, axis=ax)).all()
+            dx, do = DeviceView(hx, device), DeviceView(ok.View.empty(oshape), device)
+            cabi.call("gather_constant_index_scalar", dx.ref(), do.ref(), ctypes.c_int64(axis), ctypes.c_int64(index),
+                      ctypes.c_uint32(0), None)
+            assert_close(do.logical(), ho.logical(), exact=True, what="gather index scalar")
+        idx = rng.integers(0, 9, size=(2, 5)).astype(np.int64)
+        announce("gather_constant_indices_tensor", lin)
+        hx, hi, ho = ok.View(x, lin), ok.View(idx), ok.View.empty((4, 2, 5, 6))
+        ok.gather_indices_tensor(hx, hi, ho, 1)
+        assert (ho.logical() == np.take(x, idx, axis=1)).all()
+        dx, di, do = DeviceView(hx, device), DeviceView(hi, device), DeviceView(ok.View.empty((4, 2, 5, 6)), device)
+        cabi.call("gather_constant_indices_tensor", dx.ref(), di.ref(), do.ref(), ctypes.c_int64(1), None)
+        assert_close(do.logical(), ho.logical(), exact=True, what="gather indices tensor")
+
+
+# --------------------------------------------------------------------------- row reductions
+
+SOFTMAX_CASES = [((1, 12, 128, 128), 3), ((1, 8, 256, 256), 3), ((2, 3, 9), 2), ((2, 17, 5), 1), ((4, 1500), 1),
+                 ((1, 6, 128, 9), 3), ((3, 40), 0)]
+
+
+@pytest.mark.parametrize("shape,axis", SOFTMAX_CASES, ids=str)
+def test_softmax(device, shape, axis):
+    cabi = _cabi()
+    rng = np.random.default_rng(seed_of(shape, axis))
+    x = rand(rng, shape, -6, 6)
+    for lin in some_layouts(len(shape), rng, 3):
+        for lout in some_layouts(len(shape), rng, 2):
+            announce("softmax", shape, axis, lin, lout)
+            hx, ho = ok.View(x, lin), ok.View.empty(shape, np.float32, lout)
+            ok.softmax(hx, ho, axis)
+            dx, do = DeviceView(hx, device), DeviceView(ok.View.empty(shape, np.float32, lout), device)
+            cabi.call("softmax", dx.ref(), do.ref(), None, 0, ctypes.c_int64(axis), None)
+            assert_close(do.logical(), ho.logical(), what=f"softmax {shape} {lin}->{lout}")
+
+
+LN_CASES = [((1, 128, 768), 2, 1e-12), ((1, 256, 512), 2, 1e-5), ((2, 7, 33), 2, 1e-5), ((3, 20, 5), 1, 1e-5),
+            ((2, 5000), 1, 1e-5)]
+
+
+@pytest.mark.parametrize("shape,axis,eps", LN_CASES, ids=str)
+def test_layer_norm(device, shape, axis, eps):
+    cabi = _cabi()
+    rng = np.random.default_rng(seed_of(shape, axis))
+    x = rand(rng, shape, -3, 3)
+    pshape = shape[axis:]
+    g, b = rand(rng, pshape, 0.5, 1.5), rand(rng, pshape, -0.5, 0.5)
+    rows = int(np.prod(shape)) // shape[axis]
+    for lin in some_layouts(len(shape), rng, 3):
+        for lout in some_layouts(len(shape), rng, 2):
+            announce("layer_norm", shape, axis, lin, lout)
+            hx, hg, hb = ok.View(x, lin), ok.View(g), ok.View(b)
+            ho = ok.View.empty(shape, np.float32, lout)
+            ok.layer_norm(hx, hg, hb, ho, axis, eps)
+            dx, dg, db = DeviceView(hx, device), DeviceView(hg, device), DeviceView(hb, device)
+            do = DeviceView(ok.View.empty(shape, np.float32, lout), device)
+            cabi.call("layer_normalization_constant_scale_bias", dx.ref(), dg.ref(), db.ref(), do.ref(), None, 0,
+                      ctypes.c_int64(axis), ctypes.c_double(eps), ctypes.c_uint32(0), None)
+            assert_close(do.logical(), ho.logical(), what=f"layer_norm {shape} {lin}->{lout}")
+    # literal mode: the row sum starts from what the scratch holds
+    import torch
+
+    stale = rng.uniform(-50, 50, size=rows).astype(np.float32)
+    hx, hg, hb = ok.View(x), ok.View(g), ok.View(b)
+    ho = ok.View.empty(shape)
+    ok.layer_norm(hx, hg, hb, ho, axis, eps, scratch=stale)
+    dx, dg, db = DeviceView(hx, device), DeviceView(hg, device), DeviceView(hb, device)
+    do = DeviceView(ok.View.empty(shape), device)
+    dscratch = torch.from_numpy(stale).to(device)
+    announce("layer_norm stale scratch", shape)
+    cabi.call("layer_normalization_constant_scale_bias", dx.ref(), dg.ref(), db.ref(), do.ref(),
+              ctypes.c_void_p(dscratch.data_ptr()), rows * 4, ctypes.c_int64(axis), ctypes.c_double(eps),
+              ctypes.c_uint32(cabi.FL_REF_LN_STALE_SCRATCH), None)
+    assert_close(do.logical(), ho.logical(), what="layer_norm stale scratch")
+
+
+def test_reduce_mean(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(41)
+    for shape, axes in [((1, 32, 14, 14), [2, 3]), ((1, 128, 768), [2]), ((3, 4, 5), [0]), ((2, 6, 5, 3), [1, 3])]:
+        x = rand(rng, shape)
+        oshape = tuple(1 if i in axes else s for i, s in enumerate(shape))
+        for lin in some_layouts(len(shape), rng, 3):
+            announce("reduce_mean", shape, axes, lin)
+            hx, ho = ok.View(x, lin), ok.View.empty(oshape)
+            ok.reduce_mean(hx, ho, axes)
+            dx, do = DeviceView(hx, device), DeviceView(ok.View.empty(oshape), device)
+            cabi.call("reduce_mean", dx.ref(), do.ref(), cabi.i64_array(axes), len(axes), None)
+            assert_close(do.logical(), ho.logical(), what="reduce_mean")
+
+
+def test_pools(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(42)
+    cases = [((1, 8, 56, 56), (2, 2), (2, 2)), ((1, 40, 7, 7), (7, 7), (1, 1)), ((2, 3, 9, 11), (3, 2), (2, 3)),
+             ((1, 4, 30), (3,), (2,))]
+    for shape, k, s in cases:
+        x = rand(rng, shape)
+        n = len(k)
+        oshape = tuple(shape[: len(shape) - n]) + tuple((shape[len(shape) - n + i] - k[i]) // s[i] + 1 for i in range(n))
+        for lin in some_layouts(len(shape), rng, 3):
+            for is_max, name in [(True, "max_pool_without_padding"), (False, "average_pool_without_padding")]:
+                announce(name, shape, k, s, lin)
+                hx, ho = ok.View(x, lin), ok.View.empty(oshape, np.float32, lin)
+                ok.pool(is_max, hx, ho, k, s)
+                dx, do = DeviceView(hx, device), DeviceView(ok.View.empty(oshape, np.float32, lin), device)
+                cabi.call(name, dx.ref(), do.ref(), cabi.i64_array(k), cabi.i64_array(s), n, None)
+                assert_close(do.logical(), ho.logical(), exact=True, what=name)
+
+
+# --------------------------------------------------------------------------- contractions
+
+MATMUL_CASES = [
+    ((1, 12, 128, 64), (1, 12, 64, 128)),  # reference matmul0.py
+    ((1, 128, 768), (768, 768)),  # reference matmul1.py
+    ((1, 12, 128, 128), (1, 12, 128, 64)),
+    ((2, 1, 33, 17), (3, 17, 29)),  # broadcast both ways, ragged
+    ((5, 7), (7, 3)),
+    ((1, 130, 70), (70, 258)),  # tile edges
+    ((64, 6), (6, 64)),  # K not a multiple of 4
+]
+
+
+@pytest.mark.parametrize("lshape,rshape", MATMUL_CASES, ids=str)
+def test_matmul(device, lshape, rshape):
+    cabi = _cabi()
+    rng = np.random.default_rng(seed_of(lshape, rshape))
+    a, b = rand(rng, lshape, -1, 1), rand(rng, rshape, -1, 1)
+    oshape = np.matmul(np.zeros(lshape, np.int8), np.zeros(rshape, np.int8)).shape
+    for la in some_layouts(len(lshape), rng, 3):
+        for lb in some_layouts(len(rshape), rng, 3):
+            for lo in some_layouts(len(oshape), rng, 2):
+                announce("matmul", lshape, rshape, la, lb, lo)
+                ha, hb, ho = ok.View(a, la), ok.View(b, lb), ok.View.empty(oshape, np.float32, lo)
+                ok.matmul(ha, hb, ho)
+                da, db = DeviceView(ha, device), DeviceView(hb, device)
+                do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=9), device)
+                cabi.call("matmul", da.ref(), db.ref(), do.ref(), None)
+                assert_close(do.logical(), ho.logical(), what=f"matmul {la} {lb} {lo}")
+
+
+def test_matmul_large_tiles(device):
+    """Shapes that select the 64x64 and 128x128 workgroup tiles."""
+    cabi = _cabi()
+    rng = np.random.default_rng(77)
+    for M, K, N in [(1024, 96, 1024), (2048, 64, 2048), (520, 40, 1000)]:
+        a, b = rand(rng, (M, K), -1, 1), rand(rng, (K, N), -1, 1)
+        want = a.astype(np.float64) @ b.astype(np.float64)
+        for la, lb in [([0, 1], [0, 1]), ([1, 0], [1, 0]), ([0, 1], [1, 0])]:
+            announce("matmul large", M, K, N, la, lb)
+            da, db = DeviceView(ok.View(a, la), device), DeviceView(ok.View(b, lb), device)
+            do = DeviceView(ok.View.empty((M, N)), device)
+            cabi.call("matmul", da.ref(), db.ref(), do.ref(), None)
+            assert_close(do.logical(), want.astype(np.float32), what="matmul large vs float64 numpy")
+
+
+def test_matmul_unaligned(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(78)
+    a, b = rand(rng, (40, 24), -1, 1), rand(rng, (24, 36), -1, 1)
+    ha, hb, ho = ok.View(a), ok.View(b), ok.View.empty((40, 36))
+    ok.matmul(ha, hb, ho)
+    announce("matmul unaligned")
+    da, db = DeviceView(ha, device, misalign_elems=1), DeviceView(hb, device, misalign_elems=3)
+    do = DeviceView(ok.View.empty((40, 36)), device, misalign_elems=1)
+    cabi.call("matmul", da.ref(), db.ref(), do.ref(), None)
+    assert_close(do.logical(), ho.logical(), what="matmul unaligned bases")
+
+
+def test_gemm(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(51)
+    # reference gemm.py: [1,768] x [768,768]^T + [768], alpha = beta = 1
+    cases = [((1, 768), (768, 768), (768,), 1.0, 1.0, 0, 1), ((8, 100), (100, 50), (50,), 0.5, 2.0, 0, 0),
+             ((100, 8), (50, 100), (8, 50), 1.5, 0.25, 1, 1), ((33, 65), (65, 17), (33, 17), 2.0, 3.0, 0, 0)]
+    for ashape, bshape, cshape, alpha, beta, ta, tb in cases:
+        a, b, c = rand(rng, ashape, -1, 1), rand(rng, bshape, -1, 1), rand(rng, cshape, -1, 1)
+        M = ashape[1] if ta else ashape[0]
+        N = bshape[0] if tb else bshape[1]
+        for flags in (0, cabi.FL_REF_GEMM_SWAPPED_SCALARS):
+            for la, lb in [([0, 1], [0, 1]), ([1, 0], [1, 0])]:
+                announce("gemm", ashape, bshape, cshape, alpha, beta, ta, tb, flags, la, lb)
+                ha, hb, hc, ho = ok.View(a, la), ok.View(b, lb), ok.View(c), ok.View.empty((M, N))
+                ok.gemm(ha, hb, hc, ho, alpha, beta, ta, tb, flags)
+                da, db, dc = DeviceView(ha, device), DeviceView(hb, device), DeviceView(hc, device)
+                do = DeviceView(ok.View.empty((M, N)), device)
+                cabi.call("gemm_constant_weights_bias", da.ref(), db.ref(), dc.ref(), do.ref(), ctypes.c_double(alpha),
+                          ctypes.c_double(beta), ta, tb, ctypes.c_uint32(flags), None)
+                assert_close(do.logical(), ho.logical(), what="gemm")
+
+
+CONV_CASES = [
+    # x shape, w shape, pads, strides, dilations, group, bias
+    ((1, 768, 128), (768, 1, 9), [4, 4], [1], [1], 768, False),  # reference conv0.py (depthwise 1-d, pad 4)
+    ((1, 768, 128), (384, 768, 1), None, [1], [1], 1, True),  # reference conv1.py (pointwise + bias)
+    ((1, 3, 34, 34), (8, 3, 3, 3), [1, 1, 1, 1], [1, 1], [1, 1], 1, True),  # VGG-style 3x3 pad 1
+    ((2, 4, 19, 17), (6, 4, 3, 5), [1, 2, 1, 2], [2, 2], [1, 1], 1, True),  # stride 2
+    ((1, 6, 15, 15), (6, 1, 5, 5), [2, 2, 2, 2], [2, 2], [1, 1], 6, True),  # depthwise 5x5 stride 2
+    ((1, 2, 12, 12), (3, 2, 3, 3), [2, 2, 2, 2], [1, 1], [2, 2], 1, False),  # dilation 2
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: str(c[:2]))
+def test_conv(device, case):
+    cabi = _cabi()
+    xshape, wshape, pads, strides, dilations, group, with_bias = case
+    rng = np.random.default_rng(seed_of(xshape, wshape))
+    x, w = rand(rng, xshape, -1, 1), rand(rng, wshape, -1, 1)
+    bias = rand(rng, (wshape[0],), -1, 1) if with_bias else None
+    ns = len(xshape) - 2
+    p = pads if pads is not None else [0] * (2 * ns)
+
+    def out_dims(st, di):
+        return tuple((xshape[2 + d] + p[d] + p[d + ns] - di[d] * (wshape[2 + d] - 1) - 1) // st[d] + 1 for d in range(ns))
+
+    for flags in (0, cabi.FL_REF_CONV_UNIT_STRIDE | (cabi.FL_REF_CONV_BIAS_INDEX1 if with_bias else 0)):
+        # the output shape comes from the graph's value_info (ONNX semantics) in both modes
+        oshape = (xshape[0], wshape[0]) + out_dims(strides, dilations)
+        for lx in some_layouts(len(xshape), rng, 2):
+            for lo in some_layouts(len(xshape), rng, 2):
+                announce("conv", case[:2], flags, lx, lo)
+                hx, hw, ho = ok.View(x, lx), ok.View(w), ok.View.empty(oshape, np.float32, lo)
+                hb = ok.View(bias) if with_bias else None
+                ok.conv(hx, hw, hb, ho, pads, strides, dilations, group, flags)
+                dx, dw = DeviceView(hx, device), DeviceView(hw, device)
+                db = DeviceView(hb, device) if with_bias else None
+                do = DeviceView(ok.View.empty(oshape, np.float32, lo), device)
+                bref = db.ref() if with_bias else None
+                if pads is None:
+                    cabi.call("conv_without_padding", dx.ref(), dw.ref(), bref, do.ref(), cabi.i64_array(strides),
+                              cabi.i64_array(dilations), ctypes.c_int64(group), ctypes.c_uint32(flags), None)
+                else:
+                    cabi.call("conv_with_padding", dx.ref(), dw.ref(), bref, do.ref(), None, 0, cabi.i64_array(pads),
+                              cabi.i64_array(strides), cabi.i64_array(dilations), ctypes.c_int64(group),
+                              ctypes.c_uint32(flags), None)
+                assert_close(do.logical(), ho.logical(), what=f"conv flags={flags}")
+
+
+def test_argument_errors(device):
+    """Rejected arguments return negative codes and launch nothing."""
+    cabi = _cabi()
+    a = DeviceView(ok.View.empty((4, 5)), device)
+    b = DeviceView(ok.View.empty((6, 3)), device)
+    o = DeviceView(ok.View.empty((4, 3)), device)
+    assert cabi.lib.fluidml_hip_matmul(a.ref(), b.ref(), o.ref(), None) == -3  # FL_ERR_SHAPE
+    assert cabi.lib.fluidml_hip_matmul(None, b.ref(), o.ref(), None) == -1  # FL_ERR_NULL
+    assert cabi.lib.fluidml_hip_softmax(a.ref(), a.ref(), None, 0, 5, None) == -5  # FL_ERR_ATTR
+    i = DeviceView(ok.View.empty((4, 5), np.int64), device)
+    assert cabi.lib.fluidml_hip_erf(i.ref(), a.ref(), None) == -4  # FL_ERR_DTYPE
+    with pytest.raises(cabi.FluidmlHipError):
+        cabi.call("add_common", a.ref(), b.ref(), o.ref(), None)

@@ -1,0 +1,299 @@
+#include "evaluation/eval.h"
+
+#include <algorithm>
+#include <fstream>
+#include <limits>
+#include <sstream>
+#include <stdexcept>
+
+#include "fluidml_hip.h"
+#include "utils/json.h"
+#include "utils/utils.h"
+
+namespace fluidml {
+namespace evaluation {
+namespace {
+
+std::string JoinInts(const std::vector<int64_t> &v) {
+  std::string s = "[";
+  for (size_t i = 0; i < v.size(); ++i) s += (i ? "," : "") + std::to_string(v[i]);
+  return s + "]";
+}
+std::string JoinLayout(const Layout &v) {
+  std::string s = "[";
+  for (size_t i = 0; i < v.size(); ++i) s += (i ? "," : "") + std::to_string(v[i]);
+  return s + "]";
+}
+
+// identity of one table row: kernel name, operand shapes, operand layouts
+std::string RowKey(const std::string &kernel, const std::vector<std::vector<int64_t>> &shapes, const LayoutKey &layouts) {
+  std::string s = kernel;
+  for (const auto &shape : shapes) s += "|" + JoinInts(shape);
+  for (const Layout &l : layouts) s += "|" + JoinLayout(l);
+  return s;
+}
+
+std::vector<std::vector<int64_t>> ShapesOf(const kernel::KernelGenerator &g) {
+  std::vector<std::vector<int64_t>> shapes{g.GetLhsMeta().GetShape()};
+  if (!g.IsSingleInput()) shapes.push_back(g.GetRhsMeta().GetShape());
+  shapes.push_back(g.GetOutputMeta().GetShape());
+  return shapes;
+}
+
+class ConstantCostModel : public CostModel {
+ public:
+  size_t Cost(KernelEval &, const LayoutKey &) override { return 1; }
+};
+
+class TableCostModel : public CostModel {
+ public:
+  explicit TableCostModel(const std::string &text) {
+    json::Value doc = json::Parse(text);
+    const json::Value *table = &doc;
+    if (table->Has("dp_table")) table = &table->At("dp_table");
+    if (table->Has("evaluator")) table = &table->At("evaluator");
+    if (table->kind != json::Value::Kind::Object) throw std::runtime_error("cost table: no evaluator object");
+    auto ints = [](const json::Value &v) {
+      std::vector<int64_t> out;
+      for (const json::Value &e : v.array) out.push_back(static_cast<int64_t>(e.number));
+      return out;
+    };
+    auto layout = [](const json::Value &v) {
+      Layout out;
+      for (const json::Value &e : v.array) out.push_back(static_cast<size_t>(e.number));
+      return out;
+    };
+    for (const auto &kernel : table->object) {
+      for (const json::Value &row : kernel.second.array) {
+        std::vector<std::vector<int64_t>> shapes;
+        LayoutKey layouts;
+        if (row.Has("input_shape")) {
+          shapes = {ints(row.At("input_shape")), ints(row.At("output_shape"))};
+          layouts = {layout(row.At("input_layout")), layout(row.At("output_layout"))};
+        } else {
+          shapes = {ints(row.At("lhs_shape")), ints(row.At("rhs_shape")), ints(row.At("output_shape"))};
+          layouts = {layout(row.At("lhs_layout")), layout(row.At("rhs_layout")), layout(row.At("output_layout"))};
+        }
+        costs_[RowKey(kernel.first, shapes, layouts)] = static_cast<size_t>(row.At("time_cost").number);
+      }
+    }
+  }
+  size_t Cost(KernelEval &eval, const LayoutKey &key) override {
+    const kernel::KernelGenerator &g = eval.GetKernelGenerator();
+    auto it = costs_.find(RowKey(g.GetKernelName(), ShapesOf(g), key));
+    if (it == costs_.end()) throw std::runtime_error("cost table has no entry for " + RowKey(g.GetKernelName(), ShapesOf(g), key));
+    return it->second;
+  }
+
+ private:
+  std::unordered_map<std::string, size_t> costs_;
+};
+
+void Check(int rc, const char *what) {
+  if (rc != 0) throw std::runtime_error(std::string("measuring a kernel: ") + what + ": " + fluidml_hip_error_string(rc));
+}
+
+// Times launches of the real kernel on zero-filled device buffers.
+class MeasuredCostModel : public CostModel {
+ public:
+  explicit MeasuredCostModel(uint32_t flags) : flags_(flags) {}
+  ~MeasuredCostModel() override {
+    for (auto &kv : buffers_) {
+      for (void *p : {kv.second.lhs, kv.second.rhs, kv.second.out, kv.second.scratch}) fluidml_hip_free(p);
+    }
+    fluidml_hip_event_destroy(start_);
+    fluidml_hip_event_destroy(stop_);
+    fluidml_hip_stream_destroy(stream_);
+  }
+
+  size_t Cost(KernelEval &eval, const LayoutKey &key) override {
+    kernel::KernelGenerator &g = eval.GetKernelGenerator();
+    if (stream_ == nullptr) {
+      Check(fluidml_hip_stream_create(&stream_), "stream");
+      Check(fluidml_hip_event_create(&start_), "event");
+      Check(fluidml_hip_event_create(&stop_), "event");
+    }
+    Buffers &b = buffers_[&eval];
+    if (b.out == nullptr) {
+      Check(fluidml_hip_arena_create(g.GetLhsMeta().GetSize(), &b.lhs), "lhs buffer");
+      if (!g.IsSingleInput()) Check(fluidml_hip_arena_create(g.GetRhsMeta().GetSize(), &b.rhs), "rhs buffer");
+      Check(fluidml_hip_arena_create(g.GetOutputMeta().GetSize(), &b.out), "output buffer");
+      Check(fluidml_hip_arena_create(g.GetBufferSize(), &b.scratch), "scratch buffer");
+    }
+    const bool single = g.IsSingleInput();
+    const Layout &lhs_layout = key[0], &out_layout = key.back();
+    std::shared_ptr<kernel::Kernel> k = g.Yield(lhs_layout, single ? Layout{} : key[1], out_layout);
+    k->Prepare();
+    const kernel::TensorView lhs(b.lhs, g.GetLhsMeta(), lhs_layout), out(b.out, g.GetOutputMeta(), out_layout);
+    kernel::TensorView rhs;
+    if (!single) rhs = kernel::TensorView(b.rhs, g.GetRhsMeta(), key[1]);
+    const kernel::Buffer scratch{b.scratch, g.GetBufferSize()};
+    kernel::LaunchContext ctx;
+    ctx.stream = stream_;
+    ctx.flags = flags_;
+    auto launch = [&]() {
+      if (single) {
+        if (g.HasBuffer()) dynamic_cast<kernel::SingleInputWithBufferKernel &>(*k).Run(ctx, lhs, out, scratch);
+        else dynamic_cast<kernel::SingleInputWithoutBufferKernel &>(*k).Run(ctx, lhs, out);
+      } else {
+        if (g.HasBuffer()) dynamic_cast<kernel::DoubleInputsWithBufferKernel &>(*k).Run(ctx, lhs, rhs, out, scratch);
+        else dynamic_cast<kernel::DoubleInputsWithoutBufferKernel &>(*k).Run(ctx, lhs, rhs, out);
+      }
+      Check(ctx.status, ctx.failed.c_str());
+    };
+    launch();  // warm: code object load, caches
+    constexpr int kBatch = 4, kRounds = 3;
+    double best = std::numeric_limits<double>::max();
+    for (int r = 0; r < kRounds; ++r) {
+      Check(fluidml_hip_event_record(start_, stream_), "record");
+      for (int i = 0; i < kBatch; ++i) launch();
+      Check(fluidml_hip_event_record(stop_, stream_), "record");
+      double ns = 0;
+      Check(fluidml_hip_event_elapsed_ns(start_, stop_, &ns), "elapsed");
+      best = std::min(best, ns / kBatch);
+    }
+    return std::max<size_t>(1, static_cast<size_t>(best));
+  }
+
+ private:
+  struct Buffers {
+    void *lhs = nullptr, *rhs = nullptr, *out = nullptr, *scratch = nullptr;
+  };
+  uint32_t flags_;
+  void *stream_ = nullptr, *start_ = nullptr, *stop_ = nullptr;
+  std::unordered_map<KernelEval *, Buffers> buffers_;
+};
+
+}  // namespace
+
+std::shared_ptr<CostModel> CostModel::MakeConstant() { return std::make_shared<ConstantCostModel>(); }
+std::shared_ptr<CostModel> CostModel::MakeMeasured(uint32_t ref_flags) { return std::make_shared<MeasuredCostModel>(ref_flags); }
+std::shared_ptr<CostModel> CostModel::MakeFromTable(const std::string &json_text) {
+  return std::make_shared<TableCostModel>(json_text);
+}
+
+std::shared_ptr<CostModel> CostModel::Make(context::Context &context) {
+  switch (context->cost_mode) {
+    case context::CostMode::Constant: return MakeConstant();
+    case context::CostMode::Table: {
+      std::ifstream ifs(context->cost_table_path);
+      if (!ifs) throw std::runtime_error("cannot open cost table " + context->cost_table_path);
+      std::stringstream ss;
+      ss << ifs.rdbuf();
+      return MakeFromTable(ss.str());
+    }
+    default: return MakeMeasured(context->ref_flags);
+  }
+}
+
+KernelEval::KernelEval(std::shared_ptr<kernel::KernelGenerator> generator, std::shared_ptr<CostModel> model)
+    : generator_(std::move(generator)), model_(std::move(model)) {}
+
+size_t KernelEval::Lookup(LayoutKey &&key) {
+  auto it = time_costs_.find(key);
+  if (it != time_costs_.end()) return it->second;
+  const size_t cost = model_->Cost(*this, key);
+  time_costs_.insert({std::move(key), cost});
+  return cost;
+}
+
+size_t KernelEval::GetTimeCost(const Layout &input_layout, const Layout &output_layout) {
+  if (!IsSingleInput()) throw std::logic_error("KernelEval: two layouts given to a double-input kernel");
+  return Lookup({input_layout, output_layout});
+}
+
+size_t KernelEval::GetTimeCost(const Layout &lhs_layout, const Layout &rhs_layout, const Layout &output_layout) {
+  if (IsSingleInput()) throw std::logic_error("KernelEval: three layouts given to a single-input kernel");
+  return Lookup({lhs_layout, rhs_layout, output_layout});
+}
+
+size_t KernelEval::GetShortestTimeCost() {
+  size_t shortest = std::numeric_limits<size_t>::max();
+  const auto lhs = utils::GenAllOrders(generator_->GetLhsMeta().GetShape().size());
+  const auto out = utils::GenAllOrders(generator_->GetOutputMeta().GetShape().size());
+  if (IsSingleInput()) {
+    for (const Layout &a : lhs)
+      for (const Layout &o : out) shortest = std::min(shortest, GetTimeCost(a, o));
+  } else {
+    const auto rhs = utils::GenAllOrders(generator_->GetRhsMeta().GetShape().size());
+    for (const Layout &a : lhs)
+      for (const Layout &b : rhs)
+        for (const Layout &o : out) shortest = std::min(shortest, GetTimeCost(a, b, o));
+  }
+  return shortest;
+}
+
+std::string KernelEval::ToJson() const {
+  const kernel::KernelGenerator &g = *generator_;
+  std::string s = "[";
+  bool first = true;
+  for (const auto &kv : time_costs_) {
+    s += first ? "" : ",";
+    first = false;
+    if (g.IsSingleInput()) {
+      s += "{\"input_shape\":" + JoinInts(g.GetLhsMeta().GetShape()) + ",\"output_shape\":" + JoinInts(g.GetOutputMeta().GetShape()) +
+           ",\"input_layout\":" + JoinLayout(kv.first[0]) + ",\"output_layout\":" + JoinLayout(kv.first[1]);
+    } else {
+      s += "{\"lhs_shape\":" + JoinInts(g.GetLhsMeta().GetShape()) + ",\"rhs_shape\":" + JoinInts(g.GetRhsMeta().GetShape()) +
+           ",\"output_shape\":" + JoinInts(g.GetOutputMeta().GetShape()) + ",\"lhs_layout\":" + JoinLayout(kv.first[0]) +
+           ",\"rhs_layout\":" + JoinLayout(kv.first[1]) + ",\"output_layout\":" + JoinLayout(kv.first[2]);
+    }
+    s += ",\"time_cost\":" + std::to_string(kv.second) + "}";
+  }
+  return s + "]";
+}
+
+}  // namespace evaluation
+
+namespace worker {
+
+std::shared_ptr<Evaluator> Evaluator::Make() { return std::make_shared<Evaluator>(); }
+
+void Evaluator::RegisterEval(std::string &&name, std::shared_ptr<evaluation::KernelEval> &&eval) {
+  const size_t h = eval->GetKernelGenerator().GetShapeHashCode();
+  auto range = by_shape_hash_.equal_range(h);
+  for (auto it = range.first; it != range.second; ++it) {
+    if (evals_[it->second]->GetKernelGenerator().ShapeEquals(eval->GetKernelGenerator())) {
+      by_name_.insert_or_assign(std::move(name), evals_[it->second]);  // share the first one's costs
+      return;
+    }
+  }
+  by_shape_hash_.insert({h, evals_.size()});
+  evals_.push_back(eval);
+  by_name_.insert_or_assign(std::move(name), std::move(eval));
+}
+
+evaluation::KernelEval &Evaluator::GetEval(const std::string &name) { return *by_name_.at(name); }
+
+evaluation::KernelEval &Evaluator::GetSingleInputEval(const std::string &name) {
+  evaluation::KernelEval &e = GetEval(name);
+  if (!e.IsSingleInput()) throw std::logic_error("Evaluator: " + name + " is not a single-input node");
+  return e;
+}
+
+evaluation::KernelEval &Evaluator::GetDoubleInputsEval(const std::string &name) {
+  evaluation::KernelEval &e = GetEval(name);
+  if (e.IsSingleInput()) throw std::logic_error("Evaluator: " + name + " is not a double-input node");
+  return e;
+}
+
+std::string Evaluator::ToJson() const {
+  std::map<std::string, std::string> by_kernel;  // kernel name -> comma-joined rows
+  for (const auto &eval : evals_) {
+    std::string rows = eval->ToJson();
+    rows = rows.substr(1, rows.size() - 2);  // strip [ ]
+    if (rows.empty()) continue;
+    std::string &slot = by_kernel[eval->GetKernelGenerator().GetKernelName()];
+    slot += (slot.empty() ? "" : ",") + rows;
+  }
+  std::string s = "{";
+  bool first = true;
+  for (const auto &kv : by_kernel) {
+    s += (first ? "" : ",") + json::Quote(kv.first) + ":[" + kv.second + "]";
+    first = false;
+  }
+  return s + "}";
+}
+
+}  // namespace worker
+}  // namespace fluidml

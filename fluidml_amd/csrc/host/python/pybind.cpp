@@ -1,0 +1,239 @@
+// Python module `fluidml`: the reference's surface (src/python/pybind.cpp:23-109;
+// checklist test/python/import_test.py:10-61) over the MI355X backend, plus
+// read-only inspection helpers (names starting with a lower-case verb on
+// Executor, and module functions starting with "_") that the tests and the
+// benchmark use to look at plans, layouts and per-kernel times.
+#include <pybind11/numpy.h>
+#include <pybind11/pybind11.h>
+#include <pybind11/stl.h>
+
+#include <optional>
+#include <string_view>
+
+#include "evaluation/dp.h"
+#include "evaluation/eval.h"
+#include "structure/context/context.h"
+#include "structure/flow/flow.h"
+#include "structure/graph/graph.h"
+#include "structure/memory/memory.h"
+#include "structure/tensor/meta.h"
+#include "utils/utils.h"
+#include "worker/builder.h"
+#include "worker/converter.h"
+#include "worker/executor.h"
+#include "worker/launcher.h"
+#include "worker/lower.h"
+#include "worker/parser.h"
+#include "worker/planner.h"
+#include "worker/runner.h"
+
+namespace py = pybind11;
+using namespace fluidml;
+
+namespace {
+
+py::dict StepsOf(worker::LaunchPlan &plan) {
+  py::list steps;
+  for (const worker::Step &s : plan.GetSteps()) {
+    py::dict d;
+    d["node"] = s.node->GetName();
+    d["kernel"] = s.kernel->GetKernelName();
+    d["bytes"] = s.bytes;
+    d["flops"] = s.flops;
+    d["output"] = s.out.name;
+    d["output_layout"] = s.out.layout;
+    steps.append(d);
+  }
+  py::dict out;
+  out["name"] = plan.GetName();
+  out["arena_bytes"] = plan.GetArenaBytes();
+  out["constant_bytes"] = plan.GetConstantBytes();
+  out["interface_bytes"] = plan.GetInterfaceBytes();
+  out["peak_device_bytes"] = plan.GetPeakDeviceBytes();
+  out["steps"] = steps;
+  return out;
+}
+
+std::optional<Meta> MetaOf(const std::vector<int64_t> &shape) { return Meta(Type::kFloat32, shape); }
+
+}  // namespace
+
+PYBIND11_MODULE(fluidml, m) {
+  m.doc() = "FluidML on MI355X: compile an ONNX graph into a HIP launch plan over one HBM arena and run it";
+
+  py::class_<context::Context>(m, "Context")
+      .def(py::init<>())
+      .def("make_plain_general_builder", &context::Context::MakePlainGeneralBuilder, py::arg("function_name"))
+      .def("make_dp_general_builder", &context::Context::MakeDPGeneralBuilder, py::arg("function_name"))
+      .def("make_kernel_builder", &context::Context::MakeKernelBuilder, py::arg("function_name"))
+      .def("make_plain_linear_planner", &context::Context::MakePlainLinearPlanner)
+      .def("make_plain_greedy_planner", &context::Context::MakePlainGreedyPlanner)
+      .def("make_dp_greedy_planner", &context::Context::MakeDPGreedyPlanner)
+      .def("make_lower", &context::Context::MakeLower)
+      .def("make_runner", &context::Context::MakeRunner)
+      .def("set_cost_mode",
+           [](context::Context &c, const std::string &mode) {
+             c->cost_model.reset();
+             if (mode == "constant") {
+               c->cost_mode = context::CostMode::Constant;
+             } else if (mode == "measure") {
+               c->cost_mode = context::CostMode::Measure;
+             } else {
+               c->cost_mode = context::CostMode::Table;
+               c->cost_table_path = mode;
+             }
+           },
+           py::arg("mode"), "\"measure\", \"constant\" or the path of a saved cost table")
+      .def("set_ref_flags", [](context::Context &c, uint32_t flags) { c->ref_flags = flags; }, py::arg("flags"))
+      .def("set_use_graph", [](context::Context &c, bool use) { c->use_graph = use; }, py::arg("use"))
+      .def("plan_text", [](context::Context &c) { return c->GetModule().ToText(); });
+
+  py::class_<flow::Flow, std::unique_ptr<flow::Flow>>(m, "Flow")
+      .def("node_names", [](const flow::Flow &f) {
+        std::vector<std::string> names;
+        for (const auto &n : f.GetNodes()) names.push_back(n->GetName());
+        return names;
+      });
+
+  py::class_<flow::Sequence, std::unique_ptr<flow::Sequence>>(m, "Sequence")
+      .def("node_names",
+           [](const flow::Sequence &s) {
+             std::vector<std::string> names;
+             for (const auto &n : s.GetNodes()) names.push_back(n->GetName());
+             return names;
+           })
+      .def("kernel_names",
+           [](const flow::Sequence &s) {
+             std::vector<std::string> names;
+             for (const auto &n : s.GetNodes()) names.push_back(std::string(n->GetKindName()) + "Kernel");
+             return names;
+           })
+      .def("layouts", [](const flow::Sequence &s) {
+        std::map<std::string, std::vector<size_t>> out;
+        for (const auto &r : s.GetRegions()) out[r->GetName()] = r->GetLayout();
+        return out;
+      });
+
+  py::class_<graph::Graph, std::unique_ptr<graph::Graph>>(m, "Graph");
+
+  py::class_<memory::Index, std::unique_ptr<memory::Index>>(m, "Index")
+      .def("get", &memory::Index::Get, py::arg("name"))
+      .def("get_maximum", &memory::Index::GetMaximum)
+      .def("items", [](const memory::Index &index) {
+        std::map<std::string, std::pair<size_t, size_t>> out;
+        for (const auto &kv : index.GetAll()) out[kv.first] = {std::get<0>(kv.second), std::get<1>(kv.second)};
+        return out;
+      });
+
+  py::class_<worker::Builder, std::unique_ptr<worker::Builder>>(m, "Builder");
+
+  py::class_<worker::GeneralBuilder, worker::Builder, std::unique_ptr<worker::GeneralBuilder>>(m, "GeneralBuilder")
+      .def("run", &worker::GeneralBuilder::Run, py::arg("sequence"), py::arg("index"));
+
+  py::class_<worker::KernelBuilder, worker::Builder, std::unique_ptr<worker::KernelBuilder>>(m, "KernelBuilder");
+
+  py::class_<worker::Converter, std::unique_ptr<worker::Converter>>(m, "Converter")
+      .def("run", &worker::Converter::Run, py::arg("graph"))
+      .def_static("make", &worker::Converter::Make);
+
+  py::class_<worker::Executor, std::unique_ptr<worker::Executor>>(m, "Executor")
+      .def("compile",
+           py::overload_cast<std::string_view, std::optional<std::string_view>, std::optional<std::string_view>,
+                             std::optional<std::string_view>>(&worker::Executor::Compile),
+           py::arg("input"), py::arg("mlir") = std::nullopt, py::arg("llvm") = std::nullopt,
+           py::arg("json") = std::nullopt)
+      .def("invoke",
+           py::overload_cast<const std::unordered_map<std::string, py::array> &>(&worker::Executor::Invoke),
+           py::arg("args"))
+      .def_static("make_plain_linear", &worker::Executor::MakePlainLinear, py::arg("name"), py::arg("epoch") = 1)
+      .def_static("make_plain_greedy", &worker::Executor::MakePlainGreedy, py::arg("name"), py::arg("epoch") = 1)
+      .def_static("make_dp_greedy", &worker::Executor::MakeDPGreedy, py::arg("name"), py::arg("epoch") = 1)
+      // ---- inspection (not in the reference) ----
+      .def("context", [](worker::Executor &e) { return e.GetContext(); })
+      .def("plan", [](worker::Executor &e) { return StepsOf(e.GetContext()->GetModule()); },
+           "launch plan summary: arena/constant/interface bytes and one dict per step")
+      .def("plan_text", [](worker::Executor &e) { return e.GetContext()->GetModule().ToText(); })
+      .def("profile",
+           [](worker::Executor &e, size_t warmup, size_t iters) {
+             py::list out;
+             for (const worker::StepTime &t : e.GetContext()->GetModule().Profile(warmup, iters)) {
+               py::dict d;
+               d["node"] = t.node;
+               d["kernel"] = t.kernel;
+               d["ns"] = t.ns;
+               d["bytes"] = t.bytes;
+               d["flops"] = t.flops;
+               out.append(d);
+             }
+             return out;
+           },
+           py::arg("warmup") = 3, py::arg("iters") = 20, "median hipEvent nanoseconds of every step")
+      .def("time_replay_ns",
+           [](worker::Executor &e, size_t warmup, size_t iters) {
+             return e.GetContext()->GetModule().TimeReplayNs(warmup, iters);
+           },
+           py::arg("warmup") = 3, py::arg("iters") = 20,
+           "mean device nanoseconds of one replay of the whole plan (inputs resident in HBM)")
+      .def("materialize", [](worker::Executor &e) { e.GetContext()->GetModule().Materialize(); });
+
+  py::class_<worker::Lower, std::unique_ptr<worker::Lower>>(m, "Lower").def("run", &worker::Lower::Run);
+
+  py::class_<worker::Parser, std::unique_ptr<worker::Parser>>(m, "Parser")
+      .def("run", py::overload_cast<std::string_view>(&worker::Parser::Run), py::arg("input"))
+      .def_static("make", &worker::Parser::Make);
+
+  py::class_<worker::Planner, std::unique_ptr<worker::Planner>>(m, "Planner")
+      .def("run", &worker::Planner::Run, py::arg("flow"));
+
+  py::class_<worker::Runner, std::unique_ptr<worker::Runner>>(m, "Runner")
+      .def("run",
+           py::overload_cast<const std::unordered_map<std::string, py::array> &, size_t>(&worker::Runner::Run),
+           py::arg("args"), py::arg("epoch") = 1);
+
+  // ---- module-level helpers for tests of the planning core ----
+  m.def(
+      "_plan_memory",
+      [](int kind, const std::vector<size_t> &starts, const std::vector<size_t> &ends, const std::vector<size_t> &sizes) {
+        std::unique_ptr<memory::Infos> infos;
+        std::unique_ptr<memory::Plan> plan;
+        if (kind == 0) {
+          infos = std::make_unique<memory::PlainInfos>();
+          plan = std::make_unique<memory::LinearPlan>();
+        } else {
+          infos = std::make_unique<memory::GreedyInfos>();
+          plan = std::make_unique<memory::GreedyPlan>();
+        }
+        for (size_t i = 0; i < sizes.size(); ++i) infos->Push(memory::Info("t" + std::to_string(i), starts[i], ends[i], sizes[i]));
+        memory::Index index = plan->Run(*infos);
+        std::vector<size_t> offsets;
+        for (size_t i = 0; i < sizes.size(); ++i) offsets.push_back(index.Get("t" + std::to_string(i)));
+        return std::make_pair(offsets, index.GetMaximum());
+      },
+      py::arg("kind"), py::arg("starts"), py::arg("ends"), py::arg("sizes"),
+      "kind 0 = PlainInfos+LinearPlan, 1 = GreedyInfos+GreedyPlan; tensors are named t0, t1, ... in push order");
+  m.def("_gen_all_orders", &utils::GenAllOrders);
+  m.def("_gen_all_indices_in_order", &utils::GenAllIndicesInOrder);
+  m.def("_gen_physical_shape", &utils::GenPhysicalShape);
+  m.def("_gen_strides", py::overload_cast<const std::vector<int64_t> &>(&utils::GenStrides));
+  m.def("_gen_strides_layout",
+        py::overload_cast<const std::vector<int64_t> &, const std::vector<size_t> &>(&utils::GenStrides));
+  m.def("_broadcast_shape", [](const std::vector<int64_t> &a, const std::vector<int64_t> &b) {
+    std::optional<Meta> r = BroadcastShape(*MetaOf(a), *MetaOf(b), Type::kFloat32);
+    return r ? std::optional<std::vector<int64_t>>(r->GetShape()) : std::nullopt;
+  });
+  m.def("_broadcast_matmul_shape", [](const std::vector<int64_t> &a, const std::vector<int64_t> &b) {
+    std::optional<Meta> r = BroadcastMatMulShape(*MetaOf(a), *MetaOf(b), Type::kFloat32);
+    return r ? std::optional<std::vector<int64_t>>(r->GetShape()) : std::nullopt;
+  });
+  m.def(
+      "_dp_layouts",
+      [](const flow::Flow &flow, const std::string &cost) {
+        std::shared_ptr<evaluation::CostModel> model = cost == "constant" ? evaluation::CostModel::MakeConstant()
+                                                                          : evaluation::CostModel::MakeFromTable(cost);
+        auto table = evaluation::DynamicProgrammingTable::Make(model);
+        evaluation::DynamicProgrammingPlan plan = table->Run(flow);
+        return std::map<std::string, std::vector<size_t>>(plan.GetAll().begin(), plan.GetAll().end());
+      },
+      py::arg("flow"), py::arg("cost") = "constant",
+      "layout DP on a flow with constant costs or with the JSON text of a cost table");
+}

@@ -1,0 +1,118 @@
+// Shared state of one compilation: the launch plan ("module"), its function
+// attributes and the options of this backend (reference
+// include/structure/context/{context,attr}.h).  `Context` is a cheap handle;
+// every worker made from it sees the same ContextImpl.
+#ifndef FLUIDML_AMD_HOST_STRUCTURE_CONTEXT_CONTEXT_H_
+#define FLUIDML_AMD_HOST_STRUCTURE_CONTEXT_CONTEXT_H_
+
+#include <memory>
+#include <optional>
+#include <ostream>
+#include <string>
+#include <vector>
+
+#include "structure/tensor/meta.h"
+
+namespace fluidml {
+namespace worker {
+class GeneralBuilder;
+class KernelBuilder;
+class Planner;
+class Lower;
+class Runner;
+class LaunchPlan;
+}  // namespace worker
+namespace evaluation {
+class DynamicProgrammingTable;
+class CostModel;
+}  // namespace evaluation
+
+namespace context {
+
+// One interface tensor of the compiled function (reference attr.h:13-36).
+class ArgumentAttr {
+ public:
+  enum class Type { Input, Output };
+  ArgumentAttr(Type type, std::string &&name, Meta &&meta) : type_(type), name_(std::move(name)), meta_(std::move(meta)) {}
+  Type GetType() const { return type_; }
+  const std::string &GetName() const { return name_; }
+  const Meta &GetMeta() const { return meta_; }
+
+ private:
+  Type type_;
+  std::string name_;
+  Meta meta_;
+};
+
+// Name, arena bytes and argument list of the compiled function (reference attr.h:38-58).
+class FuncAttr {
+ public:
+  FuncAttr(std::string &&name, size_t buffer) : name_(std::move(name)), buffer_(buffer) {}
+  const std::string &GetName() const { return name_; }
+  size_t GetBuffer() const { return buffer_; }
+  const std::vector<ArgumentAttr> &GetArguments() const { return arguments_; }
+  void PutArgument(ArgumentAttr &&arg) { arguments_.push_back(std::move(arg)); }
+
+ private:
+  std::string name_;
+  size_t buffer_;
+  std::vector<ArgumentAttr> arguments_;
+};
+
+// How the layout DP obtains kernel costs.
+enum class CostMode {
+  Measure,   // time every (kernel, layouts) on the GPU with hipEvents
+  Constant,  // every cost is 1 (the reference's DP_DEBUG build, eval.cpp:73-76)
+  Table      // read costs from a JSON cost table written by an earlier compile
+};
+
+class ContextImpl {
+ public:
+  ContextImpl();
+  ~ContextImpl();
+  worker::LaunchPlan &GetModule();
+  bool HasModule() const { return module_ != nullptr; }
+  void SetModule(std::unique_ptr<worker::LaunchPlan> &&module);
+  FuncAttr &GetFuncAttr();
+  void SetFuncAttr(FuncAttr &&attr);
+
+  // FL_REF_* literal-reference switches (env FLUIDML_REF_QUIRKS=<int>, default 0)
+  uint32_t ref_flags = 0;
+  // replay the plan as a captured hipGraph (env FLUIDML_HIP_GRAPH=0 disables)
+  bool use_graph = true;
+  // cost source of the layout DP (env FLUIDML_DP_COST=measure|constant|<path to table json>)
+  CostMode cost_mode = CostMode::Measure;
+  std::string cost_table_path;
+  std::shared_ptr<evaluation::CostModel> cost_model;  // created on first use
+
+ private:
+  std::unique_ptr<worker::LaunchPlan> module_;
+  std::optional<FuncAttr> func_attr_;
+};
+
+class Context {
+ public:
+  Context();
+  ContextImpl &operator*() { return *impl_; }
+  ContextImpl *operator->() { return impl_.get(); }
+  std::unique_ptr<evaluation::DynamicProgrammingTable> MakeDynamicProgrammingTable();
+  std::unique_ptr<worker::GeneralBuilder> MakePlainGeneralBuilder(std::string &&function_name);
+  std::unique_ptr<worker::GeneralBuilder> MakeDPGeneralBuilder(std::string &&function_name);
+  std::unique_ptr<worker::KernelBuilder> MakeKernelBuilder(std::string &&function_name);
+  std::unique_ptr<worker::Planner> MakePlainLinearPlanner();
+  std::unique_ptr<worker::Planner> MakePlainGreedyPlanner();
+  std::unique_ptr<worker::Planner> MakeDPGreedyPlanner();
+  std::unique_ptr<worker::Lower> MakeLower();
+  std::unique_ptr<worker::Runner> MakeRunner();
+  // textual dump of the launch plan (what `*mlir << context_` prints in the
+  // reference, executor.cpp:106-112)
+  friend std::ostream &operator<<(std::ostream &os, Context &context);
+
+ private:
+  std::shared_ptr<ContextImpl> impl_;
+};
+
+}  // namespace context
+}  // namespace fluidml
+
+#endif

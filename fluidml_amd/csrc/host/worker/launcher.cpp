@@ -1,0 +1,309 @@
+#include "worker/launcher.h"
+
+#include <algorithm>
+#include <chrono>
+#include <sstream>
+#include <stdexcept>
+
+#include "fluidml_hip.h"
+
+namespace fluidml {
+namespace worker {
+
+namespace {
+void Check(int rc, const char *what) {
+  if (rc != 0) throw std::runtime_error(std::string(what) + ": " + fluidml_hip_error_string(rc));
+}
+
+kernel::TensorView ViewOf(void *base, const Operand &op) { return kernel::TensorView(base, op.meta, op.layout); }
+
+const char *SpaceName(Operand::Space s) {
+  switch (s) {
+    case Operand::Space::Arena: return "arena";
+    case Operand::Space::Interface: return "interface";
+    case Operand::Space::Constant: return "constant";
+    default: return "private";
+  }
+}
+}  // namespace
+
+LaunchPlan::LaunchPlan(std::string &&name, size_t arena_bytes) : name_(std::move(name)), arena_bytes_(arena_bytes) {}
+
+LaunchPlan::~LaunchPlan() {
+  if (graph_) fluidml_hip_graph_destroy(graph_);
+  for (auto &kv : constants_) fluidml_hip_free(kv.second.device);
+  for (auto &kv : privates_) fluidml_hip_free(kv.second.device);
+  for (auto &kv : interfaces_) fluidml_hip_free(kv.second.device);
+  if (arena_) fluidml_hip_arena_destroy(arena_);
+  if (stream_) fluidml_hip_stream_destroy(stream_);
+}
+
+void LaunchPlan::AddArgument(Argument &&arg) {
+  interfaces_[arg.name].bytes = arg.meta.GetSize();
+  arguments_.push_back(std::move(arg));
+}
+
+void LaunchPlan::AddConstant(const std::string &name, const Tensor &tensor, const std::vector<size_t> &layout) {
+  constants_.insert({name, ConstantSlot{tensor, layout, nullptr}});
+}
+
+void LaunchPlan::AddPrivate(const std::string &name, size_t bytes) { privates_[name].bytes = bytes; }
+
+void LaunchPlan::AddStep(Step &&step) { steps_.push_back(std::move(step)); }
+
+size_t LaunchPlan::GetConstantBytes() const {
+  size_t n = 0;
+  for (const auto &kv : constants_) n += kv.second.tensor.GetMeta().GetSize();
+  for (const Step &s : steps_) n += s.kernel->GetConstantBytes();
+  return n;
+}
+
+size_t LaunchPlan::GetInterfaceBytes() const {
+  size_t n = 0;
+  for (const auto &kv : interfaces_) n += kv.second.bytes;
+  return n;
+}
+
+void LaunchPlan::Validate() const {
+  auto check_operand = [&](const Step &s, const Operand &op) {
+    switch (op.space) {
+      case Operand::Space::Arena:
+        if (op.offset + op.meta.GetSize() > arena_bytes_) throw std::logic_error("plan: " + s.node->GetName() + " operand " + op.name + " leaves the arena");
+        break;
+      case Operand::Space::Interface:
+        if (!interfaces_.count(op.name)) throw std::logic_error("plan: unknown interface tensor " + op.name);
+        break;
+      case Operand::Space::Constant:
+        if (!constants_.count(op.name)) throw std::logic_error("plan: unknown constant " + op.name);
+        break;
+      case Operand::Space::Private:
+        if (!privates_.count(op.name)) throw std::logic_error("plan: unknown private tensor " + op.name);
+        break;
+    }
+  };
+  for (const Step &s : steps_) {
+    if (!s.kernel) throw std::logic_error("plan: " + s.node->GetName() + " has no kernel");
+    check_operand(s, s.in0);
+    if (s.node->IsDoubleInputs()) check_operand(s, s.in1);
+    check_operand(s, s.out);
+    if (s.has_buffer && s.buffer_offset + s.buffer_bytes > arena_bytes_) {
+      throw std::logic_error("plan: scratch of " + s.node->GetName() + " leaves the arena");
+    }
+  }
+}
+
+std::string LaunchPlan::ToText() const {
+  std::ostringstream os;
+  auto operand = [&](const Operand &op) {
+    os << op.name << "@" << SpaceName(op.space);
+    if (op.space == Operand::Space::Arena) os << "+" << op.offset;
+    os << ":" << GetStringFromType(op.meta.GetType()) << "[";
+    for (size_t i = 0; i < op.meta.GetShape().size(); ++i) os << (i ? "," : "") << op.meta.GetShape()[i];
+    os << "]/(";
+    for (size_t i = 0; i < op.layout.size(); ++i) os << (i ? "," : "") << op.layout[i];
+    os << ")";
+  };
+  os << "launch_plan @" << name_ << " arena_bytes=" << arena_bytes_ << " constant_bytes=" << GetConstantBytes()
+     << " interface_bytes=" << GetInterfaceBytes() << "\n";
+  for (const Argument &a : arguments_) {
+    os << "  arg " << (a.type == Argument::Type::Input ? "in  " : "out ") << a.name << " bytes=" << a.meta.GetSize() << "\n";
+  }
+  for (size_t i = 0; i < steps_.size(); ++i) {
+    const Step &s = steps_[i];
+    os << "  %" << i << " " << s.kernel->GetKernelName() << " \"" << s.node->GetName() << "\" (";
+    operand(s.in0);
+    if (s.node->IsDoubleInputs()) {
+      os << ", ";
+      operand(s.in1);
+    }
+    os << ") -> ";
+    operand(s.out);
+    if (s.has_buffer) os << " scratch@arena+" << s.buffer_offset << ":" << s.buffer_bytes;
+    os << "\n";
+  }
+  return os.str();
+}
+
+void LaunchPlan::Materialize() {
+  if (arena_ != nullptr) return;
+  Validate();
+  Check(fluidml_hip_stream_create(&stream_), "creating the plan's stream");
+  for (auto &kv : constants_) {
+    const std::vector<uint8_t> bytes = kv.second.tensor.Pack(kv.second.layout);
+    Check(fluidml_hip_upload_constant(bytes.data(), bytes.size(), &kv.second.device), "uploading a constant region");
+  }
+  for (auto *slots : {&privates_, &interfaces_}) {
+    for (auto &kv : *slots) Check(fluidml_hip_arena_create(kv.second.bytes, &kv.second.device), "allocating a device buffer");
+  }
+  for (Step &s : steps_) s.kernel->Prepare();
+  Check(fluidml_hip_arena_create(arena_bytes_, &arena_), "allocating the arena");
+}
+
+void *LaunchPlan::Resolve(const Operand &op) const {
+  switch (op.space) {
+    case Operand::Space::Arena: return static_cast<char *>(arena_) + op.offset;
+    case Operand::Space::Interface: return interfaces_.at(op.name).device;
+    case Operand::Space::Constant: return constants_.at(op.name).device;
+    default: return privates_.at(op.name).device;
+  }
+}
+
+void *LaunchPlan::GetDeviceAddress(const std::string &name) const {
+  auto it = interfaces_.find(name);
+  if (it != interfaces_.end()) return it->second.device;
+  auto ct = constants_.find(name);
+  if (ct != constants_.end()) return ct->second.device;
+  return nullptr;
+}
+
+void LaunchPlan::LaunchAll(kernel::LaunchContext &ctx) const {
+  for (const Step &s : steps_) {
+    const kernel::TensorView in0 = ViewOf(Resolve(s.in0), s.in0), out = ViewOf(Resolve(s.out), s.out);
+    const kernel::Buffer buffer{s.has_buffer ? static_cast<char *>(arena_) + s.buffer_offset : nullptr, s.buffer_bytes};
+    kernel::Kernel *k = s.kernel.get();
+    if (s.node->IsSingleInput()) {
+      if (s.has_buffer) dynamic_cast<kernel::SingleInputWithBufferKernel &>(*k).Run(ctx, in0, out, buffer);
+      else dynamic_cast<kernel::SingleInputWithoutBufferKernel &>(*k).Run(ctx, in0, out);
+    } else {
+      const kernel::TensorView in1 = ViewOf(Resolve(s.in1), s.in1);
+      if (s.has_buffer) dynamic_cast<kernel::DoubleInputsWithBufferKernel &>(*k).Run(ctx, in0, in1, out, buffer);
+      else dynamic_cast<kernel::DoubleInputsWithoutBufferKernel &>(*k).Run(ctx, in0, in1, out);
+    }
+    if (ctx.status != 0) {
+      throw std::runtime_error("launching " + ctx.failed + " for node '" + s.node->GetName() + "': " +
+                               fluidml_hip_error_string(ctx.status));
+    }
+  }
+}
+
+// One replay of the whole sequence on the plan's stream: the captured graph
+// when capture is enabled (recorded on first use), plain launches otherwise.
+void LaunchPlan::Replay(kernel::LaunchContext &ctx) {
+  if (!use_graph_) {
+    LaunchAll(ctx);
+    return;
+  }
+  if (graph_ == nullptr) {
+    Check(fluidml_hip_graph_begin_capture(stream_), "starting launch-plan capture");
+    try {
+      LaunchAll(ctx);
+    } catch (...) {
+      void *discard = nullptr;
+      fluidml_hip_graph_end_capture(stream_, &discard);
+      if (discard) fluidml_hip_graph_destroy(discard);
+      throw;
+    }
+    Check(fluidml_hip_graph_end_capture(stream_, &graph_), "finishing launch-plan capture");
+  }
+  Check(fluidml_hip_graph_launch(graph_, stream_), "launching the captured plan");
+}
+
+size_t LaunchPlan::Run(const std::unordered_map<std::string, void *> &args, size_t epoch) {
+  if (epoch == 0) epoch = 1;
+  Materialize();
+  // the literal LayerNorm mode reads its scratch before writing it: give every
+  // call the zero-filled arena the reference allocates per Invoke (runner.cpp:87-88)
+  if (flags_ & FL_REF_LN_STALE_SCRATCH) Check(fluidml_hip_arena_zero(arena_, arena_bytes_, stream_), "zeroing the arena");
+  for (const Argument &a : arguments_) {
+    void *host = args.at(a.name);
+    if (a.type == Argument::Type::Input) {
+      Check(fluidml_hip_memcpy_h2d(interfaces_.at(a.name).device, host, a.meta.GetSize(), stream_), "copying an input to HBM");
+    }
+  }
+  Check(fluidml_hip_stream_synchronize(stream_), "waiting for input copies");
+  kernel::LaunchContext ctx;
+  ctx.stream = stream_;
+  ctx.flags = flags_;
+  if (use_graph_ && graph_ == nullptr) {  // record outside the timed region
+    Replay(ctx);
+    Check(fluidml_hip_stream_synchronize(stream_), "waiting for the first replay");
+  }
+  const auto t0 = std::chrono::high_resolution_clock::now();
+  for (size_t e = 0; e < epoch; ++e) Replay(ctx);
+  Check(fluidml_hip_stream_synchronize(stream_), "waiting for the replays");
+  const auto t1 = std::chrono::high_resolution_clock::now();
+  for (const Argument &a : arguments_) {
+    if (a.type == Argument::Type::Output) {
+      Check(fluidml_hip_memcpy_d2h(args.at(a.name), interfaces_.at(a.name).device, a.meta.GetSize(), stream_), "copying an output to the host");
+    }
+  }
+  Check(fluidml_hip_stream_synchronize(stream_), "waiting for output copies");
+  return static_cast<size_t>(std::chrono::duration_cast<std::chrono::nanoseconds>(t1 - t0).count()) / epoch;
+}
+
+double LaunchPlan::TimeReplayNs(size_t warmup, size_t iters) {
+  Materialize();
+  kernel::LaunchContext ctx;
+  ctx.stream = stream_;
+  ctx.flags = flags_;
+  for (size_t i = 0; i < warmup + 1; ++i) Replay(ctx);
+  void *e0 = nullptr, *e1 = nullptr;
+  Check(fluidml_hip_event_create(&e0), "event");
+  Check(fluidml_hip_event_create(&e1), "event");
+  Check(fluidml_hip_event_record(e0, stream_), "event record");
+  for (size_t i = 0; i < iters; ++i) Replay(ctx);
+  Check(fluidml_hip_event_record(e1, stream_), "event record");
+  double ns = 0;
+  Check(fluidml_hip_event_elapsed_ns(e0, e1, &ns), "event elapsed");
+  fluidml_hip_event_destroy(e0);
+  fluidml_hip_event_destroy(e1);
+  return ns / static_cast<double>(std::max<size_t>(iters, 1));
+}
+
+std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
+  Materialize();
+  kernel::LaunchContext ctx;
+  ctx.stream = stream_;
+  ctx.flags = flags_;
+  const bool saved = use_graph_;
+  use_graph_ = false;
+  std::vector<std::vector<double>> samples(steps_.size());
+  std::vector<void *> events(steps_.size() + 1, nullptr);
+  for (void *&e : events) Check(fluidml_hip_event_create(&e), "event");
+  for (size_t it = 0; it < warmup + iters; ++it) {
+    Check(fluidml_hip_event_record(events[0], stream_), "event record");
+    for (size_t i = 0; i < steps_.size(); ++i) {
+      // launch one step at a time between event pairs
+      const Step &s = steps_[i];
+      const kernel::TensorView in0 = ViewOf(Resolve(s.in0), s.in0), out = ViewOf(Resolve(s.out), s.out);
+      const kernel::Buffer buffer{s.has_buffer ? static_cast<char *>(arena_) + s.buffer_offset : nullptr, s.buffer_bytes};
+      kernel::Kernel *k = s.kernel.get();
+      if (s.node->IsSingleInput()) {
+        if (s.has_buffer) dynamic_cast<kernel::SingleInputWithBufferKernel &>(*k).Run(ctx, in0, out, buffer);
+        else dynamic_cast<kernel::SingleInputWithoutBufferKernel &>(*k).Run(ctx, in0, out);
+      } else {
+        const kernel::TensorView in1 = ViewOf(Resolve(s.in1), s.in1);
+        if (s.has_buffer) dynamic_cast<kernel::DoubleInputsWithBufferKernel &>(*k).Run(ctx, in0, in1, out, buffer);
+        else dynamic_cast<kernel::DoubleInputsWithoutBufferKernel &>(*k).Run(ctx, in0, in1, out);
+      }
+      Check(ctx.status, "profiling launch");
+      Check(fluidml_hip_event_record(events[i + 1], stream_), "event record");
+    }
+    Check(fluidml_hip_stream_synchronize(stream_), "profiling sync");
+    if (it >= warmup) {
+      for (size_t i = 0; i < steps_.size(); ++i) {
+        double ns = 0;
+        Check(fluidml_hip_event_elapsed_ns(events[i], events[i + 1], &ns), "event elapsed");
+        samples[i].push_back(ns);
+      }
+    }
+  }
+  for (void *e : events) fluidml_hip_event_destroy(e);
+  use_graph_ = saved;
+  std::vector<StepTime> out;
+  for (size_t i = 0; i < steps_.size(); ++i) {
+    std::vector<double> &v = samples[i];
+    std::sort(v.begin(), v.end());
+    StepTime t;
+    t.node = steps_[i].node->GetName();
+    t.kernel = steps_[i].kernel->GetKernelName();
+    t.ns = v.empty() ? 0 : v[v.size() / 2];
+    t.bytes = steps_[i].bytes;
+    t.flops = steps_[i].flops;
+    out.push_back(std::move(t));
+  }
+  return out;
+}
+
+}  // namespace worker
+}  // namespace fluidml

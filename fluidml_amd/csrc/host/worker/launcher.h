@@ -1,0 +1,139 @@
+// The compiled artefact of this backend: an ordered list of kernel launches
+// over one HBM arena.  It stands where the reference keeps an MLIR module plus
+// a JIT engine (src/structure/context/context.cpp:152-166): GeneralBuilder
+// fills it (reference builder.cpp:149-394 lays memref views over the arena
+// argument), Lower validates it, Runner materialises it on the device and
+// replays it.
+#ifndef FLUIDML_AMD_HOST_WORKER_LAUNCHER_H_
+#define FLUIDML_AMD_HOST_WORKER_LAUNCHER_H_
+
+#include <map>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "structure/flow/flow.h"
+#include "structure/kernel/kernel.h"
+
+namespace fluidml {
+namespace worker {
+
+// Where an operand of a step lives.
+struct Operand {
+  enum class Space {
+    Arena,      // inner region: arena base + offset from the memory plan
+    Interface,  // graph input/output: device staging buffer (GeneralBuilder gives it the identity layout)
+    Constant,   // constant region: its own HBM allocation, region layout applied
+    Private     // inner region no Memory edge uses: its own HBM allocation
+  };
+  Space space = Space::Arena;
+  std::string name;
+  size_t offset = 0;  // Arena only
+  Meta meta{Type::kUnknown, std::vector<int64_t>{}};
+  std::vector<size_t> layout;
+};
+
+struct Step {
+  std::shared_ptr<flow::Node> node;
+  std::shared_ptr<kernel::Kernel> kernel;
+  Operand in0, in1, out;  // in1 unused for single-input nodes
+  bool has_buffer = false;
+  size_t buffer_offset = 0, buffer_bytes = 0;
+  // algorithmic work of the step: bytes = unique operand bytes + output bytes
+  // (scratch excluded), flops = 2*MACs for contractions, 0 otherwise
+  double bytes = 0, flops = 0;
+};
+
+struct Argument {
+  enum class Type { Input, Output };
+  Type type;
+  std::string name;
+  Meta meta;
+};
+
+struct StepTime {
+  std::string node, kernel;
+  double ns = 0, bytes = 0, flops = 0;
+};
+
+class LaunchPlan {
+ public:
+  LaunchPlan(std::string &&name, size_t arena_bytes);
+  ~LaunchPlan();
+  LaunchPlan(const LaunchPlan &) = delete;
+
+  // ---- filled by the builders (host only, no device needed) ----
+  void AddArgument(Argument &&arg);
+  void AddConstant(const std::string &name, const Tensor &tensor, const std::vector<size_t> &layout);
+  void AddPrivate(const std::string &name, size_t bytes);
+  void AddStep(Step &&step);
+
+  const std::string &GetName() const { return name_; }
+  size_t GetArenaBytes() const { return arena_bytes_; }
+  size_t GetConstantBytes() const;   // constant regions + constants kernels own
+  size_t GetInterfaceBytes() const;  // device staging of graph inputs and outputs
+  size_t GetPeakDeviceBytes() const { return arena_bytes_ + GetConstantBytes() + GetInterfaceBytes(); }
+  const std::vector<Step> &GetSteps() const { return steps_; }
+  const std::vector<Argument> &GetArguments() const { return arguments_; }
+  // Every arena operand and scratch buffer lies inside [0, arena_bytes); every
+  // named constant / interface / private operand exists. Throws std::logic_error otherwise.
+  void Validate() const;
+  // Human-readable listing (what the `mlir` / `llvm` sinks of Executor::Compile receive).
+  std::string ToText() const;
+
+  // ---- device side ----
+  // Allocates the arena, uploads constants, allocates interface staging and
+  // prepares kernels. Idempotent. Throws std::runtime_error on HIP errors.
+  void Materialize();
+  bool IsMaterialized() const { return arena_ != nullptr; }
+  // H2D inputs, `epoch` replays of all steps, D2H outputs; returns mean wall
+  // nanoseconds per replay of the launch-and-wait loop alone (reference
+  // runner.cpp:101-119). `args` maps every argument name to a host buffer of
+  // exactly Meta::GetSize() bytes; a missing name throws std::out_of_range
+  // (reference runner.cpp:70).
+  size_t Run(const std::unordered_map<std::string, void *> &args, size_t epoch);
+  // hipEvent time of every step, median of `iters` runs after `warmup`.
+  std::vector<StepTime> Profile(size_t warmup, size_t iters);
+  // mean device time of one whole replay measured with events on the plan's stream
+  double TimeReplayNs(size_t warmup, size_t iters);
+
+  void SetFlags(uint32_t flags) { flags_ = flags; }
+  uint32_t GetFlags() const { return flags_; }
+  void SetUseGraph(bool use) { use_graph_ = use; }
+  // device address of a named interface / constant operand (tests)
+  void *GetDeviceAddress(const std::string &name) const;
+  void *GetArenaBase() const { return arena_; }
+  void *GetStream() const { return stream_; }
+
+ private:
+  struct ConstantSlot {
+    Tensor tensor;
+    std::vector<size_t> layout;
+    void *device = nullptr;
+  };
+  struct RawSlot {
+    size_t bytes = 0;
+    void *device = nullptr;
+  };
+  void *Resolve(const Operand &op) const;
+  void LaunchAll(kernel::LaunchContext &ctx) const;
+  void Replay(kernel::LaunchContext &ctx);
+
+  std::string name_;
+  size_t arena_bytes_;
+  std::vector<Argument> arguments_;
+  std::vector<Step> steps_;
+  std::map<std::string, ConstantSlot> constants_;
+  std::map<std::string, RawSlot> privates_, interfaces_;
+  uint32_t flags_ = 0;
+  bool use_graph_ = true;
+  void *arena_ = nullptr;
+  void *stream_ = nullptr;
+  void *graph_ = nullptr;
+};
+
+}  // namespace worker
+}  // namespace fluidml
+
+#endif

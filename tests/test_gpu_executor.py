@@ -1,0 +1,120 @@
+"""Whole-graph parity on the GPU: Executor.compile + invoke (the reference's entry points,
+include/worker/executor.h:18-36) against the oracle's graph runner on the same seeded weights
+and inputs, for the three executor flavours, with and without launch-plan capture, and with
+DP-chosen (non-identity) layouts -- which the reference itself never tests numerically
+(test/python/node/node_test.py only drives make_plain_greedy)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+from oracle import graph_runner
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _mods():
+    from fluidml_amd import fluidml, models
+
+    return fluidml, models
+
+
+def announce(*what):
+    print("[case]", *what, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def tiny_bert(tmp_path_factory):
+    fluidml, models = _mods()
+    net = models.bert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32, seed=5)
+    path = str(tmp_path_factory.mktemp("onnx") / "tiny_bert.onnx")
+    net.save(path)
+    feeds = models.bert_inputs(16, 100, seed=6)
+    feeds["attention_mask"][0, 12:] = 0.0  # exercise the additive mask
+    want = graph_runner.run_graph(net, feeds)
+    return net, path, feeds, want
+
+
+def _invoke(ex, net, feeds):
+    args = {k: np.ascontiguousarray(v) for k, v in feeds.items()}
+    outs = {v.name: np.full(v.shape, np.nan, dtype=v.dtype) for v in net.outputs}
+    args.update(outs)
+    ns = ex.invoke(args)
+    assert ns > 0
+    return outs
+
+
+@pytest.mark.parametrize("flavour", ["plain_linear", "plain_greedy", "dp_greedy"])
+@pytest.mark.parametrize("graph", [False, True], ids=["launches", "captured"])
+def test_tiny_bert_matches_oracle(device, tiny_bert, flavour, graph, monkeypatch):
+    fluidml, _ = _mods()
+    net, path, feeds, want = tiny_bert
+    monkeypatch.setenv("FLUIDML_HIP_GRAPH", "1" if graph else "0")
+    monkeypatch.setenv("FLUIDML_DP_COST", "constant")  # every tensor gets the reversed layout
+    announce("tiny bert", flavour, "graph" if graph else "launches")
+    ex = getattr(fluidml.Executor, "make_" + flavour)("tiny_" + flavour, 3)
+    ex.compile(path)
+    if flavour == "dp_greedy":
+        layouts = {s["output"]: s["output_layout"] for s in ex.plan()["steps"]}
+        assert any(l != sorted(l) for l in layouts.values()), "DP plan should use non-identity layouts"
+    for _ in range(2):  # second call replays the captured plan
+        got = _invoke(ex, net, feeds)
+        for name, ref in want.items():
+            assert_close(got[name], ref, what=f"{flavour} {name}")
+
+
+def test_dp_measured_layouts_match_oracle(device, tiny_bert, monkeypatch, tmp_path):
+    """Layouts picked from hipEvent-measured costs, then replayed from the saved cost table."""
+    fluidml, _ = _mods()
+    net, path, feeds, want = tiny_bert
+    monkeypatch.setenv("FLUIDML_DP_COST", "measure")
+    announce("tiny bert dp measured")
+    ex = fluidml.Executor.make_dp_greedy("tiny_dp_measured")
+    json_path = str(tmp_path / "dp.json")
+    ex.compile(path, None, None, json_path)
+    got = _invoke(ex, net, feeds)
+    for name, ref in want.items():
+        assert_close(got[name], ref, what=f"dp measured {name}")
+    first = {s["output"]: s["output_layout"] for s in ex.plan()["steps"]}
+    # same cost table -> same layouts
+    monkeypatch.setenv("FLUIDML_DP_COST", json_path)
+    announce("tiny bert dp replay from table")
+    ex2 = fluidml.Executor.make_dp_greedy("tiny_dp_replay")
+    ex2.compile(path)
+    second = {s["output"]: s["output_layout"] for s in ex2.plan()["steps"]}
+    assert first == second
+    got = _invoke(ex2, net, feeds)
+    for name, ref in want.items():
+        assert_close(got[name], ref, what=f"dp replay {name}")
+
+
+def test_invoke_errors(device, tiny_bert):
+    fluidml, _ = _mods()
+    net, path, feeds, _ = tiny_bert
+    ex = fluidml.Executor.make_plain_greedy("tiny_err")
+    ex.compile(path)
+    args = {k: v for k, v in feeds.items()}
+    with pytest.raises((KeyError, IndexError)):  # missing output name: std::out_of_range (reference runner.cpp:70)
+        ex.invoke(args)
+    args[net.outputs[0].name] = np.zeros((3,), np.float32)
+    with pytest.raises(ValueError):
+        ex.invoke(args)
+
+
+def test_profile_and_accounting(device, tiny_bert):
+    fluidml, _ = _mods()
+    net, path, feeds, _ = tiny_bert
+    ex = fluidml.Executor.make_plain_greedy("tiny_prof")
+    ex.compile(path)
+    plan = ex.plan()
+    assert plan["peak_device_bytes"] == plan["arena_bytes"] + plan["constant_bytes"] + plan["interface_bytes"]
+    _invoke(ex, net, feeds)
+    times = ex.profile(2, 5)
+    assert len(times) == len(net.nodes)
+    assert all(t["ns"] > 0 for t in times)
+    mm = [t for t in times if t["kernel"] == "MatMulKernel"]
+    assert mm and all(t["flops"] > 0 for t in mm)
+    assert ex.time_replay_ns(2, 5) > 0

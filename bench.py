@@ -1,0 +1,169 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path: BERT-base encoder (batch 1, seq 128, fp32) compiled by
+Executor.make_dp_greedy-equivalent planning and replayed as HIP launches over one HBM arena.
+
+A "step" is one inference: one replay of the whole launch plan (416 kernels) on inputs that are
+already resident in HBM.  Prints ONE JSON line; see DESIGN.md for how every field is derived.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--executor plain_greedy|dp_greedy]
+                    [--no-cpu-baseline] [--layers 12]
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
+HBM_PEAK_GBS = 8000.0
+
+
+def cpu_baseline(layers_total: int, sample_layers: int, seq: int):
+    """The oracle's loop nests (the FluidML-equivalent CPU execution) on one core, timed on
+    `sample_layers` encoder layers of the same configuration plus the embedding/mask prologue;
+    the per-layer time is extrapolated to `layers_total` layers."""
+    from fluidml_amd import models
+    from oracle import graph_runner
+
+    net = models.bert_base(seq=seq, layers=sample_layers)
+    feeds = models.bert_inputs(seq)
+    timings = {}
+    graph_runner.run_graph(net, feeds, timings=timings)
+    names = [n.name for n in net.nodes]
+    per_layer = (len(names) - 8) // sample_layers  # 5 embedding nodes + 3 mask nodes come first
+    prologue = sum(timings[n][1] for n in names[:8])
+    layer_time = sum(timings[n][1] for n in names[8:]) / sample_layers
+    total = prologue + layers_total * layer_time
+    return {
+        "value": 1.0 / total,
+        "unit": "inferences/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"{sample_layers} of {layers_total} encoder layers + embeddings at seq {seq} (one inference each), "
+                  f"{per_layer} kernels per layer; per-layer time {layer_time:.3f} s extrapolated to {layers_total} layers",
+        "seconds_per_inference": total,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--executor", default="plain_greedy", choices=["plain_linear", "plain_greedy", "dp_greedy"])
+    ap.add_argument("--layers", type=int, default=12)
+    ap.add_argument("--seq", type=int, default=128)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-layers", type=int, default=3)
+    ap.add_argument("--per-kernel", action="store_true", help="also print a per-kernel table to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the reference has no multi-device path); use --gpus 1")
+
+    import numpy as np
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    from fluidml_amd import fluidml, models
+
+    net = models.bert_base(seq=args.seq, layers=args.layers)
+    feeds = models.bert_inputs(args.seq)
+    with tempfile.TemporaryDirectory() as tmp:
+        path = net.save(os.path.join(tmp, "bert_base.onnx"))
+        ex = getattr(fluidml.Executor, "make_" + args.executor)("bert_base", 1)
+        t0 = time.perf_counter()
+        ex.compile(path)
+        compile_s = time.perf_counter() - t0
+    plan = ex.plan()
+
+    # one full Invoke: H2D inputs, replay, D2H output (also records the launch plan)
+    io = {k: np.ascontiguousarray(v) for k, v in feeds.items()}
+    outs = {v.name: np.zeros(v.shape, v.dtype) for v in net.outputs}
+    io.update(outs)
+    ex.invoke(io)
+    assert np.isfinite(next(iter(outs.values()))).all()
+
+    ex.replay(args.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ex.replay(args.steps)  # ends with a wait on the plan's stream
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    value = args.steps / elapsed
+
+    # Invoke as the reference defines it (host buffers in and out): PCIe-inclusive
+    t0 = time.perf_counter()
+    for _ in range(10):
+        ex.invoke(io)
+    invoke_ms = (time.perf_counter() - t0) / 10 * 1e3
+
+    # per-kernel durations with hipEvent pairs on the plan's stream, same steps
+    times = ex.profile(3, min(args.steps, 30))
+    by_kernel = {}
+    for t in times:
+        k = by_kernel.setdefault(t["kernel"], {"ns": 0.0, "bytes": 0.0, "flops": 0.0, "launches": 0})
+        k["ns"] += t["ns"]
+        k["bytes"] += t["bytes"]
+        k["flops"] += t["flops"]
+        k["launches"] += 1
+    dominant = max(by_kernel.items(), key=lambda kv: kv[1]["ns"])
+    dname, d = dominant
+    if d["flops"] > 0:
+        achieved = d["flops"] / d["ns"] / 1e3  # flop/ns = GFLOP/s -> TFLOP/s
+        roofline = {"bound": "mfma", "kernel": dname, "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
+                    "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
+                    "avg_launch_us": d["ns"] / d["launches"] / 1e3, "launches_per_step": d["launches"],
+                    "flops_per_launch": d["flops"] / d["launches"]}
+    else:
+        achieved = d["bytes"] / d["ns"]  # B/ns = GB/s
+        roofline = {"bound": "hbm", "kernel": dname, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                    "avg_launch_us": d["ns"] / d["launches"] / 1e3, "launches_per_step": d["launches"],
+                    "bytes_per_launch": d["bytes"] / d["launches"]}
+    total_flops = sum(t["flops"] for t in times)
+    total_bytes = sum(t["bytes"] for t in times)
+    kernel_sum_ms = sum(t["ns"] for t in times) / 1e6
+
+    if args.per_kernel:
+        print(f"{'kernel':48s} {'launches':>8s} {'total us':>10s} {'avg us':>8s} {'GB/s':>9s} {'TFLOP/s':>8s}", file=sys.stderr)
+        for name, k in sorted(by_kernel.items(), key=lambda kv: -kv[1]["ns"]):
+            print(f"{name:48s} {k['launches']:8d} {k['ns'] / 1e3:10.1f} {k['ns'] / k['launches'] / 1e3:8.2f} "
+                  f"{k['bytes'] / k['ns']:9.1f} {k['flops'] / k['ns'] / 1e3:8.2f}", file=sys.stderr)
+
+    result = {
+        "metric": "inferences/sec at BERT-base seq128 fp32 on 1 MI355X",
+        "value": value,
+        "unit": "inferences/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic: seeded N(0,0.02) weights, input_ids uniform in [0,30522), mask ones",
+        "config": {"workload": f"BERT-base encoder ONNX graph, batch 1, seq {args.seq}, {args.layers} layers, fp32",
+                   "executor": args.executor, "kernels_per_step": len(times), "launch": "captured hipGraph replay"},
+        "roofline": roofline,
+        "peak_hbm_bytes": {"arena": plan["arena_bytes"], "constants": plan["constant_bytes"],
+                           "interface": plan["interface_bytes"], "total": plan["peak_device_bytes"]},
+        "whole_graph": {"flops_per_step": total_flops, "algorithmic_bytes_per_step": total_bytes,
+                        "tflops": total_flops / (ms_per_step * 1e-3) / 1e12,
+                        "sum_of_kernel_ms": kernel_sum_ms, "invoke_with_host_copies_ms": invoke_ms,
+                        "compile_s": compile_s},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.layers, min(args.cpu_sample_layers, args.layers), args.seq)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -108,6 +108,18 @@ PYBIND11_MODULE(fluidml, m) {
              for (const auto &n : s.GetNodes()) names.push_back(std::string(n->GetKindName()) + "Kernel");
              return names;
            })
+      .def("region_names",
+           [](const flow::Sequence &s) {
+             std::vector<std::string> names;
+             for (const auto &r : s.GetRegions()) names.push_back(r->GetName());
+             return names;
+           })
+      .def("buffer_sizes",
+           [](const flow::Sequence &s) {
+             std::vector<size_t> sizes;
+             for (const auto &n : s.GetNodes()) sizes.push_back(n->GetBufferSize());
+             return sizes;
+           })
       .def("layouts", [](const flow::Sequence &s) {
         std::map<std::string, std::vector<size_t>> out;
         for (const auto &r : s.GetRegions()) out[r->GetName()] = r->GetLayout();
@@ -174,6 +186,8 @@ PYBIND11_MODULE(fluidml, m) {
            },
            py::arg("warmup") = 3, py::arg("iters") = 20,
            "mean device nanoseconds of one replay of the whole plan (inputs resident in HBM)")
+      .def("replay", [](worker::Executor &e, size_t n) { e.GetContext()->GetModule().ReplayResident(n); }, py::arg("n") = 1,
+           "n replays of the plan on the tensors already in HBM, then a stream wait (no host copies)")
       .def("materialize", [](worker::Executor &e) { e.GetContext()->GetModule().Materialize(); });
 
   py::class_<worker::Lower, std::unique_ptr<worker::Lower>>(m, "Lower").def("run", &worker::Lower::Run);

@@ -231,6 +231,15 @@ size_t LaunchPlan::Run(const std::unordered_map<std::string, void *> &args, size
   return static_cast<size_t>(std::chrono::duration_cast<std::chrono::nanoseconds>(t1 - t0).count()) / epoch;
 }
 
+void LaunchPlan::ReplayResident(size_t n) {
+  Materialize();
+  kernel::LaunchContext ctx;
+  ctx.stream = stream_;
+  ctx.flags = flags_;
+  for (size_t i = 0; i < n; ++i) Replay(ctx);
+  Check(fluidml_hip_stream_synchronize(stream_), "waiting for the replays");
+}
+
 double LaunchPlan::TimeReplayNs(size_t warmup, size_t iters) {
   Materialize();
   kernel::LaunchContext ctx;

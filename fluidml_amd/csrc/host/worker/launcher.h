@@ -93,6 +93,8 @@ class LaunchPlan {
   // exactly Meta::GetSize() bytes; a missing name throws std::out_of_range
   // (reference runner.cpp:70).
   size_t Run(const std::unordered_map<std::string, void *> &args, size_t epoch);
+  // `n` replays on inputs already resident in HBM, then a stream wait; no host copies.
+  void ReplayResident(size_t n);
   // hipEvent time of every step, median of `iters` runs after `warmup`.
   std::vector<StepTime> Profile(size_t warmup, size_t iters);
   // mean device time of one whole replay measured with events on the plan's stream

@@ -28,7 +28,9 @@ class Net(GraphBuilder):
 
     # ---- weights
     def normal(self, shape, std=0.02, name=None) -> Value:
-        return self.const((self.rng.standard_normal(shape) * std).astype(np.float32), name)
+        w = self.rng.standard_normal(shape, dtype=np.float32)
+        w *= np.float32(std)
+        return self.const(w, name)
 
     def zeros(self, shape, name=None) -> Value:
         return self.const(np.zeros(shape, np.float32), name)
@@ -135,7 +137,7 @@ def bert_base(seq: int = 128, layers: int = 12, hidden: int = 768, heads: int = 
 
     word = g.gather(g.normal((vocab, hidden), name="embeddings.word_embeddings.weight"), ids)
     typ = g.gather(g.normal((types, hidden), name="embeddings.token_type_embeddings.weight"), tok)
-    pos_table = (g.rng.standard_normal((max_pos, hidden)) * 0.02).astype(np.float32)
+    pos_table = g.rng.standard_normal((max_pos, hidden), dtype=np.float32) * np.float32(0.02)
     x = g.add(word, typ)
     x = g.add(x, g.const(pos_table[:seq][None], name="embeddings.position_embeddings.slice"))
     x = g.layer_norm(x, g.ones((hidden,)), g.zeros((hidden,)), eps)

@@ -187,22 +187,20 @@ class GraphBuilder:
 
     def serialize(self) -> bytes:
         out_names = {v.name for v in self.outputs}
-        graph = b"".join(_f_bytes(1, encode_node(n.op_type, n.name, [i.name for i in n.inputs],
-                                                 [o.name for o in n.outputs], n.attrs)) for n in self.nodes)
-        graph += _f_string(2, self.name)
-        graph += b"".join(_f_bytes(5, encode_tensor(v.name, v.const)) for v in self.initializers)
-        graph += b"".join(_f_bytes(11, encode_value_info(v.name, NP_TO_ONNX[v.dtype], v.shape)) for v in self.inputs)
-        graph += b"".join(_f_bytes(12, encode_value_info(v.name, NP_TO_ONNX[v.dtype], v.shape)) for v in self.outputs)
+        parts = [_f_bytes(1, encode_node(n.op_type, n.name, [i.name for i in n.inputs], [o.name for o in n.outputs],
+                                         n.attrs)) for n in self.nodes]
+        parts.append(_f_string(2, self.name))
+        parts += [_f_bytes(5, encode_tensor(v.name, v.const)) for v in self.initializers]
+        parts += [_f_bytes(11, encode_value_info(v.name, NP_TO_ONNX[v.dtype], v.shape)) for v in self.inputs]
+        parts += [_f_bytes(12, encode_value_info(v.name, NP_TO_ONNX[v.dtype], v.shape)) for v in self.outputs]
         for n in self.nodes:
             for o in n.outputs:
                 if o.name not in out_names:
-                    graph += _f_bytes(13, encode_value_info(o.name, NP_TO_ONNX[o.dtype], o.shape))
+                    parts.append(_f_bytes(13, encode_value_info(o.name, NP_TO_ONNX[o.dtype], o.shape)))
+        graph_len = sum(len(p) for p in parts)
         opset = _f_string(1, "") + _f_varint(2, self.opset)
-        model = _f_varint(1, 8)  # ir_version
-        model += _f_string(2, "fluidml_amd.onnx_writer")
-        model += _f_bytes(7, graph)
-        model += _f_bytes(8, opset)
-        return model
+        head = _f_varint(1, 8) + _f_string(2, "fluidml_amd.onnx_writer")  # ir_version, producer_name
+        return b"".join([head, _key(7, 2), _varint(graph_len)] + parts + [_f_bytes(8, opset)])
 
     def save(self, path: str) -> str:
         with open(path, "wb") as f:

@@ -1,0 +1,339 @@
+"""Host pipeline without a GPU: ONNX codec, graph -> flow conversion, execution order, lifetimes,
+arena plan and layout DP.  Nothing here launches a kernel."""
+import itertools
+import json
+import os
+import zlib
+
+import numpy as np
+import pytest
+
+from oracle import memory_plan, ref_memory
+
+
+@pytest.fixture(scope="module")
+def mods():
+    from fluidml_amd import fluidml, models, onnx_writer
+
+    return fluidml, models, onnx_writer
+
+
+@pytest.fixture(scope="module")
+def tiny(mods, tmp_path_factory):
+    fluidml, models, _ = mods
+    net = models.bert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32, seed=5)
+    path = str(tmp_path_factory.mktemp("onnx") / "tiny_bert.onnx")
+    net.save(path)
+    return net, path
+
+
+def staged(fluidml, path, planner="make_plain_greedy_planner"):
+    graph = fluidml.Parser.make().run(path)
+    flow = fluidml.Converter.make().run(graph)
+    ctx = fluidml.Context()
+    ctx.set_cost_mode("constant")
+    sequence, index, report = getattr(ctx, planner)().run(flow)
+    return flow, sequence, index, report
+
+
+# ------------------------------------------------------------------ ONNX codec
+
+def _onnx_messages():
+    """The slice of onnx.proto this backend reads, declared to the protobuf runtime so that the
+    protobuf library itself (not this repository's codec) produces and parses the bytes."""
+    pytest.importorskip("google.protobuf")
+    from google.protobuf import descriptor_pb2, descriptor_pool, message_factory
+
+    f = descriptor_pb2.FileDescriptorProto(name="onnx_subset.proto", package="onnxsub", syntax="proto2")
+    T = descriptor_pb2.FieldDescriptorProto
+
+    def msg(name, fields):
+        m = f.message_type.add(name=name)
+        for fname, number, ftype, label, type_name in fields:
+            fd = m.field.add(name=fname, number=number, type=ftype, label=label)
+            if type_name:
+                fd.type_name = ".onnxsub." + type_name
+        return m
+
+    O, R = T.LABEL_OPTIONAL, T.LABEL_REPEATED
+    msg("TensorProto", [("dims", 1, T.TYPE_INT64, R, None), ("data_type", 2, T.TYPE_INT32, O, None),
+                        ("float_data", 4, T.TYPE_FLOAT, R, None), ("int32_data", 5, T.TYPE_INT32, R, None),
+                        ("int64_data", 7, T.TYPE_INT64, R, None), ("name", 8, T.TYPE_STRING, O, None),
+                        ("raw_data", 9, T.TYPE_BYTES, O, None), ("double_data", 10, T.TYPE_DOUBLE, R, None)])
+    msg("AttributeProto", [("name", 1, T.TYPE_STRING, O, None), ("f", 2, T.TYPE_FLOAT, O, None),
+                           ("i", 3, T.TYPE_INT64, O, None), ("s", 4, T.TYPE_BYTES, O, None),
+                           ("t", 5, T.TYPE_MESSAGE, O, "TensorProto"), ("floats", 7, T.TYPE_FLOAT, R, None),
+                           ("ints", 8, T.TYPE_INT64, R, None), ("type", 20, T.TYPE_INT32, O, None)])
+    msg("NodeProto", [("input", 1, T.TYPE_STRING, R, None), ("output", 2, T.TYPE_STRING, R, None),
+                      ("name", 3, T.TYPE_STRING, O, None), ("op_type", 4, T.TYPE_STRING, O, None),
+                      ("attribute", 5, T.TYPE_MESSAGE, R, "AttributeProto")])
+    msg("Dimension", [("dim_value", 1, T.TYPE_INT64, O, None), ("dim_param", 2, T.TYPE_STRING, O, None)])
+    msg("TensorShapeProto", [("dim", 1, T.TYPE_MESSAGE, R, "Dimension")])
+    msg("TypeTensor", [("elem_type", 1, T.TYPE_INT32, O, None), ("shape", 2, T.TYPE_MESSAGE, O, "TensorShapeProto")])
+    msg("TypeProto", [("tensor_type", 1, T.TYPE_MESSAGE, O, "TypeTensor")])
+    msg("ValueInfoProto", [("name", 1, T.TYPE_STRING, O, None), ("type", 2, T.TYPE_MESSAGE, O, "TypeProto")])
+    msg("GraphProto", [("node", 1, T.TYPE_MESSAGE, R, "NodeProto"), ("name", 2, T.TYPE_STRING, O, None),
+                       ("initializer", 5, T.TYPE_MESSAGE, R, "TensorProto"), ("input", 11, T.TYPE_MESSAGE, R, "ValueInfoProto"),
+                       ("output", 12, T.TYPE_MESSAGE, R, "ValueInfoProto"), ("value_info", 13, T.TYPE_MESSAGE, R, "ValueInfoProto")])
+    msg("OperatorSetId", [("domain", 1, T.TYPE_STRING, O, None), ("version", 2, T.TYPE_INT64, O, None)])
+    msg("ModelProto", [("ir_version", 1, T.TYPE_INT64, O, None), ("producer_name", 2, T.TYPE_STRING, O, None),
+                       ("graph", 7, T.TYPE_MESSAGE, O, "GraphProto"), ("opset_import", 8, T.TYPE_MESSAGE, R, "OperatorSetId")])
+    pool = descriptor_pool.DescriptorPool()
+    pool.Add(f)
+    get = getattr(message_factory, "GetMessageClass", None)
+    if get is None:
+        factory = message_factory.MessageFactory(pool)
+        return lambda n: factory.GetPrototype(pool.FindMessageTypeByName("onnxsub." + n))
+    return lambda n: get(pool.FindMessageTypeByName("onnxsub." + n))
+
+
+def test_writer_output_parses_with_the_protobuf_library(mods, tiny):
+    """The writer's bytes, read back by google.protobuf against onnx.proto's field numbers."""
+    net, path = tiny
+    Model = _onnx_messages()("ModelProto")
+    m = Model()
+    m.ParseFromString(open(path, "rb").read())
+    assert m.ir_version == 8 and m.opset_import[0].version == 17
+    g = m.graph
+    assert [n.name for n in g.node] == [n.name for n in net.nodes]
+    assert [n.op_type for n in g.node] == [n.op_type for n in net.nodes]
+    assert [i.name for i in g.input] == [v.name for v in net.inputs]
+    assert [tuple(d.dim_value for d in i.type.tensor_type.shape.dim) for i in g.input] == [v.shape for v in net.inputs]
+    assert len(g.value_info) == len(net.nodes) - len(net.outputs)
+    init = {t.name: t for t in g.initializer}
+    for v in net.initializers[:20]:
+        t = init[v.name]
+        assert tuple(t.dims) == v.shape
+        assert np.array_equal(np.frombuffer(t.raw_data, dtype=v.dtype).reshape(v.shape), v.const)
+    ln = next(n for n in g.node if n.op_type == "LayerNormalization")
+    attrs = {a.name: a for a in ln.attribute}
+    assert attrs["axis"].i == -1 and attrs["axis"].type == 2
+    assert abs(attrs["epsilon"].f - 1e-12) < 1e-18 and attrs["epsilon"].type == 1
+
+
+def test_reader_accepts_bytes_from_the_protobuf_library(mods, tmp_path):
+    """A model serialised by google.protobuf (typed repeated fields, unpacked and packed, negative ints,
+    rank-0 initialisers) goes through Parser -> Converter -> Planner."""
+    fluidml, _, _ = mods
+    cls = _onnx_messages()
+    m = cls("ModelProto")()
+    m.ir_version = 8
+    g = m.graph
+    g.name = "pb"
+
+    def vi(lst, name, elem, shape):
+        v = lst.add()
+        v.name = name
+        v.type.tensor_type.elem_type = elem
+        for d in shape:
+            v.type.tensor_type.shape.dim.add().dim_value = d
+
+    vi(g.input, "x", 1, [2, 3, 4])
+    vi(g.output, "y", 1, [2, 4, 3])
+    vi(g.value_info, "t0", 1, [2, 3, 4])
+    vi(g.value_info, "t1", 1, [2, 3, 4])
+    c = g.initializer.add()
+    c.name, c.data_type = "half", 1
+    c.float_data.append(0.5)  # typed field, rank 0 -> scalar operand
+    b = g.initializer.add()
+    b.name, b.data_type = "bias", 1
+    b.dims.append(4)
+    b.float_data.extend([1.0, 2.0, 3.0, 4.0])
+    n = g.node.add(name="mul", op_type="Mul")
+    n.input.extend(["x", "half"])
+    n.output.append("t0")
+    n = g.node.add(name="add", op_type="Add")
+    n.input.extend(["t0", "bias"])
+    n.output.append("t1")
+    n = g.node.add(name="tr", op_type="Transpose")
+    n.input.append("t1")
+    n.output.append("y")
+    a = n.attribute.add(name="perm", type=7)
+    a.ints.extend([0, 2, 1])
+    path = str(tmp_path / "pb.onnx")
+    open(path, "wb").write(m.SerializeToString())
+    flow, seq, index, _ = staged(fluidml, path)
+    assert seq.node_names() == ["mul", "add", "tr"]
+    assert seq.kernel_names() == ["MulConstantKernel", "AddCommonKernel", "TransposeKernel"]
+    assert index.get_maximum() == 2 * 96  # t0 and t1 live in adjacent steps
+
+
+def test_converter_rejects_what_the_reference_leaves_unreachable(mods, tmp_path):
+    fluidml, models, _ = mods
+    g = models.Net("bad", 0)
+    x = g.input("x", np.float32, (2, 3))
+    y = g.node("Sub", [x, g.scalar(1.0)], (2, 3))  # x - scalar has no FluidML kernel
+    g.output(y)
+    path = g.save(str(tmp_path / "bad.onnx"))
+    with pytest.raises(RuntimeError, match="scalar - x"):
+        staged(fluidml, path)
+    g = models.Net("bad2", 0)
+    x = g.input("x", np.float32, (2, 3))
+    g.output(g.node("Sigmoid", [x], (2, 3)))
+    with pytest.raises(RuntimeError, match="not supported"):
+        staged(fluidml, g.save(str(tmp_path / "bad2.onnx")))
+
+
+# ------------------------------------------------------------------ order, lifetimes, plan
+
+def users_of(net):
+    producer, consumers = {}, {}
+    for n in net.nodes:
+        producer[n.outputs[0].name] = n.name
+        for i in n.inputs:
+            consumers.setdefault(i.name, []).append(n.name)
+    return producer, consumers
+
+
+@pytest.mark.parametrize("planner", ["make_plain_linear_planner", "make_plain_greedy_planner", "make_dp_greedy_planner"])
+def test_order_lifetimes_and_plan(mods, tiny, planner):
+    fluidml, _, _ = mods
+    net, path = tiny
+    flow, seq, index, _ = staged(fluidml, path, planner)
+    order = seq.node_names()
+    assert sorted(order) == sorted(n.name for n in net.nodes)
+    pos = {name: i for i, name in enumerate(order)}
+    producer, consumers = users_of(net)
+    inner = {n.outputs[0].name: n.outputs[0] for n in net.nodes} 
+    for out in net.outputs:
+        inner.pop(out.name)
+    # valid topological order
+    for n in net.nodes:
+        for i in n.inputs:
+            if i.name in producer:
+                assert pos[producer[i.name]] < pos[n.name]
+    # rebuild the planner's requests from first principles, in the planner's push order
+    # (reference planner.cpp:236-293): regions in Sequence::GetRegions() order, then node scratch
+    requests, names = [], []
+    for name in seq.region_names():
+        if name in inner and consumers.get(name):
+            steps = [pos[producer[name]]] + [pos[c] for c in consumers[name]]
+            v = inner[name]
+            requests.append((min(steps), max(steps), int(np.prod(v.shape)) * v.dtype.itemsize))
+            names.append(name)
+    for i, (name, scratch) in enumerate(zip(order, seq.buffer_sizes())):
+        if scratch:
+            requests.append((i, i, scratch))
+            names.append(name)
+    got = index.items()
+    assert sorted(got) == sorted(names)
+    kind = 0 if planner == "make_plain_linear_planner" else 1
+    want_offsets, want_max = (memory_plan.linear_plan if kind == 0 else memory_plan.greedy_plan)(requests)
+    assert [got[n][0] for n in names] == want_offsets
+    assert index.get_maximum() == want_max
+    if ref_memory.available():  # and the reference's own planner sources agree on the same requests
+        assert ref_memory.plan(kind, requests) == (want_offsets, want_max)
+    # tensors alive at a common step never share bytes
+    for (a, ra), (b, rb) in itertools.combinations(zip(names, requests), 2):
+        if ra[0] <= rb[1] and rb[0] <= ra[1]:
+            oa, ob = got[a][0], got[b][0]
+            assert oa + ra[2] <= ob or ob + rb[2] <= oa, (a, b)
+    # scratch sizes: softmax / layernorm = input shape with the axis collapsed (reference flow/node.cpp:972-985, 1355-1368)
+    sizes = dict(zip(order, seq.buffer_sizes()))
+    for n in net.nodes:
+        if n.op_type in ("Softmax", "LayerNormalization"):
+            assert sizes[n.name] == int(np.prod(n.inputs[0].shape[:-1])) * 4
+        else:
+            assert sizes[n.name] == 0
+
+
+def test_plan_is_independent_of_layouts(mods, tiny):
+    """Layouts change strides, never sizes: DP and plain greedy plans coincide (reference meta.cpp:38-40)."""
+    fluidml, _, _ = mods
+    _, path = tiny
+    _, s1, i1, _ = staged(fluidml, path, "make_plain_greedy_planner")
+    _, s2, i2, _ = staged(fluidml, path, "make_dp_greedy_planner")
+    assert s1.node_names() == s2.node_names()
+    assert i1.items() == i2.items()
+
+
+def test_golden_bert_base_plan(mods, tmp_path):
+    """Arena plan of the headline workload, frozen: a change of container order, heap ties or best-fit
+    behaviour shows up here.  (Regenerate with tests/golden/make_plan_fixture.py.)"""
+    fluidml, models, _ = mods
+    golden_path = os.path.join(os.path.dirname(__file__), "golden", "bert_base_s128_plan.json")
+    golden = json.load(open(golden_path))
+    net = models.bert_base()
+    path = net.save(str(tmp_path / "bert.onnx"))
+    _, seq, index, _ = staged(fluidml, path)
+    assert index.get_maximum() == golden["arena_bytes"]
+    assert len(seq.node_names()) == golden["nodes"]
+    items = index.items()
+    digest = zlib.crc32(json.dumps(sorted((k, v[0], v[1]) for k, v in items.items())).encode())
+    assert digest == golden["offsets_crc32"]
+    assert zlib.crc32("\n".join(seq.node_names()).encode()) == golden["order_crc32"]
+    for name, (offset, size) in golden["sample"].items():
+        assert items[name] == (offset, size), name
+
+
+# ------------------------------------------------------------------ layout DP
+
+def test_dp_constant_cost_closed_form(mods, tiny):
+    """With every kernel cost equal, every tensor gets GenAllOrders(rank)[0], the reversed permutation
+    (ties keep the first enumerated layout, reference dp.cpp:705-709, 787, 820)."""
+    fluidml, _, _ = mods
+    net, path = tiny
+    flow, seq, _, report = staged(fluidml, path, "make_dp_greedy_planner")
+    layouts = fluidml._dp_layouts(flow, "constant")
+    shapes = {v.name: v.shape for n in net.nodes for v in n.outputs + n.inputs}
+    assert len(layouts) >= len(net.nodes)
+    for name, layout in layouts.items():
+        assert layout == list(range(len(shapes[name])))[::-1], name
+    doc = json.loads(report)
+    assert set(doc) == {"dp_table", "plan"} and "evaluator" in doc["dp_table"]
+    assert doc["plan"] == {k: v for k, v in layouts.items()}
+    row = doc["dp_table"]["evaluator"]["SoftmaxKernel"][0]
+    assert set(row) == {"input_shape", "output_shape", "input_layout", "output_layout", "time_cost"}
+
+
+def synthetic_cost(kernel, layouts):
+    return 1 + zlib.crc32(repr((kernel, layouts)).encode()) % 1000
+
+
+def test_dp_is_optimal_on_a_chain(mods, tmp_path):
+    """Brute force over every layout assignment of a 3-kernel chain with a synthetic cost table."""
+    fluidml, models, _ = mods
+    g = models.Net("chain", 0)
+    x = g.input("x", np.float32, (2, 3, 4))
+    t1 = g.unary("Relu", x)
+    t2 = g.transpose(t1, (2, 0, 1))
+    y = g.unary("Erf", t2)
+    g.output(y)
+    path = g.save(str(tmp_path / "chain.onnx"))
+    flow, _, _, _ = staged(fluidml, path)
+    perms = fluidml._gen_all_orders(3)
+    kernels = [("ReluKernel", (2, 3, 4), (2, 3, 4)), ("TransposeKernel", (2, 3, 4), (4, 2, 3)), ("ErfKernel", (4, 2, 3), (4, 2, 3))]
+    table = {}
+    for name, ishape, oshape in kernels:
+        table[name] = [{"input_shape": list(ishape), "output_shape": list(oshape), "input_layout": a, "output_layout": b,
+                        "time_cost": synthetic_cost(name, (a, b))} for a in perms for b in perms]
+    layouts = fluidml._dp_layouts(flow, json.dumps({"evaluator": table}))
+    tensors = [x.name, t1.name, t2.name, y.name]
+    assert sorted(layouts) == sorted(tensors)
+    assert layouts[y.name] == perms[0]  # the result keeps the first enumerated layout
+
+    def total(assign):
+        return sum(synthetic_cost(k[0], (assign[i], assign[i + 1])) for i, k in enumerate(kernels))
+
+    best = min(total([a, b, c, perms[0]]) for a in perms for b in perms for c in perms)
+    assert total([layouts[t] for t in tensors]) == best
+
+
+def test_dp_on_a_branching_flow_covers_every_tensor(mods, tmp_path):
+    """Residual pattern (a value with two consumers): main chain + branch, merged first-writer-wins."""
+    fluidml, models, _ = mods
+    g = models.Net("residual", 0)
+    x = g.input("x", np.float32, (2, 3, 4))
+    a = g.unary("Relu", x)
+    b = g.unary("Erf", a)
+    c = g.unary("Tanh", b)
+    d = g.add(c, a)  # `a` feeds both Erf and Add
+    g.output(g.unary("Neg", d))
+    path = g.save(str(tmp_path / "residual.onnx"))
+    flow, _, _, _ = staged(fluidml, path)
+    layouts = fluidml._dp_layouts(flow, "constant")
+    produced = {n.outputs[0].name for n in g.nodes} | {x.name}
+    assert produced <= set(layouts)
+    assert all(sorted(l) == [0, 1, 2] for l in layouts.values())
+    # determinism: same flow, same answer
+    assert fluidml._dp_layouts(flow, "constant") == layouts

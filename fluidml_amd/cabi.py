@@ -80,6 +80,7 @@ SIGNATURES = {
     "fluidml_hip_memcpy_h2d": [_vp, _vp, _sz, _vp],
     "fluidml_hip_memcpy_d2h": [_vp, _vp, _sz, _vp],
     "fluidml_hip_memcpy_d2d": [_vp, _vp, _sz, _vp],
+    "fluidml_hip_time_kernels": [_vp, _vp],
     "fluidml_hip_stream_create": [_P(_vp)],
     "fluidml_hip_stream_destroy": [_vp],
     "fluidml_hip_stream_synchronize": [_vp],
@@ -139,6 +140,10 @@ SIGNATURES = {
     "fluidml_hip_matmul": [_T, _T, _T, _vp],
     "fluidml_hip_matmul_bf16": [_T, _T, _T, _vp],
     "fluidml_hip_gemm_constant_weights_bias": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _u32, _vp],
+    "fluidml_hip_matmul_add": [_T, _T, _T, _T, _vp],
+    "fluidml_hip_matmul_add_div_erf_add_mul_mul": [_T, _T, _T, _T, _f64, _f64, _f64, _vp],
+    "fluidml_hip_div_add_softmax": [_T, _f64, _T, _T, _i64, _vp],
+    "fluidml_hip_add_layer_normalization": [_T, _T, _T, _T, _T, _i64, _f64, _vp],
     "fluidml_hip_conv_without_padding": [_T, _T, _T, _T, _i64p, _i64p, _i64, _u32, _vp],
     "fluidml_hip_conv_with_padding": [_T, _T, _T, _T, _vp, _sz, _i64p, _i64p, _i64p, _i64, _u32, _vp],
 }

@@ -194,9 +194,9 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
   const float *w = static_cast<const float *>(weights->base);
   hipStream_t s = AsStream(stream);
   switch (ns) {
-    case 1: hipLaunchKernelGGL(ConvDirect<1>, grid, block, 0, s, p, o, x, w, b); break;
-    case 2: hipLaunchKernelGGL(ConvDirect<2>, grid, block, 0, s, p, o, x, w, b); break;
-    case 3: hipLaunchKernelGGL(ConvDirect<3>, grid, block, 0, s, p, o, x, w, b); break;
+    case 1: FL_LAUNCH(ConvDirect<1>, grid, block, 0, s, p, o, x, w, b); break;
+    case 2: FL_LAUNCH(ConvDirect<2>, grid, block, 0, s, p, o, x, w, b); break;
+    case 3: FL_LAUNCH(ConvDirect<3>, grid, block, 0, s, p, o, x, w, b); break;
     default: return FL_ERR_RANK;
   }
   return LaunchStatus();

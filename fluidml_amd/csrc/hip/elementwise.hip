@@ -132,11 +132,11 @@ int LaunchNest(LoopNest nest, void *out, const void *in0, const void *in1, const
   const int64_t blocks_needed = (n_items + kBlock - 1) / kBlock;
   const uint32_t grid = static_cast<uint32_t>(std::min<int64_t>(blocks_needed, 256 * 32));
   if (vec_ok) {
-    hipLaunchKernelGGL((EwKernel<NIN, kVec, TO, T0, T1, T2, Op>), dim3(grid), dim3(kBlock), 0, stream, args,
+    FL_LAUNCH((EwKernel<NIN, kVec, TO, T0, T1, T2, Op>), dim3(grid), dim3(kBlock), 0, stream, args,
                        static_cast<uint32_t>(n_items), bcast, static_cast<TO *>(out), static_cast<const T0 *>(in0),
                        static_cast<const T1 *>(in1), static_cast<const T2 *>(in2), op);
   } else {
-    hipLaunchKernelGGL((EwKernel<NIN, 1, TO, T0, T1, T2, Op>), dim3(grid), dim3(kBlock), 0, stream, args,
+    FL_LAUNCH((EwKernel<NIN, 1, TO, T0, T1, T2, Op>), dim3(grid), dim3(kBlock), 0, stream, args,
                        static_cast<uint32_t>(n_items), 0u, static_cast<TO *>(out), static_cast<const T0 *>(in0),
                        static_cast<const T1 *>(in1), static_cast<const T2 *>(in2), op);
   }

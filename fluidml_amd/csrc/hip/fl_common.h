@@ -10,6 +10,7 @@
 #define FLUIDML_AMD_CSRC_HIP_FL_COMMON_H_
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <algorithm>
 #include <cstdint>
@@ -39,6 +40,24 @@ constexpr int kWave = 64;  // CDNA wavefront
   } while (0)
 
 inline hipStream_t AsStream(void *stream) { return static_cast<hipStream_t>(stream); }
+
+// Kernel-exact timing: while a thread has a pair of events installed, every kernel it launches through
+// FL_LAUNCH updates them with the dispatch's own begin/end timestamps (hipExtLaunchKernelGGL), which
+// excludes launch latency and queue gaps -- the same interval a profiler reports for the kernel.
+struct KernelTimer {
+  hipEvent_t start = nullptr, stop = nullptr;
+};
+KernelTimer &ThreadKernelTimer();  // runtime.hip
+
+#define FL_LAUNCH(kernel, grid, block, shmem, stream, ...)                                                       \
+  do {                                                                                                           \
+    const ::fl::KernelTimer &fl_timer_ = ::fl::ThreadKernelTimer();                                              \
+    if (fl_timer_.start != nullptr) {                                                                            \
+      hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, fl_timer_.start, fl_timer_.stop, 0, __VA_ARGS__); \
+    } else {                                                                                                     \
+      hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                                       \
+    }                                                                                                            \
+  } while (0)
 
 inline int LaunchStatus() {
   hipError_t err = hipGetLastError();
@@ -127,7 +146,7 @@ inline bool IsAligned(const void *p, size_t bytes) {
 // canonicalised: unit dims dropped, dims ordered by descending output stride
 // (so the innermost loop walks the output's fastest physical dimension), and
 // neighbours merged when every operand agrees they are contiguous.
-constexpr int kMaxOperands = 5;
+constexpr int kMaxOperands = 6;
 
 struct LoopNest {
   int rank = 0;
@@ -214,6 +233,7 @@ struct NestArgs {
 
 template <int NOPS>
 inline NestArgs<NOPS> MakeNestArgs(const LoopNest &nest) {
+  static_assert(NOPS <= kMaxOperands, "LoopNest holds strides for kMaxOperands operands");
   NestArgs<NOPS> a;
   std::memset(&a, 0, sizeof(a));
   a.rank = nest.rank;

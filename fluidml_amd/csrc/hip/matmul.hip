@@ -41,6 +41,9 @@ struct MatmulArgs {
   float ca, cb;
   const float *bias;
   int32_t sDm, sDn;
+  // optional activation after the bias: v * (erf(v / g_div) + g_add) * g_mul  (the erf-GELU chain)
+  int32_t act;
+  float g_div, g_add, g_mul;
 };
 
 template <int VEC>
@@ -105,7 +108,7 @@ struct TileLoader {
 
 // LA: 0 = A tile kept [m][k] (A is k-contiguous), 1 = kept [k][m].
 // LB: 0 = B tile kept [k][n] (B is n-contiguous), 1 = kept [n][k].
-template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC>
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH>
 __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, float *__restrict__ C,
                                                                 const float *__restrict__ A,
                                                                 const float *__restrict__ B) {
@@ -164,38 +167,35 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  VecF<VEC> ra[LoaderA::kPerThread], rb[LoaderB::kPerThread];
+  // DEPTH chunks are in flight in registers: the loads of chunk c+DEPTH are issued while chunk c is
+  // consumed, so a workgroup keeps DEPTH * (A tile + B tile) bytes outstanding instead of one chunk --
+  // with only a few workgroups per CU that is what hides the L2/HBM latency.
+  static_assert(DEPTH % 2 == 0, "the LDS buffer index must be a compile-time function of the stage");
+  VecF<VEC> ra[DEPTH][LoaderA::kPerThread], rb[DEPTH][LoaderB::kPerThread];
   const int rows_m = p.M - m0, cols_n = p.N - n0;
   const int n_chunks = (p.K + BK - 1) / BK;
 
-  auto load_chunk = [&](int c) {
+  auto load_chunk = [&](int c, VecF<VEC>(&qa)[LoaderA::kPerThread], VecF<VEC>(&qb)[LoaderB::kPerThread]) {
     const int k0 = c * BK, k_valid = p.K - k0;
     if constexpr (LA == 0) {
-      LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAm, p.sAk, rows_m, k_valid, ra);
+      LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAm, p.sAk, rows_m, k_valid, qa);
     } else {
-      LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAk, p.sAm, k_valid, rows_m, ra);
+      LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAk, p.sAm, k_valid, rows_m, qa);
     }
     if constexpr (LB == 0) {
-      LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBk, p.sBn, k_valid, cols_n, rb);
+      LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBk, p.sBn, k_valid, cols_n, qb);
     } else {
-      LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBn, p.sBk, cols_n, k_valid, rb);
+      LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBn, p.sBk, cols_n, k_valid, qb);
     }
   };
-  auto store_chunk = [&](int buf) {
+  auto store_chunk = [&](int buf, const VecF<VEC>(&qa)[LoaderA::kPerThread], const VecF<VEC>(&qb)[LoaderB::kPerThread]) {
     float *as = lds + buf * (A_ELEMS + B_ELEMS);
     float *bs = as + A_ELEMS;
-    LoaderA::Store(as, LDA, ra);
-    LoaderB::Store(bs, LDB, rb);
+    LoaderA::Store(as, LDA, qa);
+    LoaderB::Store(bs, LDB, qb);
   };
-
-  load_chunk(0);
-  store_chunk(0);
-  __syncthreads();
-
-  for (int c = 0; c < n_chunks; ++c) {
-    const bool more = c + 1 < n_chunks;
-    if (more) load_chunk(c + 1);
-    const float *as = lds + (c & 1) * (A_ELEMS + B_ELEMS);
+  auto compute_chunk = [&](int buf) {
+    const float *as = lds + buf * (A_ELEMS + B_ELEMS);
     const float *bs = as + A_ELEMS;
 #pragma unroll
     for (int kk = 0; kk < KW; kk += 8) {
@@ -237,13 +237,30 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
           for (int j = 0; j < TN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][e], b[j][e], acc[i][j], 0, 0, 0);
     }
-    if (more) store_chunk((c + 1) & 1);
-    __syncthreads();
+  };
+
+#pragma unroll
+  for (int s = 0; s < DEPTH; ++s) {
+    if (s < n_chunks) load_chunk(s, ra[s], rb[s]);
   }
+  for (int c0 = 0; c0 < n_chunks; c0 += DEPTH) {
+#pragma unroll
+    for (int s = 0; s < DEPTH; ++s) {
+      const int c = c0 + s;
+      if (c < n_chunks) {  // uniform over the workgroup
+        store_chunk(s & 1, ra[s], rb[s]);
+        if (c + DEPTH < n_chunks) load_chunk(c + DEPTH, ra[s], rb[s]);
+        // one barrier per chunk: buffer (s&1) was last read two chunks ago, and every wave
+        // passed the previous barrier only after finishing that read
+        __syncthreads();
+        compute_chunk(s & 1);
+      }
+    }
+  }
+  __syncthreads();  // staging area is reused below
 
   // ---- combine the K slices of a workgroup through LDS ------------------------
   if constexpr (KS > 1) {
-    // the final barrier of the loop above makes the staging area free
     if (ks > 0) {
       float *red = lds + (ks - 1) * BM * BN;
 #pragma unroll
@@ -289,18 +306,21 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
           if (p.bias != nullptr) {
             v = p.ca * v + p.cb * p.bias[m * p.sDm + n * p.sDn];
           }
+          if (p.act != 0) {
+            v = (v * (erff(v / p.g_div) + p.g_add)) * p.g_mul;
+          }
           Cb[static_cast<int64_t>(m) * p.sCm + static_cast<int64_t>(n) * p.sCn] = v;
         }
       }
     }
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC>
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH>
 void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   MatmulArgs q = p;
   q.tiles_m = (p.M + BM - 1) / BM;
   q.tiles_n = (p.N + BN - 1) / BN;
-  hipLaunchKernelGGL((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC>), dim3(q.tiles_m * q.tiles_n, n_batch),
+  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH>), dim3(q.tiles_m * q.tiles_n, n_batch),
                      dim3(64 * WM * WN * KS), 0, s, q, C, A, B);
 }
 
@@ -309,16 +329,21 @@ void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
   const int64_t tiles_l = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * n_batch;
   const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
   if (tiles_l >= 192) {
-    LaunchConfig<128, 128, 16, 2, 2, 1, LA, LB, VEC>(p, n_batch, C, A, B, s);
+    LaunchConfig<128, 128, 16, 2, 2, 1, LA, LB, VEC, 2>(p, n_batch, C, A, B, s);
   } else if (tiles_m >= 192) {
-    LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC>(p, n_batch, C, A, B, s);
+    LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4>(p, n_batch, C, A, B, s);
   } else {
-    LaunchConfig<32, 32, 32, 1, 1, 4, LA, LB, VEC>(p, n_batch, C, A, B, s);
+    LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2>(p, n_batch, C, A, B, s);
   }
 }
 
+struct Activation {
+  int32_t kind = 0;  // 0 none, 1 erf-GELU chain
+  float div = 1.0f, add = 0.0f, mul = 1.0f;
+};
+
 int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, bool trans_a, bool trans_b, float ca,
-             float cb, const fl_tensor *bias, void *stream) {
+             float cb, const fl_tensor *bias, void *stream, Activation act = Activation()) {
   FL_CHECK(CheckView(lhs));
   FL_CHECK(CheckView(rhs));
   FL_CHECK(CheckView(out));
@@ -374,6 +399,10 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   p.batch = MakeNestArgs<3>(nest);
   p.ca = ca;
   p.cb = cb;
+  p.act = act.kind;
+  p.g_div = act.div;
+  p.g_add = act.add;
+  p.g_mul = act.mul;
   if (bias != nullptr) {
     FL_CHECK(CheckView(bias));
     if (bias->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
@@ -430,6 +459,25 @@ extern "C" {
 
 int fluidml_hip_matmul(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
   return fl::Contract(lhs, rhs, out, false, false, 1.0f, 0.0f, nullptr, stream);
+}
+
+int fluidml_hip_matmul_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
+                           void *stream) {
+  if (!lhs || !rhs || !bias || !out) return FL_ERR_NULL;
+  if (bias->rank != 1) return FL_ERR_RANK;
+  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream);
+}
+
+int fluidml_hip_matmul_add_div_erf_add_mul_mul(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias,
+                                               const fl_tensor *out, double div, double add, double mul, void *stream) {
+  if (!lhs || !rhs || !bias || !out) return FL_ERR_NULL;
+  if (bias->rank != 1) return FL_ERR_RANK;
+  fl::Activation act;
+  act.kind = 1;
+  act.div = static_cast<float>(div);
+  act.add = static_cast<float>(add);
+  act.mul = static_cast<float>(mul);
+  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, act);
 }
 
 int fluidml_hip_matmul_bf16(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {

@@ -112,19 +112,19 @@ int LogicalReshape(const fl_tensor *in, const fl_tensor *out, void *stream) {
   hipStream_t st = AsStream(stream);
   switch (DtypeSize(in->dtype)) {
     case 1:
-      hipLaunchKernelGGL(ReshapeKernel<uint8_t>, dim3(grid), dim3(kBlock), 0, st, a, s, static_cast<uint32_t>(n),
+      FL_LAUNCH(ReshapeKernel<uint8_t>, dim3(grid), dim3(kBlock), 0, st, a, s, static_cast<uint32_t>(n),
                          static_cast<uint8_t *>(out->base), static_cast<const uint8_t *>(in->base));
       break;
     case 2:
-      hipLaunchKernelGGL(ReshapeKernel<uint16_t>, dim3(grid), dim3(kBlock), 0, st, a, s, static_cast<uint32_t>(n),
+      FL_LAUNCH(ReshapeKernel<uint16_t>, dim3(grid), dim3(kBlock), 0, st, a, s, static_cast<uint32_t>(n),
                          static_cast<uint16_t *>(out->base), static_cast<const uint16_t *>(in->base));
       break;
     case 4:
-      hipLaunchKernelGGL(ReshapeKernel<uint32_t>, dim3(grid), dim3(kBlock), 0, st, a, s, static_cast<uint32_t>(n),
+      FL_LAUNCH(ReshapeKernel<uint32_t>, dim3(grid), dim3(kBlock), 0, st, a, s, static_cast<uint32_t>(n),
                          static_cast<uint32_t *>(out->base), static_cast<const uint32_t *>(in->base));
       break;
     case 8:
-      hipLaunchKernelGGL(ReshapeKernel<uint64_t>, dim3(grid), dim3(kBlock), 0, st, a, s, static_cast<uint32_t>(n),
+      FL_LAUNCH(ReshapeKernel<uint64_t>, dim3(grid), dim3(kBlock), 0, st, a, s, static_cast<uint32_t>(n),
                          static_cast<uint64_t *>(out->base), static_cast<const uint64_t *>(in->base));
       break;
     default: return FL_ERR_DTYPE;
@@ -195,12 +195,12 @@ int LaunchGather(LoopNest nest, int64_t axis_stride, int64_t axis_len, void *out
   NestArgs<3 + NADD> a = MakeNestArgs<3 + NADD>(nest);
   const uint32_t grid = static_cast<uint32_t>((n_items + kBlock - 1) / kBlock);
   if (vec_ok) {
-    hipLaunchKernelGGL((GatherKernel<T, kVec, NADD>), dim3(grid), dim3(kBlock), 0, stream, a,
+    FL_LAUNCH((GatherKernel<T, kVec, NADD>), dim3(grid), dim3(kBlock), 0, stream, a,
                        static_cast<uint32_t>(n_items), static_cast<int32_t>(axis_stride), axis_len,
                        static_cast<T *>(out), static_cast<const int64_t *>(indices), static_cast<const T *>(data),
                        static_cast<const T *>(add0), static_cast<const T *>(add1));
   } else {
-    hipLaunchKernelGGL((GatherKernel<T, 1, NADD>), dim3(grid), dim3(kBlock), 0, stream, a,
+    FL_LAUNCH((GatherKernel<T, 1, NADD>), dim3(grid), dim3(kBlock), 0, stream, a,
                        static_cast<uint32_t>(n_items), static_cast<int32_t>(axis_stride), axis_len,
                        static_cast<T *>(out), static_cast<const int64_t *>(indices), static_cast<const T *>(data),
                        static_cast<const T *>(add0), static_cast<const T *>(add1));
@@ -349,10 +349,10 @@ int fluidml_hip_cum_sum(const fl_tensor *in, const fl_tensor *out, int64_t axis,
   const uint32_t len = static_cast<uint32_t>(in->shape[axis]);
   const int32_t so = static_cast<int32_t>(out->strides[axis]), si = static_cast<int32_t>(in->strides[axis]);
   if (in->dtype == FL_INT64) {
-    hipLaunchKernelGGL(CumSumKernel<int64_t>, dim3(grid), dim3(kBlock), 0, s, a, static_cast<uint32_t>(rows), len, so,
+    FL_LAUNCH(CumSumKernel<int64_t>, dim3(grid), dim3(kBlock), 0, s, a, static_cast<uint32_t>(rows), len, so,
                        si, static_cast<int64_t *>(out->base), static_cast<const int64_t *>(in->base));
   } else if (in->dtype == FL_INT32) {
-    hipLaunchKernelGGL(CumSumKernel<int32_t>, dim3(grid), dim3(kBlock), 0, s, a, static_cast<uint32_t>(rows), len, so,
+    FL_LAUNCH(CumSumKernel<int32_t>, dim3(grid), dim3(kBlock), 0, s, a, static_cast<uint32_t>(rows), len, so,
                        si, static_cast<int32_t *>(out->base), static_cast<const int32_t *>(in->base));
   } else {
     return FL_ERR_DTYPE;  // reference cum_sum.cpp uses arith.addi only

@@ -100,7 +100,7 @@ int Pool(const fl_tensor *in, const fl_tensor *out, const int64_t *kernel_shape,
   p.window = MakeNestArgs<1>(window);
   p.n_out = static_cast<uint32_t>(Numel(out));
   p.n_window = static_cast<uint32_t>(n_window);
-  hipLaunchKernelGGL(PoolKernel<IS_MAX>, dim3((p.n_out + kBlock - 1) / kBlock), dim3(kBlock), 0, AsStream(stream), p,
+  FL_LAUNCH(PoolKernel<IS_MAX>, dim3((p.n_out + kBlock - 1) / kBlock), dim3(kBlock), 0, AsStream(stream), p,
                      static_cast<float *>(out->base), static_cast<const float *>(in->base));
   return LaunchStatus();
 }

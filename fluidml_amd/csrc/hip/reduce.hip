@@ -45,6 +45,7 @@ __device__ __forceinline__ void RowOffsets(const NestArgs<NOPS> &a, uint32_t row
 // Build the outer nest (all dims but `axis`) for the given operands' strides.
 template <int NOPS>
 RowArgs<NOPS> MakeRowArgs(int rank, const int64_t *shape, int axis, const int64_t (*strides)[kMaxRank]) {
+  static_assert(NOPS <= kMaxOperands, "LoopNest holds strides for kMaxOperands operands");
   LoopNest nest;
   nest.n_operands = NOPS;
   nest.rank = 0;
@@ -68,22 +69,33 @@ RowArgs<NOPS> MakeRowArgs(int rank, const int64_t *shape, int axis, const int64_
 // ---- Softmax ----------------------------------------------------------------
 
 // One wave per row, row cached in registers: len <= 64 * ITEMS.
+// Optional prologue shared by the softmax kernels: x / div + mask (operand 2 of the nest, broadcast
+// strides), i.e. the DivConstantRhs -> AddCommon -> Softmax chain of an attention block in one pass.
+struct SoftmaxPre {
+  const float *mask;  // nullptr = plain softmax
+  float div;
+  __device__ __forceinline__ float operator()(float x, int32_t mask_off) const {
+    return mask != nullptr ? x / div + mask[mask_off] : x;
+  }
+};
+
 template <int ITEMS>
-__global__ __launch_bounds__(kBlock) void SoftmaxRowWave(RowArgs<2> a, float *__restrict__ out,
-                                                         const float *__restrict__ in) {
+__global__ __launch_bounds__(kBlock) void SoftmaxRowWave(RowArgs<3> a, float *__restrict__ out,
+                                                         const float *__restrict__ in, SoftmaxPre pre) {
   const uint32_t lane = threadIdx.x % kWave;
   const uint32_t row = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   if (row >= a.n_rows) return;
-  int32_t off[2];
-  RowOffsets<2>(a.outer, row, off);
+  int32_t off[3];
+  RowOffsets<3>(a.outer, row, off);
   const float *src = in + off[1];
   float *dst = out + off[0];
+  const int32_t sm = a.axis_stride[2];
   float x[ITEMS];
   float m = -__FLT_MAX__;
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t j = lane + i * kWave;
-    x[i] = j < a.len ? src[j] : -__FLT_MAX__;
+    x[i] = j < a.len ? pre(src[j], off[2] + static_cast<int32_t>(j) * sm) : -__FLT_MAX__;
     m = fmaxf(m, x[i]);
   }
   m = WaveReduce(m, MaxOp{});
@@ -103,52 +115,55 @@ __global__ __launch_bounds__(kBlock) void SoftmaxRowWave(RowArgs<2> a, float *__
 }
 
 // One block per row, any length, three passes over the (cache-resident) row.
-__global__ __launch_bounds__(kBlock) void SoftmaxRowBlock(RowArgs<2> a, float *__restrict__ out,
-                                                          const float *__restrict__ in) {
+__global__ __launch_bounds__(kBlock) void SoftmaxRowBlock(RowArgs<3> a, float *__restrict__ out,
+                                                          const float *__restrict__ in, SoftmaxPre pre) {
   __shared__ float smem[kBlock / kWave];
-  int32_t off[2];
-  RowOffsets<2>(a.outer, blockIdx.x, off);
+  int32_t off[3];
+  RowOffsets<3>(a.outer, blockIdx.x, off);
   const float *src = in + off[1];
   float *dst = out + off[0];
+  const int32_t sm = a.axis_stride[2];
+  auto at = [&](uint32_t j) { return pre(src[j], off[2] + static_cast<int32_t>(j) * sm); };
   float m = -__FLT_MAX__;
-  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) m = fmaxf(m, src[j]);
+  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) m = fmaxf(m, at(j));
   m = BlockReduce<kBlock / kWave>(m, MaxOp{}, smem);
   float s = 0.0f;
-  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) s += expf(src[j] - m);
+  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) s += expf(at(j) - m);
   s = BlockReduce<kBlock / kWave>(s, SumOp{}, smem);
-  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) dst[j] = expf(src[j] - m) / s;
+  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) dst[j] = expf(at(j) - m) / s;
 }
 
 // One lane per row; the axis is walked with its stride.
-__global__ __launch_bounds__(kBlock) void SoftmaxColumn(RowArgs<2> a, float *__restrict__ out,
-                                                        const float *__restrict__ in) {
+__global__ __launch_bounds__(kBlock) void SoftmaxColumn(RowArgs<3> a, float *__restrict__ out,
+                                                        const float *__restrict__ in, SoftmaxPre pre) {
   const uint32_t row = blockIdx.x * kBlock + threadIdx.x;
   if (row >= a.n_rows) return;
-  int32_t off[2];
-  RowOffsets<2>(a.outer, row, off);
+  int32_t off[3];
+  RowOffsets<3>(a.outer, row, off);
   const float *src = in + off[1];
   float *dst = out + off[0];
-  const int32_t si = a.axis_stride[1], so = a.axis_stride[0];
+  const int32_t si = a.axis_stride[1], so = a.axis_stride[0], sm = a.axis_stride[2];
+  auto at = [&](uint32_t j) { return pre(src[static_cast<int32_t>(j) * si], off[2] + static_cast<int32_t>(j) * sm); };
   float m = -__FLT_MAX__;
-  for (uint32_t j = 0; j < a.len; ++j) m = fmaxf(m, src[static_cast<int32_t>(j) * si]);
+  for (uint32_t j = 0; j < a.len; ++j) m = fmaxf(m, at(j));
   float s = 0.0f;
-  for (uint32_t j = 0; j < a.len; ++j) s += expf(src[static_cast<int32_t>(j) * si] - m);
-  for (uint32_t j = 0; j < a.len; ++j) dst[static_cast<int32_t>(j) * so] = expf(src[static_cast<int32_t>(j) * si] - m) / s;
+  for (uint32_t j = 0; j < a.len; ++j) s += expf(at(j) - m);
+  for (uint32_t j = 0; j < a.len; ++j) dst[static_cast<int32_t>(j) * so] = expf(at(j) - m) / s;
 }
 
 // ---- LayerNormalization -------------------------------------------------------
 
-// operands: 0 out, 1 in, 2 scale, 3 bias, 4 scratch (one float per row)
+// operands: 0 out, 1 in, 2 scale, 3 bias, 4 scratch (one float per row), 5 optional addend y: LN(in + y)
 template <int ITEMS>
-__global__ __launch_bounds__(kBlock) void LayerNormRowBlock(RowArgs<5> a, float *__restrict__ out,
+__global__ __launch_bounds__(kBlock) void LayerNormRowBlock(RowArgs<6> a, float *__restrict__ out,
                                                             const float *__restrict__ in,
                                                             const float *__restrict__ scale,
                                                             const float *__restrict__ bias,
                                                             const float *__restrict__ scratch, float eps,
-                                                            int stale_scratch) {
+                                                            int stale_scratch, const float *__restrict__ addend) {
   __shared__ float smem[kBlock / kWave];
-  int32_t off[5];
-  RowOffsets<5>(a.outer, blockIdx.x, off);
+  int32_t off[6];
+  RowOffsets<6>(a.outer, blockIdx.x, off);
   const float *src = in + off[1];
   const float n = static_cast<float>(a.len);
   float x[ITEMS];
@@ -157,6 +172,7 @@ __global__ __launch_bounds__(kBlock) void LayerNormRowBlock(RowArgs<5> a, float 
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t j = threadIdx.x + i * kBlock;
     x[i] = j < a.len ? src[j] : 0.0f;
+    if (addend != nullptr && j < a.len) x[i] = x[i] + addend[off[5] + static_cast<int32_t>(j) * a.axis_stride[5]];
     s += x[i];
   }
   s = BlockReduce<kBlock / kWave>(s, SumOp{}, smem);
@@ -183,26 +199,31 @@ __global__ __launch_bounds__(kBlock) void LayerNormRowBlock(RowArgs<5> a, float 
 }
 
 // Any length / any axis stride: lanes of a block stride the row three times.
-__global__ __launch_bounds__(kBlock) void LayerNormRowLoop(RowArgs<5> a, float *__restrict__ out,
+__global__ __launch_bounds__(kBlock) void LayerNormRowLoop(RowArgs<6> a, float *__restrict__ out,
                                                            const float *__restrict__ in,
                                                            const float *__restrict__ scale,
                                                            const float *__restrict__ bias,
                                                            const float *__restrict__ scratch, float eps,
-                                                           int stale_scratch) {
+                                                           int stale_scratch, const float *__restrict__ addend) {
   __shared__ float smem[kBlock / kWave];
-  int32_t off[5];
-  RowOffsets<5>(a.outer, blockIdx.x, off);
+  int32_t off[6];
+  RowOffsets<6>(a.outer, blockIdx.x, off);
   const float *src = in + off[1];
   const int32_t si = a.axis_stride[1], so = a.axis_stride[0], sg = a.axis_stride[2], sb = a.axis_stride[3];
+  const int32_t sy = a.axis_stride[5];
+  auto at = [&](uint32_t j) {
+    const int32_t jj = static_cast<int32_t>(j);
+    return addend != nullptr ? src[jj * si] + addend[off[5] + jj * sy] : src[jj * si];
+  };
   const float n = static_cast<float>(a.len);
   float s = 0.0f;
-  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) s += src[static_cast<int32_t>(j) * si];
+  for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) s += at(j);
   s = BlockReduce<kBlock / kWave>(s, SumOp{}, smem);
   if (stale_scratch) s += scratch[off[4]];
   const float mean = s / n;
   float v = 0.0f;
   for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) {
-    const float d = src[static_cast<int32_t>(j) * si] - mean;
+    const float d = at(j) - mean;
     v += d * d;
   }
   v = BlockReduce<kBlock / kWave>(v, SumOp{}, smem);
@@ -212,30 +233,35 @@ __global__ __launch_bounds__(kBlock) void LayerNormRowLoop(RowArgs<5> a, float *
   const float *b = bias + off[3];
   for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) {
     const int32_t jj = static_cast<int32_t>(j);
-    dst[jj * so] = ((src[jj * si] - mean) * inv) * g[jj * sg] + b[jj * sb];
+    dst[jj * so] = ((at(j) - mean) * inv) * g[jj * sg] + b[jj * sb];
   }
 }
 
 // One lane per row (strided axis, many rows).
-__global__ __launch_bounds__(kBlock) void LayerNormColumn(RowArgs<5> a, float *__restrict__ out,
+__global__ __launch_bounds__(kBlock) void LayerNormColumn(RowArgs<6> a, float *__restrict__ out,
                                                           const float *__restrict__ in,
                                                           const float *__restrict__ scale,
                                                           const float *__restrict__ bias,
                                                           const float *__restrict__ scratch, float eps,
-                                                          int stale_scratch) {
+                                                          int stale_scratch, const float *__restrict__ addend) {
   const uint32_t row = blockIdx.x * kBlock + threadIdx.x;
   if (row >= a.n_rows) return;
-  int32_t off[5];
-  RowOffsets<5>(a.outer, row, off);
+  int32_t off[6];
+  RowOffsets<6>(a.outer, row, off);
   const float *src = in + off[1];
   const int32_t si = a.axis_stride[1], so = a.axis_stride[0], sg = a.axis_stride[2], sb = a.axis_stride[3];
+  const int32_t sy = a.axis_stride[5];
+  auto at = [&](uint32_t j) {
+    const int32_t jj = static_cast<int32_t>(j);
+    return addend != nullptr ? src[jj * si] + addend[off[5] + jj * sy] : src[jj * si];
+  };
   const float n = static_cast<float>(a.len);
   float s = stale_scratch ? scratch[off[4]] : 0.0f;
-  for (uint32_t j = 0; j < a.len; ++j) s += src[static_cast<int32_t>(j) * si];
+  for (uint32_t j = 0; j < a.len; ++j) s += at(j);
   const float mean = s / n;
   float v = 0.0f;
   for (uint32_t j = 0; j < a.len; ++j) {
-    const float d = src[static_cast<int32_t>(j) * si] - mean;
+    const float d = at(j) - mean;
     v += d * d;
   }
   const float inv = 1.0f / sqrtf(v / n + eps);
@@ -244,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void LayerNormColumn(RowArgs<5> a, float *_
   const float *b = bias + off[3];
   for (uint32_t j = 0; j < a.len; ++j) {
     const int32_t jj = static_cast<int32_t>(j);
-    dst[jj * so] = ((src[jj * si] - mean) * inv) * g[jj * sg] + b[jj * sb];
+    dst[jj * so] = ((at(j) - mean) * inv) * g[jj * sg] + b[jj * sb];
   }
 }
 
@@ -305,21 +331,28 @@ using namespace fl;
 
 extern "C" {
 
-int fluidml_hip_softmax(const fl_tensor *in, const fl_tensor *out, void *scratch, size_t scratch_bytes, int64_t axis,
-                        void *stream) {
-  (void)scratch;
-  (void)scratch_bytes;
+static int SoftmaxImpl(const fl_tensor *in, const fl_tensor *mask, float div, const fl_tensor *out, int64_t axis,
+                       void *stream) {
   FL_CHECK(CheckView(in));
   FL_CHECK(CheckView(out));
   if (in->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
   if (!SameShape(in, out)) return FL_ERR_SHAPE;
   if (axis < 0 || axis >= in->rank) return FL_ERR_ATTR;  // reference normalises before the kernel
-  int64_t strides[2][kMaxRank];
+  int64_t strides[3][kMaxRank];
   for (int i = 0; i < in->rank; ++i) {
     strides[0][i] = out->strides[i];
     strides[1][i] = in->strides[i];
+    strides[2][i] = 0;
   }
-  RowArgs<2> a = MakeRowArgs<2>(in->rank, in->shape, static_cast<int>(axis), strides);
+  SoftmaxPre pre{nullptr, 1.0f};
+  if (mask != nullptr) {
+    FL_CHECK(CheckView(mask));
+    if (mask->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+    FL_CHECK(BroadcastStrides(mask, in->rank, in->shape, strides[2]));
+    pre.mask = static_cast<const float *>(mask->base);
+    pre.div = div;
+  }
+  RowArgs<3> a = MakeRowArgs<3>(in->rank, in->shape, static_cast<int>(axis), strides);
   float *o = static_cast<float *>(out->base);
   const float *x = static_cast<const float *>(in->base);
   hipStream_t s = AsStream(stream);
@@ -327,28 +360,40 @@ int fluidml_hip_softmax(const fl_tensor *in, const fl_tensor *out, void *scratch
   if (row_contig && a.len > 16) {
     const uint32_t wave_blocks = (a.n_rows + kBlock / kWave - 1) / (kBlock / kWave);
     if (a.len <= 64) {
-      hipLaunchKernelGGL(SoftmaxRowWave<1>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x);
+      FL_LAUNCH(SoftmaxRowWave<1>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x, pre);
     } else if (a.len <= 128) {
-      hipLaunchKernelGGL(SoftmaxRowWave<2>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x);
+      FL_LAUNCH(SoftmaxRowWave<2>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x, pre);
     } else if (a.len <= 256) {
-      hipLaunchKernelGGL(SoftmaxRowWave<4>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x);
+      FL_LAUNCH(SoftmaxRowWave<4>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x, pre);
     } else if (a.len <= 512) {
-      hipLaunchKernelGGL(SoftmaxRowWave<8>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x);
+      FL_LAUNCH(SoftmaxRowWave<8>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x, pre);
     } else if (a.len <= 1024) {
-      hipLaunchKernelGGL(SoftmaxRowWave<16>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x);
+      FL_LAUNCH(SoftmaxRowWave<16>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x, pre);
     } else {
-      hipLaunchKernelGGL(SoftmaxRowBlock, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x);
+      FL_LAUNCH(SoftmaxRowBlock, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, pre);
     }
   } else {
-    hipLaunchKernelGGL(SoftmaxColumn, dim3((a.n_rows + kBlock - 1) / kBlock), dim3(kBlock), 0, s, a, o, x);
+    FL_LAUNCH(SoftmaxColumn, dim3((a.n_rows + kBlock - 1) / kBlock), dim3(kBlock), 0, s, a, o, x, pre);
   }
   return LaunchStatus();
 }
 
-int fluidml_hip_layer_normalization_constant_scale_bias(const fl_tensor *in, const fl_tensor *scale,
-                                                        const fl_tensor *bias, const fl_tensor *out, void *scratch,
-                                                        size_t scratch_bytes, int64_t axis, double epsilon,
-                                                        uint32_t flags, void *stream) {
+int fluidml_hip_softmax(const fl_tensor *in, const fl_tensor *out, void *scratch, size_t scratch_bytes, int64_t axis,
+                        void *stream) {
+  (void)scratch;
+  (void)scratch_bytes;
+  return SoftmaxImpl(in, nullptr, 1.0f, out, axis, stream);
+}
+
+int fluidml_hip_div_add_softmax(const fl_tensor *in, double div, const fl_tensor *mask, const fl_tensor *out,
+                                int64_t axis, void *stream) {
+  if (mask == nullptr) return FL_ERR_NULL;
+  return SoftmaxImpl(in, mask, static_cast<float>(div), out, axis, stream);
+}
+
+static int LayerNormImpl(const fl_tensor *in, const fl_tensor *addend, const fl_tensor *scale, const fl_tensor *bias,
+                         const fl_tensor *out, void *scratch, size_t scratch_bytes, int64_t axis, double epsilon,
+                         uint32_t flags, void *stream) {
   FL_CHECK(CheckView(in));
   FL_CHECK(CheckView(scale));
   FL_CHECK(CheckView(bias));
@@ -359,9 +404,18 @@ int fluidml_hip_layer_normalization_constant_scale_bias(const fl_tensor *in, con
   if (axis < 0) axis += in->rank;  // reference flow/node.cpp:931-933
   if (axis < 0 || axis >= in->rank) return FL_ERR_ATTR;
   const int stale = (flags & FL_REF_LN_STALE_SCRATCH) ? 1 : 0;
-  int64_t strides[5][kMaxRank];
+  int64_t strides[6][kMaxRank];
   FL_CHECK(BroadcastStrides(scale, in->rank, in->shape, strides[2]));
   FL_CHECK(BroadcastStrides(bias, in->rank, in->shape, strides[3]));
+  const float *y = nullptr;
+  if (addend != nullptr) {
+    FL_CHECK(CheckView(addend));
+    if (addend->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+    FL_CHECK(BroadcastStrides(addend, in->rank, in->shape, strides[5]));
+    y = static_cast<const float *>(addend->base);
+  } else {
+    for (int i = 0; i < in->rank; ++i) strides[5][i] = 0;
+  }
   // scratch: dense row-major tensor of the input shape with axis -> 1
   int64_t acc = 1, rows = 1;
   for (int i = in->rank - 1; i >= 0; --i) {
@@ -379,7 +433,7 @@ int fluidml_hip_layer_normalization_constant_scale_bias(const fl_tensor *in, con
     if (scratch == nullptr) return FL_ERR_NULL;
     if (scratch_bytes < static_cast<size_t>(rows) * sizeof(float)) return FL_ERR_SCRATCH;
   }
-  RowArgs<5> a = MakeRowArgs<5>(in->rank, in->shape, static_cast<int>(axis), strides);
+  RowArgs<6> a = MakeRowArgs<6>(in->rank, in->shape, static_cast<int>(axis), strides);
   float *o = static_cast<float *>(out->base);
   const float *x = static_cast<const float *>(in->base);
   const float *g = static_cast<const float *>(scale->base);
@@ -390,23 +444,37 @@ int fluidml_hip_layer_normalization_constant_scale_bias(const fl_tensor *in, con
   const bool row_contig = a.axis_stride[0] == 1 && a.axis_stride[1] == 1;
   if (row_contig && a.len > 64) {
     if (a.len <= kBlock) {
-      hipLaunchKernelGGL(LayerNormRowBlock<1>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+      FL_LAUNCH(LayerNormRowBlock<1>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
     } else if (a.len <= 2 * kBlock) {
-      hipLaunchKernelGGL(LayerNormRowBlock<2>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+      FL_LAUNCH(LayerNormRowBlock<2>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
     } else if (a.len <= 4 * kBlock) {
-      hipLaunchKernelGGL(LayerNormRowBlock<4>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+      FL_LAUNCH(LayerNormRowBlock<4>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
     } else if (a.len <= 8 * kBlock) {
-      hipLaunchKernelGGL(LayerNormRowBlock<8>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+      FL_LAUNCH(LayerNormRowBlock<8>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
     } else {
-      hipLaunchKernelGGL(LayerNormRowLoop, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+      FL_LAUNCH(LayerNormRowLoop, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
     }
   } else if (a.n_rows >= 4096 || a.len <= 64) {
-    hipLaunchKernelGGL(LayerNormColumn, dim3((a.n_rows + kBlock - 1) / kBlock), dim3(kBlock), 0, s, a, o, x, g, b, sc,
-                       eps, stale);
+    FL_LAUNCH(LayerNormColumn, dim3((a.n_rows + kBlock - 1) / kBlock), dim3(kBlock), 0, s, a, o, x, g, b, sc,
+                       eps, stale, y);
   } else {
-    hipLaunchKernelGGL(LayerNormRowLoop, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale);
+    FL_LAUNCH(LayerNormRowLoop, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
   }
   return LaunchStatus();
+}
+
+int fluidml_hip_layer_normalization_constant_scale_bias(const fl_tensor *in, const fl_tensor *scale,
+                                                        const fl_tensor *bias, const fl_tensor *out, void *scratch,
+                                                        size_t scratch_bytes, int64_t axis, double epsilon,
+                                                        uint32_t flags, void *stream) {
+  return LayerNormImpl(in, nullptr, scale, bias, out, scratch, scratch_bytes, axis, epsilon, flags, stream);
+}
+
+int fluidml_hip_add_layer_normalization(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *scale,
+                                        const fl_tensor *bias, const fl_tensor *out, int64_t axis, double epsilon,
+                                        void *stream) {
+  if (rhs == nullptr) return FL_ERR_NULL;
+  return LayerNormImpl(lhs, rhs, scale, bias, out, nullptr, 0, axis, epsilon, 0, stream);
 }
 
 int fluidml_hip_reduce_mean(const fl_tensor *in, const fl_tensor *out, const int64_t *axes, int32_t n_axes,
@@ -456,10 +524,10 @@ int fluidml_hip_reduce_mean(const fl_tensor *in, const fl_tensor *out, const int
   hipStream_t s = AsStream(stream);
   const bool inner_contig = inner.strides[0][inner.rank - 1] == 1;
   if ((inner_contig && n_red >= 32) || n_out < 1024) {
-    hipLaunchKernelGGL(ReduceMeanWave, dim3((a.n_out + kBlock / kWave - 1) / (kBlock / kWave)), dim3(kBlock), 0, s, a, o,
+    FL_LAUNCH(ReduceMeanWave, dim3((a.n_out + kBlock / kWave - 1) / (kBlock / kWave)), dim3(kBlock), 0, s, a, o,
                        x);
   } else {
-    hipLaunchKernelGGL(ReduceMeanThread, dim3((a.n_out + kBlock - 1) / kBlock), dim3(kBlock), 0, s, a, o, x);
+    FL_LAUNCH(ReduceMeanThread, dim3((a.n_out + kBlock - 1) / kBlock), dim3(kBlock), 0, s, a, o, x);
   }
   return LaunchStatus();
 }

@@ -18,6 +18,13 @@ __global__ __launch_bounds__(256) void FillZero(uint32_t *p, size_t n_words, uin
 
 }  // namespace
 
+namespace fl {
+KernelTimer &ThreadKernelTimer() {
+  static thread_local KernelTimer timer;
+  return timer;
+}
+}  // namespace fl
+
 extern "C" {
 
 int fluidml_hip_abi_version(void) { return 1; }
@@ -91,7 +98,7 @@ int fluidml_hip_arena_zero(void *arena, size_t bytes, void *stream) {
   if (bytes == 0) return FL_OK;
   const size_t n_words = bytes / 4, n_tail = bytes % 4;
   const size_t blocks = std::min<size_t>((n_words + 255) / 256 + 1, 4096);
-  hipLaunchKernelGGL(FillZero, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, AsStream(stream),
+  FL_LAUNCH(FillZero, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, AsStream(stream),
                      static_cast<uint32_t *>(arena), n_words, static_cast<uint8_t *>(arena) + n_words * 4, n_tail);
   return LaunchStatus();
 }
@@ -185,6 +192,14 @@ int fluidml_hip_event_elapsed_ns(void *start, void *stop, double *ns) {
   float ms = 0.0f;
   FL_HIP_CHECK(hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
   *ns = static_cast<double>(ms) * 1.0e6;
+  return FL_OK;
+}
+
+int fluidml_hip_time_kernels(void *start, void *stop) {
+  if ((start == nullptr) != (stop == nullptr)) return FL_ERR_NULL;
+  fl::KernelTimer &t = fl::ThreadKernelTimer();
+  t.start = static_cast<hipEvent_t>(start);
+  t.stop = static_cast<hipEvent_t>(stop);
   return FL_OK;
 }
 

@@ -142,16 +142,23 @@ class MeasuredCostModel : public CostModel {
       Check(ctx.status, ctx.failed.c_str());
     };
     launch();  // warm: code object load, caches
-    constexpr int kBatch = 4, kRounds = 3;
+    // the dispatch's own begin/end timestamps: launch latency and queue gaps would otherwise swamp
+    // the differences between layouts for the many kernels that run only a few microseconds
+    constexpr int kRounds = 5;
     double best = std::numeric_limits<double>::max();
-    for (int r = 0; r < kRounds; ++r) {
-      Check(fluidml_hip_event_record(start_, stream_), "record");
-      for (int i = 0; i < kBatch; ++i) launch();
-      Check(fluidml_hip_event_record(stop_, stream_), "record");
-      double ns = 0;
-      Check(fluidml_hip_event_elapsed_ns(start_, stop_, &ns), "elapsed");
-      best = std::min(best, ns / kBatch);
+    Check(fluidml_hip_time_kernels(start_, stop_), "kernel timing on");
+    try {
+      for (int r = 0; r < kRounds; ++r) {
+        launch();
+        double ns = 0;
+        Check(fluidml_hip_event_elapsed_ns(start_, stop_, &ns), "elapsed");
+        best = std::min(best, ns);
+      }
+    } catch (...) {
+      fluidml_hip_time_kernels(nullptr, nullptr);
+      throw;
     }
+    Check(fluidml_hip_time_kernels(nullptr, nullptr), "kernel timing off");
     return std::max<size_t>(1, static_cast<size_t>(best));
   }
 

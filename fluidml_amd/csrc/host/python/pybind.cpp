@@ -32,10 +32,27 @@ using namespace fluidml;
 
 namespace {
 
+py::dict OperandOf(const worker::Operand &op) {
+  static const char *kSpaces[] = {"arena", "interface", "constant", "private"};
+  py::dict d;
+  d["name"] = op.name;
+  d["space"] = kSpaces[static_cast<int>(op.space)];
+  d["offset"] = op.offset;
+  d["bytes"] = op.meta.GetSize();
+  d["shape"] = op.meta.GetShape();
+  d["layout"] = op.layout;
+  return d;
+}
+
 py::dict StepsOf(worker::LaunchPlan &plan) {
   py::list steps;
   for (const worker::Step &s : plan.GetSteps()) {
     py::dict d;
+    py::list inputs;
+    inputs.append(OperandOf(s.in0));
+    if (s.node->IsDoubleInputs()) inputs.append(OperandOf(s.in1));
+    d["inputs"] = inputs;
+    d["out"] = OperandOf(s.out);
     d["node"] = s.node->GetName();
     d["kernel"] = s.kernel->GetKernelName();
     d["bytes"] = s.bytes;
@@ -51,6 +68,16 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
   out["interface_bytes"] = plan.GetInterfaceBytes();
   out["peak_device_bytes"] = plan.GetPeakDeviceBytes();
   out["steps"] = steps;
+  py::list launches;
+  for (const worker::Launch &l : plan.GetSchedule()) {
+    py::dict d;
+    d["kind"] = worker::LaunchKindName(l.kind);
+    d["members"] = l.members;
+    d["bytes"] = l.bytes;
+    d["flops"] = l.flops;
+    launches.append(d);
+  }
+  out["launches"] = launches;
   return out;
 }
 
@@ -86,6 +113,7 @@ PYBIND11_MODULE(fluidml, m) {
            py::arg("mode"), "\"measure\", \"constant\" or the path of a saved cost table")
       .def("set_ref_flags", [](context::Context &c, uint32_t flags) { c->ref_flags = flags; }, py::arg("flags"))
       .def("set_use_graph", [](context::Context &c, bool use) { c->use_graph = use; }, py::arg("use"))
+      .def("set_fuse", [](context::Context &c, bool fuse) { c->fuse = fuse; }, py::arg("fuse"))
       .def("plan_text", [](context::Context &c) { return c->GetModule().ToText(); });
 
   py::class_<flow::Flow, std::unique_ptr<flow::Flow>>(m, "Flow")

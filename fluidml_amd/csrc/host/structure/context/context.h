@@ -80,6 +80,8 @@ class ContextImpl {
   uint32_t ref_flags = 0;
   // replay the plan as a captured hipGraph (env FLUIDML_HIP_GRAPH=0 disables)
   bool use_graph = true;
+  // launch-level fusion of single-reader kernel chains (env FLUIDML_FUSE=0 disables)
+  bool fuse = true;
   // cost source of the layout DP (env FLUIDML_DP_COST=measure|constant|<path to table json>)
   CostMode cost_mode = CostMode::Measure;
   std::string cost_table_path;

@@ -78,6 +78,9 @@ class Base : virtual public Kernel {
       if (c) c->Upload();
     }
   }
+  const DeviceConstant *GetConstant(int i) const override {
+    return i == 0 ? c0_.get() : i == 1 ? c1_.get() : i == 2 ? c2_.get() : nullptr;
+  }
   size_t GetConstantBytes() const override {
     size_t n = 0;
     for (const DeviceConstant *c : {c0_.get(), c1_.get(), c2_.get()}) {

@@ -76,6 +76,12 @@ class Kernel {
   virtual void Prepare() {}
   // bytes of HBM the kernel's own constants occupy
   virtual size_t GetConstantBytes() const { return 0; }
+  // i-th constant the kernel owns (0..2), nullptr if it has none there; lets a fused launch reuse
+  // the uploaded LayerNorm scale/bias of the node it absorbs
+  virtual const DeviceConstant *GetConstant(int i) const {
+    (void)i;
+    return nullptr;
+  }
 };
 
 class SingleInputKernel : virtual public Kernel {};

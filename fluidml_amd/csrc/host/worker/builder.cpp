@@ -151,6 +151,7 @@ class GeneralBuilderImpl : public GeneralBuilder {
     }
     plan->SetFlags(context_->ref_flags);
     plan->SetUseGraph(context_->use_graph);
+    plan->SetFuse(context_->fuse);
     context_->SetModule(std::move(plan));
     context_->SetFuncAttr(std::move(func_attr));
   }
@@ -242,6 +243,7 @@ class KernelBuilderImpl : public KernelBuilder {
     plan->AddStep(std::move(step));
     plan->SetFlags(context_->ref_flags);
     plan->SetUseGraph(false);
+    plan->SetFuse(false);
     context_->SetModule(std::move(plan));
     context_->SetFuncAttr(std::move(func_attr));
   }

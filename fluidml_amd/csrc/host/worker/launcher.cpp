@@ -121,6 +121,14 @@ std::string LaunchPlan::ToText() const {
     if (s.has_buffer) os << " scratch@arena+" << s.buffer_offset << ":" << s.buffer_bytes;
     os << "\n";
   }
+  const std::vector<Launch> &schedule = GetSchedule();
+  os << "  schedule launches=" << schedule.size() << "\n";
+  for (const Launch &l : schedule) {
+    if (l.kind == Launch::Kind::Step) continue;
+    os << "    fused " << LaunchKindName(l.kind) << " {";
+    for (size_t m = 0; m < l.members.size(); ++m) os << (m ? "," : "") << "%" << l.members[m];
+    os << "}\n";
+  }
   return os.str();
 }
 
@@ -156,24 +164,105 @@ void *LaunchPlan::GetDeviceAddress(const std::string &name) const {
   return nullptr;
 }
 
-void LaunchPlan::LaunchAll(kernel::LaunchContext &ctx) const {
-  for (const Step &s : steps_) {
-    const kernel::TensorView in0 = ViewOf(Resolve(s.in0), s.in0), out = ViewOf(Resolve(s.out), s.out);
-    const kernel::Buffer buffer{s.has_buffer ? static_cast<char *>(arena_) + s.buffer_offset : nullptr, s.buffer_bytes};
-    kernel::Kernel *k = s.kernel.get();
-    if (s.node->IsSingleInput()) {
-      if (s.has_buffer) dynamic_cast<kernel::SingleInputWithBufferKernel &>(*k).Run(ctx, in0, out, buffer);
-      else dynamic_cast<kernel::SingleInputWithoutBufferKernel &>(*k).Run(ctx, in0, out);
+const std::vector<Launch> &LaunchPlan::GetSchedule() const {
+  if (!schedule_built_) {
+    schedule_ = BuildSchedule(steps_, fuse_ && flags_ == 0);
+    schedule_built_ = true;
+  }
+  return schedule_;
+}
+
+void LaunchPlan::IssueStep(kernel::LaunchContext &ctx, const Step &s) const {
+  const kernel::TensorView in0 = ViewOf(Resolve(s.in0), s.in0), out = ViewOf(Resolve(s.out), s.out);
+  const kernel::Buffer buffer{s.has_buffer ? static_cast<char *>(arena_) + s.buffer_offset : nullptr, s.buffer_bytes};
+  kernel::Kernel *k = s.kernel.get();
+  if (s.node->IsSingleInput()) {
+    if (s.has_buffer) dynamic_cast<kernel::SingleInputWithBufferKernel &>(*k).Run(ctx, in0, out, buffer);
+    else dynamic_cast<kernel::SingleInputWithoutBufferKernel &>(*k).Run(ctx, in0, out);
+  } else {
+    const kernel::TensorView in1 = ViewOf(Resolve(s.in1), s.in1);
+    if (s.has_buffer) dynamic_cast<kernel::DoubleInputsWithBufferKernel &>(*k).Run(ctx, in0, in1, out, buffer);
+    else dynamic_cast<kernel::DoubleInputsWithoutBufferKernel &>(*k).Run(ctx, in0, in1, out);
+  }
+  if (ctx.status != 0) {
+    throw std::runtime_error("launching " + ctx.failed + " for node '" + s.node->GetName() + "': " +
+                             fluidml_hip_error_string(ctx.status));
+  }
+}
+
+namespace {
+// `t` seen through a transpose: result[k] walks t's dim perm[k]
+fl_tensor Permuted(const fl_tensor &t, const std::vector<int64_t> &perm, bool inverse) {
+  fl_tensor v = t;
+  for (int32_t k = 0; k < t.rank; ++k) {
+    const int64_t p = perm.empty() ? t.rank - 1 - k : perm[static_cast<size_t>(k)];
+    if (inverse) {
+      v.shape[p] = t.shape[k];
+      v.strides[p] = t.strides[k];
     } else {
-      const kernel::TensorView in1 = ViewOf(Resolve(s.in1), s.in1);
-      if (s.has_buffer) dynamic_cast<kernel::DoubleInputsWithBufferKernel &>(*k).Run(ctx, in0, in1, out, buffer);
-      else dynamic_cast<kernel::DoubleInputsWithoutBufferKernel &>(*k).Run(ctx, in0, in1, out);
-    }
-    if (ctx.status != 0) {
-      throw std::runtime_error("launching " + ctx.failed + " for node '" + s.node->GetName() + "': " +
-                               fluidml_hip_error_string(ctx.status));
+      v.shape[k] = t.shape[p];
+      v.strides[k] = t.strides[p];
     }
   }
+  return v;
+}
+}  // namespace
+
+void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
+  if (l.kind == Launch::Kind::Step) {
+    IssueStep(ctx, steps_[l.members[0]]);
+    return;
+  }
+  const kernel::TensorView a = ViewOf(Resolve(l.a), l.a), out = ViewOf(Resolve(l.out), l.out);
+  int rc = FL_ERR_UNSUPPORTED;
+  switch (l.kind) {
+    case Launch::Kind::MatMulAdd: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b), c = ViewOf(Resolve(l.c), l.c);
+      rc = fluidml_hip_matmul_add(&a.t, &b.t, &c.t, &out.t, ctx.stream);
+      break;
+    }
+    case Launch::Kind::MatMulAddGelu: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b), c = ViewOf(Resolve(l.c), l.c);
+      rc = fluidml_hip_matmul_add_div_erf_add_mul_mul(&a.t, &b.t, &c.t, &out.t, l.s0, l.s1, l.s2, ctx.stream);
+      break;
+    }
+    case Launch::Kind::DivAddSoftmax: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
+      rc = fluidml_hip_div_add_softmax(&a.t, l.s0, &b.t, &out.t, l.axis, ctx.stream);
+      break;
+    }
+    case Launch::Kind::AddLayerNorm: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
+      const kernel::Kernel &ln = *steps_[l.owner].kernel;
+      const kernel::DeviceConstant *scale = ln.GetConstant(0), *bias = ln.GetConstant(1);
+      if (scale == nullptr || bias == nullptr) throw std::logic_error("fused LayerNorm: the node holds no scale/bias");
+      const kernel::TensorView g = scale->View(), h = bias->View();
+      rc = fluidml_hip_add_layer_normalization(&a.t, &b.t, &g.t, &h.t, &out.t, l.axis, l.s0, ctx.stream);
+      break;
+    }
+    case Launch::Kind::ReshapeTranspose: {
+      // the Transpose's output buffer addressed by the Reshape's logical index
+      const fl_tensor dst = Permuted(out.t, l.perm, true);
+      rc = fluidml_hip_reshape(&a.t, &dst, ctx.stream);
+      break;
+    }
+    case Launch::Kind::TransposeReshape: {
+      // the Transpose's input buffer addressed by the Transpose's logical output index
+      const fl_tensor src = Permuted(a.t, l.perm, false);
+      rc = fluidml_hip_reshape(&src, &out.t, ctx.stream);
+      break;
+    }
+    default: break;
+  }
+  if (rc != 0) {
+    ctx.Note(rc, LaunchKindName(l.kind));
+    throw std::runtime_error(std::string("launching fused ") + LaunchKindName(l.kind) + " ending at node '" +
+                             steps_[l.members.back()].node->GetName() + "': " + fluidml_hip_error_string(rc));
+  }
+}
+
+void LaunchPlan::LaunchAll(kernel::LaunchContext &ctx) const {
+  for (const Launch &l : GetSchedule()) Issue(ctx, l);
 }
 
 // One replay of the whole sequence on the plan's stream: the captured graph
@@ -264,51 +353,45 @@ std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
   kernel::LaunchContext ctx;
   ctx.stream = stream_;
   ctx.flags = flags_;
-  const bool saved = use_graph_;
-  use_graph_ = false;
-  std::vector<std::vector<double>> samples(steps_.size());
-  std::vector<void *> events(steps_.size() + 1, nullptr);
+  const std::vector<Launch> &schedule = GetSchedule();
+  std::vector<std::vector<double>> samples(schedule.size());
+  // one start/stop pair per launch, stamped by the dispatch itself (kernel-exact durations)
+  std::vector<void *> events(2 * schedule.size(), nullptr);
   for (void *&e : events) Check(fluidml_hip_event_create(&e), "event");
   for (size_t it = 0; it < warmup + iters; ++it) {
-    Check(fluidml_hip_event_record(events[0], stream_), "event record");
-    for (size_t i = 0; i < steps_.size(); ++i) {
-      // launch one step at a time between event pairs
-      const Step &s = steps_[i];
-      const kernel::TensorView in0 = ViewOf(Resolve(s.in0), s.in0), out = ViewOf(Resolve(s.out), s.out);
-      const kernel::Buffer buffer{s.has_buffer ? static_cast<char *>(arena_) + s.buffer_offset : nullptr, s.buffer_bytes};
-      kernel::Kernel *k = s.kernel.get();
-      if (s.node->IsSingleInput()) {
-        if (s.has_buffer) dynamic_cast<kernel::SingleInputWithBufferKernel &>(*k).Run(ctx, in0, out, buffer);
-        else dynamic_cast<kernel::SingleInputWithoutBufferKernel &>(*k).Run(ctx, in0, out);
-      } else {
-        const kernel::TensorView in1 = ViewOf(Resolve(s.in1), s.in1);
-        if (s.has_buffer) dynamic_cast<kernel::DoubleInputsWithBufferKernel &>(*k).Run(ctx, in0, in1, out, buffer);
-        else dynamic_cast<kernel::DoubleInputsWithoutBufferKernel &>(*k).Run(ctx, in0, in1, out);
+    try {
+      for (size_t i = 0; i < schedule.size(); ++i) {
+        Check(fluidml_hip_time_kernels(events[2 * i], events[2 * i + 1]), "kernel timing on");
+        Issue(ctx, schedule[i]);
       }
-      Check(ctx.status, "profiling launch");
-      Check(fluidml_hip_event_record(events[i + 1], stream_), "event record");
+    } catch (...) {
+      fluidml_hip_time_kernels(nullptr, nullptr);
+      throw;
     }
+    Check(fluidml_hip_time_kernels(nullptr, nullptr), "kernel timing off");
     Check(fluidml_hip_stream_synchronize(stream_), "profiling sync");
     if (it >= warmup) {
-      for (size_t i = 0; i < steps_.size(); ++i) {
+      for (size_t i = 0; i < schedule.size(); ++i) {
         double ns = 0;
-        Check(fluidml_hip_event_elapsed_ns(events[i], events[i + 1], &ns), "event elapsed");
+        Check(fluidml_hip_event_elapsed_ns(events[2 * i], events[2 * i + 1], &ns), "event elapsed");
         samples[i].push_back(ns);
       }
     }
   }
   for (void *e : events) fluidml_hip_event_destroy(e);
-  use_graph_ = saved;
   std::vector<StepTime> out;
-  for (size_t i = 0; i < steps_.size(); ++i) {
+  for (size_t i = 0; i < schedule.size(); ++i) {
     std::vector<double> &v = samples[i];
     std::sort(v.begin(), v.end());
+    const Launch &l = schedule[i];
     StepTime t;
-    t.node = steps_[i].node->GetName();
-    t.kernel = steps_[i].kernel->GetKernelName();
+    for (size_t m : l.members) {
+      t.node += (t.node.empty() ? "" : "+") + steps_[m].node->GetName();
+      t.kernel += (t.kernel.empty() ? "" : "+") + steps_[m].kernel->GetKernelName();
+    }
     t.ns = v.empty() ? 0 : v[v.size() / 2];
-    t.bytes = steps_[i].bytes;
-    t.flops = steps_[i].flops;
+    t.bytes = l.bytes;
+    t.flops = l.flops;
     out.push_back(std::move(t));
   }
   return out;

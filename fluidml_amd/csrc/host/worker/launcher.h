@@ -45,6 +45,37 @@ struct Step {
   double bytes = 0, flops = 0;
 };
 
+// One launch of the replayed schedule: a single step, or a chain of steps whose
+// intermediate tensors each have exactly one reader inside the chain.  A chain
+// is issued at the position of its last member, reads only what enters the
+// chain from outside, and writes only the last member's output; the elided
+// intermediates keep their slots in the memory plan but are never touched.
+struct Launch {
+  enum class Kind {
+    Step,              // members = {i}
+    MatMulAdd,         // MatMul -> AddCommon(rank-1 constant bias)
+    MatMulAddGelu,     // MatMul -> AddCommon(bias) -> DivConstantRhs -> Erf -> AddConstant -> MulCommon -> MulConstant
+    DivAddSoftmax,     // DivConstantRhs -> AddCommon(mask) -> Softmax
+    AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias
+    ReshapeTranspose,  // Reshape -> Transpose, one strided copy
+    TransposeReshape   // Transpose -> Reshape, one strided copy
+  };
+  Kind kind = Kind::Step;
+  std::vector<size_t> members;  // indices into the step list, ascending
+  Operand a, b, c, out;         // external operands, role by kind (see fusion.cpp)
+  double s0 = 0, s1 = 0, s2 = 0;
+  int64_t axis = 0;
+  std::vector<int64_t> perm;
+  size_t owner = 0;  // member whose kernel owns constants the launch needs (LayerNorm scale/bias)
+  double bytes = 0, flops = 0;
+};
+const char *LaunchKindName(Launch::Kind kind);
+// Groups `steps` into launches.  With `fuse` false every step is its own launch.
+// A chain is only formed when no step between its first and last member writes
+// bytes that alias one of the chain's external inputs (arena intervals from the
+// memory plan), so that issuing the reads late is safe.
+std::vector<Launch> BuildSchedule(const std::vector<Step> &steps, bool fuse);
+
 struct Argument {
   enum class Type { Input, Output };
   Type type;
@@ -75,6 +106,8 @@ class LaunchPlan {
   size_t GetInterfaceBytes() const;  // device staging of graph inputs and outputs
   size_t GetPeakDeviceBytes() const { return arena_bytes_ + GetConstantBytes() + GetInterfaceBytes(); }
   const std::vector<Step> &GetSteps() const { return steps_; }
+  // the launches actually replayed (steps grouped into chains when fusion is on)
+  const std::vector<Launch> &GetSchedule() const;
   const std::vector<Argument> &GetArguments() const { return arguments_; }
   // Every arena operand and scratch buffer lies inside [0, arena_bytes); every
   // named constant / interface / private operand exists. Throws std::logic_error otherwise.
@@ -95,7 +128,7 @@ class LaunchPlan {
   size_t Run(const std::unordered_map<std::string, void *> &args, size_t epoch);
   // `n` replays on inputs already resident in HBM, then a stream wait; no host copies.
   void ReplayResident(size_t n);
-  // hipEvent time of every step, median of `iters` runs after `warmup`.
+  // kernel-exact hipEvent duration of every launch of the schedule, median of `iters` runs after `warmup`.
   std::vector<StepTime> Profile(size_t warmup, size_t iters);
   // mean device time of one whole replay measured with events on the plan's stream
   double TimeReplayNs(size_t warmup, size_t iters);
@@ -103,6 +136,8 @@ class LaunchPlan {
   void SetFlags(uint32_t flags) { flags_ = flags; }
   uint32_t GetFlags() const { return flags_; }
   void SetUseGraph(bool use) { use_graph_ = use; }
+  // launch-level fusion of single-reader chains; off whenever literal-reference flags are set
+  void SetFuse(bool fuse) { fuse_ = fuse; }
   // device address of a named interface / constant operand (tests)
   void *GetDeviceAddress(const std::string &name) const;
   void *GetArenaBase() const { return arena_; }
@@ -119,6 +154,8 @@ class LaunchPlan {
     void *device = nullptr;
   };
   void *Resolve(const Operand &op) const;
+  void IssueStep(kernel::LaunchContext &ctx, const Step &s) const;
+  void Issue(kernel::LaunchContext &ctx, const Launch &l) const;
   void LaunchAll(kernel::LaunchContext &ctx) const;
   void Replay(kernel::LaunchContext &ctx);
 
@@ -130,6 +167,9 @@ class LaunchPlan {
   std::map<std::string, RawSlot> privates_, interfaces_;
   uint32_t flags_ = 0;
   bool use_graph_ = true;
+  bool fuse_ = true;
+  mutable std::vector<Launch> schedule_;
+  mutable bool schedule_built_ = false;
   void *arena_ = nullptr;
   void *stream_ = nullptr;
   void *graph_ = nullptr;

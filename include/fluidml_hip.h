@@ -128,6 +128,13 @@ int fluidml_hip_event_create(void **event);
 int fluidml_hip_event_destroy(void *event);
 int fluidml_hip_event_record(void *event, void *stream);
 int fluidml_hip_event_elapsed_ns(void *start, void *stop, double *ns);
+/* Kernel-exact timing for the calling thread: until cleared with (NULL, NULL),
+ * every kernel an entry point below launches stamps `start`/`stop` with the
+ * dispatch's own begin and end, so their elapsed time excludes launch latency
+ * and queue gaps (what eval.cpp:64-100 cannot separate on the CPU).  If one call
+ * launches several kernels the events describe the last one.  Not for use
+ * during launch-plan capture. */
+int fluidml_hip_time_kernels(void *start, void *stop);
 /* Launch-plan capture: the node sequence of one Invoke recorded once and
  * replayed (the counterpart of re-running `_mlir_ciface_<name>`,
  * reference runner.cpp:101-109). */
@@ -269,6 +276,29 @@ int fluidml_hip_conv_without_padding(const fl_tensor *in, const fl_tensor *weigh
  * input in `scratch`; here padding is applied on the fly and scratch is
  * untouched. */
 int fluidml_hip_conv_with_padding(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, void *scratch, size_t scratch_bytes, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, uint32_t flags, void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* Launch-level fusions.  Each computes exactly what the named chain of        */
+/* kernels above computes, operation for operation, without writing the        */
+/* chain's intermediate tensors; the launcher uses them where an intermediate  */
+/* has one reader (the reference fuses at graph level instead, e.g.            */
+/* add_div_erf_add_mul_mul.cpp, and has no launch-level counterpart).          */
+
+/* MatMulKernel -> AddCommonKernel with a rank-1 bias over the last dim
+ * (reference matmul.cpp:28-59 + add.cpp:75-137). */
+int fluidml_hip_matmul_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, void *stream);
+/* MatMulKernel -> AddCommonKernel(bias) -> Div -> Erf -> Add -> Mul -> Mul:
+ * t = lhs.rhs + bias; out = t * (erf(t / div) + add) * mul
+ * (reference matmul.cpp:28-59 + add_div_erf_add_mul_mul.cpp:29-132). */
+int fluidml_hip_matmul_add_div_erf_add_mul_mul(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double div, double add, double mul, void *stream);
+/* DivConstantRhsKernel -> AddCommonKernel(mask, broadcast) -> SoftmaxKernel:
+ * out = softmax(in / div + mask, axis)
+ * (reference div.cpp:24-56 + add.cpp:75-137 + softmax.cpp:22-139). */
+int fluidml_hip_div_add_softmax(const fl_tensor *in, double div, const fl_tensor *mask, const fl_tensor *out, int64_t axis, void *stream);
+/* AddCommonKernel -> LayerNormalizationConstantScaleBiasKernel:
+ * out = LayerNorm(lhs + rhs) (reference add.cpp:75-137 +
+ * layer_normalization.cpp:33-220, ONNX semantics). */
+int fluidml_hip_add_layer_normalization(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *scale, const fl_tensor *bias, const fl_tensor *out, int64_t axis, double epsilon, void *stream);
 
 #ifdef __cplusplus
 }

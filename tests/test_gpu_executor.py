@@ -49,14 +49,21 @@ def _invoke(ex, net, feeds):
 
 @pytest.mark.parametrize("flavour", ["plain_linear", "plain_greedy", "dp_greedy"])
 @pytest.mark.parametrize("graph", [False, True], ids=["launches", "captured"])
-def test_tiny_bert_matches_oracle(device, tiny_bert, flavour, graph, monkeypatch):
+@pytest.mark.parametrize("fuse", [True, False], ids=["fused", "unfused"])
+def test_tiny_bert_matches_oracle(device, tiny_bert, flavour, graph, fuse, monkeypatch):
     fluidml, _ = _mods()
     net, path, feeds, want = tiny_bert
     monkeypatch.setenv("FLUIDML_HIP_GRAPH", "1" if graph else "0")
+    monkeypatch.setenv("FLUIDML_FUSE", "1" if fuse else "0")
     monkeypatch.setenv("FLUIDML_DP_COST", "constant")  # every tensor gets the reversed layout
-    announce("tiny bert", flavour, "graph" if graph else "launches")
+    announce("tiny bert", flavour, "graph" if graph else "launches", "fused" if fuse else "unfused")
     ex = getattr(fluidml.Executor, "make_" + flavour)("tiny_" + flavour, 3)
     ex.compile(path)
+    plan = ex.plan()
+    if fuse:
+        assert len(plan["launches"]) < len(plan["steps"])
+    else:
+        assert len(plan["launches"]) == len(plan["steps"])
     if flavour == "dp_greedy":
         layouts = {s["output"]: s["output_layout"] for s in ex.plan()["steps"]}
         assert any(l != sorted(l) for l in layouts.values()), "DP plan should use non-identity layouts"
@@ -113,8 +120,9 @@ def test_profile_and_accounting(device, tiny_bert):
     assert plan["peak_device_bytes"] == plan["arena_bytes"] + plan["constant_bytes"] + plan["interface_bytes"]
     _invoke(ex, net, feeds)
     times = ex.profile(2, 5)
-    assert len(times) == len(net.nodes)
+    assert len(times) == len(plan["launches"])  # one entry per launch of the schedule
+    assert sum(len(t["node"].split("+")) for t in times) == len(net.nodes)
     assert all(t["ns"] > 0 for t in times)
-    mm = [t for t in times if t["kernel"] == "MatMulKernel"]
+    mm = [t for t in times if t["kernel"].startswith("MatMulKernel")]
     assert mm and all(t["flops"] > 0 for t in mm)
     assert ex.time_replay_ns(2, 5) > 0

@@ -554,6 +554,90 @@ def test_gemm(device):
                 assert_close(do.logical(), ho.logical(), what="gemm")
 
 
+# --------------------------------------------------------------------------- launch-level fusions
+# Each fused entry point is checked against the oracle's UNFUSED chain of kernels.
+
+def test_fused_matmul_add_and_gelu(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(91)
+    for ashape, bshape in [((1, 128, 768), (768, 3072)), ((1, 128, 768), (768, 768)), ((2, 3, 17, 40), (40, 29)),
+                           ((1, 5, 64), (64, 8))]:
+        a, b = rand(rng, ashape, -1, 1), rand(rng, bshape, -0.05, 0.05)
+        oshape = ashape[:-1] + (bshape[-1],)
+        bias = rand(rng, (bshape[-1],), -0.5, 0.5)
+        for la, lb, lo in [(None, None, None), (list(range(len(ashape)))[::-1], [1, 0], list(range(len(oshape)))[::-1])]:
+            announce("fused matmul+add(+gelu)", ashape, bshape, la, lb, lo)
+            ha, hb, hbias = ok.View(a, la), ok.View(b, lb), ok.View(bias)
+            t0, t1 = ok.View.empty(oshape), ok.View.empty(oshape)
+            ok.matmul(ha, hb, t0)
+            ok.binary_f32(ok.BOP_ADD, hbias, t0, t1)  # bias first, like the exported graphs
+            da, db, dbias = DeviceView(ha, device), DeviceView(hb, device), DeviceView(hbias, device)
+            do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
+            cabi.call("matmul_add", da.ref(), db.ref(), dbias.ref(), do.ref(), None)
+            assert_close(do.logical(), t1.logical(), what="matmul_add")
+            # Div -> Erf -> Add -> Mul(t, .) -> Mul
+            u0, u1, u2, u3, u4 = (ok.View.empty(oshape) for _ in range(5))
+            ok.unary_f32(ok.OP_DIV_C, t1, u0, 1.4142135381698608)
+            ok.unary_f32(ok.OP_ERF, u0, u1)
+            ok.unary_f32(ok.OP_ADD_C, u1, u2, 1.0)
+            ok.binary_f32(ok.BOP_MUL, t1, u2, u3)
+            ok.unary_f32(ok.OP_MUL_C, u3, u4, 0.5)
+            do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
+            cabi.call("matmul_add_div_erf_add_mul_mul", da.ref(), db.ref(), dbias.ref(), do.ref(),
+                      ctypes.c_double(1.4142135381698608), ctypes.c_double(1.0), ctypes.c_double(0.5), None)
+            assert_close(do.logical(), u4.logical(), what="matmul_add_div_erf_add_mul_mul")
+
+
+def test_fused_div_add_softmax(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(92)
+    for shape, mshape, axis in [((1, 12, 128, 128), (1, 1, 1, 128), 3), ((2, 3, 9, 70), (2, 1, 9, 70), 3),
+                                ((2, 17, 5), (17, 1), 1), ((4, 1500), (1500,), 1)]:
+        x, mask = rand(rng, shape, -40, 40), rand(rng, mshape, -5, 0)
+        for lin, lout in [(None, None), (list(range(len(shape)))[::-1], None), (None, list(range(len(shape)))[::-1])]:
+            announce("fused div+add+softmax", shape, mshape, axis, lin, lout)
+            hx, hm = ok.View(x, lin), ok.View(mask)
+            t0, t1, ho = ok.View.empty(shape), ok.View.empty(shape), ok.View.empty(shape, np.float32, lout)
+            ok.unary_f32(ok.OP_DIV_C, hx, t0, 8.0)
+            ok.binary_f32(ok.BOP_ADD, t0, hm, t1)
+            ok.softmax(t1, ho, axis)
+            dx, dm = DeviceView(hx, device), DeviceView(hm, device)
+            do = DeviceView(ok.View.empty(shape, np.float32, lout), device)
+            cabi.call("div_add_softmax", dx.ref(), ctypes.c_double(8.0), dm.ref(), do.ref(), ctypes.c_int64(axis), None)
+            assert_close(do.logical(), ho.logical(), what="div_add_softmax")
+    # in place on the input (what the launcher does when the plan put the output over the dead input)
+    x, mask = rand(rng, (1, 4, 64, 64), -40, 40), rand(rng, (1, 1, 1, 64), -5, 0)
+    hx, hm = ok.View(x), ok.View(mask)
+    t0, t1, ho = (ok.View.empty(x.shape) for _ in range(3))
+    ok.unary_f32(ok.OP_DIV_C, hx, t0, 8.0)
+    ok.binary_f32(ok.BOP_ADD, t0, hm, t1)
+    ok.softmax(t1, ho, 3)
+    dx, dm = DeviceView(hx, device), DeviceView(hm, device)
+    announce("fused div+add+softmax in place")
+    cabi.call("div_add_softmax", dx.ref(), ctypes.c_double(8.0), dm.ref(), dx.ref(), ctypes.c_int64(3), None)
+    assert_close(dx.logical(), ho.logical(), what="div_add_softmax in place")
+
+
+def test_fused_add_layer_norm(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(93)
+    for shape, axis, eps in [((1, 128, 768), 2, 1e-12), ((2, 7, 33), 2, 1e-5), ((3, 20, 5), 1, 1e-5), ((2, 5000), 1, 1e-5)]:
+        x, y = rand(rng, shape, -3, 3), rand(rng, shape, -3, 3)
+        g, b = rand(rng, shape[axis:], 0.5, 1.5), rand(rng, shape[axis:], -0.5, 0.5)
+        for lx, ly, lo in [(None, None, None), (list(range(len(shape)))[::-1], None, None),
+                           (None, list(range(len(shape)))[::-1], list(range(len(shape)))[::-1])]:
+            announce("fused add+layer_norm", shape, axis, lx, ly, lo)
+            hx, hy, hg, hb = ok.View(x, lx), ok.View(y, ly), ok.View(g), ok.View(b)
+            t0, ho = ok.View.empty(shape), ok.View.empty(shape, np.float32, lo)
+            ok.binary_f32(ok.BOP_ADD, hx, hy, t0)
+            ok.layer_norm(t0, hg, hb, ho, axis, eps)
+            dx, dy, dg, db = (DeviceView(h, device) for h in (hx, hy, hg, hb))
+            do = DeviceView(ok.View.empty(shape, np.float32, lo), device)
+            cabi.call("add_layer_normalization", dx.ref(), dy.ref(), dg.ref(), db.ref(), do.ref(), ctypes.c_int64(axis),
+                      ctypes.c_double(eps), None)
+            assert_close(do.logical(), ho.logical(), what="add_layer_normalization")
+
+
 CONV_CASES = [
     # x shape, w shape, pads, strides, dilations, group, bias
     ((1, 768, 128), (768, 1, 9), [4, 4], [1], [1], 768, False),  # reference conv0.py (depthwise 1-d, pad 4)

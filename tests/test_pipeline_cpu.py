@@ -266,6 +266,71 @@ def test_golden_bert_base_plan(mods, tmp_path):
         assert items[name] == (offset, size), name
 
 
+# ------------------------------------------------------------------ launch schedule (fusion)
+
+def _overlap(x, y):
+    if x["space"] != y["space"]:
+        return False
+    if x["space"] != "arena":
+        return x["name"] == y["name"]
+    return x["offset"] < y["offset"] + y["bytes"] and y["offset"] < x["offset"] + x["bytes"]
+
+
+@pytest.mark.parametrize("flavour", ["make_plain_greedy", "make_plain_linear", "make_dp_greedy"])
+def test_fused_schedule_is_safe(mods, tiny, flavour, monkeypatch):
+    """Independent re-check of what the launcher's fusion pass must guarantee: every step is issued once,
+    an elided tensor has no reader outside its chain, and moving a chain's reads to its last member's
+    position crosses no write to the bytes it reads (arena intervals of the memory plan)."""
+    fluidml, _, _ = mods
+    _, path = tiny
+    monkeypatch.setenv("FLUIDML_DP_COST", "constant")
+    ex = getattr(fluidml.Executor, flavour)("sched")
+    ex.compile(path)
+    plan = ex.plan()
+    steps, launches = plan["steps"], plan["launches"]
+    assert sorted(m for l in launches for m in l["members"]) == list(range(len(steps)))
+    assert [l["members"][-1] for l in launches] == sorted(l["members"][-1] for l in launches)
+    kinds = {l["kind"] for l in launches}
+    assert {"MatMulAdd", "MatMulAddDivErfAddMulMul", "AddLayerNormalization", "DivAddSoftmax"} <= kinds
+    readers = {}
+    for i, s in enumerate(steps):
+        for op in s["inputs"]:
+            readers.setdefault(op["name"], set()).add(i)
+    for l in launches:
+        members = l["members"]
+        assert members == sorted(members)
+        if l["kind"] == "Step":
+            assert len(members) == 1
+            continue
+        inside = {steps[m]["out"]["name"] for m in members[:-1]}
+        for m in members[:-1]:
+            out = steps[m]["out"]
+            assert out["space"] in ("arena", "private")
+            assert readers[out["name"]] <= set(members), "an elided tensor is read outside its chain"
+        final = steps[members[-1]]["out"]
+        for m in members:
+            for op in steps[m]["inputs"]:
+                if op["name"] in inside:
+                    continue
+                for s in range(m + 1, members[-1]):
+                    if s not in members:
+                        assert not _overlap(steps[s]["out"], op), "a read was moved across a write to its bytes"
+                if _overlap(final, op):  # only the in-place softmax may write over what it reads
+                    assert l["kind"] == "DivAddSoftmax" and final["offset"] == op["offset"] and final["layout"] == op["layout"]
+    # switched off: one launch per step
+    monkeypatch.setenv("FLUIDML_FUSE", "0")
+    ex = getattr(fluidml.Executor, flavour)("sched_off")
+    ex.compile(path)
+    plan = ex.plan()
+    assert [l["members"] for l in plan["launches"]] == [[i] for i in range(len(plan["steps"]))]
+    # literal-reference mode never fuses
+    monkeypatch.setenv("FLUIDML_FUSE", "1")
+    monkeypatch.setenv("FLUIDML_REF_QUIRKS", "4")
+    ex = getattr(fluidml.Executor, flavour)("sched_ref")
+    ex.compile(path)
+    assert len(ex.plan()["launches"]) == len(ex.plan()["steps"])
+
+
 # ------------------------------------------------------------------ layout DP
 
 def test_dp_constant_cost_closed_form(mods, tiny):

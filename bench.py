@@ -2,8 +2,8 @@
 """Benchmark of the hot path: BERT-base encoder (batch 1, seq 128, fp32) compiled by
 Executor.make_dp_greedy-equivalent planning and replayed as HIP launches over one HBM arena.
 
-A "step" is one inference: one replay of the whole launch plan (416 kernels) on inputs that are
-already resident in HBM.  Prints ONE JSON line; see DESIGN.md for how every field is derived.
+A "step" is one inference: one replay of the whole launch plan (416 graph nodes issued as 189 kernel
+launches after launch-level fusion) on inputs that are already resident in HBM.  Prints ONE JSON line; see DESIGN.md for how every field is derived.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--executor plain_greedy|dp_greedy]
                     [--no-cpu-baseline] [--layers 12]
@@ -21,6 +21,12 @@ if ROOT not in sys.path:
 
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per launch of the contraction kernel on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE
+# (KiB per dispatch, averaged over the 96 contraction launches of an inference), each scaled by what the
+# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x1.000): (3912.5 * 2.0 + 576.0) KiB.
+# Only valid for the default workload (BERT-base, seq 128, 12 layers, plain_greedy, fusion on).
+MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 8_601_851
 
 
 def cpu_baseline(layers_total: int, sample_layers: int, seq: int):
@@ -61,6 +67,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-layers", type=int, default=3)
     ap.add_argument("--per-kernel", action="store_true", help="also print a per-kernel table to stderr")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="instead of the benchmark, launch the identity-copy kernel 3 times on a buffer of MIB MiB "
+                         "(a kernel of known traffic, to scale profiler byte counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the reference has no multi-device path); use --gpus 1")
@@ -71,6 +80,24 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     from fluidml_amd import fluidml, models
+
+    if args.copy_calibration:
+        import ctypes
+
+        from fluidml_amd import cabi
+
+        n = args.copy_calibration * (1 << 20) // 4
+        src = torch.ones(n, dtype=torch.float32, device="cuda")
+        dst = torch.zeros(n, dtype=torch.float32, device="cuda")
+        ts = cabi.make_tensor(src.data_ptr(), cabi.FL_FLOAT32, [n], [1])
+        td = cabi.make_tensor(dst.data_ptr(), cabi.FL_FLOAT32, [n], [1])
+        torch.cuda.synchronize()
+        for _ in range(3):
+            cabi.call("dropout", ctypes.byref(ts), ctypes.byref(td), None)
+        torch.cuda.synchronize()
+        assert bool((dst == 1).all())
+        print(json.dumps({"copy_calibration_bytes_read": n * 4, "copy_calibration_bytes_written": n * 4}))
+        return
 
     net = models.bert_base(seq=args.seq, layers=args.layers)
     feeds = models.bert_inputs(args.seq)
@@ -106,9 +133,20 @@ def main():
 
     # per-kernel durations with hipEvent pairs on the plan's stream, same steps
     times = ex.profile(3, min(args.steps, 30))
+    # group launches by the device kernel that runs them: a fused launch is served by the kernel of its
+    # first member (MatMul, MatMul+bias and MatMul+bias+GELU are one MatmulKernel instantiation)
     by_kernel = {}
+    by_launch_kind = {}
     for t in times:
-        k = by_kernel.setdefault(t["kernel"], {"ns": 0.0, "bytes": 0.0, "flops": 0.0, "launches": 0})
+        k = by_launch_kind.setdefault(t["kernel"], {"ns": 0.0, "bytes": 0.0, "flops": 0.0, "launches": 0})
+        k["ns"] += t["ns"]
+        k["bytes"] += t["bytes"]
+        k["flops"] += t["flops"]
+        k["launches"] += 1
+        family = t["kernel"].split("+")[0]
+        if family in ("TransposeKernel", "ReshapeKernel") and "+" in t["kernel"]:
+            family = "ReshapeKernel"
+        k = by_kernel.setdefault(family, {"ns": 0.0, "bytes": 0.0, "flops": 0.0, "launches": 0})
         k["ns"] += t["ns"]
         k["bytes"] += t["bytes"]
         k["flops"] += t["flops"]
@@ -117,8 +155,12 @@ def main():
     dname, d = dominant
     if d["flops"] > 0:
         achieved = d["flops"] / d["ns"] / 1e3  # flop/ns = GFLOP/s -> TFLOP/s
-        roofline = {"bound": "mfma", "kernel": dname, "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
-                    "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
+        default_workload = (args.layers, args.seq, args.executor) == (12, 128, "plain_greedy") and \
+            os.environ.get("FLUIDML_FUSE", "1") != "0"
+        roofline = {"bound": "mfma", "kernel": dname + " (all launches of the contraction kernel, fused epilogues included)",
+                    "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
+                    "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
+                    "traffic": MATMUL_TRAFFIC_BYTES_PER_LAUNCH if default_workload and dname == "MatMulKernel" else None,
                     "avg_launch_us": d["ns"] / d["launches"] / 1e3, "launches_per_step": d["launches"],
                     "flops_per_launch": d["flops"] / d["launches"]}
     else:
@@ -133,7 +175,7 @@ def main():
 
     if args.per_kernel:
         print(f"{'kernel':48s} {'launches':>8s} {'total us':>10s} {'avg us':>8s} {'GB/s':>9s} {'TFLOP/s':>8s}", file=sys.stderr)
-        for name, k in sorted(by_kernel.items(), key=lambda kv: -kv[1]["ns"]):
+        for name, k in sorted(by_launch_kind.items(), key=lambda kv: -kv[1]["ns"]):
             print(f"{name:48s} {k['launches']:8d} {k['ns'] / 1e3:10.1f} {k['ns'] / k['launches'] / 1e3:8.2f} "
                   f"{k['bytes'] / k['ns']:9.1f} {k['flops'] / k['ns'] / 1e3:8.2f}", file=sys.stderr)
 

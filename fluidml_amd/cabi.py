@@ -26,6 +26,7 @@ FL_REF_CONV_BIAS_INDEX1 = 1 << 1
 FL_REF_LN_STALE_SCRATCH = 1 << 2
 FL_REF_GEMM_SWAPPED_SCALARS = 1 << 3
 FL_REF_GATHER_RAW_AXIS = 1 << 4
+FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
 
 DTYPE_SIZE = {FL_BOOL: 1, FL_INT32: 4, FL_INT64: 8, FL_FLOAT16: 2, FL_FLOAT32: 4, FL_FLOAT64: 8}
 
@@ -124,7 +125,7 @@ SIGNATURES = {
     "fluidml_hip_unsqueeze": [_T, _T, _i64p, _i32, _vp],
     "fluidml_hip_slice": [_T, _T, _i64p, _i64p, _i64p, _i32, _vp],
     "fluidml_hip_concat2": [_T, _T, _T, _i64, _vp],
-    "fluidml_hip_pad": [_T, _T, _i64p, _i32, _vp],
+    "fluidml_hip_pad": [_T, _T, _i64p, _i32, _u32, _vp],
     "fluidml_hip_gather_constant_index_scalar": [_T, _T, _i64, _i64, _u32, _vp],
     "fluidml_hip_gather_constant_indices_tensor": [_T, _T, _T, _i64, _vp],
     "fluidml_hip_gather_constant_data_tensor": [_T, _T, _T, _vp],

@@ -323,6 +323,69 @@ int StridedCopy(const fl_tensor *in, int64_t in_offset, const int64_t *in_stride
   return CopyNest(nest, &i2, &o2, stream);
 }
 
+namespace {
+
+// Pad: one lane per output element; inside the interior it copies the input, outside it writes zero.
+struct PadArgs {
+  NestArgs<2> nest;  // dims of the OUTPUT in descending output-stride order; operand 1 = input strides
+  uint32_t lo[kMaxRank], hi[kMaxRank];
+  uint32_t n;
+  int32_t in_base;  // sum lo[d] * input stride[d]
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void PadKernel(PadArgs p, T *__restrict__ out, const T *__restrict__ in) {
+  const uint32_t item = blockIdx.x * 256 + threadIdx.x;
+  if (item >= p.n) return;
+  uint32_t rem = item;
+  int32_t off_out = 0, off_in = 0;
+  bool inside = true;
+  for (int d = p.nest.rank - 1; d >= 0; --d) {
+    uint32_t q = 0, r = rem;
+    if (d > 0) p.nest.div[d].DivMod(rem, q, r);
+    rem = q;
+    off_out += static_cast<int32_t>(r) * p.nest.strides[0][d];
+    off_in += static_cast<int32_t>(r) * p.nest.strides[1][d];
+    inside = inside && r >= p.lo[d] && r < p.hi[d];
+  }
+  out[off_out] = inside ? in[off_in - p.in_base] : T(0);
+}
+
+template <typename T>
+int LaunchPad(const fl_tensor *in, const fl_tensor *out, const int64_t *before, hipStream_t stream) {
+  // dims sorted by descending output stride (innermost loop = fastest output dim), nothing merged
+  int order[kMaxRank];
+  for (int i = 0; i < out->rank; ++i) order[i] = i;
+  for (int i = 1; i < out->rank; ++i) {
+    for (int j = i; j > 0 && out->strides[order[j]] > out->strides[order[j - 1]]; --j) std::swap(order[j], order[j - 1]);
+  }
+  LoopNest nest;
+  nest.n_operands = 2;
+  nest.rank = out->rank;
+  PadArgs p;
+  std::memset(&p, 0, sizeof(p));
+  int64_t total = 1, in_base = 0;
+  for (int k = 0; k < out->rank; ++k) {
+    const int d = order[k];
+    nest.shape[k] = out->shape[d];
+    nest.strides[0][k] = out->strides[d];
+    nest.strides[1][k] = in->strides[d];
+    p.lo[k] = static_cast<uint32_t>(before[d]);
+    p.hi[k] = static_cast<uint32_t>(before[d] + in->shape[d]);
+    in_base += before[d] * in->strides[d];
+    total *= out->shape[d];
+  }
+  if (total == 0) return FL_OK;
+  if (total > 0x7fffffff) return FL_ERR_TOO_LARGE;
+  p.nest = MakeNestArgs<2>(nest);
+  p.n = static_cast<uint32_t>(total);
+  p.in_base = static_cast<int32_t>(in_base);
+  FL_LAUNCH(PadKernel<T>, dim3((p.n + 255) / 256), dim3(256), 0, stream, p, static_cast<T *>(out->base),
+            static_cast<const T *>(in->base));
+  return LaunchStatus();
+}
+
+}  // namespace
 }  // namespace fl
 
 using namespace fl;
@@ -619,17 +682,27 @@ int fluidml_hip_concat2(const fl_tensor *lhs, const fl_tensor *rhs, const fl_ten
                      out->strides, stream);
 }
 
-int fluidml_hip_pad(const fl_tensor *in, const fl_tensor *out, const int64_t *pads_before, int32_t n, void *stream) {
+int fluidml_hip_pad(const fl_tensor *in, const fl_tensor *out, const int64_t *pads_before, int32_t n, uint32_t flags,
+                    void *stream) {
   FL_CHECK(CheckView(in));
   FL_CHECK(CheckView(out));
   if (in->rank != out->rank || n != in->rank) return FL_ERR_RANK;
+  if (in->dtype != out->dtype) return FL_ERR_DTYPE;
   if (pads_before == nullptr && n > 0) return FL_ERR_NULL;
   int64_t out_offset = 0;
   for (int i = 0; i < in->rank; ++i) {
     if (pads_before[i] < 0 || pads_before[i] + in->shape[i] > out->shape[i]) return FL_ERR_SHAPE;
     out_offset += pads_before[i] * out->strides[i];
   }
-  return StridedCopy(in, 0, in->strides, out, out_offset, in->rank, in->shape, out->strides, stream);
+  if (flags & FL_REF_PAD_BORDER_UNWRITTEN) {
+    return StridedCopy(in, 0, in->strides, out, out_offset, in->rank, in->shape, out->strides, stream);
+  }
+  switch (DtypeSize(in->dtype)) {
+    case 1: return LaunchPad<uint8_t>(in, out, pads_before, AsStream(stream));
+    case 4: return LaunchPad<uint32_t>(in, out, pads_before, AsStream(stream));
+    case 8: return LaunchPad<uint64_t>(in, out, pads_before, AsStream(stream));
+    default: return FL_ERR_DTYPE;
+  }
 }
 
 int fluidml_hip_gather_constant_index_scalar(const fl_tensor *in, const fl_tensor *out, int64_t axis, int64_t index,

@@ -150,7 +150,7 @@ class SingleNoBuffer final : public SingleInputWithoutBufferKernel, public Base 
       case OpKind::Pad: {
         std::vector<int64_t> before;
         for (const auto &p : a.pad_pairs) before.push_back(std::get<0>(p));
-        rc = fluidml_hip_pad(in, out, before.data(), static_cast<int32_t>(before.size()), s);
+        rc = fluidml_hip_pad(in, out, before.data(), static_cast<int32_t>(before.size()), ctx.flags, s);
         break;
       }
       case OpKind::ReduceMean: {

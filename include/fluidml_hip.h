@@ -80,7 +80,11 @@ enum fl_ref_flags {
   FL_REF_GEMM_SWAPPED_SCALARS = 1 << 3,
   /* GatherConstantIndexScalar compares against the un-normalised axis
    * (reference gather.cpp:116). */
-  FL_REF_GATHER_RAW_AXIS = 1 << 4
+  FL_REF_GATHER_RAW_AXIS = 1 << 4,
+  /* Pad copies the input into the interior and never writes the border, which
+   * keeps whatever the arena held (reference pad.cpp:33-51 writes through a
+   * subview only); without the flag the border is written as zero. */
+  FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
 };
 
 typedef struct fl_tensor {
@@ -219,9 +223,10 @@ int fluidml_hip_unsqueeze(const fl_tensor *in, const fl_tensor *out, const int64
 int fluidml_hip_slice(const fl_tensor *in, const fl_tensor *out, const int64_t *starts, const int64_t *axes, const int64_t *steps, int32_t n, void *stream);
 /* Concat2Kernel (reference concat.cpp:18-68). */
 int fluidml_hip_concat2(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, int64_t axis, void *stream);
-/* PadKernel: copies the input into the interior; the border is not written
- * (reference pad.cpp:15-51). `pads_before[i]` per dimension. */
-int fluidml_hip_pad(const fl_tensor *in, const fl_tensor *out, const int64_t *pads_before, int32_t n, void *stream);
+/* PadKernel: input copied into the interior, border written as zero (ONNX
+ * constant mode, value 0); with FL_REF_PAD_BORDER_UNWRITTEN only the interior
+ * is written (reference pad.cpp:15-51). `pads_before[i]` per dimension. */
+int fluidml_hip_pad(const fl_tensor *in, const fl_tensor *out, const int64_t *pads_before, int32_t n, uint32_t flags, void *stream);
 /* GatherConstantIndexScalarKernel (reference gather.cpp:100-139). */
 int fluidml_hip_gather_constant_index_scalar(const fl_tensor *in, const fl_tensor *out, int64_t axis, int64_t index, uint32_t flags, void *stream);
 /* GatherConstantIndicesTensorKernel: data is the runtime input, `indices` a

@@ -119,7 +119,7 @@ def run_graph(net, feeds: Dict[str, np.ndarray], flags: int = 0, timings: Option
             ok.concat2(ok.View(val(ins[0])), ok.View(val(ins[1])), o, a["axis"] % len(out.shape))
         elif op == "Pad":
             p = [int(v) for v in val(ins[1])]
-            ok.pad(ok.View(val(ins[0])), o, p[: len(p) // 2])
+            ok.pad(ok.View(val(ins[0])), o, p[: len(p) // 2], flags & (1 << 5))
         elif op == "Softmax":
             ok.softmax(ok.View(val(ins[0])), o, a.get("axis", -1) % len(out.shape))
         elif op == "LayerNormalization":

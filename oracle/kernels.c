@@ -230,14 +230,17 @@ int oracle_unsqueeze_sub_mul(const view *in, const view *out, const int64_t *axe
 
 /* ---- data movement ---------------------------------------------------------------- */
 
-static void copy_elem(const view *dst, int64_t doff, const view *src, int64_t soff) {
-  size_t esz;
-  switch (src->dtype) {
-    case FL_BOOL: esz = 1; break;
-    case FL_FLOAT16: esz = 2; break;
-    case FL_INT32: case FL_FLOAT32: esz = 4; break;
-    default: esz = 8; break;
+static size_t dtype_size(int32_t dtype) {
+  switch (dtype) {
+    case FL_BOOL: return 1;
+    case FL_FLOAT16: return 2;
+    case FL_INT32: case FL_FLOAT32: return 4;
+    default: return 8;
   }
+}
+
+static void copy_elem(const view *dst, int64_t doff, const view *src, int64_t soff) {
+  const size_t esz = dtype_size(src->dtype);
   memcpy((char *)dst->base + doff * (int64_t)esz, (const char *)src->base + soff * (int64_t)esz, esz);
 }
 
@@ -339,9 +342,16 @@ int oracle_concat2(const view *lhs, const view *rhs, const view *out, int64_t ax
 }
 
 /* pad.cpp:15-51: input copied into the interior; the border is left as it was */
-int oracle_pad(const view *in, const view *out, const int64_t *pads_before) {
+int oracle_pad(const view *in, const view *out, const int64_t *pads_before, uint32_t flags) {
   int64_t idx[FL_MAX_RANK] = {0};
   int64_t base = 0;
+  if (!(flags & FL_REF_PAD_BORDER_UNWRITTEN)) {
+    /* ONNX constant mode with value 0: every output element starts as zero */
+    const size_t esz = dtype_size(out->dtype);
+    do {
+      memset((char *)out->base + offset_of(out, idx) * (int64_t)esz, 0, esz);
+    } while (next_index(out->rank, out->shape, idx));
+  }
   for (int i = 0; i < in->rank; ++i) base += pads_before[i] * out->strides[i];
   do {
     copy_elem(out, base + offset_of(out, idx), in, offset_of(in, idx));

@@ -174,8 +174,9 @@ def concat2(a, b, out, axis):
     _call("oracle_concat2", _ref(a), _ref(b), _ref(out), i64(axis))
 
 
-def pad(x, out, pads_before):
-    _call("oracle_pad", _ref(x), _ref(out), _i64(pads_before))
+def pad(x, out, pads_before, flags=0):
+    """flags = 0: border written as zero; FL_REF_PAD_BORDER_UNWRITTEN (1 << 5): border left as it is"""
+    _call("oracle_pad", _ref(x), _ref(out), _i64(pads_before), u32(flags))
 
 
 def gather_index_scalar(x, out, axis, index, flags=0):

@@ -320,13 +320,17 @@ def test_squeeze_unsqueeze_slice_concat_pad(device):
         cabi.call("concat2", da.ref(), db.ref(), do.ref(), ctypes.c_int64(3), None)
         assert_close(do.logical(), ho.logical(), exact=True, what="concat2")
     p = rand(rng, (2, 3, 5))
-    hp, ho = ok.View(p), ok.View.empty((2, 4, 8), np.float32, [2, 0, 1], fill=7)
-    ok.pad(hp, ho, [0, 1, 2])
-    dp = DeviceView(hp, device)
-    do = DeviceView(ok.View.empty((2, 4, 8), np.float32, [2, 0, 1], fill=7), device)
-    announce("pad")
-    cabi.call("pad", dp.ref(), do.ref(), cabi.i64_array([0, 1, 2]), 3, None)
-    assert_close(do.logical(), ho.logical(), exact=True, what="pad (border untouched)")
+    for flags, what in ((0, "pad (zero border)"), (cabi.FL_REF_PAD_BORDER_UNWRITTEN, "pad (border untouched)")):
+        for lin, lout in (([0, 1, 2], [2, 0, 1]), ([1, 2, 0], [0, 1, 2])):
+            hp, ho = ok.View(p, lin), ok.View.empty((2, 4, 8), np.float32, lout, fill=7)
+            ok.pad(hp, ho, [0, 1, 2], flags)
+            if flags == 0:
+                assert (ho.logical() == np.pad(p, [(0, 0), (1, 0), (2, 1)])).all()
+            dp = DeviceView(hp, device)
+            do = DeviceView(ok.View.empty((2, 4, 8), np.float32, lout, fill=7), device)
+            announce(what, lin, lout)
+            cabi.call("pad", dp.ref(), do.ref(), cabi.i64_array([0, 1, 2]), 3, ctypes.c_uint32(flags), None)
+            assert_close(do.logical(), ho.logical(), exact=True, what=what)
 
 
 def test_gathers(device):

@@ -1,0 +1,52 @@
+"""Whole-graph GPU parity for the other benchmark configurations (ConvBERT, GPT-NeoX prefill,
+EfficientNet-B0, VGG-16) at reduced width/depth: Executor.compile + invoke against the oracle's
+graph runner on the same seeded weights and inputs, with the reference's plain layouts and with
+DP-chosen (reversed) layouts.  The full-size graphs only differ in extents; their plans are frozen
+by the CPU suite and their throughput is reported by bench.py --config."""
+import sys
+
+import numpy as np
+import pytest
+
+from oracle import graph_runner
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _cases():
+    from fluidml_amd import models
+
+    return {
+        "convbert": (lambda: models.convbert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32),
+                     lambda: models.bert_inputs(16, 100, seed=7)),
+        "gpt_neox": (lambda: models.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120),
+                     lambda: models.gpt_neox_inputs(24, 120, seed=8)),
+        "efficientnet_b0": (lambda: models.efficientnet_b0(image=64, classes=10, width_div=4),
+                            lambda: models.image_input((1, 3, 64, 64), seed=9)),
+        "vgg16": (lambda: models.vgg16(batch=2, image=32, classes=10, width_div=8, fc=512),
+                  lambda: models.image_input((2, 3, 32, 32), seed=10)),
+    }
+
+
+@pytest.mark.parametrize("flavour", ["plain_greedy", "dp_greedy"])
+@pytest.mark.parametrize("config", ["convbert", "gpt_neox", "efficientnet_b0", "vgg16"])
+def test_config_matches_oracle(device, config, flavour, tmp_path, monkeypatch):
+    from fluidml_amd import fluidml
+
+    make_net, make_feeds = _cases()[config]
+    net, feeds = make_net(), make_feeds()
+    want = graph_runner.run_graph(net, feeds)
+    path = net.save(str(tmp_path / f"{config}.onnx"))
+    monkeypatch.setenv("FLUIDML_DP_COST", "constant")
+    print("[case]", config, flavour, len(net.nodes), "nodes", flush=True)
+    sys.stdout.flush()
+    ex = getattr(fluidml.Executor, "make_" + flavour)(config, 2)
+    ex.compile(path)
+    args = {k: np.ascontiguousarray(v) for k, v in feeds.items()}
+    outs = {v.name: np.full(v.shape, np.nan, dtype=v.dtype) for v in net.outputs}
+    args.update(outs)
+    for _ in range(2):
+        assert ex.invoke(args) > 0
+        for name, ref in want.items():
+            assert_close(outs[name], ref, what=f"{config} {flavour} {name}")

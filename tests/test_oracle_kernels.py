@@ -168,10 +168,13 @@ def test_data_movement():
     assert (ho.logical() == np.concatenate([a, b], axis=1)).all()
     p = rand(rng, (2, 3, 5))
     ho = ok.View.empty((2, 4, 8), np.float32, [2, 0, 1], fill=7)
-    ok.pad(ok.View(p), ho, [0, 1, 2])
+    ok.pad(ok.View(p), ho, [0, 1, 2], 1 << 5)  # FL_REF_PAD_BORDER_UNWRITTEN
     want = np.full((2, 4, 8), 7, np.float32)
     want[:, 1:4, 2:7] = p  # border keeps its previous contents (reference pad.cpp:15-51)
     assert (ho.logical() == want).all()
+    ho = ok.View.empty((2, 4, 8), np.float32, [2, 0, 1], fill=7)
+    ok.pad(ok.View(p, [1, 0, 2]), ho, [0, 1, 2])  # default: ONNX constant mode, value 0
+    assert (ho.logical() == np.pad(p, [(0, 0), (1, 0), (2, 1)])).all()
 
 
 def test_gathers():

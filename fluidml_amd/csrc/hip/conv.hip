@@ -111,6 +111,14 @@ __global__ __launch_bounds__(kBlock) void ConvDirect(ConvArgs p, float *__restri
   out[ooff] = acc;
 }
 
+}  // namespace
+
+// matmul.hip
+int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
+                     const int64_t *pads, const int64_t *strides, const int64_t *dilations, void *stream);
+
+namespace {
+
 int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
          const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, uint32_t flags,
          void *stream) {
@@ -167,6 +175,11 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
       if (F < 2) return FL_ERR_SHAPE;
       p.bias_fixed = 1;
     }
+  }
+  // dense contractions go to the matrix cores; depthwise, 3-d and literal-reference modes stay here
+  if (!depthwise && flags == 0 && ns <= 2) {
+    const int rc = ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, stream);
+    if (rc != FL_ERR_UNSUPPORTED) return rc;
   }
   LoopNest nest;
   nest.rank = rank;

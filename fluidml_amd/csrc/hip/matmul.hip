@@ -32,6 +32,18 @@ namespace {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
+// Geometry of a convolution run as an implicit GEMM: M = output channels, N = images x output pixels,
+// K = input channels x kernel taps.  B[k][n] is gathered from the input on the fly (padding reads as 0),
+// C[m][n] is scattered to out[image, m, oh, ow].  1-d convolutions use H = OH = KH = 1.
+struct ConvGeom {
+  int32_t H, W;                  // input extents
+  int32_t sh, sw, dh, dw, ph, pw;
+  int32_t sXn, sXc, sXh, sXw;    // input element strides
+  int32_t sOn, sOh, sOw;         // output element strides (the channel stride is sCm)
+  FastDiv div_ohw, div_ow;       // n -> (image, oh, ow)
+  FastDiv div_khw, div_kw;       // k -> (channel, kh, kw)
+};
+
 struct MatmulArgs {
   int32_t M, N, K;
   int32_t sAm, sAk, sBk, sBn, sCm, sCn;
@@ -44,6 +56,7 @@ struct MatmulArgs {
   // optional activation after the bias: v * (erf(v / g_div) + g_add) * g_mul  (the erf-GELU chain)
   int32_t act;
   float g_div, g_add, g_mul;
+  ConvGeom conv;  // read by the CONV instantiations only
 };
 
 template <int VEC>
@@ -108,7 +121,8 @@ struct TileLoader {
 
 // LA: 0 = A tile kept [m][k] (A is k-contiguous), 1 = kept [k][m].
 // LB: 0 = B tile kept [k][n] (B is n-contiguous), 1 = kept [n][k].
-template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH>
+// CONV: B is the input of a convolution addressed through p.conv (LB must be 0, scalar gathers).
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV = false>
 __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, float *__restrict__ C,
                                                                 const float *__restrict__ A,
                                                                 const float *__restrict__ B) {
@@ -125,8 +139,10 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   constexpr int LDS_ELEMS = STAGE_ELEMS > RED_ELEMS ? STAGE_ELEMS : RED_ELEMS;
   __shared__ __attribute__((aligned(16))) float lds[LDS_ELEMS];
 
+  constexpr int VB = CONV ? 1 : VEC;
+  static_assert(!CONV || (LB == 0 && NT % BN == 0), "the gather keeps one output pixel per thread");
   using LoaderA = typename std::conditional<LA == 0, TileLoader<BM, BK, VEC, NT>, TileLoader<BK, BM, VEC, NT>>::type;
-  using LoaderB = typename std::conditional<LB == 0, TileLoader<BK, BN, VEC, NT>, TileLoader<BN, BK, VEC, NT>>::type;
+  using LoaderB = typename std::conditional<LB == 0, TileLoader<BK, BN, VB, NT>, TileLoader<BN, BK, VB, NT>>::type;
 
   // ---- which tile -----------------------------------------------------------
   uint32_t bid = blockIdx.x;
@@ -152,7 +168,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
     for (int o = 0; o < 3; ++o) boff[o] += static_cast<int32_t>(rem) * p.batch.strides[o][0];
   }
   const float *Ab = A + boff[1] + static_cast<int64_t>(m0) * p.sAm;
-  const float *Bb = B + boff[2] + static_cast<int64_t>(n0) * p.sBn;
+  const float *Bb = CONV ? B : B + boff[2] + static_cast<int64_t>(n0) * p.sBn;
   float *Cb = C + boff[0];
 
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
@@ -171,24 +187,58 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   // consumed, so a workgroup keeps DEPTH * (A tile + B tile) bytes outstanding instead of one chunk --
   // with only a few workgroups per CU that is what hides the L2/HBM latency.
   static_assert(DEPTH % 2 == 0, "the LDS buffer index must be a compile-time function of the stage");
-  VecF<VEC> ra[DEPTH][LoaderA::kPerThread], rb[DEPTH][LoaderB::kPerThread];
+  VecF<VEC> ra[DEPTH][LoaderA::kPerThread];
+  VecF<VB> rb[DEPTH][LoaderB::kPerThread];
   const int rows_m = p.M - m0, cols_n = p.N - n0;
   const int n_chunks = (p.K + BK - 1) / BK;
 
-  auto load_chunk = [&](int c, VecF<VEC>(&qa)[LoaderA::kPerThread], VecF<VEC>(&qb)[LoaderB::kPerThread]) {
+  // convolution: the output pixel this thread gathers for stays the same for the whole kernel
+  bool g_valid = false;
+  int32_t g_ih0 = 0, g_iw0 = 0, g_base = 0;
+  if constexpr (CONV) {
+    const int n = n0 + static_cast<int>(threadIdx.x % BN);
+    g_valid = n < p.N;
+    uint32_t img, r, oh, ow;
+    p.conv.div_ohw.DivMod(static_cast<uint32_t>(g_valid ? n : 0), img, r);
+    p.conv.div_ow.DivMod(r, oh, ow);
+    g_ih0 = static_cast<int32_t>(oh) * p.conv.sh - p.conv.ph;
+    g_iw0 = static_cast<int32_t>(ow) * p.conv.sw - p.conv.pw;
+    g_base = static_cast<int32_t>(img) * p.conv.sXn;
+  }
+
+  auto load_chunk = [&](int c, VecF<VEC>(&qa)[LoaderA::kPerThread], VecF<VB>(&qb)[LoaderB::kPerThread]) {
     const int k0 = c * BK, k_valid = p.K - k0;
     if constexpr (LA == 0) {
       LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAm, p.sAk, rows_m, k_valid, qa);
     } else {
       LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAk, p.sAm, k_valid, rows_m, qa);
     }
-    if constexpr (LB == 0) {
+    if constexpr (CONV) {
+      // same item -> (k row, n column) mapping as TileLoader<BK, BN, 1, NT>: column = thread % BN
+#pragma unroll
+      for (int j = 0; j < LoaderB::kPerThread; ++j) {
+        const int k = k0 + static_cast<int>(threadIdx.x / BN) + j * (NT / BN);
+        float v = 0.0f;
+        if (g_valid && k < p.K) {
+          uint32_t ci, r, kh, kw;
+          p.conv.div_khw.DivMod(static_cast<uint32_t>(k), ci, r);
+          p.conv.div_kw.DivMod(r, kh, kw);
+          const int32_t ih = g_ih0 + static_cast<int32_t>(kh) * p.conv.dh;
+          const int32_t iw = g_iw0 + static_cast<int32_t>(kw) * p.conv.dw;
+          if (static_cast<uint32_t>(ih) < static_cast<uint32_t>(p.conv.H) &&
+              static_cast<uint32_t>(iw) < static_cast<uint32_t>(p.conv.W)) {
+            v = B[g_base + static_cast<int32_t>(ci) * p.conv.sXc + ih * p.conv.sXh + iw * p.conv.sXw];
+          }
+        }
+        qb[j].v[0] = v;
+      }
+    } else if constexpr (LB == 0) {
       LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBk, p.sBn, k_valid, cols_n, qb);
     } else {
       LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBn, p.sBk, cols_n, k_valid, qb);
     }
   };
-  auto store_chunk = [&](int buf, const VecF<VEC>(&qa)[LoaderA::kPerThread], const VecF<VEC>(&qb)[LoaderB::kPerThread]) {
+  auto store_chunk = [&](int buf, const VecF<VEC>(&qa)[LoaderA::kPerThread], const VecF<VB>(&qb)[LoaderB::kPerThread]) {
     float *as = lds + buf * (A_ELEMS + B_ELEMS);
     float *bs = as + A_ELEMS;
     LoaderA::Store(as, LDA, qa);
@@ -298,6 +348,14 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = n0 + (wn * TN + j) * 32 + lrow;
+      int64_t col = static_cast<int64_t>(n) * p.sCn;
+      if constexpr (CONV) {
+        uint32_t img, r, oh, ow;
+        p.conv.div_ohw.DivMod(static_cast<uint32_t>(n < p.N ? n : 0), img, r);
+        p.conv.div_ow.DivMod(r, oh, ow);
+        col = static_cast<int64_t>(img) * p.conv.sOn + static_cast<int64_t>(oh) * p.conv.sOh +
+              static_cast<int64_t>(ow) * p.conv.sOw;
+      }
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
@@ -309,31 +367,39 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
           if (p.act != 0) {
             v = (v * (erff(v / p.g_div) + p.g_add)) * p.g_mul;
           }
-          Cb[static_cast<int64_t>(m) * p.sCm + static_cast<int64_t>(n) * p.sCn] = v;
+          Cb[static_cast<int64_t>(m) * p.sCm + col] = v;
         }
       }
     }
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH>
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV>
 void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   MatmulArgs q = p;
   q.tiles_m = (p.M + BM - 1) / BM;
   q.tiles_n = (p.N + BN - 1) / BN;
-  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH>), dim3(q.tiles_m * q.tiles_n, n_batch),
+  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV>), dim3(q.tiles_m * q.tiles_n, n_batch),
                      dim3(64 * WM * WN * KS), 0, s, q, C, A, B);
 }
 
-template <int LA, int LB, int VEC>
+// Useful fraction of the MFMA work when the problem is cut into bm x bn tiles.
+inline double TileEfficiency(int64_t m, int64_t n, int64_t bm, int64_t bn) {
+  return static_cast<double>(m) * static_cast<double>(n) /
+         (static_cast<double>((m + bm - 1) / bm * bm) * static_cast<double>((n + bn - 1) / bn * bn));
+}
+
+template <int LA, int LB, int VEC, bool CONV>
 void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   const int64_t tiles_l = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * n_batch;
   const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
-  if (tiles_l >= 192) {
-    LaunchConfig<128, 128, 16, 2, 2, 1, LA, LB, VEC, 2>(p, n_batch, C, A, B, s);
+  // the big tile only when it fills the chip and does not waste much more of itself on edges than the next one
+  const bool big_ok = tiles_l >= 192 && TileEfficiency(p.M, p.N, 128, 128) + 0.15 >= TileEfficiency(p.M, p.N, 64, 64);
+  if (big_ok) {
+    LaunchConfig<128, 128, 16, 2, 2, 1, LA, LB, VEC, 2, CONV>(p, n_batch, C, A, B, s);
   } else if (tiles_m >= 192) {
-    LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4>(p, n_batch, C, A, B, s);
+    LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4, CONV>(p, n_batch, C, A, B, s);
   } else {
-    LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2>(p, n_batch, C, A, B, s);
+    LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2, CONV>(p, n_batch, C, A, B, s);
   }
 }
 
@@ -441,8 +507,8 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   const uint32_t nb = static_cast<uint32_t>(n_batch);
 #define FL_MM_DISPATCH(LA_, LB_)                              \
   if (la == LA_ && lb == LB_) {                               \
-    if (vec) LaunchBySize<LA_, LB_, 4>(p, nb, C, A, B, s);    \
-    else LaunchBySize<LA_, LB_, 1>(p, nb, C, A, B, s);        \
+    if (vec) LaunchBySize<LA_, LB_, 4, false>(p, nb, C, A, B, s); \
+    else LaunchBySize<LA_, LB_, 1, false>(p, nb, C, A, B, s);     \
   }
   FL_MM_DISPATCH(0, 0)
   FL_MM_DISPATCH(0, 1)
@@ -453,6 +519,83 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
 }
 
 }  // namespace
+
+// Convolution with group == 1 and one or two spatial dims as an implicit GEMM on the matrix cores.
+// Returns FL_ERR_UNSUPPORTED (nothing launched) when the operands do not fit this path: the caller then
+// uses the direct kernel.  `pads` may be null; `strides`/`dilations` have one entry per spatial dim.
+int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
+                     const int64_t *pads, const int64_t *strides, const int64_t *dilations, void *stream) {
+  const int ns = out->rank - 2;
+  if (ns != 1 && ns != 2) return FL_ERR_UNSUPPORTED;
+  const int hd = ns == 2 ? 2 : -1, wd = ns == 2 ? 3 : 2;  // dims of H (absent for 1-d) and W
+  const int64_t KH = ns == 2 ? weights->shape[2] : 1, KW = weights->shape[wd];
+  const int64_t Cc = in->shape[1], F = out->shape[1];
+  const int64_t OH = ns == 2 ? out->shape[2] : 1, OW = out->shape[wd];
+  const int64_t n_total = out->shape[0] * OH * OW, k_total = Cc * KH * KW;
+  if (n_total > 0x7fffffff || k_total > 0x7fffffff || n_total == 0 || F == 0) return FL_ERR_UNSUPPORTED;
+  // A = weights as an [F][K] matrix: (c, kh, kw) must be one strided run
+  const int64_t s_kw = weights->strides[wd];
+  if (ns == 2 && KH > 1 && weights->strides[2] != KW * s_kw) return FL_ERR_UNSUPPORTED;
+  if (Cc > 1 && weights->strides[1] != KH * KW * s_kw) return FL_ERR_UNSUPPORTED;
+  if (Numel(in) > 0x7fffffff || Numel(out) > 0x7fffffff) return FL_ERR_UNSUPPORTED;
+
+  MatmulArgs p;
+  std::memset(&p, 0, sizeof(p));
+  p.M = static_cast<int32_t>(F);
+  p.N = static_cast<int32_t>(n_total);
+  p.K = static_cast<int32_t>(k_total);
+  p.sAm = static_cast<int32_t>(weights->strides[0]);
+  p.sAk = static_cast<int32_t>(s_kw);
+  p.sCm = static_cast<int32_t>(out->strides[1]);
+  p.sCn = 0;
+  p.batch.rank = 0;
+  p.ca = 1.0f;
+  p.cb = 1.0f;
+  if (bias != nullptr) {
+    p.bias = static_cast<const float *>(bias->base);
+    p.sDm = static_cast<int32_t>(bias->strides[0]);
+    p.sDn = 0;
+  }
+  ConvGeom &g = p.conv;
+  g.H = ns == 2 ? static_cast<int32_t>(in->shape[2]) : 1;
+  g.W = static_cast<int32_t>(in->shape[wd]);
+  g.sh = ns == 2 && strides ? static_cast<int32_t>(strides[0]) : 1;
+  g.sw = strides ? static_cast<int32_t>(strides[ns - 1]) : 1;
+  g.dh = ns == 2 && dilations ? static_cast<int32_t>(dilations[0]) : 1;
+  g.dw = dilations ? static_cast<int32_t>(dilations[ns - 1]) : 1;
+  g.ph = ns == 2 && pads ? static_cast<int32_t>(pads[0]) : 0;
+  g.pw = pads ? static_cast<int32_t>(pads[ns - 1]) : 0;
+  g.sXn = static_cast<int32_t>(in->strides[0]);
+  g.sXc = static_cast<int32_t>(in->strides[1]);
+  g.sXh = ns == 2 ? static_cast<int32_t>(in->strides[2]) : 0;
+  g.sXw = static_cast<int32_t>(in->strides[wd]);
+  g.sOn = static_cast<int32_t>(out->strides[0]);
+  g.sOh = ns == 2 ? static_cast<int32_t>(out->strides[2]) : 0;
+  g.sOw = static_cast<int32_t>(out->strides[wd]);
+  g.div_ohw = FastDiv(static_cast<uint32_t>(OH * OW));
+  g.div_ow = FastDiv(static_cast<uint32_t>(OW));
+  g.div_khw = FastDiv(static_cast<uint32_t>(KH * KW));
+  g.div_kw = FastDiv(static_cast<uint32_t>(KW));
+  (void)hd;
+
+  float *C = static_cast<float *>(out->base);
+  const float *A = static_cast<const float *>(weights->base);
+  const float *B = static_cast<const float *>(in->base);
+  hipStream_t s = AsStream(stream);
+  const int la = (p.sAk <= p.sAm || p.M == 1) ? 0 : 1;
+  bool vec = IsAligned(A, 16);
+  if (la == 0) vec = vec && (p.sAk == 1 || p.K == 1) && p.K % 4 == 0 && p.sAm % 4 == 0;
+  else vec = vec && p.sAm == 1 && p.M % 4 == 0 && p.sAk % 4 == 0;
+  if (la == 0) {
+    if (vec) LaunchBySize<0, 0, 4, true>(p, 1, C, A, B, s);
+    else LaunchBySize<0, 0, 1, true>(p, 1, C, A, B, s);
+  } else {
+    if (vec) LaunchBySize<1, 0, 4, true>(p, 1, C, A, B, s);
+    else LaunchBySize<1, 0, 1, true>(p, 1, C, A, B, s);
+  }
+  return LaunchStatus();
+}
+
 }  // namespace fl
 
 extern "C" {

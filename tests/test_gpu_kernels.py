@@ -689,6 +689,26 @@ def test_conv(device, case):
                 assert_close(do.logical(), ho.logical(), what=f"conv flags={flags}")
 
 
+def test_conv_large_tiles(device):
+    """Shapes that select the 64x64 and 128x128 workgroup tiles of the implicit-GEMM path, and a weight
+    tensor whose layout is not (c, kh, kw)-contiguous, which has to take the direct kernel."""
+    cabi = _cabi()
+    rng = np.random.default_rng(79)
+    for xshape, wshape, lw in [((2, 8, 64, 64), (128, 8, 3, 3), None), ((4, 8, 64, 64), (256, 8, 3, 3), None),
+                               ((1, 8, 20, 20), (16, 8, 3, 3), [3, 2, 1, 0])]:
+        x, w, bias = rand(rng, xshape, -1, 1), rand(rng, wshape, -0.05, 0.05), rand(rng, (wshape[0],), -1, 1)
+        oshape = (xshape[0], wshape[0]) + xshape[2:]
+        for lx, lo in [(None, None), ([0, 3, 1, 2], [0, 3, 1, 2])]:  # NCHW and channels-last storage
+            announce("conv large", xshape, wshape, lx, lo, lw)
+            hx, hw, hb, ho = ok.View(x, lx), ok.View(w, lw), ok.View(bias), ok.View.empty(oshape, np.float32, lo)
+            ok.conv(hx, hw, hb, ho, [1, 1, 1, 1], [1, 1], [1, 1], 1, 0)
+            dx, dw, db = DeviceView(hx, device), DeviceView(hw, device), DeviceView(hb, device)
+            do = DeviceView(ok.View.empty(oshape, np.float32, lo), device)
+            cabi.call("conv_with_padding", dx.ref(), dw.ref(), db.ref(), do.ref(), None, 0, cabi.i64_array([1, 1, 1, 1]),
+                      cabi.i64_array([1, 1]), cabi.i64_array([1, 1]), ctypes.c_int64(1), ctypes.c_uint32(0), None)
+            assert_close(do.logical(), ho.logical(), what="conv large")
+
+
 def test_argument_errors(device):
     """Rejected arguments return negative codes and launch nothing."""
     cabi = _cabi()

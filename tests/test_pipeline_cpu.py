@@ -266,6 +266,22 @@ def test_golden_bert_base_plan(mods, tmp_path):
         assert items[name] == (offset, size), name
 
 
+@pytest.mark.parametrize("config", ["convbert_base_s128", "gpt_neox_s256", "efficientnet_b0", "vgg16_b1", "vgg16_b8"])
+def test_golden_config_plans(mods, tmp_path, config):
+    """Arena plans of the other benchmark configurations at full size, frozen like the BERT-base one."""
+    import importlib.util
+
+    here = os.path.join(os.path.dirname(__file__), "golden")
+    spec = importlib.util.spec_from_file_location("make_plan_fixture", os.path.join(here, "make_plan_fixture.py"))
+    fixture = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(fixture)
+    golden = json.load(open(os.path.join(here, "config_plans.json")))[config]
+    got = fixture.plan_of(fixture.CONFIGS[config][1](), str(tmp_path))
+    for key in ("nodes", "arena_bytes", "offsets_crc32", "order_crc32"):
+        assert got[key] == golden[key], key
+    assert got["sample"] == {k: list(v) for k, v in golden["sample"].items()}
+
+
 # ------------------------------------------------------------------ launch schedule (fusion)
 
 def _overlap(x, y):

@@ -142,7 +142,10 @@ SIGNATURES = {
     "fluidml_hip_matmul_bf16": [_T, _T, _T, _vp],
     "fluidml_hip_gemm_constant_weights_bias": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _u32, _vp],
     "fluidml_hip_matmul_add": [_T, _T, _T, _T, _vp],
-    "fluidml_hip_matmul_add_div_erf_add_mul_mul": [_T, _T, _T, _T, _f64, _f64, _f64, _vp],
+    "fluidml_hip_matmul_chain": [_T, _T, _T, _T, _vp, _vp],
+    "fluidml_hip_gemm_chain": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _vp, _vp],
+    "fluidml_hip_conv_chain": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _vp],
+    "fluidml_hip_elementwise_chain": [_T, _T, _vp, _vp],
     "fluidml_hip_div_add_softmax": [_T, _f64, _T, _T, _i64, _vp],
     "fluidml_hip_add_layer_normalization": [_T, _T, _T, _T, _T, _i64, _f64, _vp],
     "fluidml_hip_conv_without_padding": [_T, _T, _T, _T, _i64p, _i64p, _i64, _u32, _vp],
@@ -155,6 +158,25 @@ for _name, _argtypes in SIGNATURES.items():
     _fn.restype = ctypes.c_int
 lib.fluidml_hip_error_string.argtypes = [ctypes.c_int]
 lib.fluidml_hip_error_string.restype = ctypes.c_char_p
+
+
+(EW_ADD_C, EW_RSUB_C, EW_MUL_C, EW_DIV_C, EW_POW_C, EW_ERF, EW_RELU, EW_TANH, EW_SQRT, EW_NEG, EW_ADD_X, EW_MUL_X,
+ EW_SUB_X, EW_RSUB_X, EW_DIV_X, EW_RDIV_X) = range(16)
+
+
+class FlEwProgram(ctypes.Structure):
+    """fl_ew_program of include/fluidml_hip.h"""
+    _fields_ = [("n", ctypes.c_int32), ("op", ctypes.c_int32 * 8), ("c", ctypes.c_float * 8)]
+
+
+def make_chain(steps) -> FlEwProgram:
+    """steps: sequence of (op, constant) pairs"""
+    g = FlEwProgram()
+    g.n = len(steps)
+    for i, (op, c) in enumerate(steps):
+        g.op[i] = op
+        g.c[i] = c
+    return g
 
 
 def error_string(code: int) -> str:

@@ -35,6 +35,7 @@ struct ConvArgs {
   int32_t bias_stride;   // element stride of bias; 0 with bias_fixed
   int32_t bias_fixed;    // FL_REF_CONV_BIAS_INDEX1: every element gets bias[1]
   uint32_t n_out;
+  fl_ew_program chain;   // elementwise chain applied after the bias (n == 0: none)
 };
 
 template <int NS>
@@ -108,6 +109,7 @@ __global__ __launch_bounds__(kBlock) void ConvDirect(ConvArgs p, float *__restri
     }
   }
   if (bias != nullptr) acc += p.bias_fixed ? bias[p.bias_stride] : bias[f * p.bias_stride];
+  if (p.chain.n != 0) acc = RunChain(p.chain, acc);
   out[ooff] = acc;
 }
 
@@ -115,13 +117,15 @@ __global__ __launch_bounds__(kBlock) void ConvDirect(ConvArgs p, float *__restri
 
 // matmul.hip
 int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
-                     const int64_t *pads, const int64_t *strides, const int64_t *dilations, void *stream);
+                     const int64_t *pads, const int64_t *strides, const int64_t *dilations,
+                     const fl_ew_program *chain, void *stream);
 
 namespace {
 
 int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
          const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, uint32_t flags,
-         void *stream) {
+         void *stream, const fl_ew_program *chain = nullptr) {
+  FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(in));
   FL_CHECK(CheckView(weights));
   FL_CHECK(CheckView(out));
@@ -146,6 +150,7 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
   p.n_spatial = ns;
   p.channels = depthwise ? 1 : static_cast<int32_t>(C);
   p.depthwise = depthwise ? 1 : 0;
+  if (chain != nullptr) p.chain = *chain;
   const bool unit = (flags & FL_REF_CONV_UNIT_STRIDE) != 0;
   for (int i = 0; i < rank; ++i) {
     p.out_shape[i] = static_cast<int32_t>(out->shape[i]);
@@ -178,7 +183,7 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
   }
   // dense contractions go to the matrix cores; depthwise, 3-d and literal-reference modes stay here
   if (!depthwise && flags == 0 && ns <= 2) {
-    const int rc = ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, stream);
+    const int rc = ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, chain, stream);
     if (rc != FL_ERR_UNSUPPORTED) return rc;
   }
   LoopNest nest;
@@ -234,6 +239,12 @@ int fluidml_hip_conv_with_padding(const fl_tensor *in, const fl_tensor *weights,
   (void)scratch_bytes;
   if (pads == nullptr) return FL_ERR_NULL;
   return fl::Conv(in, weights, bias, out, pads, strides, dilations, group, flags, stream);
+}
+
+int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
+                           const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group,
+                           const fl_ew_program *chain, void *stream) {
+  return fl::Conv(in, weights, bias, out, pads, strides, dilations, group, 0, stream, chain);
 }
 
 }  // extern "C"

@@ -190,6 +190,10 @@ struct Sqrt {
 struct Neg {
   __device__ float operator()(float x, Empty, Empty) const { return -x; }
 };
+struct Chain {
+  fl_ew_program g;
+  __device__ float operator()(float x, Empty, Empty) const { return RunChain(g, x); }
+};
 struct Not {
   __device__ uint8_t operator()(uint8_t x, Empty, Empty) const { return x ^ 1u; }
 };
@@ -680,6 +684,12 @@ int fluidml_hip_concat2(const fl_tensor *lhs, const fl_tensor *rhs, const fl_ten
   FL_CHECK(StridedCopy(lhs, 0, lhs->strides, out, 0, out->rank, lhs->shape, out->strides, stream));
   return StridedCopy(rhs, 0, rhs->strides, out, lhs->shape[axis] * out->strides[axis], out->rank, rhs->shape,
                      out->strides, stream);
+}
+
+int fluidml_hip_elementwise_chain(const fl_tensor *in, const fl_tensor *out, const fl_ew_program *chain, void *stream) {
+  if (chain == nullptr) return FL_ERR_NULL;
+  FL_CHECK(CheckChain(chain));
+  return UnaryF32(in, out, Chain{*chain}, stream);
 }
 
 int fluidml_hip_pad(const fl_tensor *in, const fl_tensor *out, const int64_t *pads_before, int32_t n, uint32_t flags,

@@ -59,6 +59,44 @@ KernelTimer &ThreadKernelTimer();  // runtime.hip
     }                                                                                                            \
   } while (0)
 
+// Interpreter of fl_ew_program, shared by the elementwise-chain kernel and the contraction epilogues.
+// Each case is the expression the standalone kernel of that operation evaluates.
+__device__ __forceinline__ float RunChain(const fl_ew_program &g, float x) {
+  float v = x;
+  for (int i = 0; i < g.n; ++i) {
+    const float c = g.c[i];
+    switch (g.op[i]) {
+      case FL_EW_ADD_C: v = v + c; break;
+      case FL_EW_RSUB_C: v = c - v; break;
+      case FL_EW_MUL_C: v = v * c; break;
+      case FL_EW_DIV_C: v = v / c; break;
+      case FL_EW_POW_C: v = powf(v, c); break;
+      case FL_EW_ERF: v = erff(v); break;
+      case FL_EW_RELU: v = v != v ? v : fmaxf(v, 0.0f); break;
+      case FL_EW_TANH: v = tanhf(v); break;
+      case FL_EW_SQRT: v = sqrtf(v); break;
+      case FL_EW_NEG: v = -v; break;
+      case FL_EW_ADD_X: v = v + x; break;
+      case FL_EW_MUL_X: v = v * x; break;
+      case FL_EW_SUB_X: v = v - x; break;
+      case FL_EW_RSUB_X: v = x - v; break;
+      case FL_EW_DIV_X: v = v / x; break;
+      case FL_EW_RDIV_X: v = x / v; break;
+      default: break;
+    }
+  }
+  return v;
+}
+
+inline int CheckChain(const fl_ew_program *g) {
+  if (g == nullptr) return FL_OK;
+  if (g->n < 0 || g->n > FL_EW_MAX_STEPS) return FL_ERR_ATTR;
+  for (int i = 0; i < g->n; ++i) {
+    if (g->op[i] < FL_EW_ADD_C || g->op[i] > FL_EW_RDIV_X) return FL_ERR_ATTR;
+  }
+  return FL_OK;
+}
+
 inline int LaunchStatus() {
   hipError_t err = hipGetLastError();
   return err == hipSuccess ? FL_OK : static_cast<int>(err);

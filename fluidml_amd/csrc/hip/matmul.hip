@@ -53,9 +53,8 @@ struct MatmulArgs {
   float ca, cb;
   const float *bias;
   int32_t sDm, sDn;
-  // optional activation after the bias: v * (erf(v / g_div) + g_add) * g_mul  (the erf-GELU chain)
-  int32_t act;
-  float g_div, g_add, g_mul;
+  // optional elementwise chain applied after the bias (chain.n == 0: none)
+  fl_ew_program chain;
   ConvGeom conv;  // read by the CONV instantiations only
 };
 
@@ -364,9 +363,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
           if (p.bias != nullptr) {
             v = p.ca * v + p.cb * p.bias[m * p.sDm + n * p.sDn];
           }
-          if (p.act != 0) {
-            v = (v * (erff(v / p.g_div) + p.g_add)) * p.g_mul;
-          }
+          if (p.chain.n != 0) v = RunChain(p.chain, v);
           Cb[static_cast<int64_t>(m) * p.sCm + col] = v;
         }
       }
@@ -403,13 +400,9 @@ void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
   }
 }
 
-struct Activation {
-  int32_t kind = 0;  // 0 none, 1 erf-GELU chain
-  float div = 1.0f, add = 0.0f, mul = 1.0f;
-};
-
 int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, bool trans_a, bool trans_b, float ca,
-             float cb, const fl_tensor *bias, void *stream, Activation act = Activation()) {
+             float cb, const fl_tensor *bias, void *stream, const fl_ew_program *chain = nullptr) {
+  FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(lhs));
   FL_CHECK(CheckView(rhs));
   FL_CHECK(CheckView(out));
@@ -465,10 +458,7 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   p.batch = MakeNestArgs<3>(nest);
   p.ca = ca;
   p.cb = cb;
-  p.act = act.kind;
-  p.g_div = act.div;
-  p.g_add = act.add;
-  p.g_mul = act.mul;
+  if (chain != nullptr) p.chain = *chain;
   if (bias != nullptr) {
     FL_CHECK(CheckView(bias));
     if (bias->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
@@ -524,7 +514,8 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
 // Returns FL_ERR_UNSUPPORTED (nothing launched) when the operands do not fit this path: the caller then
 // uses the direct kernel.  `pads` may be null; `strides`/`dilations` have one entry per spatial dim.
 int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
-                     const int64_t *pads, const int64_t *strides, const int64_t *dilations, void *stream) {
+                     const int64_t *pads, const int64_t *strides, const int64_t *dilations,
+                     const fl_ew_program *chain, void *stream) {
   const int ns = out->rank - 2;
   if (ns != 1 && ns != 2) return FL_ERR_UNSUPPORTED;
   const int hd = ns == 2 ? 2 : -1, wd = ns == 2 ? 3 : 2;  // dims of H (absent for 1-d) and W
@@ -551,6 +542,7 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
   p.batch.rank = 0;
   p.ca = 1.0f;
   p.cb = 1.0f;
+  if (chain != nullptr) p.chain = *chain;
   if (bias != nullptr) {
     p.bias = static_cast<const float *>(bias->base);
     p.sDm = static_cast<int32_t>(bias->strides[0]);
@@ -611,16 +603,20 @@ int fluidml_hip_matmul_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
   return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream);
 }
 
-int fluidml_hip_matmul_add_div_erf_add_mul_mul(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias,
-                                               const fl_tensor *out, double div, double add, double mul, void *stream) {
+int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
+                             const fl_ew_program *chain, void *stream) {
+  if (!lhs || !rhs || !out) return FL_ERR_NULL;
+  if (bias != nullptr && bias->rank != 1) return FL_ERR_RANK;
+  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain);
+}
+
+int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
+                           double alpha, double beta, int32_t trans_a, int32_t trans_b, const fl_ew_program *chain,
+                           void *stream) {
   if (!lhs || !rhs || !bias || !out) return FL_ERR_NULL;
-  if (bias->rank != 1) return FL_ERR_RANK;
-  fl::Activation act;
-  act.kind = 1;
-  act.div = static_cast<float>(div);
-  act.add = static_cast<float>(add);
-  act.mul = static_cast<float>(mul);
-  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, act);
+  if (lhs->rank != 2 || rhs->rank != 2 || out->rank != 2) return FL_ERR_RANK;
+  return fl::Contract(lhs, rhs, out, trans_a != 0, trans_b != 0, static_cast<float>(alpha), static_cast<float>(beta),
+                      bias, stream, chain);
 }
 
 int fluidml_hip_matmul_bf16(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {

@@ -17,8 +17,10 @@ namespace worker {
 const char *LaunchKindName(Launch::Kind kind) {
   switch (kind) {
     case Launch::Kind::Step: return "Step";
-    case Launch::Kind::MatMulAdd: return "MatMulAdd";
-    case Launch::Kind::MatMulAddGelu: return "MatMulAddDivErfAddMulMul";
+    case Launch::Kind::MatMulChain: return "MatMulChain";
+    case Launch::Kind::GemmChain: return "GemmChain";
+    case Launch::Kind::ConvChain: return "ConvChain";
+    case Launch::Kind::ElementwiseChain: return "ElementwiseChain";
     case Launch::Kind::DivAddSoftmax: return "DivAddSoftmax";
     case Launch::Kind::AddLayerNorm: return "AddLayerNormalization";
     case Launch::Kind::ReshapeTranspose: return "ReshapeTranspose";
@@ -57,17 +59,31 @@ class Scheduler {
   std::vector<Launch> Run(bool fuse) {
     std::vector<Launch> fused;
     if (fuse) {
+      // the row-reduction patterns first: their leading Div/Add would otherwise be absorbed one at a time
+      // by the elementwise chains of the second sweep, which saves fewer launches
+      for (size_t i = 0; i < steps_.size(); ++i) {
+        if (taken_[i]) continue;
+        std::optional<Launch> l;
+        if (Kind(i) == OpKind::DivConstantRhs) l = MatchSoftmax(i);
+        else if (Kind(i) == OpKind::AddCommon) l = MatchLayerNorm(i);
+        if (l) {
+          for (size_t m : l->members) taken_[m] = true;
+          fused.push_back(std::move(*l));
+        }
+      }
       for (size_t i = 0; i < steps_.size(); ++i) {
         if (taken_[i]) continue;
         std::optional<Launch> l;
         switch (Kind(i)) {
-          case OpKind::MatMul: l = MatchMatMul(i); break;
-          case OpKind::DivConstantRhs: l = MatchSoftmax(i); break;
-          case OpKind::AddCommon: l = MatchLayerNorm(i); break;
+          case OpKind::MatMul:
+          case OpKind::GemmConstantWeightsBias:
+          case OpKind::ConvWithPadding:
+          case OpKind::ConvWithoutPadding: l = MatchContraction(i); break;
           case OpKind::Reshape: l = MatchCopyPair(i, OpKind::Transpose); break;
           case OpKind::Transpose: l = MatchCopyPair(i, OpKind::Reshape); break;
           default: break;
         }
+        if (!l && UnaryOp(i) >= 0) l = MatchElementwise(i);
         if (l) {
           for (size_t m : l->members) taken_[m] = true;
           fused.push_back(std::move(*l));
@@ -157,75 +173,166 @@ class Scheduler {
     return true;
   }
 
-  std::optional<Launch> MatchMatMul(size_t i) {
-    const Step &mm = steps_[i];
-    if (!IsFloat(mm.out)) return std::nullopt;
-    const auto j = SoleReader(i);
-    if (!j || Kind(*j) != OpKind::AddCommon) return std::nullopt;
-    const auto bias = Other(*j, mm.out);
-    const Step &add = steps_[*j];
-    if (!bias || bias->space != Operand::Space::Constant || !IsFloat(*bias)) return std::nullopt;
-    const auto &shape = mm.out.meta.GetShape();
-    if (bias->meta.GetShape().size() != 1 || bias->meta.GetShape()[0] != shape.back()) return std::nullopt;
-    if (add.out.meta.GetShape() != shape) return std::nullopt;
+  // fl_ew_op of a unary step with at most one scalar constant, -1 if the step is not one
+  int UnaryOp(size_t i) const {
+    if (!IsFloat(steps_[i].out) || !IsFloat(steps_[i].in0)) return -1;
+    switch (Kind(i)) {
+      case OpKind::AddConstant: return FL_EW_ADD_C;
+      case OpKind::SubConstantLhs: return FL_EW_RSUB_C;
+      case OpKind::MulConstant: return FL_EW_MUL_C;
+      case OpKind::DivConstantRhs: return FL_EW_DIV_C;
+      case OpKind::Pow: return FL_EW_POW_C;
+      case OpKind::Erf: return FL_EW_ERF;
+      case OpKind::Relu: return FL_EW_RELU;
+      case OpKind::Tanh: return FL_EW_TANH;
+      case OpKind::Sqrt: return FL_EW_SQRT;
+      case OpKind::Neg: return FL_EW_NEG;
+      default: return -1;
+    }
+  }
 
+  // fl_ew_op of a binary step that combines the running value `value` with the chain input `root`, -1 otherwise
+  int BinaryWithRoot(size_t j, const Operand &value, const Operand &root) const {
+    const Step &s = steps_[j];
+    if (!s.node->IsDoubleInputs() || !IsFloat(s.out)) return -1;
+    const bool value_left = SameTensor(s.in0, value) && SameTensor(s.in1, root);
+    const bool value_right = SameTensor(s.in1, value) && SameTensor(s.in0, root);
+    if (value_left == value_right) return -1;
+    switch (Kind(j)) {
+      case OpKind::AddCommon: return FL_EW_ADD_X;
+      case OpKind::MulCommon: return FL_EW_MUL_X;
+      case OpKind::SubCommon: return value_left ? FL_EW_SUB_X : FL_EW_RSUB_X;
+      case OpKind::DivCommon: return value_left ? FL_EW_DIV_X : FL_EW_RDIV_X;
+      default: return -1;
+    }
+  }
+
+  struct Chain {
+    std::vector<size_t> members;
+    fl_ew_program program{};
+  };
+
+  // The longest chain of free elementwise steps that starts at `first` (a unary step reading `root`) and
+  // whose intermediate values each have one reader.  Binary steps may combine the value with `root` again.
+  Chain Follow(const Operand &root, size_t first) const {
+    Chain c;
+    size_t cur = first;
+    c.members.push_back(first);
+    c.program.op[0] = UnaryOp(first);
+    c.program.c[0] = static_cast<float>(Attrs(first).value);
+    c.program.n = 1;
+    while (c.program.n < FL_EW_MAX_STEPS) {
+      const auto j = SoleReader(cur);
+      if (!j || steps_[*j].out.meta.GetShape() != root.meta.GetShape()) break;
+      int op = -1;
+      float value = 0.0f;
+      if (steps_[*j].node->IsSingleInput()) {
+        op = UnaryOp(*j);
+        value = static_cast<float>(Attrs(*j).value);
+      } else {
+        op = BinaryWithRoot(*j, steps_[cur].out, root);
+      }
+      if (op < 0) break;
+      c.program.op[c.program.n] = op;
+      c.program.c[c.program.n] = value;
+      ++c.program.n;
+      c.members.push_back(*j);
+      cur = *j;
+    }
+    return c;
+  }
+
+  // The chain that consumes `root` completely (every reader of `root` is a member), so `root` need not be written.
+  std::optional<Chain> ConsumingChain(size_t producer) const {
+    const Operand &root = steps_[producer].out;
+    if (!Elidable(root) || !IsFloat(root)) return std::nullopt;
+    auto it = readers_.find(root.name);
+    if (it == readers_.end()) return std::nullopt;
+    std::optional<size_t> first;
+    for (size_t r : it->second) {
+      if (r <= producer || taken_[r]) return std::nullopt;
+      if (steps_[r].node->IsSingleInput() && UnaryOp(r) >= 0 && SameTensor(steps_[r].in0, root) &&
+          steps_[r].out.meta.GetShape() == root.meta.GetShape()) {
+        if (first) return std::nullopt;  // two unary readers: two chains, keep the tensor
+        first = r;
+      }
+    }
+    if (!first) return std::nullopt;
+    Chain c = Follow(root, *first);
+    for (size_t r : it->second) {
+      if (std::find(c.members.begin(), c.members.end(), r) == c.members.end()) return std::nullopt;
+    }
+    return c;
+  }
+
+  std::optional<Launch> MatchContraction(size_t i) {
+    const Step &head = steps_[i];
+    if (!IsFloat(head.out)) return std::nullopt;
     Launch l;
-    l.a = mm.in0;
-    l.b = mm.in1;
-    l.c = *bias;
-    // try to extend through the erf-GELU chain
-    if (auto g = MatchGelu(*j)) {
-      l.kind = Launch::Kind::MatMulAddGelu;
-      l.members = {i, *j};
-      l.members.insert(l.members.end(), g->members.begin(), g->members.end());
+    l.a = head.in0;
+    l.b = head.in1;
+    l.owner = i;
+    l.members = {i};
+    size_t value_step = i;  // the step whose output the elementwise chain starts from
+    if (Kind(i) == OpKind::MatMul) {
+      l.kind = Launch::Kind::MatMulChain;
+      // MatMul -> AddCommon(rank-1 constant bias over the last dim)
+      if (const auto j = SoleReader(i); j && Kind(*j) == OpKind::AddCommon) {
+        const auto bias = Other(*j, head.out);
+        const auto &shape = head.out.meta.GetShape();
+        if (bias && bias->space == Operand::Space::Constant && IsFloat(*bias) && bias->meta.GetShape().size() == 1 &&
+            bias->meta.GetShape()[0] == shape.back() && steps_[*j].out.meta.GetShape() == shape) {
+          l.c = *bias;
+          l.has_c = true;
+          l.members.push_back(*j);
+          value_step = *j;
+        }
+      }
+    } else if (Kind(i) == OpKind::GemmConstantWeightsBias) {
+      l.kind = Launch::Kind::GemmChain;
+    } else {
+      l.kind = Launch::Kind::ConvChain;
+    }
+    const size_t without_chain = l.members.size();
+    if (const auto chain = ConsumingChain(value_step)) {
+      l.members.insert(l.members.end(), chain->members.begin(), chain->members.end());
+      l.chain = chain->program;
+    }
+    // longest variant whose late reads are safe: with the chain, then without it
+    for (int attempt = 0; attempt < 2; ++attempt) {
+      if (l.members.size() < 2) return std::nullopt;  // nothing fused
       l.out = steps_[l.members.back()].out;
-      l.s0 = g->s0;
-      l.s1 = g->s1;
-      l.s2 = g->s2;
       if (Safe(l.members, {{i, l.a}, {i, l.b}}) && OutputDisjoint(l.out, {&l.a, &l.b})) {
-        l.bytes = Bytes({&l.a, &l.b, &l.c, &l.out});
+        l.bytes = l.has_c ? Bytes({&l.a, &l.b, &l.c, &l.out}) : Bytes({&l.a, &l.b, &l.out});
+        l.bytes += static_cast<double>(steps_[i].kernel->GetConstantBytes());
         l.flops = Flops(l.members);
         return l;
       }
+      l.members.resize(without_chain);
+      l.chain = fl_ew_program{};
     }
-    l.kind = Launch::Kind::MatMulAdd;
-    l.members = {i, *j};
-    l.out = add.out;
-    if (!Safe(l.members, {{i, l.a}, {i, l.b}}) || !OutputDisjoint(l.out, {&l.a, &l.b})) return std::nullopt;
-    l.bytes = Bytes({&l.a, &l.b, &l.c, &l.out});
-    l.flops = Flops(l.members);
-    return l;
+    return std::nullopt;
   }
 
-  // t = steps[j].out; Div(t, c) -> Erf -> Add(c) -> Mul(t, .) -> Mul(c): members after j, scalars in s0..s2
-  std::optional<Launch> MatchGelu(size_t j) const {
-    const Operand &t = steps_[j].out;
-    if (!Elidable(t)) return std::nullopt;
-    auto it = readers_.find(t.name);
-    if (it == readers_.end() || it->second.size() != 2) return std::nullopt;
-    size_t d = it->second[0], m = it->second[1];
-    if (Kind(d) != OpKind::DivConstantRhs) std::swap(d, m);
-    if (Kind(d) != OpKind::DivConstantRhs || Kind(m) != OpKind::MulCommon) return std::nullopt;
-    if (d <= j || taken_[d] || taken_[m]) return std::nullopt;
-    const auto e = SoleReader(d);
-    if (!e || Kind(*e) != OpKind::Erf) return std::nullopt;
-    const auto a = SoleReader(*e);
-    if (!a || Kind(*a) != OpKind::AddConstant) return std::nullopt;
-    const auto m2 = SoleReader(*a);
-    if (!m2 || *m2 != m) return std::nullopt;
-    const auto other = Other(m, steps_[*a].out);
-    if (!other || !SameTensor(*other, t)) return std::nullopt;
-    const auto r = SoleReader(m);
-    if (!r || Kind(*r) != OpKind::MulConstant) return std::nullopt;
-    for (size_t s : {d, *e, *a, m, *r}) {
-      if (steps_[s].out.meta.GetShape() != t.meta.GetShape() || !IsFloat(steps_[s].out)) return std::nullopt;
-    }
+  // Two or more elementwise steps on a tensor that stays live (or is a graph input).
+  std::optional<Launch> MatchElementwise(size_t i) {
+    const Step &head = steps_[i];
+    if (head.in0.meta.GetShape() != head.out.meta.GetShape()) return std::nullopt;
+    Chain c = Follow(head.in0, i);
+    if (c.members.size() < 2) return std::nullopt;
     Launch l;
-    l.members = {d, *e, *a, m, *r};
-    if (!std::is_sorted(l.members.begin(), l.members.end())) return std::nullopt;
-    l.s0 = Attrs(d).value;
-    l.s1 = Attrs(*a).value;
-    l.s2 = Attrs(*r).value;
+    l.kind = Launch::Kind::ElementwiseChain;
+    l.members = c.members;
+    l.chain = c.program;
+    l.a = head.in0;
+    l.out = steps_[l.members.back()].out;
+    if (!Safe(l.members, {{i, l.a}})) return std::nullopt;
+    // in place is fine element for element (same bytes, same layout); any other overlap is not
+    if (Alias(l.out, l.a) && !(l.out.space == Operand::Space::Arena && l.a.space == Operand::Space::Arena &&
+                               l.out.offset == l.a.offset && l.out.layout == l.a.layout)) {
+      return std::nullopt;
+    }
+    l.bytes = Bytes({&l.a, &l.out});
     return l;
   }
 

@@ -216,16 +216,37 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
   const kernel::TensorView a = ViewOf(Resolve(l.a), l.a), out = ViewOf(Resolve(l.out), l.out);
   int rc = FL_ERR_UNSUPPORTED;
   switch (l.kind) {
-    case Launch::Kind::MatMulAdd: {
-      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b), c = ViewOf(Resolve(l.c), l.c);
-      rc = fluidml_hip_matmul_add(&a.t, &b.t, &c.t, &out.t, ctx.stream);
+    case Launch::Kind::MatMulChain: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
+      kernel::TensorView c;
+      if (l.has_c) c = ViewOf(Resolve(l.c), l.c);
+      rc = fluidml_hip_matmul_chain(&a.t, &b.t, l.has_c ? &c.t : nullptr, &out.t, &l.chain, ctx.stream);
       break;
     }
-    case Launch::Kind::MatMulAddGelu: {
-      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b), c = ViewOf(Resolve(l.c), l.c);
-      rc = fluidml_hip_matmul_add_div_erf_add_mul_mul(&a.t, &b.t, &c.t, &out.t, l.s0, l.s1, l.s2, ctx.stream);
+    case Launch::Kind::GemmChain: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
+      const flow::Attrs &at = steps_[l.owner].node->GetAttrs();
+      const kernel::DeviceConstant *bias = steps_[l.owner].kernel->GetConstant(0);
+      if (bias == nullptr) throw std::logic_error("fused Gemm: the node holds no bias");
+      const kernel::TensorView c = bias->View();
+      rc = fluidml_hip_gemm_chain(&a.t, &b.t, &c.t, &out.t, at.alpha, at.beta, at.trans_a ? 1 : 0, at.trans_b ? 1 : 0,
+                                  &l.chain, ctx.stream);
       break;
     }
+    case Launch::Kind::ConvChain: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
+      const flow::Attrs &at = steps_[l.owner].node->GetAttrs();
+      const kernel::DeviceConstant *bias = steps_[l.owner].kernel->GetConstant(0);
+      kernel::TensorView c;
+      if (bias != nullptr) c = bias->View();
+      const bool padded = steps_[l.owner].node->GetKind() == flow::OpKind::ConvWithPadding;
+      rc = fluidml_hip_conv_chain(&a.t, &b.t, bias ? &c.t : nullptr, &out.t, padded ? at.pads.data() : nullptr,
+                                  at.strides.data(), at.dilations.data(), at.group, &l.chain, ctx.stream);
+      break;
+    }
+    case Launch::Kind::ElementwiseChain:
+      rc = fluidml_hip_elementwise_chain(&a.t, &out.t, &l.chain, ctx.stream);
+      break;
     case Launch::Kind::DivAddSoftmax: {
       const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
       rc = fluidml_hip_div_add_softmax(&a.t, l.s0, &b.t, &out.t, l.axis, ctx.stream);

@@ -53,8 +53,10 @@ struct Step {
 struct Launch {
   enum class Kind {
     Step,              // members = {i}
-    MatMulAdd,         // MatMul -> AddCommon(rank-1 constant bias)
-    MatMulAddGelu,     // MatMul -> AddCommon(bias) -> DivConstantRhs -> Erf -> AddConstant -> MulCommon -> MulConstant
+    MatMulChain,       // MatMul [-> AddCommon(rank-1 constant bias)] [-> elementwise chain]
+    GemmChain,         // GemmConstantWeightsBias -> elementwise chain
+    ConvChain,         // Conv{With,Without}Padding -> elementwise chain
+    ElementwiseChain,  // two or more elementwise steps on one tensor
     DivAddSoftmax,     // DivConstantRhs -> AddCommon(mask) -> Softmax
     AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias
     ReshapeTranspose,  // Reshape -> Transpose, one strided copy
@@ -66,7 +68,9 @@ struct Launch {
   double s0 = 0, s1 = 0, s2 = 0;
   int64_t axis = 0;
   std::vector<int64_t> perm;
-  size_t owner = 0;  // member whose kernel owns constants the launch needs (LayerNorm scale/bias)
+  bool has_c = false;     // MatMulChain: a bias operand is present
+  fl_ew_program chain{};  // elementwise steps applied to the value (n == 0: none)
+  size_t owner = 0;  // member whose kernel owns constants / attributes the launch needs (LayerNorm, Gemm, Conv)
   double bytes = 0, flops = 0;
 };
 const char *LaunchKindName(Launch::Kind kind);

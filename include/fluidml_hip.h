@@ -87,6 +87,35 @@ enum fl_ref_flags {
   FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
 };
 
+/* A short chain of elementwise operations on one float32 value, used by the
+ * launch-level fusions below.  Step i replaces v (initially the chain's input
+ * x) by op[i](v, c[i]) or op[i](v, x); every operation is the one the
+ * standalone kernel of that name performs. */
+enum fl_ew_op {
+  FL_EW_ADD_C = 0, /* v + c   (AddConstantKernel) */
+  FL_EW_RSUB_C,    /* c - v   (SubConstantLhsKernel) */
+  FL_EW_MUL_C,     /* v * c   (MulConstantKernel) */
+  FL_EW_DIV_C,     /* v / c   (DivConstantRhsKernel) */
+  FL_EW_POW_C,     /* powf(v, c) (PowKernel) */
+  FL_EW_ERF,       /* ErfKernel */
+  FL_EW_RELU,      /* ReluKernel (NaN propagates) */
+  FL_EW_TANH,      /* TanhKernel */
+  FL_EW_SQRT,      /* SqrtKernel */
+  FL_EW_NEG,       /* NegKernel */
+  FL_EW_ADD_X,     /* v + x   (AddCommonKernel with the chain input) */
+  FL_EW_MUL_X,     /* v * x   (MulCommonKernel) */
+  FL_EW_SUB_X,     /* v - x   (SubCommonKernel, chain value on the left) */
+  FL_EW_RSUB_X,    /* x - v */
+  FL_EW_DIV_X,     /* v / x   (DivCommonKernel, chain value on the left) */
+  FL_EW_RDIV_X     /* x / v */
+};
+#define FL_EW_MAX_STEPS 8
+typedef struct fl_ew_program {
+  int32_t n; /* 0..FL_EW_MAX_STEPS */
+  int32_t op[FL_EW_MAX_STEPS];
+  float c[FL_EW_MAX_STEPS];
+} fl_ew_program;
+
 typedef struct fl_tensor {
   void *base;
   int32_t dtype; /* enum fl_dtype */
@@ -292,10 +321,18 @@ int fluidml_hip_conv_with_padding(const fl_tensor *in, const fl_tensor *weights,
 /* MatMulKernel -> AddCommonKernel with a rank-1 bias over the last dim
  * (reference matmul.cpp:28-59 + add.cpp:75-137). */
 int fluidml_hip_matmul_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, void *stream);
-/* MatMulKernel -> AddCommonKernel(bias) -> Div -> Erf -> Add -> Mul -> Mul:
- * t = lhs.rhs + bias; out = t * (erf(t / div) + add) * mul
- * (reference matmul.cpp:28-59 + add_div_erf_add_mul_mul.cpp:29-132). */
-int fluidml_hip_matmul_add_div_erf_add_mul_mul(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double div, double add, double mul, void *stream);
+/* MatMulKernel [-> AddCommonKernel(rank-1 bias)] -> elementwise chain on the
+ * result, e.g. the erf-GELU chain Div, Erf, Add, Mul(x), Mul of
+ * add_div_erf_add_mul_mul.cpp:29-132.  `bias` and `chain` may be NULL. */
+int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, const fl_ew_program *chain, void *stream);
+/* GemmConstantWeightsBiasKernel -> elementwise chain (reference gemm.cpp:39-182). */
+int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double alpha, double beta, int32_t trans_a, int32_t trans_b, const fl_ew_program *chain, void *stream);
+/* Conv{With,Without}PaddingKernel -> elementwise chain (reference conv.cpp:27-280);
+ * `pads` may be NULL.  ONNX semantics only (no literal-reference flags). */
+int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, const fl_ew_program *chain, void *stream);
+/* A chain of elementwise kernels on one float32 tensor as one launch:
+ * out = chain(in), same shape, any two layouts. */
+int fluidml_hip_elementwise_chain(const fl_tensor *in, const fl_tensor *out, const fl_ew_program *chain, void *stream);
 /* DivConstantRhsKernel -> AddCommonKernel(mask, broadcast) -> SoftmaxKernel:
  * out = softmax(in / div + mask, axis)
  * (reference div.cpp:24-56 + add.cpp:75-137 + softmax.cpp:22-139). */

@@ -587,9 +587,101 @@ def test_fused_matmul_add_and_gelu(device):
             ok.binary_f32(ok.BOP_MUL, t1, u2, u3)
             ok.unary_f32(ok.OP_MUL_C, u3, u4, 0.5)
             do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
-            cabi.call("matmul_add_div_erf_add_mul_mul", da.ref(), db.ref(), dbias.ref(), do.ref(),
-                      ctypes.c_double(1.4142135381698608), ctypes.c_double(1.0), ctypes.c_double(0.5), None)
-            assert_close(do.logical(), u4.logical(), what="matmul_add_div_erf_add_mul_mul")
+            gelu = cabi.make_chain([(cabi.EW_DIV_C, 1.4142135381698608), (cabi.EW_ERF, 0), (cabi.EW_ADD_C, 1.0),
+                                    (cabi.EW_MUL_X, 0), (cabi.EW_MUL_C, 0.5)])
+            cabi.call("matmul_chain", da.ref(), db.ref(), dbias.ref(), do.ref(), ctypes.byref(gelu), None)
+            assert_close(do.logical(), u4.logical(), what="matmul_chain bias + erf-GELU")
+            # no bias, chain only: relu(a.b) * 0.5
+            ok.unary_f32(ok.OP_RELU, t0, u0)
+            ok.unary_f32(ok.OP_MUL_C, u0, u1, 0.5)
+            do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
+            chain = cabi.make_chain([(cabi.EW_RELU, 0), (cabi.EW_MUL_C, 0.5)])
+            cabi.call("matmul_chain", da.ref(), db.ref(), None, do.ref(), ctypes.byref(chain), None)
+            assert_close(do.logical(), u1.logical(), what="matmul_chain relu, scale")
+
+
+def test_elementwise_chain(device):
+    """Every chain operation against the oracle's standalone kernels, applied one after the other."""
+    cabi = _cabi()
+    rng = np.random.default_rng(94)
+    shape = (3, 17, 40)
+    x = rand(rng, shape, 0.2, 3.0)  # positive: sqrt and pow stay real
+    unary = {cabi.EW_ADD_C: ok.OP_ADD_C, cabi.EW_RSUB_C: ok.OP_RSUB_C, cabi.EW_MUL_C: ok.OP_MUL_C, cabi.EW_DIV_C: ok.OP_DIV_C,
+             cabi.EW_POW_C: ok.OP_POW_C, cabi.EW_ERF: ok.OP_ERF, cabi.EW_RELU: ok.OP_RELU, cabi.EW_TANH: ok.OP_TANH,
+             cabi.EW_SQRT: ok.OP_SQRT, cabi.EW_NEG: ok.OP_NEG}
+    programs = [
+        [(cabi.EW_DIV_C, 2.0), (cabi.EW_TANH, 0), (cabi.EW_ADD_C, 1.0), (cabi.EW_MUL_C, 0.5), (cabi.EW_MUL_X, 0)],  # swish
+        [(cabi.EW_SQRT, 0), (cabi.EW_RSUB_C, 1.5), (cabi.EW_RELU, 0), (cabi.EW_ADD_X, 0), (cabi.EW_POW_C, 1.7), (cabi.EW_NEG, 0),
+         (cabi.EW_ERF, 0), (cabi.EW_SUB_X, 0)],
+        [(cabi.EW_MUL_C, 0.3), (cabi.EW_RSUB_X, 0), (cabi.EW_DIV_X, 0), (cabi.EW_ADD_C, 2.0), (cabi.EW_RDIV_X, 0)],
+    ]
+    for steps in programs:
+        for lin, lout in [(None, None), ([2, 1, 0], [1, 0, 2])]:
+            announce("elementwise chain", [s[0] for s in steps], lin, lout)
+            hx = ok.View(x, lin)
+            cur = hx
+            for op, c in steps:
+                nxt = ok.View.empty(shape)
+                if op in unary:
+                    ok.unary_f32(unary[op], cur, nxt, c)
+                elif op in (cabi.EW_ADD_X, cabi.EW_MUL_X):
+                    ok.binary_f32(ok.BOP_ADD if op == cabi.EW_ADD_X else ok.BOP_MUL, cur, hx, nxt)
+                elif op in (cabi.EW_SUB_X, cabi.EW_DIV_X):
+                    ok.binary_f32(ok.BOP_SUB if op == cabi.EW_SUB_X else ok.BOP_DIV, cur, hx, nxt)
+                else:
+                    ok.binary_f32(ok.BOP_SUB if op == cabi.EW_RSUB_X else ok.BOP_DIV, hx, cur, nxt)
+                cur = nxt
+            dx = DeviceView(hx, device)
+            do = DeviceView(ok.View.empty(shape, np.float32, lout), device)
+            chain = cabi.make_chain(steps)
+            cabi.call("elementwise_chain", dx.ref(), do.ref(), ctypes.byref(chain), None)
+            assert_close(do.logical(), cur.logical(), what="elementwise_chain")
+    bad = cabi.make_chain([(99, 0)])
+    assert cabi.lib.fluidml_hip_elementwise_chain(dx.ref(), do.ref(), ctypes.byref(bad), None) == -5  # FL_ERR_ATTR
+
+
+def test_conv_and_gemm_chain(device):
+    cabi = _cabi()
+    rng = np.random.default_rng(95)
+    swish = [(cabi.EW_DIV_C, 2.0), (cabi.EW_TANH, 0), (cabi.EW_ADD_C, 1.0), (cabi.EW_MUL_C, 0.5), (cabi.EW_MUL_X, 0)]
+
+    def swish_ref(t):
+        u = [ok.View.empty(t.shape) for _ in range(5)]
+        ok.unary_f32(ok.OP_DIV_C, t, u[0], 2.0)
+        ok.unary_f32(ok.OP_TANH, u[0], u[1])
+        ok.unary_f32(ok.OP_ADD_C, u[1], u[2], 1.0)
+        ok.unary_f32(ok.OP_MUL_C, u[2], u[3], 0.5)
+        ok.binary_f32(ok.BOP_MUL, u[3], t, u[4])
+        return u[4]
+
+    # dense 3x3 (matrix cores) and depthwise 5x5 stride 2 (direct kernel)
+    for xshape, wshape, pads, strides, group in [((2, 8, 20, 20), (16, 8, 3, 3), [1, 1, 1, 1], [1, 1], 1),
+                                                 ((1, 6, 15, 15), (6, 1, 5, 5), [2, 2, 2, 2], [2, 2], 6)]:
+        x, w, bias = rand(rng, xshape, -1, 1), rand(rng, wshape, -0.3, 0.3), rand(rng, (wshape[0],), -1, 1)
+        od = tuple((xshape[2 + d] + 2 * pads[d] - wshape[2 + d]) // strides[d] + 1 for d in range(2))
+        oshape = (xshape[0], wshape[0]) + od
+        hx, hw, hb, t = ok.View(x), ok.View(w), ok.View(bias), ok.View.empty(oshape)
+        ok.conv(hx, hw, hb, t, pads, strides, [1, 1], group, 0)
+        want = swish_ref(t)
+        announce("conv chain", xshape, wshape, group)
+        dx, dw, db = DeviceView(hx, device), DeviceView(hw, device), DeviceView(hb, device)
+        do = DeviceView(ok.View.empty(oshape, np.float32, [0, 3, 1, 2]), device)
+        chain = cabi.make_chain(swish)
+        cabi.call("conv_chain", dx.ref(), dw.ref(), db.ref(), do.ref(), cabi.i64_array(pads), cabi.i64_array(strides),
+                  cabi.i64_array([1, 1]), ctypes.c_int64(group), ctypes.byref(chain), None)
+        assert_close(do.logical(), want.logical(), what="conv_chain swish")
+    # Gemm -> Relu (transB, alpha = beta = 1)
+    a, b, c = rand(rng, (8, 100), -1, 1), rand(rng, (50, 100), -0.05, 0.05), rand(rng, (50,), -0.2, 0.2)
+    ha, hb, hc, t, want = ok.View(a), ok.View(b), ok.View(c), ok.View.empty((8, 50)), ok.View.empty((8, 50))
+    ok.gemm(ha, hb, hc, t, 1.0, 1.0, 0, 1, 0)
+    ok.unary_f32(ok.OP_RELU, t, want)
+    announce("gemm chain")
+    da, db, dc = DeviceView(ha, device), DeviceView(hb, device), DeviceView(hc, device)
+    do = DeviceView(ok.View.empty((8, 50)), device)
+    relu = cabi.make_chain([(cabi.EW_RELU, 0)])
+    cabi.call("gemm_chain", da.ref(), db.ref(), dc.ref(), do.ref(), ctypes.c_double(1.0), ctypes.c_double(1.0), 0, 1,
+              ctypes.byref(relu), None)
+    assert_close(do.logical(), want.logical(), what="gemm_chain relu")
 
 
 def test_fused_div_add_softmax(device):

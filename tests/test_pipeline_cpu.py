@@ -292,13 +292,26 @@ def _overlap(x, y):
     return x["offset"] < y["offset"] + y["bytes"] and y["offset"] < x["offset"] + x["bytes"]
 
 
+SCHEDULE_NETS = {
+    "bert": (lambda m: m.bert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32, seed=5),
+             {"MatMulChain", "AddLayerNormalization", "DivAddSoftmax", "ElementwiseChain"}),
+    "convbert": (lambda m: m.convbert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32),
+                 {"MatMulChain", "AddLayerNormalization", "DivAddSoftmax"}),
+    "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), {"MatMulChain"}),
+    "efficientnet_b0": (lambda m: m.efficientnet_b0(image=64, classes=10, width_div=4), {"ConvChain"}),
+    "vgg16": (lambda m: m.vgg16(batch=2, image=32, classes=10, width_div=8, fc=512), {"ConvChain", "GemmChain"}),
+}
+
+
 @pytest.mark.parametrize("flavour", ["make_plain_greedy", "make_plain_linear", "make_dp_greedy"])
-def test_fused_schedule_is_safe(mods, tiny, flavour, monkeypatch):
+@pytest.mark.parametrize("which", list(SCHEDULE_NETS))
+def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     """Independent re-check of what the launcher's fusion pass must guarantee: every step is issued once,
     an elided tensor has no reader outside its chain, and moving a chain's reads to its last member's
     position crosses no write to the bytes it reads (arena intervals of the memory plan)."""
-    fluidml, _, _ = mods
-    _, path = tiny
+    fluidml, models, _ = mods
+    make, expected_kinds = SCHEDULE_NETS[which]
+    path = make(models).save(str(tmp_path / "net.onnx"))
     monkeypatch.setenv("FLUIDML_DP_COST", "constant")
     ex = getattr(fluidml.Executor, flavour)("sched")
     ex.compile(path)
@@ -307,7 +320,7 @@ def test_fused_schedule_is_safe(mods, tiny, flavour, monkeypatch):
     assert sorted(m for l in launches for m in l["members"]) == list(range(len(steps)))
     assert [l["members"][-1] for l in launches] == sorted(l["members"][-1] for l in launches)
     kinds = {l["kind"] for l in launches}
-    assert {"MatMulAdd", "MatMulAddDivErfAddMulMul", "AddLayerNormalization", "DivAddSoftmax"} <= kinds
+    assert expected_kinds <= kinds
     readers = {}
     for i, s in enumerate(steps):
         for op in s["inputs"]:
@@ -331,8 +344,9 @@ def test_fused_schedule_is_safe(mods, tiny, flavour, monkeypatch):
                 for s in range(m + 1, members[-1]):
                     if s not in members:
                         assert not _overlap(steps[s]["out"], op), "a read was moved across a write to its bytes"
-                if _overlap(final, op):  # only the in-place softmax may write over what it reads
-                    assert l["kind"] == "DivAddSoftmax" and final["offset"] == op["offset"] and final["layout"] == op["layout"]
+                if _overlap(final, op):  # only row-wise / elementwise kernels may work in place, and only exactly
+                    assert l["kind"] in ("DivAddSoftmax", "ElementwiseChain")
+                    assert final["offset"] == op["offset"] and final["layout"] == op["layout"]
     # switched off: one launch per step
     monkeypatch.setenv("FLUIDML_FUSE", "0")
     ex = getattr(fluidml.Executor, flavour)("sched_off")

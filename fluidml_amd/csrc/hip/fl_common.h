@@ -9,6 +9,8 @@
 #ifndef FLUIDML_AMD_CSRC_HIP_FL_COMMON_H_
 #define FLUIDML_AMD_CSRC_HIP_FL_COMMON_H_
 
+#include <utility>
+
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 
@@ -59,6 +61,17 @@ KernelTimer &ThreadKernelTimer();  // runtime.hip
     }                                                                                                            \
   } while (0)
 
+// Compile-time loop: body(std::integral_constant<int, 0>) ... body(std::integral_constant<int, N - 1>).
+// Unlike `#pragma unroll` it cannot be left rolled, so register arrays indexed by the counter stay in registers.
+template <int N, typename F, int... I>
+__host__ __device__ __forceinline__ void StaticForImpl(F &&body, std::integer_sequence<int, I...>) {
+  (body(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__host__ __device__ __forceinline__ void StaticFor(F &&body) {
+  StaticForImpl<N>(static_cast<F &&>(body), std::make_integer_sequence<int, N>{});
+}
+
 // Interpreter of fl_ew_program, shared by the elementwise-chain kernel and the contraction epilogues.
 // Each case is the expression the standalone kernel of that operation evaluates.
 __device__ __forceinline__ float RunChain(const fl_ew_program &g, float x) {
@@ -86,6 +99,42 @@ __device__ __forceinline__ float RunChain(const fl_ew_program &g, float x) {
     }
   }
   return v;
+}
+
+// The same interpreter over a block of N values held in registers: one (wave-uniform) branch per chain
+// step instead of one per value.  `v` holds the chain inputs on entry and the results on exit.
+template <int N>
+__device__ __forceinline__ void RunChainBlock(const fl_ew_program &g, float (&v)[N]) {
+  float x[N];
+#pragma unroll
+  for (int e = 0; e < N; ++e) x[e] = v[e];
+  for (int i = 0; i < g.n; ++i) {
+    const float c = g.c[i];
+#define FL_EW_CASE(OP, EXPR)               \
+  case OP:                                 \
+    _Pragma("unroll") for (int e = 0; e < N; ++e) v[e] = (EXPR); \
+    break;
+    switch (g.op[i]) {
+      FL_EW_CASE(FL_EW_ADD_C, v[e] + c)
+      FL_EW_CASE(FL_EW_RSUB_C, c - v[e])
+      FL_EW_CASE(FL_EW_MUL_C, v[e] * c)
+      FL_EW_CASE(FL_EW_DIV_C, v[e] / c)
+      FL_EW_CASE(FL_EW_POW_C, powf(v[e], c))
+      FL_EW_CASE(FL_EW_ERF, erff(v[e]))
+      FL_EW_CASE(FL_EW_RELU, v[e] != v[e] ? v[e] : fmaxf(v[e], 0.0f))
+      FL_EW_CASE(FL_EW_TANH, tanhf(v[e]))
+      FL_EW_CASE(FL_EW_SQRT, sqrtf(v[e]))
+      FL_EW_CASE(FL_EW_NEG, -v[e])
+      FL_EW_CASE(FL_EW_ADD_X, v[e] + x[e])
+      FL_EW_CASE(FL_EW_MUL_X, v[e] * x[e])
+      FL_EW_CASE(FL_EW_SUB_X, v[e] - x[e])
+      FL_EW_CASE(FL_EW_RSUB_X, x[e] - v[e])
+      FL_EW_CASE(FL_EW_DIV_X, v[e] / x[e])
+      FL_EW_CASE(FL_EW_RDIV_X, x[e] / v[e])
+      default: break;
+    }
+#undef FL_EW_CASE
+  }
 }
 
 inline int CheckChain(const fl_ew_program *g) {

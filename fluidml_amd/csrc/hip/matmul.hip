@@ -342,10 +342,8 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   }
 
   // ---- epilogue ---------------------------------------------------------------
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
+  StaticFor<TM * TN>([&](auto tile) {
+      constexpr int i = decltype(tile)::value / TN, j = decltype(tile)::value % TN;
       const int n = n0 + (wn * TN + j) * 32 + lrow;
       int64_t col = static_cast<int64_t>(n) * p.sCn;
       if constexpr (CONV) {
@@ -355,19 +353,24 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
         col = static_cast<int64_t>(img) * p.conv.sOn + static_cast<int64_t>(oh) * p.conv.sOh +
               static_cast<int64_t>(ow) * p.conv.sOw;
       }
+      // bias, then the elementwise chain on the 16 values of this 32x32 tile the lane holds, then the stores
+      float vals[16];
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
-        if (m < p.M && n < p.N) {
-          float v = acc[i][j][e];
-          if (p.bias != nullptr) {
-            v = p.ca * v + p.cb * p.bias[m * p.sDm + n * p.sDn];
-          }
-          if (p.chain.n != 0) v = RunChain(p.chain, v);
-          Cb[static_cast<int64_t>(m) * p.sCm + col] = v;
+        float v = acc[i][j][e];
+        if (p.bias != nullptr && m < p.M && n < p.N) {
+          v = p.ca * v + p.cb * p.bias[m * p.sDm + n * p.sDn];
         }
+        vals[e] = v;
       }
-    }
+      if (p.chain.n != 0) RunChainBlock<16>(p.chain, vals);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
+        if (m < p.M && n < p.N) Cb[static_cast<int64_t>(m) * p.sCm + col] = vals[e];
+      }
+  });
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV>

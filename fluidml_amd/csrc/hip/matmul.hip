@@ -22,6 +22,8 @@
 //
 // A second, opt-in path rounds operands to bf16 (v_mfma_f32_32x32x8_bf16 would
 // be its instruction); it is not built yet and reports FL_ERR_UNSUPPORTED.
+#include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 #include "fl_common.h"
@@ -55,6 +57,11 @@ struct MatmulArgs {
   int32_t sDm, sDn;
   // optional elementwise chain applied after the bias (chain.n == 0: none)
   fl_ew_program chain;
+  // split K over gridDim.z workgroups per tile: each takes `chunks_per_split` chunks, writes its partial tile
+  // to `partials`, and the workgroup that arrives last at `counters[tile]` adds them up in split order
+  int32_t chunks_per_split;
+  float *partials;
+  uint32_t *counters;
   ConvGeom conv;  // read by the CONV instantiations only
 };
 
@@ -288,17 +295,20 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
     }
   };
 
+  // this workgroup's share of the chunks (all of them unless K is split over gridDim.z)
+  const int c_begin = gridDim.z > 1 ? static_cast<int>(blockIdx.z) * p.chunks_per_split : 0;
+  const int c_end = gridDim.z > 1 ? min(n_chunks, c_begin + p.chunks_per_split) : n_chunks;
 #pragma unroll
   for (int s = 0; s < DEPTH; ++s) {
-    if (s < n_chunks) load_chunk(s, ra[s], rb[s]);
+    if (c_begin + s < c_end) load_chunk(c_begin + s, ra[s], rb[s]);
   }
-  for (int c0 = 0; c0 < n_chunks; c0 += DEPTH) {
+  for (int c0 = c_begin; c0 < c_end; c0 += DEPTH) {
 #pragma unroll
     for (int s = 0; s < DEPTH; ++s) {
       const int c = c0 + s;
-      if (c < n_chunks) {  // uniform over the workgroup
+      if (c < c_end) {  // uniform over the workgroup
         store_chunk(s & 1, ra[s], rb[s]);
-        if (c + DEPTH < n_chunks) load_chunk(c + DEPTH, ra[s], rb[s]);
+        if (c + DEPTH < c_end) load_chunk(c + DEPTH, ra[s], rb[s]);
         // one barrier per chunk: buffer (s&1) was last read two chunks ago, and every wave
         // passed the previous barrier only after finishing that read
         __syncthreads();
@@ -341,6 +351,42 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
     }
   }
 
+  // ---- combine the K splits of a tile across workgroups ------------------------
+  // Only the single-wave-per-tile configuration splits (host side), so no workgroup barrier is involved:
+  // the wave publishes its partial tile, then one atomic tells it whether it arrived last; the last wave
+  // adds all partials in split order, which makes the sum independent of arrival order.
+  if constexpr (WM * WN == 1 && KS > 1) {
+    if (gridDim.z > 1) {
+      const uint32_t n_splits = gridDim.z;
+      const uint32_t tile_id = blockIdx.y * gridDim.x + blockIdx.x;
+      float *mine = p.partials + (static_cast<size_t>(tile_id) * n_splits + blockIdx.z) * (BM * BN);
+      // The partial tiles travel through device-coherent accesses (agent-scope atomics: they bypass the
+      // per-XCD L2 instead of living in it), so no cache-wide write-back or invalidate is needed: waiting
+      // for this wave's stores to be acknowledged before it counts its arrival is enough, and the last
+      // wave's loads are issued only after it has seen every other arrival.
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        __hip_atomic_store(mine + e * 64 + lane, acc[0][0][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // s_waitcnt: stores acknowledged
+      uint32_t arrived = 0;
+      if (lane == 0) arrived = __hip_atomic_fetch_add(&p.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      arrived = __shfl(arrived, 0);
+      if (arrived != n_splits - 1) return;
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // keeps the loads below behind the counter read
+      if (lane == 0) __hip_atomic_store(&p.counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const float *all = p.partials + static_cast<size_t>(tile_id) * n_splits * (BM * BN);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[0][0][e] = 0.0f;
+      for (uint32_t z = 0; z < n_splits; ++z) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          acc[0][0][e] += __hip_atomic_load(all + z * (BM * BN) + e * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+    }
+  }
+
   // ---- epilogue ---------------------------------------------------------------
   StaticFor<TM * TN>([&](auto tile) {
       constexpr int i = decltype(tile)::value / TN, j = decltype(tile)::value % TN;
@@ -373,13 +419,44 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   });
 }
 
+// Upper bound on the number of K splits per tile (environment FLUIDML_SPLITK, default 4; 1 = never split).
+inline int64_t SplitKLimit() {
+  static const int64_t limit = [] {
+    const char *v = std::getenv("FLUIDML_SPLITK");
+    const long n = v != nullptr ? std::strtol(v, nullptr, 10) : 4;
+    return static_cast<int64_t>(n < 1 ? 1 : n);
+  }();
+  return limit;
+}
+
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV>
 void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   MatmulArgs q = p;
   q.tiles_m = (p.M + BM - 1) / BM;
   q.tiles_n = (p.N + BN - 1) / BN;
-  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV>), dim3(q.tiles_m * q.tiles_n, n_batch),
-                     dim3(64 * WM * WN * KS), 0, s, q, C, A, B);
+  uint32_t splits = 1;
+  if constexpr (WM * WN == 1 && KS > 1) {
+    static_assert(BM * BN == kWorkspaceTileFloats, "a partial tile fills one workspace slot");
+    // Few tiles and a long K: give each tile to several workgroups.  Measured on MI355X (M = 128..256): with
+    // about 100 tiles, 2 splits of 3 chunks (K = 768) and 4 splits of 4..6 chunks (K = 2048, 3072) win by
+    // 8 % to 40 %; from about 400 tiles on, or with fewer than 3 chunks per split, the exchange of the
+    // partial tiles costs more than the extra workgroups bring.
+    const int64_t tiles = static_cast<int64_t>(q.tiles_m) * q.tiles_n * n_batch;
+    const int64_t n_chunks = (p.K + BK - 1) / BK;
+    int64_t want = std::min<int64_t>(n_chunks / 3, static_cast<int64_t>(kWorkspaceTiles) / tiles);
+    want = std::min<int64_t>(want, SplitKLimit());
+    if (tiles > 256) want = 1;
+    if (want >= 2) {
+      if (StreamWorkspace *ws = GetStreamWorkspace(s)) {
+        q.chunks_per_split = static_cast<int32_t>((n_chunks + want - 1) / want);
+        splits = static_cast<uint32_t>((n_chunks + q.chunks_per_split - 1) / q.chunks_per_split);
+        q.partials = ws->partials;
+        q.counters = ws->counters;
+      }
+    }
+  }
+  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV>),
+            dim3(q.tiles_m * q.tiles_n, n_batch, splits), dim3(64 * WM * WN * KS), 0, s, q, C, A, B);
 }
 
 // Useful fraction of the MFMA work when the problem is cut into bm x bn tiles.

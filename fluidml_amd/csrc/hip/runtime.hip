@@ -2,6 +2,9 @@
 // and launch-plan capture.  It replaces what the reference gets from
 // mlir::ExecutionEngine and a per-call host vector (src/worker/runner.cpp:56-120,
 // src/structure/context/context.cpp:152-166).
+#include <mutex>
+#include <unordered_map>
+
 #include "fl_common.h"
 
 using namespace fl;
@@ -19,6 +22,42 @@ __global__ __launch_bounds__(256) void FillZero(uint32_t *p, size_t n_words, uin
 }  // namespace
 
 namespace fl {
+namespace {
+std::mutex g_workspace_mutex;
+std::unordered_map<hipStream_t, StreamWorkspace> g_workspaces;
+}  // namespace
+
+StreamWorkspace *GetStreamWorkspace(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_workspace_mutex);
+  auto it = g_workspaces.find(stream);
+  if (it != g_workspaces.end()) return &it->second;
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  if (status != hipStreamCaptureStatusNone) return nullptr;  // no allocation while a graph is recorded
+  StreamWorkspace ws;
+  if (hipMalloc(reinterpret_cast<void **>(&ws.partials), kWorkspaceTiles * kWorkspaceTileFloats * sizeof(float)) != hipSuccess ||
+      hipMalloc(reinterpret_cast<void **>(&ws.counters), kWorkspaceTiles * sizeof(uint32_t)) != hipSuccess ||
+      hipMemset(ws.counters, 0, kWorkspaceTiles * sizeof(uint32_t)) != hipSuccess) {
+    (void)hipGetLastError();
+    if (ws.partials) (void)hipFree(ws.partials);
+    if (ws.counters) (void)hipFree(ws.counters);
+    return nullptr;
+  }
+  return &g_workspaces.emplace(stream, ws).first->second;
+}
+
+void DropStreamWorkspace(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_workspace_mutex);
+  auto it = g_workspaces.find(stream);
+  if (it == g_workspaces.end()) return;
+  (void)hipFree(it->second.partials);
+  (void)hipFree(it->second.counters);
+  g_workspaces.erase(it);
+}
+
 KernelTimer &ThreadKernelTimer() {
   static thread_local KernelTimer timer;
   return timer;
@@ -152,11 +191,14 @@ int fluidml_hip_stream_create(void **stream) {
   hipStream_t s = nullptr;
   FL_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
   *stream = s;
+  (void)GetStreamWorkspace(s);  // now, so that a later capture on this stream finds it
   return FL_OK;
 }
 
 int fluidml_hip_stream_destroy(void *stream) {
   if (stream == nullptr) return FL_OK;
+  FL_HIP_CHECK(hipStreamSynchronize(AsStream(stream)));
+  DropStreamWorkspace(AsStream(stream));
   FL_HIP_CHECK(hipStreamDestroy(AsStream(stream)));
   return FL_OK;
 }

@@ -523,6 +523,26 @@ def test_matmul_large_tiles(device):
             assert_close(do.logical(), want.astype(np.float32), what="matmul large vs float64 numpy")
 
 
+def test_matmul_split_k(device):
+    """Few tiles and a long K: the tile's K range is split over several workgroups whose partial tiles are
+    added in split order by the last one to arrive -- the result must not depend on arrival order."""
+    cabi = _cabi()
+    rng = np.random.default_rng(80)
+    for M, K, N in [(128, 768, 768), (128, 3072, 768), (100, 1000, 70), (1, 4096, 512)]:
+        a, b = rand(rng, (M, K), -1, 1), rand(rng, (K, N), -0.05, 0.05)
+        want = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+        announce("matmul split k", M, K, N)
+        da, db = DeviceView(ok.View(a), device), DeviceView(ok.View(b), device)
+        runs = []
+        for _ in range(4):
+            do = DeviceView(ok.View.empty((M, N), fill=3), device)
+            cabi.call("matmul", da.ref(), db.ref(), do.ref(), None)
+            runs.append(do.logical())
+        assert_close(runs[0], want, what="matmul split k vs float64 numpy")
+        for r in runs[1:]:
+            assert (r == runs[0]).all(), "split-K sum depends on the run"
+
+
 def test_matmul_unaligned(device):
     cabi = _cabi()
     rng = np.random.default_rng(78)

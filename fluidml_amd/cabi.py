@@ -143,6 +143,7 @@ SIGNATURES = {
     "fluidml_hip_gemm_constant_weights_bias": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _u32, _vp],
     "fluidml_hip_matmul_add": [_T, _T, _T, _T, _vp],
     "fluidml_hip_matmul_chain": [_T, _T, _T, _T, _vp, _vp],
+    "fluidml_hip_matmul_chain_view": [_T, _T, _T, _T, _i64, _i64, _vp, _vp],
     "fluidml_hip_gemm_chain": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _vp, _vp],
     "fluidml_hip_conv_chain": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _vp],
     "fluidml_hip_elementwise_chain": [_T, _T, _vp, _vp],

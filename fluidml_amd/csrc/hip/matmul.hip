@@ -59,6 +59,10 @@ struct MatmulArgs {
   fl_ew_program chain;
   // split K over gridDim.z workgroups per tile: each takes `chunks_per_split` chunks, writes its partial tile
   // to `partials`, and the workgroup that arrives last at `counters[tile]` adds them up in split order
+  // optional two-level column addressing of C: column n lives at (n / n_inner) * sCn_outer + (n % n_inner) * sCn
+  // (the last output dim reshaped into two dims that a transpose moved apart); n_inner == 0: n * sCn
+  int32_t n_inner, sCn_outer;
+  FastDiv div_inner;
   int32_t chunks_per_split;
   float *partials;
   uint32_t *counters;
@@ -392,6 +396,11 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
       constexpr int i = decltype(tile)::value / TN, j = decltype(tile)::value % TN;
       const int n = n0 + (wn * TN + j) * 32 + lrow;
       int64_t col = static_cast<int64_t>(n) * p.sCn;
+      if (!CONV && p.n_inner != 0) {
+        uint32_t hi, lo;
+        p.div_inner.DivMod(static_cast<uint32_t>(n < p.N ? n : 0), hi, lo);
+        col = static_cast<int64_t>(hi) * p.sCn_outer + static_cast<int64_t>(lo) * p.sCn;
+      }
       if constexpr (CONV) {
         uint32_t img, r, oh, ow;
         p.conv.div_ohw.DivMod(static_cast<uint32_t>(n < p.N ? n : 0), img, r);
@@ -481,7 +490,8 @@ void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
 }
 
 int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, bool trans_a, bool trans_b, float ca,
-             float cb, const fl_tensor *bias, void *stream, const fl_ew_program *chain = nullptr) {
+             float cb, const fl_tensor *bias, void *stream, const fl_ew_program *chain = nullptr, int64_t n_inner = 0,
+             int64_t stride_outer = 0) {
   FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(lhs));
   FL_CHECK(CheckView(rhs));
@@ -539,6 +549,12 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   p.ca = ca;
   p.cb = cb;
   if (chain != nullptr) p.chain = *chain;
+  if (n_inner != 0) {
+    if (n_inner < 0 || p.N % n_inner != 0 || stride_outer < 0 || stride_outer > INT32_MAX) return FL_ERR_ATTR;
+    p.n_inner = static_cast<int32_t>(n_inner);
+    p.sCn_outer = static_cast<int32_t>(stride_outer);
+    p.div_inner = FastDiv(static_cast<uint32_t>(n_inner));
+  }
   if (bias != nullptr) {
     FL_CHECK(CheckView(bias));
     if (bias->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
@@ -688,6 +704,13 @@ int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const f
   if (!lhs || !rhs || !out) return FL_ERR_NULL;
   if (bias != nullptr && bias->rank != 1) return FL_ERR_RANK;
   return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain);
+}
+
+int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
+                                  int64_t n_inner, int64_t stride_outer, const fl_ew_program *chain, void *stream) {
+  if (!lhs || !rhs || !out) return FL_ERR_NULL;
+  if (bias != nullptr && bias->rank != 1) return FL_ERR_RANK;
+  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, n_inner, stride_outer);
 }
 
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,

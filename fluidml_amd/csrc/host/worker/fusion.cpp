@@ -9,6 +9,7 @@
 #include <optional>
 #include <unordered_map>
 
+#include "utils/utils.h"
 #include "worker/launcher.h"
 
 namespace fluidml {
@@ -45,6 +46,131 @@ bool Alias(const Operand &x, const Operand &y) {
 }
 
 bool IsFloat(const Operand &o) { return o.meta.GetType() == Type::kFloat32; }
+
+// Follows a tensor through Reshape / Transpose steps and answers whether the result is just the source tensor
+// re-addressed.  Every source dim is kept as a run of "atoms" (factors of its extent, outermost first); a reshape
+// regroups the row-major sequence of atoms and may cut one in two, a transpose permutes groups.
+class ViewTracker {
+ public:
+  explicit ViewTracker(const std::vector<int64_t> &source_shape) {
+    for (size_t d = 0; d < source_shape.size(); ++d) {
+      atoms_.push_back({static_cast<int>(d), source_shape[d]});
+      dims_.push_back({static_cast<int>(atoms_.size()) - 1});
+    }
+    n_source_dims_ = source_shape.size();
+  }
+
+  // row-major reshape to `shape`; false (state unusable) if an atom would have to be cut unevenly
+  bool Reshape(const std::vector<int64_t> &shape) {
+    std::vector<int> flat;
+    for (const auto &d : dims_) flat.insert(flat.end(), d.begin(), d.end());
+    std::vector<std::vector<int>> out;
+    size_t pos = 0;
+    for (int64_t extent : shape) {
+      std::vector<int> group;
+      int64_t need = extent;
+      while (need > 1) {
+        if (pos >= flat.size()) return false;
+        const int a = flat[pos];
+        const int64_t e = atoms_[a].extent;
+        if (e == 1) {
+          ++pos;
+        } else if (need % e == 0) {
+          group.push_back(a);
+          need /= e;
+          ++pos;
+        } else if (e % need == 0) {
+          // the outer part of the atom completes this dim, the inner part stays for the next one
+          atoms_.push_back({atoms_[a].source_dim, e / need});
+          const int inner = static_cast<int>(atoms_.size()) - 1;
+          atoms_[a].extent = need;
+          if (auto it = inner_of_.find(a); it != inner_of_.end()) inner_of_[inner] = it->second;
+          inner_of_[a] = inner;
+          group.push_back(a);
+          flat[pos] = inner;
+          need = 1;
+        } else {
+          return false;
+        }
+      }
+      out.push_back(std::move(group));
+    }
+    for (; pos < flat.size(); ++pos) {
+      if (atoms_[flat[pos]].extent != 1) return false;
+    }
+    dims_ = std::move(out);
+    return true;
+  }
+
+  bool Transpose(const std::vector<int64_t> &perm) {
+    if (perm.size() != dims_.size()) return false;
+    std::vector<std::vector<int>> out;
+    for (int64_t p : perm) {
+      if (p < 0 || static_cast<size_t>(p) >= dims_.size()) return false;
+      out.push_back(dims_[static_cast<size_t>(p)]);
+    }
+    dims_ = std::move(out);
+    return true;
+  }
+
+  struct View {
+    std::vector<int64_t> strides;  // per source dim
+    int64_t n_inner = 0, stride_outer = 0;  // split of the last source dim, if any
+  };
+
+  // Strides of the source dims inside a tensor of the current shape stored with `strides`.  Every source dim
+  // must come out as one stride, except the last one which may be two (outer, inner).
+  std::optional<View> Resolve(const std::vector<int64_t> &strides) const {
+    if (strides.size() != dims_.size()) return std::nullopt;
+    std::vector<int64_t> atom_stride(atoms_.size(), 0);
+    for (size_t d = 0; d < dims_.size(); ++d) {
+      int64_t run = strides[d];
+      for (size_t k = dims_[d].size(); k-- > 0;) {
+        atom_stride[dims_[d][k]] = run;
+        run *= atoms_[dims_[d][k]].extent;
+      }
+    }
+    View v;
+    v.strides.assign(n_source_dims_, 0);
+    for (size_t d = 0; d < n_source_dims_; ++d) {
+      // atoms of this source dim, outermost first, merged where contiguous, unit extents dropped
+      std::vector<std::pair<int64_t, int64_t>> parts;  // (extent, stride)
+      for (int a = static_cast<int>(d); a >= 0;) {
+        if (atoms_[a].extent != 1) {
+          if (!parts.empty() && parts.back().second == atom_stride[a] * atoms_[a].extent) {
+            parts.back().first *= atoms_[a].extent;
+            parts.back().second = atom_stride[a];
+          } else {
+            parts.push_back({atoms_[a].extent, atom_stride[a]});
+          }
+        }
+        auto it = inner_of_.find(a);
+        a = it == inner_of_.end() ? -1 : it->second;
+      }
+      if (parts.empty()) continue;
+      if (parts.size() == 1) {
+        v.strides[d] = parts[0].second;
+      } else if (parts.size() == 2 && d + 1 == n_source_dims_) {
+        v.stride_outer = parts[0].second;
+        v.n_inner = parts[1].first;
+        v.strides[d] = parts[1].second;
+      } else {
+        return std::nullopt;
+      }
+    }
+    return v;
+  }
+
+ private:
+  struct Atom {
+    int source_dim;
+    int64_t extent;
+  };
+  std::vector<Atom> atoms_;                  // atoms 0..n_source_dims-1 are the outermost atom of each source dim
+  std::unordered_map<int, int> inner_of_;    // atom -> the atom cut off its inner side
+  std::vector<std::vector<int>> dims_;       // current dims, each a run of atoms (outermost first)
+  size_t n_source_dims_ = 0;
+};
 
 class Scheduler {
  public:
@@ -298,6 +424,17 @@ class Scheduler {
       l.members.insert(l.members.end(), chain->members.begin(), chain->members.end());
       l.chain = chain->program;
     }
+    // MatMul only: trailing Reshape / Transpose steps that merely re-address the result are folded into the
+    // kernel's output strides (the head split and merge copies of an attention block)
+    if (l.kind == Launch::Kind::MatMulChain) {
+      Launch with_views = l;
+      if (AppendViews(i, &with_views) && with_views.members.size() >= 2 &&
+          Safe(with_views.members, {{i, l.a}, {i, l.b}}) && OutputDisjoint(with_views.out, {&l.a, &l.b})) {
+        with_views.bytes = l.has_c ? Bytes({&l.a, &l.b, &l.c, &with_views.out}) : Bytes({&l.a, &l.b, &with_views.out});
+        with_views.flops = Flops(with_views.members);
+        return with_views;
+      }
+    }
     // longest variant whose late reads are safe: with the chain, then without it
     for (int attempt = 0; attempt < 2; ++attempt) {
       if (l.members.size() < 2) return std::nullopt;  // nothing fused
@@ -312,6 +449,51 @@ class Scheduler {
       l.chain = fl_ew_program{};
     }
     return std::nullopt;
+  }
+
+  // Extends `l` (a MatMulChain headed by step `head`) by the longest run of single-reader Reshape / Transpose
+  // steps after which the contraction's logical output is still a strided view of the final tensor.
+  bool AppendViews(size_t head, Launch *l) const {
+    ViewTracker tracker(steps_[head].out.meta.GetShape());
+    size_t cur = l->members.back();
+    std::vector<size_t> views;
+    size_t best = 0;
+    ViewTracker::View best_view;
+    while (true) {
+      const auto j = SoleReader(cur);
+      if (!j || !IsFloat(steps_[*j].out)) break;
+      bool ok = false;
+      switch (Kind(*j)) {
+        case OpKind::Reshape:
+        case OpKind::Flatten:
+        case OpKind::Squeeze:
+        case OpKind::Unsqueeze: ok = tracker.Reshape(steps_[*j].out.meta.GetShape()); break;
+        case OpKind::Transpose: {
+          std::vector<int64_t> perm = Attrs(*j).perm;
+          if (perm.empty()) {
+            for (int64_t d = static_cast<int64_t>(steps_[*j].out.meta.GetShape().size()); d-- > 0;) perm.push_back(d);
+          }
+          ok = tracker.Transpose(perm);
+          break;
+        }
+        default: break;
+      }
+      if (!ok) break;
+      views.push_back(*j);
+      cur = *j;
+      const Operand &o = steps_[*j].out;
+      if (auto v = tracker.Resolve(utils::GenStrides(o.meta.GetShape(), o.layout))) {
+        best = views.size();
+        best_view = *v;
+      }
+    }
+    if (best == 0) return false;
+    l->members.insert(l->members.end(), views.begin(), views.begin() + static_cast<std::ptrdiff_t>(best));
+    l->out = steps_[l->members.back()].out;
+    l->view_strides = best_view.strides;
+    l->n_inner = best_view.n_inner;
+    l->stride_outer = best_view.stride_outer;
+    return true;
   }
 
   // Two or more elementwise steps on a tensor that stays live (or is a graph input).

@@ -220,7 +220,15 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
       kernel::TensorView c;
       if (l.has_c) c = ViewOf(Resolve(l.c), l.c);
-      rc = fluidml_hip_matmul_chain(&a.t, &b.t, l.has_c ? &c.t : nullptr, &out.t, &l.chain, ctx.stream);
+      if (l.view_strides.empty()) {
+        rc = fluidml_hip_matmul_chain(&a.t, &b.t, l.has_c ? &c.t : nullptr, &out.t, &l.chain, ctx.stream);
+      } else {
+        // the contraction's logical output addressed inside the buffer of the last folded Reshape / Transpose
+        kernel::TensorView dst(out.t.base, steps_[l.members[0]].out.meta);
+        for (size_t d = 0; d < l.view_strides.size(); ++d) dst.t.strides[d] = l.view_strides[d];
+        rc = fluidml_hip_matmul_chain_view(&a.t, &b.t, l.has_c ? &c.t : nullptr, &dst.t, l.n_inner, l.stride_outer,
+                                           &l.chain, ctx.stream);
+      }
       break;
     }
     case Launch::Kind::GemmChain: {

@@ -69,6 +69,11 @@ struct Launch {
   int64_t axis = 0;
   std::vector<int64_t> perm;
   bool has_c = false;     // MatMulChain: a bias operand is present
+  // MatMulChain followed by Reshape/Transpose steps that only re-address the result: element strides of the
+  // contraction's logical output dims inside `out` (empty: `out` is the contraction's own output tensor),
+  // and the optional split of the last dim (see fluidml_hip_matmul_chain_view)
+  std::vector<int64_t> view_strides;
+  int64_t n_inner = 0, stride_outer = 0;
   fl_ew_program chain{};  // elementwise steps applied to the value (n == 0: none)
   size_t owner = 0;  // member whose kernel owns constants / attributes the launch needs (LayerNorm, Gemm, Conv)
   double bytes = 0, flops = 0;

@@ -325,6 +325,14 @@ int fluidml_hip_matmul_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
  * result, e.g. the erf-GELU chain Div, Erf, Add, Mul(x), Mul of
  * add_div_erf_add_mul_mul.cpp:29-132.  `bias` and `chain` may be NULL. */
 int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, const fl_ew_program *chain, void *stream);
+/* The same, followed by Reshape / Transpose steps that only re-address the
+ * result (reference reshape.cpp:18-64, transpose.cpp:19-48): `out` carries the
+ * contraction's logical shape [..., M, N] with the element strides each of
+ * those dims has inside the final buffer.  If the reshape split N into
+ * (N / n_inner, n_inner) and the transpose moved the two apart, column n is
+ * stored at (n / n_inner) * stride_outer + (n % n_inner) * out->strides[last];
+ * n_inner == 0 means plain strides. */
+int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, int64_t n_inner, int64_t stride_outer, const fl_ew_program *chain, void *stream);
 /* GemmConstantWeightsBiasKernel -> elementwise chain (reference gemm.cpp:39-182). */
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double alpha, double beta, int32_t trans_a, int32_t trans_b, const fl_ew_program *chain, void *stream);
 /* Conv{With,Without}PaddingKernel -> elementwise chain (reference conv.cpp:27-280);

@@ -620,6 +620,35 @@ def test_fused_matmul_add_and_gelu(device):
             assert_close(do.logical(), u1.logical(), what="matmul_chain relu, scale")
 
 
+def test_matmul_chain_view(device):
+    """MatMul + bias written straight into the buffer of a following Reshape (last dim split into heads) and
+    Transpose: the head-split copies of an attention block folded into the contraction's output addressing."""
+    cabi = _cabi()
+    rng = np.random.default_rng(96)
+    S, H, heads, d = 24, 48, 4, 12
+    a, b, bias = rand(rng, (1, S, H), -1, 1), rand(rng, (H, H), -0.2, 0.2), rand(rng, (H,), -0.5, 0.5)
+    t0, t1 = ok.View.empty((1, S, H)), ok.View.empty((1, S, H))
+    ok.matmul(ok.View(a), ok.View(b), t0)
+    ok.binary_f32(ok.BOP_ADD, ok.View(bias), t0, t1)
+    r = ok.View.empty((1, S, heads, d))
+    ok.reshape(t1, r)
+    for perm, lout in [((0, 2, 1, 3), None), ((0, 2, 3, 1), None), ((0, 2, 1, 3), [3, 1, 0, 2])]:
+        oshape = tuple((1, S, heads, d)[p] for p in perm)
+        want = ok.View.empty(oshape)
+        ok.transpose(r, want, list(perm))
+        announce("matmul chain view", perm, lout)
+        final = ok.View.empty(oshape, np.float32, lout, fill=5)
+        dfinal = DeviceView(final, device)
+        fs = final.strides  # strides of the transposed tensor's dims
+        pos = {p: k for k, p in enumerate(perm)}  # reshape dim -> transposed dim
+        # logical [1, S, H]: dim 0 and dim 1 map to reshape dims 0 and 1, H splits into (heads, d)
+        view = cabi.make_tensor(dfinal.tensor.base, cabi.FL_FLOAT32, [1, S, H], [fs[pos[0]], fs[pos[1]], fs[pos[3]]])
+        da, db, dbias = DeviceView(ok.View(a), device), DeviceView(ok.View(b), device), DeviceView(ok.View(bias), device)
+        cabi.call("matmul_chain_view", da.ref(), db.ref(), dbias.ref(), ctypes.byref(view), ctypes.c_int64(d),
+                  ctypes.c_int64(fs[pos[2]]), None, None)
+        assert_close(dfinal.logical(), want.logical(), what="matmul_chain_view")
+
+
 def test_elementwise_chain(device):
     """Every chain operation against the oracle's standalone kernels, applied one after the other."""
     cabi = _cabi()

@@ -63,6 +63,13 @@ struct MatmulArgs {
   // (the last output dim reshaped into two dims that a transpose moved apart); n_inner == 0: n * sCn
   int32_t n_inner, sCn_outer;
   FastDiv div_inner;
+  // sibling contractions that share A and every extent, one per blockIdx.y (n_groups <= 1: none; batch
+  // dims are then absent).  Member 0 uses the fields above, member g > 0 the entries g - 1 below.
+  int32_t n_groups;
+  const float *gB[3];
+  float *gC[3];
+  const float *gbias[3];
+  int32_t g_sCm[3], g_sCn[3], g_sCn_outer[3];
   int32_t chunks_per_split;
   float *partials;
   uint32_t *counters;
@@ -133,9 +140,11 @@ struct TileLoader {
 // LB: 0 = B tile kept [k][n] (B is n-contiguous), 1 = kept [n][k].
 // CONV: B is the input of a convolution addressed through p.conv (LB must be 0, scalar gathers).
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV = false>
-__global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, float *__restrict__ C,
+__global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, float *__restrict__ C_,
                                                                 const float *__restrict__ A,
-                                                                const float *__restrict__ B) {
+                                                                const float *__restrict__ B_) {
+  float *__restrict__ C = C_;
+  const float *__restrict__ B = B_;
   constexpr int NT = 64 * WM * WN * KS;
   constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);
   constexpr int KW = BK / KS;  // k extent one wave covers per chunk
@@ -164,9 +173,25 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   const int tile_m = bid % p.tiles_m, tile_n = bid / p.tiles_m;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
+  // which sibling of a grouped launch this workgroup serves
+  const float *bias = p.bias;
+  int32_t sCm = p.sCm, sCn = p.sCn, sCn_outer = p.sCn_outer;
+  uint32_t batch_id = blockIdx.y;
+  if (p.n_groups > 1) {
+    if (batch_id > 0) {
+      const uint32_t g = batch_id - 1;
+      B = p.gB[g];
+      C = p.gC[g];
+      bias = p.gbias[g];
+      sCm = p.g_sCm[g];
+      sCn = p.g_sCn[g];
+      sCn_outer = p.g_sCn_outer[g];
+    }
+    batch_id = 0;
+  }
   int32_t boff[3] = {0, 0, 0};
   {
-    uint32_t rem = blockIdx.y;
+    uint32_t rem = batch_id;
     for (int d = p.batch.rank - 1; d > 0; --d) {
       uint32_t q, r;
       p.batch.div[d].DivMod(rem, q, r);
@@ -395,11 +420,11 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   StaticFor<TM * TN>([&](auto tile) {
       constexpr int i = decltype(tile)::value / TN, j = decltype(tile)::value % TN;
       const int n = n0 + (wn * TN + j) * 32 + lrow;
-      int64_t col = static_cast<int64_t>(n) * p.sCn;
+      int64_t col = static_cast<int64_t>(n) * sCn;
       if (!CONV && p.n_inner != 0) {
         uint32_t hi, lo;
         p.div_inner.DivMod(static_cast<uint32_t>(n < p.N ? n : 0), hi, lo);
-        col = static_cast<int64_t>(hi) * p.sCn_outer + static_cast<int64_t>(lo) * p.sCn;
+        col = static_cast<int64_t>(hi) * sCn_outer + static_cast<int64_t>(lo) * sCn;
       }
       if constexpr (CONV) {
         uint32_t img, r, oh, ow;
@@ -414,8 +439,8 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
         float v = acc[i][j][e];
-        if (p.bias != nullptr && m < p.M && n < p.N) {
-          v = p.ca * v + p.cb * p.bias[m * p.sDm + n * p.sDn];
+        if (bias != nullptr && m < p.M && n < p.N) {
+          v = p.ca * v + p.cb * bias[m * p.sDm + n * p.sDn];
         }
         vals[e] = v;
       }
@@ -423,7 +448,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
-        if (m < p.M && n < p.N) Cb[static_cast<int64_t>(m) * p.sCm + col] = vals[e];
+        if (m < p.M && n < p.N) Cb[static_cast<int64_t>(m) * sCm + col] = vals[e];
       }
   });
 }
@@ -489,9 +514,18 @@ void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
   }
 }
 
+// Siblings of a grouped launch: same lhs, same extents and rhs strides, own rhs / bias / out buffers.
+struct Siblings {
+  int count = 0;  // members beyond the first, at most 3
+  const fl_tensor *rhs[3];
+  const fl_tensor *bias[3];
+  const fl_tensor *out[3];
+  int64_t stride_outer[3];
+};
+
 int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, bool trans_a, bool trans_b, float ca,
              float cb, const fl_tensor *bias, void *stream, const fl_ew_program *chain = nullptr, int64_t n_inner = 0,
-             int64_t stride_outer = 0) {
+             int64_t stride_outer = 0, const Siblings *siblings = nullptr) {
   FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(lhs));
   FL_CHECK(CheckView(rhs));
@@ -577,12 +611,44 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   const float *B = static_cast<const float *>(rhs->base);
   hipStream_t s = AsStream(stream);
 
+  bool siblings_aligned = true;
+  if (siblings != nullptr && siblings->count > 0) {
+    if (siblings->count > 3 || n_batch != 1) return FL_ERR_UNSUPPORTED;
+    for (int g = 0; g < siblings->count; ++g) {
+      const fl_tensor *r = siblings->rhs[g], *o = siblings->out[g], *bs = siblings->bias[g];
+      FL_CHECK(CheckView(r));
+      FL_CHECK(CheckView(o));
+      if (r->dtype != FL_FLOAT32 || o->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+      if (r->rank != rhs->rank || o->rank != out->rank || (bs == nullptr) != (bias == nullptr)) return FL_ERR_SHAPE;
+      for (int i = 0; i < rr; ++i) {
+        if (r->shape[i] != rhs->shape[i] || r->strides[i] != rhs->strides[i]) return FL_ERR_SHAPE;
+      }
+      for (int i = 0; i < orank; ++i) {
+        if (o->shape[i] != out->shape[i]) return FL_ERR_SHAPE;
+      }
+      if (bs != nullptr) {
+        FL_CHECK(CheckView(bs));
+        if (bs->dtype != FL_FLOAT32 || bs->rank != bias->rank || bs->shape[0] != bias->shape[0] ||
+            bs->strides[0] != bias->strides[0]) return FL_ERR_SHAPE;
+        p.gbias[g] = static_cast<const float *>(bs->base);
+      }
+      p.gB[g] = static_cast<const float *>(r->base);
+      p.gC[g] = static_cast<float *>(o->base);
+      p.g_sCm[g] = static_cast<int32_t>(o->strides[orank - 2]);
+      p.g_sCn[g] = static_cast<int32_t>(o->strides[orank - 1]);
+      p.g_sCn_outer[g] = static_cast<int32_t>(siblings->stride_outer[g]);
+      siblings_aligned = siblings_aligned && IsAligned(r->base, 16);
+    }
+    p.n_groups = siblings->count + 1;
+    n_batch = p.n_groups;  // one grid row per sibling
+  }
+
   // Layout of each staged tile follows the operand's fast dimension; 128-bit
   // loads need that dimension to have unit stride and everything else to keep
   // 16-byte alignment.
   const int la = (p.sAk <= p.sAm || p.M == 1) ? 0 : 1;
   const int lb = (p.sBn <= p.sBk || p.K == 1) ? 0 : 1;
-  bool vec = IsAligned(A, 16) && IsAligned(B, 16);
+  bool vec = IsAligned(A, 16) && IsAligned(B, 16) && siblings_aligned;
   if (la == 0) vec = vec && (p.sAk == 1 || p.K == 1) && p.K % 4 == 0 && p.sAm % 4 == 0;
   else vec = vec && p.sAm == 1 && p.M % 4 == 0 && p.sAk % 4 == 0;
   if (lb == 0) vec = vec && (p.sBn == 1 || p.N == 1) && p.N % 4 == 0 && p.sBk % 4 == 0;
@@ -711,6 +777,27 @@ int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, co
   if (!lhs || !rhs || !out) return FL_ERR_NULL;
   if (bias != nullptr && bias->rank != 1) return FL_ERR_RANK;
   return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, n_inner, stride_outer);
+}
+
+int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs,
+                                   const fl_tensor *const *bias, const fl_tensor *const *out, int64_t n_inner,
+                                   const int64_t *stride_outer, const fl_ew_program *chain, void *stream) {
+  if (!lhs || !rhs || !out) return FL_ERR_NULL;
+  if (count < 1 || count > 4) return FL_ERR_ATTR;
+  fl::Siblings sib;
+  sib.count = count - 1;
+  for (int g = 0; g < count; ++g) {
+    if (!rhs[g] || !out[g]) return FL_ERR_NULL;
+    if (bias != nullptr && bias[g] != nullptr && bias[g]->rank != 1) return FL_ERR_RANK;
+    if (g > 0) {
+      sib.rhs[g - 1] = rhs[g];
+      sib.out[g - 1] = out[g];
+      sib.bias[g - 1] = bias != nullptr ? bias[g] : nullptr;
+      sib.stride_outer[g - 1] = stride_outer != nullptr ? stride_outer[g] : 0;
+    }
+  }
+  return fl::Contract(lhs, rhs[0], out[0], false, false, 1.0f, 1.0f, bias != nullptr ? bias[0] : nullptr, stream, chain,
+                      n_inner, stride_outer != nullptr ? stride_outer[0] : 0, &sib);
 }
 
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,

@@ -73,6 +73,12 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
     py::dict d;
     d["kind"] = worker::LaunchKindName(l.kind);
     d["members"] = l.members;
+    // members whose output tensor the launch writes (the rest are elided intermediates)
+    std::vector<size_t> written;
+    if (l.group.empty()) written.push_back(l.members.back());
+    for (const worker::Launch &m : l.group) written.push_back(m.members.back());
+    d["written"] = written;
+    d["position"] = l.group.empty() ? l.members.back() : l.position;
     d["bytes"] = l.bytes;
     d["flops"] = l.flops;
     launches.append(d);

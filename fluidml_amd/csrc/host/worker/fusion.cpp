@@ -19,6 +19,7 @@ const char *LaunchKindName(Launch::Kind kind) {
   switch (kind) {
     case Launch::Kind::Step: return "Step";
     case Launch::Kind::MatMulChain: return "MatMulChain";
+    case Launch::Kind::MatMulGroup: return "MatMulGroup";
     case Launch::Kind::GemmChain: return "GemmChain";
     case Launch::Kind::ConvChain: return "ConvChain";
     case Launch::Kind::ElementwiseChain: return "ElementwiseChain";
@@ -216,9 +217,10 @@ class Scheduler {
         }
       }
     }
+    if (fuse) GroupSiblings(&fused);
     // a chain is issued where its last member stood; everything else keeps its place
     std::vector<const Launch *> at(steps_.size(), nullptr);
-    for (const Launch &l : fused) at[l.members.back()] = &l;
+    for (const Launch &l : fused) at[l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back()] = &l;
     std::vector<Launch> schedule;
     for (size_t i = 0; i < steps_.size(); ++i) {
       if (at[i] != nullptr) {
@@ -493,6 +495,134 @@ class Scheduler {
     l->view_strides = best_view.strides;
     l->n_inner = best_view.n_inner;
     l->stride_outer = best_view.stride_outer;
+    return true;
+  }
+
+  // MatMulChains that read the same left operand with the same extents (the query / key / value projections)
+  // become one launch at the position of the last of them, provided that moving the earlier ones there
+  // crosses no reader of their outputs and no write to what they read.
+  void GroupSiblings(std::vector<Launch> *fused) const {
+    auto compatible = [&](const Launch &x, const Launch &y) {
+      if (x.kind != Launch::Kind::MatMulChain || y.kind != Launch::Kind::MatMulChain) return false;
+      const Step &hx = steps_[x.members[0]], &hy = steps_[y.members[0]];
+      const auto &shape = hx.out.meta.GetShape();
+      int64_t batch = 1;
+      for (size_t d = 0; d + 2 < shape.size(); ++d) batch *= shape[d];
+      return SameTensor(x.a, y.a) && x.a.layout == y.a.layout && batch == 1 && shape == hy.out.meta.GetShape() &&
+             x.b.space == Operand::Space::Constant && y.b.space == Operand::Space::Constant &&
+             x.b.meta.GetShape() == y.b.meta.GetShape() && x.b.layout == y.b.layout && x.has_c == y.has_c &&
+             x.n_inner == y.n_inner && x.view_strides.empty() == y.view_strides.empty() && x.chain.n == y.chain.n &&
+             std::equal(x.chain.op, x.chain.op + x.chain.n, y.chain.op) &&
+             std::equal(x.chain.c, x.chain.c + x.chain.n, y.chain.c);
+    };
+    std::vector<bool> used(fused->size(), false);
+    std::vector<Launch> result;
+    for (size_t i = 0; i < fused->size(); ++i) {
+      if (used[i]) continue;
+      std::vector<size_t> set = {i};
+      for (size_t j = i + 1; j < fused->size() && set.size() < 4; ++j) {
+        if (!used[j] && compatible((*fused)[i], (*fused)[j])) set.push_back(j);
+      }
+      // the largest prefix of the candidates that can meet at the position of one of them
+      size_t position = 0;
+      while (set.size() >= 2) {
+        bool found = false;
+        for (size_t k : set) {
+          if (CanGroupAt(*fused, set, (*fused)[k].members.back())) {
+            position = (*fused)[k].members.back();
+            found = true;
+            break;
+          }
+        }
+        if (found) break;
+        set.pop_back();
+      }
+      if (set.size() < 2) {
+        result.push_back((*fused)[i]);
+        used[i] = true;
+        continue;
+      }
+      Launch g;
+      g.kind = Launch::Kind::MatMulGroup;
+      for (size_t k : set) {
+        used[k] = true;
+        const Launch &m = (*fused)[k];
+        g.members.insert(g.members.end(), m.members.begin(), m.members.end());
+        g.flops += m.flops;
+        g.bytes += m.bytes - (k == set[0] ? 0.0 : static_cast<double>(m.a.meta.GetSize()));
+        g.group.push_back(m);
+      }
+      std::sort(g.members.begin(), g.members.end());
+      std::sort(g.group.begin(), g.group.end(), [](const Launch &x, const Launch &y) { return x.members.back() < y.members.back(); });
+      g.a = g.group[0].a;
+      g.out = g.group.back().out;
+      g.position = position;
+      result.push_back(std::move(g));
+    }
+    *fused = std::move(result);
+  }
+
+  // Can every launch of `set` be issued at step position `position` (the last member of one of them)?
+  bool CanGroupAt(const std::vector<Launch> &fused, const std::vector<size_t> &set, size_t position) const {
+    std::vector<size_t> members;
+    for (size_t k : set) members.insert(members.end(), fused[k].members.begin(), fused[k].members.end());
+    auto is_member = [&](size_t s) { return std::find(members.begin(), members.end(), s) != members.end(); };
+    for (size_t k : set) {
+      const Launch &l = fused[k];
+      const size_t own = l.members.back();
+      if (own <= position) {
+        // delayed: its reads of the left operand (weights and bias are constants) move from the chain's head
+        // to `position`, and its output appears later than planned
+        for (size_t s = l.members[0] + 1; s < position; ++s) {
+          if (!is_member(s) && Alias(steps_[s].out, l.a)) return false;
+        }
+        auto it = readers_.find(l.out.name);
+        if (it != readers_.end()) {
+          for (size_t r : it->second) {
+            if (r <= position) return false;
+          }
+        }
+      } else {
+        // hoisted: the left operand must exist already, and the output's bytes, reserved only from `own` on,
+        // must not be touched by anything that runs between the new and the planned position
+        if (l.members[0] <= position) return false;  // part of the chain already ran: not a pure hoist
+        auto producer_before = [&](const Operand &op) {
+          if (op.space == Operand::Space::Constant || op.space == Operand::Space::Interface) {
+            // constants always exist; interface tensors are graph inputs unless a step writes them
+            for (size_t s = position; s < steps_.size(); ++s) {
+              if (SameTensor(steps_[s].out, op)) return false;
+            }
+            return true;
+          }
+          for (size_t s = 0; s < position; ++s) {
+            if (SameTensor(steps_[s].out, op)) return true;
+          }
+          return false;
+        };
+        if (!producer_before(l.a)) return false;
+        for (size_t s = position; s <= own; ++s) {
+          if (is_member(s)) continue;
+          const Step &st = steps_[s];
+          if (Alias(st.out, l.out) || Alias(st.in0, l.out)) return false;
+          if (st.node->IsDoubleInputs() && Alias(st.in1, l.out)) return false;
+          if (st.has_buffer && l.out.space == Operand::Space::Arena && st.buffer_offset < l.out.offset + l.out.meta.GetSize() &&
+              l.out.offset < st.buffer_offset + st.buffer_bytes) {
+            return false;  // scratch of a step in between (untouched by these kernels, but reserved)
+          }
+        }
+      }
+      // the output must not overlap what a member reads at the common position
+      for (size_t other : set) {
+        if (Alias(l.out, fused[other].a)) return false;
+      }
+    }
+    // outputs of different members are live together from the later one's planned position on, but a hoisted
+    // output and a not-yet-dead neighbour could still collide: all outputs pairwise disjoint
+    for (size_t x : set) {
+      for (size_t y : set) {
+        if (x < y && Alias(fused[x].out, fused[y].out)) return false;
+      }
+    }
     return true;
   }
 

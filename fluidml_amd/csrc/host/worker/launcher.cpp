@@ -231,6 +231,30 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       }
       break;
     }
+    case Launch::Kind::MatMulGroup: {
+      const size_t n = l.group.size();
+      std::vector<kernel::TensorView> rhs(n), bias(n), dst(n);
+      std::vector<const fl_tensor *> rhs_p(n), bias_p(n), dst_p(n);
+      std::vector<int64_t> outer(n);
+      for (size_t g = 0; g < n; ++g) {
+        const Launch &m = l.group[g];
+        rhs[g] = ViewOf(Resolve(m.b), m.b);
+        if (m.has_c) bias[g] = ViewOf(Resolve(m.c), m.c);
+        if (m.view_strides.empty()) {
+          dst[g] = ViewOf(Resolve(m.out), m.out);
+        } else {
+          dst[g] = kernel::TensorView(Resolve(m.out), steps_[m.members[0]].out.meta);
+          for (size_t d = 0; d < m.view_strides.size(); ++d) dst[g].t.strides[d] = m.view_strides[d];
+        }
+        rhs_p[g] = &rhs[g].t;
+        bias_p[g] = m.has_c ? &bias[g].t : nullptr;
+        dst_p[g] = &dst[g].t;
+        outer[g] = m.stride_outer;
+      }
+      rc = fluidml_hip_matmul_chain_group(static_cast<int32_t>(n), &a.t, rhs_p.data(), bias_p.data(), dst_p.data(),
+                                          l.group[0].n_inner, outer.data(), &l.group[0].chain, ctx.stream);
+      break;
+    }
     case Launch::Kind::GemmChain: {
       const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
       const flow::Attrs &at = steps_[l.owner].node->GetAttrs();

@@ -56,6 +56,7 @@ struct Launch {
     MatMulChain,       // MatMul [-> AddCommon(rank-1 constant bias)] [-> elementwise chain]
     GemmChain,         // GemmConstantWeightsBias -> elementwise chain
     ConvChain,         // Conv{With,Without}Padding -> elementwise chain
+    MatMulGroup,       // up to four MatMulChains that share the left operand and all extents, one launch
     ElementwiseChain,  // two or more elementwise steps on one tensor
     DivAddSoftmax,     // DivConstantRhs -> AddCommon(mask) -> Softmax
     AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias
@@ -74,6 +75,9 @@ struct Launch {
   // and the optional split of the last dim (see fluidml_hip_matmul_chain_view)
   std::vector<int64_t> view_strides;
   int64_t n_inner = 0, stride_outer = 0;
+  // MatMulGroup: the grouped chains (members = union of theirs; every chain's `out` is written)
+  std::vector<Launch> group;
+  size_t position = 0;  // MatMulGroup: step index where the launch is issued (one of the members)
   fl_ew_program chain{};  // elementwise steps applied to the value (n == 0: none)
   size_t owner = 0;  // member whose kernel owns constants / attributes the launch needs (LayerNorm, Gemm, Conv)
   double bytes = 0, flops = 0;

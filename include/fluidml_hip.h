@@ -333,6 +333,11 @@ int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const f
  * stored at (n / n_inner) * stride_outer + (n % n_inner) * out->strides[last];
  * n_inner == 0 means plain strides. */
 int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, int64_t n_inner, int64_t stride_outer, const fl_ew_program *chain, void *stream);
+/* `count` (1..4) such launches that share `lhs`, every extent, the strides of
+ * `rhs`, `n_inner` and `chain`, as ONE launch (the query / key / value
+ * projections of an attention block): rhs[i], bias[i] (all NULL or none),
+ * out[i] and stride_outer[i] belong to member i.  No batch dims. */
+int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs, const fl_tensor *const *bias, const fl_tensor *const *out, int64_t n_inner, const int64_t *stride_outer, const fl_ew_program *chain, void *stream);
 /* GemmConstantWeightsBiasKernel -> elementwise chain (reference gemm.cpp:39-182). */
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double alpha, double beta, int32_t trans_a, int32_t trans_b, const fl_ew_program *chain, void *stream);
 /* Conv{With,Without}PaddingKernel -> elementwise chain (reference conv.cpp:27-280);

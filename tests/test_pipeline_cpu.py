@@ -318,7 +318,7 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     plan = ex.plan()
     steps, launches = plan["steps"], plan["launches"]
     assert sorted(m for l in launches for m in l["members"]) == list(range(len(steps)))
-    assert [l["members"][-1] for l in launches] == sorted(l["members"][-1] for l in launches)
+    assert [l["position"] for l in launches] == sorted(l["position"] for l in launches)
     kinds = {l["kind"] for l in launches}
     assert expected_kinds <= kinds
     readers = {}
@@ -331,22 +331,40 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
         if l["kind"] == "Step":
             assert len(members) == 1
             continue
-        inside = {steps[m]["out"]["name"] for m in members[:-1]}
-        for m in members[:-1]:
+        written = set(l["written"])
+        position = l["position"]  # the step index where the launch is issued
+        assert position in members
+        if l["kind"] != "MatMulGroup":
+            assert position == members[-1] and written == {members[-1]}
+        inside = {steps[m]["out"]["name"] for m in members if m not in written}
+        producer = {s["out"]["name"]: i for i, s in enumerate(steps)}
+        for m in members:
             out = steps[m]["out"]
-            assert out["space"] in ("arena", "private")
-            assert readers[out["name"]] <= set(members), "an elided tensor is read outside its chain"
-        final = steps[members[-1]]["out"]
+            if m in written:
+                # written at `position`: no reader may come earlier ...
+                assert all(r in members or r > position for r in readers.get(out["name"], ())), "read before written"
+                # ... and if that is earlier than planned, nothing in between may touch the bytes
+                for s in range(position, m):
+                    if s not in members:
+                        for op in steps[s]["inputs"] + [steps[s]["out"]]:
+                            assert not _overlap(op, out), "a hoisted output lands on bytes still in use"
+            else:
+                assert out["space"] in ("arena", "private")
+                assert readers[out["name"]] <= set(members), "an elided tensor is read outside its chain"
+        finals = [steps[m]["out"] for m in written]
         for m in members:
             for op in steps[m]["inputs"]:
                 if op["name"] in inside:
                     continue
-                for s in range(m + 1, members[-1]):
+                for s in range(m + 1, position):
                     if s not in members:
                         assert not _overlap(steps[s]["out"], op), "a read was moved across a write to its bytes"
-                if _overlap(final, op):  # only row-wise / elementwise kernels may work in place, and only exactly
-                    assert l["kind"] in ("DivAddSoftmax", "ElementwiseChain")
-                    assert final["offset"] == op["offset"] and final["layout"] == op["layout"]
+                if m > position and op["name"] in producer:
+                    assert producer[op["name"]] < position, "a hoisted read precedes its producer"
+                for final in finals:
+                    if _overlap(final, op):  # only row-wise / elementwise kernels may work in place, and only exactly
+                        assert l["kind"] in ("DivAddSoftmax", "ElementwiseChain")
+                        assert final["offset"] == op["offset"] and final["layout"] == op["layout"]
     # switched off: one launch per step
     monkeypatch.setenv("FLUIDML_FUSE", "0")
     ex = getattr(fluidml.Executor, flavour)("sched_off")

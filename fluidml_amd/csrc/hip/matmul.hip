@@ -453,6 +453,96 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   });
 }
 
+// ---- skinny contraction: M <= 8 rows against a k-contiguous B (weight streaming, HBM bound) ----------------
+// One wave owns kSkinnyRows (1, 2 or 4: fewer when N alone cannot fill the chip) consecutive columns n of C, i.e. rows of B as stored: lanes stride K with 128-bit
+// loads of those rows and of the M rows of A (small, served by the caches), keep M x kSkinnyRows partial sums
+// each and combine them with wave64 shuffles.  No LDS, no MFMA: at one to eight rows the matrix cores would
+// run 75-97 % empty while the kernel waits for the weights anyway.
+template <int MT, int kSkinnyRows>
+__global__ __launch_bounds__(256) void SkinnyGemmKernel(MatmulArgs p, float *__restrict__ C, const float *__restrict__ A,
+                                                        const float *__restrict__ B) {
+  const int lane = threadIdx.x % 64;
+  const int n0 = (blockIdx.x * 4 + threadIdx.x / 64) * kSkinnyRows;
+  if (n0 >= p.N) return;
+  float acc[MT][kSkinnyRows];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < kSkinnyRows; ++r) acc[m][r] = 0.0f;
+  const float *brow[kSkinnyRows];
+#pragma unroll
+  for (int r = 0; r < kSkinnyRows; ++r) brow[r] = B + static_cast<int64_t>(min(n0 + r, p.N - 1)) * p.sBn;
+  // two 256-wide k steps per iteration: 2 x kSkinnyRows 128-bit weight loads in flight per lane
+  for (int k = lane * 4; k < p.K; k += 512) {
+    const bool second = k + 256 < p.K;
+    floatx4 b0[kSkinnyRows], b1[kSkinnyRows], a0[MT], a1[MT];
+#pragma unroll
+    for (int r = 0; r < kSkinnyRows; ++r) {
+      b0[r] = *reinterpret_cast<const floatx4 *>(brow[r] + k);
+      b1[r] = second ? *reinterpret_cast<const floatx4 *>(brow[r] + k + 256) : floatx4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const float *arow = A + static_cast<int64_t>(m) * p.sAm + k;
+      a0[m] = m < p.M ? *reinterpret_cast<const floatx4 *>(arow) : floatx4{0, 0, 0, 0};
+      a1[m] = m < p.M && second ? *reinterpret_cast<const floatx4 *>(arow + 256) : floatx4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < kSkinnyRows; ++r) {
+        acc[m][r] += a0[m].x * b0[r].x;
+        acc[m][r] += a0[m].y * b0[r].y;
+        acc[m][r] += a0[m].z * b0[r].z;
+        acc[m][r] += a0[m].w * b0[r].w;
+        acc[m][r] += a1[m].x * b1[r].x;
+        acc[m][r] += a1[m].y * b1[r].y;
+        acc[m][r] += a1[m].z * b1[r].z;
+        acc[m][r] += a1[m].w * b1[r].w;
+      }
+  }
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < kSkinnyRows; ++r) acc[m][r] = WaveReduce(acc[m][r], SumOp{});
+  if (lane == 0) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < kSkinnyRows; ++r) {
+        const int n = n0 + r;
+        if (m < p.M && n < p.N) {
+          float v = acc[m][r];
+          if (p.bias != nullptr) v = p.ca * v + p.cb * p.bias[m * p.sDm + n * p.sDn];
+          if (p.chain.n != 0) v = RunChain(p.chain, v);
+          C[static_cast<int64_t>(m) * p.sCm + static_cast<int64_t>(n) * p.sCn] = v;
+        }
+      }
+  }
+}
+
+// Launches the skinny kernel if the problem fits it; false = use the tiled kernel.
+inline bool TrySkinnyGemm(const MatmulArgs &p, int64_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
+  if (n_batch != 1 || p.M > 8 || p.N < 256 || p.K < 256 || p.n_inner != 0 || p.n_groups > 1) return false;
+  if (p.sBk != 1 || p.sAk != 1 || p.K % 4 != 0 || p.sBn % 4 != 0 || (p.M > 1 && p.sAm % 4 != 0)) return false;
+  if (!IsAligned(A, 16) || !IsAligned(B, 16)) return false;
+  // rows per wave: as many as still leave about eight waves per compute unit
+  const int rows = p.N >= 4 * 2048 ? 4 : (p.N >= 2 * 2048 || p.M > 2) ? 2 : 1;
+  const dim3 grid((p.N + 4 * rows - 1) / (4 * rows)), block(256);
+#define FL_SKINNY(MT_)                                                                              \
+  do {                                                                                              \
+    if (rows == 4) FL_LAUNCH((SkinnyGemmKernel<MT_, 4>), grid, block, 0, s, p, C, A, B);            \
+    else if (rows == 2) FL_LAUNCH((SkinnyGemmKernel<MT_, 2>), grid, block, 0, s, p, C, A, B);       \
+    else FL_LAUNCH((SkinnyGemmKernel<MT_, 1>), grid, block, 0, s, p, C, A, B);                      \
+  } while (0)
+  if (p.M == 1) FL_SKINNY(1);
+  else if (p.M == 2) FL_SKINNY(2);
+  else if (p.M <= 4) FL_SKINNY(4);
+  else FL_SKINNY(8);
+#undef FL_SKINNY
+  return true;
+}
+
 // Upper bound on the number of K splits per tile (environment FLUIDML_SPLITK, default 4; 1 = never split).
 inline int64_t SplitKLimit() {
   static const int64_t limit = [] {
@@ -656,6 +746,7 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   for (int i = 0; i < nest.rank && vec; ++i) {
     if (nest.strides[1][i] % 4 != 0 || nest.strides[2][i] % 4 != 0) vec = false;
   }
+  if (TrySkinnyGemm(p, n_batch, C, A, B, s)) return LaunchStatus();
   const uint32_t nb = static_cast<uint32_t>(n_batch);
 #define FL_MM_DISPATCH(LA_, LB_)                              \
   if (la == LA_ && lb == LB_) {                               \

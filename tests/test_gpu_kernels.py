@@ -561,7 +561,10 @@ def test_gemm(device):
     rng = np.random.default_rng(51)
     # reference gemm.py: [1,768] x [768,768]^T + [768], alpha = beta = 1
     cases = [((1, 768), (768, 768), (768,), 1.0, 1.0, 0, 1), ((8, 100), (100, 50), (50,), 0.5, 2.0, 0, 0),
-             ((100, 8), (50, 100), (8, 50), 1.5, 0.25, 1, 1), ((33, 65), (65, 17), (33, 17), 2.0, 3.0, 0, 0)]
+             ((100, 8), (50, 100), (8, 50), 1.5, 0.25, 1, 1), ((33, 65), (65, 17), (33, 17), 2.0, 3.0, 0, 0),
+             # few rows against k-contiguous weights: the weight-streaming kernel (1, 2, 3..4 and 5..8 row variants)
+             ((8, 2048), (1000, 2048), (1000,), 1.0, 1.0, 0, 1), ((3, 4096), (515, 4096), (515,), 1.0, 1.0, 0, 1),
+             ((2, 1024), (300, 1024), (2, 300), 0.5, 2.0, 0, 1), ((5, 512), (257, 512), (257,), 1.0, 1.0, 0, 1)]
     for ashape, bshape, cshape, alpha, beta, ta, tb in cases:
         a, b, c = rand(rng, ashape, -1, 1), rand(rng, bshape, -0.05, 0.05), rand(rng, cshape, -1, 1)
         M = ashape[1] if ta else ashape[0]

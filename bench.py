@@ -2,7 +2,7 @@
 """Benchmark of the hot path: BERT-base encoder (batch 1, seq 128, fp32) compiled by
 Executor.make_dp_greedy-equivalent planning and replayed as HIP launches over one HBM arena.
 
-A "step" is one inference: one replay of the whole launch plan (416 graph nodes issued as 189 kernel
+A "step" is one inference: one replay of the whole launch plan (416 graph nodes issued as 135 kernel
 launches after launch-level fusion) on inputs that are already resident in HBM.  Prints ONE JSON line; see DESIGN.md for how every field is derived.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--executor plain_greedy|dp_greedy]
@@ -23,10 +23,10 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the contraction kernel on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch, averaged over the 96 contraction launches of an inference), each scaled by what the
-# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x1.000): (3912.5 * 2.0 + 576.0) KiB.
+# (KiB per dispatch, averaged over the 85 contraction launches of an inference), each scaled by what the
+# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x1.000): (4514.3 * 2.0 + 1308.3) KiB.
 # Only valid for the default workload (BERT-base, seq 128, 12 layers, plain_greedy, fusion on).
-MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 8_601_851
+MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 10_583_891
 
 
 def cpu_baseline(layers_total: int, sample_layers: int, seq: int):

@@ -293,10 +293,99 @@ int Binary(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, Op 
   return LaunchNest<2, T, T, T, Empty>(nest, out->base, lhs->base, rhs->base, nullptr, op, AsStream(stream));
 }
 
+// Copy whose fastest output dim is not the fastest input dim (a transposing layout change): 64x64 tiles go
+// through LDS so that both the global reads (along the input's unit-stride dim) and the global writes (along
+// the output's) are coalesced.  `outer` enumerates the remaining dims (operand 0 = out, 1 = in).
+struct TiledCopyArgs {
+  NestArgs<2> outer;
+  uint32_t n_out_fast, n_in_fast;  // extents of the output-fast dim and of the input-fast dim
+  int32_t in_stride_of_out_fast;   // input stride along the output-fast dim
+  int32_t out_stride_of_in_fast;   // output stride along the input-fast dim
+  uint32_t tiles_out_fast, tiles_in_fast;
+};
+
+__global__ __launch_bounds__(256) void TiledCopyKernel(TiledCopyArgs a, uint32_t *__restrict__ out,
+                                                       const uint32_t *__restrict__ in) {
+  __shared__ uint32_t tile[64][65];
+  const uint32_t t_of = blockIdx.x % a.tiles_out_fast, t_if = (blockIdx.x / a.tiles_out_fast) % a.tiles_in_fast;
+  uint32_t rem = blockIdx.x / (a.tiles_out_fast * a.tiles_in_fast);
+  int32_t off_out = 0, off_in = 0;
+  for (int d = a.outer.rank - 1; d >= 0; --d) {
+    uint32_t q = 0, r = rem;
+    if (d > 0) a.outer.div[d].DivMod(rem, q, r);
+    rem = q;
+    off_out += static_cast<int32_t>(r) * a.outer.strides[0][d];
+    off_in += static_cast<int32_t>(r) * a.outer.strides[1][d];
+  }
+  const uint32_t of0 = t_of * 64, if0 = t_if * 64;
+  const uint32_t lane = threadIdx.x % 64, row = threadIdx.x / 64;
+  // read: lanes run along the input-fast dim
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const uint32_t jo = of0 + row + 4 * r, ji = if0 + lane;
+    if (jo < a.n_out_fast && ji < a.n_in_fast) {
+      tile[row + 4 * r][lane] = in[off_in + static_cast<int32_t>(jo) * a.in_stride_of_out_fast + static_cast<int32_t>(ji)];
+    }
+  }
+  __syncthreads();
+  // write: lanes run along the output-fast dim
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const uint32_t ji = if0 + row + 4 * r, jo = of0 + lane;
+    if (jo < a.n_out_fast && ji < a.n_in_fast) {
+      out[off_out + static_cast<int32_t>(ji) * a.out_stride_of_in_fast + static_cast<int32_t>(jo)] = tile[lane][row + 4 * r];
+    }
+  }
+}
+
+// Launches the tiled kernel when `nest` (operand 0 = out, 1 = in, 32-bit elements) is a transposing copy of
+// useful size; false = use the generic element-per-lane path.
+bool TryTiledCopy(LoopNest nest, const fl_tensor *in, const fl_tensor *out, hipStream_t stream) {
+  nest.Canonicalise();
+  const int inner = nest.rank - 1;
+  if (nest.rank < 2 || nest.strides[0][inner] != 1 || nest.strides[1][inner] == 1) return false;
+  int in_fast = -1;
+  for (int d = 0; d < inner; ++d) {
+    if (nest.strides[1][d] == 1) in_fast = d;
+  }
+  if (in_fast < 0 || nest.shape[inner] < 32 || nest.shape[in_fast] < 32) return false;
+  TiledCopyArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.n_out_fast = static_cast<uint32_t>(nest.shape[inner]);
+  a.n_in_fast = static_cast<uint32_t>(nest.shape[in_fast]);
+  a.in_stride_of_out_fast = static_cast<int32_t>(nest.strides[1][inner]);
+  a.out_stride_of_in_fast = static_cast<int32_t>(nest.strides[0][in_fast]);
+  a.tiles_out_fast = (a.n_out_fast + 63) / 64;
+  a.tiles_in_fast = (a.n_in_fast + 63) / 64;
+  LoopNest outer;
+  outer.n_operands = 2;
+  outer.rank = 0;
+  int64_t n_outer = 1;
+  for (int d = 0; d < inner; ++d) {
+    if (d == in_fast) continue;
+    outer.shape[outer.rank] = nest.shape[d];
+    outer.strides[0][outer.rank] = nest.strides[0][d];
+    outer.strides[1][outer.rank] = nest.strides[1][d];
+    n_outer *= nest.shape[d];
+    ++outer.rank;
+  }
+  if (outer.rank == 0) {
+    outer.rank = 1;
+    outer.shape[0] = 1;
+  }
+  const int64_t blocks = n_outer * a.tiles_out_fast * a.tiles_in_fast;
+  if (blocks > INT32_MAX) return false;
+  a.outer = MakeNestArgs<2>(outer);
+  FL_LAUNCH(TiledCopyKernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, stream, a,
+            static_cast<uint32_t *>(out->base), static_cast<const uint32_t *>(in->base));
+  return true;
+}
+
 // Copy `in` (already re-strided to the output's index space) into `out`,
 // whatever the (equal) element type is.
 int CopyNest(const LoopNest &nest, const fl_tensor *in, const fl_tensor *out, void *stream) {
   if (in->dtype != out->dtype) return FL_ERR_DTYPE;
+  if (DtypeSize(out->dtype) == 4 && TryTiledCopy(nest, in, out, AsStream(stream))) return LaunchStatus();
   switch (DtypeSize(out->dtype)) {
     case 1: return Unary<uint8_t, uint8_t>(nest, in, out, Copy<uint8_t, uint8_t>{}, stream);
     case 2: return Unary<uint16_t, uint16_t>(nest, in, out, Copy<uint16_t, uint16_t>{}, stream);
@@ -328,6 +417,20 @@ int StridedCopy(const fl_tensor *in, int64_t in_offset, const int64_t *in_stride
 }
 
 namespace {
+
+// Elementwise chain on two tensors stored identically (the usual case): flat 128-bit accesses, eight values
+// per lane, one wave-uniform branch per chain step for all eight.
+__global__ __launch_bounds__(256) void ChainFlatKernel(fl_ew_program g, uint32_t n_vec8, float *__restrict__ out,
+                                                       const float *__restrict__ in) {
+  typedef float float4v __attribute__((ext_vector_type(4)));
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_vec8) return;
+  const float4v lo = reinterpret_cast<const float4v *>(in)[2 * i], hi = reinterpret_cast<const float4v *>(in)[2 * i + 1];
+  float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  RunChainBlock<8>(g, v);
+  reinterpret_cast<float4v *>(out)[2 * i] = float4v{v[0], v[1], v[2], v[3]};
+  reinterpret_cast<float4v *>(out)[2 * i + 1] = float4v{v[4], v[5], v[6], v[7]};
+}
 
 // Pad: one lane per output element; inside the interior it copies the input, outside it writes zero.
 struct PadArgs {
@@ -689,6 +792,24 @@ int fluidml_hip_concat2(const fl_tensor *lhs, const fl_tensor *rhs, const fl_ten
 int fluidml_hip_elementwise_chain(const fl_tensor *in, const fl_tensor *out, const fl_ew_program *chain, void *stream) {
   if (chain == nullptr) return FL_ERR_NULL;
   FL_CHECK(CheckChain(chain));
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (in->dtype == FL_FLOAT32 && out->dtype == FL_FLOAT32 && SameShape(in, out)) {
+    // same dense storage on both sides?
+    bool same = true;
+    int64_t numel = 1, span = 0;
+    for (int i = 0; i < in->rank; ++i) {
+      same = same && (in->strides[i] == out->strides[i] || in->shape[i] == 1);
+      numel *= in->shape[i];
+      span += (in->shape[i] - 1) * in->strides[i];
+    }
+    if (same && span + 1 == numel && numel % 8 == 0 && IsAligned(in->base, 16) && IsAligned(out->base, 16)) {
+      const uint32_t n_vec8 = static_cast<uint32_t>(numel / 8);
+      FL_LAUNCH(ChainFlatKernel, dim3((n_vec8 + 255) / 256), dim3(256), 0, AsStream(stream), *chain, n_vec8,
+                static_cast<float *>(out->base), static_cast<const float *>(in->base));
+      return LaunchStatus();
+    }
+  }
   return UnaryF32(in, out, Chain{*chain}, stream);
 }
 

@@ -133,6 +133,40 @@ __global__ __launch_bounds__(kBlock) void SoftmaxRowBlock(RowArgs<3> a, float *_
   for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) dst[j] = expf(at(j) - m) / s;
 }
 
+// One block per row, row cached in registers: len <= 256 * ITEMS (read once, written once).
+template <int ITEMS>
+__global__ __launch_bounds__(kBlock) void SoftmaxRowBlockCached(RowArgs<3> a, float *__restrict__ out,
+                                                                const float *__restrict__ in, SoftmaxPre pre) {
+  __shared__ float smem[kBlock / kWave];
+  int32_t off[3];
+  RowOffsets<3>(a.outer, blockIdx.x, off);
+  const float *src = in + off[1];
+  float *dst = out + off[0];
+  const int32_t sm = a.axis_stride[2];
+  float x[ITEMS];
+  float m = -__FLT_MAX__;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = threadIdx.x + i * kBlock;
+    x[i] = j < a.len ? pre(src[j], off[2] + static_cast<int32_t>(j) * sm) : -__FLT_MAX__;
+    m = fmaxf(m, x[i]);
+  }
+  m = BlockReduce<kBlock / kWave>(m, MaxOp{}, smem);
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = threadIdx.x + i * kBlock;
+    x[i] = j < a.len ? expf(x[i] - m) : 0.0f;
+    s += x[i];
+  }
+  s = BlockReduce<kBlock / kWave>(s, SumOp{}, smem);
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = threadIdx.x + i * kBlock;
+    if (j < a.len) dst[j] = x[i] / s;
+  }
+}
+
 // One lane per row; the axis is walked with its stride.
 __global__ __launch_bounds__(kBlock) void SoftmaxColumn(RowArgs<3> a, float *__restrict__ out,
                                                         const float *__restrict__ in, SoftmaxPre pre) {
@@ -194,6 +228,53 @@ __global__ __launch_bounds__(kBlock) void LayerNormRowBlock(RowArgs<6> a, float 
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t j = threadIdx.x + i * kBlock;
+    if (j < a.len) dst[j] = (x[i] * inv) * g[static_cast<int32_t>(j) * sg] + b[static_cast<int32_t>(j) * sb];
+  }
+}
+
+// One wave per row, row cached in registers: len <= 64 * ITEMS; no workgroup barrier at all.
+template <int ITEMS>
+__global__ __launch_bounds__(kBlock) void LayerNormRowWave(RowArgs<6> a, float *__restrict__ out,
+                                                           const float *__restrict__ in,
+                                                           const float *__restrict__ scale,
+                                                           const float *__restrict__ bias,
+                                                           const float *__restrict__ scratch, float eps,
+                                                           int stale_scratch, const float *__restrict__ addend) {
+  const uint32_t lane = threadIdx.x % kWave;
+  const uint32_t row = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  if (row >= a.n_rows) return;
+  int32_t off[6];
+  RowOffsets<6>(a.outer, row, off);
+  const float *src = in + off[1];
+  const float n = static_cast<float>(a.len);
+  float x[ITEMS];
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = lane + i * kWave;
+    x[i] = j < a.len ? src[j] : 0.0f;
+    if (addend != nullptr && j < a.len) x[i] = x[i] + addend[off[5] + static_cast<int32_t>(j) * a.axis_stride[5]];
+    s += x[i];
+  }
+  s = WaveReduce(s, SumOp{});
+  if (stale_scratch) s += scratch[off[4]];
+  const float mean = s / n;
+  float v = 0.0f;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = lane + i * kWave;
+    x[i] = j < a.len ? x[i] - mean : 0.0f;
+    v += x[i] * x[i];
+  }
+  v = WaveReduce(v, SumOp{});
+  const float inv = 1.0f / sqrtf(v / n + eps);
+  float *dst = out + off[0];
+  const float *g = scale + off[2];
+  const float *b = bias + off[3];
+  const int32_t sg = a.axis_stride[2], sb = a.axis_stride[3];
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = lane + i * kWave;
     if (j < a.len) dst[j] = (x[i] * inv) * g[static_cast<int32_t>(j) * sg] + b[static_cast<int32_t>(j) * sb];
   }
 }
@@ -369,6 +450,12 @@ static int SoftmaxImpl(const fl_tensor *in, const fl_tensor *mask, float div, co
       FL_LAUNCH(SoftmaxRowWave<8>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x, pre);
     } else if (a.len <= 1024) {
       FL_LAUNCH(SoftmaxRowWave<16>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x, pre);
+    } else if (a.len <= 8 * kBlock) {
+      FL_LAUNCH(SoftmaxRowBlockCached<8>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, pre);
+    } else if (a.len <= 16 * kBlock) {
+      FL_LAUNCH(SoftmaxRowBlockCached<16>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, pre);
+    } else if (a.len <= 32 * kBlock) {
+      FL_LAUNCH(SoftmaxRowBlockCached<32>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, pre);
     } else {
       FL_LAUNCH(SoftmaxRowBlock, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, pre);
     }
@@ -443,7 +530,16 @@ static int LayerNormImpl(const fl_tensor *in, const fl_tensor *addend, const fl_
   hipStream_t s = AsStream(stream);
   const bool row_contig = a.axis_stride[0] == 1 && a.axis_stride[1] == 1;
   if (row_contig && a.len > 64) {
-    if (a.len <= kBlock) {
+    const dim3 wave_grid((a.n_rows + kBlock / kWave - 1) / (kBlock / kWave));
+    if (a.len <= 4 * kWave) {
+      FL_LAUNCH(LayerNormRowWave<4>, wave_grid, dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
+    } else if (a.len <= 8 * kWave && a.n_rows >= 1024) {
+      FL_LAUNCH(LayerNormRowWave<8>, wave_grid, dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
+    } else if (a.len <= 12 * kWave && a.n_rows >= 1024) {
+      FL_LAUNCH(LayerNormRowWave<12>, wave_grid, dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
+    } else if (a.len <= 16 * kWave && a.n_rows >= 1024) {
+      FL_LAUNCH(LayerNormRowWave<16>, wave_grid, dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
+    } else if (a.len <= kBlock) {
       FL_LAUNCH(LayerNormRowBlock<1>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
     } else if (a.len <= 2 * kBlock) {
       FL_LAUNCH(LayerNormRowBlock<2>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
@@ -451,6 +547,10 @@ static int LayerNormImpl(const fl_tensor *in, const fl_tensor *addend, const fl_
       FL_LAUNCH(LayerNormRowBlock<4>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
     } else if (a.len <= 8 * kBlock) {
       FL_LAUNCH(LayerNormRowBlock<8>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
+    } else if (a.len <= 16 * kBlock) {
+      FL_LAUNCH(LayerNormRowBlock<16>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
+    } else if (a.len <= 32 * kBlock) {
+      FL_LAUNCH(LayerNormRowBlock<32>, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
     } else {
       FL_LAUNCH(LayerNormRowLoop, dim3(a.n_rows), dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);
     }

@@ -99,6 +99,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-layers", type=int, default=3)
     ap.add_argument("--per-kernel", action="store_true", help="also print a per-kernel table to stderr")
+    ap.add_argument("--bf16", action="store_true",
+                    help="additionally run the opt-in bf16 contraction path and report its throughput and its "
+                         "error against the fp32 result under \"bf16\" (the headline value stays fp32)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="instead of the benchmark, launch the identity-copy kernel 3 times on a buffer of MIB MiB "
                          "(a kernel of known traffic, to scale profiler byte counters) and exit")
@@ -234,6 +237,33 @@ def main():
                         "sum_of_kernel_ms": kernel_sum_ms, "invoke_with_host_copies_ms": invoke_ms,
                         "compile_s": compile_s},
     }
+    if args.bf16:
+        ref_out = {k: v.copy() for k, v in outs.items()}
+        ex.invoke(io)
+        ref_out = {k: outs[k].copy() for k in outs}
+        os.environ["FLUIDML_BF16"] = "1"
+        try:
+            with tempfile.TemporaryDirectory() as tmp:
+                path = net.save(os.path.join(tmp, args.config + ".onnx"))
+                ex16 = getattr(fluidml.Executor, "make_" + args.executor)(args.config + "_bf16", 1)
+                ex16.compile(path)
+        finally:
+            os.environ["FLUIDML_BF16"] = "0"
+        ex16.invoke(io)
+        got = {k: outs[k].copy() for k in outs}
+        ex16.replay(args.warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ex16.replay(args.steps)
+        torch.cuda.synchronize()
+        el = time.perf_counter() - t0
+        name = next(iter(got))
+        err = np.abs(got[name].astype(np.float64) - ref_out[name].astype(np.float64))
+        result["bf16"] = {"value": batch * args.steps / el, "unit": "inferences/s", "ms_per_step": el / args.steps * 1e3,
+                          "max_abs_err_vs_fp32": float(err.max()),
+                          "max_abs_err_over_max_abs_output": float(err.max() / np.abs(ref_out[name]).max()),
+                          "mean_abs_err_vs_fp32": float(err.mean()),
+                          "note": "MatMul operands rounded to bf16 (nearest even), fp32 accumulation; Gemm/Conv stay fp32"}
     if not args.no_cpu_baseline:
         if args.config == "bert_base":
             result["cpu_baseline"] = cpu_baseline(args.layers, min(args.cpu_sample_layers, args.layers), args.seq)

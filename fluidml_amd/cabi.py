@@ -27,6 +27,7 @@ FL_REF_LN_STALE_SCRATCH = 1 << 2
 FL_REF_GEMM_SWAPPED_SCALARS = 1 << 3
 FL_REF_GATHER_RAW_AXIS = 1 << 4
 FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
+FL_CONTRACT_BF16 = 1 << 0
 
 DTYPE_SIZE = {FL_BOOL: 1, FL_INT32: 4, FL_INT64: 8, FL_FLOAT16: 2, FL_FLOAT32: 4, FL_FLOAT64: 8}
 
@@ -142,9 +143,9 @@ SIGNATURES = {
     "fluidml_hip_matmul_bf16": [_T, _T, _T, _vp],
     "fluidml_hip_gemm_constant_weights_bias": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _u32, _vp],
     "fluidml_hip_matmul_add": [_T, _T, _T, _T, _vp],
-    "fluidml_hip_matmul_chain": [_T, _T, _T, _T, _vp, _vp],
-    "fluidml_hip_matmul_chain_view": [_T, _T, _T, _T, _i64, _i64, _vp, _vp],
-    "fluidml_hip_matmul_chain_group": [_i32, _T, _vp, _vp, _vp, _i64, _i64p, _vp, _vp],
+    "fluidml_hip_matmul_chain": [_T, _T, _T, _T, _vp, _u32, _vp],
+    "fluidml_hip_matmul_chain_view": [_T, _T, _T, _T, _i64, _i64, _vp, _u32, _vp],
+    "fluidml_hip_matmul_chain_group": [_i32, _T, _vp, _vp, _vp, _i64, _i64p, _vp, _u32, _vp],
     "fluidml_hip_gemm_chain": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _vp, _vp],
     "fluidml_hip_conv_chain": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _vp],
     "fluidml_hip_elementwise_chain": [_T, _T, _vp, _vp],

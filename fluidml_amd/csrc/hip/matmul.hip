@@ -20,8 +20,10 @@
 //   * workgroup ids are folded so that consecutive tiles land on one XCD and
 //     share its L2.
 //
-// A second, opt-in path rounds operands to bf16 (v_mfma_f32_32x32x8_bf16 would
-// be its instruction); it is not built yet and reports FL_ERR_UNSUPPORTED.
+// A second, opt-in path (BF16 instantiations) rounds both operands to bf16 (round to nearest even) as they
+// leave LDS and multiplies them with v_mfma_f32_32x32x8_bf16_1k; accumulation stays fp32.  The k-to-lane
+// assignment is the one the fp32 path already uses (lane half h holds k = 4h..4h+3 of a group of 8), so one
+// bf16 instruction replaces four fp32 ones.
 #include <algorithm>
 #include <cstdlib>
 #include <type_traits>
@@ -33,6 +35,15 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef short bf16x4 __attribute__((ext_vector_type(4)));
+
+// float -> bf16 bits, round to nearest even (NaN stays NaN)
+__device__ __forceinline__ short ToBf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<short>((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<short>(u >> 16);
+}
 
 // Geometry of a convolution run as an implicit GEMM: M = output channels, N = images x output pixels,
 // K = input channels x kernel taps.  B[k][n] is gathered from the input on the fly (padding reads as 0),
@@ -139,7 +150,8 @@ struct TileLoader {
 // LA: 0 = A tile kept [m][k] (A is k-contiguous), 1 = kept [k][m].
 // LB: 0 = B tile kept [k][n] (B is n-contiguous), 1 = kept [n][k].
 // CONV: B is the input of a convolution addressed through p.conv (LB must be 0, scalar gathers).
-template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV = false>
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV = false,
+          bool BF16 = false>
 __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, float *__restrict__ C_,
                                                                 const float *__restrict__ A,
                                                                 const float *__restrict__ B_) {
@@ -314,13 +326,26 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
           b[j][3] = t.w;
         }
       }
+      if constexpr (BF16) {
+        bf16x4 ah[TM], bh[TN];
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
+        for (int i = 0; i < TM; ++i) ah[i] = bf16x4{ToBf16(a[i][0]), ToBf16(a[i][1]), ToBf16(a[i][2]), ToBf16(a[i][3])};
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bh[j] = bf16x4{ToBf16(b[j][0]), ToBf16(b[j][1]), ToBf16(b[j][2]), ToBf16(b[j][3])};
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][e], b[j][e], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(ah[i], bh[j], acc[i][j], 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][e], b[j][e], acc[i][j], 0, 0, 0);
+      }
     }
   };
 
@@ -553,7 +578,7 @@ inline int64_t SplitKLimit() {
   return limit;
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV>
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV, bool BF16>
 void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   MatmulArgs q = p;
   q.tiles_m = (p.M + BM - 1) / BM;
@@ -579,7 +604,7 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
       }
     }
   }
-  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV>),
+  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV, BF16>),
             dim3(q.tiles_m * q.tiles_n, n_batch, splits), dim3(64 * WM * WN * KS), 0, s, q, C, A, B);
 }
 
@@ -589,18 +614,18 @@ inline double TileEfficiency(int64_t m, int64_t n, int64_t bm, int64_t bn) {
          (static_cast<double>((m + bm - 1) / bm * bm) * static_cast<double>((n + bn - 1) / bn * bn));
 }
 
-template <int LA, int LB, int VEC, bool CONV>
+template <int LA, int LB, int VEC, bool CONV, bool BF16 = false>
 void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   const int64_t tiles_l = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * n_batch;
   const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
   // the big tile only when it fills the chip and does not waste much more of itself on edges than the next one
   const bool big_ok = tiles_l >= 192 && TileEfficiency(p.M, p.N, 128, 128) + 0.15 >= TileEfficiency(p.M, p.N, 64, 64);
   if (big_ok) {
-    LaunchConfig<128, 128, 16, 2, 2, 1, LA, LB, VEC, 2, CONV>(p, n_batch, C, A, B, s);
+    LaunchConfig<128, 128, 16, 2, 2, 1, LA, LB, VEC, 2, CONV, BF16>(p, n_batch, C, A, B, s);
   } else if (tiles_m >= 192) {
-    LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4, CONV>(p, n_batch, C, A, B, s);
+    LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4, CONV, BF16>(p, n_batch, C, A, B, s);
   } else {
-    LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2, CONV>(p, n_batch, C, A, B, s);
+    LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2, CONV, BF16>(p, n_batch, C, A, B, s);
   }
 }
 
@@ -615,7 +640,7 @@ struct Siblings {
 
 int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, bool trans_a, bool trans_b, float ca,
              float cb, const fl_tensor *bias, void *stream, const fl_ew_program *chain = nullptr, int64_t n_inner = 0,
-             int64_t stride_outer = 0, const Siblings *siblings = nullptr) {
+             int64_t stride_outer = 0, const Siblings *siblings = nullptr, bool bf16 = false) {
   FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(lhs));
   FL_CHECK(CheckView(rhs));
@@ -746,12 +771,18 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   for (int i = 0; i < nest.rank && vec; ++i) {
     if (nest.strides[1][i] % 4 != 0 || nest.strides[2][i] % 4 != 0) vec = false;
   }
-  if (TrySkinnyGemm(p, n_batch, C, A, B, s)) return LaunchStatus();
+  if (!bf16 && TrySkinnyGemm(p, n_batch, C, A, B, s)) return LaunchStatus();
   const uint32_t nb = static_cast<uint32_t>(n_batch);
 #define FL_MM_DISPATCH(LA_, LB_)                              \
   if (la == LA_ && lb == LB_) {                               \
-    if (vec) LaunchBySize<LA_, LB_, 4, false>(p, nb, C, A, B, s); \
-    else LaunchBySize<LA_, LB_, 1, false>(p, nb, C, A, B, s);     \
+    if (bf16) {                                                   \
+      if (vec) LaunchBySize<LA_, LB_, 4, false, true>(p, nb, C, A, B, s); \
+      else LaunchBySize<LA_, LB_, 1, false, true>(p, nb, C, A, B, s);     \
+    } else if (vec) {                                             \
+      LaunchBySize<LA_, LB_, 4, false>(p, nb, C, A, B, s);        \
+    } else {                                                      \
+      LaunchBySize<LA_, LB_, 1, false>(p, nb, C, A, B, s);        \
+    }                                                             \
   }
   FL_MM_DISPATCH(0, 0)
   FL_MM_DISPATCH(0, 1)
@@ -857,22 +888,26 @@ int fluidml_hip_matmul_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
 }
 
 int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
-                             const fl_ew_program *chain, void *stream) {
+                             const fl_ew_program *chain, uint32_t flags, void *stream) {
   if (!lhs || !rhs || !out) return FL_ERR_NULL;
   if (bias != nullptr && bias->rank != 1) return FL_ERR_RANK;
-  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain);
+  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, 0, 0, nullptr,
+                      (flags & FL_CONTRACT_BF16) != 0);
 }
 
 int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
-                                  int64_t n_inner, int64_t stride_outer, const fl_ew_program *chain, void *stream) {
+                                  int64_t n_inner, int64_t stride_outer, const fl_ew_program *chain, uint32_t flags,
+                                  void *stream) {
   if (!lhs || !rhs || !out) return FL_ERR_NULL;
   if (bias != nullptr && bias->rank != 1) return FL_ERR_RANK;
-  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, n_inner, stride_outer);
+  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, n_inner, stride_outer, nullptr,
+                      (flags & FL_CONTRACT_BF16) != 0);
 }
 
 int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs,
                                    const fl_tensor *const *bias, const fl_tensor *const *out, int64_t n_inner,
-                                   const int64_t *stride_outer, const fl_ew_program *chain, void *stream) {
+                                   const int64_t *stride_outer, const fl_ew_program *chain, uint32_t flags,
+                                   void *stream) {
   if (!lhs || !rhs || !out) return FL_ERR_NULL;
   if (count < 1 || count > 4) return FL_ERR_ATTR;
   fl::Siblings sib;
@@ -888,7 +923,7 @@ int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl
     }
   }
   return fl::Contract(lhs, rhs[0], out[0], false, false, 1.0f, 1.0f, bias != nullptr ? bias[0] : nullptr, stream, chain,
-                      n_inner, stride_outer != nullptr ? stride_outer[0] : 0, &sib);
+                      n_inner, stride_outer != nullptr ? stride_outer[0] : 0, &sib, (flags & FL_CONTRACT_BF16) != 0);
 }
 
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
@@ -901,11 +936,7 @@ int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
 }
 
 int fluidml_hip_matmul_bf16(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
-  (void)lhs;
-  (void)rhs;
-  (void)out;
-  (void)stream;
-  return FL_ERR_UNSUPPORTED;
+  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 0.0f, nullptr, stream, nullptr, 0, 0, nullptr, true);
 }
 
 int fluidml_hip_gemm_constant_weights_bias(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias,

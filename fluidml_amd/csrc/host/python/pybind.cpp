@@ -120,6 +120,7 @@ PYBIND11_MODULE(fluidml, m) {
       .def("set_ref_flags", [](context::Context &c, uint32_t flags) { c->ref_flags = flags; }, py::arg("flags"))
       .def("set_use_graph", [](context::Context &c, bool use) { c->use_graph = use; }, py::arg("use"))
       .def("set_fuse", [](context::Context &c, bool fuse) { c->fuse = fuse; }, py::arg("fuse"))
+      .def("set_bf16", [](context::Context &c, bool on) { c->bf16 = on; }, py::arg("on"))
       .def("plan_text", [](context::Context &c) { return c->GetModule().ToText(); });
 
   py::class_<flow::Flow, std::unique_ptr<flow::Flow>>(m, "Flow")

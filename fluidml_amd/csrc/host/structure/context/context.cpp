@@ -18,6 +18,7 @@ ContextImpl::ContextImpl() {
   if (const char *q = std::getenv("FLUIDML_REF_QUIRKS")) ref_flags = static_cast<uint32_t>(std::strtoul(q, nullptr, 0));
   if (const char *g = std::getenv("FLUIDML_HIP_GRAPH")) use_graph = std::string(g) != "0";
   if (const char *f = std::getenv("FLUIDML_FUSE")) fuse = std::string(f) != "0";
+  if (const char *h = std::getenv("FLUIDML_BF16")) bf16 = std::string(h) != "0";
   if (const char *c = std::getenv("FLUIDML_DP_COST")) {
     const std::string mode(c);
     if (mode == "constant") {

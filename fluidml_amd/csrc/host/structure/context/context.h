@@ -82,6 +82,8 @@ class ContextImpl {
   bool use_graph = true;
   // launch-level fusion of single-reader kernel chains (env FLUIDML_FUSE=0 disables)
   bool fuse = true;
+  // MatMul nodes on the opt-in bf16 path (env FLUIDML_BF16=1)
+  bool bf16 = false;
   // cost source of the layout DP (env FLUIDML_DP_COST=measure|constant|<path to table json>)
   CostMode cost_mode = CostMode::Measure;
   std::string cost_table_path;

@@ -242,7 +242,7 @@ class DoubleNoBuffer final : public DoubleInputsWithoutBufferKernel, public Base
       case OpKind::MulCommon: rc = fluidml_hip_mul_common(l, r, out, s); break;
       case OpKind::DivCommon: rc = fluidml_hip_div_common(l, r, out, s); break;
       case OpKind::Concat2: rc = fluidml_hip_concat2(l, r, out, NormAxis(attrs_.axis, out->rank), s); break;
-      case OpKind::MatMul: rc = fluidml_hip_matmul(l, r, out, s); break;
+      case OpKind::MatMul: rc = ctx.bf16 ? fluidml_hip_matmul_bf16(l, r, out, s) : fluidml_hip_matmul(l, r, out, s); break;
       case OpKind::GemmConstantWeightsBias: {
         const TensorView bias = Const(c0_, "bias").View();
         rc = fluidml_hip_gemm_constant_weights_bias(l, r, &bias.t, out, attrs_.alpha, attrs_.beta, attrs_.trans_a ? 1 : 0,

@@ -32,6 +32,7 @@ std::vector<std::vector<Axis>> GetAxesInAllOrders();
 struct LaunchContext {
   void *stream = nullptr;  // hipStream_t
   uint32_t flags = 0;      // FL_REF_* literal-reference switches
+  bool bf16 = false;       // MatMul on the opt-in bf16 path (operands rounded to bf16, fp32 accumulation)
   int status = 0;          // first non-zero return code of the C ABI
   std::string failed;      // kernel name that produced it
   void Note(int code, const std::string &kernel_name);

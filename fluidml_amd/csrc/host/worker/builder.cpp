@@ -152,6 +152,7 @@ class GeneralBuilderImpl : public GeneralBuilder {
     plan->SetFlags(context_->ref_flags);
     plan->SetUseGraph(context_->use_graph);
     plan->SetFuse(context_->fuse);
+    plan->SetBf16(context_->bf16);
     context_->SetModule(std::move(plan));
     context_->SetFuncAttr(std::move(func_attr));
   }

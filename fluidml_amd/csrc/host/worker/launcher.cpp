@@ -214,6 +214,7 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
     return;
   }
   const kernel::TensorView a = ViewOf(Resolve(l.a), l.a), out = ViewOf(Resolve(l.out), l.out);
+  const uint32_t contract_flags = ctx.bf16 ? FL_CONTRACT_BF16 : 0u;
   int rc = FL_ERR_UNSUPPORTED;
   switch (l.kind) {
     case Launch::Kind::MatMulChain: {
@@ -221,13 +222,13 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       kernel::TensorView c;
       if (l.has_c) c = ViewOf(Resolve(l.c), l.c);
       if (l.view_strides.empty()) {
-        rc = fluidml_hip_matmul_chain(&a.t, &b.t, l.has_c ? &c.t : nullptr, &out.t, &l.chain, ctx.stream);
+        rc = fluidml_hip_matmul_chain(&a.t, &b.t, l.has_c ? &c.t : nullptr, &out.t, &l.chain, contract_flags, ctx.stream);
       } else {
         // the contraction's logical output addressed inside the buffer of the last folded Reshape / Transpose
         kernel::TensorView dst(out.t.base, steps_[l.members[0]].out.meta);
         for (size_t d = 0; d < l.view_strides.size(); ++d) dst.t.strides[d] = l.view_strides[d];
         rc = fluidml_hip_matmul_chain_view(&a.t, &b.t, l.has_c ? &c.t : nullptr, &dst.t, l.n_inner, l.stride_outer,
-                                           &l.chain, ctx.stream);
+                                           &l.chain, contract_flags, ctx.stream);
       }
       break;
     }
@@ -252,7 +253,8 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
         outer[g] = m.stride_outer;
       }
       rc = fluidml_hip_matmul_chain_group(static_cast<int32_t>(n), &a.t, rhs_p.data(), bias_p.data(), dst_p.data(),
-                                          l.group[0].n_inner, outer.data(), &l.group[0].chain, ctx.stream);
+                                          l.group[0].n_inner, outer.data(), &l.group[0].chain, contract_flags,
+                                          ctx.stream);
       break;
     }
     case Launch::Kind::GemmChain: {
@@ -356,6 +358,7 @@ size_t LaunchPlan::Run(const std::unordered_map<std::string, void *> &args, size
   kernel::LaunchContext ctx;
   ctx.stream = stream_;
   ctx.flags = flags_;
+  ctx.bf16 = bf16_;
   if (use_graph_ && graph_ == nullptr) {  // record outside the timed region
     Replay(ctx);
     Check(fluidml_hip_stream_synchronize(stream_), "waiting for the first replay");
@@ -378,6 +381,7 @@ void LaunchPlan::ReplayResident(size_t n) {
   kernel::LaunchContext ctx;
   ctx.stream = stream_;
   ctx.flags = flags_;
+  ctx.bf16 = bf16_;
   for (size_t i = 0; i < n; ++i) Replay(ctx);
   Check(fluidml_hip_stream_synchronize(stream_), "waiting for the replays");
 }
@@ -387,6 +391,7 @@ double LaunchPlan::TimeReplayNs(size_t warmup, size_t iters) {
   kernel::LaunchContext ctx;
   ctx.stream = stream_;
   ctx.flags = flags_;
+  ctx.bf16 = bf16_;
   for (size_t i = 0; i < warmup + 1; ++i) Replay(ctx);
   void *e0 = nullptr, *e1 = nullptr;
   Check(fluidml_hip_event_create(&e0), "event");
@@ -406,6 +411,7 @@ std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
   kernel::LaunchContext ctx;
   ctx.stream = stream_;
   ctx.flags = flags_;
+  ctx.bf16 = bf16_;
   const std::vector<Launch> &schedule = GetSchedule();
   std::vector<std::vector<double>> samples(schedule.size());
   // one start/stop pair per launch, stamped by the dispatch itself (kernel-exact durations)

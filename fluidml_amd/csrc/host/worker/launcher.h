@@ -151,6 +151,8 @@ class LaunchPlan {
   void SetUseGraph(bool use) { use_graph_ = use; }
   // launch-level fusion of single-reader chains; off whenever literal-reference flags are set
   void SetFuse(bool fuse) { fuse_ = fuse; }
+  // MatMul nodes on the opt-in bf16 path (operands rounded to bf16, fp32 accumulation)
+  void SetBf16(bool on) { bf16_ = on; }
   // device address of a named interface / constant operand (tests)
   void *GetDeviceAddress(const std::string &name) const;
   void *GetArenaBase() const { return arena_; }
@@ -181,6 +183,7 @@ class LaunchPlan {
   uint32_t flags_ = 0;
   bool use_graph_ = true;
   bool fuse_ = true;
+  bool bf16_ = false;
   mutable std::vector<Launch> schedule_;
   mutable bool schedule_built_ = false;
   void *arena_ = nullptr;

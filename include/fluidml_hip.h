@@ -87,6 +87,13 @@ enum fl_ref_flags {
   FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
 };
 
+/* Options of the contraction entry points that take `flags`. */
+enum fl_contract_flags {
+  /* operands rounded to bf16 (nearest even), fp32 accumulation: the opt-in
+   * reduced-precision path; its error is reported separately by bench.py */
+  FL_CONTRACT_BF16 = 1 << 0
+};
+
 /* A short chain of elementwise operations on one float32 value, used by the
  * launch-level fusions below.  Step i replaces v (initially the chain's input
  * x) by op[i](v, c[i]) or op[i](v, x); every operation is the one the
@@ -295,8 +302,9 @@ int fluidml_hip_average_pool_without_padding(const fl_tensor *in, const fl_tenso
 /* MatMulKernel: NumPy batch-broadcast matmul, fp32 MFMA
  * (reference matmul.cpp:28-59, utils.cpp:64-147). */
 int fluidml_hip_matmul(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream);
-/* Same contraction with operands rounded to bf16 and fp32 accumulation
- * (opt-in; no counterpart in the reference, error is reported separately). */
+/* Same contraction with operands rounded to bf16 (nearest even) and fp32
+ * accumulation on v_mfma_f32_32x32x8_bf16 (opt-in; no counterpart in the
+ * reference, error is reported separately). */
 int fluidml_hip_matmul_bf16(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream);
 /* GemmConstantBiasKernel (kernel name "GemmConstantWeightsBiasKernel"):
  * rank-2, bias rank 1 or 2 (reference gemm.cpp:39-182). */
@@ -324,7 +332,7 @@ int fluidml_hip_matmul_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
 /* MatMulKernel [-> AddCommonKernel(rank-1 bias)] -> elementwise chain on the
  * result, e.g. the erf-GELU chain Div, Erf, Add, Mul(x), Mul of
  * add_div_erf_add_mul_mul.cpp:29-132.  `bias` and `chain` may be NULL. */
-int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, const fl_ew_program *chain, void *stream);
+int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, const fl_ew_program *chain, uint32_t flags, void *stream);
 /* The same, followed by Reshape / Transpose steps that only re-address the
  * result (reference reshape.cpp:18-64, transpose.cpp:19-48): `out` carries the
  * contraction's logical shape [..., M, N] with the element strides each of
@@ -332,12 +340,12 @@ int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const f
  * (N / n_inner, n_inner) and the transpose moved the two apart, column n is
  * stored at (n / n_inner) * stride_outer + (n % n_inner) * out->strides[last];
  * n_inner == 0 means plain strides. */
-int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, int64_t n_inner, int64_t stride_outer, const fl_ew_program *chain, void *stream);
+int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, int64_t n_inner, int64_t stride_outer, const fl_ew_program *chain, uint32_t flags, void *stream);
 /* `count` (1..4) such launches that share `lhs`, every extent, the strides of
  * `rhs`, `n_inner` and `chain`, as ONE launch (the query / key / value
  * projections of an attention block): rhs[i], bias[i] (all NULL or none),
  * out[i] and stride_outer[i] belong to member i.  No batch dims. */
-int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs, const fl_tensor *const *bias, const fl_tensor *const *out, int64_t n_inner, const int64_t *stride_outer, const fl_ew_program *chain, void *stream);
+int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs, const fl_tensor *const *bias, const fl_tensor *const *out, int64_t n_inner, const int64_t *stride_outer, const fl_ew_program *chain, uint32_t flags, void *stream);
 /* GemmConstantWeightsBiasKernel -> elementwise chain (reference gemm.cpp:39-182). */
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double alpha, double beta, int32_t trans_a, int32_t trans_b, const fl_ew_program *chain, void *stream);
 /* Conv{With,Without}PaddingKernel -> elementwise chain (reference conv.cpp:27-280);

@@ -98,6 +98,26 @@ def test_dp_measured_layouts_match_oracle(device, tiny_bert, monkeypatch, tmp_pa
         assert_close(got[name], ref, what=f"dp replay {name}")
 
 
+def test_bf16_opt_in(device, tiny_bert, monkeypatch):
+    """FLUIDML_BF16=1 moves every MatMul to the bf16 path; the result stays close to the fp32 oracle but is not
+    held to the fp32 tolerance (its error is reported separately by bench.py --bf16)."""
+    fluidml, _ = _mods()
+    net, path, feeds, want = tiny_bert
+    monkeypatch.setenv("FLUIDML_BF16", "1")
+    announce("tiny bert bf16")
+    ex = fluidml.Executor.make_plain_greedy("tiny_bf16")
+    ex.compile(path)
+    got = _invoke(ex, net, feeds)
+    monkeypatch.setenv("FLUIDML_BF16", "0")
+    ex32 = fluidml.Executor.make_plain_greedy("tiny_fp32")
+    ex32.compile(path)
+    got32 = _invoke(ex32, net, feeds)
+    for name, ref in want.items():
+        err = np.abs(got[name] - ref).max()
+        assert 0 < err < 0.1, f"bf16 path: max abs err {err}"
+        assert np.abs(got32[name] - ref).max() < err  # and the default path is the more exact one
+
+
 def test_invoke_errors(device, tiny_bert):
     fluidml, _ = _mods()
     net, path, feeds, _ = tiny_bert

@@ -543,6 +543,37 @@ def test_matmul_split_k(device):
             assert (r == runs[0]).all(), "split-K sum depends on the run"
 
 
+def _round_bf16(x):
+    """float32 -> nearest-even bf16 -> float32"""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32).reshape(x.shape)
+
+
+def test_matmul_bf16(device):
+    """Opt-in path: both operands rounded to bf16, products and sums in fp32.  Checked to the fp32 tolerance
+    against the oracle run on the rounded operands; the distance to the unrounded fp32 result is printed."""
+    cabi = _cabi()
+    rng = np.random.default_rng(81)
+    for ashape, bshape in [((1, 128, 768), (768, 768)), ((2, 3, 70, 40), (40, 50)), ((1024, 96), (96, 1024)),
+                           ((2048, 64), (64, 2048))]:
+        a, b = rand(rng, ashape, -1, 1), rand(rng, bshape, -0.05, 0.05)
+        oshape = np.matmul(np.empty(ashape, np.int8), np.empty(bshape, np.int8)).shape
+        want = ok.View.empty(oshape)
+        ok.matmul(ok.View(_round_bf16(a)), ok.View(_round_bf16(b)), want)
+        exact = ok.View.empty(oshape)
+        ok.matmul(ok.View(a), ok.View(b), exact)
+        for la in (None, list(range(len(ashape)))[::-1]):
+            announce("matmul bf16", ashape, bshape, la)
+            da, db = DeviceView(ok.View(a, la), device), DeviceView(ok.View(b), device)
+            do = DeviceView(ok.View.empty(oshape, fill=4), device)
+            cabi.call("matmul_bf16", da.ref(), db.ref(), do.ref(), None)
+            assert_close(do.logical(), want.logical(), what="matmul_bf16 vs oracle on bf16-rounded operands")
+        err = np.abs(do.logical() - exact.logical())
+        print(f"[bf16] {ashape}x{bshape}: max abs err vs fp32 {err.max():.3e}, relative to max |c| {err.max() / np.abs(exact.logical()).max():.3e}")
+        assert err.max() / np.abs(exact.logical()).max() < 2e-2
+
+
 def test_matmul_unaligned(device):
     cabi = _cabi()
     rng = np.random.default_rng(78)
@@ -612,14 +643,14 @@ def test_fused_matmul_add_and_gelu(device):
             do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
             gelu = cabi.make_chain([(cabi.EW_DIV_C, 1.4142135381698608), (cabi.EW_ERF, 0), (cabi.EW_ADD_C, 1.0),
                                     (cabi.EW_MUL_X, 0), (cabi.EW_MUL_C, 0.5)])
-            cabi.call("matmul_chain", da.ref(), db.ref(), dbias.ref(), do.ref(), ctypes.byref(gelu), None)
+            cabi.call("matmul_chain", da.ref(), db.ref(), dbias.ref(), do.ref(), ctypes.byref(gelu), ctypes.c_uint32(0), None)
             assert_close(do.logical(), u4.logical(), what="matmul_chain bias + erf-GELU")
             # no bias, chain only: relu(a.b) * 0.5
             ok.unary_f32(ok.OP_RELU, t0, u0)
             ok.unary_f32(ok.OP_MUL_C, u0, u1, 0.5)
             do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
             chain = cabi.make_chain([(cabi.EW_RELU, 0), (cabi.EW_MUL_C, 0.5)])
-            cabi.call("matmul_chain", da.ref(), db.ref(), None, do.ref(), ctypes.byref(chain), None)
+            cabi.call("matmul_chain", da.ref(), db.ref(), None, do.ref(), ctypes.byref(chain), ctypes.c_uint32(0), None)
             assert_close(do.logical(), u1.logical(), what="matmul_chain relu, scale")
 
 
@@ -648,7 +679,7 @@ def test_matmul_chain_view(device):
         view = cabi.make_tensor(dfinal.tensor.base, cabi.FL_FLOAT32, [1, S, H], [fs[pos[0]], fs[pos[1]], fs[pos[3]]])
         da, db, dbias = DeviceView(ok.View(a), device), DeviceView(ok.View(b), device), DeviceView(ok.View(bias), device)
         cabi.call("matmul_chain_view", da.ref(), db.ref(), dbias.ref(), ctypes.byref(view), ctypes.c_int64(d),
-                  ctypes.c_int64(fs[pos[2]]), None, None)
+                  ctypes.c_int64(fs[pos[2]]), None, ctypes.c_uint32(0), None)
         assert_close(dfinal.logical(), want.logical(), what="matmul_chain_view")
 
 

@@ -20,6 +20,7 @@
 #include "utils/utils.h"
 #include "worker/builder.h"
 #include "worker/converter.h"
+#include "optimization/graph_passes.h"
 #include "worker/executor.h"
 #include "worker/launcher.h"
 #include "worker/lower.h"
@@ -120,6 +121,7 @@ PYBIND11_MODULE(fluidml, m) {
       .def("set_ref_flags", [](context::Context &c, uint32_t flags) { c->ref_flags = flags; }, py::arg("flags"))
       .def("set_use_graph", [](context::Context &c, bool use) { c->use_graph = use; }, py::arg("use"))
       .def("set_fuse", [](context::Context &c, bool fuse) { c->fuse = fuse; }, py::arg("fuse"))
+      .def("set_graph_passes", [](context::Context &c, bool on) { c->graph_passes = on; }, py::arg("on"))
       .def("set_bf16", [](context::Context &c, bool on) { c->bf16 = on; }, py::arg("on"))
       .def("plan_text", [](context::Context &c) { return c->GetModule().ToText(); });
 
@@ -161,7 +163,29 @@ PYBIND11_MODULE(fluidml, m) {
         return out;
       });
 
-  py::class_<graph::Graph, std::unique_ptr<graph::Graph>>(m, "Graph");
+  py::class_<graph::Graph, std::unique_ptr<graph::Graph>>(m, "Graph")
+      .def("nodes",
+           [](const graph::Graph &g) {
+             py::list out;
+             for (const std::shared_ptr<graph::Node> &n : g.GetAllNodes()) {
+               py::dict d;
+               d["name"] = n->GetName();
+               d["op"] = graph::OpToString(n->GetOp());
+               std::vector<std::string> ins, outs;
+               for (const auto &e : g.GetNodeFrom(n->GetName())) ins.push_back(e->GetName());
+               for (const auto &e : g.GetNodeTo(n->GetName())) outs.push_back(e->GetName());
+               d["inputs"] = ins;
+               d["outputs"] = outs;
+               out.append(d);
+             }
+             return out;
+           },
+           "nodes in container order: name, op, input and output value names");
+
+  py::class_<optimization::GraphPassesManager>(m, "GraphPassesManager")
+      .def(py::init<>())
+      .def("register_all_passes", &optimization::GraphPassesManager::RegisterAllPasses)
+      .def("run", &optimization::GraphPassesManager::Run, py::arg("graph"));
 
   py::class_<memory::Index, std::unique_ptr<memory::Index>>(m, "Index")
       .def("get", &memory::Index::Get, py::arg("name"))

@@ -19,6 +19,7 @@ ContextImpl::ContextImpl() {
   if (const char *g = std::getenv("FLUIDML_HIP_GRAPH")) use_graph = std::string(g) != "0";
   if (const char *f = std::getenv("FLUIDML_FUSE")) fuse = std::string(f) != "0";
   if (const char *h = std::getenv("FLUIDML_BF16")) bf16 = std::string(h) != "0";
+  if (const char *gp = std::getenv("FLUIDML_GRAPH_PASSES")) graph_passes = std::string(gp) != "0";
   if (const char *c = std::getenv("FLUIDML_DP_COST")) {
     const std::string mode(c);
     if (mode == "constant") {

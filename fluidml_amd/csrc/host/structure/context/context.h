@@ -82,6 +82,9 @@ class ContextImpl {
   bool use_graph = true;
   // launch-level fusion of single-reader kernel chains (env FLUIDML_FUSE=0 disables)
   bool fuse = true;
+  // run the graph-level fusion passes between parsing and conversion (env FLUIDML_GRAPH_PASSES=1);
+  // the reference ships them unwired, so the default is off
+  bool graph_passes = false;
   // MatMul nodes on the opt-in bf16 path (env FLUIDML_BF16=1)
   bool bf16 = false;
   // cost source of the layout DP (env FLUIDML_DP_COST=measure|constant|<path to table json>)

@@ -1,5 +1,7 @@
 #include "structure/graph/graph.h"
 
+#include <algorithm>
+
 #include <stdexcept>
 #include <utility>
 
@@ -146,6 +148,28 @@ bool Graph::NodeToEdge(const std::string &node_name, const std::string &edge_nam
   nodes_[node_name].to.push_back(edge_name);
   edges_[edge_name].from = node_name;
   return true;
+}
+
+namespace {
+void Scrub(std::vector<std::string> *names, const std::string &name) {
+  names->erase(std::remove(names->begin(), names->end(), name), names->end());
+}
+}  // namespace
+
+void Graph::DeleteNode(const std::string &name) {
+  if (nodes_.erase(name) == 0) return;
+  for (auto &kv : edges_) {
+    if (kv.second.from && *kv.second.from == name) kv.second.from.reset();
+    Scrub(&kv.second.to, name);
+  }
+}
+
+void Graph::DeleteEdge(const std::string &name) {
+  if (edges_.erase(name) == 0) return;
+  for (auto &kv : nodes_) {
+    Scrub(&kv.second.from, name);
+    Scrub(&kv.second.to, name);
+  }
 }
 
 }  // namespace graph

@@ -126,6 +126,10 @@ class Graph {
   // Links are silently refused when either end is unknown (graph.cpp:343-351, 357-365).
   bool EdgeToNode(const std::string &edge_name, const std::string &node_name);
   bool NodeToEdge(const std::string &node_name, const std::string &edge_name);
+  // Remove a node / a value together with every link that mentions it (what the reference's
+  // Node::Delete / Edge::Delete do for the fusion passes, node.cpp and edge.cpp of structure/graph).
+  void DeleteNode(const std::string &name);
+  void DeleteEdge(const std::string &name);
 
  private:
   struct EdgeContainer {

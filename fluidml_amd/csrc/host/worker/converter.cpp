@@ -380,9 +380,43 @@ void ConvertNode(flow::Flow &flow, const graph::Graph &graph, const graph::Node 
       c.PutDouble(padded ? OpKind::ConvWithPadding : OpKind::ConvWithoutPadding, c.in[0], c.in[1], std::move(a));
       break;
     }
+    // the fused forms only arise from the graph passes; inputs = the chain's constants, then its variable
+    case Op::AddDivErfAddMulMul: {  // add0 CT, div CS, add1 CS, mul1 CS, x (converter.cpp:455-520)
+      c.Need(5);
+      if (!c.in[0]->IsConstantTensor() || !c.in[1]->IsConstantScalar() || !c.in[2]->IsConstantScalar() ||
+          !c.in[3]->IsConstantScalar() || !c.in[4]->IsNonConstant()) Unsupported(node, "operand pattern");
+      Attrs a;
+      a.t0 = c.in[0]->GetTensor();
+      a.alpha = c.in[1]->GetScalar();
+      a.beta = c.in[2]->GetScalar();
+      a.extra = c.in[3]->GetScalar();
+      c.PutSingle(OpKind::AddDivErfAddMulMul, c.in[4], std::move(a));
+      break;
+    }
+    case Op::GatherAddAdd: {  // table CT, add0 CT, add1 CT, indices (converter.cpp:1293-1356)
+      c.Need(4);
+      if (!c.in[0]->IsConstantTensor() || !c.in[1]->IsConstantTensor() || !c.in[2]->IsConstantTensor() ||
+          !c.in[3]->IsNonConstant()) Unsupported(node, "operand pattern");
+      Attrs a;
+      a.t0 = c.in[0]->GetTensor();
+      a.t1 = c.in[1]->GetTensor();
+      a.t2 = c.in[2]->GetTensor();
+      c.PutSingle(OpKind::GatherConstantDataTensorAddTensorLhsAddTensorLhs, c.in[3], std::move(a));
+      break;
+    }
+    case Op::UnsqueezeSubMul: {  // axes CT, sub CS, mul CS, x (converter.cpp:2496-2557)
+      c.Need(4);
+      if (!c.in[0]->IsConstantTensor() || !c.in[1]->IsConstantScalar() || !c.in[2]->IsConstantScalar() ||
+          !c.in[3]->IsNonConstant()) Unsupported(node, "operand pattern");
+      Attrs a;
+      a.axes = TensorAsInt64(c.in[0]->GetTensor());
+      a.alpha = c.in[1]->GetScalar();
+      a.beta = c.in[2]->GetScalar();
+      c.PutSingle(OpKind::UnsqueezeSubLhsScalarMulRhsScalar, c.in[3], std::move(a));
+      break;
+    }
     default:
-      // ConstantOfShape is parsed but has no conversion (converter.cpp:268-274);
-      // the fused forms only arise from graph passes
+      // ConstantOfShape is parsed but has no conversion (converter.cpp:268-274)
       Unsupported(node, "no flow node for this operator");
   }
 }

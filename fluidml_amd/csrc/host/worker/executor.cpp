@@ -1,5 +1,7 @@
 #include "worker/executor.h"
 
+#include "optimization/graph_passes.h"
+
 #include <stdexcept>
 
 #include "worker/builder.h"
@@ -28,6 +30,11 @@ class ExecutorImpl : public Executor {
                                                                             : context_.MakePlainGeneralBuilder(std::move(fn));
     std::unique_ptr<Lower> lower = context_.MakeLower();
     graph::Graph graph = parser->Run(input);
+    if (context_->graph_passes) {
+      optimization::GraphPassesManager passes;
+      passes.RegisterAllPasses();
+      passes.Run(graph);
+    }
     flow::Flow flow = converter->Run(graph);
     std::unique_ptr<Planner> planner;
     switch (flavour_) {

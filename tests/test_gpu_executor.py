@@ -98,6 +98,25 @@ def test_dp_measured_layouts_match_oracle(device, tiny_bert, monkeypatch, tmp_pa
         assert_close(got[name], ref, what=f"dp replay {name}")
 
 
+@pytest.mark.parametrize("fuse", [True, False], ids=["fused", "unfused"])
+def test_graph_passes_match_oracle(device, tiny_bert, fuse, monkeypatch):
+    """With FLUIDML_GRAPH_PASSES=1 the GELU chain and the mask preparation run as the reference's fused nodes
+    (AddDivErfAddMulMul, UnsqueezeSubLhsScalarMulRhsScalar); the oracle runs the original, unfused graph."""
+    fluidml, _ = _mods()
+    net, path, feeds, want = tiny_bert
+    monkeypatch.setenv("FLUIDML_GRAPH_PASSES", "1")
+    monkeypatch.setenv("FLUIDML_FUSE", "1" if fuse else "0")
+    announce("tiny bert graph passes", fuse)
+    ex = fluidml.Executor.make_plain_greedy("tiny_passes")
+    ex.compile(path)
+    kernels = [s["kernel"] for s in ex.plan()["steps"]]
+    assert kernels.count("AddDivErfAddMulMulKernel") == 2 and kernels.count("UnsqueezeSubLhsScalarMulRhsScalarKernel") == 1
+    assert len(kernels) < len(net.nodes)
+    got = _invoke(ex, net, feeds)
+    for name, ref in want.items():
+        assert_close(got[name], ref, what=f"graph passes {name}")
+
+
 def test_bf16_opt_in(device, tiny_bert, monkeypatch):
     """FLUIDML_BF16=1 moves every MatMul to the bf16 path; the result stays close to the fp32 oracle but is not
     held to the fp32 tolerance (its error is reported separately by bench.py --bf16)."""

@@ -282,6 +282,58 @@ def test_golden_config_plans(mods, tmp_path, config):
     assert got["sample"] == {k: list(v) for k, v in golden["sample"].items()}
 
 
+# ------------------------------------------------------------------ graph-level fusion passes
+
+def test_graph_fusion_passes(mods, tmp_path, monkeypatch):
+    """The three graph passes (reference src/optimization/graph/*.cpp): each pattern collapses into one fused
+    node whose inputs are the chain's constants followed by its variable input; everything else is untouched."""
+    fluidml, models, _ = mods
+    import numpy as np
+
+    g = models.Net("passes", 11)
+    ids = g.input("ids", np.int64, (1, 8))
+    mask = g.input("mask", np.float32, (1, 8))
+    emb = g.gather(g.normal((50, 16)), ids)                       # Gather(table) -> Add(CT) -> Add(CT)
+    emb = g.add(emb, g.normal((1, 8, 16)))
+    emb = g.add(emb, g.normal((16,)))
+    ext = g.mul(g.sub(g.scalar(1.0), g.unsqueeze(mask, [1, 2])), g.scalar(-10000.0))   # Unsqueeze -> Sub -> Mul
+    h = g.erf_gelu(g.linear(emb, g.normal((16, 32)), g.zeros((32,))))                   # Add(bias) -> GELU chain
+    s = g.add(g.matmul(h, g.normal((32, 8))), g.reshape(ext, (1, 1, 8)))
+    g.output(s)
+    path = g.save(str(tmp_path / "passes.onnx"))
+    graph = fluidml.Parser.make().run(path)
+    before = {n["name"]: n for n in graph.nodes()}
+    manager = fluidml.GraphPassesManager()
+    manager.register_all_passes()
+    manager.run(graph)
+    after = {n["name"]: n for n in graph.nodes()}
+    ops = sorted(n["op"] for n in after.values())
+    assert ops == sorted(["AddDivErfAddMulMul", "GatherAddAdd", "UnsqueezeSubMul", "MatMul", "MatMul", "Add", "Reshape"])
+    assert len(before) == 3 + 3 + 1 + 6 + 1 + 1 + 1
+    gelu = next(n for n in after.values() if n["op"] == "AddDivErfAddMulMul")
+    assert len(gelu["inputs"]) == 5 and len(gelu["name"].split("-")) == 6
+    assert gelu["inputs"][4] == next(n for n in before.values() if n["op"] == "MatMul" and n["outputs"][0] == gelu["inputs"][4])["outputs"][0]
+    gather = next(n for n in after.values() if n["op"] == "GatherAddAdd")
+    assert gather["inputs"][3] == "ids" and len(gather["inputs"]) == 4
+    um = next(n for n in after.values() if n["op"] == "UnsqueezeSubMul")
+    assert um["inputs"][3] == "mask" and len(um["inputs"]) == 4
+    # the fused graph converts and plans; fewer kernels than without the passes
+    flow = fluidml.Converter.make().run(graph)
+    seq, _, _ = fluidml.Context().make_plain_greedy_planner().run(flow)
+    kernels = sorted(seq.kernel_names())
+    assert "AddDivErfAddMulMulKernel" in kernels and "UnsqueezeSubLhsScalarMulRhsScalarKernel" in kernels
+    assert "GatherConstantDataTensorAddTensorLhsAddTensorLhsKernel" in kernels
+    assert len(kernels) == 7
+    # through the Executor: off by default (the reference never calls the passes), on with the switch
+    ex = fluidml.Executor.make_plain_greedy("no_passes")
+    ex.compile(path)
+    assert len(ex.plan()["steps"]) == len(before)
+    monkeypatch.setenv("FLUIDML_GRAPH_PASSES", "1")
+    ex = fluidml.Executor.make_plain_greedy("with_passes")
+    ex.compile(path)
+    assert len(ex.plan()["steps"]) == 7
+
+
 # ------------------------------------------------------------------ launch schedule (fusion)
 
 def _overlap(x, y):

@@ -149,8 +149,10 @@ struct TileLoader {
 
 // LA: 0 = A tile kept [m][k] (A is k-contiguous), 1 = kept [k][m].
 // LB: 0 = B tile kept [k][n] (B is n-contiguous), 1 = kept [n][k].
-// CONV: B is the input of a convolution addressed through p.conv (LB must be 0, scalar gathers).
-template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV = false,
+// CONV: 0 = plain contraction; 1 = B is the input of a convolution addressed through p.conv (LB must be 0), one
+// scalar gather per element; 2 = the same with one 128-bit gather per four consecutive output pixels of a row
+// (unit stride along W in the input and in the convolution, OW a multiple of 4).
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV = 0,
           bool BF16 = false>
 __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, float *__restrict__ C_,
                                                                 const float *__restrict__ A,
@@ -170,8 +172,8 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   constexpr int LDS_ELEMS = STAGE_ELEMS > RED_ELEMS ? STAGE_ELEMS : RED_ELEMS;
   __shared__ __attribute__((aligned(16))) float lds[LDS_ELEMS];
 
-  constexpr int VB = CONV ? 1 : VEC;
-  static_assert(!CONV || (LB == 0 && NT % BN == 0), "the gather keeps one output pixel per thread");
+  constexpr int VB = CONV == 2 ? 4 : CONV == 1 ? 1 : VEC;
+  static_assert(!CONV || (LB == 0 && NT % (BN / VB) == 0), "the gather keeps one output pixel (group) per thread");
   using LoaderA = typename std::conditional<LA == 0, TileLoader<BM, BK, VEC, NT>, TileLoader<BK, BM, VEC, NT>>::type;
   using LoaderB = typename std::conditional<LB == 0, TileLoader<BK, BN, VB, NT>, TileLoader<BN, BK, VB, NT>>::type;
 
@@ -243,7 +245,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   bool g_valid = false;
   int32_t g_ih0 = 0, g_iw0 = 0, g_base = 0;
   if constexpr (CONV) {
-    const int n = n0 + static_cast<int>(threadIdx.x % BN);
+    const int n = n0 + static_cast<int>(threadIdx.x % (BN / VB)) * VB;
     g_valid = n < p.N;
     uint32_t img, r, oh, ow;
     p.conv.div_ohw.DivMod(static_cast<uint32_t>(g_valid ? n : 0), img, r);
@@ -261,23 +263,40 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
       LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAk, p.sAm, k_valid, rows_m, qa);
     }
     if constexpr (CONV) {
-      // same item -> (k row, n column) mapping as TileLoader<BK, BN, 1, NT>: column = thread % BN
+      // same item -> (k row, n column) mapping as TileLoader<BK, BN, VB, NT>: column group = thread % (BN / VB)
 #pragma unroll
       for (int j = 0; j < LoaderB::kPerThread; ++j) {
-        const int k = k0 + static_cast<int>(threadIdx.x / BN) + j * (NT / BN);
-        float v = 0.0f;
+        const int k = k0 + static_cast<int>(threadIdx.x / (BN / VB)) + j * (NT / (BN / VB));
+#pragma unroll
+        for (int e = 0; e < VB; ++e) qb[j].v[e] = 0.0f;
         if (g_valid && k < p.K) {
           uint32_t ci, r, kh, kw;
           p.conv.div_khw.DivMod(static_cast<uint32_t>(k), ci, r);
           p.conv.div_kw.DivMod(r, kh, kw);
           const int32_t ih = g_ih0 + static_cast<int32_t>(kh) * p.conv.dh;
           const int32_t iw = g_iw0 + static_cast<int32_t>(kw) * p.conv.dw;
-          if (static_cast<uint32_t>(ih) < static_cast<uint32_t>(p.conv.H) &&
-              static_cast<uint32_t>(iw) < static_cast<uint32_t>(p.conv.W)) {
-            v = B[g_base + static_cast<int32_t>(ci) * p.conv.sXc + ih * p.conv.sXh + iw * p.conv.sXw];
+          if (static_cast<uint32_t>(ih) < static_cast<uint32_t>(p.conv.H)) {
+            if constexpr (CONV == 2) {
+              // four output pixels of one row read four consecutive input elements (4-byte aligned only)
+              const float *row = B + g_base + static_cast<int32_t>(ci) * p.conv.sXc + ih * p.conv.sXh;
+              if (iw >= 0 && iw + 3 < p.conv.W) {
+                struct __attribute__((packed, aligned(4))) Quad {
+                  float v[4];
+                };
+                const Quad q = *reinterpret_cast<const Quad *>(row + iw);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) qb[j].v[e] = q.v[e];
+              } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  if (static_cast<uint32_t>(iw + e) < static_cast<uint32_t>(p.conv.W)) qb[j].v[e] = row[iw + e];
+                }
+              }
+            } else if (static_cast<uint32_t>(iw) < static_cast<uint32_t>(p.conv.W)) {
+              qb[j].v[0] = B[g_base + static_cast<int32_t>(ci) * p.conv.sXc + ih * p.conv.sXh + iw * p.conv.sXw];
+            }
           }
         }
-        qb[j].v[0] = v;
       }
     } else if constexpr (LB == 0) {
       LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBk, p.sBn, k_valid, cols_n, qb);
@@ -578,7 +597,7 @@ inline int64_t SplitKLimit() {
   return limit;
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, bool CONV, bool BF16>
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV, bool BF16>
 void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   MatmulArgs q = p;
   q.tiles_m = (p.M + BM - 1) / BM;
@@ -614,7 +633,7 @@ inline double TileEfficiency(int64_t m, int64_t n, int64_t bm, int64_t bn) {
          (static_cast<double>((m + bm - 1) / bm * bm) * static_cast<double>((n + bn - 1) / bn * bn));
 }
 
-template <int LA, int LB, int VEC, bool CONV, bool BF16 = false>
+template <int LA, int LB, int VEC, int CONV, bool BF16 = false>
 void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   const int64_t tiles_l = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * n_batch;
   const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
@@ -776,12 +795,12 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
 #define FL_MM_DISPATCH(LA_, LB_)                              \
   if (la == LA_ && lb == LB_) {                               \
     if (bf16) {                                                   \
-      if (vec) LaunchBySize<LA_, LB_, 4, false, true>(p, nb, C, A, B, s); \
-      else LaunchBySize<LA_, LB_, 1, false, true>(p, nb, C, A, B, s);     \
+      if (vec) LaunchBySize<LA_, LB_, 4, 0, true>(p, nb, C, A, B, s); \
+      else LaunchBySize<LA_, LB_, 1, 0, true>(p, nb, C, A, B, s);     \
     } else if (vec) {                                             \
-      LaunchBySize<LA_, LB_, 4, false>(p, nb, C, A, B, s);        \
+      LaunchBySize<LA_, LB_, 4, 0>(p, nb, C, A, B, s);        \
     } else {                                                      \
-      LaunchBySize<LA_, LB_, 1, false>(p, nb, C, A, B, s);        \
+      LaunchBySize<LA_, LB_, 1, 0>(p, nb, C, A, B, s);        \
     }                                                             \
   }
   FL_MM_DISPATCH(0, 0)
@@ -862,13 +881,21 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
   bool vec = IsAligned(A, 16);
   if (la == 0) vec = vec && (p.sAk == 1 || p.K == 1) && p.K % 4 == 0 && p.sAm % 4 == 0;
   else vec = vec && p.sAm == 1 && p.M % 4 == 0 && p.sAk % 4 == 0;
+  // four output pixels per gather when they sit in one input row at unit stride
+  const bool quad = g.sw == 1 && g.sXw == 1 && OW % 4 == 0;
+#define FL_CONV_DISPATCH(LA_, VEC_)                                         \
+  do {                                                                      \
+    if (quad) LaunchBySize<LA_, 0, VEC_, 2>(p, 1, C, A, B, s);              \
+    else LaunchBySize<LA_, 0, VEC_, 1>(p, 1, C, A, B, s);                   \
+  } while (0)
   if (la == 0) {
-    if (vec) LaunchBySize<0, 0, 4, true>(p, 1, C, A, B, s);
-    else LaunchBySize<0, 0, 1, true>(p, 1, C, A, B, s);
+    if (vec) FL_CONV_DISPATCH(0, 4);
+    else FL_CONV_DISPATCH(0, 1);
   } else {
-    if (vec) LaunchBySize<1, 0, 4, true>(p, 1, C, A, B, s);
-    else LaunchBySize<1, 0, 1, true>(p, 1, C, A, B, s);
+    if (vec) FL_CONV_DISPATCH(1, 4);
+    else FL_CONV_DISPATCH(1, 1);
   }
+#undef FL_CONV_DISPATCH
   return LaunchStatus();
 }
 

@@ -62,13 +62,13 @@ KernelTimer &ThreadKernelTimer();  // runtime.hip
   } while (0)
 
 // Per-stream device memory for kernels that combine partial results across workgroups (split-K
-// contractions): 1024 partial 32x32 tiles and as many arrival counters (zero between launches).
+// contractions): 4096 partial 32x32 tiles (16 MiB) and as many arrival counters (zero between launches).
 // Launches on one stream run in order, so they can share it; two streams never share.
 struct StreamWorkspace {
   float *partials = nullptr;
   uint32_t *counters = nullptr;
 };
-constexpr size_t kWorkspaceTiles = 1024;
+constexpr size_t kWorkspaceTiles = 4096;
 constexpr size_t kWorkspaceTileFloats = 1024;
 // The stream's workspace, created on first use.  nullptr when it does not exist yet and cannot be created
 // now (the stream is being captured into a graph) or the allocation fails; callers then do without.

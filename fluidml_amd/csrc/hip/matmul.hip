@@ -425,14 +425,15 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   }
 
   // ---- combine the K splits of a tile across workgroups ------------------------
-  // Only the single-wave-per-tile configuration splits (host side), so no workgroup barrier is involved:
-  // the wave publishes its partial tile, then one atomic tells it whether it arrived last; the last wave
-  // adds all partials in split order, which makes the sum independent of arrival order.
-  if constexpr (WM * WN == 1 && KS > 1) {
+  // Only configurations in which a wave ends up with exactly one 32x32 accumulator split (host side), and each
+  // wave runs the protocol on its own slot, so no workgroup barrier is involved: the wave publishes its partial
+  // tile, then one atomic tells it whether it arrived last; the last wave adds all partials in split order,
+  // which makes the sum independent of arrival order.
+  if constexpr (TM * TN == 1 && (WM * WN == 1 || KS == 1)) {
     if (gridDim.z > 1) {
       const uint32_t n_splits = gridDim.z;
-      const uint32_t tile_id = blockIdx.y * gridDim.x + blockIdx.x;
-      float *mine = p.partials + (static_cast<size_t>(tile_id) * n_splits + blockIdx.z) * (BM * BN);
+      const uint32_t tile_id = (blockIdx.y * gridDim.x + blockIdx.x) * (WM * WN) + wm * WN + wn;
+      float *mine = p.partials + (static_cast<size_t>(tile_id) * n_splits + blockIdx.z) * 1024;
       // The partial tiles travel through device-coherent accesses (agent-scope atomics: they bypass the
       // per-XCD L2 instead of living in it), so no cache-wide write-back or invalidate is needed: waiting
       // for this wave's stores to be acknowledged before it counts its arrival is enough, and the last
@@ -448,13 +449,13 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
       if (arrived != n_splits - 1) return;
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // keeps the loads below behind the counter read
       if (lane == 0) __hip_atomic_store(&p.counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const float *all = p.partials + static_cast<size_t>(tile_id) * n_splits * (BM * BN);
+      const float *all = p.partials + static_cast<size_t>(tile_id) * n_splits * 1024;
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[0][0][e] = 0.0f;
       for (uint32_t z = 0; z < n_splits; ++z) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          acc[0][0][e] += __hip_atomic_load(all + z * (BM * BN) + e * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          acc[0][0][e] += __hip_atomic_load(all + z * 1024 + e * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
     }
@@ -587,14 +588,15 @@ inline bool TrySkinnyGemm(const MatmulArgs &p, int64_t n_batch, float *C, const 
   return true;
 }
 
-// Upper bound on the number of K splits per tile (environment FLUIDML_SPLITK, default 4; 1 = never split).
-inline int64_t SplitKLimit() {
+// Upper bound on the number of K splits per tile (environment FLUIDML_SPLITK; default 4 for the 32x32 tile and
+// 8 for the 64x64 tile; 1 = never split).
+inline int64_t SplitKLimit(int64_t fallback) {
   static const int64_t limit = [] {
     const char *v = std::getenv("FLUIDML_SPLITK");
-    const long n = v != nullptr ? std::strtol(v, nullptr, 10) : 4;
-    return static_cast<int64_t>(n < 1 ? 1 : n);
+    const long n = v != nullptr ? std::strtol(v, nullptr, 10) : 0;
+    return static_cast<int64_t>(n < 0 ? 0 : n);
   }();
-  return limit;
+  return limit > 0 ? limit : fallback;
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV, bool BF16>
@@ -603,16 +605,17 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
   q.tiles_m = (p.M + BM - 1) / BM;
   q.tiles_n = (p.N + BN - 1) / BN;
   uint32_t splits = 1;
-  if constexpr (WM * WN == 1 && KS > 1) {
-    static_assert(BM * BN == kWorkspaceTileFloats, "a partial tile fills one workspace slot");
+  constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);
+  if constexpr (TM * TN == 1 && (WM * WN == 1 || KS == 1)) {
     // Few tiles and a long K: give each tile to several workgroups.  Measured on MI355X (M = 128..256): with
-    // about 100 tiles, 2 splits of 3 chunks (K = 768) and 4 splits of 4..6 chunks (K = 2048, 3072) win by
-    // 8 % to 40 %; from about 400 tiles on, or with fewer than 3 chunks per split, the exchange of the
-    // partial tiles costs more than the extra workgroups bring.
+    // about 100 tiles, 2 splits of 3 chunks of 128 (K = 768) and 4 splits of 4..6 chunks (K = 2048, 3072) win
+    // by 8 % to 40 %; from about 400 tiles on, or with shorter runs of K per split, the exchange of the
+    // partial tiles costs more than the extra workgroups bring.  One workspace slot per wave and split.
     const int64_t tiles = static_cast<int64_t>(q.tiles_m) * q.tiles_n * n_batch;
     const int64_t n_chunks = (p.K + BK - 1) / BK;
-    int64_t want = std::min<int64_t>(n_chunks / 3, static_cast<int64_t>(kWorkspaceTiles) / tiles);
-    want = std::min<int64_t>(want, SplitKLimit());
+    const int64_t min_chunks = 384 / BK;  // at least 384 values of k per split
+    int64_t want = std::min<int64_t>(n_chunks / min_chunks, static_cast<int64_t>(kWorkspaceTiles) / (tiles * WM * WN));
+    want = std::min<int64_t>(want, SplitKLimit(WM * WN == 1 ? 4 : 8));
     if (tiles > 256) want = 1;
     if (want >= 2) {
       if (StreamWorkspace *ws = GetStreamWorkspace(s)) {
@@ -638,10 +641,13 @@ void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
   const int64_t tiles_l = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * n_batch;
   const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
   // the big tile only when it fills the chip and does not waste much more of itself on edges than the next one
-  const bool big_ok = tiles_l >= 192 && TileEfficiency(p.M, p.N, 128, 128) + 0.15 >= TileEfficiency(p.M, p.N, 64, 64);
+  const bool big_ok = !CONV && tiles_l >= 192 && TileEfficiency(p.M, p.N, 128, 128) + 0.15 >= TileEfficiency(p.M, p.N, 64, 64);
   if (big_ok) {
     LaunchConfig<128, 128, 16, 2, 2, 1, LA, LB, VEC, 2, CONV, BF16>(p, n_batch, C, A, B, s);
-  } else if (tiles_m >= 192) {
+  } else if (tiles_m >= 192 ||
+             (CONV && tiles_m * std::min<int64_t>({8, p.K / 384, static_cast<int64_t>(kWorkspaceTiles) / (tiles_m * 4)}) >= 192)) {
+    // also when splitting K over up to 8 workgroups per tile fills the chip (measured on 3x3 convolutions
+    // with 32..104 tiles: 1.5x to 2x over the 32x32 tile)
     LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4, CONV, BF16>(p, n_batch, C, A, B, s);
   } else {
     LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2, CONV, BF16>(p, n_batch, C, A, B, s);

@@ -630,21 +630,13 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
             dim3(q.tiles_m * q.tiles_n, n_batch, splits), dim3(64 * WM * WN * KS), 0, s, q, C, A, B);
 }
 
-// Useful fraction of the MFMA work when the problem is cut into bm x bn tiles.
-inline double TileEfficiency(int64_t m, int64_t n, int64_t bm, int64_t bn) {
-  return static_cast<double>(m) * static_cast<double>(n) /
-         (static_cast<double>((m + bm - 1) / bm * bm) * static_cast<double>((n + bn - 1) / bn * bn));
-}
-
 template <int LA, int LB, int VEC, int CONV, bool BF16 = false>
 void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
-  const int64_t tiles_l = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * n_batch;
   const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
-  // the big tile only when it fills the chip and does not waste much more of itself on edges than the next one
-  const bool big_ok = !CONV && tiles_l >= 192 && TileEfficiency(p.M, p.N, 128, 128) + 0.15 >= TileEfficiency(p.M, p.N, 64, 64);
-  if (big_ok) {
-    LaunchConfig<128, 128, 16, 2, 2, 1, LA, LB, VEC, 2, CONV, BF16>(p, n_batch, C, A, B, s);
-  } else if (tiles_m >= 192 ||
+  // (A 128x128x16 tile with two chunks in flight was measured slower than the 64x64x32 tile with four at
+  // every size tried -- 4096^3: 101 against 123 TFLOP/s, [256,512]x[512,50304]: 69 against 108, 3x3
+  // convolutions: 50 against 67..85 -- and is not built.)
+  if (tiles_m >= 192 ||
              (CONV && tiles_m * std::min<int64_t>({8, p.K / 384, static_cast<int64_t>(kWorkspaceTiles) / (tiles_m * 4)}) >= 192)) {
     // also when splitting K over up to 8 workgroups per tile fills the chip (measured on 3x3 convolutions
     // with 32..104 tiles: 1.5x to 2x over the 32x32 tile)

@@ -159,6 +159,11 @@ def main():
     ms_per_step = elapsed / args.steps * 1e3
     value = batch * args.steps / elapsed
 
+    # distribution of single replays (device time between events on the plan's stream)
+    per_replay = np.sort(np.asarray(ex.replay_times_ns(3, min(args.steps, 200)))) / 1e6
+    percentiles = {"p10": float(np.percentile(per_replay, 10)), "p50": float(np.percentile(per_replay, 50)),
+                   "p90": float(np.percentile(per_replay, 90))}
+
     # Invoke as the reference defines it (host buffers in and out): PCIe-inclusive
     t0 = time.perf_counter()
     for _ in range(10):
@@ -222,6 +227,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "ms_per_step_percentiles": percentiles,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -245,6 +245,12 @@ PYBIND11_MODULE(fluidml, m) {
            },
            py::arg("warmup") = 3, py::arg("iters") = 20,
            "mean device nanoseconds of one replay of the whole plan (inputs resident in HBM)")
+      .def("replay_times_ns",
+           [](worker::Executor &e, size_t warmup, size_t iters) {
+             return e.GetContext()->GetModule().ReplayTimesNs(warmup, iters);
+           },
+           py::arg("warmup") = 3, py::arg("iters") = 100,
+           "device nanoseconds of each of `iters` consecutive replays (events on the plan's stream)")
       .def("replay", [](worker::Executor &e, size_t n) { e.GetContext()->GetModule().ReplayResident(n); }, py::arg("n") = 1,
            "n replays of the plan on the tensors already in HBM, then a stream wait (no host copies)")
       .def("materialize", [](worker::Executor &e) { e.GetContext()->GetModule().Materialize(); });

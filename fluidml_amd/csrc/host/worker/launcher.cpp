@@ -406,6 +406,27 @@ double LaunchPlan::TimeReplayNs(size_t warmup, size_t iters) {
   return ns / static_cast<double>(std::max<size_t>(iters, 1));
 }
 
+std::vector<double> LaunchPlan::ReplayTimesNs(size_t warmup, size_t iters) {
+  Materialize();
+  kernel::LaunchContext ctx;
+  ctx.stream = stream_;
+  ctx.flags = flags_;
+  ctx.bf16 = bf16_;
+  for (size_t i = 0; i < warmup + 1; ++i) Replay(ctx);
+  std::vector<void *> events(iters + 1, nullptr);
+  for (void *&e : events) Check(fluidml_hip_event_create(&e), "event");
+  Check(fluidml_hip_event_record(events[0], stream_), "event record");
+  for (size_t i = 0; i < iters; ++i) {
+    Replay(ctx);
+    Check(fluidml_hip_event_record(events[i + 1], stream_), "event record");
+  }
+  Check(fluidml_hip_stream_synchronize(stream_), "waiting for the replays");
+  std::vector<double> out(iters, 0.0);
+  for (size_t i = 0; i < iters; ++i) Check(fluidml_hip_event_elapsed_ns(events[i], events[i + 1], &out[i]), "event elapsed");
+  for (void *e : events) fluidml_hip_event_destroy(e);
+  return out;
+}
+
 std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
   Materialize();
   kernel::LaunchContext ctx;

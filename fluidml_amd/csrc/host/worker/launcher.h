@@ -145,6 +145,8 @@ class LaunchPlan {
   std::vector<StepTime> Profile(size_t warmup, size_t iters);
   // mean device time of one whole replay measured with events on the plan's stream
   double TimeReplayNs(size_t warmup, size_t iters);
+  // device time of each of `iters` consecutive replays (events between them on the plan's stream, no host waits)
+  std::vector<double> ReplayTimesNs(size_t warmup, size_t iters);
 
   void SetFlags(uint32_t flags) { flags_ = flags; }
   uint32_t GetFlags() const { return flags_; }

@@ -683,6 +683,40 @@ def test_matmul_chain_view(device):
         assert_close(dfinal.logical(), want.logical(), what="matmul_chain_view")
 
 
+def test_matmul_chain_group(device):
+    """Three contractions that share the left operand in one launch (query / key / value projections), each
+    with its own weights, bias and output addressing."""
+    cabi = _cabi()
+    rng = np.random.default_rng(97)
+    S, H = 40, 64
+    a = rand(rng, (1, S, H), -1, 1)
+    ws = [rand(rng, (H, H), -0.2, 0.2) for _ in range(3)]
+    bs = [rand(rng, (H,), -0.5, 0.5) for _ in range(3)]
+    louts = [None, [2, 1, 0], [0, 2, 1]]
+    wants, douts = [], []
+    for w, b, lo in zip(ws, bs, louts):
+        t0, t1 = ok.View.empty((1, S, H)), ok.View.empty((1, S, H))
+        ok.matmul(ok.View(a), ok.View(w), t0)
+        ok.binary_f32(ok.BOP_ADD, ok.View(b), t0, t1)
+        wants.append(t1.logical())
+        douts.append(DeviceView(ok.View.empty((1, S, H), np.float32, lo, fill=2), device))
+    da = DeviceView(ok.View(a), device)
+    dws = [DeviceView(ok.View(w), device) for w in ws]
+    dbs = [DeviceView(ok.View(b), device) for b in bs]
+    ptr = ctypes.POINTER(cabi.FlTensor)
+    rhs = (ptr * 3)(*[ctypes.pointer(d.tensor) for d in dws])
+    bias = (ptr * 3)(*[ctypes.pointer(d.tensor) for d in dbs])
+    out = (ptr * 3)(*[ctypes.pointer(d.tensor) for d in douts])
+    announce("matmul chain group")
+    cabi.call("matmul_chain_group", 3, da.ref(), rhs, bias, out, ctypes.c_int64(0), None, None, ctypes.c_uint32(0), None)
+    for d, want in zip(douts, wants):
+        assert_close(d.logical(), want, what="matmul_chain_group")
+    # mismatching sibling shapes are rejected
+    bad = DeviceView(ok.View(rand(rng, (H, H + 4), -1, 1)), device)
+    rhs_bad = (ptr * 2)(ctypes.pointer(dws[0].tensor), ctypes.pointer(bad.tensor))
+    assert cabi.lib.fluidml_hip_matmul_chain_group(2, da.ref(), rhs_bad, bias, out, 0, None, None, 0, None) == -3  # FL_ERR_SHAPE
+
+
 def test_elementwise_chain(device):
     """Every chain operation against the oracle's standalone kernels, applied one after the other."""
     cabi = _cabi()

@@ -24,6 +24,7 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::ConvChain: return "ConvChain";
     case Launch::Kind::ElementwiseChain: return "ElementwiseChain";
     case Launch::Kind::DivAddSoftmax: return "DivAddSoftmax";
+    case Launch::Kind::Attention: return "Attention";
     case Launch::Kind::AddLayerNorm: return "AddLayerNormalization";
     case Launch::Kind::ReshapeTranspose: return "ReshapeTranspose";
     default: return "TransposeReshape";
@@ -191,7 +192,8 @@ class Scheduler {
       for (size_t i = 0; i < steps_.size(); ++i) {
         if (taken_[i]) continue;
         std::optional<Launch> l;
-        if (Kind(i) == OpKind::DivConstantRhs) l = MatchSoftmax(i);
+        if (Kind(i) == OpKind::MatMul) l = MatchAttention(i);
+        else if (Kind(i) == OpKind::DivConstantRhs) l = MatchSoftmax(i);
         else if (Kind(i) == OpKind::AddCommon) l = MatchLayerNorm(i);
         if (l) {
           for (size_t m : l->members) taken_[m] = true;
@@ -673,6 +675,87 @@ class Scheduler {
     if (Alias(l.out, l.b)) return std::nullopt;
     l.bytes = Bytes({&l.a, &l.b, &l.out});
     return l;
+  }
+
+  // scores = MatMul(q, k^T) -> Div | Mul by a constant [-> + mask] [-> Where(cond, x, fill)] -> Softmax over
+  // the keys -> MatMul(p, v), optionally followed by the head-merging Transpose / Reshape: one launch that
+  // keeps the score rows on chip.  The kernel's limits (head size, number of keys) are checked here so that
+  // the launch can never be refused at replay time.
+  std::optional<Launch> MatchAttention(size_t i) {
+    const Step &scores = steps_[i];
+    const auto &shape = scores.out.meta.GetShape();
+    const auto &qs = scores.in0.meta.GetShape(), &ks = scores.in1.meta.GetShape();
+    const size_t rank = shape.size();
+    if (!IsFloat(scores.out) || rank < 2 || qs.size() != rank || ks.size() != rank) return std::nullopt;
+    if (!std::equal(shape.begin(), shape.end() - 2, qs.begin()) || !std::equal(shape.begin(), shape.end() - 2, ks.begin())) {
+      return std::nullopt;  // broadcast batch dims
+    }
+    const int64_t head = qs[rank - 1], keys = shape[rank - 1];
+    if (head > 64 || keys > 256 || head == 0 || keys == 0) return std::nullopt;
+    Launch l;
+    l.kind = Launch::Kind::Attention;
+    l.a = scores.in0;
+    l.b = scores.in1;
+    l.members = {i};
+    std::vector<std::pair<size_t, Operand>> external = {{i, l.a}, {i, l.b}};
+    auto next = SoleReader(i);
+    if (!next || !IsFloat(steps_[*next].out) || steps_[*next].out.meta.GetShape() != shape) return std::nullopt;
+    if (Kind(*next) == OpKind::DivConstantRhs) l.divisor = true;
+    else if (Kind(*next) != OpKind::MulConstant) return std::nullopt;
+    l.s0 = Attrs(*next).value;
+    l.members.push_back(*next);
+    size_t cur = *next;
+    next = SoleReader(cur);
+    if (next && Kind(*next) == OpKind::AddCommon && steps_[*next].out.meta.GetShape() == shape) {
+      const auto mask = Other(*next, steps_[cur].out);
+      if (!mask || !IsFloat(*mask)) return std::nullopt;
+      l.d = *mask;
+      l.has_mask = true;
+      external.push_back({*next, l.d});
+      l.members.push_back(*next);
+      cur = *next;
+      next = SoleReader(cur);
+    }
+    if (next && Kind(*next) == OpKind::WhereConstantCondConstantScalarY && IsFloat(steps_[*next].out) &&
+        steps_[*next].out.meta.GetShape() == shape) {
+      l.has_cond = true;
+      l.owner = *next;
+      l.s1 = Attrs(*next).value;
+      l.members.push_back(*next);
+      cur = *next;
+      next = SoleReader(cur);
+    }
+    if (!next || Kind(*next) != OpKind::Softmax || steps_[*next].out.meta.GetShape() != shape) return std::nullopt;
+    const int64_t axis = steps_[*next].node->GetAxis();
+    if (axis != static_cast<int64_t>(rank) - 1 && axis != -1) return std::nullopt;
+    l.members.push_back(*next);
+    const Operand &probs = steps_[*next].out;
+    next = SoleReader(*next);
+    if (!next || Kind(*next) != OpKind::MatMul || !SameTensor(steps_[*next].in0, probs) || SameTensor(steps_[*next].in1, probs)) {
+      return std::nullopt;
+    }
+    const size_t pv = *next;
+    l.c = steps_[pv].in1;
+    const auto &vs = l.c.meta.GetShape();
+    if (!IsFloat(steps_[pv].out) || vs.size() != rank || !std::equal(shape.begin(), shape.end() - 2, vs.begin()) ||
+        vs[rank - 1] != head) {
+      return std::nullopt;
+    }
+    external.push_back({pv, l.c});
+    l.members.push_back(pv);
+    auto finish = [&](Launch *x) {
+      if (!Safe(x->members, external)) return false;
+      if (!OutputDisjoint(x->out, {&x->a, &x->b, &x->c}) || (x->has_mask && Alias(x->out, x->d))) return false;
+      x->bytes = x->has_mask ? Bytes({&x->a, &x->b, &x->c, &x->d, &x->out}) : Bytes({&x->a, &x->b, &x->c, &x->out});
+      if (x->has_cond) x->bytes += static_cast<double>(steps_[x->owner].kernel->GetConstantBytes());
+      x->flops = Flops(x->members);
+      return true;
+    };
+    Launch with_views = l;
+    if (AppendViews(pv, &with_views) && with_views.n_inner == 0 && finish(&with_views)) return with_views;
+    l.out = steps_[pv].out;
+    if (finish(&l)) return l;
+    return std::nullopt;
   }
 
   std::optional<Launch> MatchLayerNorm(size_t i) {

@@ -286,6 +286,29 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       rc = fluidml_hip_div_add_softmax(&a.t, l.s0, &b.t, &out.t, l.axis, ctx.stream);
       break;
     }
+    case Launch::Kind::Attention: {
+      const kernel::TensorView kt = ViewOf(Resolve(l.b), l.b), v = ViewOf(Resolve(l.c), l.c);
+      kernel::TensorView mask, cond;
+      if (l.has_mask) mask = ViewOf(Resolve(l.d), l.d);
+      if (l.has_cond) {
+        const kernel::DeviceConstant *c = steps_[l.owner].kernel->GetConstant(0);
+        if (c == nullptr) throw std::logic_error("fused attention: the Where node holds no condition");
+        cond = c->View();
+      }
+      kernel::TensorView dst = out;
+      if (!l.view_strides.empty()) {
+        // the context's logical dims addressed inside the buffer of the last folded Transpose / Reshape
+        size_t pv = 0;
+        for (size_t m : l.members) {
+          if (steps_[m].node->GetKind() == flow::OpKind::MatMul) pv = m;
+        }
+        dst = kernel::TensorView(out.t.base, steps_[pv].out.meta);
+        for (size_t d = 0; d < l.view_strides.size(); ++d) dst.t.strides[d] = l.view_strides[d];
+      }
+      rc = fluidml_hip_attention(&a.t, &kt.t, &v.t, &dst.t, l.s0, l.divisor ? 1 : 0, l.has_mask ? &mask.t : nullptr,
+                                 l.has_cond ? &cond.t : nullptr, l.s1, ctx.stream);
+      break;
+    }
     case Launch::Kind::AddLayerNorm: {
       const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
       const kernel::Kernel &ln = *steps_[l.owner].kernel;

@@ -59,17 +59,21 @@ struct Launch {
     MatMulGroup,       // up to four MatMulChains that share the left operand and all extents, one launch
     ElementwiseChain,  // two or more elementwise steps on one tensor
     DivAddSoftmax,     // DivConstantRhs -> AddCommon(mask) -> Softmax
+    Attention,         // MatMul -> Div|Mul constant [-> AddCommon(mask)] [-> Where(cond, x, scalar)] -> Softmax -> MatMul
     AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias
     ReshapeTranspose,  // Reshape -> Transpose, one strided copy
     TransposeReshape   // Transpose -> Reshape, one strided copy
   };
   Kind kind = Kind::Step;
   std::vector<size_t> members;  // indices into the step list, ascending
-  Operand a, b, c, out;         // external operands, role by kind (see fusion.cpp)
+  Operand a, b, c, d, out;      // external operands, role by kind (see fusion.cpp)
   double s0 = 0, s1 = 0, s2 = 0;
   int64_t axis = 0;
   std::vector<int64_t> perm;
   bool has_c = false;     // MatMulChain: a bias operand is present
+  // Attention: a = queries, b = keys (transposed), c = values, d = additive mask (has_mask), the Where step
+  // `owner` holds the condition (has_cond) and s1 its fill value; s0 scales the scores, dividing if `divisor`
+  bool has_mask = false, has_cond = false, divisor = false;
   // MatMulChain followed by Reshape/Transpose steps that only re-address the result: element strides of the
   // contraction's logical output dims inside `out` (empty: `out` is the contraction's own output tensor),
   // and the optional split of the last dim (see fluidml_hip_matmul_chain_view)

@@ -358,6 +358,16 @@ int fluidml_hip_elementwise_chain(const fl_tensor *in, const fl_tensor *out, con
  * out = softmax(in / div + mask, axis)
  * (reference div.cpp:24-56 + add.cpp:75-137 + softmax.cpp:22-139). */
 int fluidml_hip_div_add_softmax(const fl_tensor *in, double div, const fl_tensor *mask, const fl_tensor *out, int64_t axis, void *stream);
+/* MatMulKernel -> DivConstantRhs | MulConstant -> [AddCommon(mask)] ->
+ * [WhereConstantCondConstantScalarY] -> SoftmaxKernel(last axis) -> MatMulKernel:
+ *   out = softmax(where(keep_cond, (q.kt) / scale (or * scale) + add_mask, fill)) . v
+ * q [..., Sq, D], kt [..., D, Skv], v [..., Skv, D], out [..., Sq, D], equal
+ * batch dims, any strides (a transposed or head-split view costs nothing);
+ * add_mask (float32) and keep_cond (bool) broadcast to [..., Sq, Skv] and may
+ * be NULL.  D <= 64 and Skv <= 256, otherwise FL_ERR_UNSUPPORTED (nothing
+ * launched).  (reference matmul.cpp:28-59, div.cpp:24-56, add.cpp:75-137,
+ * where.cpp:17-150, softmax.cpp:22-139) */
+int fluidml_hip_attention(const fl_tensor *q, const fl_tensor *kt, const fl_tensor *v, const fl_tensor *out, double scale, int32_t scale_is_divisor, const fl_tensor *add_mask, const fl_tensor *keep_cond, double fill, void *stream);
 /* AddCommonKernel -> LayerNormalizationConstantScaleBiasKernel:
  * out = LayerNorm(lhs + rhs) (reference add.cpp:75-137 +
  * layer_normalization.cpp:33-220, ONNX semantics). */

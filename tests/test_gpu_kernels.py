@@ -831,6 +831,65 @@ def test_fused_div_add_softmax(device):
     assert_close(dx.logical(), ho.logical(), what="div_add_softmax in place")
 
 
+def test_fused_attention(device):
+    """scores -> scale -> mask / where -> softmax -> context in one launch, against the oracle's chain of
+    MatMul, Div | Mul, Add | Where, Softmax, MatMul; operands as the strided views an attention block has."""
+    cabi = _cabi()
+    rng = np.random.default_rng(98)
+    # (batch dims, Sq, Skv, D, additive mask?, causal where?, scale is divisor?, keys stored transposed?)
+    # keys stored as [.., D, Skv] with every extent a multiple of four take the kernel's 128-bit path
+    cases = [((1, 12), 128, 128, 64, True, False, True, True), ((2, 3), 40, 40, 16, True, False, True, False),
+             ((1, 4), 200, 200, 64, False, True, False, True), ((3,), 33, 70, 32, False, False, True, True),
+             ((1, 2), 256, 256, 64, True, True, False, False), ((2, 2), 24, 36, 48, True, True, True, True),
+             ((1, 1), 5, 3, 7, True, False, False, False)]
+    for bdims, sq, skv, d, use_mask, use_where, divisor, kt_stored in cases:
+        q = rand(rng, bdims + (sq, d), -1, 1)
+        k = rand(rng, bdims + (skv, d), -1, 1)
+        v = rand(rng, bdims + (skv, d), -1, 1)
+        scale = float(np.sqrt(d)) if divisor else float(1.0 / np.sqrt(d))
+        mask = rand(rng, (1,) * len(bdims) + (1, skv), -8, 0) if use_mask else None
+        cond = np.tril(np.ones((sq, skv), np.bool_))[(None,) * len(bdims)] if use_where else None
+        fill = float(np.finfo(np.float32).min)
+        # oracle chain
+        kt = np.ascontiguousarray(np.swapaxes(k, -1, -2))
+        s0 = ok.View.empty(bdims + (sq, skv))
+        ok.matmul(ok.View(q), ok.View(kt), s0)
+        s1 = ok.View.empty(s0.shape)
+        ok.unary_f32(ok.OP_DIV_C if divisor else ok.OP_MUL_C, s0, s1, scale)
+        if use_mask:
+            s2 = ok.View.empty(s0.shape)
+            ok.binary_f32(ok.BOP_ADD, s1, ok.View(mask), s2)
+            s1 = s2
+        if use_where:
+            s2 = ok.View.empty(s0.shape)
+            ok.where(ok.View(cond), s1, None, fill, s2)
+            s1 = s2
+        p = ok.View.empty(s0.shape)
+        ok.softmax(s1, p, len(s0.shape) - 1)
+        want = ok.View.empty(bdims + (sq, d))
+        ok.matmul(p, ok.View(v), want)
+        announce("fused attention", bdims, sq, skv, d, use_mask, use_where, divisor, kt_stored)
+        dq, dv = DeviceView(ok.View(q), device), DeviceView(ok.View(v), device)
+        rank = len(bdims) + 2
+        if kt_stored:
+            dk = DeviceView(ok.View(kt), device)
+            ktv = dk.tensor
+        else:  # keys as the projection wrote them, [.., Skv, D]; the kernel sees K^T as a strided view
+            dk = DeviceView(ok.View(k), device)
+            kst = list(dk.tensor.strides[:rank])
+            ktv = cabi.make_tensor(dk.tensor.base, cabi.FL_FLOAT32, list(bdims) + [d, skv], kst[:-2] + [kst[-1], kst[-2]])
+        # output stored head-merged: [.., Sq, heads * D] like the Transpose + Reshape after the context matmul
+        lo = None if len(bdims) < 2 else list(range(len(bdims) - 1)) + [len(bdims), len(bdims) - 1, len(bdims) + 1]
+        do = DeviceView(ok.View.empty(bdims + (sq, d), np.float32, lo, fill=3), device)
+        dm = DeviceView(ok.View(mask), device) if use_mask else None
+        dc = DeviceView(ok.View(cond), device) if use_where else None
+        cabi.call("attention", dq.ref(), ctypes.byref(ktv), dv.ref(), do.ref(), ctypes.c_double(scale), int(divisor),
+                  dm.ref() if dm else None, dc.ref() if dc else None, ctypes.c_double(fill), None)
+        assert_close(do.logical(), want.logical(), what="attention")
+    big = DeviceView(ok.View.empty((1, 1, 8, 128)), device)
+    assert cabi.lib.fluidml_hip_attention(big.ref(), big.ref(), big.ref(), big.ref(), 1.0, 1, None, None, 0.0, None) != 0
+
+
 def test_fused_add_layer_norm(device):
     cabi = _cabi()
     rng = np.random.default_rng(93)

@@ -346,10 +346,10 @@ def _overlap(x, y):
 
 SCHEDULE_NETS = {
     "bert": (lambda m: m.bert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32, seed=5),
-             {"MatMulChain", "AddLayerNormalization", "DivAddSoftmax", "ElementwiseChain"}),
+             {"MatMulChain", "AddLayerNormalization", "Attention", "ElementwiseChain"}),
     "convbert": (lambda m: m.convbert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32),
-                 {"MatMulChain", "AddLayerNormalization", "DivAddSoftmax"}),
-    "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), {"MatMulChain"}),
+                 {"MatMulChain", "AddLayerNormalization"}),  # whether its attention fuses depends on the plan's reuse of bytes
+    "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), {"MatMulChain", "Attention"}),
     "efficientnet_b0": (lambda m: m.efficientnet_b0(image=64, classes=10, width_div=4), {"ConvChain"}),
     "vgg16": (lambda m: m.vgg16(batch=2, image=32, classes=10, width_div=8, fc=512), {"ConvChain", "GemmChain"}),
 }

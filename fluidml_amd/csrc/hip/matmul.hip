@@ -57,35 +57,60 @@ struct ConvGeom {
   FastDiv div_khw, div_kw;       // k -> (channel, kh, kw)
 };
 
+// Batch dims of a contraction after merging (operand 0 = C, 1 = A, 2 = B), innermost last.  Kept small and
+// statically indexed: the kernel's scalar loads of its arguments are a serial chain of cache misses otherwise.
+constexpr int kMaxBatchDims = 4;
+struct BatchArgs {
+  int32_t rank;  // 0: a single batch element
+  FastDiv div[kMaxBatchDims];
+  int32_t strides[3][kMaxBatchDims];
+};
+
+// Kernel arguments.  Every workgroup needs the first block before it can issue its first load, and a cold
+// 64-byte line of kernel arguments costs a few hundred nanoseconds: what every launch reads comes first and
+// is packed, what only some launches read (chain, siblings, convolution geometry) follows.
 struct MatmulArgs {
   int32_t M, N, K;
   int32_t sAm, sAk, sBk, sBn, sCm, sCn;
-  NestArgs<3> batch;  // operand 0 = C, 1 = A, 2 = B
   uint32_t tiles_m, tiles_n;
-  // epilogue: C = ca * acc + cb * bias[m * sDm + n * sDn]   (bias may be null)
-  float ca, cb;
-  const float *bias;
-  int32_t sDm, sDn;
-  // optional elementwise chain applied after the bias (chain.n == 0: none)
-  fl_ew_program chain;
-  // split K over gridDim.z workgroups per tile: each takes `chunks_per_split` chunks, writes its partial tile
-  // to `partials`, and the workgroup that arrives last at `counters[tile]` adds them up in split order
+  // split K over `n_splits` workgroups per tile (blockIdx.z): each takes `chunks_per_split` chunks, writes its
+  // partial tile to `partials`, and the workgroup that arrives last at `counters[tile]` adds them up in split order
+  uint32_t n_splits;
+  int32_t chunks_per_split;
+  // sibling contractions that share A and every extent, one per blockIdx.y (n_groups <= 1: none; batch
+  // dims are then absent).  Member 0 uses the fields here, member g > 0 the entries g - 1 of the g* arrays.
+  int32_t n_groups;
   // optional two-level column addressing of C: column n lives at (n / n_inner) * sCn_outer + (n % n_inner) * sCn
   // (the last output dim reshaped into two dims that a transpose moved apart); n_inner == 0: n * sCn
   int32_t n_inner, sCn_outer;
+  // epilogue: C = ca * acc + cb * bias[m * sDm + n * sDn]   (bias may be null)
+  const float *bias;
+  int32_t sDm, sDn;
+  float ca, cb;
+  float *partials;
+  uint32_t *counters;
+  BatchArgs batch;
   FastDiv div_inner;
-  // sibling contractions that share A and every extent, one per blockIdx.y (n_groups <= 1: none; batch
-  // dims are then absent).  Member 0 uses the fields above, member g > 0 the entries g - 1 below.
-  int32_t n_groups;
+  // optional elementwise chain applied after the bias (chain.n == 0: none)
+  fl_ew_program chain;
   const float *gB[3];
   float *gC[3];
   const float *gbias[3];
   int32_t g_sCm[3], g_sCn[3], g_sCn_outer[3];
-  int32_t chunks_per_split;
-  float *partials;
-  uint32_t *counters;
   ConvGeom conv;  // read by the CONV instantiations only
 };
+
+inline int MakeBatchArgs(const LoopNest &nest, int64_t n_batch, BatchArgs *b) {
+  std::memset(b, 0, sizeof(*b));
+  if (n_batch == 1) return FL_OK;
+  if (nest.rank > kMaxBatchDims) return FL_ERR_UNSUPPORTED;
+  b->rank = nest.rank;
+  for (int i = 0; i < nest.rank; ++i) {
+    b->div[i] = FastDiv(static_cast<uint32_t>(nest.shape[i]));
+    for (int o = 0; o < 3; ++o) b->strides[o][i] = static_cast<int32_t>(nest.strides[o][i]);
+  }
+  return FL_OK;
+}
 
 template <int VEC>
 struct VecF {
@@ -154,9 +179,8 @@ struct TileLoader {
 // (unit stride along W in the input and in the convolution, OW a multiple of 4).
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV = 0,
           bool BF16 = false>
-__global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, float *__restrict__ C_,
-                                                                const float *__restrict__ A,
-                                                                const float *__restrict__ B_) {
+__global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restrict__ C_, const float *__restrict__ A,
+                                                                const float *__restrict__ B_, MatmulArgs p) {
   float *__restrict__ C = C_;
   const float *__restrict__ B = B_;
   constexpr int NT = 64 * WM * WN * KS;
@@ -204,14 +228,17 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
     batch_id = 0;
   }
   int32_t boff[3] = {0, 0, 0};
-  {
+  if (p.batch.rank > 0) {
     uint32_t rem = batch_id;
-    for (int d = p.batch.rank - 1; d > 0; --d) {
-      uint32_t q, r;
-      p.batch.div[d].DivMod(rem, q, r);
-      rem = q;
 #pragma unroll
-      for (int o = 0; o < 3; ++o) boff[o] += static_cast<int32_t>(r) * p.batch.strides[o][d];
+    for (int d = kMaxBatchDims - 1; d > 0; --d) {
+      if (d < p.batch.rank) {
+        uint32_t q, r;
+        p.batch.div[d].DivMod(rem, q, r);
+        rem = q;
+#pragma unroll
+        for (int o = 0; o < 3; ++o) boff[o] += static_cast<int32_t>(r) * p.batch.strides[o][d];
+      }
     }
 #pragma unroll
     for (int o = 0; o < 3; ++o) boff[o] += static_cast<int32_t>(rem) * p.batch.strides[o][0];
@@ -231,6 +258,16 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  // A bias with one value per column is requested now: at the end of the kernel its load would be one more
+  // cold miss in the chain.
+  const bool bias_by_col = bias != nullptr && p.sDm == 0;
+  float bias_col[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + (wn * TN + j) * 32 + lrow;
+    bias_col[j] = bias_by_col && n < p.N ? bias[n * p.sDn] : 0.0f;
+  }
 
   // DEPTH chunks are in flight in registers: the loads of chunk c+DEPTH are issued while chunk c is
   // consumed, so a workgroup keeps DEPTH * (A tile + B tile) bytes outstanding instead of one chunk --
@@ -368,9 +405,9 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
     }
   };
 
-  // this workgroup's share of the chunks (all of them unless K is split over gridDim.z)
-  const int c_begin = gridDim.z > 1 ? static_cast<int>(blockIdx.z) * p.chunks_per_split : 0;
-  const int c_end = gridDim.z > 1 ? min(n_chunks, c_begin + p.chunks_per_split) : n_chunks;
+  // this workgroup's share of the chunks (all of them unless K is split over blockIdx.z)
+  const int c_begin = p.n_splits > 1 ? static_cast<int>(blockIdx.z) * p.chunks_per_split : 0;
+  const int c_end = p.n_splits > 1 ? min(n_chunks, c_begin + p.chunks_per_split) : n_chunks;
 #pragma unroll
   for (int s = 0; s < DEPTH; ++s) {
     if (c_begin + s < c_end) load_chunk(c_begin + s, ra[s], rb[s]);
@@ -430,9 +467,9 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
   // tile, then one atomic tells it whether it arrived last; the last wave adds all partials in split order,
   // which makes the sum independent of arrival order.
   if constexpr (TM * TN == 1 && (WM * WN == 1 || KS == 1)) {
-    if (gridDim.z > 1) {
-      const uint32_t n_splits = gridDim.z;
-      const uint32_t tile_id = (blockIdx.y * gridDim.x + blockIdx.x) * (WM * WN) + wm * WN + wn;
+    if (p.n_splits > 1) {
+      const uint32_t n_splits = p.n_splits;
+      const uint32_t tile_id = (blockIdx.y * n_tiles + blockIdx.x) * (WM * WN) + wm * WN + wn;
       float *mine = p.partials + (static_cast<size_t>(tile_id) * n_splits + blockIdx.z) * 1024;
       // The partial tiles travel through device-coherent accesses (agent-scope atomics: they bypass the
       // per-XCD L2 instead of living in it), so no cache-wide write-back or invalidate is needed: waiting
@@ -484,7 +521,9 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
         float v = acc[i][j][e];
-        if (bias != nullptr && m < p.M && n < p.N) {
+        if (bias_by_col) {
+          v = p.ca * v + p.cb * bias_col[j];
+        } else if (bias != nullptr && m < p.M && n < p.N) {
           v = p.ca * v + p.cb * bias[m * p.sDm + n * p.sDn];
         }
         vals[e] = v;
@@ -504,8 +543,8 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(MatmulArgs p, fl
 // each and combine them with wave64 shuffles.  No LDS, no MFMA: at one to eight rows the matrix cores would
 // run 75-97 % empty while the kernel waits for the weights anyway.
 template <int MT, int kSkinnyRows>
-__global__ __launch_bounds__(256) void SkinnyGemmKernel(MatmulArgs p, float *__restrict__ C, const float *__restrict__ A,
-                                                        const float *__restrict__ B) {
+__global__ __launch_bounds__(256) void SkinnyGemmKernel(float *__restrict__ C, const float *__restrict__ A,
+                                                        const float *__restrict__ B, MatmulArgs p) {
   const int lane = threadIdx.x % 64;
   const int n0 = (blockIdx.x * 4 + threadIdx.x / 64) * kSkinnyRows;
   if (n0 >= p.N) return;
@@ -576,9 +615,9 @@ inline bool TrySkinnyGemm(const MatmulArgs &p, int64_t n_batch, float *C, const 
   const dim3 grid((p.N + 4 * rows - 1) / (4 * rows)), block(256);
 #define FL_SKINNY(MT_)                                                                              \
   do {                                                                                              \
-    if (rows == 4) FL_LAUNCH((SkinnyGemmKernel<MT_, 4>), grid, block, 0, s, p, C, A, B);            \
-    else if (rows == 2) FL_LAUNCH((SkinnyGemmKernel<MT_, 2>), grid, block, 0, s, p, C, A, B);       \
-    else FL_LAUNCH((SkinnyGemmKernel<MT_, 1>), grid, block, 0, s, p, C, A, B);                      \
+    if (rows == 4) FL_LAUNCH((SkinnyGemmKernel<MT_, 4>), grid, block, 0, s, C, A, B, p);            \
+    else if (rows == 2) FL_LAUNCH((SkinnyGemmKernel<MT_, 2>), grid, block, 0, s, C, A, B, p);       \
+    else FL_LAUNCH((SkinnyGemmKernel<MT_, 1>), grid, block, 0, s, C, A, B, p);                      \
   } while (0)
   if (p.M == 1) FL_SKINNY(1);
   else if (p.M == 2) FL_SKINNY(2);
@@ -626,8 +665,9 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
       }
     }
   }
+  q.n_splits = splits;
   FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV, BF16>),
-            dim3(q.tiles_m * q.tiles_n, n_batch, splits), dim3(64 * WM * WN * KS), 0, s, q, C, A, B);
+            dim3(q.tiles_m * q.tiles_n, n_batch, splits), dim3(64 * WM * WN * KS), 0, s, C, A, B, q);
 }
 
 template <int LA, int LB, int VEC, int CONV, bool BF16 = false>
@@ -711,7 +751,7 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   int64_t n_batch = 1;
   for (int i = 0; i < nest.rank; ++i) n_batch *= nest.shape[i];
   if (n_batch > 65535) return FL_ERR_TOO_LARGE;
-  p.batch = MakeNestArgs<3>(nest);
+  FL_CHECK(MakeBatchArgs(nest, n_batch, &p.batch));
   p.ca = ca;
   p.cb = cb;
   if (chain != nullptr) p.chain = *chain;

@@ -57,16 +57,7 @@ __global__ __launch_bounds__(256) void AttentionKernel(AttentionArgs a, float *_
 
   const uint32_t qb = blockIdx.x % a.q_blocks;
   int32_t off[6] = {0, 0, 0, 0, 0, 0};
-  {
-    uint32_t rem = blockIdx.x / a.q_blocks;
-    for (int d = a.batch.rank - 1; d >= 0; --d) {
-      uint32_t qq = 0, r = rem;
-      if (d > 0) a.batch.div[d].DivMod(rem, qq, r);
-      rem = qq;
-#pragma unroll
-      for (int o = 0; o < 6; ++o) off[o] += static_cast<int32_t>(r) * a.batch.strides[o][d];
-    }
-  }
+  a.batch.AddOffsets(blockIdx.x / a.q_blocks, off);
   const int m0 = static_cast<int>(qb) * kQ;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, l16 = lane % 16, grp = lane / 16;
 

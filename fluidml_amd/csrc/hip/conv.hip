@@ -16,10 +16,9 @@ constexpr int kBlock = 256;
 constexpr int kMaxSpatial = 3;
 
 struct ConvArgs {
-  NestArgs<1> out_nest;  // canonical order of the output's (n, f, o...) index space; operand 0 = out offset
-  // logical de-linearisation of the canonical index back to (n, f, o...):
-  // stride table of a second operand that carries the logical linear index
-  int32_t lin_strides[kMaxRank];
+  // canonical order of the output's (n, f, o...) index space; operand 0 = out offset, operand 1 = the logical
+  // linear index (de-linearised back to (n, f, o...) in the kernel)
+  NestArgs<2> out_nest;
   int32_t rank;          // 2 + n_spatial
   int32_t n_spatial;
   int32_t out_shape[2 + kMaxSpatial];
@@ -44,19 +43,10 @@ __global__ __launch_bounds__(kBlock) void ConvDirect(ConvArgs p, float *__restri
   const uint32_t item = blockIdx.x * kBlock + threadIdx.x;
   if (item >= p.n_out) return;
   // canonical index -> output offset and logical linear index
-  int32_t ooff = 0, lin = 0;
-  {
-    uint32_t rem = item;
-    for (int d = p.out_nest.rank - 1; d > 0; --d) {
-      uint32_t q, r;
-      p.out_nest.div[d].DivMod(rem, q, r);
-      rem = q;
-      ooff += static_cast<int32_t>(r) * p.out_nest.strides[0][d];
-      lin += static_cast<int32_t>(r) * p.lin_strides[d];
-    }
-    ooff += static_cast<int32_t>(rem) * p.out_nest.strides[0][0];
-    lin += static_cast<int32_t>(rem) * p.lin_strides[0];
-  }
+  int32_t both[2] = {0, 0};
+  p.out_nest.AddOffsets(item, both);
+  const int32_t ooff = both[0];
+  int32_t lin = both[1];
   int32_t o[NS];
 #pragma unroll
   for (int d = NS - 1; d >= 0; --d) {
@@ -197,14 +187,7 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
     acc *= out->shape[i];
   }
   nest.Canonicalise();
-  NestArgs<2> both = MakeNestArgs<2>(nest);
-  p.out_nest.rank = both.rank;
-  for (int i = 0; i < both.rank; ++i) {
-    p.out_nest.shape[i] = both.shape[i];
-    p.out_nest.div[i] = both.div[i];
-    p.out_nest.strides[0][i] = both.strides[0][i];
-    p.lin_strides[i] = both.strides[1][i];
-  }
+  p.out_nest = MakeNestArgs<2>(nest);
   p.n_out = static_cast<uint32_t>(Numel(out));
   const dim3 grid((p.n_out + kBlock - 1) / kBlock), block(kBlock);
   float *o = static_cast<float *>(out->base);

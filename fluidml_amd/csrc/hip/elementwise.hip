@@ -31,19 +31,10 @@ __global__ __launch_bounds__(kBlock) void EwKernel(NestArgs<NIN + 1> a, uint32_t
                                                    const T1 *__restrict__ in1, const T2 *__restrict__ in2, Op op) {
   const uint32_t stride = gridDim.x * kBlock;
   for (uint32_t item = blockIdx.x * kBlock + threadIdx.x; item < n_items; item += stride) {
-    uint32_t rem = item;
     int32_t off[NIN + 1];
 #pragma unroll
     for (int o = 0; o <= NIN; ++o) off[o] = 0;
-    for (int d = a.rank - 1; d > 0; --d) {
-      uint32_t q, r;
-      a.div[d].DivMod(rem, q, r);
-      rem = q;
-#pragma unroll
-      for (int o = 0; o <= NIN; ++o) off[o] += static_cast<int32_t>(r) * a.strides[o][d];
-    }
-#pragma unroll
-    for (int o = 0; o <= NIN; ++o) off[o] += static_cast<int32_t>(rem) * a.strides[o][0];
+    a.AddOffsets(item, off);
 
     if constexpr (VEC == 1) {
       T0 x0 = in0[off[1]];
@@ -308,15 +299,9 @@ __global__ __launch_bounds__(256) void TiledCopyKernel(TiledCopyArgs a, uint32_t
                                                        const uint32_t *__restrict__ in) {
   __shared__ uint32_t tile[64][65];
   const uint32_t t_of = blockIdx.x % a.tiles_out_fast, t_if = (blockIdx.x / a.tiles_out_fast) % a.tiles_in_fast;
-  uint32_t rem = blockIdx.x / (a.tiles_out_fast * a.tiles_in_fast);
-  int32_t off_out = 0, off_in = 0;
-  for (int d = a.outer.rank - 1; d >= 0; --d) {
-    uint32_t q = 0, r = rem;
-    if (d > 0) a.outer.div[d].DivMod(rem, q, r);
-    rem = q;
-    off_out += static_cast<int32_t>(r) * a.outer.strides[0][d];
-    off_in += static_cast<int32_t>(r) * a.outer.strides[1][d];
-  }
+  int32_t off2[2] = {0, 0};
+  a.outer.AddOffsets(blockIdx.x / (a.tiles_out_fast * a.tiles_in_fast), off2);
+  const int32_t off_out = off2[0], off_in = off2[1];
   const uint32_t of0 = t_of * 64, if0 = t_if * 64;
   const uint32_t lane = threadIdx.x % 64, row = threadIdx.x / 64;
   // read: lanes run along the input-fast dim
@@ -449,10 +434,10 @@ __global__ __launch_bounds__(256) void PadKernel(PadArgs p, T *__restrict__ out,
   bool inside = true;
   for (int d = p.nest.rank - 1; d >= 0; --d) {
     uint32_t q = 0, r = rem;
-    if (d > 0) p.nest.div[d].DivMod(rem, q, r);
+    if (d > 0) p.nest.dims[d].div.DivMod(rem, q, r);
     rem = q;
-    off_out += static_cast<int32_t>(r) * p.nest.strides[0][d];
-    off_in += static_cast<int32_t>(r) * p.nest.strides[1][d];
+    off_out += static_cast<int32_t>(r) * p.nest.dims[d].strides[0];
+    off_in += static_cast<int32_t>(r) * p.nest.dims[d].strides[1];
     inside = inside && r >= p.lo[d] && r < p.hi[d];
   }
   out[off_out] = inside ? in[off_in - p.in_base] : T(0);

@@ -324,12 +324,65 @@ inline int BroadcastStrides(const fl_tensor *t, int out_rank, const int64_t *out
 }
 
 // Device-side descriptor of a canonical loop nest.
+#if defined(__HIPCC__)
+// Forces a wave-uniform value (a kernel argument) into a scalar register here.
+template <typename T>
+__device__ __forceinline__ void PinScalar(const T &x) {
+  asm volatile("" ::"s"(x));
+}
+#endif
+
+// Everything a kernel reads about one dim lies together, and the dims a kernel usually has (one to three)
+// come first: the scalar loads of the kernel arguments miss once per 64-byte line, one miss after the other
+// when the index is not a compile-time constant, and that chain sits in front of a kernel's first load.
 template <int NOPS>
 struct NestArgs {
+  struct Dim {
+    FastDiv div;  // div.divisor is the extent
+    int32_t strides[NOPS];
+  };
   int32_t rank;
-  uint32_t shape[kMaxRank];
-  FastDiv div[kMaxRank];
-  int32_t strides[NOPS][kMaxRank];
+  Dim dims[kMaxRank];
+
+#if defined(__HIPCC__)
+  // Splits `index` over the dims (innermost last) and adds operand o's offset to off[o], o < N.
+  template <int N>
+  __device__ __forceinline__ void AddOffsets(uint32_t index, int32_t (&off)[N]) const {
+    static_assert(N <= NOPS, "more offsets than operands");
+    constexpr int kStatic = 4;  // dims handled with compile-time argument offsets
+    // request the first three dims' descriptors in one batch (see the layout note above): left alone the
+    // compiler fetches each field right before its use, one scalar-cache round trip after the other
+    PinScalar(rank);
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+      PinScalar(dims[d].div.divisor);
+      PinScalar(dims[d].div.multiplier);
+      PinScalar(dims[d].div.shift);
+#pragma unroll
+      for (int o = 0; o < N; ++o) PinScalar(dims[d].strides[o]);
+    }
+    uint32_t rem = index;
+    for (int d = rank - 1; d >= kStatic; --d) {
+      uint32_t q, r;
+      dims[d].div.DivMod(rem, q, r);
+      rem = q;
+#pragma unroll
+      for (int o = 0; o < N; ++o) off[o] += static_cast<int32_t>(r) * dims[d].strides[o];
+    }
+#pragma unroll
+    for (int d = kStatic - 1; d > 0; --d) {
+      if (d < rank) {
+        uint32_t q, r;
+        dims[d].div.DivMod(rem, q, r);
+        rem = q;
+#pragma unroll
+        for (int o = 0; o < N; ++o) off[o] += static_cast<int32_t>(r) * dims[d].strides[o];
+      }
+    }
+#pragma unroll
+    for (int o = 0; o < N; ++o) off[o] += static_cast<int32_t>(rem) * dims[0].strides[o];
+  }
+#endif
 };
 
 template <int NOPS>
@@ -339,9 +392,8 @@ inline NestArgs<NOPS> MakeNestArgs(const LoopNest &nest) {
   std::memset(&a, 0, sizeof(a));
   a.rank = nest.rank;
   for (int i = 0; i < nest.rank; ++i) {
-    a.shape[i] = static_cast<uint32_t>(nest.shape[i]);
-    a.div[i] = FastDiv(static_cast<uint32_t>(nest.shape[i]));
-    for (int o = 0; o < NOPS; ++o) a.strides[o][i] = static_cast<int32_t>(nest.strides[o][i]);
+    a.dims[i].div = FastDiv(static_cast<uint32_t>(nest.shape[i]));
+    for (int o = 0; o < NOPS; ++o) a.dims[i].strides[o] = static_cast<int32_t>(nest.strides[o][i]);
   }
   return a;
 }

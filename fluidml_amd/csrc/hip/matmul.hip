@@ -201,6 +201,23 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restric
   using LoaderA = typename std::conditional<LA == 0, TileLoader<BM, BK, VEC, NT>, TileLoader<BK, BM, VEC, NT>>::type;
   using LoaderB = typename std::conditional<LB == 0, TileLoader<BK, BN, VB, NT>, TileLoader<BN, BK, VB, NT>>::type;
 
+  // Request every argument the kernel is going to read in one batch and wait for them once: left to itself the
+  // compiler loads each field right before its first use, a dozen dependent round trips to the scalar cache
+  // before the first tile load can be issued.
+  asm volatile("" ::"s"(p.M), "s"(p.N), "s"(p.K), "s"(p.sAm), "s"(p.sAk), "s"(p.sBk), "s"(p.sBn), "s"(p.sCm), "s"(p.sCn),
+               "s"(p.tiles_m), "s"(p.tiles_n), "s"(p.n_splits), "s"(p.chunks_per_split), "s"(p.n_groups), "s"(p.n_inner),
+               "s"(p.sCn_outer), "s"(p.bias), "s"(p.sDm), "s"(p.sDn), "s"(p.ca), "s"(p.cb), "s"(p.partials),
+               "s"(p.counters), "s"(p.batch.rank), "s"(p.chain.n));
+  if constexpr (CONV != 0) {
+    asm volatile("" ::"s"(p.conv.H), "s"(p.conv.W), "s"(p.conv.sh), "s"(p.conv.sw), "s"(p.conv.dh), "s"(p.conv.dw),
+                 "s"(p.conv.ph), "s"(p.conv.pw), "s"(p.conv.sXn), "s"(p.conv.sXc), "s"(p.conv.sXh), "s"(p.conv.sXw),
+                 "s"(p.conv.sOn), "s"(p.conv.sOh), "s"(p.conv.sOw), "s"(p.conv.div_ohw.divisor),
+                 "s"(p.conv.div_ohw.multiplier), "s"(p.conv.div_ohw.shift), "s"(p.conv.div_ow.divisor),
+                 "s"(p.conv.div_ow.multiplier), "s"(p.conv.div_ow.shift), "s"(p.conv.div_khw.divisor),
+                 "s"(p.conv.div_khw.multiplier), "s"(p.conv.div_khw.shift), "s"(p.conv.div_kw.divisor),
+                 "s"(p.conv.div_kw.multiplier), "s"(p.conv.div_kw.shift));
+  }
+
   // ---- which tile -----------------------------------------------------------
   uint32_t bid = blockIdx.x;
   const uint32_t n_tiles = p.tiles_m * p.tiles_n;

@@ -21,18 +21,12 @@ struct alignas(sizeof(T) * N) Vec {
 
 template <int NOPS>
 __device__ __forceinline__ void ItemOffsets(const NestArgs<NOPS> &a, uint32_t item, int32_t *off) {
+  int32_t acc[NOPS];
 #pragma unroll
-  for (int o = 0; o < NOPS; ++o) off[o] = 0;
-  uint32_t rem = item;
-  for (int d = a.rank - 1; d > 0; --d) {
-    uint32_t q, r;
-    a.div[d].DivMod(rem, q, r);
-    rem = q;
+  for (int o = 0; o < NOPS; ++o) acc[o] = 0;
+  a.AddOffsets(item, acc);
 #pragma unroll
-    for (int o = 0; o < NOPS; ++o) off[o] += static_cast<int32_t>(r) * a.strides[o][d];
-  }
-#pragma unroll
-  for (int o = 0; o < NOPS; ++o) off[o] += static_cast<int32_t>(rem) * a.strides[o][0];
+  for (int o = 0; o < NOPS; ++o) off[o] = acc[o];
 }
 
 // ---- Reshape ------------------------------------------------------------------
@@ -47,16 +41,9 @@ __global__ __launch_bounds__(kBlock) void ReshapeKernel(NestArgs<2> a, NestArgs<
   if (item >= n) return;
   int32_t off[2];
   ItemOffsets<2>(a, item, off);
-  uint32_t rem = static_cast<uint32_t>(off[1]);
-  int32_t in_off = 0;
-  for (int d = src.rank - 1; d > 0; --d) {
-    uint32_t q, r;
-    src.div[d].DivMod(rem, q, r);
-    rem = q;
-    in_off += static_cast<int32_t>(r) * src.strides[0][d];
-  }
-  in_off += static_cast<int32_t>(rem) * src.strides[0][0];
-  out[off[0]] = in[in_off];
+  int32_t in_off[1] = {0};
+  src.AddOffsets(static_cast<uint32_t>(off[1]), in_off);
+  out[off[0]] = in[in_off[0]];
 }
 
 // Merge logically adjacent dims that are contiguous, keeping logical order.

@@ -32,30 +32,15 @@ __global__ __launch_bounds__(kBlock) void PoolKernel(PoolArgs p, float *__restri
                                                      const float *__restrict__ in) {
   const uint32_t item = blockIdx.x * kBlock + threadIdx.x;
   if (item >= p.n_out) return;
-  int32_t off0 = 0, off1 = 0;
-  uint32_t rem = item;
-  for (int d = p.nest.rank - 1; d > 0; --d) {
-    uint32_t q, r;
-    p.nest.div[d].DivMod(rem, q, r);
-    rem = q;
-    off0 += static_cast<int32_t>(r) * p.nest.strides[0][d];
-    off1 += static_cast<int32_t>(r) * p.nest.strides[1][d];
-  }
-  off0 += static_cast<int32_t>(rem) * p.nest.strides[0][0];
-  off1 += static_cast<int32_t>(rem) * p.nest.strides[1][0];
-  const float *src = in + off1;
+  int32_t off[2] = {0, 0};
+  p.nest.AddOffsets(item, off);
+  const int32_t off0 = off[0];
+  const float *src = in + off[1];
   float acc = src[0];
   for (uint32_t w = 1; w < p.n_window; ++w) {
-    uint32_t wr = w;
-    int32_t woff = 0;
-    for (int d = p.window.rank - 1; d > 0; --d) {
-      uint32_t q, r;
-      p.window.div[d].DivMod(wr, q, r);
-      wr = q;
-      woff += static_cast<int32_t>(r) * p.window.strides[0][d];
-    }
-    woff += static_cast<int32_t>(wr) * p.window.strides[0][0];
-    const float v = src[woff];
+    int32_t woff[1] = {0};
+    p.window.AddOffsets(w, woff);
+    const float v = src[woff[0]];
     acc = IS_MAX ? MaximumF(acc, v) : acc + v;
   }
   out[off0] = IS_MAX ? acc : acc / static_cast<float>(p.n_window);

@@ -20,26 +20,20 @@ constexpr int kBlock = 256;
 
 template <int NOPS>
 struct RowArgs {
-  NestArgs<NOPS> outer;  // non-axis dims, canonical order (operand 0 = output)
   uint32_t n_rows;
   uint32_t len;
   int32_t axis_stride[NOPS];
+  NestArgs<NOPS> outer;  // non-axis dims, canonical order (operand 0 = output)
 };
 
 template <int NOPS>
 __device__ __forceinline__ void RowOffsets(const NestArgs<NOPS> &a, uint32_t row, int32_t *off) {
+  int32_t acc[NOPS];
 #pragma unroll
-  for (int o = 0; o < NOPS; ++o) off[o] = 0;
-  uint32_t rem = row;
-  for (int d = a.rank - 1; d > 0; --d) {
-    uint32_t q, r;
-    a.div[d].DivMod(rem, q, r);
-    rem = q;
+  for (int o = 0; o < NOPS; ++o) acc[o] = 0;
+  a.AddOffsets(row, acc);
 #pragma unroll
-    for (int o = 0; o < NOPS; ++o) off[o] += static_cast<int32_t>(r) * a.strides[o][d];
-  }
-#pragma unroll
-  for (int o = 0; o < NOPS; ++o) off[o] += static_cast<int32_t>(rem) * a.strides[o][0];
+  for (int o = 0; o < NOPS; ++o) off[o] = acc[o];
 }
 
 // Build the outer nest (all dims but `axis`) for the given operands' strides.
@@ -366,15 +360,9 @@ struct ReduceArgs {
 };
 
 __device__ __forceinline__ int32_t InnerOffset(const NestArgs<1> &a, uint32_t idx) {
-  int32_t off = 0;
-  uint32_t rem = idx;
-  for (int d = a.rank - 1; d > 0; --d) {
-    uint32_t q, r;
-    a.div[d].DivMod(rem, q, r);
-    rem = q;
-    off += static_cast<int32_t>(r) * a.strides[0][d];
-  }
-  return off + static_cast<int32_t>(rem) * a.strides[0][0];
+  int32_t off[1] = {0};
+  a.AddOffsets(idx, off);
+  return off[0];
 }
 
 // One wave per output element.

@@ -513,7 +513,7 @@ class Scheduler {
       return SameTensor(x.a, y.a) && x.a.layout == y.a.layout && batch == 1 && shape == hy.out.meta.GetShape() &&
              x.b.space == Operand::Space::Constant && y.b.space == Operand::Space::Constant &&
              x.b.meta.GetShape() == y.b.meta.GetShape() && x.b.layout == y.b.layout && x.has_c == y.has_c &&
-             x.n_inner == y.n_inner && x.view_strides.empty() == y.view_strides.empty() && x.chain.n == y.chain.n &&
+             InnerCompatible(x, y, shape.back()) && x.view_strides.empty() == y.view_strides.empty() && x.chain.n == y.chain.n &&
              std::equal(x.chain.op, x.chain.op + x.chain.n, y.chain.op) &&
              std::equal(x.chain.c, x.chain.c + x.chain.n, y.chain.c);
     };
@@ -522,8 +522,13 @@ class Scheduler {
     for (size_t i = 0; i < fused->size(); ++i) {
       if (used[i]) continue;
       std::vector<size_t> set = {i};
+      int64_t inner = (*fused)[i].n_inner;  // the one non-zero column split of the set, if any
       for (size_t j = i + 1; j < fused->size() && set.size() < 4; ++j) {
-        if (!used[j] && compatible((*fused)[i], (*fused)[j])) set.push_back(j);
+        const Launch &y = (*fused)[j];
+        if (used[j] || !compatible((*fused)[i], y)) continue;
+        if (y.n_inner != 0 && inner != 0 && y.n_inner != inner) continue;
+        if (y.n_inner != 0) inner = y.n_inner;
+        set.push_back(j);
       }
       // the largest prefix of the candidates that can meet at the position of one of them
       size_t position = 0;
@@ -553,6 +558,12 @@ class Scheduler {
         g.flops += m.flops;
         g.bytes += m.bytes - (k == set[0] ? 0.0 : static_cast<double>(m.a.meta.GetSize()));
         g.group.push_back(m);
+        // a member whose columns are one strided run joins members with split columns by splitting its run
+        Launch &added = g.group.back();
+        if (added.n_inner == 0 && inner != 0) {
+          added.n_inner = inner;
+          added.stride_outer = inner * added.view_strides.back();
+        }
       }
       std::sort(g.members.begin(), g.members.end());
       std::sort(g.group.begin(), g.group.end(), [](const Launch &x, const Launch &y) { return x.members.back() < y.members.back(); });
@@ -564,8 +575,18 @@ class Scheduler {
     *fused = std::move(result);
   }
 
+  // Two chains can share a launch if their column addressing can be made the same: equal splits of the last
+  // output dim, or one of them unsplit (its columns are then one strided run, which any split describes too).
+  static bool InnerCompatible(const Launch &x, const Launch &y, int64_t columns) {
+    if (x.n_inner == y.n_inner) return true;
+    if (x.n_inner != 0 && y.n_inner != 0) return false;
+    const int64_t inner = x.n_inner != 0 ? x.n_inner : y.n_inner;
+    return !x.view_strides.empty() && !y.view_strides.empty() && columns % inner == 0;
+  }
+
   // Can every launch of `set` be issued at step position `position` (the last member of one of them)?
   bool CanGroupAt(const std::vector<Launch> &fused, const std::vector<size_t> &set, size_t position) const {
+
     std::vector<size_t> members;
     for (size_t k : set) members.insert(members.end(), fused[k].members.begin(), fused[k].members.end());
     auto is_member = [&](size_t s) { return std::find(members.begin(), members.end(), s) != members.end(); };

@@ -506,10 +506,24 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restric
       const float *all = p.partials + static_cast<size_t>(tile_id) * n_splits * 1024;
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[0][0][e] = 0.0f;
-      for (uint32_t z = 0; z < n_splits; ++z) {
+      // four splits' loads are in flight together (one round trip for up to four splits); the sums still run
+      // in split order
+      for (uint32_t z0 = 0; z0 < n_splits; z0 += 4) {
+        float part[4][16];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          acc[0][0][e] += __hip_atomic_load(all + z * 1024 + e * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (uint32_t u = 0; u < 4; ++u) {
+          const uint32_t z = z0 + u < n_splits ? z0 + u : z0;  // repeats a valid slot, ignored below
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            part[u][e] = __hip_atomic_load(all + z * 1024 + e * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+          if (z0 + u < n_splits) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[0][0][e] += part[u][e];
+          }
         }
       }
     }

@@ -23,10 +23,10 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the contraction kernel on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch, averaged over the 85 contraction launches of an inference), each scaled by what the
-# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x1.000): (4514.3 * 2.0 + 1308.3) KiB.
+# (KiB per dispatch, averaged over the 53 contraction launches of an inference), each scaled by what the
+# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x1.000): (6101.5 * 2.0 + 1397.0) KiB.
 # Only valid for the default workload (BERT-base, seq 128, 12 layers, plain_greedy, fusion on).
-MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 10_583_891
+MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 13_924_796
 
 
 def cpu_baseline(layers_total: int, sample_layers: int, seq: int):
@@ -183,6 +183,8 @@ def main():
         k["flops"] += t["flops"]
         k["launches"] += 1
         family = t["kernel"].split("+")[0]
+        if family == "MatMulKernel" and "SoftmaxKernel" in t["kernel"]:
+            family = "AttentionKernel"  # scores, softmax and context product in one launch: its own device kernel
         if family in ("TransposeKernel", "ReshapeKernel") and "+" in t["kernel"]:
             family = "ReshapeKernel"
         k = by_kernel.setdefault(family, {"ns": 0.0, "bytes": 0.0, "flops": 0.0, "launches": 0})

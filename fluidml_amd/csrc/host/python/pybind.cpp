@@ -85,6 +85,17 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
     launches.append(d);
   }
   out["launches"] = launches;
+  py::list arguments;
+  for (const worker::Argument &arg : plan.GetArguments()) {
+    py::dict d;
+    d["name"] = arg.name;
+    d["kind"] = arg.type == worker::Argument::Type::Input ? "input" : "output";
+    d["dtype"] = static_cast<int>(arg.meta.GetType());
+    d["shape"] = arg.meta.GetShape();
+    d["bytes"] = arg.meta.GetSize();
+    arguments.append(d);
+  }
+  out["arguments"] = arguments;
   return out;
 }
 

@@ -165,3 +165,21 @@ def test_profile_and_accounting(device, tiny_bert):
     mm = [t for t in times if t["kernel"].startswith("MatMulKernel")]
     assert mm and all(t["flops"] > 0 for t in mm)
     assert ex.time_replay_ns(2, 5) > 0
+
+
+def test_compiler_cli_invoke(device, tiny_bert, tmp_path, capsys):
+    """The command-line compiler with the benchmark executables' protocol (reference benchmark/bert.cpp:11-38):
+    compile once, Invoke on zero-filled inputs, report the nanoseconds Invoke returns."""
+    import json
+
+    from fluidml_amd import compiler
+
+    _, path, _, _ = tiny_bert
+    announce("compiler cli", "dp_greedy", "--invoke 3")
+    rc = compiler.main(["-n", "cli_bert", "-i", path, "-m", "dp_greedy", "-e", "2", "--json", str(tmp_path / "dp.json"),
+                        "--invoke", "3"])
+    assert rc == 0
+    summary = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert summary["mode"] == "dp_greedy" and len(summary["invoke_ns"]) == 3
+    assert all(ns > 0 for ns in summary["invoke_ns"])
+    assert (tmp_path / "dp.json").stat().st_size > 0

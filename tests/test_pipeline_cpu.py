@@ -502,3 +502,37 @@ def test_dp_on_a_branching_flow_covers_every_tensor(mods, tmp_path):
     assert all(sorted(l) == [0, 1, 2] for l in layouts.values())
     # determinism: same flow, same answer
     assert fluidml._dp_layouts(flow, "constant") == layouts
+
+
+# ------------------------------------------------------------------ command-line compiler
+
+def test_compiler_cli(mods, tmp_path, capsys, monkeypatch):
+    """Same options as the reference's executable (reference bin/compiler.cpp:13-69); --mode selects the executor
+    (the reference parses it and then ignores it), the three sinks are written, a bad mode is refused."""
+    import json
+
+    from fluidml_amd import compiler
+
+    _, models, _ = mods
+    path = models.bert_base(seq=16, layers=1, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32, seed=5).save(
+        str(tmp_path / "net.onnx"))
+    monkeypatch.setenv("FLUIDML_DP_COST", "constant")
+    plans = {}
+    for mode in compiler.ALLOWED_MODES:
+        sinks = {k: tmp_path / f"{mode}.{k}" for k in ("mlir", "llvm", "json")}
+        rc = compiler.main(["--name", "cli_" + mode, "--input", path, "--mode", mode, "--mlir", str(sinks["mlir"]),
+                            "--llvm", str(sinks["llvm"]), "--json", str(sinks["json"])])
+        assert rc == 0
+        plans[mode] = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+        assert plans[mode]["mode"] == mode and plans[mode]["steps"] > 0
+        assert sinks["mlir"].read_text() == sinks["llvm"].read_text() != ""
+        assert "cli_" + mode in sinks["mlir"].read_text()
+        kinds = [a["kind"] for a in plans[mode]["arguments"]]
+        assert kinds.count("output") == 1 and kinds.count("input") == len(kinds) - 1 >= 2
+    # the linear plan never reuses bytes, the greedy one does: the mode reached the executor
+    assert plans["plain_linear"]["arena_bytes"] > plans["plain_greedy"]["arena_bytes"]
+    assert (tmp_path / "dp_greedy.json").stat().st_size > (tmp_path / "plain_greedy.json").stat().st_size
+    with pytest.raises(SystemExit):
+        compiler.main(["-n", "x", "-i", path, "-m", "fastest"])
+    with pytest.raises(SystemExit):
+        compiler.main(["-i", path])  # --name is required, as in the reference

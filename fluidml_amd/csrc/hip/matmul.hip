@@ -140,11 +140,12 @@ struct TileLoader {
   static constexpr int kItems = ROWS * kVecsPerRow;
   static constexpr int kPerThread = (kItems + NT - 1) / NT;
 
+  // `tid`: index of the calling thread among the NT threads that share the tile
   __device__ __forceinline__ static void Load(const float *g, int row_stride, int col_stride, int rows_valid,
-                                              int cols_valid, VecF<VEC> (&regs)[kPerThread]) {
+                                              int cols_valid, VecF<VEC> (&regs)[kPerThread], int tid) {
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
-      const int item = threadIdx.x + j * NT;
+      const int item = tid + j * NT;
       const int row = item / kVecsPerRow, col = (item % kVecsPerRow) * VEC;
       if (item < kItems && row < rows_valid && col < cols_valid) {
         regs[j] = LoadVec<VEC>(g + row * row_stride + col * col_stride);
@@ -155,10 +156,10 @@ struct TileLoader {
     }
   }
 
-  __device__ __forceinline__ static void Store(float *lds, int ld, const VecF<VEC> (&regs)[kPerThread]) {
+  __device__ __forceinline__ static void Store(float *lds, int ld, const VecF<VEC> (&regs)[kPerThread], int tid) {
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
-      const int item = threadIdx.x + j * NT;
+      const int item = tid + j * NT;
       const int row = item / kVecsPerRow, col = (item % kVecsPerRow) * VEC;
       if (item < kItems) {
         if constexpr (VEC == 4) {
@@ -177,9 +178,13 @@ struct TileLoader {
 // CONV: 0 = plain contraction; 1 = B is the input of a convolution addressed through p.conv (LB must be 0), one
 // scalar gather per element; 2 = the same with one 128-bit gather per four consecutive output pixels of a row
 // (unit stride along W in the input and in the convolution, OW a multiple of 4).
+// SPEC: the workgroup has a second set of waves that only moves tiles from global memory into LDS (producers)
+// while the first set only feeds the matrix cores from LDS (consumers).  With one workgroup per compute unit
+// the plain kernel leaves each SIMD idle while its single wave waits for loads, writes LDS or sits at the
+// barrier; here the two roles overlap.
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV = 0,
-          bool BF16 = false>
-__global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restrict__ C_, const float *__restrict__ A,
+          bool BF16 = false, bool SPEC = false>
+__global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(float *__restrict__ C_, const float *__restrict__ A,
                                                                 const float *__restrict__ B_, MatmulArgs p) {
   float *__restrict__ C = C_;
   const float *__restrict__ B = B_;
@@ -198,6 +203,9 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restric
 
   constexpr int VB = CONV == 2 ? 4 : CONV == 1 ? 1 : VEC;
   static_assert(!CONV || (LB == 0 && NT % (BN / VB) == 0), "the gather keeps one output pixel (group) per thread");
+  static_assert(!SPEC || !CONV, "the gather of the convolution runs in the consumer waves");
+  const bool producer = SPEC && threadIdx.x >= NT;
+  const int ltid = producer ? static_cast<int>(threadIdx.x) - NT : static_cast<int>(threadIdx.x);
   using LoaderA = typename std::conditional<LA == 0, TileLoader<BM, BK, VEC, NT>, TileLoader<BK, BM, VEC, NT>>::type;
   using LoaderB = typename std::conditional<LB == 0, TileLoader<BK, BN, VB, NT>, TileLoader<BN, BK, VB, NT>>::type;
 
@@ -264,7 +272,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restric
   const float *Bb = CONV ? B : B + boff[2] + static_cast<int64_t>(n0) * p.sBn;
   float *Cb = C + boff[0];
 
-  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int wave = ltid / 64, lane = threadIdx.x % 64;
   const int ks = wave % KS, wn = (wave / KS) % WN, wm = wave / (KS * WN);
   const int lrow = lane % 32, half = lane / 32;
 
@@ -312,9 +320,9 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restric
   auto load_chunk = [&](int c, VecF<VEC>(&qa)[LoaderA::kPerThread], VecF<VB>(&qb)[LoaderB::kPerThread]) {
     const int k0 = c * BK, k_valid = p.K - k0;
     if constexpr (LA == 0) {
-      LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAm, p.sAk, rows_m, k_valid, qa);
+      LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAm, p.sAk, rows_m, k_valid, qa, ltid);
     } else {
-      LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAk, p.sAm, k_valid, rows_m, qa);
+      LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAk, p.sAm, k_valid, rows_m, qa, ltid);
     }
     if constexpr (CONV) {
       // same item -> (k row, n column) mapping as TileLoader<BK, BN, VB, NT>: column group = thread % (BN / VB)
@@ -353,16 +361,16 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restric
         }
       }
     } else if constexpr (LB == 0) {
-      LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBk, p.sBn, k_valid, cols_n, qb);
+      LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBk, p.sBn, k_valid, cols_n, qb, ltid);
     } else {
-      LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBn, p.sBk, cols_n, k_valid, qb);
+      LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBn, p.sBk, cols_n, k_valid, qb, ltid);
     }
   };
   auto store_chunk = [&](int buf, const VecF<VEC>(&qa)[LoaderA::kPerThread], const VecF<VB>(&qb)[LoaderB::kPerThread]) {
     float *as = lds + buf * (A_ELEMS + B_ELEMS);
     float *bs = as + A_ELEMS;
-    LoaderA::Store(as, LDA, qa);
-    LoaderB::Store(bs, LDB, qb);
+    LoaderA::Store(as, LDA, qa, ltid);
+    LoaderB::Store(bs, LDB, qb, ltid);
   };
   auto compute_chunk = [&](int buf) {
     const float *as = lds + buf * (A_ELEMS + B_ELEMS);
@@ -425,21 +433,55 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restric
   // this workgroup's share of the chunks (all of them unless K is split over blockIdx.z)
   const int c_begin = p.n_splits > 1 ? static_cast<int>(blockIdx.z) * p.chunks_per_split : 0;
   const int c_end = p.n_splits > 1 ? min(n_chunks, c_begin + p.chunks_per_split) : n_chunks;
+  if constexpr (SPEC) {
+    // Barrier j separates "chunk j is in LDS" from "chunk j is being consumed".  Producers store chunk j after
+    // barrier j-1 (the consumers are then done with chunk j-2, the previous content of that buffer); consumers
+    // compute chunk j after barrier j.  Both sides pass one barrier per chunk.
+    if (producer) {
 #pragma unroll
-  for (int s = 0; s < DEPTH; ++s) {
-    if (c_begin + s < c_end) load_chunk(c_begin + s, ra[s], rb[s]);
-  }
-  for (int c0 = c_begin; c0 < c_end; c0 += DEPTH) {
+      for (int s = 0; s < DEPTH; ++s) {
+        if (c_begin + s < c_end) load_chunk(c_begin + s, ra[s], rb[s]);
+      }
+      for (int c0 = c_begin; c0 < c_end; c0 += DEPTH) {
+#pragma unroll
+        for (int s = 0; s < DEPTH; ++s) {
+          const int c = c0 + s;
+          if (c < c_end) {  // uniform over the workgroup
+            if (c > c_begin) __syncthreads();
+            store_chunk(s & 1, ra[s], rb[s]);
+            if (c + DEPTH < c_end) load_chunk(c + DEPTH, ra[s], rb[s]);
+          }
+        }
+      }
+      __syncthreads();  // the last chunk is in LDS
+    } else {
+      for (int c0 = c_begin; c0 < c_end; c0 += DEPTH) {
+#pragma unroll
+        for (int s = 0; s < DEPTH; ++s) {
+          if (c0 + s < c_end) {
+            __syncthreads();
+            compute_chunk(s & 1);
+          }
+        }
+      }
+    }
+  } else {
 #pragma unroll
     for (int s = 0; s < DEPTH; ++s) {
-      const int c = c0 + s;
-      if (c < c_end) {  // uniform over the workgroup
-        store_chunk(s & 1, ra[s], rb[s]);
-        if (c + DEPTH < c_end) load_chunk(c + DEPTH, ra[s], rb[s]);
-        // one barrier per chunk: buffer (s&1) was last read two chunks ago, and every wave
-        // passed the previous barrier only after finishing that read
-        __syncthreads();
-        compute_chunk(s & 1);
+      if (c_begin + s < c_end) load_chunk(c_begin + s, ra[s], rb[s]);
+    }
+    for (int c0 = c_begin; c0 < c_end; c0 += DEPTH) {
+#pragma unroll
+      for (int s = 0; s < DEPTH; ++s) {
+        const int c = c0 + s;
+        if (c < c_end) {  // uniform over the workgroup
+          store_chunk(s & 1, ra[s], rb[s]);
+          if (c + DEPTH < c_end) load_chunk(c + DEPTH, ra[s], rb[s]);
+          // one barrier per chunk: buffer (s&1) was last read two chunks ago, and every wave
+          // passed the previous barrier only after finishing that read
+          __syncthreads();
+          compute_chunk(s & 1);
+        }
       }
     }
   }
@@ -447,7 +489,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restric
 
   // ---- combine the K slices of a workgroup through LDS ------------------------
   if constexpr (KS > 1) {
-    if (ks > 0) {
+    if (ks > 0 && !producer) {
       float *red = lds + (ks - 1) * BM * BN;
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -461,7 +503,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restric
           }
     }
     __syncthreads();
-    if (ks > 0) return;
+    if (ks > 0 || producer) return;
 #pragma unroll
     for (int s = 1; s < KS; ++s) {
       const float *red = lds + (s - 1) * BM * BN;
@@ -477,6 +519,8 @@ __global__ __launch_bounds__(64 * WM *WN *KS) void MatmulKernel(float *__restric
           }
     }
   }
+
+  if (producer) return;
 
   // ---- combine the K splits of a tile across workgroups ------------------------
   // Only configurations in which a wave ends up with exactly one 32x32 accumulator split (host side), and each
@@ -669,7 +713,8 @@ inline int64_t SplitKLimit(int64_t fallback) {
   return limit > 0 ? limit : fallback;
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV, bool BF16>
+template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV, bool BF16,
+          bool SPEC = false>
 void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   MatmulArgs q = p;
   q.tiles_m = (p.M + BM - 1) / BM;
@@ -697,8 +742,8 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
     }
   }
   q.n_splits = splits;
-  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV, BF16>),
-            dim3(q.tiles_m * q.tiles_n, n_batch, splits), dim3(64 * WM * WN * KS), 0, s, C, A, B, q);
+  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV, BF16, SPEC>),
+            dim3(q.tiles_m * q.tiles_n, n_batch, splits), dim3(64 * WM * WN * KS * (SPEC ? 2 : 1)), 0, s, C, A, B, q);
 }
 
 template <int LA, int LB, int VEC, int CONV, bool BF16 = false>
@@ -713,7 +758,9 @@ void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
     // with 32..104 tiles: 1.5x to 2x over the 32x32 tile)
     LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4, CONV, BF16>(p, n_batch, C, A, B, s);
   } else {
-    LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2, CONV, BF16>(p, n_batch, C, A, B, s);
+    // plain contractions run the 32x32 tile with producer and consumer waves (measured on BERT-base: 8.9 -> 8.6,
+    // 14.5 -> 13.6 and 15.9 -> 15.0 us for its three shapes); the convolution gather stays in the consumer waves
+    LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2, CONV, BF16, CONV == 0>(p, n_batch, C, A, B, s);
   }
 }
 

@@ -949,6 +949,35 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
   if (Cc > 1 && weights->strides[1] != KH * KW * s_kw) return FL_ERR_UNSUPPORTED;
   if (Numel(in) > 0x7fffffff || Numel(out) > 0x7fffffff) return FL_ERR_UNSUPPORTED;
 
+  // A 1x1 convolution with unit stride and no padding is a plain batched contraction
+  // out[img] = W[F][C] . in[img][C][H*W]: no gather, 128-bit loads of both operands, the producer/consumer tile.
+  {
+    bool pointwise = KH == 1 && KW == 1;
+    for (int d = 0; d < ns && pointwise; ++d) {
+      pointwise = (!strides || strides[d] == 1) && (!pads || (pads[d] == 0 && pads[ns + d] == 0));
+    }
+    if (pointwise && ns == 2) {
+      pointwise = in->strides[2] == in->shape[3] * in->strides[3] && out->strides[2] == out->shape[3] * out->strides[3];
+    }
+    if (pointwise) {
+      const int64_t S = OH * OW;
+      fl_tensor a{}, b{}, c{}, d{};
+      a.base = weights->base, a.dtype = FL_FLOAT32, a.rank = 2;
+      a.shape[0] = F, a.shape[1] = Cc, a.strides[0] = weights->strides[0], a.strides[1] = weights->strides[1];
+      b.base = in->base, b.dtype = FL_FLOAT32, b.rank = 3;
+      b.shape[0] = in->shape[0], b.shape[1] = Cc, b.shape[2] = S;
+      b.strides[0] = in->strides[0], b.strides[1] = in->strides[1], b.strides[2] = in->strides[wd];
+      c.base = out->base, c.dtype = FL_FLOAT32, c.rank = 3;
+      c.shape[0] = out->shape[0], c.shape[1] = F, c.shape[2] = S;
+      c.strides[0] = out->strides[0], c.strides[1] = out->strides[1], c.strides[2] = out->strides[wd];
+      if (bias != nullptr) {
+        d.base = bias->base, d.dtype = FL_FLOAT32, d.rank = 2;
+        d.shape[0] = F, d.shape[1] = S, d.strides[0] = bias->strides[0], d.strides[1] = 0;
+      }
+      return Contract(&a, &b, &c, false, false, 1.0f, 1.0f, bias != nullptr ? &d : nullptr, stream, chain);
+    }
+  }
+
   MatmulArgs p;
   std::memset(&p, 0, sizeof(p));
   p.M = static_cast<int32_t>(F);

@@ -918,6 +918,8 @@ CONV_CASES = [
     ((2, 4, 19, 17), (6, 4, 3, 5), [1, 2, 1, 2], [2, 2], [1, 1], 1, True),  # stride 2
     ((1, 6, 15, 15), (6, 1, 5, 5), [2, 2, 2, 2], [2, 2], [1, 1], 6, True),  # depthwise 5x5 stride 2
     ((1, 2, 12, 12), (3, 2, 3, 3), [2, 2, 2, 2], [1, 1], [2, 2], 1, False),  # dilation 2
+    ((2, 24, 14, 14), (40, 24, 1, 1), None, [1, 1], [1, 1], 1, True),  # pointwise 2-d, two images (plain contraction)
+    ((1, 8, 12, 12), (16, 8, 1, 1), None, [2, 2], [1, 1], 1, True),  # pointwise with stride 2 (gather path)
 ]
 
 

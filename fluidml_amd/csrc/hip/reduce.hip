@@ -380,6 +380,55 @@ __global__ __launch_bounds__(kBlock) void ReduceMeanWave(ReduceArgs a, float *__
   if (lane == 0) out[off[0]] = s / a.divisor;
 }
 
+// The reduced dims are one unit-stride run: WAVES waves per output element (1, or the 4 of a workgroup when
+// there are few outputs with long runs), 128-bit loads where the run starts on a 16-byte boundary, four
+// independent partial sums per lane.
+template <int WAVES>
+__global__ __launch_bounds__(kBlock) void ReduceMeanRun(ReduceArgs a, float *__restrict__ out,
+                                                        const float *__restrict__ in) {
+  __shared__ float part[kBlock / kWave];
+  const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const uint32_t o = WAVES == 1 ? blockIdx.x * (kBlock / kWave) + wave : blockIdx.x;
+  const bool active = o < a.n_out;
+  int32_t off[2] = {0, 0};
+  if (active) RowOffsets<2>(a.outer, o, off);
+  const float *src = in + off[1];
+  const uint32_t t = WAVES == 1 ? lane : threadIdx.x, nt = WAVES * kWave;
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  if (active) {
+    uint32_t head = static_cast<uint32_t>((16 - (reinterpret_cast<uintptr_t>(src) & 15)) & 15) / 4;  // elements up to the boundary
+    if (head > a.n_red) head = a.n_red;
+    if (t < head) s0 += src[t];
+    const uint32_t n4 = (a.n_red - head) / 4;
+    const float *body = src + head;
+    uint32_t j = t;
+    for (; j + 3 * nt < n4; j += 4 * nt) {
+      const float4 v0 = *reinterpret_cast<const float4 *>(body + 4 * j);
+      const float4 v1 = *reinterpret_cast<const float4 *>(body + 4 * (j + nt));
+      const float4 v2 = *reinterpret_cast<const float4 *>(body + 4 * (j + 2 * nt));
+      const float4 v3 = *reinterpret_cast<const float4 *>(body + 4 * (j + 3 * nt));
+      s0 += (v0.x + v0.y) + (v0.z + v0.w);
+      s1 += (v1.x + v1.y) + (v1.z + v1.w);
+      s2 += (v2.x + v2.y) + (v2.z + v2.w);
+      s3 += (v3.x + v3.y) + (v3.z + v3.w);
+    }
+    for (; j < n4; j += nt) {
+      const float4 v = *reinterpret_cast<const float4 *>(body + 4 * j);
+      s0 += (v.x + v.y) + (v.z + v.w);
+    }
+    const uint32_t tail = head + 4 * n4;
+    if (tail + t < a.n_red) s1 += src[tail + t];
+  }
+  float s = WaveReduce((s0 + s1) + (s2 + s3), SumOp{});
+  if constexpr (WAVES == 1) {
+    if (active && lane == 0) out[off[0]] = s / a.divisor;
+  } else {
+    if (lane == 0) part[wave] = s;
+    __syncthreads();
+    if (threadIdx.x == 0 && active) out[off[0]] = (((part[0] + part[1]) + part[2]) + part[3]) / a.divisor;
+  }
+}
+
 // One lane per output element.
 __global__ __launch_bounds__(kBlock) void ReduceMeanThread(ReduceArgs a, float *__restrict__ out,
                                                            const float *__restrict__ in) {
@@ -611,7 +660,13 @@ int fluidml_hip_reduce_mean(const fl_tensor *in, const fl_tensor *out, const int
   const float *x = static_cast<const float *>(in->base);
   hipStream_t s = AsStream(stream);
   const bool inner_contig = inner.strides[0][inner.rank - 1] == 1;
-  if ((inner_contig && n_red >= 32) || n_out < 1024) {
+  if (inner.rank == 1 && inner_contig && n_red >= 64) {
+    if (n_out <= 512 && n_red >= 1024) {
+      FL_LAUNCH(ReduceMeanRun<kBlock / kWave>, dim3(a.n_out), dim3(kBlock), 0, s, a, o, x);
+    } else {
+      FL_LAUNCH(ReduceMeanRun<1>, dim3((a.n_out + kBlock / kWave - 1) / (kBlock / kWave)), dim3(kBlock), 0, s, a, o, x);
+    }
+  } else if ((inner_contig && n_red >= 32) || n_out < 1024) {
     FL_LAUNCH(ReduceMeanWave, dim3((a.n_out + kBlock / kWave - 1) / (kBlock / kWave)), dim3(kBlock), 0, s, a, o,
                        x);
   } else {

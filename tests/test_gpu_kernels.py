@@ -443,7 +443,10 @@ def test_layer_norm(device, shape, axis, eps):
 def test_reduce_mean(device):
     cabi = _cabi()
     rng = np.random.default_rng(41)
-    for shape, axes in [((1, 32, 14, 14), [2, 3]), ((1, 128, 768), [2]), ((3, 4, 5), [0]), ((2, 6, 5, 3), [1, 3])]:
+    # the last three: long unit-stride runs (a workgroup per output), runs that start off a 16-byte boundary
+    # (169 elements per channel), and many short runs
+    for shape, axes in [((1, 32, 14, 14), [2, 3]), ((1, 128, 768), [2]), ((3, 4, 5), [0]), ((2, 6, 5, 3), [1, 3]),
+                        ((1, 32, 112, 112), [2, 3]), ((1, 96, 13, 13), [2, 3]), ((2, 600, 9, 9), [2, 3])]:
         x = rand(rng, shape)
         oshape = tuple(1 if i in axes else s for i, s in enumerate(shape))
         for lin in some_layouts(len(shape), rng, 3):

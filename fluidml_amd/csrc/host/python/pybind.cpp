@@ -76,7 +76,16 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
     d["members"] = l.members;
     // members whose output tensor the launch writes (the rest are elided intermediates)
     std::vector<size_t> written;
-    if (l.group.empty()) written.push_back(l.members.back());
+    if (l.kind == worker::Launch::Kind::View) {
+      // nothing runs and nothing is written: the readers address `source` (bytes of another tensor) instead
+      py::dict src = OperandOf(l.out);
+      src["bytes"] = l.out.Extent();
+      src["view_offset"] = l.out.view_offset;
+      src["view_strides"] = l.out.view_strides;
+      d["source"] = src;
+    } else if (l.group.empty()) {
+      written.push_back(l.members.back());
+    }
     for (const worker::Launch &m : l.group) written.push_back(m.members.back());
     d["written"] = written;
     d["position"] = l.group.empty() ? l.members.back() : l.position;

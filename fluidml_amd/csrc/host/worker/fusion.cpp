@@ -27,6 +27,7 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::Attention: return "Attention";
     case Launch::Kind::AddLayerNorm: return "AddLayerNormalization";
     case Launch::Kind::ReshapeTranspose: return "ReshapeTranspose";
+    case Launch::Kind::View: return "View";
     default: return "TransposeReshape";
   }
 }
@@ -43,7 +44,7 @@ bool Elidable(const Operand &o) { return o.space == Operand::Space::Arena || o.s
 bool Alias(const Operand &x, const Operand &y) {
   if (x.space != y.space) return false;
   if (x.space != Operand::Space::Arena) return x.name == y.name;
-  const size_t x1 = x.offset + x.meta.GetSize(), y1 = y.offset + y.meta.GetSize();
+  const size_t x1 = x.offset + x.Extent(), y1 = y.offset + y.Extent();
   return x.offset < y1 && y.offset < x1;
 }
 
@@ -163,6 +164,36 @@ class ViewTracker {
     return v;
   }
 
+  // The other direction: element strides of the current dims inside the source tensor stored with
+  // `source_strides`; nullopt if a current dim is not one strided run of the source.
+  std::optional<std::vector<int64_t>> StridesInSource(const std::vector<int64_t> &source_strides) const {
+    if (source_strides.size() != n_source_dims_) return std::nullopt;
+    std::vector<int64_t> atom_stride(atoms_.size(), 0);
+    for (size_t d = 0; d < n_source_dims_; ++d) {
+      std::vector<int> chain;  // atoms of source dim d, outermost first
+      for (int a = static_cast<int>(d); a >= 0;) {
+        chain.push_back(a);
+        auto it = inner_of_.find(a);
+        a = it == inner_of_.end() ? -1 : it->second;
+      }
+      int64_t run = source_strides[d];
+      for (size_t k = chain.size(); k-- > 0;) {
+        atom_stride[chain[k]] = run;
+        run *= atoms_[chain[k]].extent;
+      }
+    }
+    std::vector<int64_t> out;
+    for (const auto &dim : dims_) {
+      int64_t stride = 0;
+      for (size_t k = 0; k < dim.size(); ++k) {
+        if (k + 1 < dim.size() && atom_stride[dim[k]] != atom_stride[dim[k + 1]] * atoms_[dim[k + 1]].extent) return std::nullopt;
+        stride = atom_stride[dim[k]];
+      }
+      out.push_back(stride);  // 0 for a unit dim
+    }
+    return out;
+  }
+
  private:
   struct Atom {
     int source_dim;
@@ -176,12 +207,9 @@ class ViewTracker {
 
 class Scheduler {
  public:
-  Scheduler(const std::vector<Step> &steps) : steps_(steps), taken_(steps.size(), false) {
-    for (size_t i = 0; i < steps_.size(); ++i) {
-      const Step &s = steps_[i];
-      readers_[s.in0.name].push_back(i);
-      if (s.node->IsDoubleInputs() && !SameTensor(s.in0, s.in1)) readers_[s.in1.name].push_back(i);
-    }
+  Scheduler(const std::vector<Step> &steps)
+      : steps_(steps), taken_(steps.size(), false), elided_(steps.size(), false), rewired_(steps.size(), false) {
+    BuildReaders();
   }
 
   std::vector<Launch> Run(bool fuse) {
@@ -220,6 +248,7 @@ class Scheduler {
       }
     }
     if (fuse) GroupSiblings(&fused);
+    if (fuse) ElideViews(&fused);
     // a chain is issued where its last member stood; everything else keeps its place
     std::vector<const Launch *> at(steps_.size(), nullptr);
     for (const Launch &l : fused) at[l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back()] = &l;
@@ -227,11 +256,22 @@ class Scheduler {
     for (size_t i = 0; i < steps_.size(); ++i) {
       if (at[i] != nullptr) {
         schedule.push_back(*at[i]);
+      } else if (elided_[i]) {
+        Launch l;
+        l.kind = Launch::Kind::View;
+        l.members = {i};
+        l.out = steps_[i].out;  // rewritten: the source seen as this step's output
+        schedule.push_back(std::move(l));
       } else if (!taken_[i]) {
         Launch l;
         l.members = {i};
         l.bytes = steps_[i].bytes;
         l.flops = steps_[i].flops;
+        if (rewired_[i]) {
+          l.rewired = true;
+          l.a = steps_[i].in0;
+          l.b = steps_[i].in1;
+        }
         schedule.push_back(std::move(l));
       }
     }
@@ -239,6 +279,210 @@ class Scheduler {
   }
 
  private:
+  void BuildReaders() {
+    readers_.clear();
+    for (size_t i = 0; i < steps_.size(); ++i) {
+      const Step &s = steps_[i];
+      readers_[s.in0.name].push_back(i);
+      if (s.node->IsDoubleInputs() && !SameTensor(s.in0, s.in1)) readers_[s.in1.name].push_back(i);
+    }
+  }
+
+  // ---- view elision -----------------------------------------------------------------------------------
+  // A Slice, Transpose, Squeeze, Unsqueeze or (where the result is still one strided pattern) Reshape / Flatten
+  // that no fusion has absorbed does not have to run: every kernel here takes element strides, so the readers
+  // can address the step's input directly.  Allowed when the tensor is internal, and the bytes of the input stay
+  // untouched from the step's position to the position where each reader is issued (the input may be dead in
+  // the memory plan by then, and its bytes reused).
+
+  static std::vector<int64_t> LogicalStrides(const Operand &op) {
+    if (op.viewed) return op.view_strides;
+    return utils::GenStrides(op.meta.GetShape(), op.layout);
+  }
+
+  // step i's output as a view of its input: (element offset, strides per output dim)
+  std::optional<std::pair<int64_t, std::vector<int64_t>>> AsView(size_t i) const {
+    const Step &s = steps_[i];
+    const std::vector<int64_t> st = LogicalStrides(s.in0);
+    const auto &ishape = s.in0.meta.GetShape();
+    const auto &oshape = s.out.meta.GetShape();
+    const int64_t irank = static_cast<int64_t>(ishape.size()), orank = static_cast<int64_t>(oshape.size());
+    if (s.in0.meta.GetType() != s.out.meta.GetType()) return std::nullopt;
+    int64_t offset = s.in0.viewed ? s.in0.view_offset : 0;
+    std::vector<int64_t> strides;
+    const flow::Attrs &at = Attrs(i);
+    switch (Kind(i)) {
+      case OpKind::Transpose: {
+        if (irank != orank) return std::nullopt;
+        std::vector<bool> seen(static_cast<size_t>(irank), false);
+        for (int64_t k = 0; k < orank; ++k) {
+          const int64_t p = at.perm.empty() ? irank - 1 - k : at.perm[static_cast<size_t>(k)];
+          if (p < 0 || p >= irank || seen[static_cast<size_t>(p)] || oshape[static_cast<size_t>(k)] != ishape[static_cast<size_t>(p)]) return std::nullopt;
+          seen[static_cast<size_t>(p)] = true;
+          strides.push_back(st[static_cast<size_t>(p)]);
+        }
+        break;
+      }
+      case OpKind::Slice: {
+        if (irank != orank || at.starts.size() != at.axes.size() || at.steps.size() != at.axes.size()) return std::nullopt;
+        std::vector<int64_t> start(static_cast<size_t>(irank), 0), step(static_cast<size_t>(irank), 1);
+        for (size_t n = 0; n < at.axes.size(); ++n) {
+          int64_t ax = at.axes[n] < 0 ? at.axes[n] + irank : at.axes[n];
+          if (ax < 0 || ax >= irank) return std::nullopt;
+          int64_t b = at.starts[n];
+          if (b < 0) b += ishape[static_cast<size_t>(ax)];
+          if (b < 0 || at.steps[n] <= 0) return std::nullopt;
+          start[static_cast<size_t>(ax)] = b;
+          step[static_cast<size_t>(ax)] = at.steps[n];
+        }
+        for (size_t d = 0; d < static_cast<size_t>(irank); ++d) {
+          if (start[d] + (oshape[d] - 1) * step[d] >= ishape[d]) return std::nullopt;
+          offset += start[d] * st[d];
+          strides.push_back(st[d] * step[d]);
+        }
+        break;
+      }
+      case OpKind::Squeeze: {
+        if (irank != orank + static_cast<int64_t>(at.axes.size())) return std::nullopt;
+        size_t j = 0;
+        for (int64_t d = 0; d < irank; ++d) {
+          bool squeezed = false;
+          for (int64_t ax : at.axes) squeezed = squeezed || (ax < 0 ? ax + irank : ax) == d;
+          if (squeezed) {
+            if (ishape[static_cast<size_t>(d)] != 1) return std::nullopt;
+          } else {
+            if (j >= oshape.size() || oshape[j] != ishape[static_cast<size_t>(d)]) return std::nullopt;
+            strides.push_back(st[static_cast<size_t>(d)]);
+            ++j;
+          }
+        }
+        if (j != oshape.size()) return std::nullopt;
+        break;
+      }
+      case OpKind::Unsqueeze: {
+        if (irank + static_cast<int64_t>(at.axes.size()) != orank) return std::nullopt;
+        size_t j = 0;
+        for (int64_t d = 0; d < orank; ++d) {
+          bool added = false;
+          for (int64_t ax : at.axes) added = added || (ax < 0 ? ax + orank : ax) == d;
+          if (added) {
+            if (oshape[static_cast<size_t>(d)] != 1) return std::nullopt;
+            strides.push_back(0);
+          } else {
+            if (j >= ishape.size() || ishape[j] != oshape[static_cast<size_t>(d)]) return std::nullopt;
+            strides.push_back(st[j++]);
+          }
+        }
+        if (j != ishape.size()) return std::nullopt;
+        break;
+      }
+      case OpKind::Reshape:
+      case OpKind::Flatten: {
+        ViewTracker tracker(ishape);
+        if (!tracker.Reshape(oshape)) return std::nullopt;
+        const auto v = tracker.StridesInSource(st);
+        if (!v || v->size() != oshape.size()) return std::nullopt;
+        strides = *v;
+        break;
+      }
+      default: return std::nullopt;
+    }
+    if (offset < 0 || offset > INT32_MAX) return std::nullopt;
+    return std::make_pair(offset, strides);
+  }
+
+  void ElideViews(std::vector<Launch> *fused) {
+    // where each step is issued: a fused launch runs at one position for all its members
+    std::vector<size_t> issued(steps_.size());
+    std::vector<const Launch *> owner(steps_.size(), nullptr);
+    for (size_t i = 0; i < steps_.size(); ++i) issued[i] = i;
+    for (const Launch &l : *fused) {
+      const size_t pos = l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back();
+      for (size_t m : l.members) {
+        issued[m] = pos;
+        owner[m] = &l;
+      }
+    }
+    // every write of the schedule: (position, bytes, launch it belongs to)
+    struct Write {
+      size_t position;
+      Operand what;
+      const Launch *launch;  // null for a single step
+      size_t step;           // the single step
+    };
+    std::vector<Write> writes;
+    for (size_t q = 0; q < steps_.size(); ++q) {
+      if (owner[q] == nullptr) writes.push_back({q, steps_[q].out, nullptr, q});
+    }
+    for (const Launch &l : *fused) {
+      const size_t pos = l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back();
+      if (l.group.empty()) writes.push_back({pos, l.out, &l, 0});
+      for (const Launch &g : l.group) writes.push_back({pos, g.out, &l, 0});
+    }
+    for (size_t i = 0; i < steps_.size(); ++i) {
+      if (taken_[i] || !Elidable(steps_[i].out) || !steps_[i].node->IsSingleInput()) continue;
+      const auto view = AsView(i);
+      if (!view) continue;
+      const Step &s = steps_[i];
+      auto it = readers_.find(s.out.name);
+      if (it == readers_.end() || it->second.empty()) continue;
+      // the source operand: the step's input, or what that input is itself a view of
+      Operand seen = s.out;  // keeps the view's meta (shape, type)
+      seen.space = s.in0.space;
+      seen.name = s.in0.name;
+      seen.offset = s.in0.offset;
+      seen.viewed = true;
+      seen.view_offset = view->first;
+      seen.view_strides = view->second;
+      seen.source_bytes = s.in0.Extent();
+      bool ok = true;
+      for (size_t r : it->second) {
+        if (r <= i) ok = false;
+        const size_t pos = issued[r];
+        if (pos < i) ok = false;  // the reader was hoisted in front of the view step: keep the copy
+        for (const Write &w : writes) {
+          // nothing may write the source's bytes after the view step and before the reader runs, and the
+          // reader's own launch must not write what it now reads through the view
+          const bool own = w.launch != nullptr ? w.launch == owner[r] : (owner[r] == nullptr && w.step == r);
+          if (w.launch == nullptr && elided_[w.step]) continue;
+          if (((w.position > i && w.position < pos) || own) && Alias(w.what, seen)) ok = false;
+        }
+        for (size_t q = i + 1; q < pos && ok; ++q) {
+          // scratch reserved by a step in between (these kernels do not touch it, but it is not ours to read under)
+          const Step &between = steps_[q];
+          if (between.has_buffer && seen.space == Operand::Space::Arena && between.buffer_offset < seen.offset + seen.Extent() &&
+              seen.offset < between.buffer_offset + between.buffer_bytes) {
+            ok = false;
+          }
+        }
+        if (!ok) break;
+      }
+      if (!ok) continue;
+      // rewrite every reader: the plan's steps (for later views of this view and for single-step launches) and
+      // the operand copies inside fused launches
+      const Operand produced = s.out;
+      for (size_t r : it->second) {
+        if (SameTensor(steps_[r].in0, produced)) steps_[r].in0 = seen;
+        if (steps_[r].node->IsDoubleInputs() && SameTensor(steps_[r].in1, produced)) steps_[r].in1 = seen;
+        rewired_[r] = true;
+      }
+      for (Launch &l : *fused) {
+        for (Operand *op : {&l.a, &l.b, &l.c, &l.d}) {
+          if (SameTensor(*op, produced) && !op->viewed) *op = seen;
+        }
+        for (Launch &g : l.group) {
+          for (Operand *op : {&g.a, &g.b, &g.c, &g.d}) {
+            if (SameTensor(*op, produced) && !op->viewed) *op = seen;
+          }
+        }
+      }
+      steps_[i].out = seen;
+      elided_[i] = true;
+      taken_[i] = true;
+      BuildReaders();  // names changed: the source gained this step's readers
+    }
+  }
+
   OpKind Kind(size_t i) const { return steps_[i].node->GetKind(); }
   const flow::Attrs &Attrs(size_t i) const { return steps_[i].node->GetAttrs(); }
 
@@ -814,8 +1058,8 @@ class Scheduler {
     return l;
   }
 
-  const std::vector<Step> &steps_;
-  std::vector<bool> taken_;
+  std::vector<Step> steps_;  // own copy: view elision rewrites the inputs of the readers
+  std::vector<bool> taken_, elided_, rewired_;
   std::unordered_map<std::string, std::vector<size_t>> readers_;
 };
 

@@ -15,7 +15,12 @@ void Check(int rc, const char *what) {
   if (rc != 0) throw std::runtime_error(std::string(what) + ": " + fluidml_hip_error_string(rc));
 }
 
-kernel::TensorView ViewOf(void *base, const Operand &op) { return kernel::TensorView(base, op.meta, op.layout); }
+kernel::TensorView ViewOf(void *base, const Operand &op) {
+  if (!op.viewed) return kernel::TensorView(base, op.meta, op.layout);
+  kernel::TensorView v(static_cast<char *>(base) + op.view_offset * static_cast<int64_t>(GetSize(op.meta.GetType())), op.meta);
+  for (size_t d = 0; d < op.view_strides.size(); ++d) v.t.strides[d] = op.view_strides[d];
+  return v;
+}
 
 const char *SpaceName(Operand::Space s) {
   switch (s) {
@@ -172,15 +177,18 @@ const std::vector<Launch> &LaunchPlan::GetSchedule() const {
   return schedule_;
 }
 
-void LaunchPlan::IssueStep(kernel::LaunchContext &ctx, const Step &s) const {
-  const kernel::TensorView in0 = ViewOf(Resolve(s.in0), s.in0), out = ViewOf(Resolve(s.out), s.out);
+void LaunchPlan::IssueStep(kernel::LaunchContext &ctx, const Step &s, const Operand *in0_view,
+                           const Operand *in1_view) const {
+  const Operand &op0 = in0_view ? *in0_view : s.in0;
+  const kernel::TensorView in0 = ViewOf(Resolve(op0), op0), out = ViewOf(Resolve(s.out), s.out);
   const kernel::Buffer buffer{s.has_buffer ? static_cast<char *>(arena_) + s.buffer_offset : nullptr, s.buffer_bytes};
   kernel::Kernel *k = s.kernel.get();
   if (s.node->IsSingleInput()) {
     if (s.has_buffer) dynamic_cast<kernel::SingleInputWithBufferKernel &>(*k).Run(ctx, in0, out, buffer);
     else dynamic_cast<kernel::SingleInputWithoutBufferKernel &>(*k).Run(ctx, in0, out);
   } else {
-    const kernel::TensorView in1 = ViewOf(Resolve(s.in1), s.in1);
+    const Operand &op1 = in1_view ? *in1_view : s.in1;
+    const kernel::TensorView in1 = ViewOf(Resolve(op1), op1);
     if (s.has_buffer) dynamic_cast<kernel::DoubleInputsWithBufferKernel &>(*k).Run(ctx, in0, in1, out, buffer);
     else dynamic_cast<kernel::DoubleInputsWithoutBufferKernel &>(*k).Run(ctx, in0, in1, out);
   }
@@ -209,8 +217,9 @@ fl_tensor Permuted(const fl_tensor &t, const std::vector<int64_t> &perm, bool in
 }  // namespace
 
 void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
+  if (l.kind == Launch::Kind::View) return;  // nothing runs: the readers address the source
   if (l.kind == Launch::Kind::Step) {
-    IssueStep(ctx, steps_[l.members[0]]);
+    IssueStep(ctx, steps_[l.members[0]], l.rewired ? &l.a : nullptr, l.rewired ? &l.b : nullptr);
     return;
   }
   const kernel::TensorView a = ViewOf(Resolve(l.a), l.a), out = ViewOf(Resolve(l.out), l.out);
@@ -464,6 +473,7 @@ std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
   for (size_t it = 0; it < warmup + iters; ++it) {
     try {
       for (size_t i = 0; i < schedule.size(); ++i) {
+        if (schedule[i].kind == Launch::Kind::View) continue;
         Check(fluidml_hip_time_kernels(events[2 * i], events[2 * i + 1]), "kernel timing on");
         Issue(ctx, schedule[i]);
       }
@@ -475,6 +485,7 @@ std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
     Check(fluidml_hip_stream_synchronize(stream_), "profiling sync");
     if (it >= warmup) {
       for (size_t i = 0; i < schedule.size(); ++i) {
+        if (schedule[i].kind == Launch::Kind::View) continue;
         double ns = 0;
         Check(fluidml_hip_event_elapsed_ns(events[2 * i], events[2 * i + 1], &ns), "event elapsed");
         samples[i].push_back(ns);
@@ -487,6 +498,7 @@ std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
     std::vector<double> &v = samples[i];
     std::sort(v.begin(), v.end());
     const Launch &l = schedule[i];
+    if (l.kind == Launch::Kind::View) continue;  // not a launch
     StepTime t;
     for (size_t m : l.members) {
       t.node += (t.node.empty() ? "" : "+") + steps_[m].node->GetName();

@@ -32,6 +32,16 @@ struct Operand {
   size_t offset = 0;  // Arena only
   Meta meta{Type::kUnknown, std::vector<int64_t>{}};
   std::vector<size_t> layout;
+  // A tensor that is not materialised but read through the bytes of another one (the output of an elided
+  // Slice / Transpose / Squeeze / Unsqueeze / Reshape): `space`, `name` and `offset` are then the source's,
+  // `meta` stays the view's own, and the view's logical element (i0, i1, ...) lives `view_offset +
+  // sum(i_d * view_strides[d])` elements into the source, whose whole extent is `source_bytes`.
+  bool viewed = false;
+  int64_t view_offset = 0;
+  std::vector<int64_t> view_strides;
+  size_t source_bytes = 0;
+  // bytes the operand may touch (its own, or its source's when it is a view)
+  size_t Extent() const { return viewed ? source_bytes : meta.GetSize(); }
 };
 
 struct Step {
@@ -62,7 +72,9 @@ struct Launch {
     Attention,         // MatMul -> Div|Mul constant [-> AddCommon(mask)] [-> Where(cond, x, scalar)] -> Softmax -> MatMul
     AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias
     ReshapeTranspose,  // Reshape -> Transpose, one strided copy
-    TransposeReshape   // Transpose -> Reshape, one strided copy
+    TransposeReshape,  // Transpose -> Reshape, one strided copy
+    View               // a Slice / Transpose / Squeeze / Unsqueeze / Reshape that is not run: its readers address
+                       // the source through strides (members = {i}, out = the source operand seen as the view)
   };
   Kind kind = Kind::Step;
   std::vector<size_t> members;  // indices into the step list, ascending
@@ -74,6 +86,8 @@ struct Launch {
   // Attention: a = queries, b = keys (transposed), c = values, d = additive mask (has_mask), the Where step
   // `owner` holds the condition (has_cond) and s1 its fill value; s0 scales the scores, dividing if `divisor`
   bool has_mask = false, has_cond = false, divisor = false;
+  // Step: the step's inputs, when one of them became a view of another tensor (rewired), replace the plan's
+  bool rewired = false;
   // MatMulChain followed by Reshape/Transpose steps that only re-address the result: element strides of the
   // contraction's logical output dims inside `out` (empty: `out` is the contraction's own output tensor),
   // and the optional split of the last dim (see fluidml_hip_matmul_chain_view)
@@ -175,7 +189,8 @@ class LaunchPlan {
     void *device = nullptr;
   };
   void *Resolve(const Operand &op) const;
-  void IssueStep(kernel::LaunchContext &ctx, const Step &s) const;
+  void IssueStep(kernel::LaunchContext &ctx, const Step &s, const Operand *in0_view = nullptr,
+                 const Operand *in1_view = nullptr) const;
   void Issue(kernel::LaunchContext &ctx, const Launch &l) const;
   void LaunchAll(kernel::LaunchContext &ctx) const;
   void Replay(kernel::LaunchContext &ctx);

@@ -377,10 +377,48 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     for i, s in enumerate(steps):
         for op in s["inputs"]:
             readers.setdefault(op["name"], set()).add(i)
+    issued = {}
+    for l in launches:
+        for m in l["members"]:
+            issued[m] = (l["position"], l)
+    # A step that is not run (kind "View"): its readers address `source`, the bytes of another tensor, when
+    # they are issued.  Everything that writes between the view step and such a reader -- outputs of single
+    # steps at their own position, outputs of fused launches at the launch's position -- must stay off those
+    # bytes, and so must the reader's own launch.
+    elided = {l["members"][0] for l in launches if l["kind"] == "View"}
+    writes = []  # (position, operand, launch id)
+    for k, l in enumerate(launches):
+        if l["kind"] != "View":
+            writes += [(l["position"], steps[m]["out"], k) for m in l["written"]]
+    for l in launches:
+        if l["kind"] != "View":
+            continue
+        (i,) = l["members"]
+        assert l["written"] == [] and steps[i]["out"]["space"] in ("arena", "private")
+        src = l["source"]
+        # a view of a view reads through to a tensor that is materialised
+        assert all(steps[j]["out"]["name"] != src["name"] for j in elided), "the source of a view is itself not run"
+        pending = list(readers.get(steps[i]["out"]["name"], ()))
+        seen = set()
+        while pending:
+            r = pending.pop()
+            if r in seen:
+                continue
+            seen.add(r)
+            assert r > i
+            if r in elided:  # reads through: its own readers are the ones that touch the bytes
+                pending += list(readers.get(steps[r]["out"]["name"], ()))
+                continue
+            pos, owner = issued[r]
+            assert pos >= i, "a reader of an elided view was hoisted in front of it"
+            for wpos, what, k in writes:
+                own = launches[k] is owner
+                if (i < wpos < pos) or own:
+                    assert not _overlap(what, src), "the source of an elided view is overwritten before a reader runs"
     for l in launches:
         members = l["members"]
         assert members == sorted(members)
-        if l["kind"] == "Step":
+        if l["kind"] in ("Step", "View"):
             assert len(members) == 1
             continue
         written = set(l["written"])

@@ -675,12 +675,19 @@ class Scheduler {
     // MatMul only: trailing Reshape / Transpose steps that merely re-address the result are folded into the
     // kernel's output strides (the head split and merge copies of an attention block)
     if (l.kind == Launch::Kind::MatMulChain) {
-      Launch with_views = l;
-      if (AppendViews(i, &with_views) && with_views.members.size() >= 2 &&
-          Safe(with_views.members, {{i, l.a}, {i, l.b}}) && OutputDisjoint(with_views.out, {&l.a, &l.b})) {
-        with_views.bytes = l.has_c ? Bytes({&l.a, &l.b, &l.c, &with_views.out}) : Bytes({&l.a, &l.b, &with_views.out});
-        with_views.flops = Flops(with_views.members);
-        return with_views;
+      // the longest run of view steps whose target buffer is safe to write from here; a shorter run leaves the
+      // rest to the view elision (a Reshape of what the kernel wrote is then read in place)
+      for (size_t limit = SIZE_MAX; limit > 0;) {
+        Launch with_views = l;
+        const size_t taken = AppendViews(i, &with_views, limit);
+        if (taken == 0) break;
+        if (with_views.members.size() >= 2 && Safe(with_views.members, {{i, l.a}, {i, l.b}}) &&
+            OutputDisjoint(with_views.out, {&l.a, &l.b})) {
+          with_views.bytes = l.has_c ? Bytes({&l.a, &l.b, &l.c, &with_views.out}) : Bytes({&l.a, &l.b, &with_views.out});
+          with_views.flops = Flops(with_views.members);
+          return with_views;
+        }
+        limit = taken - 1;
       }
     }
     // longest variant whose late reads are safe: with the chain, then without it
@@ -701,13 +708,14 @@ class Scheduler {
 
   // Extends `l` (a MatMulChain headed by step `head`) by the longest run of single-reader Reshape / Transpose
   // steps after which the contraction's logical output is still a strided view of the final tensor.
-  bool AppendViews(size_t head, Launch *l) const {
+  // At most `limit` view steps are taken; returns how many were (0: none).
+  size_t AppendViews(size_t head, Launch *l, size_t limit = SIZE_MAX) const {
     ViewTracker tracker(steps_[head].out.meta.GetShape());
     size_t cur = l->members.back();
     std::vector<size_t> views;
     size_t best = 0;
     ViewTracker::View best_view;
-    while (true) {
+    while (views.size() < limit) {
       const auto j = SoleReader(cur);
       if (!j || !IsFloat(steps_[*j].out)) break;
       bool ok = false;
@@ -735,13 +743,13 @@ class Scheduler {
         best_view = *v;
       }
     }
-    if (best == 0) return false;
+    if (best == 0) return 0;
     l->members.insert(l->members.end(), views.begin(), views.begin() + static_cast<std::ptrdiff_t>(best));
     l->out = steps_[l->members.back()].out;
     l->view_strides = best_view.strides;
     l->n_inner = best_view.n_inner;
     l->stride_outer = best_view.stride_outer;
-    return true;
+    return best;
   }
 
   // MatMulChains that read the same left operand with the same extents (the query / key / value projections)
@@ -1016,8 +1024,13 @@ class Scheduler {
       x->flops = Flops(x->members);
       return true;
     };
-    Launch with_views = l;
-    if (AppendViews(pv, &with_views) && with_views.n_inner == 0 && finish(&with_views)) return with_views;
+    for (size_t limit = SIZE_MAX; limit > 0;) {
+      Launch with_views = l;
+      const size_t taken = AppendViews(pv, &with_views, limit);
+      if (taken == 0) break;
+      if (with_views.n_inner == 0 && finish(&with_views)) return with_views;
+      limit = taken - 1;
+    }
     l.out = steps_[pv].out;
     if (finish(&l)) return l;
     return std::nullopt;

@@ -23,10 +23,10 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the contraction kernel on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch, averaged over the 53 contraction launches of an inference), each scaled by what the
-# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x1.000): (6101.5 * 2.0 + 1397.0) KiB.
+# (KiB per dispatch, averaged over the 51 contraction launches of an inference), each scaled by what the
+# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x1.000): (6279.6 * 2.0 + 1429.2) KiB.
 # Only valid for the default workload (BERT-base, seq 128, 12 layers, plain_greedy, fusion on).
-MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 13_924_796
+MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 14_322_469
 
 
 def cpu_baseline(layers_total: int, sample_layers: int, seq: int):

@@ -83,8 +83,16 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
       src["view_offset"] = l.out.view_offset;
       src["view_strides"] = l.out.view_strides;
       d["source"] = src;
+    } else if (l.kind == worker::Launch::Kind::Placed) {
+      // a Concat2 whose inputs were written in place: nothing runs
     } else if (l.group.empty()) {
       written.push_back(l.members.back());
+    }
+    // a launch that writes into a part of another tensor (an input of a Concat2 placed in its output)
+    if (l.kind != worker::Launch::Kind::View && l.out.viewed) {
+      py::dict into = OperandOf(l.out);
+      into["bytes"] = l.out.Extent();
+      d["writes_into"] = into;
     }
     for (const worker::Launch &m : l.group) written.push_back(m.members.back());
     d["written"] = written;

@@ -28,6 +28,8 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::AddLayerNorm: return "AddLayerNormalization";
     case Launch::Kind::ReshapeTranspose: return "ReshapeTranspose";
     case Launch::Kind::View: return "View";
+    case Launch::Kind::Placed: return "Placed";
+    case Launch::Kind::CopyInto: return "CopyInto";
     default: return "TransposeReshape";
   }
 }
@@ -208,7 +210,8 @@ class ViewTracker {
 class Scheduler {
  public:
   Scheduler(const std::vector<Step> &steps)
-      : steps_(steps), taken_(steps.size(), false), elided_(steps.size(), false), rewired_(steps.size(), false) {
+      : steps_(steps), taken_(steps.size(), false), elided_(steps.size(), false), rewired_(steps.size(), false),
+        placed_(steps.size(), 0) {
     BuildReaders();
   }
 
@@ -249,6 +252,7 @@ class Scheduler {
     }
     if (fuse) GroupSiblings(&fused);
     if (fuse) ElideViews(&fused);
+    if (fuse) PlaceConcatInputs(&fused);
     // a chain is issued where its last member stood; everything else keeps its place
     std::vector<const Launch *> at(steps_.size(), nullptr);
     for (const Launch &l : fused) at[l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back()] = &l;
@@ -262,6 +266,21 @@ class Scheduler {
         l.members = {i};
         l.out = steps_[i].out;  // rewritten: the source seen as this step's output
         schedule.push_back(std::move(l));
+      } else if (placed_[i] != 0) {
+        // a Concat2 with one or both inputs already in place
+        Launch l;
+        l.members = {i};
+        if (placed_[i] == 3) {
+          l.kind = Launch::Kind::Placed;
+          l.out = steps_[i].out;
+        } else {
+          l.kind = Launch::Kind::CopyInto;
+          const bool first_left = placed_[i] == 2;  // input 1 is in place: copy input 0
+          l.a = first_left ? steps_[i].in0 : steps_[i].in1;
+          l.out = ConcatPart(i, first_left ? 0 : 1);
+          l.bytes = 2.0 * static_cast<double>(l.a.meta.GetSize());
+        }
+        schedule.push_back(std::move(l));
       } else if (!taken_[i]) {
         Launch l;
         l.members = {i};
@@ -271,6 +290,7 @@ class Scheduler {
           l.rewired = true;
           l.a = steps_[i].in0;
           l.b = steps_[i].in1;
+          l.out = steps_[i].out;
         }
         schedule.push_back(std::move(l));
       }
@@ -480,6 +500,111 @@ class Scheduler {
       elided_[i] = true;
       taken_[i] = true;
       BuildReaders();  // names changed: the source gained this step's readers
+    }
+  }
+
+  // ---- Concat2 inputs written in place ---------------------------------------------------------------------
+  // The launch that produces an input of a Concat2 can write it straight into its part of the Concat2's output
+  // (every kernel takes output strides), provided nobody else reads the input, and the output's bytes -- which
+  // the memory plan reserves only from the Concat2 on -- are touched by nothing else between that launch and the
+  // Concat2.  With both inputs in place the Concat2 does not run; with one, it copies the other.
+
+  // part `side` (0: first input, 1: second) of Concat2 step c's output, as an operand
+  Operand ConcatPart(size_t c, int side) const {
+    const Step &s = steps_[c];
+    const Operand &whole = s.out;
+    const auto &shape = whole.meta.GetShape();
+    int64_t axis = Attrs(c).axis;
+    if (axis < 0) axis += static_cast<int64_t>(shape.size());
+    const std::vector<int64_t> strides = LogicalStrides(whole);
+    Operand part = whole;
+    part.meta = side == 0 ? s.in0.meta : s.in1.meta;
+    part.viewed = true;
+    part.view_strides = strides;
+    part.view_offset = (whole.viewed ? whole.view_offset : 0) +
+                       (side == 0 ? 0 : s.in0.meta.GetShape()[static_cast<size_t>(axis)] * strides[static_cast<size_t>(axis)]);
+    part.source_bytes = whole.Extent();
+    return part;
+  }
+
+  void PlaceConcatInputs(std::vector<Launch> *fused) {
+    std::vector<size_t> issued(steps_.size());
+    std::vector<Launch *> owner(steps_.size(), nullptr);
+    for (size_t i = 0; i < steps_.size(); ++i) issued[i] = i;
+    for (Launch &l : *fused) {
+      const size_t pos = l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back();
+      for (size_t m : l.members) {
+        issued[m] = pos;
+        owner[m] = &l;
+      }
+    }
+    for (size_t c = 0; c < steps_.size(); ++c) {
+      if (taken_[c] || Kind(c) != OpKind::Concat2) continue;
+      const Step &cat = steps_[c];
+      const auto &oshape = cat.out.meta.GetShape();
+      int64_t axis = Attrs(c).axis;
+      if (axis < 0) axis += static_cast<int64_t>(oshape.size());
+      if (axis < 0 || axis >= static_cast<int64_t>(oshape.size()) || cat.out.viewed || SameTensor(cat.in0, cat.in1)) continue;
+      if (cat.in0.meta.GetShape().size() != oshape.size() || cat.in1.meta.GetShape().size() != oshape.size()) continue;
+      for (int side = 0; side < 2; ++side) {
+        const Operand &x = side == 0 ? cat.in0 : cat.in1;
+        if (x.viewed || !Elidable(x) || x.meta.GetType() != cat.out.meta.GetType()) continue;
+        auto it = readers_.find(x.name);
+        if (it == readers_.end() || it->second.size() != 1 || it->second[0] != c) continue;
+        // the step that writes x, and the launch it runs in
+        std::optional<size_t> producer;
+        for (size_t q = 0; q < c; ++q) {
+          if (!elided_[q] && SameTensor(steps_[q].out, x) && !steps_[q].out.viewed) producer = q;
+        }
+        if (!producer) continue;
+        Launch *l = owner[*producer];
+        if (l != nullptr) {
+          const bool plain_out = l->group.empty() && l->view_strides.empty() && SameTensor(l->out, x) && !l->out.viewed;
+          const bool kind_ok = l->kind == Launch::Kind::MatMulChain || l->kind == Launch::Kind::GemmChain ||
+                               l->kind == Launch::Kind::ConvChain || l->kind == Launch::Kind::ElementwiseChain ||
+                               l->kind == Launch::Kind::DivAddSoftmax || l->kind == Launch::Kind::AddLayerNorm ||
+                               l->kind == Launch::Kind::Attention;
+          if (!plain_out || !kind_ok) continue;
+        } else if (taken_[*producer] || placed_[*producer] != 0) {
+          continue;
+        }
+        const size_t from = issued[*producer];
+        if (from >= c) continue;
+        // nothing else may touch the output's bytes from the producer's launch up to the Concat2
+        const Operand target = ConcatPart(c, side);
+        bool ok = true;
+        for (size_t q = 0; q < steps_.size() && ok; ++q) {
+          if (q == c || elided_[q]) continue;
+          if (l != nullptr ? owner[q] == l : q == *producer) continue;
+          const bool in_range = (q >= from && q <= c) || (issued[q] >= from && issued[q] <= c);
+          if (!in_range) continue;
+          const Step &st = steps_[q];
+          // the other input's producer may already write its own part of the same output
+          const bool other_part = st.out.viewed && SameTensor(st.out, cat.out) && placed_[c] != 0;
+          if (!other_part && Alias(st.out, target)) ok = false;
+          if (Alias(st.in0, target) || (st.node->IsDoubleInputs() && Alias(st.in1, target))) ok = false;
+          if (st.has_buffer && target.space == Operand::Space::Arena && st.buffer_offset < target.offset + target.Extent() &&
+              target.offset < st.buffer_offset + st.buffer_bytes) {
+            ok = false;
+          }
+        }
+        // the producer's own inputs must not lie under the bytes it now writes
+        for (size_t m : (l != nullptr ? l->members : std::vector<size_t>{*producer})) {
+          const Step &st = steps_[m];
+          if (Alias(st.in0, target) || (st.node->IsDoubleInputs() && Alias(st.in1, target))) ok = false;
+        }
+        if (l != nullptr) {
+          for (const Operand *op : {&l->a, &l->b, &l->c, &l->d}) {
+            if (!op->name.empty() && Alias(*op, target)) ok = false;
+          }
+        }
+        if (!ok) continue;
+        steps_[*producer].out = target;
+        if (l != nullptr) l->out = target;
+        else rewired_[*producer] = true;
+        placed_[c] |= side == 0 ? 1 : 2;
+      }
+      if (placed_[c] != 0) taken_[c] = true;
     }
   }
 
@@ -1073,6 +1198,7 @@ class Scheduler {
 
   std::vector<Step> steps_;  // own copy: view elision rewrites the inputs of the readers
   std::vector<bool> taken_, elided_, rewired_;
+  std::vector<int> placed_;  // Concat2 steps: bit 0 / 1 = input 0 / 1 is written in place by its producer
   std::unordered_map<std::string, std::vector<size_t>> readers_;
 };
 

@@ -178,9 +178,9 @@ const std::vector<Launch> &LaunchPlan::GetSchedule() const {
 }
 
 void LaunchPlan::IssueStep(kernel::LaunchContext &ctx, const Step &s, const Operand *in0_view,
-                           const Operand *in1_view) const {
-  const Operand &op0 = in0_view ? *in0_view : s.in0;
-  const kernel::TensorView in0 = ViewOf(Resolve(op0), op0), out = ViewOf(Resolve(s.out), s.out);
+                           const Operand *in1_view, const Operand *out_view) const {
+  const Operand &op0 = in0_view ? *in0_view : s.in0, &opo = out_view ? *out_view : s.out;
+  const kernel::TensorView in0 = ViewOf(Resolve(op0), op0), out = ViewOf(Resolve(opo), opo);
   const kernel::Buffer buffer{s.has_buffer ? static_cast<char *>(arena_) + s.buffer_offset : nullptr, s.buffer_bytes};
   kernel::Kernel *k = s.kernel.get();
   if (s.node->IsSingleInput()) {
@@ -217,9 +217,10 @@ fl_tensor Permuted(const fl_tensor &t, const std::vector<int64_t> &perm, bool in
 }  // namespace
 
 void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
-  if (l.kind == Launch::Kind::View) return;  // nothing runs: the readers address the source
+  if (l.kind == Launch::Kind::View || l.kind == Launch::Kind::Placed) return;  // nothing runs
   if (l.kind == Launch::Kind::Step) {
-    IssueStep(ctx, steps_[l.members[0]], l.rewired ? &l.a : nullptr, l.rewired ? &l.b : nullptr);
+    IssueStep(ctx, steps_[l.members[0]], l.rewired ? &l.a : nullptr, l.rewired ? &l.b : nullptr,
+              l.rewired ? &l.out : nullptr);
     return;
   }
   const kernel::TensorView a = ViewOf(Resolve(l.a), l.a), out = ViewOf(Resolve(l.out), l.out);
@@ -327,6 +328,9 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       rc = fluidml_hip_add_layer_normalization(&a.t, &b.t, &g.t, &h.t, &out.t, l.axis, l.s0, ctx.stream);
       break;
     }
+    case Launch::Kind::CopyInto:
+      rc = fluidml_hip_reshape(&a.t, &out.t, ctx.stream);  // same shape on both sides: a strided copy
+      break;
     case Launch::Kind::ReshapeTranspose: {
       // the Transpose's output buffer addressed by the Reshape's logical index
       const fl_tensor dst = Permuted(out.t, l.perm, true);
@@ -473,7 +477,7 @@ std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
   for (size_t it = 0; it < warmup + iters; ++it) {
     try {
       for (size_t i = 0; i < schedule.size(); ++i) {
-        if (schedule[i].kind == Launch::Kind::View) continue;
+        if (schedule[i].kind == Launch::Kind::View || schedule[i].kind == Launch::Kind::Placed) continue;
         Check(fluidml_hip_time_kernels(events[2 * i], events[2 * i + 1]), "kernel timing on");
         Issue(ctx, schedule[i]);
       }
@@ -485,7 +489,7 @@ std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
     Check(fluidml_hip_stream_synchronize(stream_), "profiling sync");
     if (it >= warmup) {
       for (size_t i = 0; i < schedule.size(); ++i) {
-        if (schedule[i].kind == Launch::Kind::View) continue;
+        if (schedule[i].kind == Launch::Kind::View || schedule[i].kind == Launch::Kind::Placed) continue;
         double ns = 0;
         Check(fluidml_hip_event_elapsed_ns(events[2 * i], events[2 * i + 1], &ns), "event elapsed");
         samples[i].push_back(ns);
@@ -498,7 +502,7 @@ std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
     std::vector<double> &v = samples[i];
     std::sort(v.begin(), v.end());
     const Launch &l = schedule[i];
-    if (l.kind == Launch::Kind::View) continue;  // not a launch
+    if (l.kind == Launch::Kind::View || l.kind == Launch::Kind::Placed) continue;  // not a launch
     StepTime t;
     for (size_t m : l.members) {
       t.node += (t.node.empty() ? "" : "+") + steps_[m].node->GetName();

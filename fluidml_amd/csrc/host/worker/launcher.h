@@ -73,8 +73,11 @@ struct Launch {
     AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias
     ReshapeTranspose,  // Reshape -> Transpose, one strided copy
     TransposeReshape,  // Transpose -> Reshape, one strided copy
-    View               // a Slice / Transpose / Squeeze / Unsqueeze / Reshape that is not run: its readers address
+    View,              // a Slice / Transpose / Squeeze / Unsqueeze / Reshape that is not run: its readers address
                        // the source through strides (members = {i}, out = the source operand seen as the view)
+    Placed,            // a Concat2 that is not run: the launches producing its inputs wrote them into its output
+    CopyInto           // a Concat2 one input of which was written in place by its producer: copies the other (a)
+                       // into its part of the output (out, a view of the Concat2's output)
   };
   Kind kind = Kind::Step;
   std::vector<size_t> members;  // indices into the step list, ascending
@@ -86,7 +89,8 @@ struct Launch {
   // Attention: a = queries, b = keys (transposed), c = values, d = additive mask (has_mask), the Where step
   // `owner` holds the condition (has_cond) and s1 its fill value; s0 scales the scores, dividing if `divisor`
   bool has_mask = false, has_cond = false, divisor = false;
-  // Step: the step's inputs, when one of them became a view of another tensor (rewired), replace the plan's
+  // Step: the step's operands a, b, out replace the plan's when an input became a view of another tensor or the
+  // output is written straight into a Concat2's output (rewired)
   bool rewired = false;
   // MatMulChain followed by Reshape/Transpose steps that only re-address the result: element strides of the
   // contraction's logical output dims inside `out` (empty: `out` is the contraction's own output tensor),
@@ -190,7 +194,7 @@ class LaunchPlan {
   };
   void *Resolve(const Operand &op) const;
   void IssueStep(kernel::LaunchContext &ctx, const Step &s, const Operand *in0_view = nullptr,
-                 const Operand *in1_view = nullptr) const;
+                 const Operand *in1_view = nullptr, const Operand *out_view = nullptr) const;
   void Issue(kernel::LaunchContext &ctx, const Launch &l) const;
   void LaunchAll(kernel::LaunchContext &ctx) const;
   void Replay(kernel::LaunchContext &ctx);

@@ -349,7 +349,7 @@ SCHEDULE_NETS = {
              {"MatMulChain", "AddLayerNormalization", "Attention", "ElementwiseChain"}),
     "convbert": (lambda m: m.convbert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32),
                  {"MatMulChain", "AddLayerNormalization"}),  # whether its attention fuses depends on the plan's reuse of bytes
-    "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), {"MatMulChain", "Attention"}),
+    "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), {"MatMulChain", "Attention", "View", "CopyInto"}),
     "efficientnet_b0": (lambda m: m.efficientnet_b0(image=64, classes=10, width_div=4), {"ConvChain"}),
     "vgg16": (lambda m: m.vgg16(batch=2, image=32, classes=10, width_div=8, fc=512), {"ConvChain", "GemmChain"}),
 }
@@ -415,10 +415,43 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
                 own = launches[k] is owner
                 if (i < wpos < pos) or own:
                     assert not _overlap(what, src), "the source of an elided view is overwritten before a reader runs"
+    # A launch that writes an input of a Concat2 straight into the Concat2's output ("writes_into"): the plan
+    # reserves those bytes only from the Concat2 on, so nothing else may read or write them between that launch
+    # and the Concat2; the input itself must have no other reader; a "Placed" Concat2 has both inputs in place,
+    # a "CopyInto" one exactly one.
+    in_place = {}
+    for l in launches:
+        if "writes_into" not in l:
+            continue
+        into = l["writes_into"]
+        cats = [i for i, s in enumerate(steps) if s["out"]["name"] == into["name"] and s["kernel"] == "Concat2Kernel"]
+        assert len(cats) == 1
+        (c,) = cats
+        in_place[c] = in_place.get(c, 0) + 1
+        if l["kind"] == "CopyInto":
+            assert l["members"] == [c]
+            continue
+        final = l["members"][-1]
+        assert readers[steps[final]["out"]["name"]] == {c}, "an input written in place has another reader"
+        pos = l["position"]
+        assert pos < c
+        for q, s in enumerate(steps):
+            if q == c or q in elided or q in l["members"]:
+                continue
+            if pos <= q <= c or pos <= issued[q][0] <= c:
+                for op in s["inputs"] + [s["out"]]:
+                    if steps[c]["out"]["name"] == issued[q][1].get("writes_into", {}).get("name") and op is s["out"]:
+                        continue  # the producer of the other input, writing its own part
+                    assert not _overlap(op, into), "bytes of a Concat2 output written early are in use"
+    for l in launches:
+        if l["kind"] == "Placed":
+            assert in_place.get(l["members"][0]) == 2 and l["written"] == []
+        if l["kind"] == "CopyInto":
+            assert in_place.get(l["members"][0]) == 2  # its own copy and the producer of the other input
     for l in launches:
         members = l["members"]
         assert members == sorted(members)
-        if l["kind"] in ("Step", "View"):
+        if l["kind"] in ("Step", "View", "Placed", "CopyInto"):
             assert len(members) == 1
             continue
         written = set(l["written"])

@@ -127,7 +127,9 @@ std::string LaunchPlan::ToText() const {
     os << "\n";
   }
   const std::vector<Launch> &schedule = GetSchedule();
-  os << "  schedule launches=" << schedule.size() << "\n";
+  size_t run = 0;
+  for (const Launch &l : schedule) run += l.kind != Launch::Kind::View && l.kind != Launch::Kind::Placed ? 1 : 0;
+  os << "  schedule launches=" << run << "\n";
   for (const Launch &l : schedule) {
     if (l.kind == Launch::Kind::Step) continue;
     os << "    fused " << LaunchKindName(l.kind) << " {";

@@ -76,10 +76,23 @@ def make_config(args):
 
 def cpu_baseline_whole(net, feeds, batch):
     """One whole inference of the oracle's loop nests on one core (configurations other than BERT-base)."""
+    import threading
+
     from oracle import graph_runner
 
+    # a whole VGG-16 pass at batch 8 takes the scalar loop nests minutes: say so while it runs
+    done = threading.Event()
+
+    def heartbeat():
+        while not done.wait(30.0):
+            print(f"[bench] cpu baseline still running ({time.perf_counter() - t0:.0f} s) ...", file=sys.stderr, flush=True)
+
     t0 = time.perf_counter()
-    graph_runner.run_graph(net, feeds)
+    threading.Thread(target=heartbeat, daemon=True).start()
+    try:
+        graph_runner.run_graph(net, feeds)
+    finally:
+        done.set()
     total = time.perf_counter() - t0
     return {"value": batch / total, "unit": "inferences/s", "cores": 1, "kind": "port",
             "sample": f"one whole forward pass of batch {batch}", "seconds_per_inference": total / batch}

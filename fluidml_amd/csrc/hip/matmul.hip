@@ -196,7 +196,13 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   constexpr int LDB = LB == 0 ? BN : BK + 4;
   constexpr int A_ELEMS = LA == 0 ? BM * LDA : BK * LDA;
   constexpr int B_ELEMS = LB == 0 ? BK * LDB : BN * LDB;
-  constexpr int RED_ELEMS = KS > 1 ? (KS - 1) * BM * BN : 0;
+  // QUARTER: one 32x32 tile per workgroup whose four waves split K.  After the K loop every wave takes a quarter of
+  // the tile (8 rows: 4 of its 16 accumulator values per lane) through the rest of the kernel -- the sum over the
+  // K slices, the exchange with the other K splits, bias, elementwise chain and stores -- instead of one wave
+  // doing all 16 values while three have left.
+  constexpr bool QUARTER = KS == 4 && TM * TN == 1 && WM * WN == 1;
+  constexpr int EV = QUARTER ? 4 : 16;  // values per lane in the tail
+  constexpr int RED_ELEMS = KS > 1 ? (QUARTER ? KS : KS - 1) * BM * BN : 0;
   constexpr int STAGE_ELEMS = 2 * (A_ELEMS + B_ELEMS);
   constexpr int LDS_ELEMS = STAGE_ELEMS > RED_ELEMS ? STAGE_ELEMS : RED_ELEMS;
   __shared__ __attribute__((aligned(16))) float lds[LDS_ELEMS];
@@ -488,7 +494,22 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   __syncthreads();  // staging area is reused below
 
   // ---- combine the K slices of a workgroup through LDS ------------------------
-  if constexpr (KS > 1) {
+  if constexpr (QUARTER) {
+    if (!producer) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        lds[ks * BM * BN + ((e / 4) * 8 + half * 4 + (e % 4)) * BN + lrow] = acc[0][0][e];
+      }
+    }
+    __syncthreads();
+    if (producer) return;
+    // value i of the quarter is accumulator element 4 ks + i: tile row 8 ks + 4 half + i; slices added in order
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int at = (ks * 8 + half * 4 + i) * BN + lrow;
+      acc[0][0][i] = ((lds[at] + lds[BM * BN + at]) + lds[2 * BM * BN + at]) + lds[3 * BM * BN + at];
+    }
+  } else if constexpr (KS > 1) {
     if (ks > 0 && !producer) {
       float *red = lds + (ks - 1) * BM * BN;
 #pragma unroll
@@ -531,34 +552,37 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
     if (p.n_splits > 1) {
       const uint32_t n_splits = p.n_splits;
       const uint32_t tile_id = (blockIdx.y * n_tiles + blockIdx.x) * (WM * WN) + wm * WN + wn;
-      float *mine = p.partials + (static_cast<size_t>(tile_id) * n_splits + blockIdx.z) * 1024;
+      // a wave's slot: the whole tile, or its quarter of it (own arrival counter per quarter)
+      const uint32_t slot = QUARTER ? tile_id * 4 + ks : tile_id;
+      const uint32_t sub = QUARTER ? ks * 256 : 0;
+      float *mine = p.partials + (static_cast<size_t>(tile_id) * n_splits + blockIdx.z) * 1024 + sub;
       // The partial tiles travel through device-coherent accesses (agent-scope atomics: they bypass the
       // per-XCD L2 instead of living in it), so no cache-wide write-back or invalidate is needed: waiting
       // for this wave's stores to be acknowledged before it counts its arrival is enough, and the last
       // wave's loads are issued only after it has seen every other arrival.
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
+      for (int e = 0; e < EV; ++e) {
         __hip_atomic_store(mine + e * 64 + lane, acc[0][0][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // s_waitcnt: stores acknowledged
       uint32_t arrived = 0;
-      if (lane == 0) arrived = __hip_atomic_fetch_add(&p.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) arrived = __hip_atomic_fetch_add(&p.counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       arrived = __shfl(arrived, 0);
       if (arrived != n_splits - 1) return;
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // keeps the loads below behind the counter read
-      if (lane == 0) __hip_atomic_store(&p.counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const float *all = p.partials + static_cast<size_t>(tile_id) * n_splits * 1024;
+      if (lane == 0) __hip_atomic_store(&p.counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const float *all = p.partials + static_cast<size_t>(tile_id) * n_splits * 1024 + sub;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[0][0][e] = 0.0f;
+      for (int e = 0; e < EV; ++e) acc[0][0][e] = 0.0f;
       // four splits' loads are in flight together (one round trip for up to four splits); the sums still run
       // in split order
       for (uint32_t z0 = 0; z0 < n_splits; z0 += 4) {
-        float part[4][16];
+        float part[4][EV];
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
           const uint32_t z = z0 + u < n_splits ? z0 + u : z0;  // repeats a valid slot, ignored below
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
+          for (int e = 0; e < EV; ++e) {
             part[u][e] = __hip_atomic_load(all + z * 1024 + e * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
         }
@@ -566,7 +590,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
         for (uint32_t u = 0; u < 4; ++u) {
           if (z0 + u < n_splits) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[0][0][e] += part[u][e];
+            for (int e = 0; e < EV; ++e) acc[0][0][e] += part[u][e];
           }
         }
       }
@@ -590,11 +614,13 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
         col = static_cast<int64_t>(img) * p.conv.sOn + static_cast<int64_t>(oh) * p.conv.sOh +
               static_cast<int64_t>(ow) * p.conv.sOw;
       }
-      // bias, then the elementwise chain on the 16 values of this 32x32 tile the lane holds, then the stores
-      float vals[16];
+      // bias, then the elementwise chain on the values of this 32x32 tile the lane holds (all 16, or the 4 of its
+      // wave's quarter), then the stores
+      auto tile_row = [&](int e) { return QUARTER ? ks * 8 + half * 4 + e : (e / 4) * 8 + half * 4 + (e % 4); };
+      float vals[EV];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = m0 + (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
+      for (int e = 0; e < EV; ++e) {
+        const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
         float v = acc[i][j][e];
         if (bias_by_col) {
           v = p.ca * v + p.cb * bias_col[j];
@@ -603,10 +629,10 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
         }
         vals[e] = v;
       }
-      if (p.chain.n != 0) RunChainBlock<16>(p.chain, vals);
+      if (p.chain.n != 0) RunChainBlock<EV>(p.chain, vals);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = m0 + (wm * TM + i) * 32 + (e / 4) * 8 + half * 4 + (e % 4);
+      for (int e = 0; e < EV; ++e) {
+        const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
         if (m < p.M && n < p.N) Cb[static_cast<int64_t>(m) * sCm + col] = vals[e];
       }
   });

@@ -24,9 +24,9 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the contraction kernel on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, averaged over the 51 contraction launches of an inference), each scaled by what the
-# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x1.000): (6279.6 * 2.0 + 1429.2) KiB.
+# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x1.000): (6245.7 * 2.0 + 1447.8) KiB.
 # Only valid for the default workload (BERT-base, seq 128, 12 layers, plain_greedy, fusion on).
-MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 14_322_469
+MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 14_271_941
 
 
 def cpu_baseline(layers_total: int, sample_layers: int, seq: int):

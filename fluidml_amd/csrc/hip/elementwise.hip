@@ -211,6 +211,14 @@ struct Mul2 {
 struct Div2 {
   __device__ float operator()(float a, float b, Empty) const { return a / b; }
 };
+// a * b + c with the product rounded before the sum, as the two separate kernels round it
+struct MulAdd3 {
+  __device__ float operator()(float a, float b, float c) const {
+#pragma clang fp contract(off)
+    const float product = a * b;
+    return product + c;
+  }
+};
 struct WhereScalarY {
   float y;
   __device__ float operator()(uint8_t c, float x, Empty) const { return c ? x : y; }
@@ -500,6 +508,15 @@ int fluidml_hip_add_common(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
   if (!lhs || !rhs || !out) return FL_ERR_NULL;
   if (lhs->dtype != FL_FLOAT32 || rhs->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
   return Binary<float>(lhs, rhs, out, Add2<float>{}, stream);
+}
+
+int fluidml_hip_mul_add(const fl_tensor *a, const fl_tensor *b, const fl_tensor *c, const fl_tensor *out, void *stream) {
+  if (!a || !b || !c || !out) return FL_ERR_NULL;
+  if (a->dtype != FL_FLOAT32 || b->dtype != FL_FLOAT32 || c->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  const fl_tensor *ins[3] = {a, b, c};
+  LoopNest nest;
+  FL_CHECK(BroadcastNest(ins, 3, out, &nest));
+  return LaunchNest<3, float, float, float, float>(nest, out->base, a->base, b->base, c->base, MulAdd3{}, AsStream(stream));
 }
 
 int fluidml_hip_sub_constant_lhs(const fl_tensor *in, const fl_tensor *out, double value, void *stream) {

@@ -23,6 +23,7 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::GemmChain: return "GemmChain";
     case Launch::Kind::ConvChain: return "ConvChain";
     case Launch::Kind::ElementwiseChain: return "ElementwiseChain";
+    case Launch::Kind::MulAdd: return "MulAdd";
     case Launch::Kind::DivAddSoftmax: return "DivAddSoftmax";
     case Launch::Kind::Attention: return "Attention";
     case Launch::Kind::AddLayerNorm: return "AddLayerNormalization";
@@ -239,6 +240,7 @@ class Scheduler {
           case OpKind::GemmConstantWeightsBias:
           case OpKind::ConvWithPadding:
           case OpKind::ConvWithoutPadding: l = MatchContraction(i); break;
+          case OpKind::MulCommon: l = MatchMulAdd(i); break;
           case OpKind::Reshape: l = MatchCopyPair(i, OpKind::Transpose); break;
           case OpKind::Transpose: l = MatchCopyPair(i, OpKind::Reshape); break;
           default: break;
@@ -563,7 +565,7 @@ class Scheduler {
           const bool kind_ok = l->kind == Launch::Kind::MatMulChain || l->kind == Launch::Kind::GemmChain ||
                                l->kind == Launch::Kind::ConvChain || l->kind == Launch::Kind::ElementwiseChain ||
                                l->kind == Launch::Kind::DivAddSoftmax || l->kind == Launch::Kind::AddLayerNorm ||
-                               l->kind == Launch::Kind::Attention;
+                               l->kind == Launch::Kind::Attention || l->kind == Launch::Kind::MulAdd;
           if (!plain_out || !kind_ok) continue;
         } else if (taken_[*producer] || placed_[*producer] != 0) {
           continue;
@@ -1045,6 +1047,26 @@ class Scheduler {
       return std::nullopt;
     }
     l.bytes = Bytes({&l.a, &l.out});
+    return l;
+  }
+
+  // MulCommon whose only reader is an AddCommon: a * b + c in one launch
+  std::optional<Launch> MatchMulAdd(size_t i) {
+    const Step &mul = steps_[i];
+    if (!IsFloat(mul.out) || !IsFloat(mul.in0) || !IsFloat(mul.in1)) return std::nullopt;
+    const auto j = SoleReader(i);
+    if (!j || Kind(*j) != OpKind::AddCommon || !IsFloat(steps_[*j].out)) return std::nullopt;
+    const auto other = Other(*j, mul.out);
+    if (!other || !IsFloat(*other)) return std::nullopt;
+    Launch l;
+    l.kind = Launch::Kind::MulAdd;
+    l.members = {i, *j};
+    l.a = mul.in0;
+    l.b = mul.in1;
+    l.c = *other;
+    l.out = steps_[*j].out;
+    if (!Safe(l.members, {{i, l.a}, {i, l.b}, {*j, l.c}}) || !OutputDisjoint(l.out, {&l.a, &l.b, &l.c})) return std::nullopt;
+    l.bytes = Bytes({&l.a, &l.b, &l.c, &l.out});
     return l;
   }
 

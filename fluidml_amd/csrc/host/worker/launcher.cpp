@@ -293,6 +293,11 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
     case Launch::Kind::ElementwiseChain:
       rc = fluidml_hip_elementwise_chain(&a.t, &out.t, &l.chain, ctx.stream);
       break;
+    case Launch::Kind::MulAdd: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b), c = ViewOf(Resolve(l.c), l.c);
+      rc = fluidml_hip_mul_add(&a.t, &b.t, &c.t, &out.t, ctx.stream);
+      break;
+    }
     case Launch::Kind::DivAddSoftmax: {
       const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
       rc = fluidml_hip_div_add_softmax(&a.t, l.s0, &b.t, &out.t, l.axis, ctx.stream);

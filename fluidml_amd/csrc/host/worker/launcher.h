@@ -68,6 +68,7 @@ struct Launch {
     ConvChain,         // Conv{With,Without}Padding -> elementwise chain
     MatMulGroup,       // up to four MatMulChains that share the left operand and all extents, one launch
     ElementwiseChain,  // two or more elementwise steps on one tensor
+    MulAdd,            // MulCommon -> AddCommon: a * b + c
     DivAddSoftmax,     // DivConstantRhs -> AddCommon(mask) -> Softmax
     Attention,         // MatMul -> Div|Mul constant [-> AddCommon(mask)] [-> Where(cond, x, scalar)] -> Softmax -> MatMul
     AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias

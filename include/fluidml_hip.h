@@ -354,6 +354,9 @@ int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const 
 /* A chain of elementwise kernels on one float32 tensor as one launch:
  * out = chain(in), same shape, any two layouts. */
 int fluidml_hip_elementwise_chain(const fl_tensor *in, const fl_tensor *out, const fl_ew_program *chain, void *stream);
+/* MulCommonKernel -> AddCommonKernel: out = a * b + c (product rounded, then the sum, like the two kernels);
+ * a, b and c broadcast to out.  (reference mul.cpp:70-132, add.cpp:75-137) */
+int fluidml_hip_mul_add(const fl_tensor *a, const fl_tensor *b, const fl_tensor *c, const fl_tensor *out, void *stream);
 /* DivConstantRhsKernel -> AddCommonKernel(mask, broadcast) -> SoftmaxKernel:
  * out = softmax(in / div + mask, axis)
  * (reference div.cpp:24-56 + add.cpp:75-137 + softmax.cpp:22-139). */

@@ -720,6 +720,25 @@ def test_matmul_chain_group(device):
     assert cabi.lib.fluidml_hip_matmul_chain_group(2, da.ref(), rhs_bad, bias, out, 0, None, None, 0, None) == -3  # FL_ERR_SHAPE
 
 
+def test_fused_mul_add(device):
+    """MulCommon -> AddCommon in one launch: the product is rounded before the sum, so the result is the two
+    kernels' bit for bit; all three inputs broadcast."""
+    cabi = _cabi()
+    rng = np.random.default_rng(171)
+    for sa, sb, sc, so in [((1, 2, 24, 8), (24, 8), (1, 2, 24, 8), (1, 2, 24, 8)), ((4, 1, 6), (1, 5, 6), (6,), (4, 5, 6)),
+                           ((1, 96, 14, 14), (1, 96, 1, 1), (1, 96, 14, 14), (1, 96, 14, 14))]:
+        a, b, c = rand(rng, sa), rand(rng, sb), rand(rng, sc)
+        for lo in some_layouts(len(so), rng, 2):
+            announce("mul_add", sa, sb, sc, lo)
+            t, want = ok.View.empty(np.broadcast_shapes(sa, sb)), ok.View.empty(so)
+            ok.binary_f32(ok.BOP_MUL, ok.View(a), ok.View(b), t)
+            ok.binary_f32(ok.BOP_ADD, t, ok.View(c), want)
+            da, db, dc = DeviceView(ok.View(a), device), DeviceView(ok.View(b), device), DeviceView(ok.View(c), device)
+            do = DeviceView(ok.View.empty(so, np.float32, lo, fill=5), device)
+            cabi.call("mul_add", da.ref(), db.ref(), dc.ref(), do.ref(), None)
+            assert_close(do.logical(), want.logical(), exact=True, what="mul_add")
+
+
 def test_elementwise_chain(device):
     """Every chain operation against the oracle's standalone kernels, applied one after the other."""
     cabi = _cabi()

@@ -219,6 +219,10 @@ struct MulAdd3 {
     return product + c;
   }
 };
+// (a + b) + c, the two sums in the order of the two separate kernels
+struct AddAdd3 {
+  __device__ float operator()(float a, float b, float c) const { return (a + b) + c; }
+};
 struct WhereScalarY {
   float y;
   __device__ float operator()(uint8_t c, float x, Empty) const { return c ? x : y; }
@@ -485,6 +489,92 @@ int LaunchPad(const fl_tensor *in, const fl_tensor *out, const int64_t *before, 
   return LaunchStatus();
 }
 
+// Rotary position embedding: one lane per output element.  Operands of the nest: 0 = out, 1 = x, 2 = cos, 3 = sin;
+// the last nest dim is the rotated axis (kept apart so that its coordinate is at hand).
+struct RotaryArgs {
+  NestArgs<4> nest;
+  uint32_t n;
+  uint32_t rot, half;  // the first `rot` values of the axis are rotated, partner at distance half = rot / 2
+  int32_t x_half;      // half * (stride of x along the axis)
+};
+
+__global__ __launch_bounds__(256) void RotaryKernel(RotaryArgs p, float *__restrict__ out, const float *__restrict__ x,
+                                                    const float *__restrict__ cos_t, const float *__restrict__ sin_t) {
+  const uint32_t item = blockIdx.x * 256 + threadIdx.x;
+  if (item >= p.n) return;
+  uint32_t rem = item, d = 0;
+  int32_t off[4] = {0, 0, 0, 0};
+  for (int k = p.nest.rank - 1; k >= 0; --k) {
+    uint32_t q = 0, r = rem;
+    if (k > 0) p.nest.dims[k].div.DivMod(rem, q, r);
+    rem = q;
+    if (k == p.nest.rank - 1) d = r;
+#pragma unroll
+    for (int o = 0; o < 4; ++o) off[o] += static_cast<int32_t>(r) * p.nest.dims[k].strides[o];
+  }
+  float v = x[off[1]];
+  if (d < p.rot) {
+    // rot = concat(-x[half:rot], x[:half]); each product is rounded before the sum, like the separate kernels
+#pragma clang fp contract(off)
+    const float partner = d < p.half ? -x[off[1] + p.x_half] : x[off[1] - p.x_half];
+    const float direct = v * cos_t[off[2]];
+    const float turned = partner * sin_t[off[3]];
+    v = direct + turned;
+  }
+  out[off[0]] = v;
+}
+
+int LaunchRotary(const fl_tensor *x, const fl_tensor *cos_t, const fl_tensor *sin_t, const fl_tensor *out,
+                 int64_t rotary_dims, hipStream_t stream) {
+  FL_CHECK(CheckView(x));
+  FL_CHECK(CheckView(cos_t));
+  FL_CHECK(CheckView(sin_t));
+  FL_CHECK(CheckView(out));
+  if (x->dtype != FL_FLOAT32 || cos_t->dtype != FL_FLOAT32 || sin_t->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32)
+    return FL_ERR_DTYPE;
+  if (!SameShape(x, out)) return FL_ERR_SHAPE;
+  const int rank = out->rank;
+  if (rank < 1) return FL_ERR_RANK;
+  const int64_t len = out->shape[rank - 1];
+  if (rotary_dims < 0 || rotary_dims > len || rotary_dims % 2 != 0) return FL_ERR_ATTR;
+  LoopNest nest;
+  nest.rank = rank;
+  nest.n_operands = 4;
+  int64_t total = 1;
+  for (int i = 0; i < rank; ++i) {
+    nest.shape[i] = out->shape[i];
+    nest.strides[0][i] = out->strides[i];
+    nest.strides[1][i] = x->strides[i];
+    total *= out->shape[i];
+  }
+  // cos and sin: [.., rotary_dims], leading dims broadcast to x's; never read beyond rotary_dims
+  const fl_tensor *tables[2] = {cos_t, sin_t};
+  for (int k = 0; k < 2; ++k) {
+    const fl_tensor *t = tables[k];
+    if (t->rank < 1 || t->rank > rank || t->shape[t->rank - 1] != rotary_dims) return FL_ERR_SHAPE;
+    for (int i = 0; i < rank; ++i) {
+      const int j = t->rank - rank + i;
+      if (i == rank - 1) nest.strides[2 + k][i] = t->strides[j];
+      else if (j < 0 || t->shape[j] == 1) nest.strides[2 + k][i] = 0;
+      else if (t->shape[j] == out->shape[i]) nest.strides[2 + k][i] = t->strides[j];
+      else return FL_ERR_SHAPE;
+    }
+  }
+  if (total == 0) return FL_OK;
+  if (total > 0x7fffffff) return FL_ERR_TOO_LARGE;
+  RotaryArgs p;
+  std::memset(&p, 0, sizeof(p));
+  p.nest = MakeNestArgs<4>(nest);
+  p.n = static_cast<uint32_t>(total);
+  p.rot = static_cast<uint32_t>(rotary_dims);
+  p.half = static_cast<uint32_t>(rotary_dims / 2);
+  p.x_half = static_cast<int32_t>((rotary_dims / 2) * x->strides[rank - 1]);
+  FL_LAUNCH(RotaryKernel, dim3((p.n + 255) / 256), dim3(256), 0, stream, p, static_cast<float *>(out->base),
+            static_cast<const float *>(x->base), static_cast<const float *>(cos_t->base),
+            static_cast<const float *>(sin_t->base));
+  return LaunchStatus();
+}
+
 }  // namespace
 }  // namespace fl
 
@@ -517,6 +607,21 @@ int fluidml_hip_mul_add(const fl_tensor *a, const fl_tensor *b, const fl_tensor 
   LoopNest nest;
   FL_CHECK(BroadcastNest(ins, 3, out, &nest));
   return LaunchNest<3, float, float, float, float>(nest, out->base, a->base, b->base, c->base, MulAdd3{}, AsStream(stream));
+}
+
+int fluidml_hip_add_add(const fl_tensor *a, const fl_tensor *b, const fl_tensor *c, const fl_tensor *out, void *stream) {
+  if (!a || !b || !c || !out) return FL_ERR_NULL;
+  if (a->dtype != FL_FLOAT32 || b->dtype != FL_FLOAT32 || c->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  const fl_tensor *ins[3] = {a, b, c};
+  LoopNest nest;
+  FL_CHECK(BroadcastNest(ins, 3, out, &nest));
+  return LaunchNest<3, float, float, float, float>(nest, out->base, a->base, b->base, c->base, AddAdd3{}, AsStream(stream));
+}
+
+int fluidml_hip_rotary(const fl_tensor *x, const fl_tensor *cos_table, const fl_tensor *sin_table, const fl_tensor *out,
+                       int64_t rotary_dims, void *stream) {
+  if (!x || !cos_table || !sin_table || !out) return FL_ERR_NULL;
+  return LaunchRotary(x, cos_table, sin_table, out, rotary_dims, AsStream(stream));
 }
 
 int fluidml_hip_sub_constant_lhs(const fl_tensor *in, const fl_tensor *out, double value, void *stream) {

@@ -6,7 +6,9 @@
 // src/structure/flow/node.cpp); it has no counterpart of this pass because it
 // pays no per-kernel launch cost.
 #include <algorithm>
+#include <cstdlib>
 #include <optional>
+#include <string>
 #include <unordered_map>
 
 #include "utils/utils.h"
@@ -24,6 +26,8 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::ConvChain: return "ConvChain";
     case Launch::Kind::ElementwiseChain: return "ElementwiseChain";
     case Launch::Kind::MulAdd: return "MulAdd";
+    case Launch::Kind::AddAdd: return "AddAdd";
+    case Launch::Kind::Rotary: return "Rotary";
     case Launch::Kind::DivAddSoftmax: return "DivAddSoftmax";
     case Launch::Kind::Attention: return "Attention";
     case Launch::Kind::AddLayerNorm: return "AddLayerNormalization";
@@ -227,6 +231,7 @@ class Scheduler {
         if (Kind(i) == OpKind::MatMul) l = MatchAttention(i);
         else if (Kind(i) == OpKind::DivConstantRhs) l = MatchSoftmax(i);
         else if (Kind(i) == OpKind::AddCommon) l = MatchLayerNorm(i);
+        if (!l && Kind(i) == OpKind::AddCommon) l = MatchRotary(i);
         if (l) {
           for (size_t m : l->members) taken_[m] = true;
           fused.push_back(std::move(*l));
@@ -241,6 +246,7 @@ class Scheduler {
           case OpKind::ConvWithPadding:
           case OpKind::ConvWithoutPadding: l = MatchContraction(i); break;
           case OpKind::MulCommon: l = MatchMulAdd(i); break;
+          case OpKind::AddCommon: l = MatchAddAdd(i); break;
           case OpKind::Reshape: l = MatchCopyPair(i, OpKind::Transpose); break;
           case OpKind::Transpose: l = MatchCopyPair(i, OpKind::Reshape); break;
           default: break;
@@ -303,8 +309,10 @@ class Scheduler {
  private:
   void BuildReaders() {
     readers_.clear();
+    producer_.clear();
     for (size_t i = 0; i < steps_.size(); ++i) {
       const Step &s = steps_[i];
+      if (!s.out.viewed) producer_[s.out.name] = i;
       readers_[s.in0.name].push_back(i);
       if (s.node->IsDoubleInputs() && !SameTensor(s.in0, s.in1)) readers_[s.in1.name].push_back(i);
     }
@@ -565,7 +573,8 @@ class Scheduler {
           const bool kind_ok = l->kind == Launch::Kind::MatMulChain || l->kind == Launch::Kind::GemmChain ||
                                l->kind == Launch::Kind::ConvChain || l->kind == Launch::Kind::ElementwiseChain ||
                                l->kind == Launch::Kind::DivAddSoftmax || l->kind == Launch::Kind::AddLayerNorm ||
-                               l->kind == Launch::Kind::Attention || l->kind == Launch::Kind::MulAdd;
+                               l->kind == Launch::Kind::Attention || l->kind == Launch::Kind::MulAdd ||
+                               l->kind == Launch::Kind::AddAdd;
           if (!plain_out || !kind_ok) continue;
         } else if (taken_[*producer] || placed_[*producer] != 0) {
           continue;
@@ -1070,6 +1079,177 @@ class Scheduler {
     return l;
   }
 
+  // ---- rotary position embedding ---------------------------------------------------------------------------
+  // The free step that produces `o` when `reader` is the only step reading it.
+  std::optional<size_t> ProducerFor(const Operand &o, size_t reader) const {
+    if (o.viewed) return std::nullopt;
+    const auto it = producer_.find(o.name);
+    if (it == producer_.end() || taken_[it->second] || it->second >= reader) return std::nullopt;
+    const auto only = SoleReader(it->second);
+    if (!only || *only != reader) return std::nullopt;
+    return it->second;
+  }
+
+  // Slice step i as the range [begin, begin + length) of the last axis with everything else whole.
+  std::optional<std::pair<int64_t, int64_t>> LastAxisRange(size_t i) const {
+    if (Kind(i) != OpKind::Slice) return std::nullopt;
+    const auto &ishape = steps_[i].in0.meta.GetShape();
+    const auto &oshape = steps_[i].out.meta.GetShape();
+    if (ishape.size() != oshape.size() || ishape.empty()) return std::nullopt;
+    const int64_t rank = static_cast<int64_t>(ishape.size());
+    for (int64_t d = 0; d + 1 < rank; ++d) {
+      if (ishape[static_cast<size_t>(d)] != oshape[static_cast<size_t>(d)]) return std::nullopt;
+    }
+    const flow::Attrs &at = Attrs(i);
+    if (at.starts.size() != at.axes.size() || at.steps.size() != at.axes.size()) return std::nullopt;
+    int64_t begin = 0;
+    for (size_t n = 0; n < at.axes.size(); ++n) {
+      const int64_t ax = at.axes[n] < 0 ? at.axes[n] + rank : at.axes[n];
+      if (ax < 0 || ax >= rank || at.steps[n] != 1) return std::nullopt;
+      int64_t b = at.starts[n];
+      if (b < 0) b += ishape[static_cast<size_t>(ax)];
+      if (ax == rank - 1) begin = b;
+      else if (b != 0) return std::nullopt;
+    }
+    if (begin < 0 || begin + oshape.back() > ishape.back()) return std::nullopt;
+    return std::make_pair(begin, oshape.back());
+  }
+
+  bool LastAxis(size_t concat) const {
+    const int64_t rank = static_cast<int64_t>(steps_[concat].out.meta.GetShape().size());
+    const int64_t axis = Attrs(concat).axis;
+    return (axis < 0 ? axis + rank : axis) == rank - 1;
+  }
+
+  // x_rot * cos + concat(-x_rot[.., h:], x_rot[.., :h]) * sin, matched from its AddCommon (step i); when x_rot is
+  // itself the slice x[.., :R] and the sum is concatenated with x[.., R:], those steps join too, and so does a
+  // Transpose of the result (written through permuted strides).  One launch of fluidml_hip_rotary.
+  std::optional<Launch> MatchRotary(size_t i) {
+    // FLUIDML_ROTARY=0 leaves the steps to the general mechanisms (views, Concat2 inputs written in place)
+    if (const char *v = std::getenv("FLUIDML_ROTARY"); v != nullptr && std::string(v) == "0") return std::nullopt;
+    const Step &add = steps_[i];
+    if (!IsFloat(add.out) || SameTensor(add.in0, add.in1)) return std::nullopt;
+    const auto p0 = ProducerFor(add.in0, i), p1 = ProducerFor(add.in1, i);
+    if (!p0 || !p1 || Kind(*p0) != OpKind::MulCommon || Kind(*p1) != OpKind::MulCommon) return std::nullopt;
+    for (int swap = 0; swap < 2; ++swap) {
+      const size_t m1 = swap ? *p1 : *p0, m2 = swap ? *p0 : *p1;  // m1: x_rot * cos, m2: turned * sin
+      for (int side = 0; side < 2; ++side) {
+        const Operand &turned = side ? steps_[m2].in1 : steps_[m2].in0;
+        const Operand &sin_t = side ? steps_[m2].in0 : steps_[m2].in1;
+        const auto c1 = ProducerFor(turned, m2);
+        if (!c1 || Kind(*c1) != OpKind::Concat2 || !LastAxis(*c1)) continue;
+        const auto neg = ProducerFor(steps_[*c1].in0, *c1), s1 = ProducerFor(steps_[*c1].in1, *c1);
+        if (!neg || !s1 || Kind(*neg) != OpKind::Neg) continue;
+        const auto s2 = ProducerFor(steps_[*neg].in0, *neg);
+        if (!s2) continue;
+        const auto r1 = LastAxisRange(*s1), r2 = LastAxisRange(*s2);
+        if (!r1 || !r2 || !SameTensor(steps_[*s1].in0, steps_[*s2].in0)) continue;
+        const Operand x_rot = steps_[*s1].in0;
+        const int64_t rot = x_rot.meta.GetShape().back(), half = rot / 2;
+        if (rot % 2 != 0 || r1->first != 0 || r1->second != half || r2->first != half || r2->second != half) continue;
+        const bool left = SameTensor(steps_[m1].in0, x_rot), right = SameTensor(steps_[m1].in1, x_rot);
+        if (left == right) continue;
+        const Operand &cos_t = left ? steps_[m1].in1 : steps_[m1].in0;
+        if (add.out.meta.GetShape() != x_rot.meta.GetShape() || !IsFloat(x_rot) || !IsFloat(cos_t) || !IsFloat(sin_t)) continue;
+        // the tables: rot values along the last axis, leading dims broadcast to x_rot's
+        bool tables = true;
+        for (const Operand *t : {&cos_t, &sin_t}) {
+          const auto &ts = t->meta.GetShape();
+          const auto &xs = x_rot.meta.GetShape();
+          tables = tables && !ts.empty() && ts.size() <= xs.size() && ts.back() == rot;
+          for (size_t d = 0; tables && d + 1 < ts.size(); ++d) {
+            const int64_t want = xs[xs.size() - ts.size() + d];
+            tables = ts[d] == 1 || ts[d] == want;
+          }
+        }
+        if (!tables) continue;
+        Launch l;
+        l.kind = Launch::Kind::Rotary;
+        l.members = {m1, *s1, *s2, *neg, *c1, m2, i};
+        l.a = x_rot;
+        l.b = cos_t;
+        l.c = sin_t;
+        l.axis = rot;
+        l.out = add.out;
+        size_t first_x = std::min({m1, *s1, *s2});
+        // the outer Slice / Concat2 pair around a partial rotation
+        Launch whole = l;
+        bool widened = false;
+        if (const auto c2 = SoleReader(i); c2 && Kind(*c2) == OpKind::Concat2 && LastAxis(*c2) &&
+                                           SameTensor(steps_[*c2].in0, add.out) && !x_rot.viewed) {
+          const auto sp = ProducerFor(steps_[*c2].in1, *c2);
+          const auto pr = producer_.find(x_rot.name);
+          if (sp && pr != producer_.end() && !taken_[pr->second] && Elidable(x_rot)) {
+            const size_t sr = pr->second;
+            const auto rr = LastAxisRange(sr), rp = LastAxisRange(*sp);
+            const auto rd = readers_.find(x_rot.name);
+            std::vector<size_t> expect = {m1, *s1, *s2};
+            std::sort(expect.begin(), expect.end());
+            std::vector<size_t> have = rd != readers_.end() ? rd->second : std::vector<size_t>{};
+            std::sort(have.begin(), have.end());
+            if (rr && rp && have == expect && SameTensor(steps_[sr].in0, steps_[*sp].in0) && rr->first == 0 &&
+                rr->second == rot && rp->first == rot && rp->first + rp->second == steps_[sr].in0.meta.GetShape().back()) {
+              whole.members.push_back(sr);
+              whole.members.push_back(*sp);
+              whole.members.push_back(*c2);
+              whole.a = steps_[sr].in0;
+              whole.out = steps_[*c2].out;
+              first_x = std::min(sr, *sp);
+              widened = true;
+            }
+          }
+        }
+        Launch &best = widened ? whole : l;
+        std::sort(best.members.begin(), best.members.end());
+        // a Transpose of the result: written through permuted strides
+        Launch turned_out = best;
+        bool transposed = false;
+        if (const auto t = SoleReader(best.members.back()); t && Kind(*t) == OpKind::Transpose &&
+                                                          Attrs(*t).perm.size() == best.out.meta.GetShape().size()) {
+          turned_out.members.push_back(*t);
+          turned_out.perm = Attrs(*t).perm;
+          turned_out.out = steps_[*t].out;
+          transposed = true;
+        }
+        auto finish = [&](Launch *x, size_t x_from) {
+          if (!Safe(x->members, {{x_from, x->a}, {m1, x->b}, {m2, x->c}})) return false;
+          if (!OutputDisjoint(x->out, {&x->a, &x->b, &x->c})) return false;
+          x->bytes = Bytes({&x->a, &x->b, &x->c, &x->out});
+          x->flops = 0;
+          return true;
+        };
+        if (transposed && finish(&turned_out, widened ? first_x : std::min({m1, *s1, *s2}))) return turned_out;
+        if (finish(&best, widened ? first_x : std::min({m1, *s1, *s2}))) return best;
+        if (widened) {
+          std::sort(l.members.begin(), l.members.end());
+          if (finish(&l, std::min({m1, *s1, *s2}))) return l;
+        }
+        return std::nullopt;
+      }
+    }
+    return std::nullopt;
+  }
+
+  // AddCommon -> AddCommon (two residuals): (a + b) + c in one launch, rounded like the two kernels
+  std::optional<Launch> MatchAddAdd(size_t i) {
+    const Step &first = steps_[i];
+    if (!IsFloat(first.out) || !IsFloat(first.in0) || !IsFloat(first.in1)) return std::nullopt;
+    const auto j = SoleReader(i);
+    if (!j || Kind(*j) != OpKind::AddCommon || !IsFloat(steps_[*j].out)) return std::nullopt;
+    const auto other = Other(*j, first.out);
+    if (!other || !IsFloat(*other)) return std::nullopt;
+    Launch l;
+    l.kind = Launch::Kind::AddAdd;
+    l.members = {i, *j};
+    l.a = first.in0;
+    l.b = first.in1;
+    l.c = *other;
+    l.out = steps_[*j].out;
+    if (!Safe(l.members, {{i, l.a}, {i, l.b}, {*j, l.c}}) || !OutputDisjoint(l.out, {&l.a, &l.b, &l.c})) return std::nullopt;
+    l.bytes = Bytes({&l.a, &l.b, &l.c, &l.out});
+    return l;
+  }
+
   std::optional<Launch> MatchSoftmax(size_t i) {
     const Step &div = steps_[i];
     if (!IsFloat(div.out)) return std::nullopt;
@@ -1222,6 +1402,7 @@ class Scheduler {
   std::vector<bool> taken_, elided_, rewired_;
   std::vector<int> placed_;  // Concat2 steps: bit 0 / 1 = input 0 / 1 is written in place by its producer
   std::unordered_map<std::string, std::vector<size_t>> readers_;
+  std::unordered_map<std::string, size_t> producer_;  // tensor name -> the step that writes it
 };
 
 }  // namespace

@@ -298,6 +298,18 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       rc = fluidml_hip_mul_add(&a.t, &b.t, &c.t, &out.t, ctx.stream);
       break;
     }
+    case Launch::Kind::AddAdd: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b), c = ViewOf(Resolve(l.c), l.c);
+      rc = fluidml_hip_add_add(&a.t, &b.t, &c.t, &out.t, ctx.stream);
+      break;
+    }
+    case Launch::Kind::Rotary: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b), c = ViewOf(Resolve(l.c), l.c);
+      // a folded Transpose: its output buffer addressed by the untransposed logical index
+      const fl_tensor dst = l.perm.empty() ? out.t : Permuted(out.t, l.perm, true);
+      rc = fluidml_hip_rotary(&a.t, &b.t, &c.t, &dst, l.axis, ctx.stream);
+      break;
+    }
     case Launch::Kind::DivAddSoftmax: {
       const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
       rc = fluidml_hip_div_add_softmax(&a.t, l.s0, &b.t, &out.t, l.axis, ctx.stream);

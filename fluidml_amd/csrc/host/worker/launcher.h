@@ -69,6 +69,10 @@ struct Launch {
     MatMulGroup,       // up to four MatMulChains that share the left operand and all extents, one launch
     ElementwiseChain,  // two or more elementwise steps on one tensor
     MulAdd,            // MulCommon -> AddCommon: a * b + c
+    AddAdd,            // AddCommon -> AddCommon: (a + b) + c
+    Rotary,            // rotary position embedding (Slice, Neg, Concat2, MulCommon, AddCommon, Concat2 [, Transpose]):
+                       // a = x, b = cosine table, c = sine table, axis = number of rotated values, perm = the
+                       // folded Transpose (empty: none)
     DivAddSoftmax,     // DivConstantRhs -> AddCommon(mask) -> Softmax
     Attention,         // MatMul -> Div|Mul constant [-> AddCommon(mask)] [-> Where(cond, x, scalar)] -> Softmax -> MatMul
     AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias

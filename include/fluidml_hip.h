@@ -357,6 +357,19 @@ int fluidml_hip_elementwise_chain(const fl_tensor *in, const fl_tensor *out, con
 /* MulCommonKernel -> AddCommonKernel: out = a * b + c (product rounded, then the sum, like the two kernels);
  * a, b and c broadcast to out.  (reference mul.cpp:70-132, add.cpp:75-137) */
 int fluidml_hip_mul_add(const fl_tensor *a, const fl_tensor *b, const fl_tensor *c, const fl_tensor *out, void *stream);
+/* AddCommonKernel -> AddCommonKernel (two residual sums): out = (a + b) + c, rounded like the two kernels;
+ * a, b and c broadcast to out.  (reference add.cpp:75-137) */
+int fluidml_hip_add_add(const fl_tensor *a, const fl_tensor *b, const fl_tensor *c, const fl_tensor *out, void *stream);
+/* The rotary position embedding of the exported GPT-NeoX graphs as one launch: Slice x[.., :R] and x[.., R:],
+ * Slice the two halves of the first, NegKernel, Concat2Kernel (-second half, first half), MulCommonKernel with
+ * the sine table, MulCommonKernel of x[.., :R] with the cosine table, AddCommonKernel, Concat2Kernel with
+ * x[.., R:] (reference slice.cpp:17-55, neg.cpp:17-40, concat.cpp:18-68, mul.cpp:70-132, add.cpp:75-137).
+ * With h = R / 2 and rot = concat(-x[.., h:R], x[.., :h]):
+ *   out[.., d] = x[.., d] * cos[.., d] + rot[.., d] * sin[.., d]   for d < R = rotary_dims (even),
+ *   out[.., d] = x[.., d]                                          beyond,
+ * both products rounded before the sum, like the separate kernels (bit-identical to them).  cos and sin have R
+ * values along the last axis; their leading dims broadcast to x's.  x and out: same shape, any strides. */
+int fluidml_hip_rotary(const fl_tensor *x, const fl_tensor *cos_table, const fl_tensor *sin_table, const fl_tensor *out, int64_t rotary_dims, void *stream);
 /* DivConstantRhsKernel -> AddCommonKernel(mask, broadcast) -> SoftmaxKernel:
  * out = softmax(in / div + mask, axis)
  * (reference div.cpp:24-56 + add.cpp:75-137 + softmax.cpp:22-139). */

@@ -737,6 +737,56 @@ def test_fused_mul_add(device):
             do = DeviceView(ok.View.empty(so, np.float32, lo, fill=5), device)
             cabi.call("mul_add", da.ref(), db.ref(), dc.ref(), do.ref(), None)
             assert_close(do.logical(), want.logical(), exact=True, what="mul_add")
+            # AddCommon -> AddCommon on the same operands
+            ok.binary_f32(ok.BOP_ADD, ok.View(a), ok.View(b), t)
+            ok.binary_f32(ok.BOP_ADD, t, ok.View(c), want)
+            do = DeviceView(ok.View.empty(so, np.float32, lo, fill=5), device)
+            cabi.call("add_add", da.ref(), db.ref(), dc.ref(), do.ref(), None)
+            assert_close(do.logical(), want.logical(), exact=True, what="add_add")
+
+
+def test_fused_rotary(device):
+    """The rotary embedding's Slice / Neg / Concat2 / MulCommon / AddCommon / Concat2 steps as one launch: the
+    result is the oracle's nine steps bit for bit, for any layouts of x and out, with and without a pass-through
+    part, tables that broadcast over heads."""
+    cabi = _cabi()
+    rng = np.random.default_rng(173)
+    for shape, rot, tshape in [((1, 8, 256, 64), 16, (1, 1, 256, 16)), ((2, 3, 10, 8), 8, (10, 8)),
+                               ((1, 2, 7, 12), 4, (1, 2, 7, 4)), ((5, 6), 6, (5, 6))]:
+        x = rand(rng, shape)
+        cos_t, sin_t = rand(rng, tshape, -1, 1), rand(rng, tshape, -1, 1)
+        rank, last, half = len(shape), len(shape) - 1, rot // 2
+        hx = ok.View(x)
+        want = ok.View.empty(shape)
+        if rot > 0:
+            head = shape[:-1]
+            xr, x1, x2, neg, turned = (ok.View.empty(head + (n,)) for n in (rot, half, half, half, rot))
+            ok.slice_(hx, xr, [0], [last], [1])
+            ok.slice_(xr, x1, [0], [last], [1])
+            ok.slice_(xr, x2, [half], [last], [1])
+            ok.unary_f32(ok.OP_NEG, x2, neg)
+            ok.concat2(neg, x1, turned, last)
+            m1, m2, summed = (ok.View.empty(head + (rot,)) for _ in range(3))
+            ok.binary_f32(ok.BOP_MUL, xr, ok.View(cos_t), m1)
+            ok.binary_f32(ok.BOP_MUL, turned, ok.View(sin_t), m2)
+            ok.binary_f32(ok.BOP_ADD, m1, m2, summed)
+            if rot == shape[-1]:
+                want = summed
+            else:
+                rest = ok.View.empty(head + (shape[-1] - rot,))
+                ok.slice_(hx, rest, [rot], [last], [1])
+                ok.concat2(summed, rest, want, last)
+        for lx, lo in [(None, None), (list(range(rank))[::-1], None), (None, list(range(rank))[::-1])]:
+            announce("rotary", shape, rot, tshape, lx, lo)
+            dx = DeviceView(ok.View(x, lx), device)
+            dc, ds = DeviceView(ok.View(cos_t), device), DeviceView(ok.View(sin_t), device)
+            do = DeviceView(ok.View.empty(shape, np.float32, lo, fill=5), device)
+            cabi.call("rotary", dx.ref(), dc.ref(), ds.ref(), do.ref(), ctypes.c_int64(rot), None)
+            assert_close(do.logical(), want.logical(), exact=True, what="rotary")
+    dx = DeviceView(ok.View.empty((2, 8)), device)
+    dt = DeviceView(ok.View.empty((2, 3)), device)
+    assert cabi.lib.fluidml_hip_rotary(dx.ref(), dt.ref(), dt.ref(), dx.ref(), 3, None) == -5  # FL_ERR_ATTR: odd
+    assert cabi.lib.fluidml_hip_rotary(dx.ref(), dt.ref(), dt.ref(), dx.ref(), 4, None) == -3  # FL_ERR_SHAPE: tables
 
 
 def test_elementwise_chain(device):

@@ -349,7 +349,10 @@ SCHEDULE_NETS = {
              {"MatMulChain", "AddLayerNormalization", "Attention", "ElementwiseChain"}),
     "convbert": (lambda m: m.convbert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32),
                  {"MatMulChain", "AddLayerNormalization"}),  # whether its attention fuses depends on the plan's reuse of bytes
-    "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), {"MatMulChain", "Attention", "View", "CopyInto"}),
+    "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), {"MatMulChain", "Attention", "View", "Rotary"}),
+    # without the rotary launch its steps go through the general mechanisms: views, Concat2 inputs written in place
+    "gpt_neox_no_rotary": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120),
+                           {"MatMulChain", "Attention", "View", "CopyInto", "MulAdd"}),
     "efficientnet_b0": (lambda m: m.efficientnet_b0(image=64, classes=10, width_div=4), {"ConvChain"}),
     "vgg16": (lambda m: m.vgg16(batch=2, image=32, classes=10, width_div=8, fc=512), {"ConvChain", "GemmChain"}),
 }
@@ -365,6 +368,8 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     make, expected_kinds = SCHEDULE_NETS[which]
     path = make(models).save(str(tmp_path / "net.onnx"))
     monkeypatch.setenv("FLUIDML_DP_COST", "constant")
+    if which.endswith("_no_rotary"):
+        monkeypatch.setenv("FLUIDML_ROTARY", "0")
     ex = getattr(fluidml.Executor, flavour)("sched")
     ex.compile(path)
     plan = ex.plan()

@@ -260,6 +260,7 @@ class Scheduler {
     }
     if (fuse) GroupSiblings(&fused);
     if (fuse) ElideViews(&fused);
+    if (fuse) RetryAttention(&fused);
     if (fuse) PlaceConcatInputs(&fused);
     // a chain is issued where its last member stood; everything else keeps its place
     std::vector<const Launch *> at(steps_.size(), nullptr);
@@ -648,7 +649,14 @@ class Scheduler {
     for (const auto &[m, op] : external) {
       for (size_t s = m + 1; s < last; ++s) {
         if (std::find(members.begin(), members.end(), s) != members.end()) continue;
+        if (!moved_.empty() && moved_[s] != SIZE_MAX && moved_[s] <= m) continue;  // runs before the first read now
+        if (elided_[s] || (!silent_.empty() && silent_[s])) continue;  // never written
         if (Alias(steps_[s].out, op)) return false;
+      }
+      // steps a group moved into the window from outside it
+      for (size_t s = 0; s < moved_.size(); ++s) {
+        if (moved_[s] == SIZE_MAX || (s > m && s < last)) continue;
+        if (moved_[s] > m && moved_[s] < last && Alias(steps_[s].out, op)) return false;
       }
     }
     // the chain's own output must not overwrite an external input another member still needs: the fused kernel
@@ -1277,6 +1285,74 @@ class Scheduler {
     return l;
   }
 
+  // Attention blocks the first sweep had to leave alone because a projection of the same block stood between
+  // the score MatMul and the rest (the value projection after Q.K^T in the sequence): once GroupSiblings has moved
+  // that projection in front, the block is matched again.  The contraction launches it overlaps are dissolved;
+  // members the attention launch does not absorb go back to being single steps.
+  void RetryAttention(std::vector<Launch> *fused) {
+    moved_.assign(steps_.size(), SIZE_MAX);
+    silent_.assign(steps_.size(), false);
+    bool any = false;
+    for (const Launch &l : *fused) {
+      for (size_t m : l.members) silent_[m] = true;
+      if (l.group.empty()) silent_[l.members.back()] = false;
+      for (const Launch &g : l.group) silent_[g.members.back()] = false;
+      if (l.kind != Launch::Kind::MatMulGroup) continue;
+      for (size_t m : l.members) moved_[m] = l.position;
+      any = true;
+    }
+    for (size_t xi = 0; any && xi < fused->size(); ++xi) {
+      const Launch &x = (*fused)[xi];
+      if (x.kind != Launch::Kind::MatMulChain || Kind(x.members[0]) != OpKind::MatMul) continue;
+      const size_t head = x.members[0];
+      const std::vector<bool> saved = taken_;
+      for (const Launch &y : *fused) {
+        if (y.kind != Launch::Kind::MatMulChain) continue;
+        for (size_t m : y.members) taken_[m] = false;
+      }
+      std::optional<Launch> l = MatchAttention(head);
+      taken_ = saved;
+      if (!l) continue;
+      std::vector<size_t> touched;
+      bool ok = true;
+      size_t absorbed_free = 0, leftovers = 0;
+      for (size_t m : l->members) {
+        bool found = false;
+        for (size_t yi = 0; yi < fused->size(); ++yi) {
+          const Launch &y = (*fused)[yi];
+          if (std::find(y.members.begin(), y.members.end(), m) == y.members.end()) continue;
+          found = true;
+          if (y.kind != Launch::Kind::MatMulChain) ok = false;
+          if (std::find(touched.begin(), touched.end(), yi) == touched.end()) touched.push_back(yi);
+        }
+        if (!found) {
+          if (taken_[m]) ok = false;
+          ++absorbed_free;
+        }
+      }
+      if (!ok) continue;
+      for (size_t yi : touched) {
+        for (size_t m : (*fused)[yi].members) {
+          if (std::find(l->members.begin(), l->members.end(), m) == l->members.end()) ++leftovers;
+        }
+      }
+      if (1 + leftovers >= touched.size() + absorbed_free) continue;  // no launch saved
+      for (size_t yi : touched) {
+        for (size_t m : (*fused)[yi].members) taken_[m] = false;
+      }
+      for (size_t m : l->members) taken_[m] = true;
+      std::vector<Launch> kept;
+      for (size_t yi = 0; yi < fused->size(); ++yi) {
+        if (std::find(touched.begin(), touched.end(), yi) == touched.end()) kept.push_back(std::move((*fused)[yi]));
+      }
+      kept.push_back(std::move(*l));
+      *fused = std::move(kept);
+      xi = static_cast<size_t>(-1);  // the list changed: start over
+    }
+    moved_.clear();
+    silent_.clear();
+  }
+
   // scores = MatMul(q, k^T) -> Div | Mul by a constant [-> + mask] [-> Where(cond, x, fill)] -> Softmax over
   // the keys -> MatMul(p, v), optionally followed by the head-merging Transpose / Reshape: one launch that
   // keeps the score rows on chip.  The kernel's limits (head size, number of keys) are checked here so that
@@ -1400,6 +1476,8 @@ class Scheduler {
 
   std::vector<Step> steps_;  // own copy: view elision rewrites the inputs of the readers
   std::vector<bool> taken_, elided_, rewired_;
+  std::vector<bool> silent_;   // per step: an intermediate of a fused launch, never written (filled by RetryAttention)
+  std::vector<size_t> moved_;  // per step: the position its launch is issued at when a group moved it (else SIZE_MAX)
   std::vector<int> placed_;  // Concat2 steps: bit 0 / 1 = input 0 / 1 is written in place by its producer
   std::unordered_map<std::string, std::vector<size_t>> readers_;
   std::unordered_map<std::string, size_t> producer_;  // tensor name -> the step that writes it

@@ -133,6 +133,7 @@ SIGNATURES = {
     "fluidml_hip_gather_constant_index_scalar": [_T, _T, _i64, _i64, _u32, _vp],
     "fluidml_hip_gather_constant_indices_tensor": [_T, _T, _T, _i64, _vp],
     "fluidml_hip_gather_constant_data_tensor": [_T, _T, _T, _vp],
+    "fluidml_hip_gather_constant_data_tensor_add": [_T, _T, _T, _T, _vp],
     "fluidml_hip_gather_constant_data_tensor_add_tensor_lhs_add_tensor_lhs": [_T, _T, _T, _T, _T, _vp],
     "fluidml_hip_cum_sum": [_T, _T, _i64, _vp],
     # row reductions

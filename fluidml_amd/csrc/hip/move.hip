@@ -293,6 +293,19 @@ int fluidml_hip_gather_constant_data_tensor(const fl_tensor *indices, const fl_t
                                 nullptr, AsStream(stream));
 }
 
+int fluidml_hip_gather_constant_data_tensor_add(const fl_tensor *indices, const fl_tensor *data, const fl_tensor *add0,
+                                                const fl_tensor *out, void *stream) {
+  LoopNest nest;
+  nest.n_operands = 4;
+  if (!indices || !data || !add0 || !out) return FL_ERR_NULL;
+  FL_CHECK(GatherNest(data, indices, out, 0, &nest));
+  FL_CHECK(CheckView(add0));
+  if (data->dtype != FL_FLOAT32 || add0->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  FL_CHECK(BroadcastStrides(add0, out->rank, out->shape, nest.strides[3]));
+  return LaunchGather<float, 1>(nest, data->strides[0], data->shape[0], out->base, indices->base, data->base,
+                                add0->base, nullptr, AsStream(stream));
+}
+
 int fluidml_hip_gather_constant_data_tensor_add_tensor_lhs_add_tensor_lhs(const fl_tensor *indices,
                                                                           const fl_tensor *data, const fl_tensor *add0,
                                                                           const fl_tensor *add1, const fl_tensor *out,

@@ -27,6 +27,7 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::ElementwiseChain: return "ElementwiseChain";
     case Launch::Kind::MulAdd: return "MulAdd";
     case Launch::Kind::AddAdd: return "AddAdd";
+    case Launch::Kind::GatherAdd: return "GatherAdd";
     case Launch::Kind::Rotary: return "Rotary";
     case Launch::Kind::DivAddSoftmax: return "DivAddSoftmax";
     case Launch::Kind::Attention: return "Attention";
@@ -247,6 +248,7 @@ class Scheduler {
           case OpKind::ConvWithoutPadding: l = MatchContraction(i); break;
           case OpKind::MulCommon: l = MatchMulAdd(i); break;
           case OpKind::AddCommon: l = MatchAddAdd(i); break;
+          case OpKind::GatherConstantDataTensor: l = MatchGatherAdd(i); break;
           case OpKind::Reshape: l = MatchCopyPair(i, OpKind::Transpose); break;
           case OpKind::Transpose: l = MatchCopyPair(i, OpKind::Reshape); break;
           default: break;
@@ -258,7 +260,11 @@ class Scheduler {
         }
       }
     }
-    if (fuse) GroupSiblings(&fused);
+    if (fuse) {
+      MarkSilent(fused);
+      GroupSiblings(&fused);
+      silent_.clear();
+    }
     if (fuse) ElideViews(&fused);
     if (fuse) RetryAttention(&fused);
     if (fuse) PlaceConcatInputs(&fused);
@@ -1019,12 +1025,21 @@ class Scheduler {
           return false;
         };
         if (!producer_before(l.a)) return false;
+        // (a step inside a fused launch that is not its last never writes its output, and what it reads from
+        // such a step is never read)
+        auto exists = [&](const Operand &op) {
+          if (silent_.empty() || op.viewed) return true;
+          const auto it = producer_.find(op.name);
+          return it == producer_.end() || !silent_[it->second];
+        };
         for (size_t s = position; s <= own; ++s) {
           if (is_member(s)) continue;
           const Step &st = steps_[s];
-          if (Alias(st.out, l.out) || Alias(st.in0, l.out)) return false;
-          if (st.node->IsDoubleInputs() && Alias(st.in1, l.out)) return false;
-          if (st.has_buffer && l.out.space == Operand::Space::Arena && st.buffer_offset < l.out.offset + l.out.meta.GetSize() &&
+          const bool unwritten = !silent_.empty() && silent_[s];
+          if (!unwritten && Alias(st.out, l.out)) return false;
+          if (exists(st.in0) && Alias(st.in0, l.out)) return false;
+          if (st.node->IsDoubleInputs() && exists(st.in1) && Alias(st.in1, l.out)) return false;
+          if (st.has_buffer && !unwritten && l.out.space == Operand::Space::Arena && st.buffer_offset < l.out.offset + l.out.meta.GetSize() &&
               l.out.offset < st.buffer_offset + st.buffer_bytes) {
             return false;  // scratch of a step in between (untouched by these kernels, but reserved)
           }
@@ -1238,6 +1253,44 @@ class Scheduler {
     return std::nullopt;
   }
 
+  // GatherConstantDataTensor -> AddCommon [-> AddCommon] (an embedding lookup and the embeddings added to it)
+  std::optional<Launch> MatchGatherAdd(size_t i) {
+    const Step &gather = steps_[i];
+    if (!IsFloat(gather.out) || steps_[i].kernel->GetConstant(0) == nullptr) return std::nullopt;
+    const auto j = SoleReader(i);
+    if (!j || Kind(*j) != OpKind::AddCommon || !IsFloat(steps_[*j].out)) return std::nullopt;
+    if (steps_[*j].out.meta.GetShape() != gather.out.meta.GetShape()) return std::nullopt;
+    const auto first = Other(*j, gather.out);
+    if (!first || !IsFloat(*first)) return std::nullopt;
+    Launch l;
+    l.kind = Launch::Kind::GatherAdd;
+    l.members = {i, *j};
+    l.a = gather.in0;
+    l.b = *first;
+    l.out = steps_[*j].out;
+    l.owner = i;
+    std::vector<std::pair<size_t, Operand>> external = {{i, l.a}, {*j, l.b}};
+    Launch longer = l;
+    if (const auto k = SoleReader(*j); k && Kind(*k) == OpKind::AddCommon && IsFloat(steps_[*k].out) &&
+                                       steps_[*k].out.meta.GetShape() == gather.out.meta.GetShape()) {
+      if (const auto second = Other(*k, steps_[*j].out); second && IsFloat(*second)) {
+        longer.members.push_back(*k);
+        longer.c = *second;
+        longer.has_c = true;
+        longer.out = steps_[*k].out;
+        auto ext = external;
+        ext.push_back({*k, longer.c});
+        if (Safe(longer.members, ext) && OutputDisjoint(longer.out, {&longer.a, &longer.b, &longer.c})) {
+          longer.bytes = Bytes({&longer.a, &longer.b, &longer.c, &longer.out}) + static_cast<double>(longer.out.meta.GetSize());
+          return longer;
+        }
+      }
+    }
+    if (!Safe(l.members, external) || !OutputDisjoint(l.out, {&l.a, &l.b})) return std::nullopt;
+    l.bytes = Bytes({&l.a, &l.b, &l.out}) + static_cast<double>(l.out.meta.GetSize());  // + the gathered rows
+    return l;
+  }
+
   // AddCommon -> AddCommon (two residuals): (a + b) + c in one launch, rounded like the two kernels
   std::optional<Launch> MatchAddAdd(size_t i) {
     const Step &first = steps_[i];
@@ -1285,18 +1338,25 @@ class Scheduler {
     return l;
   }
 
+  // silent_[s]: step s sits inside a fused launch and is not the member whose output the launch writes
+  void MarkSilent(const std::vector<Launch> &fused) {
+    silent_.assign(steps_.size(), false);
+    for (const Launch &l : fused) {
+      for (size_t m : l.members) silent_[m] = true;
+      if (l.group.empty()) silent_[l.members.back()] = false;
+      for (const Launch &g : l.group) silent_[g.members.back()] = false;
+    }
+  }
+
   // Attention blocks the first sweep had to leave alone because a projection of the same block stood between
   // the score MatMul and the rest (the value projection after Q.K^T in the sequence): once GroupSiblings has moved
   // that projection in front, the block is matched again.  The contraction launches it overlaps are dissolved;
   // members the attention launch does not absorb go back to being single steps.
   void RetryAttention(std::vector<Launch> *fused) {
     moved_.assign(steps_.size(), SIZE_MAX);
-    silent_.assign(steps_.size(), false);
+    MarkSilent(*fused);
     bool any = false;
     for (const Launch &l : *fused) {
-      for (size_t m : l.members) silent_[m] = true;
-      if (l.group.empty()) silent_[l.members.back()] = false;
-      for (const Launch &g : l.group) silent_[g.members.back()] = false;
       if (l.kind != Launch::Kind::MatMulGroup) continue;
       for (size_t m : l.members) moved_[m] = l.position;
       any = true;

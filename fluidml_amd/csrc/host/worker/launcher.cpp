@@ -298,6 +298,18 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       rc = fluidml_hip_mul_add(&a.t, &b.t, &c.t, &out.t, ctx.stream);
       break;
     }
+    case Launch::Kind::GatherAdd: {
+      const kernel::DeviceConstant *table = steps_[l.owner].kernel->GetConstant(0);
+      if (table == nullptr) throw std::logic_error("fused Gather: the node holds no data tensor");
+      const kernel::TensorView data = table->View(), b = ViewOf(Resolve(l.b), l.b);
+      if (l.has_c) {
+        const kernel::TensorView c = ViewOf(Resolve(l.c), l.c);
+        rc = fluidml_hip_gather_constant_data_tensor_add_tensor_lhs_add_tensor_lhs(&a.t, &data.t, &b.t, &c.t, &out.t, ctx.stream);
+      } else {
+        rc = fluidml_hip_gather_constant_data_tensor_add(&a.t, &data.t, &b.t, &out.t, ctx.stream);
+      }
+      break;
+    }
     case Launch::Kind::AddAdd: {
       const kernel::TensorView b = ViewOf(Resolve(l.b), l.b), c = ViewOf(Resolve(l.c), l.c);
       rc = fluidml_hip_add_add(&a.t, &b.t, &c.t, &out.t, ctx.stream);

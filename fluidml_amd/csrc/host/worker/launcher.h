@@ -70,6 +70,8 @@ struct Launch {
     ElementwiseChain,  // two or more elementwise steps on one tensor
     MulAdd,            // MulCommon -> AddCommon: a * b + c
     AddAdd,            // AddCommon -> AddCommon: (a + b) + c
+    GatherAdd,         // GatherConstantDataTensor -> AddCommon [-> AddCommon]: data[a] + b [+ c] (has_c), the
+                       // table is the constant of `owner`
     Rotary,            // rotary position embedding (Slice, Neg, Concat2, MulCommon, AddCommon, Concat2 [, Transpose]):
                        // a = x, b = cosine table, c = sine table, axis = number of rotated values, perm = the
                        // folded Transpose (empty: none)

@@ -271,6 +271,9 @@ int fluidml_hip_gather_constant_indices_tensor(const fl_tensor *in, const fl_ten
 /* GatherConstantDataTensorKernel: `data` is a constant float32 table, the
  * runtime input holds int64 indices, axis 0 (reference gather.cpp:195-272). */
 int fluidml_hip_gather_constant_data_tensor(const fl_tensor *indices, const fl_tensor *data, const fl_tensor *out, void *stream);
+/* GatherConstantDataTensorKernel -> AddCommonKernel as one launch: out = data[indices] + add0, add0 broadcast
+ * to out (reference gather.cpp:224-262, add.cpp:75-137; the one-addend form of the fused kernel below). */
+int fluidml_hip_gather_constant_data_tensor_add(const fl_tensor *indices, const fl_tensor *data, const fl_tensor *add0, const fl_tensor *out, void *stream);
 /* GatherConstantDataTensorAddTensorLhsAddTensorLhsKernel: data[ids] + add0 + add1
  * (reference gather_add_add.cpp:25-163). */
 int fluidml_hip_gather_constant_data_tensor_add_tensor_lhs_add_tensor_lhs(const fl_tensor *indices, const fl_tensor *data, const fl_tensor *add0, const fl_tensor *add1, const fl_tensor *out, void *stream);

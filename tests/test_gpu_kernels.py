@@ -356,6 +356,12 @@ def test_gathers(device):
         cabi.call("gather_constant_data_tensor_add_tensor_lhs_add_tensor_lhs", di.ref(), dt.ref(), dp.ref(), dy.ref(),
                   do2.ref(), None)
         assert_close(do2.logical(), ho2.logical(), exact=True, what="gather+add+add")
+        # one addend: Gather -> AddCommon as the separate oracle steps
+        ho3 = ok.View.empty((1, 128, 768), np.float32, lout)
+        ok.binary_f32(ok.BOP_ADD, ho, hp, ho3)
+        do3 = DeviceView(ok.View.empty((1, 128, 768), np.float32, lout), device)
+        cabi.call("gather_constant_data_tensor_add", di.ref(), dt.ref(), dp.ref(), do3.ref(), None)
+        assert_close(do3.logical(), ho3.logical(), exact=True, what="gather+add")
     x = rand(rng, (4, 9, 6))
     for lin in some_layouts(3, rng, 3):
         for axis, index in [(0, 3), (1, 0), (2, 5), (-1, 2)]:

@@ -118,6 +118,9 @@ def main():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="instead of the benchmark, launch the identity-copy kernel 3 times on a buffer of MIB MiB "
                          "(a kernel of known traffic, to scale profiler byte counters) and exit")
+    ap.add_argument("--hbm-kernels", action="store_true",
+                    help="instead of the benchmark, time every bandwidth-bound kernel class on 128-512 MiB of data "
+                         "and print its achieved HBM GB/s (table on stderr, one JSON line on stdout)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the reference has no multi-device path); use --gpus 1")
@@ -129,6 +132,11 @@ def main():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     from fluidml_amd import fluidml, models
 
+    if args.hbm_kernels:
+        from fluidml_amd import hbm_sweep
+
+        print(json.dumps(hbm_sweep.run(out=sys.stderr)))
+        return
     if args.copy_calibration:
         import ctypes
 

@@ -242,6 +242,51 @@ inline bool IsAligned(const void *p, size_t bytes) {
   return (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
 }
 
+// Outputs this large do not stay in the last-level cache until their reader runs; writing them with
+// non-temporal stores keeps them from evicting the data the kernel is still reading.  Measured on a 256 MiB
+// copy: 5.5 -> 7.0 TB/s; no difference at 64 MiB and below; non-temporal LOADS were slower at every size.
+constexpr size_t kStreamingBytes = size_t{64} << 20;
+inline bool StreamingOutput(size_t out_bytes) { return out_bytes >= kStreamingBytes; }
+
+// *p = v with a non-temporal store.  V: any trivially copyable type of 4, 8, 16 or 32 bytes aligned to its
+// size; other sizes are stored normally.
+template <typename V>
+__device__ __forceinline__ void StoreStreaming(V *p, const V &v) {
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  if constexpr (sizeof(V) == 4) {
+    __builtin_nontemporal_store(__builtin_bit_cast(uint32_t, v), reinterpret_cast<uint32_t *>(p));
+  } else if constexpr (sizeof(V) == 8) {
+    __builtin_nontemporal_store(__builtin_bit_cast(u32x2, v), reinterpret_cast<u32x2 *>(p));
+  } else if constexpr (sizeof(V) == 16) {
+    __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4 *>(p));
+  } else if constexpr (sizeof(V) == 32) {
+    struct Halves {
+      u32x4 lo, hi;
+    };
+    const Halves h = __builtin_bit_cast(Halves, v);
+    __builtin_nontemporal_store(h.lo, reinterpret_cast<u32x4 *>(p));
+    __builtin_nontemporal_store(h.hi, reinterpret_cast<u32x4 *>(p) + 1);
+  } else {
+    *p = v;
+  }
+}
+
+// *p = v, non-temporal when `streaming` (wave-uniform).
+template <typename V>
+__device__ __forceinline__ void StoreMaybeStreaming(V *p, const V &v, bool streaming) {
+  if (!streaming) {
+    *p = v;
+    return;
+  }
+  // The two empty statements (which name the address, so that the store cannot move across them even when the
+  // pointer is `__restrict__`) keep the optimiser from folding this store and the plain one above into a single
+  // store, which would silently lose the non-temporal hint (the merged store keeps only what both had).
+  asm volatile("" : : "v"(p) : "memory");
+  StoreStreaming(p, v);
+  asm volatile("" : : "v"(p) : "memory");
+}
+
 // A loop nest over up to kMaxRank dimensions and up to kMaxOperands strided
 // operands; operand 0 is the output.  Built in logical order, then
 // canonicalised: unit dims dropped, dims ordered by descending output stride

@@ -46,6 +46,77 @@ __global__ __launch_bounds__(kBlock) void PoolKernel(PoolArgs p, float *__restri
   out[off0] = IS_MAX ? acc : acc / static_cast<float>(p.n_window);
 }
 
+// 2x2 window, stride 2, unit-stride rows on both sides (the pools of the VGG/ResNet families): a lane reads
+// 2*OUTS consecutive values of two input rows with 128-bit loads and writes OUTS consecutive outputs.  The
+// window is folded in its row-major order like PoolKernel does, so the results are identical.
+template <bool IS_MAX, int OUTS>
+__global__ __launch_bounds__(kBlock) void Pool2x2Kernel(NestArgs<2> nest, uint32_t n_items, int32_t row_stride,
+                                                        bool streaming, float *__restrict__ out,
+                                                        const float *__restrict__ in) {
+  const uint32_t item = blockIdx.x * kBlock + threadIdx.x;
+  if (item >= n_items) return;
+  int32_t off[2] = {0, 0};
+  nest.AddOffsets(item, off);
+  const float *src = in + off[1];
+  struct alignas(16) Quad {
+    float v[4];
+  };
+  struct alignas(4 * OUTS) Outs {
+    float v[OUTS];
+  };
+  float top[2 * OUTS], bottom[2 * OUTS];
+#pragma unroll
+  for (int q = 0; q < OUTS / 2; ++q) {
+    const Quad t = reinterpret_cast<const Quad *>(src)[q], b = reinterpret_cast<const Quad *>(src + row_stride)[q];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      top[4 * q + k] = t.v[k];
+      bottom[4 * q + k] = b.v[k];
+    }
+  }
+  Outs r;
+#pragma unroll
+  for (int k = 0; k < OUTS; ++k) {
+    float acc = top[2 * k];
+    acc = IS_MAX ? MaximumF(acc, top[2 * k + 1]) : acc + top[2 * k + 1];
+    acc = IS_MAX ? MaximumF(acc, bottom[2 * k]) : acc + bottom[2 * k];
+    acc = IS_MAX ? MaximumF(acc, bottom[2 * k + 1]) : acc + bottom[2 * k + 1];
+    r.v[k] = IS_MAX ? acc : acc / 4.0f;
+  }
+  StoreMaybeStreaming(reinterpret_cast<Outs *>(out + off[0]), r, streaming);
+}
+
+// Launches Pool2x2Kernel when the canonical nest allows it; false = use the generic kernel.
+template <bool IS_MAX>
+bool TryPool2x2(LoopNest nest, const LoopNest &window, const fl_tensor *in, const fl_tensor *out, hipStream_t stream) {
+  if (window.rank != 2 || window.shape[0] != 2 || window.shape[1] != 2 || window.strides[0][1] != 1) return false;
+  const int inner = nest.rank - 1;
+  if (inner < 0 || nest.strides[0][inner] != 1 || nest.strides[1][inner] != 2) return false;
+  const int64_t row_stride = window.strides[0][0];
+  const int outs = nest.shape[inner] % 4 == 0 ? 4 : nest.shape[inner] % 2 == 0 ? 2 : 0;
+  if (outs == 0 || row_stride % 4 != 0 || row_stride > INT32_MAX) return false;
+  if (!IsAligned(in->base, 16) || !IsAligned(out->base, 4 * outs)) return false;
+  for (int d = 0; d < inner; ++d) {
+    if (nest.strides[1][d] % 4 != 0 || nest.strides[0][d] % outs != 0) return false;
+  }
+  const int64_t n_out = Numel(out);
+  nest.shape[inner] /= outs;
+  nest.strides[0][inner] = outs;
+  nest.strides[1][inner] = 2 * outs;
+  const uint32_t n_items = static_cast<uint32_t>(n_out / outs);
+  const NestArgs<2> args = MakeNestArgs<2>(nest);
+  const bool streaming = StreamingOutput(static_cast<size_t>(n_out) * sizeof(float));
+  const dim3 grid((n_items + kBlock - 1) / kBlock);
+  if (outs == 4) {
+    FL_LAUNCH((Pool2x2Kernel<IS_MAX, 4>), grid, dim3(kBlock), 0, stream, args, n_items, static_cast<int32_t>(row_stride),
+              streaming, static_cast<float *>(out->base), static_cast<const float *>(in->base));
+  } else {
+    FL_LAUNCH((Pool2x2Kernel<IS_MAX, 2>), grid, dim3(kBlock), 0, stream, args, n_items, static_cast<int32_t>(row_stride),
+              streaming, static_cast<float *>(out->base), static_cast<const float *>(in->base));
+  }
+  return true;
+}
+
 template <bool IS_MAX>
 int Pool(const fl_tensor *in, const fl_tensor *out, const int64_t *kernel_shape, const int64_t *strides, int32_t n,
          void *stream) {
@@ -80,6 +151,7 @@ int Pool(const fl_tensor *in, const fl_tensor *out, const int64_t *kernel_shape,
   }
   nest.Canonicalise();
   // the window keeps its logical (row-major) order: that is the fold order
+  if (Numel(out) <= INT32_MAX && TryPool2x2<IS_MAX>(nest, window, in, out, AsStream(stream))) return LaunchStatus();
   PoolArgs p;
   p.nest = MakeNestArgs<2>(nest);
   p.window = MakeNestArgs<1>(window);

@@ -22,6 +22,7 @@ template <int NOPS>
 struct RowArgs {
   uint32_t n_rows;
   uint32_t len;
+  uint32_t streaming;  // 1 = the output is large enough for non-temporal stores
   int32_t axis_stride[NOPS];
   NestArgs<NOPS> outer;  // non-axis dims, canonical order (operand 0 = output)
 };
@@ -56,9 +57,31 @@ RowArgs<NOPS> MakeRowArgs(int rank, const int64_t *shape, int axis, const int64_
   for (int i = 0; i < nest.rank; ++i) rows *= nest.shape[i];
   args.n_rows = static_cast<uint32_t>(rows);
   args.len = static_cast<uint32_t>(shape[axis]);
+  args.streaming = StreamingOutput(static_cast<size_t>(rows) * static_cast<size_t>(shape[axis]) * sizeof(float)) ? 1 : 0;
   for (int o = 0; o < NOPS; ++o) args.axis_stride[o] = static_cast<int32_t>(strides[o][axis]);
   return args;
 }
+
+// True when operand `o` of a row kernel can be read or written 16 bytes at a time along the axis: unit axis
+// stride, every row starting on a 16-byte boundary.
+inline bool RowsVectorisable(const void *base, int rank, const int64_t *shape, int axis, const int64_t *strides) {
+  if (!IsAligned(base, 16) || (shape[axis] > 1 && strides[axis] != 1)) return false;
+  for (int i = 0; i < rank; ++i) {
+    if (i != axis && shape[i] > 1 && strides[i] % 4 != 0) return false;
+  }
+  return true;
+}
+// True when an operand's address depends only on the position along the axis (scale and bias of a
+// LayerNormalization over the last dim).
+inline bool RowInvariant(int rank, const int64_t *shape, int axis, const int64_t *strides) {
+  for (int i = 0; i < rank; ++i) {
+    if (i != axis && shape[i] > 1 && strides[i] != 0) return false;
+  }
+  return true;
+}
+// Row kernels switch to the many-rows variants from this many elements on (below, the launches of the
+// transformer graphs keep the kernels they were tuned with).
+constexpr int64_t kManyRowsElements = int64_t{1} << 20;
 
 // ---- Softmax ----------------------------------------------------------------
 
@@ -104,7 +127,72 @@ __global__ __launch_bounds__(kBlock) void SoftmaxRowWave(RowArgs<3> a, float *__
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t j = lane + i * kWave;
-    if (j < a.len) dst[j] = x[i] / s;
+    if (j < a.len) StoreMaybeStreaming(dst + j, x[i] / s, a.streaming != 0);
+  }
+}
+
+// Many short rows: LANES lanes per row (64 / LANES rows per wave), 128-bit accesses, row cached in registers:
+// len <= 4 * LANES * ITEMS, len % 4 == 0, rows 16-byte aligned on both sides.
+struct alignas(16) Quad {
+  float v[4];
+};
+
+template <int LANES, typename F>
+__device__ __forceinline__ float GroupReduce(float v, F f) {
+#pragma unroll
+  for (int off = LANES / 2; off > 0; off >>= 1) v = f(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+template <int LANES, int ITEMS>
+__global__ __launch_bounds__(kBlock) void SoftmaxRowVec(RowArgs<3> a, float *__restrict__ out,
+                                                        const float *__restrict__ in, SoftmaxPre pre) {
+  const uint32_t lane = threadIdx.x % LANES;
+  const uint32_t row = blockIdx.x * (kBlock / LANES) + threadIdx.x / LANES;
+  if (row >= a.n_rows) return;  // a row's lanes leave together
+  int32_t off[3];
+  RowOffsets<3>(a.outer, row, off);
+  const Quad *src = reinterpret_cast<const Quad *>(in + off[1]);
+  Quad *dst = reinterpret_cast<Quad *>(out + off[0]);
+  const int32_t sm = a.axis_stride[2];
+  const uint32_t n_quads = a.len / 4;
+  Quad x[ITEMS];
+  float m = -__FLT_MAX__;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t q = lane + i * LANES;
+    if (q < n_quads) x[i] = src[q];
+  }
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t q = lane + i * LANES;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      x[i].v[k] = q < n_quads ? pre(x[i].v[k], off[2] + static_cast<int32_t>(4 * q + k) * sm) : -__FLT_MAX__;
+      m = fmaxf(m, x[i].v[k]);
+    }
+  }
+  m = GroupReduce<LANES>(m, MaxOp{});
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t q = lane + i * LANES;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      x[i].v[k] = q < n_quads ? expf(x[i].v[k] - m) : 0.0f;
+      s += x[i].v[k];
+    }
+  }
+  s = GroupReduce<LANES>(s, SumOp{});
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t q = lane + i * LANES;
+    if (q < n_quads) {
+      Quad r;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) r.v[k] = x[i].v[k] / s;
+      StoreMaybeStreaming(dst + q, r, a.streaming != 0);
+    }
   }
 }
 
@@ -157,7 +245,7 @@ __global__ __launch_bounds__(kBlock) void SoftmaxRowBlockCached(RowArgs<3> a, fl
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t j = threadIdx.x + i * kBlock;
-    if (j < a.len) dst[j] = x[i] / s;
+    if (j < a.len) StoreMaybeStreaming(dst + j, x[i] / s, a.streaming != 0);
   }
 }
 
@@ -222,7 +310,10 @@ __global__ __launch_bounds__(kBlock) void LayerNormRowBlock(RowArgs<6> a, float 
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t j = threadIdx.x + i * kBlock;
-    if (j < a.len) dst[j] = (x[i] * inv) * g[static_cast<int32_t>(j) * sg] + b[static_cast<int32_t>(j) * sb];
+    if (j < a.len) {
+      StoreMaybeStreaming(dst + j, (x[i] * inv) * g[static_cast<int32_t>(j) * sg] + b[static_cast<int32_t>(j) * sb],
+                          a.streaming != 0);
+    }
   }
 }
 
@@ -269,7 +360,98 @@ __global__ __launch_bounds__(kBlock) void LayerNormRowWave(RowArgs<6> a, float *
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t j = lane + i * kWave;
-    if (j < a.len) dst[j] = (x[i] * inv) * g[static_cast<int32_t>(j) * sg] + b[static_cast<int32_t>(j) * sb];
+    if (j < a.len) {
+      StoreMaybeStreaming(dst + j, (x[i] * inv) * g[static_cast<int32_t>(j) * sg] + b[static_cast<int32_t>(j) * sb],
+                          a.streaming != 0);
+    }
+  }
+}
+
+// Many rows: a workgroup copies scale and bias into LDS once, then each of its waves walks rows (one wave per
+// row, 128-bit accesses, row cached in registers): len <= 256 * ITEMS, len % 4 == 0, rows (and the addend's)
+// 16-byte aligned.  Dynamic LDS: 2 * len floats.
+template <int ITEMS>
+__global__ __launch_bounds__(kBlock) void LayerNormRowVec(RowArgs<6> a, float *__restrict__ out,
+                                                          const float *__restrict__ in,
+                                                          const float *__restrict__ scale,
+                                                          const float *__restrict__ bias,
+                                                          const float *__restrict__ scratch, float eps,
+                                                          int stale_scratch, const float *__restrict__ addend) {
+  extern __shared__ __align__(16) float ln_params[];  // scale[len], bias[len]
+  const uint32_t lane = threadIdx.x % kWave;
+  const uint32_t n_quads = a.len / 4;
+  {
+    // scale and bias do not depend on the row in this variant (the host checks it)
+    const int32_t sg = a.axis_stride[2], sb = a.axis_stride[3];
+    for (uint32_t j = threadIdx.x; j < a.len; j += kBlock) {
+      ln_params[j] = scale[static_cast<int32_t>(j) * sg];
+      ln_params[a.len + j] = bias[static_cast<int32_t>(j) * sb];
+    }
+  }
+  __syncthreads();
+  const Quad *gq = reinterpret_cast<const Quad *>(ln_params);
+  const Quad *bq = reinterpret_cast<const Quad *>(ln_params + a.len);
+  const float n = static_cast<float>(a.len);
+  const uint32_t row_step = gridDim.x * (kBlock / kWave);
+  for (uint32_t row = blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave; row < a.n_rows; row += row_step) {
+    int32_t off[6];
+    RowOffsets<6>(a.outer, row, off);
+    const Quad *src = reinterpret_cast<const Quad *>(in + off[1]);
+    Quad x[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t q = lane + i * kWave;
+      if (q < n_quads) x[i] = src[q];
+    }
+    if (addend != nullptr) {
+      const Quad *add = reinterpret_cast<const Quad *>(addend + off[5]);
+#pragma unroll
+      for (int i = 0; i < ITEMS; ++i) {
+        const uint32_t q = lane + i * kWave;
+        if (q < n_quads) {
+          const Quad y = add[q];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) x[i].v[k] = x[i].v[k] + y.v[k];
+        }
+      }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t q = lane + i * kWave;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (q >= n_quads) x[i].v[k] = 0.0f;
+        s += x[i].v[k];
+      }
+    }
+    s = WaveReduce(s, SumOp{});
+    if (stale_scratch) s += scratch[off[4]];
+    const float mean = s / n;
+    float v = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t q = lane + i * kWave;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        x[i].v[k] = q < n_quads ? x[i].v[k] - mean : 0.0f;
+        v += x[i].v[k] * x[i].v[k];
+      }
+    }
+    v = WaveReduce(v, SumOp{});
+    const float inv = 1.0f / sqrtf(v / n + eps);
+    Quad *dst = reinterpret_cast<Quad *>(out + off[0]);
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t q = lane + i * kWave;
+      if (q < n_quads) {
+        const Quad g = gq[q], b = bq[q];
+        Quad r;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) r.v[k] = (x[i].v[k] * inv) * g.v[k] + b.v[k];
+        StoreMaybeStreaming(dst + q, r, a.streaming != 0);
+      }
+    }
   }
 }
 
@@ -475,7 +657,23 @@ static int SoftmaxImpl(const fl_tensor *in, const fl_tensor *mask, float div, co
   const float *x = static_cast<const float *>(in->base);
   hipStream_t s = AsStream(stream);
   const bool row_contig = (a.axis_stride[0] == 1 && a.axis_stride[1] == 1) || a.len == 1;
-  if (row_contig && a.len > 16) {
+  const bool many_rows = static_cast<int64_t>(a.n_rows) * a.len >= kManyRowsElements && a.len % 4 == 0 && a.len >= 32 &&
+                         a.len <= 1024 && RowsVectorisable(out->base, in->rank, in->shape, static_cast<int>(axis), strides[0]) &&
+                         RowsVectorisable(in->base, in->rank, in->shape, static_cast<int>(axis), strides[1]);
+  if (many_rows) {
+    auto blocks = [&](uint32_t lanes) { return dim3((a.n_rows + kBlock / lanes - 1) / (kBlock / lanes)); };
+    if (a.len <= 64) {
+      FL_LAUNCH((SoftmaxRowVec<8, 2>), blocks(8), dim3(kBlock), 0, s, a, o, x, pre);
+    } else if (a.len <= 128) {
+      FL_LAUNCH((SoftmaxRowVec<16, 2>), blocks(16), dim3(kBlock), 0, s, a, o, x, pre);
+    } else if (a.len <= 256) {
+      FL_LAUNCH((SoftmaxRowVec<16, 4>), blocks(16), dim3(kBlock), 0, s, a, o, x, pre);
+    } else if (a.len <= 512) {
+      FL_LAUNCH((SoftmaxRowVec<32, 4>), blocks(32), dim3(kBlock), 0, s, a, o, x, pre);
+    } else {
+      FL_LAUNCH((SoftmaxRowVec<64, 4>), blocks(64), dim3(kBlock), 0, s, a, o, x, pre);
+    }
+  } else if (row_contig && a.len > 16) {
     const uint32_t wave_blocks = (a.n_rows + kBlock / kWave - 1) / (kBlock / kWave);
     if (a.len <= 64) {
       FL_LAUNCH(SoftmaxRowWave<1>, dim3(wave_blocks), dim3(kBlock), 0, s, a, o, x, pre);
@@ -566,7 +764,38 @@ static int LayerNormImpl(const fl_tensor *in, const fl_tensor *addend, const fl_
   const float eps = static_cast<float>(epsilon);
   hipStream_t s = AsStream(stream);
   const bool row_contig = a.axis_stride[0] == 1 && a.axis_stride[1] == 1;
-  if (row_contig && a.len > 64) {
+  const int ax = static_cast<int>(axis);
+  const bool many_rows = static_cast<int64_t>(a.n_rows) * a.len >= kManyRowsElements && a.len % 4 == 0 && a.len >= 256 &&
+                         a.len <= 16 * 256 && RowsVectorisable(out->base, in->rank, in->shape, ax, strides[0]) &&
+                         RowsVectorisable(in->base, in->rank, in->shape, ax, strides[1]) &&
+                         (y == nullptr || RowsVectorisable(y, in->rank, in->shape, ax, strides[5])) &&
+                         RowInvariant(in->rank, in->shape, ax, strides[2]) && RowInvariant(in->rank, in->shape, ax, strides[3]);
+  if (many_rows) {
+    // eight workgroups per compute unit at most: each keeps its copy of scale and bias for many rows
+    const dim3 wave_grid(std::min<uint32_t>((a.n_rows + kBlock / kWave - 1) / (kBlock / kWave), 256 * 8));
+    const size_t lds_bytes = 2 * static_cast<size_t>(a.len) * sizeof(float);
+    const uint32_t items = (a.len + 255) / 256;
+#define FL_LN_VEC(ITEMS) \
+  FL_LAUNCH(LayerNormRowVec<ITEMS>, wave_grid, dim3(kBlock), lds_bytes, s, a, o, x, g, b, sc, eps, stale, y)
+    if (items <= 1) {
+      FL_LN_VEC(1);
+    } else if (items <= 2) {
+      FL_LN_VEC(2);
+    } else if (items <= 3) {
+      FL_LN_VEC(3);
+    } else if (items <= 4) {
+      FL_LN_VEC(4);
+    } else if (items <= 6) {
+      FL_LN_VEC(6);
+    } else if (items <= 8) {
+      FL_LN_VEC(8);
+    } else if (items <= 12) {
+      FL_LN_VEC(12);
+    } else {
+      FL_LN_VEC(16);
+    }
+#undef FL_LN_VEC
+  } else if (row_contig && a.len > 64) {
     const dim3 wave_grid((a.n_rows + kBlock / kWave - 1) / (kBlock / kWave));
     if (a.len <= 4 * kWave) {
       FL_LAUNCH(LayerNormRowWave<4>, wave_grid, dim3(kBlock), 0, s, a, o, x, g, b, sc, eps, stale, y);

@@ -468,7 +468,8 @@ def test_pools(device):
     cabi = _cabi()
     rng = np.random.default_rng(42)
     cases = [((1, 8, 56, 56), (2, 2), (2, 2)), ((1, 40, 7, 7), (7, 7), (1, 1)), ((2, 3, 9, 11), (3, 2), (2, 3)),
-             ((1, 4, 30), (3,), (2,))]
+             ((1, 4, 30), (3,), (2,)), ((2, 5, 14, 28), (2, 2), (2, 2)), ((1, 3, 13, 12), (2, 2), (3, 2)),
+             ((1, 2, 10, 10), (2, 2), (2, 2)), ((1, 3, 8, 16), (2, 2), (2, 1))]
     for shape, k, s in cases:
         x = rand(rng, shape)
         n = len(k)
@@ -481,6 +482,58 @@ def test_pools(device):
                 dx, do = DeviceView(hx, device), DeviceView(ok.View.empty(oshape, np.float32, lin), device)
                 cabi.call(name, dx.ref(), do.ref(), cabi.i64_array(k), cabi.i64_array(s), n, None)
                 assert_close(do.logical(), ho.logical(), exact=True, what=name)
+
+
+def test_large_outputs(device):
+    """Outputs of 64 MiB and more take the non-temporal store path (and the widest launch grids): the same
+    oracle comparison as the small cases, one layout each."""
+    cabi = _cabi()
+    rng = np.random.default_rng(2718)
+
+    def run(what, host_inputs, oshape, oracle, call, exact):
+        announce("large", what, oshape)
+        ho = ok.View.empty(oshape, np.float32)
+        oracle(*host_inputs, ho)
+        devs = [DeviceView(h, device) for h in host_inputs]
+        do = DeviceView(ok.View.empty(oshape, np.float32), device)
+        call(*[d.ref() for d in devs], do.ref())
+        assert_close(do.logical(), ho.logical(), exact=exact, what=f"large {what}")
+
+    shape = (4100, 4096)  # 64.06 MiB
+    x = rand(rng, shape)
+    run("relu", [ok.View(x)], shape, lambda a, o: ok.unary_f32(ok.OP_RELU, a, o, 0, 0),
+        lambda a, o: cabi.call("relu", a, o, None), True)
+    row = rand(rng, (4096,))
+    run("add_common (row broadcast)", [ok.View(x), ok.View(row)], shape, lambda a, b, o: ok.binary_f32(ok.BOP_ADD, a, b, o),
+        lambda a, b, o: cabi.call("add_common", a, b, o, None), True)
+    chain = cabi.make_chain([(cabi.EW_MUL_C, 0.5), (cabi.EW_RELU, 0), (cabi.EW_ADD_X, 0)])
+
+    def chain_oracle(a, o):
+        t0, t1 = ok.View.empty(shape, np.float32), ok.View.empty(shape, np.float32)
+        ok.unary_f32(ok.OP_MUL_C, a, t0, 0.5, 0)
+        ok.unary_f32(ok.OP_RELU, t0, t1, 0, 0)
+        ok.binary_f32(ok.BOP_ADD, t1, a, o)
+
+    run("elementwise_chain", [ok.View(x)], shape, chain_oracle,
+        lambda a, o: cabi.call("elementwise_chain", a, o, ctypes.byref(chain), None), True)
+    for sshape in [(131080, 128), (16400, 1024)]:
+        xs = rand(rng, sshape, -6, 6)
+        run(f"softmax {sshape}", [ok.View(xs)], sshape, lambda a, o: ok.softmax(a, o, 1),
+            lambda a, o: cabi.call("softmax", a, o, None, 0, ctypes.c_int64(1), None), False)
+    lshape = (21900, 768)
+    xl, g, b = rand(rng, lshape, -3, 3), rand(rng, (768,), 0.5, 1.5), rand(rng, (768,), -0.5, 0.5)
+    run("layer_norm", [ok.View(xl), ok.View(g), ok.View(b)], lshape, lambda a, gg, bb, o: ok.layer_norm(a, gg, bb, o, 1, 1e-5),
+        lambda a, gg, bb, o: cabi.call("layer_normalization_constant_scale_bias", a, gg, bb, o, None, 0, ctypes.c_int64(1),
+                                       ctypes.c_double(1e-5), ctypes.c_uint32(0), None), False)
+    tshape = (4160, 4128)
+    xt = rand(rng, tshape)
+    run("transpose", [ok.View(xt)], (4128, 4160), lambda a, o: ok.transpose(a, o, (1, 0)),
+        lambda a, o: cabi.call("transpose", a, o, cabi.i64_array((1, 0)), 2, None), True)
+    pshape, two = (16, 64, 264, 256), cabi.i64_array((2, 2))
+    xp = rand(rng, pshape)
+    for is_max, name in [(True, "max_pool_without_padding"), (False, "average_pool_without_padding")]:
+        run(name, [ok.View(xp)], (16, 64, 132, 128), lambda a, o, m=is_max: ok.pool(m, a, o, (2, 2), (2, 2)),
+            lambda a, o, nm=name: cabi.call(nm, a, o, two, two, 2, None), True)
 
 
 # --------------------------------------------------------------------------- contractions

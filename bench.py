@@ -112,6 +112,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-layers", type=int, default=3)
     ap.add_argument("--per-kernel", action="store_true", help="also print a per-kernel table to stderr")
+    ap.add_argument("--per-launch", action="store_true", help="also print every launch of one step, in order, to stderr")
     ap.add_argument("--bf16", action="store_true",
                     help="additionally run the opt-in bf16 contraction path and report its throughput and its "
                          "error against the fp32 result under \"bf16\" (the headline value stays fp32)")
@@ -240,6 +241,12 @@ def main():
         for name, k in sorted(by_launch_kind.items(), key=lambda kv: -kv[1]["ns"]):
             print(f"{name:48s} {k['launches']:8d} {k['ns'] / 1e3:10.1f} {k['ns'] / k['launches'] / 1e3:8.2f} "
                   f"{k['bytes'] / k['ns']:9.1f} {k['flops'] / k['ns'] / 1e3:8.2f}", file=sys.stderr)
+
+    if args.per_launch:
+        print(f"{'#':>4s} {'launch':60s} {'us':>9s} {'GB/s':>9s} {'TFLOP/s':>8s}", file=sys.stderr)
+        for i, t in enumerate(times):
+            print(f"{i:4d} {t['kernel'][:60]:60s} {t['ns'] / 1e3:9.2f} {t['bytes'] / t['ns']:9.1f} {t['flops'] / t['ns'] / 1e3:8.2f}",
+                  file=sys.stderr)
 
     result = {
         "metric": "inferences/sec at BERT-base seq128 fp32 on 1 MI355X" if args.config == "bert_base"

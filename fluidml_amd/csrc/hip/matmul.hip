@@ -706,11 +706,102 @@ __global__ __launch_bounds__(256) void SkinnyGemmKernel(float *__restrict__ C, c
   }
 }
 
+// The same for long K (K >= 2048): a whole workgroup owns ROWS columns n of C and its four waves split K, so that four
+// times as many waves stream weights at once (N = 4096, K = 25088: 8 waves per compute unit with the kernel above keep
+// ~8 MB in flight, too little to cover the memory latency at the HBM rate); the four partial sums of every output are
+// added in wave order through LDS.  Every workgroup reads all of A, whatever ROWS is: with M rows of A the caches
+// deliver M / ROWS bytes of A per byte of weights, so ROWS grows with M (M = 8, ROWS = 2: 1.6 GB of A through L2 for
+// 411 MB of weights, 129 us; the weights alone take 63 us at 6.5 TB/s).  STEPS k steps of 1024 per iteration.
+template <int MT, int ROWS, int STEPS>
+__global__ __launch_bounds__(256) void SkinnyGemmBlockKernel(float *__restrict__ C, const float *__restrict__ A,
+                                                             const float *__restrict__ B, MatmulArgs p) {
+  __shared__ float partial[4][MT][ROWS];
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int n0 = blockIdx.x * ROWS;
+  float acc[MT][ROWS];
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) acc[m][r] = 0.0f;
+  const float *brow[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) brow[r] = B + static_cast<int64_t>(min(n0 + r, p.N - 1)) * p.sBn;
+  for (int k = threadIdx.x * 4; k < p.K; k += 1024 * STEPS) {
+    floatx4 b[STEPS][ROWS], a[STEPS][MT];
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+      const bool live = k + 1024 * t < p.K;
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) {
+        b[t][r] = live ? *reinterpret_cast<const floatx4 *>(brow[r] + k + 1024 * t) : floatx4{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const float *arow = A + static_cast<int64_t>(m) * p.sAm + k + 1024 * t;
+        a[t][m] = m < p.M && live ? *reinterpret_cast<const floatx4 *>(arow) : floatx4{0, 0, 0, 0};
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t)
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+          acc[m][r] += a[t][m].x * b[t][r].x;
+          acc[m][r] += a[t][m].y * b[t][r].y;
+          acc[m][r] += a[t][m].z * b[t][r].z;
+          acc[m][r] += a[t][m].w * b[t][r].w;
+        }
+  }
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      const float v = WaveReduce(acc[m][r], SumOp{});
+      if (lane == 0) partial[wave][m][r] = v;
+    }
+  __syncthreads();
+  if (threadIdx.x < MT * ROWS) {
+    const int m = threadIdx.x / ROWS, r = threadIdx.x % ROWS, n = n0 + r;
+    if (m < p.M && n < p.N) {
+      float v = ((partial[0][m][r] + partial[1][m][r]) + partial[2][m][r]) + partial[3][m][r];
+      if (p.bias != nullptr) v = p.ca * v + p.cb * p.bias[m * p.sDm + n * p.sDn];
+      if (p.chain.n != 0) v = RunChain(p.chain, v);
+      C[static_cast<int64_t>(m) * p.sCm + static_cast<int64_t>(n) * p.sCn] = v;
+    }
+  }
+}
+
 // Launches the skinny kernel if the problem fits it; false = use the tiled kernel.
 inline bool TrySkinnyGemm(const MatmulArgs &p, int64_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   if (n_batch != 1 || p.M > 8 || p.N < 256 || p.K < 256 || p.n_inner != 0 || p.n_groups > 1) return false;
   if (p.sBk != 1 || p.sAk != 1 || p.K % 4 != 0 || p.sBn % 4 != 0 || (p.M > 1 && p.sAm % 4 != 0)) return false;
   if (!IsAligned(A, 16) || !IsAligned(B, 16)) return false;
+  if (p.K >= 2048) {
+    // columns per workgroup: as many as A has rows (at least two), while two workgroups per compute unit remain
+    const int mt = p.M == 1 ? 1 : p.M == 2 ? 2 : p.M <= 4 ? 4 : 8;
+    // (with K below 8192 a workgroup runs too few iterations for the wider variants to pay: 4096 x 4096 at M = 8
+    // takes 24.7 us with two columns, 27.8 us with eight)
+    int rows = p.K >= 8192 ? std::max(mt, 2) : 2;
+    while (rows > 1 && p.N / rows < 512) rows /= 2;
+#define FL_SKINNY_BLOCK(MT_, ROWS_)                                                                              \
+  FL_LAUNCH((SkinnyGemmBlockKernel<MT_, ROWS_, (MT_ * ROWS_ <= 8 ? 2 : 1)>), dim3((p.N + ROWS_ - 1) / ROWS_), dim3(256), 0, \
+            s, C, A, B, p)
+#define FL_SKINNY_ROWS(MT_)                    \
+  do {                                         \
+    if (rows == 8) FL_SKINNY_BLOCK(MT_, 8);    \
+    else if (rows == 4) FL_SKINNY_BLOCK(MT_, 4); \
+    else if (rows == 2) FL_SKINNY_BLOCK(MT_, 2); \
+    else FL_SKINNY_BLOCK(MT_, 1);              \
+  } while (0)
+    if (mt == 1) FL_SKINNY_ROWS(1);
+    else if (mt == 2) FL_SKINNY_ROWS(2);
+    else if (mt == 4) FL_SKINNY_ROWS(4);
+    else FL_SKINNY_ROWS(8);
+#undef FL_SKINNY_ROWS
+#undef FL_SKINNY_BLOCK
+    return true;
+  }
   // rows per wave: as many as still leave about eight waves per compute unit
   const int rows = p.N >= 4 * 2048 ? 4 : (p.N >= 2 * 2048 || p.M > 2) ? 2 : 1;
   const dim3 grid((p.N + 4 * rows - 1) / (4 * rows)), block(256);

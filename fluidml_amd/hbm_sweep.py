@@ -106,6 +106,17 @@ def run(repeats: int = 20, out=None) -> dict:
     vtab, vog = view(table), view(og)
     report("Gather [128,512] rows of 768 floats",
            lambda: cabi.call("gather_constant_data_tensor", ref(vid), ref(vtab), ref(vog), None), 2 * og.numel() * 4)
+    del table, ids, og, xi, xo
+    weights = torch.randn(4096, 25088, device=dev) * 0.01
+    bias = torch.zeros(4096, device=dev)
+    for batch in (1, 8):
+        act = torch.randn(batch, 25088, device=dev)
+        res = torch.empty(batch, 4096, device=dev)
+        va, vw, vbias, vres = view(act), view(weights), view(bias), view(res)
+        report(f"Gemm [{batch},25088] x [4096,25088]^T (weight streaming)",
+               lambda: cabi.call("gemm_constant_weights_bias", ref(va), ref(vw), ref(vbias), ref(vres), ctypes.c_double(1.0),
+                                 ctypes.c_double(1.0), 0, 1, ctypes.c_uint32(0), None),
+               (weights.numel() + act.numel() + res.numel() + bias.numel()) * 4)
     return {"metric": "achieved HBM bandwidth of the bandwidth-bound kernels", "unit": "GB/s", "peak": HBM_PEAK_GBPS,
             "repeats": repeats, "kernels": rows}
 

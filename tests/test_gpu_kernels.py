@@ -657,7 +657,9 @@ def test_gemm(device):
              ((100, 8), (50, 100), (8, 50), 1.5, 0.25, 1, 1), ((33, 65), (65, 17), (33, 17), 2.0, 3.0, 0, 0),
              # few rows against k-contiguous weights: the weight-streaming kernel (1, 2, 3..4 and 5..8 row variants)
              ((8, 2048), (1000, 2048), (1000,), 1.0, 1.0, 0, 1), ((3, 4096), (515, 4096), (515,), 1.0, 1.0, 0, 1),
-             ((2, 1024), (300, 1024), (2, 300), 0.5, 2.0, 0, 1), ((5, 512), (257, 512), (257,), 1.0, 1.0, 0, 1)]
+             ((2, 1024), (300, 1024), (2, 300), 0.5, 2.0, 0, 1), ((5, 512), (257, 512), (257,), 1.0, 1.0, 0, 1),
+             # long K: a workgroup per one or two weight rows, K split over its waves (K not a multiple of the step)
+             ((1, 3588), (4099, 3588), (4099,), 1.0, 1.0, 0, 1), ((6, 2052), (4100, 2052), (4100,), 1.0, 0.5, 0, 1)]
     for ashape, bshape, cshape, alpha, beta, ta, tb in cases:
         a, b, c = rand(rng, ashape, -1, 1), rand(rng, bshape, -0.05, 0.05), rand(rng, cshape, -1, 1)
         M = ashape[1] if ta else ashape[0]

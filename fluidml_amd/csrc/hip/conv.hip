@@ -203,6 +203,222 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
   return LaunchStatus();
 }
 
+// ---- two pointwise convolutions on one pixel (squeeze-and-excitation) ---------------------------------------
+// hidden[s] = chain1(sum_c w1[s][c] * in[c] + b1[s]);  out[f] = chain2(sum_s w2[f][s] * hidden[s] + b2[f]).
+// A workgroup of 16 waves owns 1024 outputs f of one image and recomputes the whole hidden vector (a few thousand
+// multiply-adds).  Everything here is a chain of dependent round trips to memory, so each phase issues all its
+// loads before it uses any: the input goes to LDS; wave w takes hidden channels w, w + 16, .. two at a time, its
+// lanes holding up to QUADS 128-bit pieces of each weight row (wave64 shuffle sum); then one lane per output walks
+// its weight row sixteen values at a time against the hidden vector in LDS.
+constexpr int kPairBlock = 1024;
+constexpr int kPairMaxChannels = 4096, kPairMaxHidden = 512;
+
+struct ConvPairArgs {
+  int32_t channels, hidden, outputs;
+  int32_t in_n, in_c, out_n, out_f;  // element strides
+  int32_t w1_s, w1_c, w2_f, w2_s;
+  int32_t b1_stride, b2_stride;      // 0: no bias (the pointer is null)
+  int32_t vec1, vec2;                // rows of w1 / w2 can be read 16 bytes at a time
+  fl_ew_program chain1, chain2;
+};
+
+struct alignas(16) PairQuad {
+  float v[4];
+};
+
+template <int QUADS>
+__global__ __launch_bounds__(kPairBlock) void ConvPairKernel(ConvPairArgs p, float *__restrict__ out,
+                                                             const float *__restrict__ in,
+                                                             const float *__restrict__ w1, const float *__restrict__ b1,
+                                                             const float *__restrict__ w2, const float *__restrict__ b2) {
+  __shared__ __align__(16) float x[kPairMaxChannels];
+  __shared__ __align__(16) float hidden[kPairMaxHidden];
+  constexpr int kWaves = kPairBlock / kWave;
+  const int image = blockIdx.y;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int f = blockIdx.x * kPairBlock + threadIdx.x;
+  const bool live = f < p.outputs;
+  const float *row2 = w2 + static_cast<int64_t>(live ? f : 0) * p.w2_f;
+  const int n_quads = p.channels / 4, hidden_quads = p.hidden / 4;
+  // the first loads of both phases do not depend on anything computed here: they are issued before the input
+  // is staged, so that the common case (at most 32 channels in between) waits for memory once
+  PairQuad a0[QUADS], a1[QUADS], wq[4];
+  float ws[16];
+  auto load_rows = [&](int s0) {
+    const int s1 = s0 + kWaves < p.hidden ? s0 + kWaves : s0;
+    const PairQuad *row0 = reinterpret_cast<const PairQuad *>(w1 + static_cast<int64_t>(s0) * p.w1_s);
+    const PairQuad *row1 = reinterpret_cast<const PairQuad *>(w1 + static_cast<int64_t>(s1) * p.w1_s);
+#pragma unroll
+    for (int k = 0; k < QUADS; ++k) {
+      const int q = lane + k * kWave;
+      a0[k] = q < n_quads ? row0[q] : PairQuad{{0, 0, 0, 0}};
+      a1[k] = q < n_quads ? row1[q] : PairQuad{{0, 0, 0, 0}};
+    }
+  };
+  auto load_quads = [&](int q0) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) wq[k] = q0 + k < hidden_quads ? reinterpret_cast<const PairQuad *>(row2)[q0 + k] : PairQuad{{0, 0, 0, 0}};
+  };
+  auto load_scalars = [&](int s0) {
+#pragma unroll
+    for (int k = 0; k < 16; ++k) ws[k] = s0 + k < p.hidden ? row2[(s0 + k) * p.w2_s] : 0.0f;
+  };
+  if (p.vec1 && wave < p.hidden) load_rows(wave);
+  if (live) {
+    if (p.vec2) load_quads(0);
+    else load_scalars(0);
+  }
+  // the biases too: a load issued only after the sums are known would be one more trip to memory each
+  float bias_first0 = 0.0f, bias_first1 = 0.0f, bias_out = 0.0f;
+  if (b1 != nullptr && wave < p.hidden) {
+    bias_first0 = b1[wave * p.b1_stride];
+    if (wave + kWaves < p.hidden) bias_first1 = b1[(wave + kWaves) * p.b1_stride];
+  }
+  if (b2 != nullptr && live) bias_out = b2[f * p.b2_stride];
+  const float *src = in + static_cast<int64_t>(image) * p.in_n;
+  for (int c = threadIdx.x; c < p.channels; c += kPairBlock) x[c] = src[c * p.in_c];
+  __syncthreads();
+  if (p.vec1) {
+    for (int s0 = wave; s0 < p.hidden; s0 += 2 * kWaves) {
+      const int s1 = s0 + kWaves;
+      const bool second = s1 < p.hidden;
+      if (s0 != wave) load_rows(s0);
+      float acc0 = 0.0f, acc1 = 0.0f;
+#pragma unroll
+      for (int k = 0; k < QUADS; ++k) {
+        const int q = lane + k * kWave;
+        if (q < n_quads) {
+          const PairQuad xv = reinterpret_cast<const PairQuad *>(x)[q];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            acc0 += a0[k].v[e] * xv.v[e];
+            acc1 += a1[k].v[e] * xv.v[e];
+          }
+        }
+      }
+      acc0 = WaveReduce(acc0, SumOp{});
+      acc1 = WaveReduce(acc1, SumOp{});
+      if (lane == 0) {
+        if (b1 != nullptr) acc0 += s0 == wave ? bias_first0 : b1[s0 * p.b1_stride];
+        hidden[s0] = p.chain1.n != 0 ? RunChain(p.chain1, acc0) : acc0;
+        if (second) {
+          if (b1 != nullptr) acc1 += s0 == wave ? bias_first1 : b1[s1 * p.b1_stride];
+          hidden[s1] = p.chain1.n != 0 ? RunChain(p.chain1, acc1) : acc1;
+        }
+      }
+    }
+  } else {
+    for (int s = wave; s < p.hidden; s += kWaves) {
+      const float *row = w1 + static_cast<int64_t>(s) * p.w1_s;
+      float acc = 0.0f;
+#pragma unroll 8
+      for (int c = lane; c < p.channels; c += kWave) acc += row[c * p.w1_c] * x[c];
+      acc = WaveReduce(acc, SumOp{});
+      if (lane == 0) {
+        if (b1 != nullptr) acc += b1[s * p.b1_stride];
+        hidden[s] = p.chain1.n != 0 ? RunChain(p.chain1, acc) : acc;
+      }
+    }
+  }
+  __syncthreads();
+  if (!live) return;
+  float acc = 0.0f;
+  if (p.vec2) {
+    for (int q0 = 0; q0 < hidden_quads; q0 += 4) {
+      if (q0 != 0) load_quads(q0);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (q0 + k < hidden_quads) {
+          const PairQuad h = reinterpret_cast<const PairQuad *>(hidden)[q0 + k];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc += wq[k].v[e] * h.v[e];
+        }
+      }
+    }
+  } else {
+    for (int s0 = 0; s0 < p.hidden; s0 += 16) {
+      if (s0 != 0) load_scalars(s0);
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        if (s0 + k < p.hidden) acc += ws[k] * hidden[s0 + k];
+      }
+    }
+  }
+  acc += bias_out;
+  if (p.chain2.n != 0) acc = RunChain(p.chain2, acc);
+  out[static_cast<int64_t>(image) * p.out_n + static_cast<int64_t>(f) * p.out_f] = acc;
+}
+
+// [N, C, 1...] tensors: every dim from the third on has extent 1
+inline bool OnePixel(const fl_tensor *t) {
+  if (t->rank < 2) return false;
+  for (int i = 2; i < t->rank; ++i) {
+    if (t->shape[i] != 1) return false;
+  }
+  return true;
+}
+
+int ConvPair(const fl_tensor *in, const fl_tensor *w1, const fl_tensor *b1, const fl_ew_program *chain1,
+             const fl_tensor *w2, const fl_tensor *b2, const fl_ew_program *chain2, const fl_tensor *out, void *stream) {
+  if (!in || !w1 || !w2 || !out) return FL_ERR_NULL;
+  const fl_tensor *all[6] = {in, w1, w2, out, b1, b2};
+  for (const fl_tensor *t : all) {
+    if (t == nullptr) continue;
+    FL_CHECK(CheckView(t));
+    if (t->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  }
+  if (!OnePixel(in) || !OnePixel(w1) || !OnePixel(w2) || !OnePixel(out)) return FL_ERR_SHAPE;
+  const int64_t n = in->shape[0], c = in->shape[1], s = w1->shape[0], f = w2->shape[0];
+  if (w1->shape[1] != c || w2->shape[1] != s || out->shape[0] != n || out->shape[1] != f) return FL_ERR_SHAPE;
+  if ((b1 && Numel(b1) != s) || (b2 && Numel(b2) != f)) return FL_ERR_SHAPE;
+  if (c > kPairMaxChannels || s > kPairMaxHidden || n > 65535) return FL_ERR_UNSUPPORTED;
+  if (n == 0 || f == 0) return FL_OK;
+  auto last_stride = [](const fl_tensor *t) {  // element stride of a tensor with one non-unit dim
+    for (int i = 0; i < t->rank; ++i) {
+      if (t->shape[i] != 1) return static_cast<int32_t>(t->strides[i]);
+    }
+    return int32_t{1};
+  };
+  ConvPairArgs p;
+  std::memset(&p, 0, sizeof(p));
+  p.channels = static_cast<int32_t>(c);
+  p.hidden = static_cast<int32_t>(s);
+  p.outputs = static_cast<int32_t>(f);
+  p.in_n = static_cast<int32_t>(in->strides[0]);
+  p.in_c = static_cast<int32_t>(in->strides[1]);
+  p.out_n = static_cast<int32_t>(out->strides[0]);
+  p.out_f = static_cast<int32_t>(out->strides[1]);
+  p.w1_s = static_cast<int32_t>(w1->strides[0]);
+  p.w1_c = static_cast<int32_t>(w1->strides[1]);
+  p.w2_f = static_cast<int32_t>(w2->strides[0]);
+  p.w2_s = static_cast<int32_t>(w2->strides[1]);
+  p.b1_stride = b1 ? last_stride(b1) : 0;
+  p.b2_stride = b2 ? last_stride(b2) : 0;
+  if (chain1 != nullptr) p.chain1 = *chain1;
+  if (chain2 != nullptr) p.chain2 = *chain2;
+  if (p.chain1.n > FL_EW_MAX_STEPS || p.chain2.n > FL_EW_MAX_STEPS) return FL_ERR_ATTR;
+  p.vec1 = c % 4 == 0 && p.w1_c == 1 && p.w1_s % 4 == 0 && IsAligned(w1->base, 16) ? 1 : 0;
+  p.vec2 = s % 4 == 0 && p.w2_s == 1 && p.w2_f % 4 == 0 && IsAligned(w2->base, 16) ? 1 : 0;
+  const dim3 grid(static_cast<uint32_t>((f + kPairBlock - 1) / kPairBlock), static_cast<uint32_t>(n));
+#define FL_CONV_PAIR(QUADS)                                                                                        \
+  FL_LAUNCH(ConvPairKernel<QUADS>, grid, dim3(kPairBlock), 0, AsStream(stream), p, static_cast<float *>(out->base), \
+            static_cast<const float *>(in->base), static_cast<const float *>(w1->base),                           \
+            b1 ? static_cast<const float *>(b1->base) : nullptr, static_cast<const float *>(w2->base),            \
+            b2 ? static_cast<const float *>(b2->base) : nullptr)
+  if (c > 8 * 256) p.vec1 = 0;  // two rows of more than 2048 values do not fit a wave's registers: strided loop
+  if (c <= 4 * 256) {
+    FL_CONV_PAIR(4);
+  } else if (c <= 5 * 256) {
+    FL_CONV_PAIR(5);
+  } else if (c <= 6 * 256) {
+    FL_CONV_PAIR(6);
+  } else {
+    FL_CONV_PAIR(8);
+  }
+#undef FL_CONV_PAIR
+  return LaunchStatus();
+}
+
 }  // namespace
 }  // namespace fl
 
@@ -228,6 +444,12 @@ int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const 
                            const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group,
                            const fl_ew_program *chain, void *stream) {
   return fl::Conv(in, weights, bias, out, pads, strides, dilations, group, 0, stream, chain);
+}
+
+int fluidml_hip_pointwise_conv_pair(const fl_tensor *in, const fl_tensor *weights1, const fl_tensor *bias1,
+                                    const fl_ew_program *chain1, const fl_tensor *weights2, const fl_tensor *bias2,
+                                    const fl_ew_program *chain2, const fl_tensor *out, void *stream) {
+  return fl::ConvPair(in, weights1, bias1, chain1, weights2, bias2, chain2, out, stream);
 }
 
 }  // extern "C"

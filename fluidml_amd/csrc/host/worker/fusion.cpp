@@ -24,6 +24,7 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::MatMulGroup: return "MatMulGroup";
     case Launch::Kind::GemmChain: return "GemmChain";
     case Launch::Kind::ConvChain: return "ConvChain";
+    case Launch::Kind::ConvPair: return "ConvPair";
     case Launch::Kind::ElementwiseChain: return "ElementwiseChain";
     case Launch::Kind::MulAdd: return "MulAdd";
     case Launch::Kind::AddAdd: return "AddAdd";
@@ -245,7 +246,10 @@ class Scheduler {
           case OpKind::MatMul:
           case OpKind::GemmConstantWeightsBias:
           case OpKind::ConvWithPadding:
-          case OpKind::ConvWithoutPadding: l = MatchContraction(i); break;
+          case OpKind::ConvWithoutPadding:
+            l = MatchConvPair(i);
+            if (!l) l = MatchContraction(i);
+            break;
           case OpKind::MulCommon: l = MatchMulAdd(i); break;
           case OpKind::AddCommon: l = MatchAddAdd(i); break;
           case OpKind::GatherConstantDataTensor: l = MatchGatherAdd(i); break;
@@ -854,6 +858,58 @@ class Scheduler {
       l.chain = fl_ew_program{};
     }
     return std::nullopt;
+  }
+
+  // A convolution that is a matrix-vector product per image: group 1, one input pixel, one tap, no padding
+  // (the two convolutions of a squeeze-and-excitation block behind the global pooling).
+  bool PointwiseOnOnePixel(size_t i) const {
+    if (Kind(i) != OpKind::ConvWithoutPadding) return false;
+    const Step &st = steps_[i];
+    const auto &in = st.in0.meta.GetShape(), &w = st.in1.meta.GetShape(), &out = st.out.meta.GetShape();
+    if (!IsFloat(st.in0) || !IsFloat(st.in1) || !IsFloat(st.out) || Attrs(i).group != 1) return false;
+    if (in.size() < 3 || w.size() != in.size() || out.size() != in.size() || w[1] != in[1]) return false;
+    for (size_t d = 2; d < in.size(); ++d) {
+      if (in[d] != 1 || w[d] != 1 || out[d] != 1) return false;
+    }
+    return true;
+  }
+
+  // Conv -> chain -> Conv -> chain on one-pixel tensors: one launch of fluidml_hip_pointwise_conv_pair
+  std::optional<Launch> MatchConvPair(size_t i) {
+    if (!PointwiseOnOnePixel(i)) return std::nullopt;
+    Launch l;
+    l.kind = Launch::Kind::ConvPair;
+    l.a = steps_[i].in0;
+    l.b = steps_[i].in1;
+    l.owner = i;
+    l.members = {i};
+    size_t last = i;
+    if (const auto chain = ConsumingChain(i)) {
+      l.members.insert(l.members.end(), chain->members.begin(), chain->members.end());
+      l.chain = chain->program;
+      last = chain->members.back();
+    }
+    const auto j = SoleReader(last);
+    if (!j || !PointwiseOnOnePixel(*j) || !SameTensor(steps_[*j].in0, steps_[last].out)) return std::nullopt;
+    // the kernel's limits, so that the launch can never be refused at replay time
+    if (steps_[i].in0.meta.GetShape()[1] > 4096 || steps_[*j].in0.meta.GetShape()[1] > 512 ||
+        steps_[i].in0.meta.GetShape()[0] > 65535) {
+      return std::nullopt;
+    }
+    l.members.push_back(*j);
+    l.c = steps_[*j].in1;
+    l.owner2 = *j;
+    if (const auto chain = ConsumingChain(*j)) {
+      l.members.insert(l.members.end(), chain->members.begin(), chain->members.end());
+      l.chain2 = chain->program;
+    }
+    std::sort(l.members.begin(), l.members.end());
+    l.out = steps_[l.members.back()].out;
+    if (!Safe(l.members, {{i, l.a}, {i, l.b}, {*j, l.c}}) || !OutputDisjoint(l.out, {&l.a, &l.b, &l.c})) return std::nullopt;
+    l.bytes = Bytes({&l.a, &l.b, &l.c, &l.out}) + static_cast<double>(steps_[i].kernel->GetConstantBytes()) +
+              static_cast<double>(steps_[*j].kernel->GetConstantBytes());
+    l.flops = Flops(l.members);
+    return l;
   }
 
   // Extends `l` (a MatMulChain headed by step `head`) by the longest run of single-reader Reshape / Transpose

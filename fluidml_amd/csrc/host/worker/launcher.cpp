@@ -290,6 +290,17 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
                                   at.strides.data(), at.dilations.data(), at.group, &l.chain, ctx.stream);
       break;
     }
+    case Launch::Kind::ConvPair: {
+      const kernel::TensorView w1 = ViewOf(Resolve(l.b), l.b), w2 = ViewOf(Resolve(l.c), l.c);
+      const kernel::DeviceConstant *bias1 = steps_[l.owner].kernel->GetConstant(0);
+      const kernel::DeviceConstant *bias2 = steps_[l.owner2].kernel->GetConstant(0);
+      kernel::TensorView b1, b2;
+      if (bias1 != nullptr) b1 = bias1->View();
+      if (bias2 != nullptr) b2 = bias2->View();
+      rc = fluidml_hip_pointwise_conv_pair(&a.t, &w1.t, bias1 ? &b1.t : nullptr, &l.chain, &w2.t, bias2 ? &b2.t : nullptr,
+                                           &l.chain2, &out.t, ctx.stream);
+      break;
+    }
     case Launch::Kind::ElementwiseChain:
       rc = fluidml_hip_elementwise_chain(&a.t, &out.t, &l.chain, ctx.stream);
       break;

@@ -66,6 +66,9 @@ struct Launch {
     MatMulChain,       // MatMul [-> AddCommon(rank-1 constant bias)] [-> elementwise chain]
     GemmChain,         // GemmConstantWeightsBias -> elementwise chain
     ConvChain,         // Conv{With,Without}Padding -> elementwise chain
+    ConvPair,          // two pointwise convolutions on one-pixel tensors, each with its elementwise chain
+                       // (squeeze-and-excitation): a = input, b = weights of `owner`, c = weights of `owner2`,
+                       // `chain` follows the first, `chain2` the second
     MatMulGroup,       // up to four MatMulChains that share the left operand and all extents, one launch
     ElementwiseChain,  // two or more elementwise steps on one tensor
     MulAdd,            // MulCommon -> AddCommon: a * b + c
@@ -108,7 +111,9 @@ struct Launch {
   std::vector<Launch> group;
   size_t position = 0;  // MatMulGroup: step index where the launch is issued (one of the members)
   fl_ew_program chain{};  // elementwise steps applied to the value (n == 0: none)
+  fl_ew_program chain2{};  // ConvPair: the steps after the second convolution
   size_t owner = 0;  // member whose kernel owns constants / attributes the launch needs (LayerNorm, Gemm, Conv)
+  size_t owner2 = 0;  // ConvPair: the second convolution
   double bytes = 0, flops = 0;
 };
 const char *LaunchKindName(Launch::Kind kind);

@@ -354,6 +354,11 @@ int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
 /* Conv{With,Without}PaddingKernel -> elementwise chain (reference conv.cpp:27-280);
  * `pads` may be NULL.  ONNX semantics only (no literal-reference flags). */
 int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, const fl_ew_program *chain, void *stream);
+/* Two pointwise convolutions on tensors of one pixel ([N, C, 1, ..]), each followed by an elementwise chain, as
+ * ONE launch: the squeeze-and-excitation pair Conv -> activation -> Conv -> activation behind a global pooling
+ * (reference conv.cpp:27-218 twice; both must have kernel size 1 and group 1, biases and chains may be NULL).
+ * At most 4096 input channels and 512 channels in between, else FL_ERR_UNSUPPORTED and nothing is launched. */
+int fluidml_hip_pointwise_conv_pair(const fl_tensor *in, const fl_tensor *weights1, const fl_tensor *bias1, const fl_ew_program *chain1, const fl_tensor *weights2, const fl_tensor *bias2, const fl_ew_program *chain2, const fl_tensor *out, void *stream);
 /* A chain of elementwise kernels on one float32 tensor as one launch:
  * out = chain(in), same shape, any two layouts. */
 int fluidml_hip_elementwise_chain(const fl_tensor *in, const fl_tensor *out, const fl_ew_program *chain, void *stream);

@@ -781,6 +781,44 @@ def test_matmul_chain_group(device):
     assert cabi.lib.fluidml_hip_matmul_chain_group(2, da.ref(), rhs_bad, bias, out, 0, None, None, 0, None) == -3  # FL_ERR_SHAPE
 
 
+def test_fused_pointwise_conv_pair(device):
+    """Conv 1x1 -> swish -> Conv 1x1 -> sigmoid on one-pixel tensors against the oracle's separate kernels."""
+    cabi = _cabi()
+    rng = np.random.default_rng(77)
+    swish = [(cabi.EW_DIV_C, 2.0), (cabi.EW_TANH, 0), (cabi.EW_ADD_C, 1.0), (cabi.EW_MUL_C, 0.5), (cabi.EW_MUL_X, 0)]
+    sigmoid = swish[:4]
+    oracle_op = {cabi.EW_DIV_C: ok.OP_DIV_C, cabi.EW_TANH: ok.OP_TANH, cabi.EW_ADD_C: ok.OP_ADD_C, cabi.EW_MUL_C: ok.OP_MUL_C}
+
+    def chain_on_host(v, steps):
+        cur = v
+        for op, c in steps:
+            nxt = ok.View.empty(v.shape, np.float32)
+            if op == cabi.EW_MUL_X:
+                ok.binary_f32(ok.BOP_MUL, cur, v, nxt)
+            else:
+                ok.unary_f32(oracle_op[op], cur, nxt, c, 0)
+            cur = nxt
+        return cur
+
+    for n, c, hidden, f, with_bias in [(1, 96, 4, 96, True), (2, 1152, 48, 1152, True), (3, 40, 10, 300, False),
+                                          (1, 2600, 6, 1030, True), (2, 37, 5, 9, True)]:
+        announce("pointwise_conv_pair", n, c, hidden, f, with_bias)
+        x = rand(rng, (n, c, 1, 1))
+        w1, w2 = rand(rng, (hidden, c, 1, 1), -0.2, 0.2), rand(rng, (f, hidden, 1, 1), -0.5, 0.5)
+        b1, b2 = rand(rng, (hidden,)), rand(rng, (f,))
+        hx, hw1, hw2, hb1, hb2 = ok.View(x), ok.View(w1), ok.View(w2), ok.View(b1), ok.View(b2)
+        mid, res = ok.View.empty((n, hidden, 1, 1), np.float32), ok.View.empty((n, f, 1, 1), np.float32)
+        ok.conv(hx, hw1, hb1 if with_bias else None, mid, None, (1, 1), (1, 1), 1, 0)
+        ok.conv(chain_on_host(mid, swish), hw2, hb2 if with_bias else None, res, None, (1, 1), (1, 1), 1, 0)
+        want = chain_on_host(res, sigmoid)
+        dx, dw1, dw2, db1, db2 = (DeviceView(h, device) for h in (hx, hw1, hw2, hb1, hb2))
+        do = DeviceView(ok.View.empty((n, f, 1, 1), np.float32), device)
+        p1, p2 = cabi.make_chain(swish), cabi.make_chain(sigmoid)
+        cabi.call("pointwise_conv_pair", dx.ref(), dw1.ref(), db1.ref() if with_bias else None, ctypes.byref(p1), dw2.ref(),
+                  db2.ref() if with_bias else None, ctypes.byref(p2), do.ref(), None)
+        assert_close(do.logical(), want.logical(), what="pointwise_conv_pair")
+
+
 def test_fused_mul_add(device):
     """MulCommon -> AddCommon in one launch: the product is rounded before the sum, so the result is the two
     kernels' bit for bit; all three inputs broadcast."""

@@ -355,7 +355,7 @@ SCHEDULE_NETS = {
     # without the rotary launch its steps go through the general mechanisms: views, Concat2 inputs written in place
     "gpt_neox_no_rotary": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120),
                            {"MatMulChain", "Attention", "View", "CopyInto", "MulAdd"}),
-    "efficientnet_b0": (lambda m: m.efficientnet_b0(image=64, classes=10, width_div=4), {"ConvChain"}),
+    "efficientnet_b0": (lambda m: m.efficientnet_b0(image=64, classes=10, width_div=4), {"ConvChain", "ConvPair"}),
     "vgg16": (lambda m: m.vgg16(batch=2, image=32, classes=10, width_div=8, fc=512), {"ConvChain", "GemmChain"}),
 }
 

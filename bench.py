@@ -23,10 +23,10 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the contraction kernel on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch, averaged over the 51 contraction launches of an inference), each scaled by what the
-# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x1.000): (6245.7 * 2.0 + 1447.8) KiB.
+# (KiB per dispatch, averaged over the 48 contraction launches of an inference), each scaled by what the
+# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x0.996): (6519.6 * 2.000 + 1464.0 * 0.996) KiB.
 # Only valid for the default workload (BERT-base, seq 128, 12 layers, plain_greedy, fusion on).
-MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 14_271_941
+MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 14_844_165
 
 
 def cpu_baseline(layers_total: int, sample_layers: int, seq: int):

@@ -303,6 +303,11 @@ def main():
     if not args.no_cpu_baseline:
         if args.config == "bert_base":
             result["cpu_baseline"] = cpu_baseline(args.layers, min(args.cpu_sample_layers, args.layers), args.seq)
+        elif batch > 1:
+            # the scalar loop nests take the same time for every image of a batch: time one image
+            one = {k: np.ascontiguousarray(v[:1]) for k, v in feeds.items()}
+            result["cpu_baseline"] = cpu_baseline_whole(models.vgg16(1), one, 1)
+            result["cpu_baseline"]["sample"] = f"one whole forward pass of ONE image of the batch of {batch} (the batch-1 graph)"
         else:
             result["cpu_baseline"] = cpu_baseline_whole(net, feeds, batch)
     print(json.dumps(result))

@@ -1,12 +1,15 @@
 #!/usr/bin/env python3
-"""Benchmark of the hot path: BERT-base encoder (batch 1, seq 128, fp32) compiled by
-Executor.make_dp_greedy-equivalent planning and replayed as HIP launches over one HBM arena.
+"""Benchmark of the hot path: BERT-base encoder (batch 1, seq 128, fp32) planned like the reference's
+Executor (plain_greedy by default) and replayed as HIP launches over one HBM arena.
 
-A "step" is one inference: one replay of the whole launch plan (416 graph nodes issued as 135 kernel
-launches after launch-level fusion) on inputs that are already resident in HBM.  Prints ONE JSON line; see DESIGN.md for how every field is derived.
+A "step" is one inference: one replay of the whole launch plan (416 graph nodes issued as 89 kernel
+launches after launch-level fusion) on inputs that are already resident in HBM.  Prints ONE JSON line:
+`value` = inferences/s over the timed replays; `roofline` = the contraction kernel's flops over its launch
+durations (dispatch begin/end timestamps) against the fp32 MFMA peak; `cpu_baseline` = the oracle's scalar loop
+nests on one host core for a bounded sample; `peak_hbm_bytes` = arena + constants + interface staging.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--executor plain_greedy|dp_greedy]
-                    [--no-cpu-baseline] [--layers 12]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--executor plain_greedy|dp_greedy]
+                    [--no-cpu-baseline] [--per-kernel] [--per-launch] [--bf16] [--hbm-kernels]
 """
 import argparse
 import json

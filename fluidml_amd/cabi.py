@@ -153,6 +153,7 @@ SIGNATURES = {
     "fluidml_hip_gemm_chain": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _vp, _vp],
     "fluidml_hip_conv_chain": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _vp],
     "fluidml_hip_pointwise_conv_pair": [_T, _T, _T, _vp, _T, _T, _vp, _T, _vp],
+    "fluidml_hip_softmax_matvec": [_T, _T, _T, _vp],
     "fluidml_hip_elementwise_chain": [_T, _T, _vp, _vp],
     "fluidml_hip_attention": [_T, _T, _T, _T, _f64, _i32, _T, _T, _f64, _vp],
     "fluidml_hip_div_add_softmax": [_T, _f64, _T, _T, _i64, _vp],

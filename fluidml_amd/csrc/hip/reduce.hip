@@ -629,6 +629,53 @@ __global__ __launch_bounds__(kBlock) void ReduceMeanThread(ReduceArgs a, float *
 
 using namespace fl;
 
+namespace fl {
+namespace {
+
+// ---- softmax over a short vector, then a matrix-vector product with it ------------------------------------------
+// out[b, m] = sum_k a[b, m, k] * softmax_k(v[b, :])  (the per-position kernel of a span-based dynamic
+// convolution: a handful of taps, softmaxed, applied to a window of values).  One lane per (b, m); the K <= 16
+// logits of batch b are read by every lane of that batch (served by the cache) and normalised in registers.
+constexpr int kMatVecMaxK = 16;
+
+struct SoftmaxMatVecArgs {
+  uint32_t n_items, rows;  // B * M, M
+  FastDiv div_rows;
+  int32_t k;
+  int32_t a_b, a_m, a_k, v_b, v_k, out_b, out_m;  // element strides
+};
+
+__global__ __launch_bounds__(kBlock) void SoftmaxMatVecKernel(SoftmaxMatVecArgs p, float *__restrict__ out,
+                                                              const float *__restrict__ a, const float *__restrict__ v) {
+  const uint32_t item = blockIdx.x * kBlock + threadIdx.x;
+  if (item >= p.n_items) return;
+  uint32_t b, m;
+  p.div_rows.DivMod(item, b, m);
+  const float *logits = v + static_cast<int64_t>(b) * p.v_b;
+  const float *row = a + static_cast<int64_t>(b) * p.a_b + static_cast<int64_t>(m) * p.a_m;
+  float x[kMatVecMaxK], w[kMatVecMaxK];
+  float top = -__FLT_MAX__;
+#pragma unroll
+  for (int t = 0; t < kMatVecMaxK; ++t) {
+    x[t] = t < p.k ? logits[t * p.v_k] : -__FLT_MAX__;
+    w[t] = t < p.k ? row[t * p.a_k] : 0.0f;
+    top = fmaxf(top, x[t]);
+  }
+  float sum = 0.0f;
+#pragma unroll
+  for (int t = 0; t < kMatVecMaxK; ++t) {
+    x[t] = t < p.k ? expf(x[t] - top) : 0.0f;
+    sum += x[t];
+  }
+  float acc = 0.0f;
+#pragma unroll
+  for (int t = 0; t < kMatVecMaxK; ++t) acc += w[t] * (x[t] / sum);
+  out[static_cast<int64_t>(b) * p.out_b + static_cast<int64_t>(m) * p.out_m] = acc;
+}
+
+}  // namespace
+}  // namespace fl
+
 extern "C" {
 
 static int SoftmaxImpl(const fl_tensor *in, const fl_tensor *mask, float div, const fl_tensor *out, int64_t axis,
@@ -901,6 +948,36 @@ int fluidml_hip_reduce_mean(const fl_tensor *in, const fl_tensor *out, const int
   } else {
     FL_LAUNCH(ReduceMeanThread, dim3((a.n_out + kBlock - 1) / kBlock), dim3(kBlock), 0, s, a, o, x);
   }
+  return LaunchStatus();
+}
+
+int fluidml_hip_softmax_matvec(const fl_tensor *a, const fl_tensor *logits, const fl_tensor *out, void *stream) {
+  using namespace fl;
+  FL_CHECK(CheckView(a));
+  FL_CHECK(CheckView(logits));
+  FL_CHECK(CheckView(out));
+  if (a->dtype != FL_FLOAT32 || logits->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  if (a->rank != 3 || logits->rank != 3 || out->rank != 3) return FL_ERR_RANK;
+  const int64_t batch = a->shape[0], rows = a->shape[1], k = a->shape[2];
+  if (logits->shape[0] != batch || logits->shape[1] != k || logits->shape[2] != 1 || out->shape[0] != batch ||
+      out->shape[1] != rows || out->shape[2] != 1) {
+    return FL_ERR_SHAPE;
+  }
+  if (k > kMatVecMaxK) return FL_ERR_UNSUPPORTED;
+  SoftmaxMatVecArgs p;
+  p.n_items = static_cast<uint32_t>(batch * rows);
+  p.rows = static_cast<uint32_t>(rows);
+  p.div_rows = FastDiv(static_cast<uint32_t>(rows));
+  p.k = static_cast<int32_t>(k);
+  p.a_b = static_cast<int32_t>(a->strides[0]);
+  p.a_m = static_cast<int32_t>(a->strides[1]);
+  p.a_k = static_cast<int32_t>(a->strides[2]);
+  p.v_b = static_cast<int32_t>(logits->strides[0]);
+  p.v_k = static_cast<int32_t>(logits->strides[1]);
+  p.out_b = static_cast<int32_t>(out->strides[0]);
+  p.out_m = static_cast<int32_t>(out->strides[1]);
+  FL_LAUNCH(SoftmaxMatVecKernel, dim3((p.n_items + kBlock - 1) / kBlock), dim3(kBlock), 0, AsStream(stream), p,
+            static_cast<float *>(out->base), static_cast<const float *>(a->base), static_cast<const float *>(logits->base));
   return LaunchStatus();
 }
 

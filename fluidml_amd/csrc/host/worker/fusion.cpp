@@ -25,6 +25,7 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::GemmChain: return "GemmChain";
     case Launch::Kind::ConvChain: return "ConvChain";
     case Launch::Kind::ConvPair: return "ConvPair";
+    case Launch::Kind::SoftmaxMatVec: return "SoftmaxMatVec";
     case Launch::Kind::ElementwiseChain: return "ElementwiseChain";
     case Launch::Kind::MulAdd: return "MulAdd";
     case Launch::Kind::AddAdd: return "AddAdd";
@@ -250,6 +251,7 @@ class Scheduler {
             l = MatchConvPair(i);
             if (!l) l = MatchContraction(i);
             break;
+          case OpKind::Softmax: l = MatchSoftmaxMatVec(i); break;
           case OpKind::MulCommon: l = MatchMulAdd(i); break;
           case OpKind::AddCommon: l = MatchAddAdd(i); break;
           case OpKind::GatherConstantDataTensor: l = MatchGatherAdd(i); break;
@@ -858,6 +860,39 @@ class Scheduler {
       l.chain = fl_ew_program{};
     }
     return std::nullopt;
+  }
+
+  // Softmax over the K <= 16 logits of [B, K, 1] whose only reader multiplies [B, M, K] with it (and whatever
+  // Reshape / Transpose views MatchContraction folds behind that MatMul): one launch of fluidml_hip_softmax_matvec
+  std::optional<Launch> MatchSoftmaxMatVec(size_t i) {
+    const Step &soft = steps_[i];
+    const auto &vs = soft.in0.meta.GetShape();
+    if (!IsFloat(soft.in0) || !IsFloat(soft.out) || vs.size() != 3 || vs[2] != 1 || vs[1] > 16) return std::nullopt;
+    const int64_t axis = Attrs(i).axis < 0 ? Attrs(i).axis + 3 : Attrs(i).axis;
+    if (axis != 1) return std::nullopt;
+    const auto j = SoleReader(i);
+    if (!j || Kind(*j) != OpKind::MatMul || !SameTensor(steps_[*j].in1, soft.out) || SameTensor(steps_[*j].in0, soft.out)) {
+      return std::nullopt;
+    }
+    const auto &as = steps_[*j].in0.meta.GetShape();
+    if (!IsFloat(steps_[*j].in0) || as.size() != 3 || as[0] != vs[0] || as[2] != vs[1]) return std::nullopt;
+    Launch l;
+    if (auto chain = MatchContraction(*j); chain && chain->kind == Launch::Kind::MatMulChain && !chain->has_c &&
+                                           chain->chain.n == 0 && chain->n_inner == 0) {
+      l = *chain;  // MatMul + the views folded behind it
+    } else {
+      l.members = {*j};
+      l.a = steps_[*j].in0;
+      l.out = steps_[*j].out;
+    }
+    l.kind = Launch::Kind::SoftmaxMatVec;
+    l.owner = *j;
+    l.b = soft.in0;
+    l.members.insert(l.members.begin(), i);
+    if (!Safe(l.members, {{i, l.b}, {*j, l.a}}) || !OutputDisjoint(l.out, {&l.a, &l.b})) return std::nullopt;
+    l.bytes = Bytes({&l.a, &l.b, &l.out});
+    l.flops = Flops(l.members);
+    return l;
   }
 
   // A convolution that is a matrix-vector product per image: group 1, one input pixel, one tap, no padding

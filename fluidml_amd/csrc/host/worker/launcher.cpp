@@ -290,6 +290,17 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
                                   at.strides.data(), at.dilations.data(), at.group, &l.chain, ctx.stream);
       break;
     }
+    case Launch::Kind::SoftmaxMatVec: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
+      if (l.view_strides.empty()) {
+        rc = fluidml_hip_softmax_matvec(&a.t, &b.t, &out.t, ctx.stream);
+      } else {
+        kernel::TensorView dst(out.t.base, steps_[l.owner].out.meta);
+        for (size_t d = 0; d < l.view_strides.size(); ++d) dst.t.strides[d] = l.view_strides[d];
+        rc = fluidml_hip_softmax_matvec(&a.t, &b.t, &dst.t, ctx.stream);
+      }
+      break;
+    }
     case Launch::Kind::ConvPair: {
       const kernel::TensorView w1 = ViewOf(Resolve(l.b), l.b), w2 = ViewOf(Resolve(l.c), l.c);
       const kernel::DeviceConstant *bias1 = steps_[l.owner].kernel->GetConstant(0);

@@ -69,6 +69,8 @@ struct Launch {
     ConvPair,          // two pointwise convolutions on one-pixel tensors, each with its elementwise chain
                        // (squeeze-and-excitation): a = input, b = weights of `owner`, c = weights of `owner2`,
                        // `chain` follows the first, `chain2` the second
+    SoftmaxMatVec,     // Softmax over <= 16 logits [B, K, 1] -> MatMul [B, M, K] x [B, K, 1] [-> Reshape views]:
+                       // a = the matrix, b = the logits, view_strides as for MatMulChain
     MatMulGroup,       // up to four MatMulChains that share the left operand and all extents, one launch
     ElementwiseChain,  // two or more elementwise steps on one tensor
     MulAdd,            // MulCommon -> AddCommon: a * b + c

@@ -354,6 +354,11 @@ int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
 /* Conv{With,Without}PaddingKernel -> elementwise chain (reference conv.cpp:27-280);
  * `pads` may be NULL.  ONNX semantics only (no literal-reference flags). */
 int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, const fl_ew_program *chain, void *stream);
+/* SoftmaxKernel over K <= 16 logits [B, K, 1] -> MatMulKernel [B, M, K] x [B, K, 1] as ONE launch:
+ * out[b, m, 0] = sum_k a[b, m, k] * softmax_k(logits[b, :, 0]) (reference softmax.cpp, matmul.cpp:28-59; the
+ * per-position kernel of a span-based dynamic convolution).  `out` is [B, M, 1] with the element strides
+ * these dims have inside the final buffer (a following Reshape is free).  K > 16: FL_ERR_UNSUPPORTED. */
+int fluidml_hip_softmax_matvec(const fl_tensor *a, const fl_tensor *logits, const fl_tensor *out, void *stream);
 /* Two pointwise convolutions on tensors of one pixel ([N, C, 1, ..]), each followed by an elementwise chain, as
  * ONE launch: the squeeze-and-excitation pair Conv -> activation -> Conv -> activation behind a global pooling
  * (reference conv.cpp:27-218 twice; both must have kernel size 1 and group 1, biases and chains may be NULL).

@@ -71,6 +71,11 @@ def test_full_size_fused_matches_unfused(device, config, tmp_path, monkeypatch):
     monkeypatch.setenv("FLUIDML_FUSE", "1")
     fused, fused_plan = _run(fluidml, net, feeds, path, config + "_fused")
     assert len(plain_plan["launches"]) == len(net.nodes) > len(fused_plan["launches"])
+    # the launch kinds each configuration is expected to exercise at full size
+    expected = {"bert_base": {"Attention", "MatMulGroup", "GatherAdd"}, "convbert_base": {"Attention", "SoftmaxMatVec"},
+                "gpt_neox": {"Attention", "Rotary", "AddAdd"}, "efficientnet_b0": {"ConvChain", "ConvPair"},
+                "vgg16_b1": {"ConvChain", "GemmChain"}}[config]
+    assert expected <= {l["kind"] for l in fused_plan["launches"]}
     for name, ref in plain.items():
         assert np.isfinite(ref).all()
         assert_close(fused[name], ref, what=f"{config} fused vs per-node {name}")

@@ -819,6 +819,35 @@ def test_fused_pointwise_conv_pair(device):
         assert_close(do.logical(), want.logical(), what="pointwise_conv_pair")
 
 
+def test_fused_softmax_matvec(device):
+    """Softmax over a few logits -> MatMul with the result against the oracle's two kernels; the output is written
+    through the strides of a reshaped buffer."""
+    cabi = _cabi()
+    rng = np.random.default_rng(123)
+    for batch, rows, k in [(768, 64, 9), (32, 16, 9), (5, 7, 16), (3, 130, 1)]:
+        announce("softmax_matvec", batch, rows, k)
+        a, v = rand(rng, (batch, rows, k)), rand(rng, (batch, k, 1), -4, 4)
+        ha, hv = ok.View(a), ok.View(v)
+        hs, ho = ok.View.empty((batch, k, 1), np.float32), ok.View.empty((batch, rows, 1), np.float32)
+        ok.softmax(hv, hs, 1)
+        ok.matmul(ha, hs, ho)
+        da, dv = DeviceView(ha, device), DeviceView(hv, device)
+        do = DeviceView(ok.View.empty((batch, rows, 1), np.float32), device)
+        cabi.call("softmax_matvec", da.ref(), dv.ref(), do.ref(), None)
+        assert_close(do.logical(), ho.logical(), what="softmax_matvec")
+        # transposed storage of the matrix and of the output
+        ha2 = ok.View(a, [2, 0, 1])
+        da2 = DeviceView(ha2, device)
+        do2 = DeviceView(ok.View.empty((batch, rows, 1), np.float32, [1, 0, 2]), device)
+        cabi.call("softmax_matvec", da2.ref(), dv.ref(), do2.ref(), None)
+        assert_close(do2.logical(), ho.logical(), what="softmax_matvec (strided)")
+    big = DeviceView(ok.View(rand(rng, (2, 3, 17))), device)
+    logits = DeviceView(ok.View(rand(rng, (2, 17, 1))), device)
+    res = DeviceView(ok.View.empty((2, 3, 1), np.float32), device)
+    with pytest.raises(cabi.FluidmlHipError):
+        cabi.call("softmax_matvec", big.ref(), logits.ref(), res.ref(), None)
+
+
 def test_fused_mul_add(device):
     """MulCommon -> AddCommon in one launch: the product is rounded before the sum, so the result is the two
     kernels' bit for bit; all three inputs broadcast."""

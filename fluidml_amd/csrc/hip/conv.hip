@@ -22,6 +22,7 @@ struct ConvArgs {
   int32_t rank;          // 2 + n_spatial
   int32_t n_spatial;
   int32_t out_shape[2 + kMaxSpatial];
+  FastDiv out_div[2 + kMaxSpatial];  // division by out_shape[i]
   int32_t in_shape[2 + kMaxSpatial];
   int32_t in_strides[2 + kMaxSpatial];
   int32_t w_strides[2 + kMaxSpatial];
@@ -37,7 +38,9 @@ struct ConvArgs {
   fl_ew_program chain;   // elementwise chain applied after the bias (n == 0: none)
 };
 
-template <int NS>
+// KH, KW: the window of the first two spatial dims when known at compile time (0 = read from the arguments): the tap
+// loops then unroll and their loads are issued together instead of one round trip per tap.  Same order of the sums.
+template <int NS, int KH = 0, int KW = 0>
 __global__ __launch_bounds__(kBlock) void ConvDirect(ConvArgs p, float *__restrict__ out, const float *__restrict__ in,
                                                      const float *__restrict__ w, const float *__restrict__ bias) {
   const uint32_t item = blockIdx.x * kBlock + threadIdx.x;
@@ -46,15 +49,18 @@ __global__ __launch_bounds__(kBlock) void ConvDirect(ConvArgs p, float *__restri
   int32_t both[2] = {0, 0};
   p.out_nest.AddOffsets(item, both);
   const int32_t ooff = both[0];
-  int32_t lin = both[1];
+  uint32_t lin = static_cast<uint32_t>(both[1]);
   int32_t o[NS];
 #pragma unroll
   for (int d = NS - 1; d >= 0; --d) {
-    o[d] = lin % p.out_shape[2 + d];
-    lin /= p.out_shape[2 + d];
+    uint32_t q, r;
+    p.out_div[2 + d].DivMod(lin, q, r);
+    o[d] = static_cast<int32_t>(r);
+    lin = q;
   }
-  const int32_t f = lin % p.out_shape[1];
-  const int32_t n = lin / p.out_shape[1];
+  uint32_t n_u, f_u;
+  p.out_div[1].DivMod(lin, n_u, f_u);
+  const int32_t f = static_cast<int32_t>(f_u), n = static_cast<int32_t>(n_u);
 
   const float *wf = w + f * p.w_strides[0];
   const float *inn = in + n * p.in_strides[0];
@@ -67,15 +73,20 @@ __global__ __launch_bounds__(kBlock) void ConvDirect(ConvArgs p, float *__restri
     const float *inc = inn + (p.depthwise ? f : c) * p.in_strides[1];
     const float *wc = wf + c * p.w_strides[1];
     if constexpr (NS == 1) {
-      for (int32_t k0 = 0; k0 < p.k_shape[0]; ++k0) {
+      const int32_t kh = KH > 0 ? KH : p.k_shape[0];
+#pragma unroll
+      for (int32_t k0 = 0; k0 < kh; ++k0) {
         const int32_t i0 = base[0] + k0 * p.dilation[0];
         if (i0 >= 0 && i0 < p.in_shape[2]) acc += inc[i0 * p.in_strides[2]] * wc[k0 * p.w_strides[2]];
       }
     } else if constexpr (NS == 2) {
-      for (int32_t k0 = 0; k0 < p.k_shape[0]; ++k0) {
+      const int32_t kh = KH > 0 ? KH : p.k_shape[0], kw = KW > 0 ? KW : p.k_shape[1];
+#pragma unroll
+      for (int32_t k0 = 0; k0 < kh; ++k0) {
         const int32_t i0 = base[0] + k0 * p.dilation[0];
         if (i0 < 0 || i0 >= p.in_shape[2]) continue;
-        for (int32_t k1 = 0; k1 < p.k_shape[1]; ++k1) {
+#pragma unroll
+        for (int32_t k1 = 0; k1 < kw; ++k1) {
           const int32_t i1 = base[1] + k1 * p.dilation[1];
           if (i1 >= 0 && i1 < p.in_shape[3])
             acc += inc[i0 * p.in_strides[2] + i1 * p.in_strides[3]] * wc[k0 * p.w_strides[2] + k1 * p.w_strides[3]];
@@ -144,6 +155,7 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
   const bool unit = (flags & FL_REF_CONV_UNIT_STRIDE) != 0;
   for (int i = 0; i < rank; ++i) {
     p.out_shape[i] = static_cast<int32_t>(out->shape[i]);
+    p.out_div[i] = FastDiv(static_cast<uint32_t>(out->shape[i]));
     p.in_shape[i] = static_cast<int32_t>(in->shape[i]);
     p.in_strides[i] = static_cast<int32_t>(in->strides[i]);
     p.w_strides[i] = static_cast<int32_t>(weights->strides[i]);
@@ -195,8 +207,24 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
   const float *w = static_cast<const float *>(weights->base);
   hipStream_t s = AsStream(stream);
   switch (ns) {
-    case 1: FL_LAUNCH(ConvDirect<1>, grid, block, 0, s, p, o, x, w, b); break;
-    case 2: FL_LAUNCH(ConvDirect<2>, grid, block, 0, s, p, o, x, w, b); break;
+    case 1:
+      if (p.k_shape[0] == 9) {
+        FL_LAUNCH((ConvDirect<1, 9>), grid, block, 0, s, p, o, x, w, b);
+      } else if (p.k_shape[0] == 3) {
+        FL_LAUNCH((ConvDirect<1, 3>), grid, block, 0, s, p, o, x, w, b);
+      } else {
+        FL_LAUNCH(ConvDirect<1>, grid, block, 0, s, p, o, x, w, b);
+      }
+      break;
+    case 2:
+      if (p.k_shape[0] == 3 && p.k_shape[1] == 3) {
+        FL_LAUNCH((ConvDirect<2, 3, 3>), grid, block, 0, s, p, o, x, w, b);
+      } else if (p.k_shape[0] == 5 && p.k_shape[1] == 5) {
+        FL_LAUNCH((ConvDirect<2, 5, 5>), grid, block, 0, s, p, o, x, w, b);
+      } else {
+        FL_LAUNCH(ConvDirect<2>, grid, block, 0, s, p, o, x, w, b);
+      }
+      break;
     case 3: FL_LAUNCH(ConvDirect<3>, grid, block, 0, s, p, o, x, w, b); break;
     default: return FL_ERR_RANK;
   }

@@ -9,7 +9,7 @@ durations (dispatch begin/end timestamps) against the fp32 MFMA peak; `cpu_basel
 nests on one host core for a bounded sample; `peak_hbm_bytes` = arena + constants + interface staging.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--executor plain_greedy|dp_greedy]
-                    [--no-cpu-baseline] [--per-kernel] [--per-launch] [--bf16] [--hbm-kernels]
+                    [--no-cpu-baseline] [--per-kernel] [--per-launch] [--bf16] [--hbm-kernels] [--mfma-kernels]
 """
 import argparse
 import json
@@ -125,6 +125,9 @@ def main():
     ap.add_argument("--hbm-kernels", action="store_true",
                     help="instead of the benchmark, time every bandwidth-bound kernel class on 128-512 MiB of data "
                          "and print its achieved HBM GB/s (table on stderr, one JSON line on stdout)")
+    ap.add_argument("--mfma-kernels", action="store_true",
+                    help="instead of the benchmark, time the contraction kernel (MatMul, 3x3 convolution) on problems of "
+                         "growing size and print its TFLOP/s against the fp32 MFMA peak")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the reference has no multi-device path); use --gpus 1")
@@ -136,6 +139,11 @@ def main():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     from fluidml_amd import fluidml, models
 
+    if args.mfma_kernels:
+        from fluidml_amd import mfma_sweep
+
+        print(json.dumps(mfma_sweep.run(out=sys.stderr)))
+        return
     if args.hbm_kernels:
         from fluidml_amd import hbm_sweep
 

@@ -556,20 +556,25 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
       const uint32_t slot = QUARTER ? tile_id * 4 + ks : tile_id;
       const uint32_t sub = QUARTER ? ks * 256 : 0;
       float *mine = p.partials + (static_cast<size_t>(tile_id) * n_splits + blockIdx.z) * 1024 + sub;
-      // The partial tiles travel through device-coherent accesses (agent-scope atomics: they bypass the
-      // per-XCD L2 instead of living in it), so no cache-wide write-back or invalidate is needed: waiting
-      // for this wave's stores to be acknowledged before it counts its arrival is enough, and the last
-      // wave's loads are issued only after it has seen every other arrival.
+      // The partial tiles travel through device-coherent accesses (agent-scope atomics: write-through stores
+      // and loads that miss in the per-XCD L2), so no cache-wide write-back or invalidate is needed.
+      // Release side: a fence of workgroup scope emits no wait on this target (the L1 keeps one workgroup's
+      // accesses in order), and the stores and the counter go to different L2 channels, so the wave itself
+      // waits until every vector memory operation it has issued is acknowledged (s_waitcnt vmcnt(0); stores
+      // count in vmcnt on gfx9) before it counts its arrival.  The "memory" clobber keeps the compiler from
+      // moving the stores below the wait or the counter update above it.
+      // Acquire side: the partial loads are issued after the branch on the counter's returned value, which
+      // the wave has to wait for; the compiler-only fence below keeps them behind it in program order.
 #pragma unroll
       for (int e = 0; e < EV; ++e) {
         __hip_atomic_store(mine + e * 64 + lane, acc[0][0][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // s_waitcnt: stores acknowledged
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       uint32_t arrived = 0;
       if (lane == 0) arrived = __hip_atomic_fetch_add(&p.counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       arrived = __shfl(arrived, 0);
       if (arrived != n_splits - 1) return;
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // keeps the loads below behind the counter read
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // compiler ordering only: no instruction on gfx9
       if (lane == 0) __hip_atomic_store(&p.counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const float *all = p.partials + static_cast<size_t>(tile_id) * n_splits * 1024 + sub;
 #pragma unroll

@@ -318,6 +318,14 @@ PYBIND11_MODULE(fluidml, m) {
       },
       py::arg("kind"), py::arg("starts"), py::arg("ends"), py::arg("sizes"),
       "kind 0 = PlainInfos+LinearPlan, 1 = GreedyInfos+GreedyPlan; tensors are named t0, t1, ... in push order");
+  m.def("_kernel_names", [] {
+    // GetKernelName() of every kernel class, in the order of flow::OpKind
+    std::vector<std::string> names;
+    for (int k = 0; k <= static_cast<int>(flow::OpKind::WhereConstantCondConstantTensorY); ++k) {
+      names.push_back(kernel::KernelNameOf(static_cast<flow::OpKind>(k)));
+    }
+    return names;
+  });
   m.def("_gen_all_orders", &utils::GenAllOrders);
   m.def("_gen_all_indices_in_order", &utils::GenAllIndicesInOrder);
   m.def("_gen_physical_shape", &utils::GenPhysicalShape);

@@ -19,3 +19,15 @@ def device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def progress(capsys):
+    """print(...) that reaches the terminal while output capture is on: long CPU legs (the oracle on a full-size
+    graph) show that the run is alive."""
+
+    def say(*args):
+        with capsys.disabled():
+            print(*args, flush=True)
+
+    return say

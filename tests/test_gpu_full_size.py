@@ -1,15 +1,19 @@
-"""The benchmark configurations at their full extents.
+"""The benchmark configurations at their full extents and full depth, against the oracle.
 
-* BERT-base with its real extents (seq 128, hidden 768, 12 heads, FFN 3072, vocab 30522) and two of its
-  twelve layers against the oracle's graph runner (a few seconds of scalar loop nests): every launch of a
-  layer at the shape bench.py times it at.
-* Every configuration at full size and full depth, where the oracle would take minutes: the fused launch
-  schedule against the one-launch-per-node schedule (FLUIDML_FUSE=0) of the same plan on the same inputs.
-  The per-node kernels are the ones the kernel tests pin against the oracle; the fused launches re-associate
-  sums (attention, split K, grouped projections), so the two agree within the fp32 tolerance the
-  configurations are specified with (rel 1e-4 / abs 1e-5), not bit for bit.
+Every configuration (BERT-base, ConvBERT-base, GPT-NeoX prefill, EfficientNet-B0, VGG-16 at batch 1 and at
+batch 8) is compiled from its ONNX file and run three ways on the same seeded weights and inputs:
+
+* the oracle's graph runner on the CPU (scalar loop nests: 1 s for EfficientNet-B0, 30-90 s for the others),
+* the fused launch schedule (what bench.py times),
+* the one-launch-per-node schedule (FLUIDML_FUSE=0) of the same plan.
+
+Both GPU schedules have to meet the oracle within the tolerance the configurations are specified with
+(rel 1e-4 / abs 1e-5, fp32).  For VGG-16 at batch 8 the oracle runs the batch-1 graph (same seed, hence the
+same weights; tests/test_oracle_graphs.py checks that rows of a batch are independent images) on images 0
+and 7.  A BERT-base case with the layouts of the DP executor (constant costs: every tensor stored with its
+dimensions reversed) runs the same comparison on non-identity strides at real extents.
 """
-import sys
+import functools
 
 import numpy as np
 import pytest
@@ -20,29 +24,14 @@ from tests.util import assert_close
 pytestmark = pytest.mark.gpu
 
 
-def _run(fluidml, net, feeds, path, name):
-    ex = fluidml.Executor.make_plain_greedy(name, 1)
+def _run(fluidml, net, feeds, path, name, flavour="plain_greedy"):
+    ex = getattr(fluidml.Executor, "make_" + flavour)(name, 1)
     ex.compile(path)
     args = {k: np.ascontiguousarray(v) for k, v in feeds.items()}
     outs = {v.name: np.full(v.shape, np.nan, dtype=v.dtype) for v in net.outputs}
     args.update(outs)
     assert ex.invoke(args) > 0
     return outs, ex.plan()
-
-
-def test_bert_base_extents_match_oracle(device, tmp_path):
-    from fluidml_amd import fluidml, models
-
-    net = models.bert_base(layers=2)
-    feeds = models.bert_inputs(128, 30522, seed=11)
-    print("[case] bert_base extents, 2 layers,", len(net.nodes), "nodes", flush=True)
-    sys.stdout.flush()
-    want = graph_runner.run_graph(net, feeds)
-    outs, plan = _run(fluidml, net, feeds, net.save(str(tmp_path / "bert2.onnx")), "bert2")
-    kinds = {l["kind"] for l in plan["launches"]}
-    assert {"Attention", "MatMulGroup", "AddLayerNormalization"} <= kinds
-    for name, ref in want.items():
-        assert_close(outs[name], ref, what=f"bert_base (2 layers) {name}")
 
 
 def _full_configs():
@@ -53,29 +42,93 @@ def _full_configs():
         "convbert_base": (models.convbert_base, lambda: models.bert_inputs(128, 30522, seed=13)),
         "gpt_neox": (models.gpt_neox, lambda: models.gpt_neox_inputs(256, 50304, seed=14)),
         "efficientnet_b0": (models.efficientnet_b0, lambda: models.image_input((1, 3, 224, 224), seed=15)),
-        "vgg16_b1": (lambda: models.vgg16(batch=1), lambda: models.image_input((1, 3, 224, 224), seed=16)),
+        # batch 1 runs image 0 of the batch of 8, so the oracle's pass over that image serves both
+        "vgg16_b1": (lambda: models.vgg16(batch=1), lambda: {"input": _vgg_images()[:1].copy()}),
+        "vgg16_b8": (lambda: models.vgg16(batch=8), lambda: {"input": _vgg_images()}),
     }
 
 
-@pytest.mark.parametrize("config", ["bert_base", "convbert_base", "gpt_neox", "efficientnet_b0", "vgg16_b1"])
-def test_full_size_fused_matches_unfused(device, config, tmp_path, monkeypatch):
+# the launch kinds each configuration is expected to exercise at full size
+_EXPECTED_KINDS = {
+    "bert_base": {"Attention", "MatMulGroup", "GatherAdd", "AddLayerNormalization"},
+    "convbert_base": {"Attention", "SoftmaxMatVec"},
+    "gpt_neox": {"Attention", "Rotary", "AddAdd"},
+    "efficientnet_b0": {"ConvChain", "ConvPair"},
+    "vgg16_b1": {"ConvChain", "GemmChain"},
+    "vgg16_b8": {"ConvChain", "GemmChain"},
+}
+
+
+@functools.lru_cache(maxsize=None)
+def _vgg_images():
+    from fluidml_amd import models
+
+    return models.image_input((8, 3, 224, 224), seed=17)["input"]
+
+
+@functools.lru_cache(maxsize=None)
+def _vgg_oracle(image):
+    """the oracle's VGG-16 (batch-1 graph) on one image of the batch: about a minute and a half of loop nests"""
+    from fluidml_amd import models
+
+    (ref,) = graph_runner.run_graph(models.vgg16(batch=1), {"input": _vgg_images()[image:image + 1].copy()}).values()
+    return ref
+
+
+def _oracle(config, net, feeds, progress):
+    """name -> (rows of the output the oracle computed, expected values)"""
+    if not config.startswith("vgg16"):
+        return {name: (slice(None), ref) for name, ref in graph_runner.run_graph(net, feeds).items()}
+    (out_name,) = [v.name for v in net.outputs]
+    rows, refs = ([0], []) if config == "vgg16_b1" else ([0, 7], [])
+    for b in rows:
+        progress("[oracle] vgg16 image", b)
+        refs.append(_vgg_oracle(b))
+    return {out_name: (rows, np.concatenate(refs, axis=0))}
+
+
+@pytest.mark.parametrize("config", ["efficientnet_b0", "bert_base", "convbert_base", "gpt_neox", "vgg16_b1", "vgg16_b8"])
+def test_full_size_matches_oracle(device, config, tmp_path, monkeypatch, progress):
     from fluidml_amd import fluidml
 
     make_net, make_feeds = _full_configs()[config]
     net, feeds = make_net(), make_feeds()
     path = net.save(str(tmp_path / f"{config}.onnx"))
-    print("[case] full size", config, len(net.nodes), "nodes", flush=True)
-    sys.stdout.flush()
+    progress("[case] full size", config, len(net.nodes), "nodes: oracle")
+    want = _oracle(config, net, feeds, progress)
+    progress("[case] full size", config, "per-node launches")
     monkeypatch.setenv("FLUIDML_FUSE", "0")
     plain, plain_plan = _run(fluidml, net, feeds, path, config + "_plain")
+    progress("[case] full size", config, "fused launches")
     monkeypatch.setenv("FLUIDML_FUSE", "1")
     fused, fused_plan = _run(fluidml, net, feeds, path, config + "_fused")
     assert len(plain_plan["launches"]) == len(net.nodes) > len(fused_plan["launches"])
-    # the launch kinds each configuration is expected to exercise at full size
-    expected = {"bert_base": {"Attention", "MatMulGroup", "GatherAdd"}, "convbert_base": {"Attention", "SoftmaxMatVec"},
-                "gpt_neox": {"Attention", "Rotary", "AddAdd"}, "efficientnet_b0": {"ConvChain", "ConvPair"},
-                "vgg16_b1": {"ConvChain", "GemmChain"}}[config]
-    assert expected <= {l["kind"] for l in fused_plan["launches"]}
-    for name, ref in plain.items():
+    assert _EXPECTED_KINDS[config] <= {l["kind"] for l in fused_plan["launches"]}
+    for name, (rows, ref) in want.items():
+        assert np.isfinite(ref).all()
+        assert_close(plain[name][rows], ref, what=f"{config} per-node launches vs oracle, {name}")
+        assert_close(fused[name][rows], ref, what=f"{config} fused launches vs oracle, {name}")
+    for name, ref in plain.items():  # every row, also those the oracle did not compute
         assert np.isfinite(ref).all()
         assert_close(fused[name], ref, what=f"{config} fused vs per-node {name}")
+
+
+def test_bert_base_dp_layouts_match_oracle(device, tmp_path, monkeypatch, progress):
+    """DP executor at BERT-base extents (4 layers): with constant costs every internal tensor is stored with its
+    dimensions reversed, so every kernel and every fused launch runs on non-identity strides at the real shapes."""
+    from fluidml_amd import fluidml, models
+
+    net = models.bert_base(layers=4)
+    feeds = models.bert_inputs(128, 30522, seed=18)
+    path = net.save(str(tmp_path / "bert4.onnx"))
+    progress("[case] bert_base extents, 4 layers, dp_greedy with constant costs: oracle")
+    want = graph_runner.run_graph(net, feeds)
+    monkeypatch.setenv("FLUIDML_DP_COST", "constant")
+    for fuse in ("0", "1"):
+        progress("[case] bert_base extents, dp_greedy, FLUIDML_FUSE =", fuse)
+        monkeypatch.setenv("FLUIDML_FUSE", fuse)
+        outs, plan = _run(fluidml, net, feeds, path, "bert4_dp" + fuse, flavour="dp_greedy")
+        layouts = [list(s["output_layout"]) for s in plan["steps"]]
+        assert sum(l != sorted(l) for l in layouts) > len(layouts) // 2, "the DP plan should hold non-identity layouts"
+        for name, ref in want.items():
+            assert_close(outs[name], ref, what=f"bert_base (4 layers) dp_greedy fuse={fuse} {name}")

@@ -82,6 +82,36 @@ def test_python_surface(fluidml):
         assert hasattr(fluidml.Context, attr), attr
 
 
+def test_top_level_module_name(fluidml):
+    """the reference's module is called `fluidml` (pybind.cpp:23): the same import line works here"""
+    import fluidml as top
+
+    for name in ["Context", "Flow", "Sequence", "Graph", "Index", "Builder", "GeneralBuilder", "Converter", "Executor",
+                 "Lower", "Parser", "Planner", "Runner"]:
+        assert getattr(top, name) is getattr(fluidml, name)
+    assert top.Executor.make_dp_greedy is fluidml.Executor.make_dp_greedy
+
+
+# kKernelName of every kernel class of the reference (include/structure/kernel/kernel/*.h; e.g. gemm.h:13
+# "GemmConstantWeightsBiasKernel" for class GemmConstantBiasKernel, where.h:13-14, 34-35, gather_add_add.h:13-14)
+REFERENCE_KERNEL_NAMES = """
+AddCommonKernel AddConstantKernel AddDivErfAddMulMulKernel AveragePoolWithoutPaddingKernel CastKernel ClipKernel
+Concat2Kernel ConvWithPaddingKernel ConvWithoutPaddingKernel CumSumKernel DivCommonKernel DivConstantRhsKernel
+DropoutKernel EqualKernel ErfKernel FlattenKernel GatherConstantDataTensorKernel GatherConstantIndexScalarKernel
+GatherConstantIndicesTensorKernel GemmConstantWeightsBiasKernel MatMulKernel MaxPoolWithoutPaddingKernel
+MulCommonKernel MulConstantKernel NegKernel NotKernel PadKernel PowKernel ReduceMeanKernel ReluKernel ReshapeKernel
+SliceKernel SoftmaxKernel SqrtKernel SqueezeKernel SubCommonKernel SubConstantLhsKernel TanhKernel TransposeKernel
+UnsqueezeKernel GatherConstantDataTensorAddTensorLhsAddTensorLhsKernel LayerNormalizationConstantScaleBiasKernel
+UnsqueezeSubLhsScalarMulRhsScalarKernel WhereConstantCondConstantScalarYKernel WhereConstantCondConstantTensorYKernel
+""".split()
+
+
+def test_kernel_names_are_the_references(fluidml):
+    names = fluidml._kernel_names()
+    assert len(names) == len(set(names)) == len(REFERENCE_KERNEL_NAMES) == 45
+    assert set(names) == set(REFERENCE_KERNEL_NAMES)
+
+
 def test_c_abi_exports_every_declared_symbol():
     """The shared library loads and exports each entry point include/fluidml_hip.h declares (no compute call)."""
     header = open(os.path.join(ROOT, "include", "fluidml_hip.h")).read()

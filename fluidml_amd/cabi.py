@@ -28,6 +28,8 @@ FL_REF_GEMM_SWAPPED_SCALARS = 1 << 3
 FL_REF_GATHER_RAW_AXIS = 1 << 4
 FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
 FL_CONTRACT_BF16 = 1 << 0
+FL_ERR_STATIC_SCRATCH = -9
+FL_NO_ALLOC_SCRATCH_BYTES = 2 << 20
 
 DTYPE_SIZE = {FL_BOOL: 1, FL_INT32: 4, FL_INT64: 8, FL_FLOAT16: 2, FL_FLOAT32: 4, FL_FLOAT64: 8}
 
@@ -144,6 +146,7 @@ SIGNATURES = {
     "fluidml_hip_average_pool_without_padding": [_T, _T, _i64p, _i64p, _i32, _vp],
     # contractions
     "fluidml_hip_matmul": [_T, _T, _T, _vp],
+    "fluidml_hip_matmul_no_alloc": [_T, _T, _T, _vp],
     "fluidml_hip_matmul_bf16": [_T, _T, _T, _vp],
     "fluidml_hip_gemm_constant_weights_bias": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _u32, _vp],
     "fluidml_hip_matmul_add": [_T, _T, _T, _T, _vp],

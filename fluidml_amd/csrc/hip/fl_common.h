@@ -74,6 +74,9 @@ constexpr size_t kWorkspaceTileFloats = 1024;
 // now (the stream is being captured into a graph) or the allocation fails; callers then do without.
 StreamWorkspace *GetStreamWorkspace(hipStream_t stream);  // runtime.hip
 void DropStreamWorkspace(hipStream_t stream);
+// Device address of the current device's fixed split-K scratch (fluidml_hip_matmul_no_alloc), looked up on
+// the first call per device; `ptr` may be null.  matmul.hip
+int StaticScratch(void **ptr);
 
 // Compile-time loop: body(std::integral_constant<int, 0>) ... body(std::integral_constant<int, N - 1>).
 // Unlike `#pragma unroll` it cannot be left rolled, so register arrays indexed by the counter stay in registers.

@@ -26,6 +26,7 @@
 // bf16 instruction replaces four fp32 ones.
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
 
 #include "fl_common.h"
@@ -824,6 +825,37 @@ inline bool TrySkinnyGemm(const MatmulArgs &p, int64_t n_batch, float *C, const 
   return true;
 }
 
+// ---- split-K workspace of the entry point that allocates nothing ------------------------------------------
+// fluidml_hip_matmul_no_alloc takes the partial tiles and arrival counters of a split-K launch from this
+// file-scope array instead of the stream's workspace (which is allocated on a stream's first use).  Every GPU
+// the library runs on holds its own copy of the array, at its own address, until the process ends.  In host
+// code the array's NAME is only a stand-in for the symbol, not a device address: the address is looked up once
+// per device with hipGetSymbolAddress (StaticScratch below) and only that pointer is handed to kernels.
+constexpr size_t kStaticSlots = FL_NO_ALLOC_SCRATCH_BYTES / (kWorkspaceTileFloats * sizeof(float));  // partial tiles
+constexpr size_t kStaticCounters = 2048;
+static __device__ __align__(256) unsigned char scratch[FL_NO_ALLOC_SCRATCH_BYTES + kStaticCounters * sizeof(uint32_t)];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Workspace a caller on this thread wants LaunchConfig to use instead of the stream's (null: the stream's).
+struct WorkspaceOverride {
+  float *partials;
+  uint32_t *counters;
+  size_t slots;     // partial tiles `partials` holds
+  size_t n_counters;
+  int error;        // set by LaunchConfig when the launch needs more than that; nothing is launched then
+};
+thread_local WorkspaceOverride *t_workspace_override = nullptr;
+
+// The counters a split-K launch on the shared static scratch is about to use must start at zero whatever an
+// earlier call left there.  A fill kernel, not hipMemsetAsync: the caller may be recording a graph.
+__global__ __launch_bounds__(256) void ZeroWordsKernel(uint32_t *p, uint32_t n) {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
 // Upper bound on the number of K splits per tile (environment FLUIDML_SPLITK; default 4 for the 32x32 tile and
 // 16 for the 64x64 tile; 1 = never split).
 inline int64_t SplitKLimit(int64_t fallback) {
@@ -857,7 +889,21 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
     want = std::min<int64_t>(want, SplitKLimit(WM * WN == 1 ? 4 : 16));
     if (tiles > 256) want = 1;
     if (want >= 2) {
-      if (StreamWorkspace *ws = GetStreamWorkspace(s)) {
+      if (WorkspaceOverride *fixed = t_workspace_override) {
+        // same split as with the stream's workspace, so the result is the same bit for bit; refused when
+        // the fixed workspace cannot hold it
+        q.chunks_per_split = static_cast<int32_t>((n_chunks + want - 1) / want);
+        splits = static_cast<uint32_t>((n_chunks + q.chunks_per_split - 1) / q.chunks_per_split);
+        const size_t waves = static_cast<size_t>(tiles) * WM * WN;  // one slot per wave and split
+        if (waves * splits > fixed->slots || waves * 4 > fixed->n_counters) {
+          fixed->error = FL_ERR_STATIC_SCRATCH;
+          return;
+        }
+        q.partials = fixed->partials;
+        q.counters = fixed->counters;
+        const uint32_t n_zero = static_cast<uint32_t>(waves * 4);  // a wave owns up to four quarter counters
+        hipLaunchKernelGGL(ZeroWordsKernel, dim3((n_zero + 255) / 256), dim3(256), 0, s, fixed->counters, n_zero);
+      } else if (StreamWorkspace *ws = GetStreamWorkspace(s)) {
         q.chunks_per_split = static_cast<int32_t>((n_chunks + want - 1) / want);
         splits = static_cast<uint32_t>((n_chunks + q.chunks_per_split - 1) / q.chunks_per_split);
         q.partials = ws->partials;
@@ -1168,12 +1214,44 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
   return LaunchStatus();
 }
 
+// Device address of the current device's copy of `scratch`, looked up on the first call per device.
+int StaticScratch(void **ptr) {
+  int dev = -1;
+  FL_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return FL_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *p = nullptr;
+    FL_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (p == nullptr) return FL_ERR_NULL;
+    g_scratch_ptr[dev] = p;
+  }
+  if (ptr != nullptr) *ptr = g_scratch_ptr[dev];
+  return FL_OK;
+}
+
 }  // namespace fl
 
 extern "C" {
 
 int fluidml_hip_matmul(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
   return fl::Contract(lhs, rhs, out, false, false, 1.0f, 0.0f, nullptr, stream);
+}
+
+int fluidml_hip_matmul_no_alloc(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
+  if (!lhs || !rhs || !out) return FL_ERR_NULL;
+  void *base = nullptr;
+  FL_CHECK(fl::StaticScratch(&base));
+  fl::WorkspaceOverride fixed;
+  fixed.partials = static_cast<float *>(base);
+  fixed.counters = reinterpret_cast<uint32_t *>(static_cast<unsigned char *>(base) + FL_NO_ALLOC_SCRATCH_BYTES);
+  fixed.slots = fl::kStaticSlots;
+  fixed.n_counters = fl::kStaticCounters;
+  fixed.error = FL_OK;
+  fl::t_workspace_override = &fixed;
+  const int rc = fl::Contract(lhs, rhs, out, false, false, 1.0f, 0.0f, nullptr, stream);
+  fl::t_workspace_override = nullptr;
+  return fixed.error != FL_OK ? fixed.error : rc;
 }
 
 int fluidml_hip_matmul_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,

@@ -79,6 +79,9 @@ const char *fluidml_hip_error_string(int code) {
     case FL_ERR_TOO_LARGE: return "view larger than 2^31-1 elements";
     case FL_ERR_SCRATCH: return "scratch buffer too small";
     case FL_ERR_UNSUPPORTED: return "not supported by this backend";
+    case FL_ERR_STATIC_SCRATCH:
+      return "split-K workspace of this problem exceeds the fixed scratch of fluidml_hip_matmul_no_alloc "
+             "(FL_NO_ALLOC_SCRATCH_BYTES); use fluidml_hip_matmul";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -192,6 +195,7 @@ int fluidml_hip_stream_create(void **stream) {
   FL_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
   *stream = s;
   (void)GetStreamWorkspace(s);  // now, so that a later capture on this stream finds it
+  (void)StaticScratch(nullptr);  // likewise the address of this device's fixed scratch
   return FL_OK;
 }
 

@@ -60,7 +60,9 @@ enum fl_error {
   FL_ERR_ATTR = -5,        /* attribute out of range (axis, pads, strides, ...) */
   FL_ERR_TOO_LARGE = -6,   /* more than 2^31-1 elements or offsets in one view */
   FL_ERR_SCRATCH = -7,     /* scratch smaller than the kernel needs */
-  FL_ERR_UNSUPPORTED = -8  /* legal in ONNX, unreachable in the reference, not built */
+  FL_ERR_UNSUPPORTED = -8, /* legal in ONNX, unreachable in the reference, not built */
+  FL_ERR_STATIC_SCRATCH = -9 /* the launch needs more split-K workspace than the fixed
+                              * FL_NO_ALLOC_SCRATCH_BYTES of fluidml_hip_matmul_no_alloc */
 };
 
 /* Literal-reference switches (each cites the reference lines it reproduces). */
@@ -305,6 +307,21 @@ int fluidml_hip_average_pool_without_padding(const fl_tensor *in, const fl_tenso
 /* MatMulKernel: NumPy batch-broadcast matmul, fp32 MFMA
  * (reference matmul.cpp:28-59, utils.cpp:64-147). */
 int fluidml_hip_matmul(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream);
+/* fluidml_hip_matmul for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It
+ * has no counterpart in the reference.  Same arguments, same kernels and the
+ * same result bit for bit as fluidml_hip_matmul, but a launch that splits K
+ * over several workgroups keeps its partial tiles and arrival counters in a
+ * fixed device array inside the library (FL_NO_ALLOC_SCRATCH_BYTES of partial
+ * tiles plus 8 KiB of counters per GPU, held until the process ends) instead
+ * of the stream's workspace, and the call allocates nothing.  A problem whose
+ * split needs more than the array holds (tiles x splits partial 32x32 tiles of
+ * 4 KiB each: 96 tiles x 4 splits fit, 160 tiles x 4 splits do not) is refused with
+ * FL_ERR_STATIC_SCRATCH and nothing is launched.  All calls on one GPU share
+ * the array: calls that overlap in time on one GPU (two streams, two threads)
+ * race; calls on one stream are ordered and safe. */
+#define FL_NO_ALLOC_SCRATCH_BYTES (2u << 20)
+int fluidml_hip_matmul_no_alloc(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream);
 /* Same contraction with operands rounded to bf16 (nearest even) and fp32
  * accumulation on v_mfma_f32_32x32x8_bf16 (opt-in; no counterpart in the
  * reference, error is reported separately). */

@@ -2,11 +2,14 @@
 """Benchmark of the hot path: BERT-base encoder (batch 1, seq 128, fp32) planned like the reference's
 Executor (plain_greedy by default) and replayed as HIP launches over one HBM arena.
 
-A "step" is one inference: one replay of the whole launch plan (416 graph nodes issued as 89 kernel
+A "step" is one inference: one replay of the whole launch plan (416 graph nodes issued as a few dozen kernel
 launches after launch-level fusion) on inputs that are already resident in HBM.  Prints ONE JSON line:
 `value` = inferences/s over the timed replays; `roofline` = the contraction kernel's flops over its launch
-durations (dispatch begin/end timestamps) against the fp32 MFMA peak; `cpu_baseline` = the oracle's scalar loop
-nests on one host core for a bounded sample; `peak_hbm_bytes` = arena + constants + interface staging.
+durations (dispatch begin/end timestamps) against the fp32 MFMA peak, `roofline.traffic` = the HBM bytes per
+launch the tracked profiler summary (`roofline.traffic_source`) holds for exactly this workload, else null;
+`cpu_baseline` = the oracle's scalar loop nests on one host core for a bounded sample;
+`peak_hbm_bytes` = arena + constants + interface staging.  The default run adds `configs`: the same
+measurement (GPU legs only) for the other five configurations and for BERT-base under the DP executor.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--executor plain_greedy|dp_greedy]
                     [--no-cpu-baseline] [--per-kernel] [--per-launch] [--bf16] [--hbm-kernels] [--mfma-kernels]
@@ -25,11 +28,29 @@ if ROOT not in sys.path:
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the contraction kernel on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch, averaged over the 48 contraction launches of an inference), each scaled by what the
-# same counter reads for the identity-copy kernel on 256 MiB (x2.000 and x0.996): (6519.6 * 2.000 + 1464.0 * 0.996) KiB.
-# Only valid for the default workload (BERT-base, seq 128, 12 layers, plain_greedy, fusion on).
-MATMUL_TRAFFIC_BYTES_PER_LAUNCH = 14_844_165
+# HBM bytes per launch of the contraction kernel come from the tracked profiler summary of the default workload
+# (BERT-base, seq 128, 12 layers, plain_greedy, fusion on): rocprofv3 FETCH_SIZE / WRITE_SIZE per dispatch, each
+# scaled by what the same counter reads for the identity-copy kernel.  The summary carries one line
+# "traffic_bytes_per_launch = N" for bench.py; any other workload reports null.
+TRAFFIC_SUMMARY = os.path.join("profiles", "matmul_bert_base_s128.md")
+
+
+def traffic_from_summary():
+    import re
+
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_SUMMARY)).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic_bytes_per_launch\s*=\s*([0-9][0-9,_]*)", text)
+    return int(m.group(1).replace(",", "").replace("_", "")) if m else None
+
+
+def host_cores():
+    try:
+        return len(os.sched_getaffinity(0))
+    except AttributeError:
+        return os.cpu_count() or 1
 
 
 def cpu_baseline(layers_total: int, sample_layers: int, seq: int):
@@ -52,9 +73,10 @@ def cpu_baseline(layers_total: int, sample_layers: int, seq: int):
         "value": 1.0 / total,
         "unit": "inferences/s",
         "cores": 1,
+        "host_cores": host_cores(),
         "kind": "port",
-        "sample": f"{sample_layers} of {layers_total} encoder layers + embeddings at seq {seq} (one inference each), "
-                  f"{per_layer} kernels per layer; per-layer time {layer_time:.3f} s extrapolated to {layers_total} layers",
+        "sample": f"{sample_layers} of {layers_total} encoder layers + embeddings at seq {seq} (one inference each) on 1 of "
+                  f"{host_cores()} host cores, {per_layer} kernels per layer; per-layer time {layer_time:.3f} s extrapolated to {layers_total} layers",
         "seconds_per_inference": total,
     }
 
@@ -97,76 +119,20 @@ def cpu_baseline_whole(net, feeds, batch):
     finally:
         done.set()
     total = time.perf_counter() - t0
-    return {"value": batch / total, "unit": "inferences/s", "cores": 1, "kind": "port",
-            "sample": f"one whole forward pass of batch {batch}", "seconds_per_inference": total / batch}
+    return {"value": batch / total, "unit": "inferences/s", "cores": 1, "host_cores": host_cores(), "kind": "port",
+            "sample": f"one whole forward pass of batch {batch} on 1 of {host_cores()} host cores", "seconds_per_inference": total / batch}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--config", default="bert_base",
-                    choices=["bert_base", "convbert_base", "gpt_neox", "efficientnet_b0", "vgg16_b1", "vgg16_b8"],
-                    help="bert_base is the configuration the headline metric is quoted on")
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--executor", default="plain_greedy", choices=["plain_linear", "plain_greedy", "dp_greedy"])
-    ap.add_argument("--layers", type=int, default=12)
-    ap.add_argument("--seq", type=int, default=128)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-layers", type=int, default=3)
-    ap.add_argument("--per-kernel", action="store_true", help="also print a per-kernel table to stderr")
-    ap.add_argument("--per-launch", action="store_true", help="also print every launch of one step, in order, to stderr")
-    ap.add_argument("--bf16", action="store_true",
-                    help="additionally run the opt-in bf16 contraction path and report its throughput and its "
-                         "error against the fp32 result under \"bf16\" (the headline value stays fp32)")
-    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
-                    help="instead of the benchmark, launch the identity-copy kernel 3 times on a buffer of MIB MiB "
-                         "(a kernel of known traffic, to scale profiler byte counters) and exit")
-    ap.add_argument("--hbm-kernels", action="store_true",
-                    help="instead of the benchmark, time every bandwidth-bound kernel class on 128-512 MiB of data "
-                         "and print its achieved HBM GB/s (table on stderr, one JSON line on stdout)")
-    ap.add_argument("--mfma-kernels", action="store_true",
-                    help="instead of the benchmark, time the contraction kernel (MatMul, 3x3 convolution) on problems of "
-                         "growing size and print its TFLOP/s against the fp32 MFMA peak")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU (the reference has no multi-device path); use --gpus 1")
+def measure(args, config, executor, per_kernel=False, per_launch=False):
+    """Compile `config` with `executor`, replay it args.steps times and return (result dict, objects for more legs)."""
+    import types
 
     import numpy as np
     import torch
 
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
-    from fluidml_amd import fluidml, models
+    from fluidml_amd import fluidml
 
-    if args.mfma_kernels:
-        from fluidml_amd import mfma_sweep
-
-        print(json.dumps(mfma_sweep.run(out=sys.stderr)))
-        return
-    if args.hbm_kernels:
-        from fluidml_amd import hbm_sweep
-
-        print(json.dumps(hbm_sweep.run(out=sys.stderr)))
-        return
-    if args.copy_calibration:
-        import ctypes
-
-        from fluidml_amd import cabi
-
-        n = args.copy_calibration * (1 << 20) // 4
-        src = torch.ones(n, dtype=torch.float32, device="cuda")
-        dst = torch.zeros(n, dtype=torch.float32, device="cuda")
-        ts = cabi.make_tensor(src.data_ptr(), cabi.FL_FLOAT32, [n], [1])
-        td = cabi.make_tensor(dst.data_ptr(), cabi.FL_FLOAT32, [n], [1])
-        torch.cuda.synchronize()
-        for _ in range(3):
-            cabi.call("dropout", ctypes.byref(ts), ctypes.byref(td), None)
-        torch.cuda.synchronize()
-        assert bool((dst == 1).all())
-        print(json.dumps({"copy_calibration_bytes_read": n * 4, "copy_calibration_bytes_written": n * 4}))
-        return
-
+    args = types.SimpleNamespace(**{**vars(args), "config": config, "executor": executor})
     net, feeds, workload, batch = make_config(args)
     with tempfile.TemporaryDirectory() as tmp:
         path = net.save(os.path.join(tmp, args.config + ".onnx"))
@@ -234,7 +200,10 @@ def main():
         roofline = {"bound": "mfma", "kernel": dname + " (all launches of the contraction kernel, fused epilogues included)",
                     "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
                     "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
-                    "traffic": MATMUL_TRAFFIC_BYTES_PER_LAUNCH if default_workload and dname == "MatMulKernel" else None,
+                    "traffic": traffic_from_summary() if default_workload and dname == "MatMulKernel" else None,
+                    "traffic_source": TRAFFIC_SUMMARY + (" (rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch, scaled by the "
+                                                         "identity-copy kernel's readings)" if default_workload else
+                                                         " covers the default workload only: not measured for this one"),
                     "avg_launch_us": d["ns"] / d["launches"] / 1e3, "launches_per_step": d["launches"],
                     "flops_per_launch": d["flops"] / d["launches"]}
     else:
@@ -247,13 +216,13 @@ def main():
     total_bytes = sum(t["bytes"] for t in times)
     kernel_sum_ms = sum(t["ns"] for t in times) / 1e6
 
-    if args.per_kernel:
+    if per_kernel:
         print(f"{'kernel':48s} {'launches':>8s} {'total us':>10s} {'avg us':>8s} {'GB/s':>9s} {'TFLOP/s':>8s}", file=sys.stderr)
         for name, k in sorted(by_launch_kind.items(), key=lambda kv: -kv[1]["ns"]):
             print(f"{name:48s} {k['launches']:8d} {k['ns'] / 1e3:10.1f} {k['ns'] / k['launches'] / 1e3:8.2f} "
                   f"{k['bytes'] / k['ns']:9.1f} {k['flops'] / k['ns'] / 1e3:8.2f}", file=sys.stderr)
 
-    if args.per_launch:
+    if per_launch:
         print(f"{'#':>4s} {'launch':60s} {'us':>9s} {'GB/s':>9s} {'TFLOP/s':>8s}", file=sys.stderr)
         for i, t in enumerate(times):
             print(f"{i:4d} {t['kernel'][:60]:60s} {t['ns'] / 1e3:9.2f} {t['bytes'] / t['ns']:9.1f} {t['flops'] / t['ns'] / 1e3:8.2f}",
@@ -284,6 +253,98 @@ def main():
                         "sum_of_kernel_ms": kernel_sum_ms, "invoke_with_host_copies_ms": invoke_ms,
                         "compile_s": compile_s},
     }
+    return result, (net, feeds, batch, ex, io, outs)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--config", default="bert_base",
+                    choices=["bert_base", "convbert_base", "gpt_neox", "efficientnet_b0", "vgg16_b1", "vgg16_b8"],
+                    help="bert_base is the configuration the headline metric is quoted on")
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--executor", default="plain_greedy", choices=["plain_linear", "plain_greedy", "dp_greedy"])
+    ap.add_argument("--layers", type=int, default=12)
+    ap.add_argument("--seq", type=int, default=128)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="default workload only: skip the `configs` key (the other configurations and the DP executor)")
+    ap.add_argument("--cpu-sample-layers", type=int, default=3)
+    ap.add_argument("--per-kernel", action="store_true", help="also print a per-kernel table to stderr")
+    ap.add_argument("--per-launch", action="store_true", help="also print every launch of one step, in order, to stderr")
+    ap.add_argument("--bf16", action="store_true",
+                    help="additionally run the opt-in bf16 contraction path and report its throughput and its "
+                         "error against the fp32 result under \"bf16\" (the headline value stays fp32)")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="instead of the benchmark, launch the identity-copy kernel 3 times on a buffer of MIB MiB "
+                         "(a kernel of known traffic, to scale profiler byte counters) and exit")
+    ap.add_argument("--hbm-kernels", action="store_true",
+                    help="instead of the benchmark, time every bandwidth-bound kernel class on 128-512 MiB of data "
+                         "and print its achieved HBM GB/s (table on stderr, one JSON line on stdout)")
+    ap.add_argument("--mfma-kernels", action="store_true",
+                    help="instead of the benchmark, time the contraction kernel (MatMul, 3x3 convolution) on problems of "
+                         "growing size and print its TFLOP/s against the fp32 MFMA peak")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the reference has no multi-device path); use --gpus 1")
+
+    import numpy as np
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    from fluidml_amd import fluidml, models
+
+    if args.mfma_kernels:
+        from bench_sweeps import mfma_sweep
+
+        print(json.dumps(mfma_sweep.run(out=sys.stderr)))
+        return
+    if args.hbm_kernels:
+        from bench_sweeps import hbm_sweep
+
+        print(json.dumps(hbm_sweep.run(out=sys.stderr)))
+        return
+    if args.copy_calibration:
+        import ctypes
+
+        from fluidml_amd import cabi
+
+        n = args.copy_calibration * (1 << 20) // 4
+        src = torch.ones(n, dtype=torch.float32, device="cuda")
+        dst = torch.zeros(n, dtype=torch.float32, device="cuda")
+        ts = cabi.make_tensor(src.data_ptr(), cabi.FL_FLOAT32, [n], [1])
+        td = cabi.make_tensor(dst.data_ptr(), cabi.FL_FLOAT32, [n], [1])
+        torch.cuda.synchronize()
+        for _ in range(3):
+            cabi.call("dropout", ctypes.byref(ts), ctypes.byref(td), None)
+        torch.cuda.synchronize()
+        assert bool((dst == 1).all())
+        print(json.dumps({"copy_calibration_bytes_read": n * 4, "copy_calibration_bytes_written": n * 4}))
+        return
+
+    result, (net, feeds, batch, ex, io, outs) = measure(args, args.config, args.executor, args.per_kernel, args.per_launch)
+    default_run = (args.config, args.layers, args.seq, args.executor) == ("bert_base", 12, 128, "plain_greedy")
+    if default_run and not args.no_configs:
+        # the other configurations and the DP executor, GPU legs only (no CPU baseline), fewer steps
+        import types
+
+        short = types.SimpleNamespace(**{**vars(args), "steps": max(20, args.steps // 4), "warmup": max(5, args.warmup // 4)})
+        result["configs"] = {}
+        del ex
+        for name, executor in [("bert_base", "dp_greedy"), ("convbert_base", "plain_greedy"), ("gpt_neox", "plain_greedy"),
+                               ("efficientnet_b0", "plain_greedy"), ("vgg16_b1", "plain_greedy"), ("vgg16_b8", "plain_greedy")]:
+            print(f"[bench] {name} ({executor}) ...", file=sys.stderr, flush=True)
+            r, keep = measure(short, name, executor)
+            del keep
+            key = name if executor == "plain_greedy" else f"{name}:{executor}"
+            result["configs"][key] = {"value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"], "steps": r["steps"],
+                                      "kernels_per_step": r["config"]["kernels_per_step"],
+                                      "roofline": {k: r["roofline"][k] for k in ("bound", "kernel", "achieved", "peak", "unit", "frac")},
+                                      "whole_graph_tflops": r["whole_graph"]["tflops"],
+                                      "peak_hbm_bytes": r["peak_hbm_bytes"]}
+        ex = None
     if args.bf16:
         ref_out = {k: v.copy() for k, v in outs.items()}
         ex.invoke(io)
@@ -318,7 +379,7 @@ def main():
             # the scalar loop nests take the same time for every image of a batch: time one image
             one = {k: np.ascontiguousarray(v[:1]) for k, v in feeds.items()}
             result["cpu_baseline"] = cpu_baseline_whole(models.vgg16(1), one, 1)
-            result["cpu_baseline"]["sample"] = f"one whole forward pass of ONE image of the batch of {batch} (the batch-1 graph)"
+            result["cpu_baseline"]["sample"] = f"one whole forward pass of ONE image of the batch of {batch} (the batch-1 graph) on 1 of {host_cores()} host cores"
         else:
             result["cpu_baseline"] = cpu_baseline_whole(net, feeds, batch)
     print(json.dumps(result))

@@ -119,7 +119,7 @@ __global__ __launch_bounds__(kBlock) void ConvDirect(ConvArgs p, float *__restri
 // matmul.hip
 int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
                      const int64_t *pads, const int64_t *strides, const int64_t *dilations,
-                     const fl_ew_program *chain, void *stream);
+                     const fl_ew_program *chain, bool bf16, void *stream);
 
 namespace {
 
@@ -131,6 +131,9 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
   FL_CHECK(CheckView(weights));
   FL_CHECK(CheckView(out));
   if (in->dtype != FL_FLOAT32 || weights->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  // the upper half of `flags` carries fl_contract_flags, the lower half fl_ref_flags
+  const bool bf16 = ((flags >> FL_CONTRACT_SHIFT) & FL_CONTRACT_BF16) != 0;
+  flags &= (1u << FL_CONTRACT_SHIFT) - 1;
   const int rank = out->rank;
   if (rank < 3 || rank > 2 + kMaxSpatial) return FL_ERR_RANK;
   if (in->rank != rank || weights->rank != rank) return FL_ERR_RANK;
@@ -185,7 +188,7 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
   }
   // dense contractions go to the matrix cores; depthwise, 3-d and literal-reference modes stay here
   if (!depthwise && flags == 0 && ns <= 2) {
-    const int rc = ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, chain, stream);
+    const int rc = ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, chain, bf16, stream);
     if (rc != FL_ERR_UNSUPPORTED) return rc;
   }
   LoopNest nest;
@@ -470,8 +473,9 @@ int fluidml_hip_conv_with_padding(const fl_tensor *in, const fl_tensor *weights,
 
 int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
                            const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group,
-                           const fl_ew_program *chain, void *stream) {
-  return fl::Conv(in, weights, bias, out, pads, strides, dilations, group, 0, stream, chain);
+                           const fl_ew_program *chain, uint32_t flags, void *stream) {
+  return fl::Conv(in, weights, bias, out, pads, strides, dilations, group, (flags & FL_CONTRACT_BF16) << FL_CONTRACT_SHIFT, stream,
+                  chain);
 }
 
 int fluidml_hip_pointwise_conv_pair(const fl_tensor *in, const fl_tensor *weights1, const fl_tensor *bias1,

@@ -1076,7 +1076,8 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   for (int i = 0; i < nest.rank && vec; ++i) {
     if (nest.strides[1][i] % 4 != 0 || nest.strides[2][i] % 4 != 0) vec = false;
   }
-  if (!bf16 && TrySkinnyGemm(p, n_batch, C, A, B, s)) return LaunchStatus();
+  // at most 8 rows against k-contiguous weights: HBM-bound weight streaming, fp32 whatever `bf16` says
+  if (TrySkinnyGemm(p, n_batch, C, A, B, s)) return LaunchStatus();
   const uint32_t nb = static_cast<uint32_t>(n_batch);
 #define FL_MM_DISPATCH(LA_, LB_)                              \
   if (la == LA_ && lb == LB_) {                               \
@@ -1104,7 +1105,7 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
 // uses the direct kernel.  `pads` may be null; `strides`/`dilations` have one entry per spatial dim.
 int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
                      const int64_t *pads, const int64_t *strides, const int64_t *dilations,
-                     const fl_ew_program *chain, void *stream) {
+                     const fl_ew_program *chain, bool bf16, void *stream) {
   const int ns = out->rank - 2;
   if (ns != 1 && ns != 2) return FL_ERR_UNSUPPORTED;
   const int hd = ns == 2 ? 2 : -1, wd = ns == 2 ? 3 : 2;  // dims of H (absent for 1-d) and W
@@ -1144,7 +1145,8 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
         d.base = bias->base, d.dtype = FL_FLOAT32, d.rank = 2;
         d.shape[0] = F, d.shape[1] = S, d.strides[0] = bias->strides[0], d.strides[1] = 0;
       }
-      return Contract(&a, &b, &c, false, false, 1.0f, 1.0f, bias != nullptr ? &d : nullptr, stream, chain);
+      return Contract(&a, &b, &c, false, false, 1.0f, 1.0f, bias != nullptr ? &d : nullptr, stream, chain, 0, 0, nullptr,
+                      bf16);
     }
   }
 
@@ -1200,8 +1202,14 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
   const bool quad = g.sw == 1 && g.sXw == 1 && OW % 4 == 0;
 #define FL_CONV_DISPATCH(LA_, VEC_)                                         \
   do {                                                                      \
-    if (quad) LaunchBySize<LA_, 0, VEC_, 2>(p, 1, C, A, B, s);              \
-    else LaunchBySize<LA_, 0, VEC_, 1>(p, 1, C, A, B, s);                   \
+    if (bf16) {                                                             \
+      if (quad) LaunchBySize<LA_, 0, VEC_, 2, true>(p, 1, C, A, B, s);      \
+      else LaunchBySize<LA_, 0, VEC_, 1, true>(p, 1, C, A, B, s);           \
+    } else if (quad) {                                                      \
+      LaunchBySize<LA_, 0, VEC_, 2>(p, 1, C, A, B, s);                      \
+    } else {                                                                \
+      LaunchBySize<LA_, 0, VEC_, 1>(p, 1, C, A, B, s);                      \
+    }                                                                       \
   } while (0)
   if (la == 0) {
     if (vec) FL_CONV_DISPATCH(0, 4);
@@ -1302,11 +1310,11 @@ int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl
 
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
                            double alpha, double beta, int32_t trans_a, int32_t trans_b, const fl_ew_program *chain,
-                           void *stream) {
+                           uint32_t flags, void *stream) {
   if (!lhs || !rhs || !bias || !out) return FL_ERR_NULL;
   if (lhs->rank != 2 || rhs->rank != 2 || out->rank != 2) return FL_ERR_RANK;
   return fl::Contract(lhs, rhs, out, trans_a != 0, trans_b != 0, static_cast<float>(alpha), static_cast<float>(beta),
-                      bias, stream, chain);
+                      bias, stream, chain, 0, 0, nullptr, (flags & FL_CONTRACT_BF16) != 0);
 }
 
 int fluidml_hip_matmul_bf16(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
@@ -1322,7 +1330,8 @@ int fluidml_hip_gemm_constant_weights_bias(const fl_tensor *lhs, const fl_tensor
   const bool swapped = (flags & FL_REF_GEMM_SWAPPED_SCALARS) != 0;
   const float ca = static_cast<float>(swapped ? beta : alpha);
   const float cb = static_cast<float>(swapped ? alpha : beta);
-  return fl::Contract(lhs, rhs, out, trans_a != 0, trans_b != 0, ca, cb, bias, stream);
+  const bool bf16 = ((flags >> FL_CONTRACT_SHIFT) & FL_CONTRACT_BF16) != 0;
+  return fl::Contract(lhs, rhs, out, trans_a != 0, trans_b != 0, ca, cb, bias, stream, nullptr, 0, 0, nullptr, bf16);
 }
 
 }  // extern "C"

@@ -229,6 +229,11 @@ class SingleWithBuffer final : public SingleInputWithBufferKernel, public Base {
   }
 };
 
+// fl_contract_flags of the launch context, placed where the entry points that also take fl_ref_flags expect them
+inline uint32_t ContractBits(const LaunchContext &ctx) {
+  return ctx.bf16 ? static_cast<uint32_t>(FL_CONTRACT_BF16) << FL_CONTRACT_SHIFT : 0u;
+}
+
 class DoubleNoBuffer final : public DoubleInputsWithoutBufferKernel, public Base {
  public:
   using Base::Base;
@@ -246,14 +251,14 @@ class DoubleNoBuffer final : public DoubleInputsWithoutBufferKernel, public Base
       case OpKind::GemmConstantWeightsBias: {
         const TensorView bias = Const(c0_, "bias").View();
         rc = fluidml_hip_gemm_constant_weights_bias(l, r, &bias.t, out, attrs_.alpha, attrs_.beta, attrs_.trans_a ? 1 : 0,
-                                                    attrs_.trans_b ? 1 : 0, ctx.flags, s);
+                                                    attrs_.trans_b ? 1 : 0, ctx.flags | ContractBits(ctx), s);
         break;
       }
       case OpKind::ConvWithoutPadding: {
         TensorView bias;
         if (c0_) bias = c0_->View();
         rc = fluidml_hip_conv_without_padding(l, r, c0_ ? &bias.t : nullptr, out, attrs_.strides.data(),
-                                              attrs_.dilations.data(), attrs_.group, ctx.flags, s);
+                                              attrs_.dilations.data(), attrs_.group, ctx.flags | ContractBits(ctx), s);
         break;
       }
       default: break;
@@ -273,7 +278,7 @@ class DoubleWithBuffer final : public DoubleInputsWithBufferKernel, public Base 
       if (c0_) bias = c0_->View();
       rc = fluidml_hip_conv_with_padding(&lhs.t, &rhs.t, c0_ ? &bias.t : nullptr, &output.t, buffer.ptr, buffer.bytes,
                                          attrs_.pads.data(), attrs_.strides.data(), attrs_.dilations.data(), attrs_.group,
-                                         ctx.flags, ctx.stream);
+                                         ctx.flags | ContractBits(ctx), ctx.stream);
     }
     ctx.Note(rc, GetKernelName());
   }

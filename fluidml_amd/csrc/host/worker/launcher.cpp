@@ -276,7 +276,7 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       if (bias == nullptr) throw std::logic_error("fused Gemm: the node holds no bias");
       const kernel::TensorView c = bias->View();
       rc = fluidml_hip_gemm_chain(&a.t, &b.t, &c.t, &out.t, at.alpha, at.beta, at.trans_a ? 1 : 0, at.trans_b ? 1 : 0,
-                                  &l.chain, ctx.stream);
+                                  &l.chain, contract_flags, ctx.stream);
       break;
     }
     case Launch::Kind::ConvChain: {
@@ -287,7 +287,7 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       if (bias != nullptr) c = bias->View();
       const bool padded = steps_[l.owner].node->GetKind() == flow::OpKind::ConvWithPadding;
       rc = fluidml_hip_conv_chain(&a.t, &b.t, bias ? &c.t : nullptr, &out.t, padded ? at.pads.data() : nullptr,
-                                  at.strides.data(), at.dilations.data(), at.group, &l.chain, ctx.stream);
+                                  at.strides.data(), at.dilations.data(), at.group, &l.chain, contract_flags, ctx.stream);
       break;
     }
     case Launch::Kind::SoftmaxMatVec: {

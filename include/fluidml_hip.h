@@ -89,12 +89,18 @@ enum fl_ref_flags {
   FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
 };
 
-/* Options of the contraction entry points that take `flags`. */
+/* Options of the contraction entry points (MatMul, Gemm, Conv with group 1).  The fused
+ * entry points take them as their `flags`; the entry points whose `flags` carry
+ * fl_ref_flags take them shifted left by FL_CONTRACT_SHIFT in the same word. */
 enum fl_contract_flags {
-  /* operands rounded to bf16 (nearest even), fp32 accumulation: the opt-in
-   * reduced-precision path; its error is reported separately by bench.py */
+  /* operands rounded to bf16 (nearest even), fp32 accumulation on the matrix
+   * cores: the opt-in reduced-precision path; its error is reported separately
+   * by bench.py.  Launches that do not run on the matrix cores ignore it
+   * (at most 8 rows against k-contiguous weights: the weights are streamed in
+   * fp32; depthwise and 3-d convolutions: the direct kernel). */
   FL_CONTRACT_BF16 = 1 << 0
 };
+#define FL_CONTRACT_SHIFT 16
 
 /* A short chain of elementwise operations on one float32 value, used by the
  * launch-level fusions below.  Step i replaces v (initially the chain's input
@@ -137,7 +143,7 @@ typedef struct fl_tensor {
 /* Library / device plumbing (replaces the MLIR ExecutionEngine + the per-call
  * host arena of reference src/worker/runner.cpp:56-120).                     */
 
-/* Version of this ABI; bumped on any signature change. */
+/* Version of this ABI; bumped on any signature change (2: `flags` of the fused Gemm and Conv entry points). */
 int fluidml_hip_abi_version(void);
 /* Human-readable text for a return code of this library (static storage). */
 const char *fluidml_hip_error_string(int code);
@@ -366,11 +372,11 @@ int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, co
  * projections of an attention block): rhs[i], bias[i] (all NULL or none),
  * out[i] and stride_outer[i] belong to member i.  No batch dims. */
 int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs, const fl_tensor *const *bias, const fl_tensor *const *out, int64_t n_inner, const int64_t *stride_outer, const fl_ew_program *chain, uint32_t flags, void *stream);
-/* GemmConstantWeightsBiasKernel -> elementwise chain (reference gemm.cpp:39-182). */
-int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double alpha, double beta, int32_t trans_a, int32_t trans_b, const fl_ew_program *chain, void *stream);
+/* GemmConstantWeightsBiasKernel -> elementwise chain (reference gemm.cpp:39-182); `flags` = fl_contract_flags. */
+int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double alpha, double beta, int32_t trans_a, int32_t trans_b, const fl_ew_program *chain, uint32_t flags, void *stream);
 /* Conv{With,Without}PaddingKernel -> elementwise chain (reference conv.cpp:27-280);
- * `pads` may be NULL.  ONNX semantics only (no literal-reference flags). */
-int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, const fl_ew_program *chain, void *stream);
+ * `pads` may be NULL.  ONNX semantics only (no literal-reference flags); `flags` = fl_contract_flags. */
+int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, const fl_ew_program *chain, uint32_t flags, void *stream);
 /* SoftmaxKernel over K <= 16 logits [B, K, 1] -> MatMulKernel [B, M, K] x [B, K, 1] as ONE launch:
  * out[b, m, 0] = sum_k a[b, m, k] * softmax_k(logits[b, :, 0]) (reference softmax.cpp, matmul.cpp:28-59; the
  * per-position kernel of a span-based dynamic convolution).  `out` is [B, M, 1] with the element strides

@@ -8,7 +8,11 @@ batch 8) is compiled from its ONNX file and run three ways on the same seeded we
 * the one-launch-per-node schedule (FLUIDML_FUSE=0) of the same plan.
 
 Both GPU schedules have to meet the oracle within the tolerance the configurations are specified with
-(rel 1e-4 / abs 1e-5, fp32).  For VGG-16 at batch 8 the oracle runs the batch-1 graph (same seed, hence the
+(rel 1e-4 / abs 1e-5, fp32), element by element.  An element outside it passes only if the GPU value is within
+the same tolerance of the float64 evaluation of the network (tests/torch_reference.py, pinned against the oracle
+on small instances by tests/test_oracle_graphs.py): the oracle adds the products of each dot product one after
+the other in fp32 like the reference's loop nests, and over the 4,608 to 25,088 terms of VGG-16's late layers
+that rounding alone exceeds the tolerance on a few logits whose terms cancel (the test prints how many).  For VGG-16 at batch 8 the oracle runs the batch-1 graph (same seed, hence the
 same weights; tests/test_oracle_graphs.py checks that rows of a batch are independent images) on images 0
 and 7.  A BERT-base case with the layouts of the DP executor (constant costs: every tensor stored with its
 dimensions reversed) runs the same comparison on non-identity strides at real extents.
@@ -19,7 +23,7 @@ import numpy as np
 import pytest
 
 from oracle import graph_runner
-from tests.util import assert_close
+from tests.util import assert_close, assert_close_or_exact
 
 pytestmark = pytest.mark.gpu
 
@@ -75,6 +79,23 @@ def _vgg_oracle(image):
     return ref
 
 
+def _exact(config, net, feeds, rows):
+    """float64 torch forward pass of the configuration (tests/torch_reference.py), rows `rows` of its output"""
+    from tests import torch_reference as tr
+
+    if config == "bert_base":
+        out = tr.bert(net, feeds, seq=128, layers=12, hidden=768, heads=12, ffn=3072, vocab=30522)
+    elif config == "convbert_base":
+        out = tr.convbert(net, feeds, seq=128, layers=12, hidden=768, heads=12, ffn=3072, vocab=30522)
+    elif config == "gpt_neox":
+        out = tr.gpt_neox(net, feeds, seq=256, layers=6, hidden=512, heads=8, ffn=2048, vocab=50304)
+    elif config == "efficientnet_b0":
+        out = tr.efficientnet_b0(net, feeds)
+    else:
+        out = tr.vgg16(net, feeds)
+    return out.numpy()[rows]
+
+
 def _oracle(config, net, feeds, progress):
     """name -> (rows of the output the oracle computed, expected values)"""
     if not config.startswith("vgg16"):
@@ -104,10 +125,19 @@ def test_full_size_matches_oracle(device, config, tmp_path, monkeypatch, progres
     fused, fused_plan = _run(fluidml, net, feeds, path, config + "_fused")
     assert len(plain_plan["launches"]) == len(net.nodes) > len(fused_plan["launches"])
     assert _EXPECTED_KINDS[config] <= {l["kind"] for l in fused_plan["launches"]}
+    cache = {}
+
+    def exact_rows(rows):
+        if "out" not in cache:
+            progress("[case] full size", config, "float64 torch forward pass")
+            cache["out"] = _exact(config, net, feeds, slice(None))
+        return cache["out"][rows]
+
     for name, (rows, ref) in want.items():
         assert np.isfinite(ref).all()
-        assert_close(plain[name][rows], ref, what=f"{config} per-node launches vs oracle, {name}")
-        assert_close(fused[name][rows], ref, what=f"{config} fused launches vs oracle, {name}")
+        for what, got in (("per-node launches", plain), ("fused launches", fused)):
+            assert_close_or_exact(got[name][rows], ref, lambda: exact_rows(rows), what=f"{config} {what} vs oracle, {name}",
+                                  report=progress)
     for name, ref in plain.items():  # every row, also those the oracle did not compute
         assert np.isfinite(ref).all()
         assert_close(fused[name], ref, what=f"{config} fused vs per-node {name}")

@@ -985,7 +985,7 @@ def test_conv_and_gemm_chain(device):
         do = DeviceView(ok.View.empty(oshape, np.float32, [0, 3, 1, 2]), device)
         chain = cabi.make_chain(swish)
         cabi.call("conv_chain", dx.ref(), dw.ref(), db.ref(), do.ref(), cabi.i64_array(pads), cabi.i64_array(strides),
-                  cabi.i64_array([1, 1]), ctypes.c_int64(group), ctypes.byref(chain), None)
+                  cabi.i64_array([1, 1]), ctypes.c_int64(group), ctypes.byref(chain), ctypes.c_uint32(0), None)
         assert_close(do.logical(), want.logical(), what="conv_chain swish")
     # Gemm -> Relu (transB, alpha = beta = 1)
     a, b, c = rand(rng, (8, 100), -1, 1), rand(rng, (50, 100), -0.05, 0.05), rand(rng, (50,), -0.2, 0.2)
@@ -997,8 +997,66 @@ def test_conv_and_gemm_chain(device):
     do = DeviceView(ok.View.empty((8, 50)), device)
     relu = cabi.make_chain([(cabi.EW_RELU, 0)])
     cabi.call("gemm_chain", da.ref(), db.ref(), dc.ref(), do.ref(), ctypes.c_double(1.0), ctypes.c_double(1.0), 0, 1,
-              ctypes.byref(relu), None)
+              ctypes.byref(relu), ctypes.c_uint32(0), None)
     assert_close(do.logical(), want.logical(), what="gemm_chain relu")
+
+
+def test_gemm_and_conv_bf16(device):
+    """The opt-in path on Gemm and on convolutions that run as implicit GEMM: operands rounded to bf16, products and
+    sums in fp32.  Checked to the fp32 tolerance against the oracle run on the rounded operands (bias unrounded), through
+    the plain entry points (option in the upper half of `flags`) and the fused ones."""
+    cabi = _cabi()
+    rng = np.random.default_rng(96)
+    bits = cabi.FL_CONTRACT_BF16 << cabi.FL_CONTRACT_SHIFT
+    # Gemm with more than 8 rows (matrix cores); transB, alpha = beta = 1
+    for M, K, N in [(64, 256, 96), (200, 1000, 130)]:
+        a, b, c = rand(rng, (M, K), -1, 1), rand(rng, (N, K), -0.05, 0.05), rand(rng, (N,), -0.2, 0.2)
+        want, exact = ok.View.empty((M, N)), ok.View.empty((M, N))
+        ok.gemm(ok.View(_round_bf16(a)), ok.View(_round_bf16(b)), ok.View(c), want, 1.0, 1.0, 0, 1, 0)
+        ok.gemm(ok.View(a), ok.View(b), ok.View(c), exact, 1.0, 1.0, 0, 1, 0)
+        announce("gemm bf16", M, K, N)
+        da, db, dc = DeviceView(ok.View(a), device), DeviceView(ok.View(b), device), DeviceView(ok.View(c), device)
+        do = DeviceView(ok.View.empty((M, N), fill=4), device)
+        cabi.call("gemm_constant_weights_bias", da.ref(), db.ref(), dc.ref(), do.ref(), ctypes.c_double(1.0), ctypes.c_double(1.0),
+                  0, 1, ctypes.c_uint32(bits), None)
+        assert_close(do.logical(), want.logical(), what="gemm bf16 vs oracle on bf16-rounded operands")
+        assert not np.array_equal(do.logical(), exact.logical()), "the bf16 option had no effect"
+        do2 = DeviceView(ok.View.empty((M, N), fill=4), device)
+        none = cabi.make_chain([])
+        cabi.call("gemm_chain", da.ref(), db.ref(), dc.ref(), do2.ref(), ctypes.c_double(1.0), ctypes.c_double(1.0), 0, 1,
+                  ctypes.byref(none), ctypes.c_uint32(cabi.FL_CONTRACT_BF16), None)
+        assert_close(do2.logical(), do.logical(), exact=True, what="gemm_chain bf16 vs gemm bf16")
+        err = np.abs(do.logical().astype(np.float64) - exact.logical())
+        print(f"[bf16] gemm {M}x{K}x{N}: max abs err vs fp32 {err.max():.3e}, relative to max |c| {err.max() / np.abs(exact.logical()).max():.3e}")
+    # 3x3 pad 1 (gather path, 32x32 and 64x64 tiles), 1x1 (plain batched contraction), strided 3x3; depthwise ignores the option
+    for xshape, wshape, pads, strides, group in [((2, 8, 20, 20), (16, 8, 3, 3), [1, 1, 1, 1], [1, 1], 1),
+                                                 ((4, 16, 64, 64), (128, 16, 3, 3), [1, 1, 1, 1], [1, 1], 1),
+                                                 ((2, 24, 14, 14), (40, 24, 1, 1), [0, 0, 0, 0], [1, 1], 1),
+                                                 ((1, 8, 21, 21), (12, 8, 3, 3), [1, 1, 1, 1], [2, 2], 1),
+                                                 ((1, 6, 15, 15), (6, 1, 5, 5), [2, 2, 2, 2], [2, 2], 6)]:
+        x, w, bias = rand(rng, xshape, -1, 1), rand(rng, wshape, -0.3, 0.3), rand(rng, (wshape[0],), -1, 1)
+        od = tuple((xshape[2 + d] + 2 * pads[d] - wshape[2 + d]) // strides[d] + 1 for d in range(2))
+        oshape = (xshape[0], wshape[0]) + od
+        want, exact = ok.View.empty(oshape), ok.View.empty(oshape)
+        rounded = group == 1
+        ok.conv(ok.View(_round_bf16(x) if rounded else x), ok.View(_round_bf16(w) if rounded else w), ok.View(bias), want, pads, strides,
+                [1, 1], group, 0)
+        ok.conv(ok.View(x), ok.View(w), ok.View(bias), exact, pads, strides, [1, 1], group, 0)
+        announce("conv bf16", xshape, wshape, group)
+        dx, dw, db = DeviceView(ok.View(x), device), DeviceView(ok.View(w), device), DeviceView(ok.View(bias), device)
+        do = DeviceView(ok.View.empty(oshape, fill=4), device)
+        cabi.call("conv_with_padding", dx.ref(), dw.ref(), db.ref(), do.ref(), None, 0, cabi.i64_array(pads), cabi.i64_array(strides),
+                  cabi.i64_array([1, 1]), ctypes.c_int64(group), ctypes.c_uint32(bits), None)
+        assert_close(do.logical(), want.logical(), what="conv bf16 vs oracle on bf16-rounded operands")
+        if rounded:
+            assert not np.array_equal(do.logical(), exact.logical()), "the bf16 option had no effect"
+        do2 = DeviceView(ok.View.empty(oshape, fill=4), device)
+        none = cabi.make_chain([])
+        cabi.call("conv_chain", dx.ref(), dw.ref(), db.ref(), do2.ref(), cabi.i64_array(pads), cabi.i64_array(strides),
+                  cabi.i64_array([1, 1]), ctypes.c_int64(group), ctypes.byref(none), ctypes.c_uint32(cabi.FL_CONTRACT_BF16), None)
+        assert_close(do2.logical(), do.logical(), exact=True, what="conv_chain bf16 vs conv bf16")
+        err = np.abs(do.logical().astype(np.float64) - exact.logical())
+        print(f"[bf16] conv {xshape} * {wshape}: max abs err vs fp32 {err.max():.3e}, relative to max |out| {err.max() / np.abs(exact.logical()).max():.3e}")
 
 
 def test_fused_div_add_softmax(device):

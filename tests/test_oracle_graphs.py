@@ -3,7 +3,7 @@ fluidml_amd/models.py WITHOUT the product beside them.
 
 For a small instance of each of the five architectures the graph generator's output, executed by the
 oracle's loop nests, has to agree with an independent float64 torch-functional forward pass that is
-written here from the architecture descriptions alone (BERT: post-LN, erf-GELU, additive mask;
+written in tests/torch_reference.py from the architecture descriptions alone (BERT: post-LN, erf-GELU, additive mask;
 ConvBERT: mixed attention with span-based dynamic convolution, kernel 9; GPT-NeoX: rotary embedding on
 a quarter of each head, causal mask, parallel residual; EfficientNet-B0: MBConv with squeeze-excite and
 swish; VGG-16).  The forward passes take the weights from the graph's initializers in creation order,
@@ -16,8 +16,6 @@ include/structure/flow/node.h:672-673 LayerNormalization axis 1 / epsilon 1e-5, 
 :389/:517 Gather axis 0, :504 Flatten axis 1; converter.cpp:2413-2438 Transpose perm reversed;
 converter.cpp:551-592 AveragePool strides 1), each on a graph that omits the attribute.
 """
-import math
-
 import numpy as np
 import pytest
 import torch
@@ -26,34 +24,10 @@ import torch.nn.functional as F
 from fluidml_amd import models
 from fluidml_amd.onnx_writer import GraphBuilder
 from oracle import graph_runner
+from tests import torch_reference
 
 # float64 forward against the oracle's fp32 loop nests on small nets: fp32 rounding only
 RTOL, ATOL = 2e-4, 2e-5
-
-
-class Params:
-    """The float initializers of rank >= 1 in creation order, handed out one by one as float64 tensors."""
-
-    def __init__(self, net, seed):
-        rng = np.random.Generator(np.random.PCG64(seed))
-        self.items = []
-        for v in net.initializers:
-            c = v.const
-            if c.dtype != np.float32 or c.ndim == 0:
-                continue
-            if c.size > 1 and (not c.any() or (c == 1).all()):  # the generators' zero biases and unit scales
-                c[...] = rng.standard_normal(c.shape).astype(np.float32) * np.float32(0.5) + (1 if c.flat[0] == 1 else 0)
-            self.items.append(c)
-        self.at = 0
-
-    def take(self, *shape):
-        c = self.items[self.at]
-        self.at += 1
-        assert tuple(c.shape) == tuple(shape), f"initializer {self.at - 1}: shape {c.shape}, architecture wants {shape}"
-        return torch.from_numpy(c.astype(np.float64))
-
-    def done(self):
-        assert self.at == len(self.items), f"{len(self.items) - self.at} float initializers were never used"
 
 
 def _check(net, feeds, want):
@@ -68,182 +42,41 @@ def _check(net, feeds, want):
     assert np.abs(want).max() > 1e-2  # a forward pass that collapsed to zero would pin nothing
 
 
-def _gelu(x):
-    return x * 0.5 * (1.0 + torch.erf(x / math.sqrt(2.0)))
-
-
-def _attention(q, k, v, heads, bias=None, causal=False):
-    """q, k, v [1, S, heads*d] -> context [1, S, heads, d]"""
-    S, d = q.shape[1], q.shape[2] // heads
-    qh, kh, vh = (t.view(1, S, heads, d).permute(0, 2, 1, 3) for t in (q, k, v))
-    s = qh @ kh.transpose(-1, -2) / math.sqrt(d)
-    if bias is not None:
-        s = s + bias
-    if causal:
-        s = torch.where(torch.tril(torch.ones(S, S, dtype=torch.bool)), s, torch.tensor(torch.finfo(torch.float32).min, dtype=s.dtype))
-    return (torch.softmax(s, -1) @ vh).permute(0, 2, 1, 3)
-
-
-def _embeddings(p, feeds, vocab, types, hidden, seq, eps):
-    ids = torch.from_numpy(feeds["input_ids"])
-    tok = torch.from_numpy(feeds["token_type_ids"])
-    word, typ, pos = p.take(vocab, hidden), p.take(types, hidden), p.take(1, seq, hidden)
-    x = word[ids] + typ[tok] + pos
-    return F.layer_norm(x, (hidden,), p.take(hidden), p.take(hidden), eps)
-
-
 def test_bert_generator_and_runner_against_torch():
-    seq, layers, hidden, heads, ffn, vocab, eps = 16, 2, 32, 4, 64, 50, 1e-12
-    net = models.bert_base(seq=seq, layers=layers, hidden=hidden, heads=heads, ffn=ffn, vocab=vocab, max_pos=32, seed=5)
-    feeds = models.bert_inputs(seq, vocab, seed=6)
+    dims = dict(seq=16, layers=2, hidden=32, heads=4, ffn=64, vocab=50)
+    net = models.bert_base(max_pos=32, seed=5, **dims)
+    feeds = models.bert_inputs(16, 50, seed=6)
     feeds["attention_mask"][0, -3:] = 0  # the additive mask must matter
-    feeds["token_type_ids"][0, seq // 2:] = 1
-    p = Params(net, 7)
-    x = _embeddings(p, feeds, vocab, 2, hidden, seq, eps)
-    bias = (1.0 - torch.from_numpy(feeds["attention_mask"]).double())[:, None, None, :] * -10000.0
-    for _ in range(layers):
-        q = x @ p.take(hidden, hidden) + p.take(hidden)
-        k = x @ p.take(hidden, hidden) + p.take(hidden)
-        v = x @ p.take(hidden, hidden) + p.take(hidden)
-        c = _attention(q, k, v, heads, bias).reshape(1, seq, hidden)
-        o = c @ p.take(hidden, hidden) + p.take(hidden)
-        x = F.layer_norm(o + x, (hidden,), p.take(hidden), p.take(hidden), eps)
-        h = _gelu(x @ p.take(hidden, ffn) + p.take(ffn))
-        f = h @ p.take(ffn, hidden) + p.take(hidden)
-        x = F.layer_norm(f + x, (hidden,), p.take(hidden), p.take(hidden), eps)
-    p.done()
-    _check(net, feeds, x)
+    feeds["token_type_ids"][0, 8:] = 1
+    _check(net, feeds, torch_reference.bert(net, feeds, randomize_seed=7, **dims))
 
 
 def test_convbert_generator_and_runner_against_torch():
-    seq, layers, hidden, heads, ffn, vocab, eps, ck = 16, 2, 32, 4, 64, 50, 1e-12, 9
-    net = models.convbert_base(seq=seq, layers=layers, hidden=hidden, heads=heads, ffn=ffn, vocab=vocab, max_pos=32, seed=8)
-    feeds = models.bert_inputs(seq, vocab, seed=9)
+    dims = dict(seq=16, layers=2, hidden=32, heads=4, ffn=64, vocab=50)
+    net = models.convbert_base(max_pos=32, seed=8, **dims)
+    feeds = models.bert_inputs(16, 50, seed=9)
     feeds["attention_mask"][0, :2] = 0
-    p = Params(net, 10)
-    nh = heads // 2
-    hd = hidden // heads
-    inner = nh * hd
-    x = _embeddings(p, feeds, vocab, 2, hidden, seq, eps)
-    bias = (1.0 - torch.from_numpy(feeds["attention_mask"]).double())[:, None, None, :] * -10000.0
-    for _ in range(layers):
-        q = x @ p.take(hidden, inner) + p.take(inner)
-        k = x @ p.take(hidden, inner) + p.take(inner)
-        v = x @ p.take(hidden, inner) + p.take(inner)
-        # separable convolution of the layer input over the sequence: depthwise k=9 (no bias), pointwise (+ bias)
-        dw = F.conv1d(x.transpose(1, 2), p.take(hidden, 1, ck), None, padding=ck // 2, groups=hidden)
-        key_conv = F.conv1d(dw, p.take(inner, hidden, 1), p.take(inner)).transpose(1, 2)
-        conv_attn = key_conv * q
-        kernel = conv_attn @ p.take(inner, nh * ck) + p.take(nh * ck)
-        kernel = torch.softmax(kernel.reshape(seq * nh, ck, 1), dim=1)
-        conv_out = x @ p.take(hidden, inner) + p.take(inner)
-        windows = F.pad(conv_out, (0, 0, ck // 2, ck // 2)).unfold(1, ck, 1)        # [1, S, inner, k]
-        conv_out = (windows.reshape(seq * nh, hd, ck) @ kernel).reshape(1, seq, nh, hd)
-        c = torch.cat([_attention(q, k, v, nh, bias), conv_out], dim=2).reshape(1, seq, hidden)
-        o = c @ p.take(hidden, hidden) + p.take(hidden)
-        x = F.layer_norm(o + x, (hidden,), p.take(hidden), p.take(hidden), eps)
-        h = _gelu(x @ p.take(hidden, ffn) + p.take(ffn))
-        f = h @ p.take(ffn, hidden) + p.take(hidden)
-        x = F.layer_norm(f + x, (hidden,), p.take(hidden), p.take(hidden), eps)
-    p.done()
-    _check(net, feeds, x)
+    _check(net, feeds, torch_reference.convbert(net, feeds, randomize_seed=10, **dims))
 
 
 def test_gpt_neox_generator_and_runner_against_torch():
-    seq, layers, hidden, heads, ffn, vocab, eps = 24, 2, 64, 2, 128, 70, 1e-5
-    net = models.gpt_neox(seq=seq, layers=layers, hidden=hidden, heads=heads, ffn=ffn, vocab=vocab, seed=11)
-    feeds = models.gpt_neox_inputs(seq, vocab, seed=12)
-    p = Params(net, 13)
-    hd = hidden // heads
-    rot = hd // 4
-    x = p.take(vocab, hidden)[torch.from_numpy(feeds["input_ids"])]
-    # rotary tables, base 10000, over the first quarter of each head; the graph's constants must equal them
-    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot))
-    ang = torch.arange(seq, dtype=torch.float64)[:, None] * inv_freq[None, :]
-    emb = torch.cat([ang, ang], dim=-1)
-    cos, sin = p.take(1, 1, seq, rot), p.take(1, 1, seq, rot)
-    assert torch.allclose(cos[0, 0], emb.cos(), atol=1e-6, rtol=0) and torch.allclose(sin[0, 0], emb.sin(), atol=1e-6, rtol=0)
-
-    def rotary(t):  # [1, heads, S, hd]
-        t_rot, t_pass = t[..., :rot], t[..., rot:]
-        half = torch.cat([-t_rot[..., rot // 2:], t_rot[..., : rot // 2]], dim=-1)
-        return torch.cat([t_rot * emb.cos() + half * emb.sin(), t_pass], dim=-1)
-
-    for _ in range(layers):
-        a_in = F.layer_norm(x, (hidden,), p.take(hidden), p.take(hidden), eps)
-        qkv = (a_in @ p.take(hidden, 3 * hidden) + p.take(3 * hidden)).view(1, seq, heads, 3 * hd)
-        q, k, v = (qkv[..., i * hd:(i + 1) * hd].permute(0, 2, 1, 3) for i in range(3))
-        q, k = rotary(q), rotary(k)
-        s = (q @ k.transpose(-1, -2)) * (1.0 / math.sqrt(hd))
-        s = torch.where(torch.tril(torch.ones(seq, seq, dtype=torch.bool)), s, torch.tensor(float(np.finfo(np.float32).min), dtype=s.dtype))
-        c = (torch.softmax(s, -1) @ v).permute(0, 2, 1, 3).reshape(1, seq, hidden)
-        attn = c @ p.take(hidden, hidden) + p.take(hidden)
-        m_in = F.layer_norm(x, (hidden,), p.take(hidden), p.take(hidden), eps)
-        h = _gelu(m_in @ p.take(hidden, ffn) + p.take(ffn))
-        mlp = h @ p.take(ffn, hidden) + p.take(hidden)
-        x = mlp + attn + x
-    x = F.layer_norm(x, (hidden,), p.take(hidden), p.take(hidden), eps)
-    logits = x @ p.take(hidden, vocab)
-    p.done()
-    _check(net, feeds, logits)
-
-
-def _swish(x):
-    return x * torch.sigmoid(x)
+    dims = dict(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=70)
+    net = models.gpt_neox(seed=11, **dims)
+    feeds = models.gpt_neox_inputs(24, 70, seed=12)
+    _check(net, feeds, torch_reference.gpt_neox(net, feeds, randomize_seed=13, **dims))
 
 
 def test_efficientnet_generator_and_runner_against_torch():
-    image, classes, div = 32, 10, 4
-    net = models.efficientnet_b0(image=image, classes=classes, width_div=div, seed=14)
-    feeds = models.image_input((1, 3, image, image), seed=15)
-    p = Params(net, 16)
-
-    def ch(c):
-        return max(4, c // div)
-
-    def conv(x, cout, k, stride, groups=1):
-        cin = x.shape[1]
-        return F.conv2d(x, p.take(cout, cin // groups, k, k), p.take(cout), stride=stride, padding=(k - 1) // 2, groups=groups)
-
-    x = _swish(conv(torch.from_numpy(feeds["input"]).double(), ch(32), 3, 2))
-    stages = [(1, 3, 1, 16, 1), (6, 3, 2, 24, 2), (6, 5, 2, 40, 2), (6, 3, 2, 80, 3), (6, 5, 1, 112, 3), (6, 5, 2, 192, 4), (6, 3, 1, 320, 1)]
-    for expand, k, stride, cout, repeats in stages:
-        for r in range(repeats):
-            inp, cin = x, x.shape[1]
-            mid = cin * expand
-            h = _swish(conv(x, mid, 1, 1)) if expand != 1 else x
-            h = _swish(conv(h, mid, k, stride if r == 0 else 1, groups=mid))
-            se = h.mean(dim=(2, 3), keepdim=True)
-            se = _swish(conv(se, max(1, cin // 4), 1, 1))
-            se = torch.sigmoid(conv(se, mid, 1, 1))
-            h = conv(h * se, ch(cout), 1, 1)
-            x = h + inp if h.shape == inp.shape and (r > 0 or stride == 1) else h
-    x = _swish(conv(x, ch(1280), 1, 1)).mean(dim=(2, 3))
-    logits = x @ p.take(classes, x.shape[1]).T + p.take(classes)
-    p.done()
-    _check(net, feeds, logits)
+    net = models.efficientnet_b0(image=32, classes=10, width_div=4, seed=14)
+    feeds = models.image_input((1, 3, 32, 32), seed=15)
+    _check(net, feeds, torch_reference.efficientnet_b0(net, feeds, classes=10, div=4, randomize_seed=16))
 
 
 @pytest.mark.parametrize("batch", [1, 2])
 def test_vgg16_generator_and_runner_against_torch(batch):
-    image, classes, div = 32, 10, 8
-    net = models.vgg16(batch=batch, image=image, classes=classes, width_div=div, seed=17)
-    feeds = models.image_input((batch, 3, image, image), seed=18)
-    p = Params(net, 19)
-    x = torch.from_numpy(feeds["input"]).double()
-    for item in [64, 64, "M", 128, 128, "M", 256, 256, 256, "M", 512, 512, 512, "M", 512, 512, 512, "M"]:
-        if item == "M":
-            x = F.max_pool2d(x, 2, 2)
-        else:
-            cout = max(4, item // div)
-            x = F.relu(F.conv2d(x, p.take(cout, x.shape[1], 3, 3), p.take(cout), padding=1))
-    x = x.flatten(1)
-    for i, n in enumerate([4096 // div, 4096 // div, classes]):
-        x = x @ p.take(n, x.shape[1]).T + p.take(n)
-        if i < 2:
-            x = F.relu(x)
-    p.done()
-    _check(net, feeds, x)
+    net = models.vgg16(batch=batch, image=32, classes=10, width_div=8, seed=17)
+    feeds = models.image_input((batch, 3, 32, 32), seed=18)
+    _check(net, feeds, torch_reference.vgg16(net, feeds, classes=10, div=8, randomize_seed=19))
 
 
 def test_vgg16_batch_rows_are_independent_images():

@@ -20,6 +20,7 @@ ContextImpl::ContextImpl() {
   if (const char *f = std::getenv("FLUIDML_FUSE")) fuse = std::string(f) != "0";
   if (const char *h = std::getenv("FLUIDML_BF16")) bf16 = std::string(h) != "0";
   if (const char *gp = std::getenv("FLUIDML_GRAPH_PASSES")) graph_passes = std::string(gp) != "0";
+  if (const char *k = std::getenv("FLUIDML_DP_CHECK")) dp_check_whole_plan = std::string(k) != "0";
   if (const char *c = std::getenv("FLUIDML_DP_COST")) {
     const std::string mode(c);
     if (mode == "constant") {
@@ -41,6 +42,8 @@ worker::LaunchPlan &ContextImpl::GetModule() {
 }
 
 void ContextImpl::SetModule(std::unique_ptr<worker::LaunchPlan> &&module) { module_ = std::move(module); }
+
+std::unique_ptr<worker::LaunchPlan> ContextImpl::ReleaseModule() { return std::move(module_); }
 
 FuncAttr &ContextImpl::GetFuncAttr() {
   if (!func_attr_) throw std::logic_error("Context: no function attributes yet (run a builder first)");

@@ -73,6 +73,7 @@ class ContextImpl {
   worker::LaunchPlan &GetModule();
   bool HasModule() const { return module_ != nullptr; }
   void SetModule(std::unique_ptr<worker::LaunchPlan> &&module);
+  std::unique_ptr<worker::LaunchPlan> ReleaseModule();
   FuncAttr &GetFuncAttr();
   void SetFuncAttr(FuncAttr &&attr);
 
@@ -90,6 +91,9 @@ class ContextImpl {
   // cost source of the layout DP (env FLUIDML_DP_COST=measure|constant|<path to table json>)
   CostMode cost_mode = CostMode::Measure;
   std::string cost_table_path;
+  // DP executor with measured costs: time the proposed plan as a whole against the default layouts and keep the
+  // faster (env FLUIDML_DP_CHECK=0 keeps the DP's proposal whatever it costs)
+  bool dp_check_whole_plan = true;
   std::shared_ptr<evaluation::CostModel> cost_model;  // created on first use
 
  private:

@@ -2,10 +2,17 @@
 
 #include "optimization/graph_passes.h"
 
+#include <algorithm>
+#include <fstream>
+#include <iterator>
+#include <sstream>
 #include <stdexcept>
+
+#include "utils/json.h"
 
 #include "worker/builder.h"
 #include "worker/converter.h"
+#include "worker/launcher.h"
 #include "worker/lower.h"
 #include "worker/parser.h"
 #include "worker/planner.h"
@@ -23,30 +30,15 @@ class ExecutorImpl : public Executor {
       : name_(std::move(name)), epoch_(epoch), flavour_(flavour) {}
 
   void Compile(std::istream &input, std::ofstream *mlir, std::ofstream *llvm, std::ofstream *json) override {
-    std::unique_ptr<Parser> parser = Parser::Make();
-    std::unique_ptr<Converter> converter = Converter::Make();
-    std::string fn = name_;
-    std::unique_ptr<GeneralBuilder> builder = flavour_ == Flavour::DPGreedy ? context_.MakeDPGeneralBuilder(std::move(fn))
-                                                                            : context_.MakePlainGeneralBuilder(std::move(fn));
-    std::unique_ptr<Lower> lower = context_.MakeLower();
-    graph::Graph graph = parser->Run(input);
-    if (context_->graph_passes) {
-      optimization::GraphPassesManager passes;
-      passes.RegisterAllPasses();
-      passes.Run(graph);
+    const std::string model((std::istreambuf_iterator<char>(input)), std::istreambuf_iterator<char>());
+    std::string dp_json = Build(context_, flavour_, model);
+    if (flavour_ == Flavour::DPGreedy && context_->cost_mode == context::CostMode::Measure && context_->dp_check_whole_plan) {
+      dp_json = KeepTheFasterPlan(model, std::move(dp_json));
+    } else if (flavour_ == Flavour::DPGreedy && context_->cost_mode == context::CostMode::Table && context_->dp_check_whole_plan) {
+      dp_json = ReplayDecision(model, std::move(dp_json));
     }
-    flow::Flow flow = converter->Run(graph);
-    std::unique_ptr<Planner> planner;
-    switch (flavour_) {
-      case Flavour::PlainLinear: planner = context_.MakePlainLinearPlanner(); break;
-      case Flavour::PlainGreedy: planner = context_.MakePlainGreedyPlanner(); break;
-      case Flavour::DPGreedy: planner = context_.MakeDPGreedyPlanner(); break;
-    }
-    auto [sequence, index, dp_json] = planner->Run(flow);
     if (json) *json << dp_json;
-    builder->Run(sequence, index);
     if (mlir) *mlir << context_;
-    lower->Run();
     if (llvm) *llvm << context_;
   }
 
@@ -59,6 +51,111 @@ class ExecutorImpl : public Executor {
     if (llvm) llvm_ofs.open(std::string(*llvm));
     if (json) json_ofs.open(std::string(*json));
     Compile(ifs, mlir ? &mlir_ofs : nullptr, llvm ? &llvm_ofs : nullptr, json ? &json_ofs : nullptr);
+  }
+
+  // parse -> [graph passes] -> convert -> plan -> build -> validate, all inside `context`; returns the planner's JSON
+  std::string Build(context::Context &context, Flavour flavour, const std::string &model) {
+    std::unique_ptr<Parser> parser = Parser::Make();
+    std::unique_ptr<Converter> converter = Converter::Make();
+    std::string fn = name_;
+    std::unique_ptr<GeneralBuilder> builder = flavour == Flavour::DPGreedy ? context.MakeDPGeneralBuilder(std::move(fn))
+                                                                           : context.MakePlainGeneralBuilder(std::move(fn));
+    std::unique_ptr<Lower> lower = context.MakeLower();
+    std::istringstream stream(model);
+    graph::Graph graph = parser->Run(stream);
+    if (context->graph_passes) {
+      optimization::GraphPassesManager passes;
+      passes.RegisterAllPasses();
+      passes.Run(graph);
+    }
+    flow::Flow flow = converter->Run(graph);
+    std::unique_ptr<Planner> planner;
+    switch (flavour) {
+      case Flavour::PlainLinear: planner = context.MakePlainLinearPlanner(); break;
+      case Flavour::PlainGreedy: planner = context.MakePlainGreedyPlanner(); break;
+      case Flavour::DPGreedy: planner = context.MakeDPGreedyPlanner(); break;
+    }
+    auto [sequence, index, dp_json] = planner->Run(flow);
+    builder->Run(sequence, index);
+    lower->Run();
+    return dp_json;
+  }
+
+  // The DP sums costs of kernels timed one by one, but what runs is the fused launch schedule, and a layout that
+  // wins a few hundred nanoseconds for one kernel can cost a whole launch when it keeps a chain from being fused.
+  // So the plan the DP proposes is timed as a whole (replays of its launch schedule on zero-filled inputs) against
+  // the plan with default layouts, and the faster one is kept.  The memory plan is the same for both: offsets do
+  // not depend on layouts.  The JSON keeps the reference's two keys -- "plan" lists the layouts in use -- and gains
+  // "whole_graph_ns" (both timings, which plan was kept) and, when the default layouts won, the DP's proposal
+  // under "dp_plan".
+  std::string KeepTheFasterPlan(const std::string &model, std::string &&dp_json) {
+    context::Context plain = PlainTwin();
+    Build(plain, Flavour::PlainGreedy, model);
+    constexpr size_t kWarmup = 3, kIters = 20;
+    double dp_ns = context_->GetModule().TimeReplayNs(kWarmup, kIters);
+    double plain_ns = plain->GetModule().TimeReplayNs(kWarmup, kIters);
+    dp_ns = std::min(dp_ns, context_->GetModule().TimeReplayNs(1, kIters));  // best of two rounds each
+    plain_ns = std::min(plain_ns, plain->GetModule().TimeReplayNs(1, kIters));
+    const bool keep_dp = dp_ns <= plain_ns;
+    const std::string timing = "\"whole_graph_ns\":{\"dp\":" + std::to_string(static_cast<long long>(dp_ns)) +
+                               ",\"default_layouts\":" + std::to_string(static_cast<long long>(plain_ns)) + ",\"kept\":\"" +
+                               (keep_dp ? "dp" : "default_layouts") + "\"}";
+    return Decide(keep_dp, plain, std::move(dp_json), timing);
+  }
+
+  // A cost table written by a compile that kept the default layouts replays that decision (no timing).
+  std::string ReplayDecision(const std::string &model, std::string &&dp_json) {
+    std::ifstream ifs(context_->cost_table_path);
+    std::stringstream text;
+    text << ifs.rdbuf();
+    const json::Value doc = json::Parse(text.str());
+    if (!doc.Has("whole_graph_ns")) return std::move(dp_json);
+    const json::Value &t = doc.At("whole_graph_ns");
+    const bool keep_dp = !(t.Has("kept") && t.At("kept").string == "default_layouts");
+    const std::string timing = "\"whole_graph_ns\":{\"dp\":" + std::to_string(static_cast<long long>(t.At("dp").number)) +
+                               ",\"default_layouts\":" + std::to_string(static_cast<long long>(t.At("default_layouts").number)) +
+                               ",\"kept\":\"" + (keep_dp ? "dp" : "default_layouts") + "\"}";
+    context::Context plain = PlainTwin();
+    if (!keep_dp) Build(plain, Flavour::PlainGreedy, model);
+    return Decide(keep_dp, plain, std::move(dp_json), timing);
+  }
+
+  // a context with this one's switches and nothing built
+  context::Context PlainTwin() {
+    context::Context plain;
+    plain->ref_flags = context_->ref_flags;
+    plain->use_graph = context_->use_graph;
+    plain->fuse = context_->fuse;
+    plain->graph_passes = context_->graph_passes;
+    plain->bf16 = context_->bf16;
+    return plain;
+  }
+
+  // Rewrites the planner's JSON for the plan that stays and, if that is the one with default layouts, moves it
+  // from `plain` into this executor's context.
+  std::string Decide(bool keep_dp, context::Context &plain, std::string &&dp_json, const std::string &timing) {
+    const std::string key = ",\"plan\":";
+    const size_t at = dp_json.rfind(key);
+    if (at == std::string::npos || dp_json.empty() || dp_json.back() != '}') {
+      throw std::logic_error("Executor: the planner's JSON does not end with its \"plan\" object");
+    }
+    const std::string head = dp_json.substr(0, at);
+    const std::string proposal = dp_json.substr(at + key.size(), dp_json.size() - at - key.size() - 1);
+    if (keep_dp) return head + key + proposal + "," + timing + "}";
+    // default layouts: every tensor of the proposal with the identity permutation of its rank
+    const json::Value plan = json::Parse(proposal);
+    std::string identity = "{";
+    bool first = true;
+    for (const auto &kv : plan.object) {
+      identity += (first ? "" : ",") + json::Quote(kv.first) + ":[";
+      for (size_t i = 0; i < kv.second.array.size(); ++i) identity += (i ? "," : "") + std::to_string(i);
+      identity += "]";
+      first = false;
+    }
+    identity += "}";
+    context_->SetFuncAttr(context::FuncAttr(plain->GetFuncAttr()));
+    context_->SetModule(plain->ReleaseModule());
+    return head + key + identity + "," + timing + ",\"dp_plan\":" + proposal + "}";
   }
 
   size_t Invoke(const std::unordered_map<std::string, void *> &args) override {

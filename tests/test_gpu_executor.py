@@ -86,7 +86,18 @@ def test_dp_measured_layouts_match_oracle(device, tiny_bert, monkeypatch, tmp_pa
     for name, ref in want.items():
         assert_close(got[name], ref, what=f"dp measured {name}")
     first = {s["output"]: s["output_layout"] for s in ex.plan()["steps"]}
-    # same cost table -> same layouts
+    # the proposal was timed as a whole against the default layouts and the faster plan kept; "plan" lists what runs
+    import json
+
+    doc = json.load(open(json_path))
+    assert {"dp_table", "plan", "whole_graph_ns"} <= set(doc)
+    timing = doc["whole_graph_ns"]
+    assert timing["kept"] == ("dp" if timing["dp"] <= timing["default_layouts"] else "default_layouts")
+    assert ("dp_plan" in doc) == (timing["kept"] == "default_layouts")
+    for name, layout in first.items():
+        if name in doc["plan"] and name not in {v.name for v in net.outputs}:
+            assert doc["plan"][name] == layout, name
+    # same cost table -> same decision, same layouts
     monkeypatch.setenv("FLUIDML_DP_COST", json_path)
     announce("tiny bert dp replay from table")
     ex2 = fluidml.Executor.make_dp_greedy("tiny_dp_replay")

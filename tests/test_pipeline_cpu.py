@@ -536,6 +536,65 @@ def test_dp_constant_cost_closed_form(mods, tiny):
     assert set(row) == {"input_shape", "output_shape", "input_layout", "output_layout", "time_cost"}
 
 
+def test_dp_json_serves_the_reference_analyzer(mods, tiny):
+    """The JSON a DP compile emits is what the reference's tools/analyzer.py reads (its `onnx` import is absent
+    here, so its lookups are replayed on the generated graph): for every graph node, the row of the node's kernel
+    with the operands' shapes and the DEFAULT layouts, and the row with the layouts of data["plan"], both found
+    by the equality tests of find_single_input / find_double_inputs (reference tools/analyzer.py:19-93), operand
+    names chosen per operator as in its main loop (:150-700): single-input kernels by their one runtime tensor,
+    Add/Mul with a rank-0 initializer as the *Constant kernels, MatMul/Add with a weight by (lhs, rhs, output)
+    with the weight's layout taken from data["plan"] too."""
+    fluidml, _, _ = mods
+    net, path = tiny
+    _, _, _, report = staged(fluidml, path, "make_dp_greedy_planner")
+    data = json.loads(report)
+    dp_table, plan = data["dp_table"]["evaluator"], data["plan"]
+    infos = {v.name: list(v.shape) for n in net.nodes for v in n.outputs + n.inputs}
+    consts = {v.name for v in net.initializers}
+
+    def single(kernel, x, out):
+        rows = dp_table[kernel]
+        for layouts in ([list(range(len(infos[x]))), list(range(len(infos[out])))], [plan[x], plan[out]]):
+            hit = [r for r in rows if r["input_shape"] == infos[x] and r["output_shape"] == infos[out] and
+                   r["input_layout"] == layouts[0] and r["output_layout"] == layouts[1]]
+            assert hit and isinstance(hit[0]["time_cost"], int), (kernel, x, out, layouts)
+
+    def double(kernel, lhs, rhs, out):
+        rows = dp_table[kernel]
+        for layouts in ([list(range(len(infos[t]))) for t in (lhs, rhs, out)], [plan[lhs], plan[rhs], plan[out]]):
+            hit = [r for r in rows if r["lhs_shape"] == infos[lhs] and r["rhs_shape"] == infos[rhs] and
+                   r["output_shape"] == infos[out] and r["lhs_layout"] == layouts[0] and r["rhs_layout"] == layouts[1] and
+                   r["output_layout"] == layouts[2]]
+            assert hit and isinstance(hit[0]["time_cost"], int), (kernel, lhs, rhs, out, layouts)
+
+    seen = set()
+    for n in net.nodes:
+        ins, out, op = [v.name for v in n.inputs], n.outputs[0].name, n.op_type
+        runtime = [i for i in ins if i not in consts]
+        scalars = [i for i in ins if i in consts and infos[i] == []]
+        seen.add(op)
+        if op in ("Add", "Mul"):
+            if scalars:
+                single(op + "ConstantKernel", runtime[0], out)
+            else:
+                double(op + "CommonKernel", ins[0], ins[1], out)
+        elif op == "Sub":
+            single("SubConstantLhsKernel", ins[1], out)
+        elif op == "Div":
+            single("DivConstantRhsKernel", ins[0], out)
+        elif op == "Gather":
+            single("GatherConstantDataTensorKernel", ins[1], out)
+        elif op == "MatMul":
+            double("MatMulKernel", ins[0], ins[1], out)
+        elif op == "LayerNormalization":
+            single("LayerNormalizationConstantScaleBiasKernel", ins[0], out)
+        else:
+            assert op in ("Erf", "Softmax", "Reshape", "Transpose", "Unsqueeze"), op
+            single(op + "Kernel", ins[0], out)
+    assert {"Add", "Mul", "Sub", "Div", "Gather", "MatMul", "LayerNormalization", "Erf", "Softmax", "Reshape", "Transpose",
+            "Unsqueeze"} <= seen
+
+
 def synthetic_cost(kernel, layouts):
     return 1 + zlib.crc32(repr((kernel, layouts)).encode()) % 1000
 

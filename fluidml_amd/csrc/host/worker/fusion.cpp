@@ -332,8 +332,9 @@ class Scheduler {
   }
 
   // ---- view elision -----------------------------------------------------------------------------------
-  // A Slice, Transpose, Squeeze, Unsqueeze or (where the result is still one strided pattern) Reshape / Flatten
-  // that no fusion has absorbed does not have to run: every kernel here takes element strides, so the readers
+  // A Slice, Transpose, Squeeze, Unsqueeze, a Gather whose constant indices form an arithmetic pattern (sliding
+  // windows), or (where the result is still one strided pattern) a Reshape / Flatten that no fusion has absorbed
+  // does not have to run: every kernel here takes element strides, so the readers
   // can address the step's input directly.  Allowed when the tensor is internal, and the bytes of the input stay
   // untouched from the step's position to the position where each reader is issued (the input may be dead in
   // the memory plan by then, and its bytes reused).
@@ -419,6 +420,54 @@ class Scheduler {
         if (j != ishape.size()) return std::nullopt;
         break;
       }
+      case OpKind::GatherConstantIndicesTensor: {
+        // indices that form an arithmetic pattern, index[j0, j1, ..] = base + sum_d j_d * step_d with every step
+        // >= 0 (the sliding windows of an unfolded convolution: index[s, k] = s + k), turn the gathered axis into
+        // one strided dim per index dim; the windows may overlap, which a reader does not mind
+        if (!at.t0) return std::nullopt;
+        const Tensor &index = *at.t0;
+        const auto &qshape = index.GetShape();
+        const int64_t q = static_cast<int64_t>(qshape.size());
+        int64_t axis = at.axis < 0 ? at.axis + irank : at.axis;
+        if (axis < 0 || axis >= irank || orank != irank - 1 + q || q == 0) return std::nullopt;
+        const std::vector<float64_t> &values = index.Get();
+        int64_t count = 1;
+        for (int64_t d : qshape) count *= d;
+        if (count <= 0 || static_cast<int64_t>(values.size()) != count) return std::nullopt;
+        const int64_t base = static_cast<int64_t>(values[0]);
+        std::vector<int64_t> step(static_cast<size_t>(q), 0), unit(static_cast<size_t>(q), 1);
+        for (int64_t d = q - 2; d >= 0; --d) unit[static_cast<size_t>(d)] = unit[static_cast<size_t>(d + 1)] * qshape[static_cast<size_t>(d + 1)];
+        for (int64_t d = 0; d < q; ++d) {
+          if (qshape[static_cast<size_t>(d)] > 1) step[static_cast<size_t>(d)] = static_cast<int64_t>(values[static_cast<size_t>(unit[static_cast<size_t>(d)])]) - base;
+          if (step[static_cast<size_t>(d)] < 0) return std::nullopt;
+        }
+        for (int64_t n = 0; n < count; ++n) {
+          int64_t rem = n, want = base;
+          for (int64_t d = 0; d < q; ++d) {
+            want += (rem / unit[static_cast<size_t>(d)]) * step[static_cast<size_t>(d)];
+            rem %= unit[static_cast<size_t>(d)];
+          }
+          const int64_t have = static_cast<int64_t>(values[static_cast<size_t>(n)]);
+          if (have != want || static_cast<float64_t>(have) != values[static_cast<size_t>(n)] || have < 0 ||
+              have >= ishape[static_cast<size_t>(axis)]) {
+            return std::nullopt;
+          }
+        }
+        for (int64_t d = 0; d < irank; ++d) {
+          if (d != axis) {
+            strides.push_back(st[static_cast<size_t>(d)]);
+          } else {
+            for (int64_t e = 0; e < q; ++e) strides.push_back(step[static_cast<size_t>(e)] * st[static_cast<size_t>(axis)]);
+          }
+        }
+        for (int64_t d = 0, k = 0; d < irank; ++d) {  // the output's extents have to be the ones these strides describe
+          for (int64_t e = 0; e < (d == axis ? q : 1); ++e, ++k) {
+            if (oshape[static_cast<size_t>(k)] != (d == axis ? qshape[static_cast<size_t>(e)] : ishape[static_cast<size_t>(d)])) return std::nullopt;
+          }
+        }
+        offset += base * st[static_cast<size_t>(axis)];
+        break;
+      }
       case OpKind::Reshape:
       case OpKind::Flatten: {
         ViewTracker tracker(ishape);
@@ -462,49 +511,54 @@ class Scheduler {
       if (l.group.empty()) writes.push_back({pos, l.out, &l, 0});
       for (const Launch &g : l.group) writes.push_back({pos, g.out, &l, 0});
     }
-    for (size_t i = 0; i < steps_.size(); ++i) {
-      if (taken_[i] || !Elidable(steps_[i].out) || !steps_[i].node->IsSingleInput()) continue;
-      const auto view = AsView(i);
-      if (!view) continue;
+    std::vector<const Launch *> dissolved;  // copy launches both of whose steps became views
+    auto is_dissolved = [&](const Launch *l) { return std::find(dissolved.begin(), dissolved.end(), l) != dissolved.end(); };
+
+    // `seen` = the output of view step(s) starting at position `first`, described inside the source tensor.  Can
+    // every reader of `produced` read the source instead?  `skip`: a copy launch that would no longer run.
+    auto readers_can_see = [&](size_t first, const Operand &produced, const Operand &seen, const Launch *skip) {
+      auto it = readers_.find(produced.name);
+      if (it == readers_.end() || it->second.empty()) return false;
+      for (size_t r : it->second) {
+        if (r <= first) return false;
+        const size_t pos = issued[r];
+        if (pos < first) return false;  // the reader was hoisted in front of the view step: keep the copy
+        for (const Write &w : writes) {
+          // nothing may write the source's bytes after the view step and before the reader runs, and the
+          // reader's own launch must not write what it now reads through the view
+          if (w.launch != nullptr && (w.launch == skip || is_dissolved(w.launch))) continue;
+          const bool own = w.launch != nullptr ? w.launch == owner[r] : (owner[r] == nullptr && w.step == r);
+          if (w.launch == nullptr && elided_[w.step]) continue;
+          if (((w.position > first && w.position < pos) || own) && Alias(w.what, seen)) return false;
+        }
+        for (size_t q = first + 1; q < pos; ++q) {
+          // scratch reserved by a step in between (these kernels do not touch it, but it is not ours to read under)
+          const Step &between = steps_[q];
+          if (between.has_buffer && seen.space == Operand::Space::Arena && between.buffer_offset < seen.offset + seen.Extent() &&
+              seen.offset < between.buffer_offset + between.buffer_bytes) {
+            return false;
+          }
+        }
+      }
+      return true;
+    };
+    // step i's output (meta of the step's own output) as the operand its readers would use instead
+    auto seen_through = [&](size_t i, const std::pair<int64_t, std::vector<int64_t>> &view) {
       const Step &s = steps_[i];
-      auto it = readers_.find(s.out.name);
-      if (it == readers_.end() || it->second.empty()) continue;
-      // the source operand: the step's input, or what that input is itself a view of
       Operand seen = s.out;  // keeps the view's meta (shape, type)
       seen.space = s.in0.space;
       seen.name = s.in0.name;
       seen.offset = s.in0.offset;
       seen.viewed = true;
-      seen.view_offset = view->first;
-      seen.view_strides = view->second;
+      seen.view_offset = view.first;
+      seen.view_strides = view.second;
       seen.source_bytes = s.in0.Extent();
-      bool ok = true;
-      for (size_t r : it->second) {
-        if (r <= i) ok = false;
-        const size_t pos = issued[r];
-        if (pos < i) ok = false;  // the reader was hoisted in front of the view step: keep the copy
-        for (const Write &w : writes) {
-          // nothing may write the source's bytes after the view step and before the reader runs, and the
-          // reader's own launch must not write what it now reads through the view
-          const bool own = w.launch != nullptr ? w.launch == owner[r] : (owner[r] == nullptr && w.step == r);
-          if (w.launch == nullptr && elided_[w.step]) continue;
-          if (((w.position > i && w.position < pos) || own) && Alias(w.what, seen)) ok = false;
-        }
-        for (size_t q = i + 1; q < pos && ok; ++q) {
-          // scratch reserved by a step in between (these kernels do not touch it, but it is not ours to read under)
-          const Step &between = steps_[q];
-          if (between.has_buffer && seen.space == Operand::Space::Arena && between.buffer_offset < seen.offset + seen.Extent() &&
-              seen.offset < between.buffer_offset + between.buffer_bytes) {
-            ok = false;
-          }
-        }
-        if (!ok) break;
-      }
-      if (!ok) continue;
-      // rewrite every reader: the plan's steps (for later views of this view and for single-step launches) and
-      // the operand copies inside fused launches
-      const Operand produced = s.out;
-      for (size_t r : it->second) {
+      return seen;
+    };
+    // rewrite every reader of `produced`: the plan's steps (for later views of this view and for single-step
+    // launches) and the operand copies inside fused launches
+    auto rewire = [&](const Operand &produced, const Operand &seen) {
+      for (size_t r : readers_.at(produced.name)) {
         if (SameTensor(steps_[r].in0, produced)) steps_[r].in0 = seen;
         if (steps_[r].node->IsDoubleInputs() && SameTensor(steps_[r].in1, produced)) steps_[r].in1 = seen;
         rewired_[r] = true;
@@ -519,11 +573,62 @@ class Scheduler {
           }
         }
       }
+    };
+
+    for (size_t i = 0; i < steps_.size(); ++i) {
+      if (!steps_[i].node->IsSingleInput()) continue;
+      if (taken_[i]) {
+        // A Reshape + Transpose (or Transpose + Reshape) pair fused into one strided copy: if the two steps in a
+        // row are still one strided view of the source, and the source's bytes last until the readers run, the
+        // copy does not have to run either.
+        const Launch *l = owner[i];
+        if (l == nullptr || is_dissolved(l) || l->members.size() != 2 || l->members[0] != i ||
+            (l->kind != Launch::Kind::ReshapeTranspose && l->kind != Launch::Kind::TransposeReshape)) {
+          continue;
+        }
+        const size_t j = l->members[1];
+        if (!Elidable(steps_[i].out) || !Elidable(steps_[j].out) || !steps_[j].node->IsSingleInput()) continue;
+        const auto first_view = AsView(i);
+        if (!first_view) continue;
+        const Operand seen_first = seen_through(i, *first_view);
+        const Operand saved = steps_[j].in0;
+        steps_[j].in0 = seen_first;
+        const auto second_view = AsView(j);
+        if (!second_view) {
+          steps_[j].in0 = saved;
+          continue;
+        }
+        Operand seen = seen_through(j, *second_view);
+        seen.source_bytes = seen_first.source_bytes;
+        const Operand produced = steps_[j].out;
+        if (!readers_can_see(i, produced, seen, l)) {
+          steps_[j].in0 = saved;
+          continue;
+        }
+        rewire(produced, seen);
+        steps_[i].out = seen_first;
+        steps_[j].out = seen;
+        elided_[i] = elided_[j] = true;
+        dissolved.push_back(l);
+        owner[i] = owner[j] = nullptr;
+        issued[i] = i;
+        issued[j] = j;
+        BuildReaders();
+        continue;
+      }
+      if (!Elidable(steps_[i].out)) continue;
+      const auto view = AsView(i);
+      if (!view) continue;
+      const Operand seen = seen_through(i, *view);
+      const Operand produced = steps_[i].out;
+      if (!readers_can_see(i, produced, seen, nullptr)) continue;
+      rewire(produced, seen);
       steps_[i].out = seen;
       elided_[i] = true;
       taken_[i] = true;
       BuildReaders();  // names changed: the source gained this step's readers
     }
+    fused->erase(std::remove_if(fused->begin(), fused->end(), [&](const Launch &l) { return is_dissolved(&l); }), fused->end());
   }
 
   // ---- Concat2 inputs written in place ---------------------------------------------------------------------

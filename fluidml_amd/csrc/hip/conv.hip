@@ -121,6 +121,10 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
                      const int64_t *pads, const int64_t *strides, const int64_t *dilations,
                      const fl_ew_program *chain, bool bf16, void *stream);
 
+int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
+                const int64_t *pads, const int64_t *strides, const int64_t *dilations, const fl_ew_program *chain,
+                void *stream);  // conv_halo.hip
+
 namespace {
 
 int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
@@ -187,6 +191,11 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
     }
   }
   // dense contractions go to the matrix cores; depthwise, 3-d and literal-reference modes stay here
+  if (!depthwise && flags == 0 && ns == 2 && !bf16) {
+    // 3x3, unit stride: the input patch is staged once per workgroup instead of gathered tap by tap
+    const int rc = ConvHalo3x3(in, weights, bias, out, pads, strides, dilations, chain, stream);
+    if (rc != FL_ERR_UNSUPPORTED) return rc;
+  }
   if (!depthwise && flags == 0 && ns <= 2) {
     const int rc = ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, chain, bf16, stream);
     if (rc != FL_ERR_UNSUPPORTED) return rc;

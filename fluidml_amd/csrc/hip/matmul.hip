@@ -790,6 +790,8 @@ inline bool TrySkinnyGemm(const MatmulArgs &p, int64_t n_batch, float *C, const 
     // takes 24.7 us with two columns, 27.8 us with eight)
     int rows = p.K >= 8192 ? std::max(mt, 2) : 2;
     while (rows > 1 && p.N / rows < 512) rows /= 2;
+    // (sixteen columns per workgroup at M = 8 -- half the re-reads of A -- were measured slower: 106 against 90.5 us for
+    // [8,25088] x [4096,25088]^T; with 128 accumulators only four waves per compute unit stream weights)
 #define FL_SKINNY_BLOCK(MT_, ROWS_)                                                                              \
   FL_LAUNCH((SkinnyGemmBlockKernel<MT_, ROWS_, (MT_ * ROWS_ <= 8 ? 2 : 1)>), dim3((p.N + ROWS_ - 1) / ROWS_), dim3(256), 0, \
             s, C, A, B, p)

@@ -284,11 +284,19 @@ __global__ __launch_bounds__(kBlock) void LayerNormRowBlock(RowArgs<6> a, float 
   const float n = static_cast<float>(a.len);
   float x[ITEMS];
   float s = 0.0f;
+  // scale and bias are requested together with the row: asked for after the two reductions they would be one more
+  // memory round trip at the end of a kernel that is nothing but a chain of round trips
+  const float *g = scale + off[2];
+  const float *b = bias + off[3];
+  const int32_t sg = a.axis_stride[2], sb = a.axis_stride[3];
+  float gv[ITEMS], bv[ITEMS];
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t j = threadIdx.x + i * kBlock;
     x[i] = j < a.len ? src[j] : 0.0f;
     if (addend != nullptr && j < a.len) x[i] = x[i] + addend[off[5] + static_cast<int32_t>(j) * a.axis_stride[5]];
+    gv[i] = j < a.len ? g[static_cast<int32_t>(j) * sg] : 0.0f;
+    bv[i] = j < a.len ? b[static_cast<int32_t>(j) * sb] : 0.0f;
     s += x[i];
   }
   s = BlockReduce<kBlock / kWave>(s, SumOp{}, smem);
@@ -304,16 +312,10 @@ __global__ __launch_bounds__(kBlock) void LayerNormRowBlock(RowArgs<6> a, float 
   v = BlockReduce<kBlock / kWave>(v, SumOp{}, smem);
   const float inv = 1.0f / sqrtf(v / n + eps);
   float *dst = out + off[0];
-  const float *g = scale + off[2];
-  const float *b = bias + off[3];
-  const int32_t sg = a.axis_stride[2], sb = a.axis_stride[3];
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t j = threadIdx.x + i * kBlock;
-    if (j < a.len) {
-      StoreMaybeStreaming(dst + j, (x[i] * inv) * g[static_cast<int32_t>(j) * sg] + b[static_cast<int32_t>(j) * sb],
-                          a.streaming != 0);
-    }
+    if (j < a.len) StoreMaybeStreaming(dst + j, (x[i] * inv) * gv[i] + bv[i], a.streaming != 0);
   }
 }
 

@@ -8,11 +8,14 @@ batch 8) is compiled from its ONNX file and run three ways on the same seeded we
 * the one-launch-per-node schedule (FLUIDML_FUSE=0) of the same plan.
 
 Both GPU schedules have to meet the oracle within the tolerance the configurations are specified with
-(rel 1e-4 / abs 1e-5, fp32), element by element.  An element outside it passes only if the GPU value is within
-the same tolerance of the float64 evaluation of the network (tests/torch_reference.py, pinned against the oracle
-on small instances by tests/test_oracle_graphs.py): the oracle adds the products of each dot product one after
-the other in fp32 like the reference's loop nests, and over the 4,608 to 25,088 terms of VGG-16's late layers
-that rounding alone exceeds the tolerance on a few logits whose terms cancel (the test prints how many).  For VGG-16 at batch 8 the oracle runs the batch-1 graph (same seed, hence the
+(rel 1e-4 / abs 1e-5, fp32), element by element.  For an element outside it the float64 evaluation of the
+network (tests/torch_reference.py, pinned against the oracle on small instances by tests/test_oracle_graphs.py)
+decides whose rounding the difference is: the element passes if the GPU value is within the same tolerance of the
+float64 value, or no farther from it than the oracle's own worst element of that output.  The oracle adds the
+products of each dot product one after the other in fp32 like the reference's loop nests, and over the 4,608 to
+25,088 terms of VGG-16's late layers that rounding alone exceeds the tolerance on a few logits whose terms cancel
+(the test prints the counts: about 10 of 1000 oracle logits are outside the tolerance of the float64 value, with
+errors up to 4e-5, against 2e-5 for the GPU).  For VGG-16 at batch 8 the oracle runs the batch-1 graph (same seed, hence the
 same weights; tests/test_oracle_graphs.py checks that rows of a batch are independent images) on images 0
 and 7.  A BERT-base case with the layouts of the DP executor (constant costs: every tensor stored with its
 dimensions reversed) runs the same comparison on non-identity strides at real extents.

@@ -1237,6 +1237,35 @@ def test_conv_large_tiles(device):
             assert_close(do.logical(), ho.logical(), what="conv large")
 
 
+def test_conv_staged_patch(device):
+    """3x3 unit-stride convolutions that take the kernel with the input patch staged in LDS: one and two pixel tiles per
+    wave, image extents that leave the last tiles ragged, a filter count that leaves the last filter tile half empty,
+    no padding, channels-last output, bias and a ReLU chain."""
+    cabi = _cabi()
+    rng = np.random.default_rng(83)
+    relu = cabi.make_chain([(cabi.EW_RELU, 0)])
+    for xshape, filters, pads, lo, with_chain in [((8, 8, 96, 150), 96, [1, 1, 1, 1], None, True),     # two tiles per wave
+                                                  ((3, 16, 30, 62), 160, [1, 1, 1, 1], [0, 3, 1, 2], False),  # ragged rows
+                                                  ((2, 8, 66, 66), 128, [0, 0, 0, 0], None, True)]:    # no padding
+        wshape = (filters, xshape[1], 3, 3)
+        x, w, bias = rand(rng, xshape, -1, 1), rand(rng, wshape, -0.1, 0.1), rand(rng, (filters,), -1, 1)
+        oh, ow = xshape[2] + 2 * pads[0] - 2, xshape[3] + 2 * pads[1] - 2
+        oshape = (xshape[0], filters, oh, ow)
+        announce("conv staged patch", xshape, wshape, pads, lo)
+        hx, hw, hb, ho = ok.View(x), ok.View(w), ok.View(bias), ok.View.empty(oshape, np.float32, lo)
+        ok.conv(hx, hw, hb, ho, pads if any(pads) else None, [1, 1], [1, 1], 1, 0)
+        want = ho
+        if with_chain:
+            want = ok.View.empty(oshape, np.float32, lo)
+            ok.unary_f32(ok.OP_RELU, ho, want)
+        dx, dw, db = DeviceView(hx, device), DeviceView(hw, device), DeviceView(hb, device)
+        do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
+        none = cabi.make_chain([])
+        cabi.call("conv_chain", dx.ref(), dw.ref(), db.ref(), do.ref(), cabi.i64_array(pads), cabi.i64_array([1, 1]),
+                  cabi.i64_array([1, 1]), ctypes.c_int64(1), ctypes.byref(relu if with_chain else none), ctypes.c_uint32(0), None)
+        assert_close(do.logical(), want.logical(), what="conv with staged patch")
+
+
 def test_argument_errors(device):
     """Rejected arguments return negative codes and launch nothing."""
     cabi = _cabi()

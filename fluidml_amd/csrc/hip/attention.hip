@@ -55,9 +55,13 @@ __global__ __launch_bounds__(256) void AttentionKernel(AttentionArgs a, float *_
   __shared__ __attribute__((aligned(16))) float ps[kQ * kLdP];
   __shared__ float row_sum[kQ];
 
-  const uint32_t qb = blockIdx.x % a.q_blocks;
+  // Workgroup ids go round the 8 XCDs; renumbered so that each XCD takes a contiguous run of (head, query block)
+  // pairs, a head's K and V are fetched by one or two of the L2s instead of all eight.
+  uint32_t bid = blockIdx.x;
+  if (gridDim.x % 8 == 0) bid = (bid % 8) * (gridDim.x / 8) + bid / 8;
+  const uint32_t qb = bid % a.q_blocks;
   int32_t off[6] = {0, 0, 0, 0, 0, 0};
-  a.batch.AddOffsets(blockIdx.x / a.q_blocks, off);
+  a.batch.AddOffsets(bid / a.q_blocks, off);
   const int m0 = static_cast<int>(qb) * kQ;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, l16 = lane % 16, grp = lane / 16;
 

@@ -781,6 +781,13 @@ __global__ __launch_bounds__(256) void SkinnyGemmBlockKernel(float *__restrict__
 // Launches the skinny kernel if the problem fits it; false = use the tiled kernel.
 inline bool TrySkinnyGemm(const MatmulArgs &p, int64_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   if (n_batch != 1 || p.M > 8 || p.N < 256 || p.K < 256 || p.n_inner != 0 || p.n_groups > 1) return false;
+  // Five to eight rows against many long weight rows: every lane of the kernels below loads M values of A per
+  // weight value, and from five rows on those cache reads, not HBM, set the pace; the tiled kernel shares A through
+  // LDS and splits K over workgroups ([8,25088] x [4096,25088]^T: 78.7 against 89.8 us, [8,4096] x [4096,4096]^T:
+  // 17.3 against 21.6; with fewer weight rows or a shorter K it has too few tiles: [8,4096] x [1000,4096]^T 11.3
+  // against 8.8 us).  A 16x16x4 MFMA formulation of the streaming kernel (16 weight rows per wave, both operands
+  // loaded 128 bits along k) was measured as well: 91 us at eight rows.
+  if (p.M >= 5 && p.N >= 2048 && p.K >= 2048) return false;
   if (p.sBk != 1 || p.sAk != 1 || p.K % 4 != 0 || p.sBn % 4 != 0 || (p.M > 1 && p.sAm % 4 != 0)) return false;
   if (!IsAligned(A, 16) || !IsAligned(B, 16)) return false;
   if (p.K >= 2048) {

@@ -29,6 +29,7 @@ FL_REF_GATHER_RAW_AXIS = 1 << 4
 FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
 FL_CONTRACT_BF16 = 1 << 0
 FL_CONTRACT_SHIFT = 16
+FL_ERR_UNSUPPORTED = -8
 FL_ERR_STATIC_SCRATCH = -9
 FL_NO_ALLOC_SCRATCH_BYTES = 2 << 20
 
@@ -156,6 +157,7 @@ SIGNATURES = {
     "fluidml_hip_matmul_chain_group": [_i32, _T, _vp, _vp, _vp, _i64, _i64p, _vp, _u32, _vp],
     "fluidml_hip_gemm_chain": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _vp, _u32, _vp],
     "fluidml_hip_conv_chain": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _u32, _vp],
+    "fluidml_hip_conv_chain_scale_add": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _T, _T, _u32, _vp],
     "fluidml_hip_pointwise_conv_pair": [_T, _T, _T, _vp, _T, _T, _vp, _T, _vp],
     "fluidml_hip_softmax_matvec": [_T, _T, _T, _vp],
     "fluidml_hip_elementwise_chain": [_T, _T, _vp, _vp],

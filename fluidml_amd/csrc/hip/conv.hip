@@ -119,7 +119,7 @@ __global__ __launch_bounds__(kBlock) void ConvDirect(ConvArgs p, float *__restri
 // matmul.hip
 int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
                      const int64_t *pads, const int64_t *strides, const int64_t *dilations,
-                     const fl_ew_program *chain, bool bf16, void *stream);
+                     const fl_ew_program *chain, bool bf16, void *stream, const ConvExtras *extras);
 
 int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
                 const int64_t *pads, const int64_t *strides, const int64_t *dilations, const fl_ew_program *chain,
@@ -129,7 +129,8 @@ namespace {
 
 int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
          const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, uint32_t flags,
-         void *stream, const fl_ew_program *chain = nullptr) {
+         void *stream, const fl_ew_program *chain = nullptr, const ConvExtras *extras = nullptr) {
+  if (extras != nullptr && extras->channel_scale == nullptr && extras->addend == nullptr) extras = nullptr;
   FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(in));
   FL_CHECK(CheckView(weights));
@@ -191,13 +192,18 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
     }
   }
   // dense contractions go to the matrix cores; depthwise, 3-d and literal-reference modes stay here
+  if (extras != nullptr) {
+    // the extra operands exist in the matrix-core path only
+    if (depthwise || flags != 0 || ns > 2) return FL_ERR_UNSUPPORTED;
+    return ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, chain, bf16, stream, extras);
+  }
   if (!depthwise && flags == 0 && ns == 2 && !bf16) {
     // 3x3, unit stride: the input patch is staged once per workgroup instead of gathered tap by tap
     const int rc = ConvHalo3x3(in, weights, bias, out, pads, strides, dilations, chain, stream);
     if (rc != FL_ERR_UNSUPPORTED) return rc;
   }
   if (!depthwise && flags == 0 && ns <= 2) {
-    const int rc = ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, chain, bf16, stream);
+    const int rc = ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, chain, bf16, stream, nullptr);
     if (rc != FL_ERR_UNSUPPORTED) return rc;
   }
   LoopNest nest;
@@ -247,9 +253,9 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
 // hidden[s] = chain1(sum_c w1[s][c] * in[c] + b1[s]);  out[f] = chain2(sum_s w2[f][s] * hidden[s] + b2[f]).
 // A workgroup of 16 waves owns 1024 outputs f of one image and recomputes the whole hidden vector (a few thousand
 // multiply-adds).  Everything here is a chain of dependent round trips to memory, so each phase issues all its
-// loads before it uses any: the input goes to LDS; wave w takes hidden channels w, w + 16, .. two at a time, its
+// loads before it uses any: the input goes to LDS; wave w takes hidden channels w, w + 16, .. ROWS at a time, its
 // lanes holding up to QUADS 128-bit pieces of each weight row (wave64 shuffle sum); then one lane per output walks
-// its weight row sixteen values at a time against the hidden vector in LDS.
+// its weight row (up to 48 values of it requested ahead) against the hidden vector in LDS.
 constexpr int kPairBlock = 1024;
 constexpr int kPairMaxChannels = 4096, kPairMaxHidden = 512;
 
@@ -266,7 +272,7 @@ struct alignas(16) PairQuad {
   float v[4];
 };
 
-template <int QUADS>
+template <int QUADS, int ROWS>
 __global__ __launch_bounds__(kPairBlock) void ConvPairKernel(ConvPairArgs p, float *__restrict__ out,
                                                              const float *__restrict__ in,
                                                              const float *__restrict__ w1, const float *__restrict__ b1,
@@ -274,80 +280,92 @@ __global__ __launch_bounds__(kPairBlock) void ConvPairKernel(ConvPairArgs p, flo
   __shared__ __align__(16) float x[kPairMaxChannels];
   __shared__ __align__(16) float hidden[kPairMaxHidden];
   constexpr int kWaves = kPairBlock / kWave;
+  // 128-bit pieces of an output's weight row requested before the hidden vector is known (fewer where the rows of
+  // the first phase leave fewer registers)
+  constexpr int kAhead = ROWS * QUADS > 8 ? 8 : 12;
   const int image = blockIdx.y;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int f = blockIdx.x * kPairBlock + threadIdx.x;
   const bool live = f < p.outputs;
   const float *row2 = w2 + static_cast<int64_t>(live ? f : 0) * p.w2_f;
   const int n_quads = p.channels / 4, hidden_quads = p.hidden / 4;
-  // the first loads of both phases do not depend on anything computed here: they are issued before the input
-  // is staged, so that the common case (at most 32 channels in between) waits for memory once
-  PairQuad a0[QUADS], a1[QUADS], wq[4];
-  float ws[16];
+  // Every round trip to memory counts here (the weights are cold: nothing has read them since the last
+  // inference), so the loads of both phases are requested as early as their registers allow: a wave's ROWS rows
+  // of the first weight matrix and the first four pieces of the output's row before the input is staged, the
+  // next eight pieces as soon as the first phase's products are done.
+  PairQuad a[ROWS][QUADS], wq[kAhead];  // (wq[0..3] double as the sixteen scalars of a row that cannot be read 128 bits at a time)
   auto load_rows = [&](int s0) {
-    const int s1 = s0 + kWaves < p.hidden ? s0 + kWaves : s0;
-    const PairQuad *row0 = reinterpret_cast<const PairQuad *>(w1 + static_cast<int64_t>(s0) * p.w1_s);
-    const PairQuad *row1 = reinterpret_cast<const PairQuad *>(w1 + static_cast<int64_t>(s1) * p.w1_s);
 #pragma unroll
-    for (int k = 0; k < QUADS; ++k) {
-      const int q = lane + k * kWave;
-      a0[k] = q < n_quads ? row0[q] : PairQuad{{0, 0, 0, 0}};
-      a1[k] = q < n_quads ? row1[q] : PairQuad{{0, 0, 0, 0}};
+    for (int r = 0; r < ROWS; ++r) {
+      const int s = s0 + r * kWaves < p.hidden ? s0 + r * kWaves : s0;
+      const PairQuad *row = reinterpret_cast<const PairQuad *>(w1 + static_cast<int64_t>(s) * p.w1_s);
+#pragma unroll
+      for (int k = 0; k < QUADS; ++k) {
+        const int q = lane + k * kWave;
+        a[r][k] = q < n_quads ? row[q] : PairQuad{{0, 0, 0, 0}};
+      }
     }
   };
-  auto load_quads = [&](int q0) {
+  auto load_quads = [&](int q0, int k0, int k1) {  // pieces q0 + k0 .. q0 + k1 - 1 into wq[k0 .. k1 - 1]
 #pragma unroll
-    for (int k = 0; k < 4; ++k) wq[k] = q0 + k < hidden_quads ? reinterpret_cast<const PairQuad *>(row2)[q0 + k] : PairQuad{{0, 0, 0, 0}};
+    for (int k = 0; k < kAhead; ++k) {
+      if (k >= k0 && k < k1) wq[k] = q0 + k < hidden_quads ? reinterpret_cast<const PairQuad *>(row2)[q0 + k] : PairQuad{{0, 0, 0, 0}};
+    }
   };
   auto load_scalars = [&](int s0) {
 #pragma unroll
-    for (int k = 0; k < 16; ++k) ws[k] = s0 + k < p.hidden ? row2[(s0 + k) * p.w2_s] : 0.0f;
+    for (int k = 0; k < 16; ++k) wq[k / 4].v[k % 4] = s0 + k < p.hidden ? row2[(s0 + k) * p.w2_s] : 0.0f;
   };
   if (p.vec1 && wave < p.hidden) load_rows(wave);
   if (live) {
-    if (p.vec2) load_quads(0);
+    if (p.vec2) load_quads(0, 0, 4);
     else load_scalars(0);
   }
   // the biases too: a load issued only after the sums are known would be one more trip to memory each
-  float bias_first0 = 0.0f, bias_first1 = 0.0f, bias_out = 0.0f;
-  if (b1 != nullptr && wave < p.hidden) {
-    bias_first0 = b1[wave * p.b1_stride];
-    if (wave + kWaves < p.hidden) bias_first1 = b1[(wave + kWaves) * p.b1_stride];
+  float bias_first[ROWS], bias_out = 0.0f;
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    bias_first[r] = b1 != nullptr && wave + r * kWaves < p.hidden ? b1[(wave + r * kWaves) * p.b1_stride] : 0.0f;
   }
   if (b2 != nullptr && live) bias_out = b2[f * p.b2_stride];
   const float *src = in + static_cast<int64_t>(image) * p.in_n;
   for (int c = threadIdx.x; c < p.channels; c += kPairBlock) x[c] = src[c * p.in_c];
   __syncthreads();
   if (p.vec1) {
-    for (int s0 = wave; s0 < p.hidden; s0 += 2 * kWaves) {
-      const int s1 = s0 + kWaves;
-      const bool second = s1 < p.hidden;
+    for (int s0 = wave; s0 < p.hidden; s0 += ROWS * kWaves) {
       if (s0 != wave) load_rows(s0);
-      float acc0 = 0.0f, acc1 = 0.0f;
+      float acc[ROWS];
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) acc[r] = 0.0f;
 #pragma unroll
       for (int k = 0; k < QUADS; ++k) {
         const int q = lane + k * kWave;
         if (q < n_quads) {
           const PairQuad xv = reinterpret_cast<const PairQuad *>(x)[q];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            acc0 += a0[k].v[e] * xv.v[e];
-            acc1 += a1[k].v[e] * xv.v[e];
+          for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[r] += a[r][k].v[e] * xv.v[e];
+        }
+      }
+      if (s0 == wave && p.vec2 && live) load_quads(0, 4, kAhead);
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) acc[r] = WaveReduce(acc[r], SumOp{});
+      if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+          const int s = s0 + r * kWaves;
+          if (s < p.hidden) {
+            float v = acc[r];
+            if (b1 != nullptr) v += s0 == wave ? bias_first[r] : b1[s * p.b1_stride];
+            hidden[s] = p.chain1.n != 0 ? RunChain(p.chain1, v) : v;
           }
         }
       }
-      acc0 = WaveReduce(acc0, SumOp{});
-      acc1 = WaveReduce(acc1, SumOp{});
-      if (lane == 0) {
-        if (b1 != nullptr) acc0 += s0 == wave ? bias_first0 : b1[s0 * p.b1_stride];
-        hidden[s0] = p.chain1.n != 0 ? RunChain(p.chain1, acc0) : acc0;
-        if (second) {
-          if (b1 != nullptr) acc1 += s0 == wave ? bias_first1 : b1[s1 * p.b1_stride];
-          hidden[s1] = p.chain1.n != 0 ? RunChain(p.chain1, acc1) : acc1;
-        }
-      }
     }
+    if (wave >= p.hidden && p.vec2 && live) load_quads(0, 4, kAhead);  // waves without a row of the first phase
   } else {
+    if (p.vec2 && live) load_quads(0, 4, kAhead);
     for (int s = wave; s < p.hidden; s += kWaves) {
       const float *row = w1 + static_cast<int64_t>(s) * p.w1_s;
       float acc = 0.0f;
@@ -364,10 +382,10 @@ __global__ __launch_bounds__(kPairBlock) void ConvPairKernel(ConvPairArgs p, flo
   if (!live) return;
   float acc = 0.0f;
   if (p.vec2) {
-    for (int q0 = 0; q0 < hidden_quads; q0 += 4) {
-      if (q0 != 0) load_quads(q0);
+    for (int q0 = 0; q0 < hidden_quads; q0 += kAhead) {
+      if (q0 != 0) load_quads(q0, 0, kAhead);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
+      for (int k = 0; k < kAhead; ++k) {
         if (q0 + k < hidden_quads) {
           const PairQuad h = reinterpret_cast<const PairQuad *>(hidden)[q0 + k];
 #pragma unroll
@@ -380,7 +398,7 @@ __global__ __launch_bounds__(kPairBlock) void ConvPairKernel(ConvPairArgs p, flo
       if (s0 != 0) load_scalars(s0);
 #pragma unroll
       for (int k = 0; k < 16; ++k) {
-        if (s0 + k < p.hidden) acc += ws[k] * hidden[s0 + k];
+        if (s0 + k < p.hidden) acc += wq[k / 4].v[k % 4] * hidden[s0 + k];
       }
     }
   }
@@ -440,20 +458,32 @@ int ConvPair(const fl_tensor *in, const fl_tensor *w1, const fl_tensor *b1, cons
   p.vec1 = c % 4 == 0 && p.w1_c == 1 && p.w1_s % 4 == 0 && IsAligned(w1->base, 16) ? 1 : 0;
   p.vec2 = s % 4 == 0 && p.w2_s == 1 && p.w2_f % 4 == 0 && IsAligned(w2->base, 16) ? 1 : 0;
   const dim3 grid(static_cast<uint32_t>((f + kPairBlock - 1) / kPairBlock), static_cast<uint32_t>(n));
-#define FL_CONV_PAIR(QUADS)                                                                                        \
-  FL_LAUNCH(ConvPairKernel<QUADS>, grid, dim3(kPairBlock), 0, AsStream(stream), p, static_cast<float *>(out->base), \
+#define FL_CONV_PAIR(QUADS, ROWS)                                                                                  \
+  FL_LAUNCH((ConvPairKernel<QUADS, ROWS>), grid, dim3(kPairBlock), 0, AsStream(stream), p, static_cast<float *>(out->base), \
             static_cast<const float *>(in->base), static_cast<const float *>(w1->base),                           \
             b1 ? static_cast<const float *>(b1->base) : nullptr, static_cast<const float *>(w2->base),            \
             b2 ? static_cast<const float *>(b2->base) : nullptr)
-  if (c > 8 * 256) p.vec1 = 0;  // two rows of more than 2048 values do not fit a wave's registers: strided loop
-  if (c <= 4 * 256) {
-    FL_CONV_PAIR(4);
-  } else if (c <= 5 * 256) {
-    FL_CONV_PAIR(5);
-  } else if (c <= 6 * 256) {
-    FL_CONV_PAIR(6);
+  if (c > 8 * 256) p.vec1 = 0;  // rows of more than 2048 values do not fit a wave's registers: strided loop
+  // 128-bit pieces per lane and row, and rows of the first matrix per wave and trip (16 waves share them): all of
+  // them in one trip while the registers last
+  const int rows = s <= 16 ? 1 : s <= 32 ? 2 : 3;
+  if (c <= 256) {
+    if (rows == 1) FL_CONV_PAIR(1, 1);
+    else if (rows == 2) FL_CONV_PAIR(1, 2);
+    else FL_CONV_PAIR(1, 3);
+  } else if (c <= 2 * 256) {
+    if (rows == 1) FL_CONV_PAIR(2, 1);
+    else if (rows == 2) FL_CONV_PAIR(2, 2);
+    else FL_CONV_PAIR(2, 3);
+  } else if (c <= 3 * 256) {
+    if (rows == 1) FL_CONV_PAIR(3, 1);
+    else if (rows == 2) FL_CONV_PAIR(3, 2);
+    else FL_CONV_PAIR(3, 3);
+  } else if (c <= 5 * 256) {  // (three rows of five pieces spill registers and were measured no faster)
+    if (rows == 1) FL_CONV_PAIR(5, 1);
+    else FL_CONV_PAIR(5, 2);
   } else {
-    FL_CONV_PAIR(8);
+    FL_CONV_PAIR(8, 1);
   }
 #undef FL_CONV_PAIR
   return LaunchStatus();
@@ -485,6 +515,18 @@ int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const 
                            const fl_ew_program *chain, uint32_t flags, void *stream) {
   return fl::Conv(in, weights, bias, out, pads, strides, dilations, group, (flags & FL_CONTRACT_BF16) << FL_CONTRACT_SHIFT, stream,
                   chain);
+}
+
+int fluidml_hip_conv_chain_scale_add(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias,
+                                     const fl_tensor *out, const int64_t *pads, const int64_t *strides,
+                                     const int64_t *dilations, int64_t group, const fl_ew_program *chain,
+                                     const fl_tensor *channel_scale, const fl_tensor *addend, uint32_t flags,
+                                     void *stream) {
+  fl::ConvExtras extras;
+  extras.channel_scale = channel_scale;
+  extras.addend = addend;
+  return fl::Conv(in, weights, bias, out, pads, strides, dilations, group, (flags & FL_CONTRACT_BF16) << FL_CONTRACT_SHIFT, stream,
+                  chain, &extras);
 }
 
 int fluidml_hip_pointwise_conv_pair(const fl_tensor *in, const fl_tensor *weights1, const fl_tensor *bias1,

@@ -78,6 +78,15 @@ void DropStreamWorkspace(hipStream_t stream);
 // the first call per device; `ptr` may be null.  matmul.hip
 int StaticScratch(void **ptr);
 
+// Operands a fused convolution launch may carry besides the reference kernel's own (both optional).
+struct ConvExtras {
+  // multiplier of the input, one value per channel ([1, C, 1, ..]: the MulCommon of a squeeze-and-excitation block in
+  // front of a pointwise convolution); each product is rounded like the separate kernel's
+  const fl_tensor *channel_scale = nullptr;
+  // tensor of the output's shape and strides, added after the elementwise chain (a residual AddCommon behind it)
+  const fl_tensor *addend = nullptr;
+};
+
 // Compile-time loop: body(std::integral_constant<int, 0>) ... body(std::integral_constant<int, N - 1>).
 // Unlike `#pragma unroll` it cannot be left rolled, so register arrays indexed by the counter stay in registers.
 template <int N, typename F, int... I>

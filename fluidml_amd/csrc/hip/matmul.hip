@@ -94,6 +94,14 @@ struct MatmulArgs {
   FastDiv div_inner;
   // optional elementwise chain applied after the bias (chain.n == 0: none)
   fl_ew_program chain;
+  // EXTRA instantiations only (plain contraction, B kept [k][n]), both optional:
+  // a tensor with the strides of C, added to the value after the chain (read at the element offset the value is
+  // stored at);
+  const float *addend;
+  // one batch element: row k of B is multiplied by k_scale[k * sKs] while it is staged, each product rounded like
+  // a separate Mul kernel's
+  const float *k_scale;
+  int32_t sKs;
   const float *gB[3];
   float *gC[3];
   const float *gbias[3];
@@ -184,7 +192,7 @@ struct TileLoader {
 // the plain kernel leaves each SIMD idle while its single wave waits for loads, writes LDS or sits at the
 // barrier; here the two roles overlap.
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV = 0,
-          bool BF16 = false, bool SPEC = false>
+          bool BF16 = false, bool SPEC = false, bool EXTRA = false>
 __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(float *__restrict__ C_, const float *__restrict__ A,
                                                                 const float *__restrict__ B_, MatmulArgs p) {
   float *__restrict__ C = C_;
@@ -211,6 +219,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   constexpr int VB = CONV == 2 ? 4 : CONV == 1 ? 1 : VEC;
   static_assert(!CONV || (LB == 0 && NT % (BN / VB) == 0), "the gather keeps one output pixel (group) per thread");
   static_assert(!SPEC || !CONV, "the gather of the convolution runs in the consumer waves");
+  static_assert(!EXTRA || (LB == 0 && CONV == 0), "the extra operands exist for plain contractions with B kept [k][n]");
   const bool producer = SPEC && threadIdx.x >= NT;
   const int ltid = producer ? static_cast<int>(threadIdx.x) - NT : static_cast<int>(threadIdx.x);
   using LoaderA = typename std::conditional<LA == 0, TileLoader<BM, BK, VEC, NT>, TileLoader<BK, BM, VEC, NT>>::type;
@@ -307,6 +316,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   static_assert(DEPTH % 2 == 0, "the LDS buffer index must be a compile-time function of the stage");
   VecF<VEC> ra[DEPTH][LoaderA::kPerThread];
   VecF<VB> rb[DEPTH][LoaderB::kPerThread];
+  float rs[DEPTH][LoaderB::kPerThread];  // EXTRA: the scale of the row each item of the B tile belongs to
   const int rows_m = p.M - m0, cols_n = p.N - n0;
   const int n_chunks = (p.K + BK - 1) / BK;
 
@@ -324,8 +334,18 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
     g_base = static_cast<int32_t>(img) * p.conv.sXn;
   }
 
-  auto load_chunk = [&](int c, VecF<VEC>(&qa)[LoaderA::kPerThread], VecF<VB>(&qb)[LoaderB::kPerThread]) {
+  auto load_chunk = [&](int c, VecF<VEC>(&qa)[LoaderA::kPerThread], VecF<VB>(&qb)[LoaderB::kPerThread],
+                        float(&qs)[LoaderB::kPerThread]) {
     const int k0 = c * BK, k_valid = p.K - k0;
+    if constexpr (EXTRA) {
+      if (p.k_scale != nullptr) {
+#pragma unroll
+        for (int j = 0; j < LoaderB::kPerThread; ++j) {
+          const int k = k0 + (ltid + j * NT) / LoaderB::kVecsPerRow;
+          qs[j] = k < p.K ? p.k_scale[static_cast<int64_t>(k) * p.sKs] : 0.0f;
+        }
+      }
+    }
     if constexpr (LA == 0) {
       LoaderA::Load(Ab + static_cast<int64_t>(k0) * p.sAk, p.sAm, p.sAk, rows_m, k_valid, qa, ltid);
     } else {
@@ -373,10 +393,22 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
       LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBn, p.sBk, cols_n, k_valid, qb, ltid);
     }
   };
-  auto store_chunk = [&](int buf, const VecF<VEC>(&qa)[LoaderA::kPerThread], const VecF<VB>(&qb)[LoaderB::kPerThread]) {
+  auto store_chunk = [&](int buf, const VecF<VEC>(&qa)[LoaderA::kPerThread], const VecF<VB>(&qb)[LoaderB::kPerThread],
+                         const float(&qs)[LoaderB::kPerThread]) {
     float *as = lds + buf * (A_ELEMS + B_ELEMS);
     float *bs = as + A_ELEMS;
     LoaderA::Store(as, LDA, qa, ltid);
+    if constexpr (EXTRA) {
+      if (p.k_scale != nullptr) {
+        VecF<VB> scaled[LoaderB::kPerThread];
+#pragma unroll
+        for (int j = 0; j < LoaderB::kPerThread; ++j)
+#pragma unroll
+          for (int e = 0; e < VB; ++e) scaled[j].v[e] = qb[j].v[e] * qs[j];
+        LoaderB::Store(bs, LDB, scaled, ltid);
+        return;
+      }
+    }
     LoaderB::Store(bs, LDB, qb, ltid);
   };
   auto compute_chunk = [&](int buf) {
@@ -447,7 +479,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
     if (producer) {
 #pragma unroll
       for (int s = 0; s < DEPTH; ++s) {
-        if (c_begin + s < c_end) load_chunk(c_begin + s, ra[s], rb[s]);
+        if (c_begin + s < c_end) load_chunk(c_begin + s, ra[s], rb[s], rs[s]);
       }
       for (int c0 = c_begin; c0 < c_end; c0 += DEPTH) {
 #pragma unroll
@@ -455,8 +487,8 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
           const int c = c0 + s;
           if (c < c_end) {  // uniform over the workgroup
             if (c > c_begin) __syncthreads();
-            store_chunk(s & 1, ra[s], rb[s]);
-            if (c + DEPTH < c_end) load_chunk(c + DEPTH, ra[s], rb[s]);
+            store_chunk(s & 1, ra[s], rb[s], rs[s]);
+            if (c + DEPTH < c_end) load_chunk(c + DEPTH, ra[s], rb[s], rs[s]);
           }
         }
       }
@@ -475,15 +507,15 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   } else {
 #pragma unroll
     for (int s = 0; s < DEPTH; ++s) {
-      if (c_begin + s < c_end) load_chunk(c_begin + s, ra[s], rb[s]);
+      if (c_begin + s < c_end) load_chunk(c_begin + s, ra[s], rb[s], rs[s]);
     }
     for (int c0 = c_begin; c0 < c_end; c0 += DEPTH) {
 #pragma unroll
       for (int s = 0; s < DEPTH; ++s) {
         const int c = c0 + s;
         if (c < c_end) {  // uniform over the workgroup
-          store_chunk(s & 1, ra[s], rb[s]);
-          if (c + DEPTH < c_end) load_chunk(c + DEPTH, ra[s], rb[s]);
+          store_chunk(s & 1, ra[s], rb[s], rs[s]);
+          if (c + DEPTH < c_end) load_chunk(c + DEPTH, ra[s], rb[s], rs[s]);
           // one barrier per chunk: buffer (s&1) was last read two chunks ago, and every wave
           // passed the previous barrier only after finishing that read
           __syncthreads();
@@ -623,7 +655,16 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
       // bias, then the elementwise chain on the values of this 32x32 tile the lane holds (all 16, or the 4 of its
       // wave's quarter), then the stores
       auto tile_row = [&](int e) { return QUARTER ? ks * 8 + half * 4 + e : (e / 4) * 8 + half * 4 + (e % 4); };
-      float vals[EV];
+      float vals[EV], add[EV];
+      const float *Eb = nullptr;
+      if constexpr (EXTRA) {
+        Eb = p.addend != nullptr ? p.addend + boff[0] : nullptr;
+#pragma unroll
+        for (int e = 0; e < EV; ++e) {
+          const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
+          add[e] = Eb != nullptr && m < p.M && n < p.N ? Eb[static_cast<int64_t>(m) * sCm + col] : 0.0f;
+        }
+      }
 #pragma unroll
       for (int e = 0; e < EV; ++e) {
         const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
@@ -636,6 +677,12 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
         vals[e] = v;
       }
       if (p.chain.n != 0) RunChainBlock<EV>(p.chain, vals);
+      if constexpr (EXTRA) {
+        if (Eb != nullptr) {
+#pragma unroll
+          for (int e = 0; e < EV; ++e) vals[e] += add[e];
+        }
+      }
 #pragma unroll
       for (int e = 0; e < EV; ++e) {
         const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
@@ -877,7 +924,7 @@ inline int64_t SplitKLimit(int64_t fallback) {
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV, bool BF16,
-          bool SPEC = false>
+          bool SPEC = false, bool EXTRA = false>
 void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   MatmulArgs q = p;
   q.tiles_m = (p.M + BM - 1) / BM;
@@ -921,11 +968,11 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
     }
   }
   q.n_splits = splits;
-  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV, BF16, SPEC>),
+  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV, BF16, SPEC, EXTRA>),
             dim3(q.tiles_m * q.tiles_n, n_batch, splits), dim3(64 * WM * WN * KS * (SPEC ? 2 : 1)), 0, s, C, A, B, q);
 }
 
-template <int LA, int LB, int VEC, int CONV, bool BF16 = false>
+template <int LA, int LB, int VEC, int CONV, bool BF16 = false, bool EXTRA = false>
 void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
   // (A 128x128x16 tile with two chunks in flight was measured slower than the 64x64x32 tile with four at
@@ -935,11 +982,11 @@ void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
              (CONV && tiles_m * std::min<int64_t>({8, p.K / 384, static_cast<int64_t>(kWorkspaceTiles) / (tiles_m * 4)}) >= 192)) {
     // also when splitting K over up to 8 workgroups per tile fills the chip (measured on 3x3 convolutions
     // with 32..104 tiles: 1.5x to 2x over the 32x32 tile)
-    LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4, CONV, BF16>(p, n_batch, C, A, B, s);
+    LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4, CONV, BF16, false, EXTRA>(p, n_batch, C, A, B, s);
   } else {
     // plain contractions run the 32x32 tile with producer and consumer waves (measured on BERT-base: 8.9 -> 8.6,
     // 14.5 -> 13.6 and 15.9 -> 15.0 us for its three shapes); the convolution gather stays in the consumer waves
-    LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2, CONV, BF16, CONV == 0>(p, n_batch, C, A, B, s);
+    LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2, CONV, BF16, CONV == 0, EXTRA>(p, n_batch, C, A, B, s);
   }
 }
 
@@ -954,7 +1001,8 @@ struct Siblings {
 
 int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, bool trans_a, bool trans_b, float ca,
              float cb, const fl_tensor *bias, void *stream, const fl_ew_program *chain = nullptr, int64_t n_inner = 0,
-             int64_t stride_outer = 0, const Siblings *siblings = nullptr, bool bf16 = false) {
+             int64_t stride_outer = 0, const Siblings *siblings = nullptr, bool bf16 = false,
+             const float *addend = nullptr, const float *k_scale = nullptr, int64_t k_scale_stride = 0) {
   FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(lhs));
   FL_CHECK(CheckView(rhs));
@@ -1085,9 +1133,27 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   for (int i = 0; i < nest.rank && vec; ++i) {
     if (nest.strides[1][i] % 4 != 0 || nest.strides[2][i] % 4 != 0) vec = false;
   }
+  // a second addend with the strides of C / a scale per row of B: the tiled kernel's own instantiations (fp32)
+  const bool extra = addend != nullptr || k_scale != nullptr;
+  if (extra) {
+    if (lb != 0 || p.n_groups > 1 || p.n_inner != 0) return FL_ERR_UNSUPPORTED;
+    p.addend = addend;
+  }
+  if (k_scale != nullptr) {
+    if (n_batch != 1 || k_scale_stride > INT32_MAX || k_scale_stride < 0) return FL_ERR_UNSUPPORTED;
+    p.k_scale = k_scale;
+    p.sKs = static_cast<int32_t>(k_scale_stride);
+  }
   // at most 8 rows against k-contiguous weights: HBM-bound weight streaming, fp32 whatever `bf16` says
-  if (TrySkinnyGemm(p, n_batch, C, A, B, s)) return LaunchStatus();
+  if (!extra && TrySkinnyGemm(p, n_batch, C, A, B, s)) return LaunchStatus();
   const uint32_t nb = static_cast<uint32_t>(n_batch);
+  if (extra) {
+    if (la == 0 && vec) LaunchBySize<0, 0, 4, 0, false, true>(p, nb, C, A, B, s);
+    else if (la == 0) LaunchBySize<0, 0, 1, 0, false, true>(p, nb, C, A, B, s);
+    else if (vec) LaunchBySize<1, 0, 4, 0, false, true>(p, nb, C, A, B, s);
+    else LaunchBySize<1, 0, 1, 0, false, true>(p, nb, C, A, B, s);
+    return LaunchStatus();
+  }
 #define FL_MM_DISPATCH(LA_, LB_)                              \
   if (la == LA_ && lb == LB_) {                               \
     if (bf16) {                                                   \
@@ -1114,9 +1180,31 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
 // uses the direct kernel.  `pads` may be null; `strides`/`dilations` have one entry per spatial dim.
 int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
                      const int64_t *pads, const int64_t *strides, const int64_t *dilations,
-                     const fl_ew_program *chain, bool bf16, void *stream) {
+                     const fl_ew_program *chain, bool bf16, void *stream, const ConvExtras *extras) {
   const int ns = out->rank - 2;
   if (ns != 1 && ns != 2) return FL_ERR_UNSUPPORTED;
+  const float *addend = nullptr;
+  if (extras != nullptr && extras->addend != nullptr) {
+    const fl_tensor *e = extras->addend;
+    FL_CHECK(CheckView(e));
+    if (e->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+    if (e->rank != out->rank) return FL_ERR_SHAPE;
+    for (int i = 0; i < out->rank; ++i) {
+      if (e->shape[i] != out->shape[i]) return FL_ERR_SHAPE;
+      if (out->shape[i] > 1 && e->strides[i] != out->strides[i]) return FL_ERR_UNSUPPORTED;
+    }
+    addend = static_cast<const float *>(e->base);
+  }
+  const fl_tensor *scale = extras != nullptr ? extras->channel_scale : nullptr;
+  if (scale != nullptr) {
+    FL_CHECK(CheckView(scale));
+    if (scale->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+    if (scale->rank != in->rank || scale->shape[1] != in->shape[1]) return FL_ERR_SHAPE;
+    for (int i = 0; i < scale->rank; ++i) {
+      if (i != 1 && scale->shape[i] != 1) return FL_ERR_SHAPE;
+    }
+    if (in->shape[0] != 1) return FL_ERR_UNSUPPORTED;  // one scale vector per image: one image per launch
+  }
   const int hd = ns == 2 ? 2 : -1, wd = ns == 2 ? 3 : 2;  // dims of H (absent for 1-d) and W
   const int64_t KH = ns == 2 ? weights->shape[2] : 1, KW = weights->shape[wd];
   const int64_t Cc = in->shape[1], F = out->shape[1];
@@ -1155,9 +1243,11 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
         d.shape[0] = F, d.shape[1] = S, d.strides[0] = bias->strides[0], d.strides[1] = 0;
       }
       return Contract(&a, &b, &c, false, false, 1.0f, 1.0f, bias != nullptr ? &d : nullptr, stream, chain, 0, 0, nullptr,
-                      bf16);
+                      bf16, addend, scale != nullptr ? static_cast<const float *>(scale->base) : nullptr,
+                      scale != nullptr ? scale->strides[1] : 0);
     }
   }
+  if (scale != nullptr || addend != nullptr) return FL_ERR_UNSUPPORTED;  // only the pointwise form carries them
 
   MatmulArgs p;
   std::memset(&p, 0, sizeof(p));

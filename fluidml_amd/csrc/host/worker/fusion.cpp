@@ -951,6 +951,9 @@ class Scheduler {
         limit = taken - 1;
       }
     }
+    if (l.kind == Launch::Kind::ConvChain) {
+      if (auto wider = WithGateAndSkip(i, l)) return wider;
+    }
     // longest variant whose late reads are safe: with the chain, then without it
     for (int attempt = 0; attempt < 2; ++attempt) {
       if (l.members.size() < 2) return std::nullopt;  // nothing fused
@@ -963,6 +966,105 @@ class Scheduler {
       }
       l.members.resize(without_chain);
       l.chain = fl_ew_program{};
+    }
+    return std::nullopt;
+  }
+
+  static bool DefaultLayout(const Operand &o) {
+    if (o.viewed) return false;
+    for (size_t d = 0; d < o.layout.size(); ++d) {
+      if (o.layout[d] != d) return false;
+    }
+    return true;
+  }
+
+  // A convolution `i` (with the chain already matched in `plain`) whose input is a MulCommon of a tensor with one
+  // factor per channel (the gate of a squeeze-and-excitation block) and / or whose result goes into an AddCommon
+  // with a tensor of its own shape (a skip connection): both become operands of the launch.  Only where the launch
+  // is a plain contraction (1x1, unit stride, no padding, default layouts): that kernel scales the rows of its
+  // right operand while staging them (one image) and adds a tensor with the output's strides in its epilogue.
+  std::optional<Launch> WithGateAndSkip(size_t i, const Launch &plain) {
+    const Step &conv = steps_[i];
+    const flow::Attrs &at = Attrs(i);
+    const auto &in_shape = conv.in0.meta.GetShape();
+    bool pointwise = at.group == 1 && in_shape.size() <= 4 && IsFloat(conv.in0) && DefaultLayout(conv.in1) &&
+                     DefaultLayout(conv.out) && (conv.in0.viewed ? false : DefaultLayout(conv.in0));
+    const auto &w_shape = conv.in1.meta.GetShape();
+    for (size_t d = 2; d < w_shape.size() && pointwise; ++d) pointwise = w_shape[d] == 1;
+    for (size_t d = 0; d < at.strides.size() && pointwise; ++d) pointwise = at.strides[d] == 1;
+    if (Kind(i) == OpKind::ConvWithPadding) {
+      for (size_t d = 0; d < at.pads.size() && pointwise; ++d) pointwise = at.pads[d] == 0;
+    }
+    if (!pointwise) return std::nullopt;
+    // the gate
+    std::optional<size_t> mul;
+    Operand x, gate;
+    if (auto it = producer_.find(conv.in0.name); it != producer_.end() && in_shape[0] == 1) {
+      const size_t m = it->second;
+      bool gated = Kind(m) == OpKind::MulCommon && !taken_[m] && m < i;
+      if (gated) {
+        const auto reader = SoleReader(m);
+        gated = reader && *reader == i;
+      }
+      if (gated) {
+        const Step &ms = steps_[m];
+        for (int side = 0; side < 2 && !mul; ++side) {
+          const Operand &full = side == 0 ? ms.in0 : ms.in1, &factor = side == 0 ? ms.in1 : ms.in0;
+          const auto &fs = factor.meta.GetShape();
+          bool ok = IsFloat(full) && IsFloat(factor) && full.meta.GetShape() == in_shape && fs.size() == in_shape.size() &&
+                    fs[1] == in_shape[1] && DefaultLayout(full) && !SameTensor(full, factor);
+          for (size_t d = 0; d < fs.size() && ok; ++d) ok = d == 1 || fs[d] == 1;
+          if (ok) {
+            mul = m;
+            x = full;
+            gate = factor;
+          }
+        }
+      }
+    }
+    // the skip connection
+    std::optional<size_t> add;
+    Operand skip;
+    if (const auto j = SoleReader(plain.members.back()); j && Kind(*j) == OpKind::AddCommon) {
+      const Operand &value = steps_[plain.members.back()].out;
+      const auto other = Other(*j, value);
+      if (other && IsFloat(*other) && !other->viewed && other->meta.GetShape() == value.meta.GetShape() &&
+          steps_[*j].out.meta.GetShape() == value.meta.GetShape() && other->layout == steps_[*j].out.layout &&
+          other->space != Operand::Space::Constant) {
+        add = *j;
+        skip = *other;
+      }
+    }
+    // the widest variant whose late reads are safe
+    for (int variant = 0; variant < 3; ++variant) {
+      const bool with_gate = variant != 2, with_skip = variant != 1;
+      if ((with_gate && !mul) || (with_skip && !add) || (!with_gate && !with_skip)) continue;
+      Launch l = plain;
+      std::vector<std::pair<size_t, Operand>> external = {{i, l.b}};
+      if (with_gate) {
+        l.members.insert(l.members.begin(), *mul);
+        l.a = x;
+        l.c = gate;
+        l.has_gate = true;
+        external.push_back({*mul, x});
+        external.push_back({*mul, gate});
+      } else {
+        external.push_back({i, l.a});
+      }
+      if (with_skip) {
+        l.members.push_back(*add);
+        l.d = skip;
+        l.has_skip = true;
+        external.push_back({*add, skip});
+      }
+      l.out = steps_[l.members.back()].out;
+      if (!Safe(l.members, external) || !OutputDisjoint(l.out, {&l.a, &l.b})) continue;
+      if ((with_gate && Alias(l.out, l.c)) || (with_skip && Alias(l.out, l.d))) continue;
+      l.bytes = Bytes({&l.a, &l.b, &l.out}) + static_cast<double>(steps_[i].kernel->GetConstantBytes());
+      if (with_gate) l.bytes += static_cast<double>(l.c.meta.GetSize());
+      if (with_skip) l.bytes += static_cast<double>(l.d.meta.GetSize());
+      l.flops = Flops(l.members);
+      return l;
     }
     return std::nullopt;
   }

@@ -286,6 +286,16 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       kernel::TensorView c;
       if (bias != nullptr) c = bias->View();
       const bool padded = steps_[l.owner].node->GetKind() == flow::OpKind::ConvWithPadding;
+      if (l.has_gate || l.has_skip) {
+        kernel::TensorView gate, skip;
+        if (l.has_gate) gate = ViewOf(Resolve(l.c), l.c);
+        if (l.has_skip) skip = ViewOf(Resolve(l.d), l.d);
+        rc = fluidml_hip_conv_chain_scale_add(&a.t, &b.t, bias ? &c.t : nullptr, &out.t, padded ? at.pads.data() : nullptr,
+                                              at.strides.data(), at.dilations.data(), at.group, &l.chain,
+                                              l.has_gate ? &gate.t : nullptr, l.has_skip ? &skip.t : nullptr, contract_flags,
+                                              ctx.stream);
+        break;
+      }
       rc = fluidml_hip_conv_chain(&a.t, &b.t, bias ? &c.t : nullptr, &out.t, padded ? at.pads.data() : nullptr,
                                   at.strides.data(), at.dilations.data(), at.group, &l.chain, contract_flags, ctx.stream);
       break;

@@ -65,7 +65,8 @@ struct Launch {
     Step,              // members = {i}
     MatMulChain,       // MatMul [-> AddCommon(rank-1 constant bias)] [-> elementwise chain]
     GemmChain,         // GemmConstantWeightsBias -> elementwise chain
-    ConvChain,         // Conv{With,Without}Padding -> elementwise chain
+    ConvChain,         // [MulCommon(x, factor per channel) ->] Conv{With,Without}Padding -> elementwise chain
+                       // [-> AddCommon(tensor of the output's shape)]
     ConvPair,          // two pointwise convolutions on one-pixel tensors, each with its elementwise chain
                        // (squeeze-and-excitation): a = input, b = weights of `owner`, c = weights of `owner2`,
                        // `chain` follows the first, `chain2` the second
@@ -98,6 +99,9 @@ struct Launch {
   int64_t axis = 0;
   std::vector<int64_t> perm;
   bool has_c = false;     // MatMulChain: a bias operand is present
+  // ConvChain: c = a per-channel factor of the input (the MulCommon in front of the convolution is a member),
+  // d = a tensor of the output's shape added after the chain (the AddCommon behind it is a member)
+  bool has_gate = false, has_skip = false;
   // Attention: a = queries, b = keys (transposed), c = values, d = additive mask (has_mask), the Where step
   // `owner` holds the condition (has_cond) and s1 its fill value; s0 scales the scores, dividing if `divisor`
   bool has_mask = false, has_cond = false, divisor = false;

@@ -377,6 +377,14 @@ int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
 /* Conv{With,Without}PaddingKernel -> elementwise chain (reference conv.cpp:27-280);
  * `pads` may be NULL.  ONNX semantics only (no literal-reference flags); `flags` = fl_contract_flags. */
 int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, const fl_ew_program *chain, uint32_t flags, void *stream);
+/* [MulCommonKernel(x, scale per channel) ->] Conv{With,Without}PaddingKernel -> elementwise chain [-> AddCommonKernel
+ * with a tensor of the output's shape] as ONE launch (reference mul.cpp, conv.cpp:27-280, add.cpp:75-137: the
+ * projection of an inverted-residual block behind its squeeze-and-excitation gate, with the skip connection).
+ * Only for a 1x1 convolution with unit stride, no padding and group 1 whose pixels are one strided run in `in`
+ * and `out` (it runs as a plain contraction; fp32 whatever `flags` say).  `channel_scale` ([1, C, 1, ..], NULL:
+ * none) multiplies the input, each product rounded as the separate kernel rounds it; one image only.  `addend`
+ * (NULL: none) has the shape and strides of `out`.  Anything else: FL_ERR_UNSUPPORTED, nothing launched. */
+int fluidml_hip_conv_chain_scale_add(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, const fl_ew_program *chain, const fl_tensor *channel_scale, const fl_tensor *addend, uint32_t flags, void *stream);
 /* SoftmaxKernel over K <= 16 logits [B, K, 1] -> MatMulKernel [B, M, K] x [B, K, 1] as ONE launch:
  * out[b, m, 0] = sum_k a[b, m, k] * softmax_k(logits[b, :, 0]) (reference softmax.cpp, matmul.cpp:28-59; the
  * per-position kernel of a span-based dynamic convolution).  `out` is [B, M, 1] with the element strides

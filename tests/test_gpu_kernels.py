@@ -1266,6 +1266,55 @@ def test_conv_staged_patch(device):
         assert_close(do.logical(), want.logical(), what="conv with staged patch")
 
 
+def test_conv_scale_add(device):
+    """MulCommon (one factor per channel) -> Conv -> chain -> AddCommon (tensor of the output's shape) as one launch, against
+    the oracle's four kernels: pointwise convolutions on both tile sizes with the gate, the skip connection or both,
+    two images, a 1-d convolution."""
+    cabi = _cabi()
+    rng = np.random.default_rng(97)
+    relu = cabi.make_chain([(cabi.EW_RELU, 0)])
+    none = cabi.make_chain([])
+    cases = [((1, 96, 28, 28), 40, 1, True, True, False, None),      # small tile, gate and skip connection
+             ((1, 240, 56, 56), 80, 1, True, False, True, None),     # 64x64 tile, gate, ReLU
+             ((1, 37, 9, 11), 50, 1, True, True, False, None),       # ragged extents, scalar loads
+             ((2, 64, 20, 20), 64, 1, False, True, True, None)]      # two images, skip connection
+    for xshape, filters, k, gate, skip, with_chain, lo in cases:
+        pads = [k // 2] * 4
+        wshape = (filters, xshape[1], k, k)
+        oshape = (xshape[0], filters, xshape[2], xshape[3])
+        x, w, bias = rand(rng, xshape, -1, 1), rand(rng, wshape, -0.2, 0.2), rand(rng, (filters,), -1, 1)
+        scale, res = rand(rng, (1, xshape[1], 1, 1), 0, 1), rand(rng, oshape, -1, 1)
+        announce("conv scale/add", xshape, wshape, gate, skip, with_chain, lo)
+        hx = ok.View(x)
+        if gate:
+            hx = ok.View.empty(xshape)
+            ok.binary_f32(ok.BOP_MUL, ok.View(x), ok.View(scale), hx)
+        want = ok.View.empty(oshape, np.float32, lo)
+        ok.conv(hx, ok.View(w), ok.View(bias), want, pads if k > 1 else None, [1, 1], [1, 1], 1, 0)
+        if with_chain:
+            t = ok.View.empty(oshape, np.float32, lo)
+            ok.unary_f32(ok.OP_RELU, want, t)
+            want = t
+        hres = ok.View.empty(oshape, np.float32, lo)
+        hres.logical()[...] = res
+        if skip:
+            t = ok.View.empty(oshape, np.float32, lo)
+            ok.binary_f32(ok.BOP_ADD, want, hres, t)
+            want = t
+        dx, dw, db = DeviceView(ok.View(x), device), DeviceView(ok.View(w), device), DeviceView(ok.View(bias), device)
+        ds, dr = DeviceView(ok.View(scale), device), DeviceView(hres, device)
+        do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
+        cabi.call("conv_chain_scale_add", dx.ref(), dw.ref(), db.ref(), do.ref(), cabi.i64_array(pads) if k > 1 else None,
+                  cabi.i64_array([1, 1]), cabi.i64_array([1, 1]), ctypes.c_int64(1), ctypes.byref(relu if with_chain else none),
+                  ds.ref() if gate else None, dr.ref() if skip else None, ctypes.c_uint32(0), None)
+        assert_close(do.logical(), want.logical(), what="conv with channel scale / addend")
+    # what the entry point refuses: anything but a pointwise convolution
+    x, w = DeviceView(ok.View(rand(rng, (1, 8, 6, 6))), device), DeviceView(ok.View(rand(rng, (8, 8, 3, 3))), device)
+    o, sc = DeviceView(ok.View.empty((1, 8, 6, 6)), device), DeviceView(ok.View(rand(rng, (1, 8, 1, 1))), device)
+    assert cabi.lib.fluidml_hip_conv_chain_scale_add(x.ref(), w.ref(), None, o.ref(), cabi.i64_array([1, 1, 1, 1]), cabi.i64_array([1, 1]),
+                                                     cabi.i64_array([1, 1]), 1, ctypes.byref(none), sc.ref(), None, 0, None) == cabi.FL_ERR_UNSUPPORTED
+
+
 def test_argument_errors(device):
     """Rejected arguments return negative codes and launch nothing."""
     cabi = _cabi()

@@ -53,7 +53,10 @@ struct HaloArgs {
 
 // NV: pixel tiles (4 rows x 8 columns each) a wave owns, one below the other: the workgroup covers 4 NV x 16 pixels.
 // With two, the weights a wave reads from LDS serve twice the products and a barrier separates twice the work.
-template <int NV>
+// FEW: fewer than eight input channels (the first layer of an image network): one chunk whose missing channels read
+// as zero; the filters' rows are then shorter than a chunk and not 16-byte aligned, so the weights are loaded
+// value by value.
+template <int NV, bool FEW>
 __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict__ out, const float *__restrict__ in,
                                                               const float *__restrict__ weights, HaloArgs p) {
   constexpr int kTH = 4 * NV;
@@ -103,8 +106,8 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
     const int r = rem / kPCols, s = rem % kPCols;
     const int ih = oh0 - p.ph + r, iw = ow0 - p.pw + s;
     x_ok[t] = i < kXItems && static_cast<uint32_t>(ih) < static_cast<uint32_t>(p.H) &&
-              static_cast<uint32_t>(iw) < static_cast<uint32_t>(p.W);
-    x_src[t] = image + static_cast<int64_t>(ch) * p.sXc + (x_ok[t] ? ih * p.sXh + iw * p.sXw : 0);
+              static_cast<uint32_t>(iw) < static_cast<uint32_t>(p.W) && (!FEW || ch < p.C);
+    x_src[t] = image + (x_ok[t] ? static_cast<int64_t>(ch) * p.sXc + ih * p.sXh + iw * p.sXw : 0);
     x_dst[t] = i < kXItems ? ch * kPlane + r * kPitch + s : -1;
   }
 
@@ -114,7 +117,13 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
     const int c0 = c * kCC;
 #pragma unroll
     for (int t = 0; t < kWPer; ++t) {
-      wr[t] = w_ok[t] ? *reinterpret_cast<const floatx4 *>(w_src[t] + c0 * 9) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+      if constexpr (FEW) {
+        const int q4 = ((tid + t * kThreads) % 18) * 4, n_w = p.C * 9;  // position of the piece inside the filter's row
+        wr[t] = floatx4{w_ok[t] && q4 < n_w ? w_src[t][0] : 0.0f, w_ok[t] && q4 + 1 < n_w ? w_src[t][1] : 0.0f,
+                        w_ok[t] && q4 + 2 < n_w ? w_src[t][2] : 0.0f, w_ok[t] && q4 + 3 < n_w ? w_src[t][3] : 0.0f};
+      } else {
+        wr[t] = w_ok[t] ? *reinterpret_cast<const floatx4 *>(w_src[t] + c0 * 9) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+      }
     }
 #pragma unroll
     for (int t = 0; t < kXPer; ++t) xr[t] = x_ok[t] ? x_src[t][static_cast<int64_t>(c0) * p.sXc] : 0.0f;
@@ -141,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
   const int a_base = (wm * 32 + lrow) * kWPitch + half * 36;
   const int b_base = half * 4 * kPlane + py * kPitch + px;
 
-  const int n_chunks = p.C / kCC;
+  const int n_chunks = FEW ? 1 : p.C / kCC;
   load_chunk(0);
   store_chunk(0);
   __syncthreads();
@@ -217,10 +226,11 @@ int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *
   }
   const int64_t N = in->shape[0], C = in->shape[1], H = in->shape[2], W = in->shape[3];
   const int64_t F = out->shape[1], OH = out->shape[2], OW = out->shape[3];
-  if (C % kCC != 0 || F < 32) return FL_ERR_UNSUPPORTED;
+  const bool few = C < kCC;
+  if ((C % kCC != 0 && !few) || F < 32) return FL_ERR_UNSUPPORTED;
   // weights (c, kh, kw)-contiguous inside a filter, filters 16-byte aligned
   if (weights->strides[3] != 1 || weights->strides[2] != 3 || weights->strides[1] != 9) return FL_ERR_UNSUPPORTED;
-  if (weights->strides[0] % 4 != 0 || !IsAligned(weights->base, 16)) return FL_ERR_UNSUPPORTED;
+  if (!few && (weights->strides[0] % 4 != 0 || !IsAligned(weights->base, 16))) return FL_ERR_UNSUPPORTED;
   if (Numel(in) > 0x7fffffff || Numel(out) > 0x7fffffff || Numel(weights) > 0x7fffffff) return FL_ERR_UNSUPPORTED;
   const int64_t ph = pads ? pads[0] : 0, pw = pads ? pads[1] : 0;
   if (ph < 0 || pw < 0 || ph > 2 || pw > 2) return FL_ERR_UNSUPPORTED;
@@ -255,15 +265,19 @@ int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *
     p.sB = static_cast<int32_t>(bias->strides[0]);
   }
   if (chain != nullptr) p.chain = *chain;
-  if (nv == 2) {
-    FL_LAUNCH(ConvHalo3x3Kernel<2>, dim3(static_cast<uint32_t>(n_tiles)), dim3(kThreads), 0, AsStream(stream),
-              static_cast<float *>(out->base), static_cast<const float *>(in->base),
-              static_cast<const float *>(weights->base), p);
+#define FL_HALO(NV_, FEW_)                                                                                          \
+  FL_LAUNCH((ConvHalo3x3Kernel<NV_, FEW_>), dim3(static_cast<uint32_t>(n_tiles)), dim3(kThreads), 0, AsStream(stream), \
+            static_cast<float *>(out->base), static_cast<const float *>(in->base),                                  \
+            static_cast<const float *>(weights->base), p)
+  if (few) {
+    if (nv == 2) FL_HALO(2, true);
+    else FL_HALO(1, true);
+  } else if (nv == 2) {
+    FL_HALO(2, false);
   } else {
-    FL_LAUNCH(ConvHalo3x3Kernel<1>, dim3(static_cast<uint32_t>(n_tiles)), dim3(kThreads), 0, AsStream(stream),
-              static_cast<float *>(out->base), static_cast<const float *>(in->base),
-              static_cast<const float *>(weights->base), p);
+    FL_HALO(1, false);
   }
+#undef FL_HALO
   return LaunchStatus();
 }
 

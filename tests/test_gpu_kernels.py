@@ -1240,13 +1240,15 @@ def test_conv_large_tiles(device):
 def test_conv_staged_patch(device):
     """3x3 unit-stride convolutions that take the kernel with the input patch staged in LDS: one and two pixel tiles per
     wave, image extents that leave the last tiles ragged, a filter count that leaves the last filter tile half empty,
-    no padding, channels-last output, bias and a ReLU chain."""
+    no padding, channels-last output, bias and a ReLU chain, fewer than eight input channels."""
     cabi = _cabi()
     rng = np.random.default_rng(83)
     relu = cabi.make_chain([(cabi.EW_RELU, 0)])
     for xshape, filters, pads, lo, with_chain in [((8, 8, 96, 150), 96, [1, 1, 1, 1], None, True),     # two tiles per wave
                                                   ((3, 16, 30, 62), 160, [1, 1, 1, 1], [0, 3, 1, 2], False),  # ragged rows
-                                                  ((2, 8, 66, 66), 128, [0, 0, 0, 0], None, True)]:    # no padding
+                                                  ((2, 8, 66, 66), 128, [0, 0, 0, 0], None, True),     # no padding
+                                                  ((4, 3, 64, 80), 64, [1, 1, 1, 1], None, True),      # three channels, two tiles per wave
+                                                  ((2, 5, 33, 70), 40, [1, 1, 1, 1], None, False)]:    # five channels, ragged
         wshape = (filters, xshape[1], 3, 3)
         x, w, bias = rand(rng, xshape, -1, 1), rand(rng, wshape, -0.1, 0.1), rand(rng, (filters,), -1, 1)
         oh, ow = xshape[2] + 2 * pads[0] - 2, xshape[3] + 2 * pads[1] - 2

@@ -153,6 +153,7 @@ SIGNATURES = {
     "fluidml_hip_gemm_constant_weights_bias": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _u32, _vp],
     "fluidml_hip_matmul_add": [_T, _T, _T, _T, _vp],
     "fluidml_hip_matmul_chain": [_T, _T, _T, _T, _vp, _u32, _vp],
+    "fluidml_hip_matmul_chain_add": [_T, _T, _T, _T, _vp, _T, _T, _u32, _vp],
     "fluidml_hip_matmul_chain_view": [_T, _T, _T, _T, _i64, _i64, _vp, _u32, _vp],
     "fluidml_hip_matmul_chain_group": [_i32, _T, _vp, _vp, _vp, _i64, _i64p, _vp, _u32, _vp],
     "fluidml_hip_gemm_chain": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _vp, _u32, _vp],

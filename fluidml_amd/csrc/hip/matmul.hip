@@ -94,10 +94,12 @@ struct MatmulArgs {
   FastDiv div_inner;
   // optional elementwise chain applied after the bias (chain.n == 0: none)
   fl_ew_program chain;
-  // EXTRA instantiations only (plain contraction, B kept [k][n]), both optional:
+  // EXTRA instantiations only (plain contraction, B kept [k][n]), all optional:
   // a tensor with the strides of C, added to the value after the chain (read at the element offset the value is
   // stored at);
   const float *addend;
+  // a second one, added after the first;
+  const float *addend2;
   // one batch element: row k of B is multiplied by k_scale[k * sKs] while it is staged, each product rounded like
   // a separate Mul kernel's
   const float *k_scale;
@@ -192,7 +194,7 @@ struct TileLoader {
 // the plain kernel leaves each SIMD idle while its single wave waits for loads, writes LDS or sits at the
 // barrier; here the two roles overlap.
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV = 0,
-          bool BF16 = false, bool SPEC = false, bool EXTRA = false>
+          bool BF16 = false, bool SPEC = false, int EXTRA = 0>
 __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(float *__restrict__ C_, const float *__restrict__ A,
                                                                 const float *__restrict__ B_, MatmulArgs p) {
   float *__restrict__ C = C_;
@@ -219,7 +221,8 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   constexpr int VB = CONV == 2 ? 4 : CONV == 1 ? 1 : VEC;
   static_assert(!CONV || (LB == 0 && NT % (BN / VB) == 0), "the gather keeps one output pixel (group) per thread");
   static_assert(!SPEC || !CONV, "the gather of the convolution runs in the consumer waves");
-  static_assert(!EXTRA || (LB == 0 && CONV == 0), "the extra operands exist for plain contractions with B kept [k][n]");
+  // EXTRA: 0 = none, 1 = addends in the epilogue, 2 = addends and a scale per row of B
+  static_assert(EXTRA == 0 || (LB == 0 && CONV == 0), "the extra operands exist for plain contractions with B kept [k][n]");
   const bool producer = SPEC && threadIdx.x >= NT;
   const int ltid = producer ? static_cast<int>(threadIdx.x) - NT : static_cast<int>(threadIdx.x);
   using LoaderA = typename std::conditional<LA == 0, TileLoader<BM, BK, VEC, NT>, TileLoader<BK, BM, VEC, NT>>::type;
@@ -316,7 +319,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   static_assert(DEPTH % 2 == 0, "the LDS buffer index must be a compile-time function of the stage");
   VecF<VEC> ra[DEPTH][LoaderA::kPerThread];
   VecF<VB> rb[DEPTH][LoaderB::kPerThread];
-  float rs[DEPTH][LoaderB::kPerThread];  // EXTRA: the scale of the row each item of the B tile belongs to
+  float rs[DEPTH][LoaderB::kPerThread];  // EXTRA == 2: the scale of the row each item of the B tile belongs to
   const int rows_m = p.M - m0, cols_n = p.N - n0;
   const int n_chunks = (p.K + BK - 1) / BK;
 
@@ -337,7 +340,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   auto load_chunk = [&](int c, VecF<VEC>(&qa)[LoaderA::kPerThread], VecF<VB>(&qb)[LoaderB::kPerThread],
                         float(&qs)[LoaderB::kPerThread]) {
     const int k0 = c * BK, k_valid = p.K - k0;
-    if constexpr (EXTRA) {
+    if constexpr (EXTRA == 2) {
       if (p.k_scale != nullptr) {
 #pragma unroll
         for (int j = 0; j < LoaderB::kPerThread; ++j) {
@@ -398,7 +401,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
     float *as = lds + buf * (A_ELEMS + B_ELEMS);
     float *bs = as + A_ELEMS;
     LoaderA::Store(as, LDA, qa, ltid);
-    if constexpr (EXTRA) {
+    if constexpr (EXTRA == 2) {
       if (p.k_scale != nullptr) {
         VecF<VB> scaled[LoaderB::kPerThread];
 #pragma unroll
@@ -655,16 +658,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
       // bias, then the elementwise chain on the values of this 32x32 tile the lane holds (all 16, or the 4 of its
       // wave's quarter), then the stores
       auto tile_row = [&](int e) { return QUARTER ? ks * 8 + half * 4 + e : (e / 4) * 8 + half * 4 + (e % 4); };
-      float vals[EV], add[EV];
-      const float *Eb = nullptr;
-      if constexpr (EXTRA) {
-        Eb = p.addend != nullptr ? p.addend + boff[0] : nullptr;
-#pragma unroll
-        for (int e = 0; e < EV; ++e) {
-          const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
-          add[e] = Eb != nullptr && m < p.M && n < p.N ? Eb[static_cast<int64_t>(m) * sCm + col] : 0.0f;
-        }
-      }
+      float vals[EV];
 #pragma unroll
       for (int e = 0; e < EV; ++e) {
         const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
@@ -677,10 +671,24 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
         vals[e] = v;
       }
       if (p.chain.n != 0) RunChainBlock<EV>(p.chain, vals);
-      if constexpr (EXTRA) {
-        if (Eb != nullptr) {
+      if constexpr (EXTRA != 0) {
+        // both tensors are requested before either is added
+        if (p.addend != nullptr) {
+          const float *Eb = p.addend + boff[0], *Eb2 = p.addend2 != nullptr ? p.addend2 + boff[0] : nullptr;
+          float add[EV], add2[EV];
+#pragma unroll
+          for (int e = 0; e < EV; ++e) {
+            const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
+            const bool inside = m < p.M && n < p.N;
+            add[e] = inside ? Eb[static_cast<int64_t>(m) * sCm + col] : 0.0f;
+            add2[e] = Eb2 != nullptr && inside ? Eb2[static_cast<int64_t>(m) * sCm + col] : 0.0f;
+          }
 #pragma unroll
           for (int e = 0; e < EV; ++e) vals[e] += add[e];
+          if (Eb2 != nullptr) {
+#pragma unroll
+            for (int e = 0; e < EV; ++e) vals[e] += add2[e];
+          }
         }
       }
 #pragma unroll
@@ -924,7 +932,7 @@ inline int64_t SplitKLimit(int64_t fallback) {
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV, bool BF16,
-          bool SPEC = false, bool EXTRA = false>
+          bool SPEC = false, int EXTRA = 0>
 void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   MatmulArgs q = p;
   q.tiles_m = (p.M + BM - 1) / BM;
@@ -972,7 +980,7 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
             dim3(q.tiles_m * q.tiles_n, n_batch, splits), dim3(64 * WM * WN * KS * (SPEC ? 2 : 1)), 0, s, C, A, B, q);
 }
 
-template <int LA, int LB, int VEC, int CONV, bool BF16 = false, bool EXTRA = false>
+template <int LA, int LB, int VEC, int CONV, bool BF16 = false, int EXTRA = 0>
 void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
   const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
   // (A 128x128x16 tile with two chunks in flight was measured slower than the 64x64x32 tile with four at
@@ -1005,7 +1013,8 @@ struct Siblings {
 int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, bool trans_a, bool trans_b, float ca,
              float cb, const fl_tensor *bias, void *stream, const fl_ew_program *chain = nullptr, int64_t n_inner = 0,
              int64_t stride_outer = 0, const Siblings *siblings = nullptr, bool bf16 = false,
-             const float *addend = nullptr, const float *k_scale = nullptr, int64_t k_scale_stride = 0) {
+             const float *addend = nullptr, const float *k_scale = nullptr, int64_t k_scale_stride = 0,
+             const float *addend2 = nullptr) {
   FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(lhs));
   FL_CHECK(CheckView(rhs));
@@ -1139,8 +1148,9 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   // a second addend with the strides of C / a scale per row of B: the tiled kernel's own instantiations (fp32)
   const bool extra = addend != nullptr || k_scale != nullptr;
   if (extra) {
-    if (lb != 0 || p.n_groups > 1 || p.n_inner != 0) return FL_ERR_UNSUPPORTED;
+    if (lb != 0 || p.n_groups > 1 || p.n_inner != 0 || (addend2 != nullptr && addend == nullptr)) return FL_ERR_UNSUPPORTED;
     p.addend = addend;
+    p.addend2 = addend2;
   }
   if (k_scale != nullptr) {
     if (n_batch != 1 || k_scale_stride > INT32_MAX || k_scale_stride < 0) return FL_ERR_UNSUPPORTED;
@@ -1151,10 +1161,16 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   if (!extra && TrySkinnyGemm(p, n_batch, C, A, B, s)) return LaunchStatus();
   const uint32_t nb = static_cast<uint32_t>(n_batch);
   if (extra) {
-    if (la == 0 && vec) LaunchBySize<0, 0, 4, 0, false, true>(p, nb, C, A, B, s);
-    else if (la == 0) LaunchBySize<0, 0, 1, 0, false, true>(p, nb, C, A, B, s);
-    else if (vec) LaunchBySize<1, 0, 4, 0, false, true>(p, nb, C, A, B, s);
-    else LaunchBySize<1, 0, 1, 0, false, true>(p, nb, C, A, B, s);
+#define FL_MM_EXTRA(E_)                                                     \
+  do {                                                                      \
+    if (la == 0 && vec) LaunchBySize<0, 0, 4, 0, false, E_>(p, nb, C, A, B, s);  \
+    else if (la == 0) LaunchBySize<0, 0, 1, 0, false, E_>(p, nb, C, A, B, s);    \
+    else if (vec) LaunchBySize<1, 0, 4, 0, false, E_>(p, nb, C, A, B, s);        \
+    else LaunchBySize<1, 0, 1, 0, false, E_>(p, nb, C, A, B, s);                 \
+  } while (0)
+    if (k_scale != nullptr) FL_MM_EXTRA(2);
+    else FL_MM_EXTRA(1);
+#undef FL_MM_EXTRA
     return LaunchStatus();
   }
 #define FL_MM_DISPATCH(LA_, LB_)                              \
@@ -1377,6 +1393,29 @@ int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const f
   if (bias != nullptr && bias->rank != 1) return FL_ERR_RANK;
   return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, 0, 0, nullptr,
                       (flags & FL_CONTRACT_BF16) != 0);
+}
+
+int fluidml_hip_matmul_chain_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
+                                 const fl_ew_program *chain, const fl_tensor *addend, const fl_tensor *addend2,
+                                 uint32_t flags, void *stream) {
+  if (!lhs || !rhs || !out || !addend) return FL_ERR_NULL;
+  if (bias != nullptr && bias->rank != 1) return FL_ERR_RANK;
+  const float *e[2] = {nullptr, nullptr};
+  const fl_tensor *t[2] = {addend, addend2};
+  for (int i = 0; i < 2; ++i) {
+    if (t[i] == nullptr) continue;
+    FL_CHECK(fl::CheckView(t[i]));
+    if (t[i]->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+    if (t[i]->rank != out->rank) return FL_ERR_SHAPE;
+    for (int d = 0; d < out->rank; ++d) {
+      if (t[i]->shape[d] != out->shape[d]) return FL_ERR_SHAPE;
+      if (out->shape[d] > 1 && t[i]->strides[d] != out->strides[d]) return FL_ERR_UNSUPPORTED;
+    }
+    e[i] = static_cast<const float *>(t[i]->base);
+  }
+  (void)flags;  // fp32 whatever the flags say: the extra operands exist in the fp32 instantiations only
+  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, 0, 0, nullptr, false, e[0], nullptr, 0,
+                      e[1]);
 }
 
 int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,

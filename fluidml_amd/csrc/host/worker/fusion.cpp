@@ -564,11 +564,11 @@ class Scheduler {
         rewired_[r] = true;
       }
       for (Launch &l : *fused) {
-        for (Operand *op : {&l.a, &l.b, &l.c, &l.d}) {
+        for (Operand *op : {&l.a, &l.b, &l.c, &l.d, &l.e}) {
           if (SameTensor(*op, produced) && !op->viewed) *op = seen;
         }
         for (Launch &g : l.group) {
-          for (Operand *op : {&g.a, &g.b, &g.c, &g.d}) {
+          for (Operand *op : {&g.a, &g.b, &g.c, &g.d, &g.e}) {
             if (SameTensor(*op, produced) && !op->viewed) *op = seen;
           }
         }
@@ -723,7 +723,7 @@ class Scheduler {
           if (Alias(st.in0, target) || (st.node->IsDoubleInputs() && Alias(st.in1, target))) ok = false;
         }
         if (l != nullptr) {
-          for (const Operand *op : {&l->a, &l->b, &l->c, &l->d}) {
+          for (const Operand *op : {&l->a, &l->b, &l->c, &l->d, &l->e}) {
             if (!op->name.empty() && Alias(*op, target)) ok = false;
           }
         }
@@ -933,6 +933,9 @@ class Scheduler {
       l.members.insert(l.members.end(), chain->members.begin(), chain->members.end());
       l.chain = chain->program;
     }
+    if (l.kind == Launch::Kind::MatMulChain) {
+      if (auto wider = WithAddends(i, l)) return wider;
+    }
     // MatMul only: trailing Reshape / Transpose steps that merely re-address the result are folded into the
     // kernel's output strides (the head split and merge copies of an attention block)
     if (l.kind == Launch::Kind::MatMulChain) {
@@ -966,6 +969,55 @@ class Scheduler {
       }
       l.members.resize(without_chain);
       l.chain = fl_ew_program{};
+    }
+    return std::nullopt;
+  }
+
+  // A MatMul chain (already matched in `plain`) whose value goes through one or two AddCommon with tensors of its
+  // own shape and layout (a residual connection; GPT-NeoX's x + attention + mlp): the tensors become operands of
+  // the launch, added in the epilogue in the order of the steps.  The kernel's instantiations with extra operands
+  // want the right operand stored n-fastest.
+  std::optional<Launch> WithAddends(size_t i, const Launch &plain) {
+    if (const char *v = std::getenv("FLUIDML_MATMUL_ADDENDS"); v != nullptr && std::string(v) == "0") return std::nullopt;
+    const Step &head = steps_[i];
+    if (!IsFloat(head.in1) || head.in1.viewed || !DefaultLayout(head.in1) || head.in1.meta.GetShape().size() < 2) return std::nullopt;
+    std::vector<size_t> adds;
+    std::vector<Operand> tensors;
+    size_t value = plain.members.back();
+    while (adds.size() < 2) {
+      const auto j = SoleReader(value);
+      if (!j || Kind(*j) != OpKind::AddCommon) break;
+      const Operand &v = steps_[value].out;
+      const auto other = Other(*j, v);
+      if (!other || !IsFloat(*other) || other->viewed || other->space == Operand::Space::Constant ||
+          other->meta.GetShape() != v.meta.GetShape() || steps_[*j].out.meta.GetShape() != v.meta.GetShape()) {
+        break;
+      }
+      adds.push_back(*j);
+      tensors.push_back(*other);
+      value = *j;
+    }
+    for (size_t n = adds.size(); n >= 1; --n) {
+      Launch l = plain;
+      std::vector<std::pair<size_t, Operand>> external = {{i, l.a}, {i, l.b}};
+      bool ok = true;
+      for (size_t k = 0; k < n; ++k) {
+        l.members.push_back(adds[k]);
+        external.push_back({adds[k], tensors[k]});
+      }
+      l.out = steps_[l.members.back()].out;
+      for (size_t k = 0; k < n; ++k) ok = ok && tensors[k].layout == l.out.layout && !Alias(l.out, tensors[k]);
+      if (!ok || !Safe(l.members, external) || !OutputDisjoint(l.out, {&l.a, &l.b})) continue;
+      l.d = tensors[0];
+      l.has_skip = true;
+      if (n == 2) {
+        l.e = tensors[1];
+        l.has_skip2 = true;
+      }
+      l.bytes = l.has_c ? Bytes({&l.a, &l.b, &l.c, &l.out}) : Bytes({&l.a, &l.b, &l.out});
+      for (size_t k = 0; k < n; ++k) l.bytes += static_cast<double>(tensors[k].meta.GetSize());
+      l.flops = Flops(l.members);
+      return l;
     }
     return std::nullopt;
   }
@@ -1205,7 +1257,7 @@ class Scheduler {
   // crosses no reader of their outputs and no write to what they read.
   void GroupSiblings(std::vector<Launch> *fused) const {
     auto compatible = [&](const Launch &x, const Launch &y) {
-      if (x.kind != Launch::Kind::MatMulChain || y.kind != Launch::Kind::MatMulChain) return false;
+      if (x.kind != Launch::Kind::MatMulChain || y.kind != Launch::Kind::MatMulChain || x.has_skip || y.has_skip) return false;
       const Step &hx = steps_[x.members[0]], &hy = steps_[y.members[0]];
       const auto &shape = hx.out.meta.GetShape();
       int64_t batch = 1;

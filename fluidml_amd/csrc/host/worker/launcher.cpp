@@ -233,7 +233,13 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
       kernel::TensorView c;
       if (l.has_c) c = ViewOf(Resolve(l.c), l.c);
-      if (l.view_strides.empty()) {
+      if (l.has_skip) {
+        const kernel::TensorView d = ViewOf(Resolve(l.d), l.d);
+        kernel::TensorView e;
+        if (l.has_skip2) e = ViewOf(Resolve(l.e), l.e);
+        rc = fluidml_hip_matmul_chain_add(&a.t, &b.t, l.has_c ? &c.t : nullptr, &out.t, &l.chain, &d.t,
+                                          l.has_skip2 ? &e.t : nullptr, contract_flags, ctx.stream);
+      } else if (l.view_strides.empty()) {
         rc = fluidml_hip_matmul_chain(&a.t, &b.t, l.has_c ? &c.t : nullptr, &out.t, &l.chain, contract_flags, ctx.stream);
       } else {
         // the contraction's logical output addressed inside the buffer of the last folded Reshape / Transpose

@@ -64,6 +64,7 @@ struct Launch {
   enum class Kind {
     Step,              // members = {i}
     MatMulChain,       // MatMul [-> AddCommon(rank-1 constant bias)] [-> elementwise chain]
+                       // [-> AddCommon(tensor) [-> AddCommon(tensor)]]
     GemmChain,         // GemmConstantWeightsBias -> elementwise chain
     ConvChain,         // [MulCommon(x, factor per channel) ->] Conv{With,Without}Padding -> elementwise chain
                        // [-> AddCommon(tensor of the output's shape)]
@@ -94,14 +95,16 @@ struct Launch {
   };
   Kind kind = Kind::Step;
   std::vector<size_t> members;  // indices into the step list, ascending
-  Operand a, b, c, d, out;      // external operands, role by kind (see fusion.cpp)
+  Operand a, b, c, d, e, out;   // external operands, role by kind (see fusion.cpp)
   double s0 = 0, s1 = 0, s2 = 0;
   int64_t axis = 0;
   std::vector<int64_t> perm;
   bool has_c = false;     // MatMulChain: a bias operand is present
   // ConvChain: c = a per-channel factor of the input (the MulCommon in front of the convolution is a member),
   // d = a tensor of the output's shape added after the chain (the AddCommon behind it is a member)
-  bool has_gate = false, has_skip = false;
+  // MatMulChain: d [and e] = tensors of the output's shape added after the chain, in this order (the AddCommon
+  // steps are members): has_skip [and has_skip2]
+  bool has_gate = false, has_skip = false, has_skip2 = false;
   // Attention: a = queries, b = keys (transposed), c = values, d = additive mask (has_mask), the Where step
   // `owner` holds the condition (has_cond) and s1 its fill value; s0 scales the scores, dividing if `divisor`
   bool has_mask = false, has_cond = false, divisor = false;

@@ -359,6 +359,11 @@ int fluidml_hip_matmul_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
  * result, e.g. the erf-GELU chain Div, Erf, Add, Mul(x), Mul of
  * add_div_erf_add_mul_mul.cpp:29-132.  `bias` and `chain` may be NULL. */
 int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, const fl_ew_program *chain, uint32_t flags, void *stream);
+/* The same followed by one or two AddCommonKernel with tensors of the output's shape and strides (a residual
+ * connection, or GPT-NeoX's parallel residual x + attention + mlp): out = (chain(lhs . rhs + bias) + addend) + addend2,
+ * each sum rounded like the separate kernels' (reference matmul.cpp:28-59, add.cpp:75-137).  `addend2` may be NULL.
+ * `rhs` must be unit-stride along its last dim; fp32 whatever `flags` say.  Otherwise FL_ERR_UNSUPPORTED. */
+int fluidml_hip_matmul_chain_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, const fl_ew_program *chain, const fl_tensor *addend, const fl_tensor *addend2, uint32_t flags, void *stream);
 /* The same, followed by Reshape / Transpose steps that only re-address the
  * result (reference reshape.cpp:18-64, transpose.cpp:19-48): `out` carries the
  * contraction's logical shape [..., M, N] with the element strides each of

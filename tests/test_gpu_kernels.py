@@ -718,6 +718,50 @@ def test_fused_matmul_add_and_gelu(device):
             assert_close(do.logical(), u1.logical(), what="matmul_chain relu, scale")
 
 
+def test_matmul_chain_add(device):
+    """MatMul + bias [+ chain] followed by one or two AddCommon with tensors of the output's shape, as one launch; the
+    sums are taken in the order of the separate kernels.  Small and large tiles, batch dims, a transposed output."""
+    cabi = _cabi()
+    rng = np.random.default_rng(93)
+    relu = cabi.make_chain([(cabi.EW_RELU, 0)])
+    none = cabi.make_chain([])
+    for ashape, bshape, lo, two, with_chain in [((1, 256, 512), (512, 512), None, True, False),
+                                                ((1, 128, 768), (768, 768), None, False, False),
+                                                ((2, 3, 70, 40), (40, 96), None, True, True),
+                                                ((1, 300, 256), (256, 1024), [0, 2, 1], True, False)]:
+        a, b = rand(rng, ashape, -1, 1), rand(rng, bshape, -0.05, 0.05)
+        oshape = ashape[:-1] + (bshape[-1],)
+        bias, r1, r2 = rand(rng, (bshape[-1],), -0.5, 0.5), rand(rng, oshape, -1, 1), rand(rng, oshape, -1, 1)
+        announce("matmul_chain_add", ashape, bshape, lo, two, with_chain)
+        t0, t1 = ok.View.empty(oshape), ok.View.empty(oshape)
+        ok.matmul(ok.View(a), ok.View(b), t0)
+        ok.binary_f32(ok.BOP_ADD, ok.View(bias), t0, t1)
+        if with_chain:
+            t = ok.View.empty(oshape)
+            ok.unary_f32(ok.OP_RELU, t1, t)
+            t1 = t
+        want = ok.View.empty(oshape)
+        ok.binary_f32(ok.BOP_ADD, ok.View(r1), t1, want)
+        if two:
+            t = ok.View.empty(oshape)
+            ok.binary_f32(ok.BOP_ADD, want, ok.View(r2), t)
+            want = t
+        h1, h2 = ok.View.empty(oshape, np.float32, lo), ok.View.empty(oshape, np.float32, lo)
+        h1.logical()[...] = r1
+        h2.logical()[...] = r2
+        da, db, dbias = DeviceView(ok.View(a), device), DeviceView(ok.View(b), device), DeviceView(ok.View(bias), device)
+        d1, d2 = DeviceView(h1, device), DeviceView(h2, device)
+        do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
+        cabi.call("matmul_chain_add", da.ref(), db.ref(), dbias.ref(), do.ref(), ctypes.byref(relu if with_chain else none),
+                  d1.ref(), d2.ref() if two else None, ctypes.c_uint32(0), None)
+        assert_close(do.logical(), want.logical(), what="matmul_chain_add")
+    # a right operand stored k-fastest is refused
+    bt = DeviceView(ok.View(rand(rng, (40, 96)), [1, 0]), device)
+    a = DeviceView(ok.View(rand(rng, (70, 40))), device)
+    o, r = DeviceView(ok.View.empty((70, 96)), device), DeviceView(ok.View(rand(rng, (70, 96))), device)
+    assert cabi.lib.fluidml_hip_matmul_chain_add(a.ref(), bt.ref(), None, o.ref(), ctypes.byref(none), r.ref(), None, 0, None) == cabi.FL_ERR_UNSUPPORTED
+
+
 def test_matmul_chain_view(device):
     """MatMul + bias written straight into the buffer of a following Reshape (last dim split into heads) and
     Transpose: the head-split copies of an attention block folded into the contraction's output addressing."""

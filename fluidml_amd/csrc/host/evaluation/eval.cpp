@@ -120,6 +120,23 @@ class MeasuredCostModel : public CostModel {
       Check(fluidml_hip_arena_create(g.GetOutputMeta().GetSize(), &b.out), "output buffer");
       Check(fluidml_hip_arena_create(g.GetBufferSize(), &b.scratch), "scratch buffer");
     }
+    // A rank-4 tensor has 24 layouts and a convolution three tensors: most of the combinations are far from any
+    // fast path of the kernels and take tens of milliseconds each on a large layer.  Every combination of the
+    // layouts a kernel is written for (default and channels-last; every layout of tensors of rank <= 3) is always
+    // timed; the others only while the kernel's measuring budget (1.5 s of device time) lasts, after that they
+    // are priced at eight times the default layouts' time, i.e. never chosen.
+    auto natural = [](const Layout &l) {
+      if (l.size() < 4) return true;
+      bool identity = true, channels_last = l[0] == 0 && l.back() == 1;
+      for (size_t i = 0; i < l.size(); ++i) identity = identity && l[i] == i;
+      for (size_t i = 1; i + 1 < l.size(); ++i) channels_last = channels_last && l[i] == i + 1;
+      return identity || channels_last;
+    };
+    bool all_natural = true;
+    for (const Layout &l : key) all_natural = all_natural && natural(l);
+    if (!all_natural && b.spent_ns > kBudgetPerKernelNs) {
+      return std::max<size_t>(1, static_cast<size_t>((b.default_ns > 0 ? b.default_ns : 1e8) * 8.0));
+    }
     const bool single = g.IsSingleInput();
     const Layout &lhs_layout = key[0], &out_layout = key.back();
     std::shared_ptr<kernel::Kernel> k = g.Yield(lhs_layout, single ? Layout{} : key[1], out_layout);
@@ -141,19 +158,33 @@ class MeasuredCostModel : public CostModel {
       }
       Check(ctx.status, ctx.failed.c_str());
     };
-    launch();  // warm: code object load, caches
     // the dispatch's own begin/end timestamps: launch latency and queue gaps would otherwise swamp
-    // the differences between layouts for the many kernels that run only a few microseconds
+    // the differences between layouts for the many kernels that run only a few microseconds.  The first launch
+    // warms up (code object load, caches); a candidate that takes more than a millisecond even so is timed by that
+    // launch alone -- a 4-d tensor has 24 layouts, most of them far from the kernels' fast paths, and five rounds of
+    // each would take minutes on the large convolutions -- the others get up to five more rounds or 2 ms.
     constexpr int kRounds = 5;
+    constexpr double kSlowNs = 1e6, kBudgetNs = 2e6;
     double best = std::numeric_limits<double>::max();
     Check(fluidml_hip_time_kernels(start_, stop_), "kernel timing on");
     try {
-      for (int r = 0; r < kRounds; ++r) {
-        launch();
-        double ns = 0;
-        Check(fluidml_hip_event_elapsed_ns(start_, stop_, &ns), "elapsed");
-        best = std::min(best, ns);
+      launch();
+      double warm = 0;
+      Check(fluidml_hip_event_elapsed_ns(start_, stop_, &warm), "elapsed");
+      if (warm > kSlowNs) {
+        best = warm;
+      } else {
+        double spent = 0;
+        for (int r = 0; r < kRounds && spent < kBudgetNs; ++r) {
+          launch();
+          double ns = 0;
+          Check(fluidml_hip_event_elapsed_ns(start_, stop_, &ns), "elapsed");
+          best = std::min(best, ns);
+          spent += ns;
+        }
+        b.spent_ns += spent;
       }
+      b.spent_ns += warm;
     } catch (...) {
       fluidml_hip_time_kernels(nullptr, nullptr);
       throw;
@@ -167,6 +198,7 @@ class MeasuredCostModel : public CostModel {
     for (const Layout &l : key) {
       for (size_t i = 0; i < l.size(); ++i) all_default = all_default && l[i] == i;
     }
+    if (all_default) b.default_ns = best;
     if (!all_default) best = best * 1.02 + 200.0;
     return std::max<size_t>(1, static_cast<size_t>(best));
   }
@@ -174,7 +206,10 @@ class MeasuredCostModel : public CostModel {
  private:
   struct Buffers {
     void *lhs = nullptr, *rhs = nullptr, *out = nullptr, *scratch = nullptr;
+    double spent_ns = 0;    // device time spent timing this kernel's candidates
+    double default_ns = 0;  // its time with default layouts, once measured
   };
+  static constexpr double kBudgetPerKernelNs = 1.5e9;
   uint32_t flags_;
   void *stream_ = nullptr, *start_ = nullptr, *stop_ = nullptr;
   std::unordered_map<KernelEval *, Buffers> buffers_;

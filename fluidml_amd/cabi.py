@@ -134,6 +134,7 @@ SIGNATURES = {
     "fluidml_hip_slice": [_T, _T, _i64p, _i64p, _i64p, _i32, _vp],
     "fluidml_hip_concat2": [_T, _T, _T, _i64, _vp],
     "fluidml_hip_pad": [_T, _T, _i64p, _i32, _u32, _vp],
+    "fluidml_hip_pad_view_copy": [_T, _i64p, _i64p, _i32, _i64, _i64p, _T, _vp],
     "fluidml_hip_gather_constant_index_scalar": [_T, _T, _i64, _i64, _u32, _vp],
     "fluidml_hip_gather_constant_indices_tensor": [_T, _T, _T, _i64, _vp],
     "fluidml_hip_gather_constant_data_tensor": [_T, _T, _T, _vp],

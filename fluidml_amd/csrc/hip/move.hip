@@ -241,12 +241,107 @@ __global__ __launch_bounds__(kBlock) void CumSumKernel(NestArgs<2> outer, uint32
   }
 }
 
+// ---- Pad followed by steps that only re-address its result, as one copy ---------------------------------
+// out[i0, i1, ..] = padded[view_offset + sum(i_k * view_strides[k])] where `padded` is the Pad's output taken as a
+// dense row-major tensor that is never written: the element is read from the Pad's input when it lies in the
+// interior and is zero otherwise.  (ConvBERT unfolds the values of its span-based convolution this way: Pad along
+// the sequence, a Gather of sliding windows, Transpose, Reshape.)
+struct PadViewArgs {
+  int32_t out_rank, pad_rank;
+  uint32_t n;
+  int32_t view_offset;
+  FastDiv out_div[kMaxRank];      // out logical extents
+  int32_t out_strides[kMaxRank];
+  int32_t view_strides[kMaxRank];
+  FastDiv pad_div[kMaxRank];      // padded extents
+  int32_t before[kMaxRank];       // padding in front, per dim
+  int32_t src_shape[kMaxRank], src_strides[kMaxRank];
+};
+
+__global__ __launch_bounds__(kBlock) void PadViewCopyKernel(PadViewArgs a, uint32_t *__restrict__ out,
+                                                            const uint32_t *__restrict__ src) {
+  const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= a.n) return;
+  uint32_t rem = idx;
+  int32_t out_off = 0, lin = a.view_offset;
+#pragma unroll
+  for (int d = kMaxRank - 1; d >= 0; --d) {
+    if (d < a.out_rank) {
+      uint32_t q, r;
+      a.out_div[d].DivMod(rem, q, r);
+      rem = q;
+      out_off += static_cast<int32_t>(r) * a.out_strides[d];
+      lin += static_cast<int32_t>(r) * a.view_strides[d];
+    }
+  }
+  uint32_t left = static_cast<uint32_t>(lin);
+  int32_t src_off = 0;
+  bool inside = true;
+#pragma unroll
+  for (int d = kMaxRank - 1; d >= 0; --d) {
+    if (d < a.pad_rank) {
+      uint32_t q, r;
+      a.pad_div[d].DivMod(left, q, r);
+      left = q;
+      const int32_t c = static_cast<int32_t>(r) - a.before[d];
+      inside = inside && static_cast<uint32_t>(c) < static_cast<uint32_t>(a.src_shape[d]);
+      src_off += c * a.src_strides[d];
+    }
+  }
+  out[out_off] = inside ? src[src_off] : 0u;
+}
+
+int PadViewCopy(const fl_tensor *in, const int64_t *pads_before, const int64_t *padded_shape, int32_t n_dims,
+                int64_t view_offset, const int64_t *view_strides, const fl_tensor *out, void *stream) {
+  if (!in || !pads_before || !padded_shape || !view_strides || !out) return FL_ERR_NULL;
+  FL_CHECK(CheckView(in));
+  FL_CHECK(CheckView(out));
+  if (in->dtype != out->dtype) return FL_ERR_DTYPE;
+  if (DtypeSize(in->dtype) != 4) return FL_ERR_UNSUPPORTED;
+  if (n_dims != in->rank) return FL_ERR_RANK;
+  PadViewArgs a;
+  std::memset(&a, 0, sizeof(a));
+  int64_t padded_numel = 1;
+  for (int d = 0; d < in->rank; ++d) {
+    if (pads_before[d] < 0 || padded_shape[d] < pads_before[d] + in->shape[d]) return FL_ERR_ATTR;
+    padded_numel *= padded_shape[d];
+    a.pad_div[d] = FastDiv(static_cast<uint32_t>(padded_shape[d]));
+    a.before[d] = static_cast<int32_t>(pads_before[d]);
+    a.src_shape[d] = static_cast<int32_t>(in->shape[d]);
+    a.src_strides[d] = static_cast<int32_t>(in->strides[d]);
+  }
+  const int64_t n = Numel(out);
+  if (n == 0) return FL_OK;
+  if (padded_numel > 0x7fffffff || n > 0x7fffffff || view_offset < 0) return FL_ERR_TOO_LARGE;
+  int64_t last = view_offset;
+  for (int d = 0; d < out->rank; ++d) {
+    if (view_strides[d] < 0 || view_strides[d] > 0x7fffffff) return FL_ERR_ATTR;
+    last += (out->shape[d] - 1) * view_strides[d];
+    a.out_div[d] = FastDiv(static_cast<uint32_t>(out->shape[d]));
+    a.out_strides[d] = static_cast<int32_t>(out->strides[d]);
+    a.view_strides[d] = static_cast<int32_t>(view_strides[d]);
+  }
+  if (last >= padded_numel) return FL_ERR_SHAPE;  // the view reaches outside the padded tensor
+  a.out_rank = out->rank;
+  a.pad_rank = in->rank;
+  a.n = static_cast<uint32_t>(n);
+  a.view_offset = static_cast<int32_t>(view_offset);
+  FL_LAUNCH(PadViewCopyKernel, dim3(static_cast<uint32_t>((n + kBlock - 1) / kBlock)), dim3(kBlock), 0, AsStream(stream), a,
+            static_cast<uint32_t *>(out->base), static_cast<const uint32_t *>(in->base));
+  return LaunchStatus();
+}
+
 }  // namespace
 }  // namespace fl
 
 using namespace fl;
 
 extern "C" {
+
+int fluidml_hip_pad_view_copy(const fl_tensor *in, const int64_t *pads_before, const int64_t *padded_shape, int32_t n_dims,
+                              int64_t view_offset, const int64_t *view_strides, const fl_tensor *out, void *stream) {
+  return PadViewCopy(in, pads_before, padded_shape, n_dims, view_offset, view_strides, out, stream);
+}
 
 int fluidml_hip_reshape(const fl_tensor *in, const fl_tensor *out, void *stream) {
   return LogicalReshape(in, out, stream);

@@ -24,6 +24,7 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::MatMulGroup: return "MatMulGroup";
     case Launch::Kind::GemmChain: return "GemmChain";
     case Launch::Kind::ConvChain: return "ConvChain";
+    case Launch::Kind::PadViewCopy: return "PadViewCopy";
     case Launch::Kind::ConvPair: return "ConvPair";
     case Launch::Kind::SoftmaxMatVec: return "SoftmaxMatVec";
     case Launch::Kind::ElementwiseChain: return "ElementwiseChain";
@@ -255,6 +256,7 @@ class Scheduler {
           case OpKind::MulCommon: l = MatchMulAdd(i); break;
           case OpKind::AddCommon: l = MatchAddAdd(i); break;
           case OpKind::GatherConstantDataTensor: l = MatchGatherAdd(i); break;
+          case OpKind::Pad: l = MatchPadViewCopy(i); break;
           case OpKind::Reshape: l = MatchCopyPair(i, OpKind::Transpose); break;
           case OpKind::Transpose: l = MatchCopyPair(i, OpKind::Reshape); break;
           default: break;
@@ -345,8 +347,12 @@ class Scheduler {
   }
 
   // step i's output as a view of its input: (element offset, strides per output dim)
-  std::optional<std::pair<int64_t, std::vector<int64_t>>> AsView(size_t i) const {
-    const Step &s = steps_[i];
+  std::optional<std::pair<int64_t, std::vector<int64_t>>> AsView(size_t i) const { return AsViewOf(i, steps_[i].in0); }
+
+  // the same with the step's input taken to be `in0` (the step's own input, possibly seen through earlier views)
+  std::optional<std::pair<int64_t, std::vector<int64_t>>> AsViewOf(size_t i, const Operand &in0) const {
+    Step s = steps_[i];
+    s.in0 = in0;
     const std::vector<int64_t> st = LogicalStrides(s.in0);
     const auto &ishape = s.in0.meta.GetShape();
     const auto &oshape = s.out.meta.GetShape();
@@ -1868,6 +1874,52 @@ class Scheduler {
     if (Alias(l.out, l.a) || Alias(l.out, l.b)) return std::nullopt;
     l.bytes = Bytes({&l.a, &l.b, &l.out}) + static_cast<double>(steps_[*j].kernel->GetConstantBytes());
     return l;
+  }
+
+  // Pad (constant zero) whose result only goes through steps that re-address it -- Gather with sliding-window
+  // indices, Slice, Transpose, Reshape, each the only reader of the one before -- until the last of them: one copy
+  // that reads the Pad's input and writes the last step's output; the padded tensor and the views are never written.
+  std::optional<Launch> MatchPadViewCopy(size_t i) {
+    const Step &pad = steps_[i];
+    if (pad.in0.meta.GetType() != Type::kFloat32 || pad.in0.viewed || !DefaultLayout(pad.out)) return std::nullopt;
+    const auto &pshape = pad.out.meta.GetShape();
+    if (Attrs(i).pad_pairs.size() != pshape.size()) return std::nullopt;
+    Launch l;
+    l.kind = Launch::Kind::PadViewCopy;
+    l.members = {i};
+    l.a = pad.in0;
+    Operand cur = pad.out;  // what the next step reads, as a view of the padded tensor
+    std::optional<Launch> best;
+    size_t at = i;
+    while (true) {
+      const auto j = SoleReader(at);
+      if (!j || !steps_[*j].node->IsSingleInput() || !SameTensor(steps_[*j].in0, steps_[at].out)) break;
+      // the step's input: the padded tensor itself, then the previous view step's output seen inside it
+      const auto view = AsViewOf(*j, at == i ? pad.out : cur);
+      if (!view) break;
+      Operand seen = steps_[*j].out;
+      seen.space = pad.out.space;
+      seen.name = pad.out.name;
+      seen.offset = pad.out.offset;
+      seen.viewed = true;
+      seen.view_offset = view->first;
+      seen.view_strides = view->second;
+      seen.source_bytes = pad.out.meta.GetSize();
+      cur = seen;
+      l.members.push_back(*j);
+      at = *j;
+      // a launch that ends here: the view materialised into this step's own output
+      Launch candidate = l;
+      candidate.out = steps_[at].out;
+      candidate.view_offset = view->first;
+      candidate.view_strides = view->second;
+      if (candidate.members.size() >= 3 && Elidable(steps_[at].out) && Safe(candidate.members, {{i, l.a}}) &&
+          !Alias(candidate.out, l.a)) {
+        candidate.bytes = Bytes({&l.a, &candidate.out});
+        best = candidate;
+      }
+    }
+    return best;
   }
 
   std::optional<Launch> MatchCopyPair(size_t i, OpKind second) {

@@ -400,6 +400,14 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
     case Launch::Kind::CopyInto:
       rc = fluidml_hip_reshape(&a.t, &out.t, ctx.stream);  // same shape on both sides: a strided copy
       break;
+    case Launch::Kind::PadViewCopy: {
+      const Step &pad = steps_[l.members.front()];
+      std::vector<int64_t> before, padded(pad.out.meta.GetShape());
+      for (const auto &pr : pad.node->GetAttrs().pad_pairs) before.push_back(std::get<0>(pr));
+      rc = fluidml_hip_pad_view_copy(&a.t, before.data(), padded.data(), static_cast<int32_t>(before.size()), l.view_offset,
+                                     l.view_strides.data(), &out.t, ctx.stream);
+      break;
+    }
     case Launch::Kind::ReshapeTranspose: {
       // the Transpose's output buffer addressed by the Reshape's logical index
       const fl_tensor dst = Permuted(out.t, l.perm, true);

@@ -87,6 +87,9 @@ struct Launch {
     AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias
     ReshapeTranspose,  // Reshape -> Transpose, one strided copy
     TransposeReshape,  // Transpose -> Reshape, one strided copy
+    PadViewCopy,       // Pad -> steps that only re-address its result (Gather of sliding windows, Slice, Transpose,
+                       // Reshape): a = the Pad's input, `view_offset` / `view_strides` = the last step's output inside
+                       // the padded tensor (never written), out = the last step's output
     View,              // a Slice / Transpose / Squeeze / Unsqueeze / Reshape that is not run: its readers address
                        // the source through strides (members = {i}, out = the source operand seen as the view)
     Placed,            // a Concat2 that is not run: the launches producing its inputs wrote them into its output
@@ -116,6 +119,7 @@ struct Launch {
   // and the optional split of the last dim (see fluidml_hip_matmul_chain_view)
   std::vector<int64_t> view_strides;
   int64_t n_inner = 0, stride_outer = 0;
+  int64_t view_offset = 0;  // PadViewCopy
   // MatMulGroup: the grouped chains (members = union of theirs; every chain's `out` is written)
   std::vector<Launch> group;
   size_t position = 0;  // MatMulGroup: step index where the launch is issued (one of the members)

@@ -271,6 +271,12 @@ int fluidml_hip_concat2(const fl_tensor *lhs, const fl_tensor *rhs, const fl_ten
  * constant mode, value 0); with FL_REF_PAD_BORDER_UNWRITTEN only the interior
  * is written (reference pad.cpp:15-51). `pads_before[i]` per dimension. */
 int fluidml_hip_pad(const fl_tensor *in, const fl_tensor *out, const int64_t *pads_before, int32_t n, uint32_t flags, void *stream);
+/* PadKernel followed by kernels that only re-address its result (Gather with sliding-window indices, Slice,
+ * Transpose, Reshape, ...) as ONE copy (reference pad.cpp:15-51, gather.cpp, transpose.cpp, reshape.cpp): the padded
+ * tensor -- `in` with `pads_before[d]` zeros in front of dim d, extents `padded_shape`, dense row-major -- is never
+ * written; out[i0, i1, ..] is its element view_offset + sum(i_k * view_strides[k]), read from `in` when it lies in
+ * the interior and zero otherwise.  One view stride per dim of `out`; 4-byte element types. */
+int fluidml_hip_pad_view_copy(const fl_tensor *in, const int64_t *pads_before, const int64_t *padded_shape, int32_t n_dims, int64_t view_offset, const int64_t *view_strides, const fl_tensor *out, void *stream);
 /* GatherConstantIndexScalarKernel (reference gather.cpp:100-139). */
 int fluidml_hip_gather_constant_index_scalar(const fl_tensor *in, const fl_tensor *out, int64_t axis, int64_t index, uint32_t flags, void *stream);
 /* GatherConstantIndicesTensorKernel: data is the runtime input, `indices` a

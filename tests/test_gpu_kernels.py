@@ -333,6 +333,43 @@ def test_squeeze_unsqueeze_slice_concat_pad(device):
             assert_close(do.logical(), ho.logical(), exact=True, what=what)
 
 
+def test_pad_view_copy(device):
+    """Pad along the sequence -> Gather of sliding windows -> Transpose -> Reshape as one copy that reads the Pad's
+    input (the unfold of ConvBERT's span-based convolution), and a Pad on two dims seen through a Slice and a
+    Transpose; checked against numpy on the padded tensor."""
+    cabi = _cabi()
+    rng = np.random.default_rng(29)
+    # [1, S, C] padded by 4 on both sides of S, windows of 9 -> [1, S, 9, C] -> [1, S, C, 9] -> [S * H, C / H, 9]
+    S, C, H, K = 40, 96, 6, 9
+    x = rand(rng, (1, S, C))
+    padded = np.zeros((1, S + K - 1, C), np.float32)
+    padded[:, 4:4 + S] = x
+    windows = np.stack([padded[:, j:j + S] for j in range(K)], axis=2)  # [1, S, K, C]
+    want = np.transpose(windows, (0, 1, 3, 2)).reshape(S * H, C // H, K)
+    # strides of the result inside the padded tensor: row b = (s, h) -> s * C + h * (C / H) = b * (C / H)
+    strides = [C // H, 1, C]
+    dx = DeviceView(ok.View(x), device)
+    for lo in (None, [2, 0, 1]):
+        announce("pad_view_copy unfold", lo)
+        do = DeviceView(ok.View.empty(want.shape, np.float32, lo, fill=7), device)
+        cabi.call("pad_view_copy", dx.ref(), cabi.i64_array([0, 4, 0]), cabi.i64_array([1, S + K - 1, C]), 3, ctypes.c_int64(0),
+                  cabi.i64_array(strides), do.ref(), None)
+        assert_close(do.logical(), want, exact=True, what="pad_view_copy unfold")
+    # two padded dims, then Slice [1:, 2:9] and Transpose
+    y = rand(rng, (5, 7))
+    py = np.zeros((8, 12), np.float32)
+    py[2:7, 3:10] = y
+    want = py[1:, 2:9].T  # [7, 7]
+    dy = DeviceView(ok.View(y), device)
+    do = DeviceView(ok.View.empty(want.shape, np.float32, None, fill=7), device)
+    cabi.call("pad_view_copy", dy.ref(), cabi.i64_array([2, 3]), cabi.i64_array([8, 12]), 2, ctypes.c_int64(1 * 12 + 2),
+              cabi.i64_array([1, 12]), do.ref(), None)
+    assert_close(do.logical(), np.ascontiguousarray(want), exact=True, what="pad_view_copy slice + transpose")
+    # a view that leaves the padded tensor is refused
+    assert cabi.lib.fluidml_hip_pad_view_copy(dy.ref(), cabi.i64_array([2, 3]), cabi.i64_array([8, 12]), 2, 30, cabi.i64_array([1, 12]),
+                                              do.ref(), None) == -3  # FL_ERR_SHAPE
+
+
 def test_gathers(device):
     cabi = _cabi()
     rng = np.random.default_rng(34)

@@ -197,8 +197,10 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
     if (depthwise || flags != 0 || ns > 2) return FL_ERR_UNSUPPORTED;
     return ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, chain, bf16, stream, extras);
   }
-  if (!depthwise && flags == 0 && ns == 2 && !bf16) {
-    // 3x3, unit stride: the input patch is staged once per workgroup instead of gathered tap by tap
+  if (!depthwise && flags == 0 && ns == 2) {
+    // 3x3, unit stride: the input patch is staged once per workgroup instead of gathered tap by tap (fp32 also
+    // where bf16 operands are allowed: it is faster than the implicit GEMM on bf16 -- VGG-16 at batch 8: 2794
+    // against 2358 images/s)
     const int rc = ConvHalo3x3(in, weights, bias, out, pads, strides, dilations, chain, stream);
     if (rc != FL_ERR_UNSUPPORTED) return rc;
   }

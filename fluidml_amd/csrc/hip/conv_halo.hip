@@ -258,7 +258,9 @@ int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *
   // worth it when the pixel tiles are mostly full and there are enough workgroups to fill the chip
   // (14 x 14 images fill 77 % of their tiles: measured slower than the implicit-GEMM path, 113.7 against 107.9 us)
   const double fill = static_cast<double>(OH * OW) / static_cast<double>(p.tiles_h * kTH * p.tiles_w * kTW);
-  if (n_tiles > 0x7fffffff || n_tiles < 256 || fill < 0.8) return FL_ERR_UNSUPPORTED;
+  // (workgroups: 224 at batch 1 on 256 x 56 x 56 still win, 40.7 -> 30.3 us with 128 input channels and 56.7 -> 54.3
+  // with 256; 112 on 512 x 28 x 28 lose against the implicit GEMM with K split over workgroups, 60 -> 100 us)
+  if (n_tiles > 0x7fffffff || n_tiles < 192 || fill < 0.8) return FL_ERR_UNSUPPORTED;
   p.tiles_pix = static_cast<uint32_t>(tiles_pix);
   if (bias != nullptr) {
     p.bias = static_cast<const float *>(bias->base);

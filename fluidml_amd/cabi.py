@@ -160,6 +160,7 @@ SIGNATURES = {
     "fluidml_hip_gemm_chain": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _vp, _u32, _vp],
     "fluidml_hip_conv_chain": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _u32, _vp],
     "fluidml_hip_conv_chain_scale_add": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _T, _T, _u32, _vp],
+    "fluidml_hip_conv_chain_mean": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _T, _u32, _vp],
     "fluidml_hip_pointwise_conv_pair": [_T, _T, _T, _vp, _T, _T, _vp, _T, _vp],
     "fluidml_hip_softmax_matvec": [_T, _T, _T, _vp],
     "fluidml_hip_elementwise_chain": [_T, _T, _vp, _vp],

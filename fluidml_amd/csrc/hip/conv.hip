@@ -114,6 +114,127 @@ __global__ __launch_bounds__(kBlock) void ConvDirect(ConvArgs p, float *__restri
   out[ooff] = acc;
 }
 
+// ---- depthwise 2-d convolution, one workgroup per channel plane ----------------------------------------------
+// The kernel above gives every output element its own thread, which then walks its K x K window through global
+// memory.  For a depthwise convolution whose zero-padded input plane fits LDS a workgroup stages the plane of one
+// (image, channel) once and its threads compute that plane's outputs from there; taps are added in the same
+// (kh, kw) order.  Owning a whole plane, the workgroup can also deliver the mean of its outputs -- what a
+// ReduceMean over the spatial dims behind the convolution (a squeeze-and-excitation block) would compute.
+struct PlaneArgs {
+  int32_t H, W, OH, OW, stride, pad_h, pad_w, rows, pitch;  // rows x pitch floats are staged
+  int32_t sXn, sXc, sXh, sXw, sOn, sOc, sOh, sOw, sWc, sWh, sWw;
+  const float *bias;
+  int32_t sB;
+  float *mean;  // optional: [image, channel] -> mean of the plane's outputs
+  int32_t sMn, sMc;
+  float count;
+  FastDiv div_ow, div_pitch;
+  fl_ew_program chain;
+};
+
+template <int K>
+__global__ __launch_bounds__(kBlock) void ConvDepthwisePlaneKernel(PlaneArgs p, float *__restrict__ out,
+                                                                   const float *__restrict__ in,
+                                                                   const float *__restrict__ w) {
+  extern __shared__ __align__(16) float plane[];
+  __shared__ float partial[kBlock / kWave];
+  const int32_t c = blockIdx.x, n = blockIdx.y;
+  const int tid = threadIdx.x;
+  float wv[K * K];
+#pragma unroll
+  for (int t = 0; t < K * K; ++t) wv[t] = w[c * p.sWc + (t / K) * p.sWh + (t % K) * p.sWw];
+  const float bias = p.bias != nullptr ? p.bias[c * p.sB] : 0.0f;
+  const float *src = in + static_cast<int64_t>(n) * p.sXn + static_cast<int64_t>(c) * p.sXc;
+  const uint32_t n_stage = static_cast<uint32_t>(p.rows * p.pitch);
+  for (uint32_t i = tid; i < n_stage; i += kBlock) {
+    uint32_t r, cc;
+    p.div_pitch.DivMod(i, r, cc);
+    const int32_t ih = static_cast<int32_t>(r) - p.pad_h, iw = static_cast<int32_t>(cc) - p.pad_w;
+    const bool inside = static_cast<uint32_t>(ih) < static_cast<uint32_t>(p.H) && static_cast<uint32_t>(iw) < static_cast<uint32_t>(p.W);
+    plane[i] = inside ? src[ih * p.sXh + iw * p.sXw] : 0.0f;
+  }
+  __syncthreads();
+  float *dst = out + static_cast<int64_t>(n) * p.sOn + static_cast<int64_t>(c) * p.sOc;
+  const uint32_t n_out = static_cast<uint32_t>(p.OH * p.OW);
+  float sum = 0.0f;
+  for (uint32_t o = tid; o < n_out; o += kBlock) {
+    uint32_t oh, ow;
+    p.div_ow.DivMod(o, oh, ow);
+    const float *win = plane + static_cast<int32_t>(oh) * p.stride * p.pitch + static_cast<int32_t>(ow) * p.stride;
+    float acc = 0.0f;
+#pragma unroll
+    for (int kh = 0; kh < K; ++kh)
+#pragma unroll
+      for (int kw = 0; kw < K; ++kw) acc += win[kh * p.pitch + kw] * wv[kh * K + kw];
+    if (p.bias != nullptr) acc += bias;
+    if (p.chain.n != 0) acc = RunChain(p.chain, acc);
+    dst[static_cast<int32_t>(oh) * p.sOh + static_cast<int32_t>(ow) * p.sOw] = acc;
+    sum += acc;
+  }
+  if (p.mean != nullptr) {
+    sum = BlockReduce<kBlock / kWave>(sum, SumOp{}, partial);
+    if (tid == 0) p.mean[static_cast<int64_t>(n) * p.sMn + static_cast<int64_t>(c) * p.sMc] = sum / p.count;
+  }
+}
+
+// FL_ERR_UNSUPPORTED (nothing launched) when the convolution does not fit: the caller goes on to the kernel above.
+// `mean_out` (may be null): [N, C, 1, 1].
+int ConvDepthwisePlane(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
+                       const int64_t *pads, const int64_t *strides, const int64_t *dilations, const fl_ew_program *chain,
+                       const fl_tensor *mean_out, void *stream) {
+  static const bool on = [] {
+    const char *v = std::getenv("FLUIDML_CONV_PLANE");
+    return v == nullptr || std::strtol(v, nullptr, 10) != 0;
+  }();
+  if (!on || out->rank != 4) return FL_ERR_UNSUPPORTED;
+  const int64_t N = in->shape[0], C = in->shape[1], H = in->shape[2], W = in->shape[3];
+  const int64_t OH = out->shape[2], OW = out->shape[3], K = weights->shape[2];
+  if (weights->shape[3] != K || (K != 3 && K != 5)) return FL_ERR_UNSUPPORTED;
+  const int64_t st = strides ? strides[0] : 1;
+  if ((strides && strides[1] != st) || st < 1 || st > 2) return FL_ERR_UNSUPPORTED;
+  if (dilations && (dilations[0] != 1 || dilations[1] != 1)) return FL_ERR_UNSUPPORTED;
+  const int64_t ph = pads ? pads[0] : 0, pw = pads ? pads[1] : 0;
+  if (ph < 0 || pw < 0 || OH <= 0 || OW <= 0) return FL_ERR_UNSUPPORTED;
+  const int64_t rows = (OH - 1) * st + K, pitch = (OW - 1) * st + K;
+  // the plane has to be small and there have to be enough planes to fill the chip
+  // (measured on EfficientNet-B0 at batch 1: planes of 14 x 14 to 30 x 30 with 240 to 1152 channels 4.3-6.5 against
+  // 4.9-7.6 us for the kernel above plus 4 us for the separate mean; 144 planes of 60 x 60 11 against 8 us, 96 planes
+  // of 114 x 114 29 against 7 us: too few workgroups, each staging too much)
+  if (rows * pitch > 48 * 48 || N * C < 192 || N > 65535) return FL_ERR_UNSUPPORTED;
+  if (Numel(in) > 0x7fffffff || Numel(out) > 0x7fffffff) return FL_ERR_UNSUPPORTED;
+  PlaneArgs p;
+  std::memset(&p, 0, sizeof(p));
+  p.H = static_cast<int32_t>(H), p.W = static_cast<int32_t>(W), p.OH = static_cast<int32_t>(OH), p.OW = static_cast<int32_t>(OW);
+  p.stride = static_cast<int32_t>(st), p.pad_h = static_cast<int32_t>(ph), p.pad_w = static_cast<int32_t>(pw);
+  p.rows = static_cast<int32_t>(rows), p.pitch = static_cast<int32_t>(pitch);
+  p.sXn = static_cast<int32_t>(in->strides[0]), p.sXc = static_cast<int32_t>(in->strides[1]);
+  p.sXh = static_cast<int32_t>(in->strides[2]), p.sXw = static_cast<int32_t>(in->strides[3]);
+  p.sOn = static_cast<int32_t>(out->strides[0]), p.sOc = static_cast<int32_t>(out->strides[1]);
+  p.sOh = static_cast<int32_t>(out->strides[2]), p.sOw = static_cast<int32_t>(out->strides[3]);
+  p.sWc = static_cast<int32_t>(weights->strides[0]), p.sWh = static_cast<int32_t>(weights->strides[2]);
+  p.sWw = static_cast<int32_t>(weights->strides[3]);
+  if (bias != nullptr) {
+    p.bias = static_cast<const float *>(bias->base);
+    p.sB = static_cast<int32_t>(bias->strides[0]);
+  }
+  if (mean_out != nullptr) {
+    p.mean = static_cast<float *>(mean_out->base);
+    p.sMn = static_cast<int32_t>(mean_out->strides[0]);
+    p.sMc = static_cast<int32_t>(mean_out->strides[1]);
+  }
+  p.count = static_cast<float>(OH * OW);
+  p.div_ow = FastDiv(static_cast<uint32_t>(OW));
+  p.div_pitch = FastDiv(static_cast<uint32_t>(pitch));
+  if (chain != nullptr) p.chain = *chain;
+  const dim3 grid(static_cast<uint32_t>(C), static_cast<uint32_t>(N));
+  const size_t lds = static_cast<size_t>(rows * pitch) * sizeof(float);
+  float *o = static_cast<float *>(out->base);
+  const float *x = static_cast<const float *>(in->base), *wp = static_cast<const float *>(weights->base);
+  if (K == 3) FL_LAUNCH(ConvDepthwisePlaneKernel<3>, grid, dim3(kBlock), lds, AsStream(stream), p, o, x, wp);
+  else FL_LAUNCH(ConvDepthwisePlaneKernel<5>, grid, dim3(kBlock), lds, AsStream(stream), p, o, x, wp);
+  return LaunchStatus();
+}
+
 }  // namespace
 
 // matmul.hip
@@ -130,6 +251,16 @@ namespace {
 int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
          const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, uint32_t flags,
          void *stream, const fl_ew_program *chain = nullptr, const ConvExtras *extras = nullptr) {
+  const fl_tensor *mean_out = extras != nullptr ? extras->mean_out : nullptr;
+  if (mean_out != nullptr) {
+    FL_CHECK(CheckView(mean_out));
+    if (mean_out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+    if (mean_out->rank != out->rank || mean_out->shape[0] != out->shape[0] || mean_out->shape[1] != out->shape[1]) return FL_ERR_SHAPE;
+    for (int i = 2; i < mean_out->rank; ++i) {
+      if (mean_out->shape[i] != 1) return FL_ERR_SHAPE;
+    }
+    if (extras->channel_scale != nullptr || extras->addend != nullptr) return FL_ERR_UNSUPPORTED;
+  }
   if (extras != nullptr && extras->channel_scale == nullptr && extras->addend == nullptr) extras = nullptr;
   FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(in));
@@ -192,6 +323,19 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
     }
   }
   // dense contractions go to the matrix cores; depthwise, 3-d and literal-reference modes stay here
+  if (depthwise && flags == 0 && ns == 2) {
+    const int rc = ConvDepthwisePlane(in, weights, bias, out, pads, strides, dilations, chain, mean_out, stream);
+    if (rc != FL_ERR_UNSUPPORTED) return rc;
+  }
+  if (mean_out != nullptr) {
+    // no kernel delivers the mean with the result here: the convolution, then the reduction
+    ConvExtras none;
+    FL_CHECK(Conv(in, weights, bias, out, pads, strides, dilations, group, flags | (bf16 ? FL_CONTRACT_BF16 << FL_CONTRACT_SHIFT : 0u),
+                  stream, chain, &none));
+    int64_t axes[kMaxSpatial];
+    for (int d = 0; d < ns; ++d) axes[d] = 2 + d;
+    return fluidml_hip_reduce_mean(out, mean_out, axes, ns, stream);
+  }
   if (extras != nullptr) {
     // the extra operands exist in the matrix-core path only
     if (depthwise || flags != 0 || ns > 2) return FL_ERR_UNSUPPORTED;
@@ -527,6 +671,16 @@ int fluidml_hip_conv_chain_scale_add(const fl_tensor *in, const fl_tensor *weigh
   fl::ConvExtras extras;
   extras.channel_scale = channel_scale;
   extras.addend = addend;
+  return fl::Conv(in, weights, bias, out, pads, strides, dilations, group, (flags & FL_CONTRACT_BF16) << FL_CONTRACT_SHIFT, stream,
+                  chain, &extras);
+}
+
+int fluidml_hip_conv_chain_mean(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
+                                const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group,
+                                const fl_ew_program *chain, const fl_tensor *mean_out, uint32_t flags, void *stream) {
+  if (mean_out == nullptr) return FL_ERR_NULL;
+  fl::ConvExtras extras;
+  extras.mean_out = mean_out;
   return fl::Conv(in, weights, bias, out, pads, strides, dilations, group, (flags & FL_CONTRACT_BF16) << FL_CONTRACT_SHIFT, stream,
                   chain, &extras);
 }

@@ -86,6 +86,8 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
     } else if (l.kind == worker::Launch::Kind::Placed) {
       // a Concat2 whose inputs were written in place: nothing runs
     } else if (l.group.empty()) {
+      // (a launch with a second output writes the tensor its last member reads as well: the member before it)
+      if (l.has_out2 && l.members.size() >= 2) written.push_back(l.members[l.members.size() - 2]);
       written.push_back(l.members.back());
     }
     // a launch that writes into a part of another tensor (an input of a Concat2 placed in its output)

@@ -515,6 +515,7 @@ class Scheduler {
     for (const Launch &l : *fused) {
       const size_t pos = l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back();
       if (l.group.empty()) writes.push_back({pos, l.out, &l, 0});
+      if (l.has_out2) writes.push_back({pos, l.out2, &l, 0});
       for (const Launch &g : l.group) writes.push_back({pos, g.out, &l, 0});
     }
     std::vector<const Launch *> dissolved;  // copy launches both of whose steps became views
@@ -693,7 +694,7 @@ class Scheduler {
         if (!producer) continue;
         Launch *l = owner[*producer];
         if (l != nullptr) {
-          const bool plain_out = l->group.empty() && l->view_strides.empty() && SameTensor(l->out, x) && !l->out.viewed;
+          const bool plain_out = l->group.empty() && l->view_strides.empty() && SameTensor(l->out, x) && !l->out.viewed && !l->has_out2;
           const bool kind_ok = l->kind == Launch::Kind::MatMulChain || l->kind == Launch::Kind::GemmChain ||
                                l->kind == Launch::Kind::ConvChain || l->kind == Launch::Kind::ElementwiseChain ||
                                l->kind == Launch::Kind::DivAddSoftmax || l->kind == Launch::Kind::AddLayerNorm ||
@@ -962,6 +963,7 @@ class Scheduler {
     }
     if (l.kind == Launch::Kind::ConvChain) {
       if (auto wider = WithGateAndSkip(i, l)) return wider;
+      if (auto wider = WithMean(i, l)) return wider;
     }
     // longest variant whose late reads are safe: with the chain, then without it
     for (int attempt = 0; attempt < 2; ++attempt) {
@@ -1026,6 +1028,45 @@ class Scheduler {
       return l;
     }
     return std::nullopt;
+  }
+
+  // A depthwise 2-d convolution (with the chain already matched in `plain`) one of whose readers is the ReduceMean
+  // over both spatial dims (the squeeze of a squeeze-and-excitation block): the kernel that owns a whole channel
+  // plane per workgroup delivers the mean with the result.  The launch runs at the ReduceMean's position and writes
+  // both tensors, so every other reader of the result has to come after it.
+  std::optional<Launch> WithMean(size_t i, const Launch &plain) {
+    const Step &conv = steps_[i];
+    const auto &in_shape = conv.in0.meta.GetShape();
+    const auto &w_shape = conv.in1.meta.GetShape();
+    if (in_shape.size() != 4 || w_shape.size() != 4 || Attrs(i).group == 1 || Attrs(i).group != in_shape[1] || w_shape[1] != 1) return std::nullopt;
+    const size_t value = plain.members.back();
+    const Operand &result = steps_[value].out;
+    if (!Elidable(result) || !IsFloat(result)) return std::nullopt;
+    auto it = readers_.find(result.name);
+    if (it == readers_.end()) return std::nullopt;
+    std::optional<size_t> mean;
+    for (size_t r : it->second) {
+      if (Kind(r) != OpKind::ReduceMean || taken_[r] || r <= value) continue;
+      const flow::Attrs &at = Attrs(r);
+      std::vector<int64_t> axes(at.axes);
+      for (int64_t &ax : axes) ax = ax < 0 ? ax + 4 : ax;
+      std::sort(axes.begin(), axes.end());
+      if (at.keepdims && axes == std::vector<int64_t>{2, 3} && (!mean || r < *mean)) mean = r;
+    }
+    if (!mean) return std::nullopt;
+    for (size_t r : it->second) {
+      if (r != *mean && std::find(plain.members.begin(), plain.members.end(), r) == plain.members.end() && r < *mean) return std::nullopt;
+    }
+    Launch l = plain;
+    l.members.push_back(*mean);
+    l.out = result;
+    l.out2 = steps_[*mean].out;
+    l.has_out2 = true;
+    if (!IsFloat(l.out2) || !Elidable(l.out2)) return std::nullopt;
+    if (!Safe(l.members, {{i, l.a}, {i, l.b}}) || !OutputDisjoint(l.out, {&l.a, &l.b}) || !OutputDisjoint(l.out2, {&l.a, &l.b, &l.out})) return std::nullopt;
+    l.bytes = Bytes({&l.a, &l.b, &l.out}) + static_cast<double>(steps_[i].kernel->GetConstantBytes()) + static_cast<double>(l.out2.meta.GetSize());
+    l.flops = Flops(l.members);
+    return l;
   }
 
   static bool DefaultLayout(const Operand &o) {

@@ -292,6 +292,13 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       kernel::TensorView c;
       if (bias != nullptr) c = bias->View();
       const bool padded = steps_[l.owner].node->GetKind() == flow::OpKind::ConvWithPadding;
+      if (l.has_out2) {
+        const kernel::TensorView mean = ViewOf(Resolve(l.out2), l.out2);
+        rc = fluidml_hip_conv_chain_mean(&a.t, &b.t, bias ? &c.t : nullptr, &out.t, padded ? at.pads.data() : nullptr,
+                                         at.strides.data(), at.dilations.data(), at.group, &l.chain, &mean.t, contract_flags,
+                                         ctx.stream);
+        break;
+      }
       if (l.has_gate || l.has_skip) {
         kernel::TensorView gate, skip;
         if (l.has_gate) gate = ViewOf(Resolve(l.c), l.c);

@@ -67,7 +67,7 @@ struct Launch {
                        // [-> AddCommon(tensor) [-> AddCommon(tensor)]]
     GemmChain,         // GemmConstantWeightsBias -> elementwise chain
     ConvChain,         // [MulCommon(x, factor per channel) ->] Conv{With,Without}Padding -> elementwise chain
-                       // [-> AddCommon(tensor of the output's shape)]
+                       // [-> AddCommon(tensor of the output's shape)] | [+ ReduceMean over the spatial dims, second output]
     ConvPair,          // two pointwise convolutions on one-pixel tensors, each with its elementwise chain
                        // (squeeze-and-excitation): a = input, b = weights of `owner`, c = weights of `owner2`,
                        // `chain` follows the first, `chain2` the second
@@ -99,6 +99,10 @@ struct Launch {
   Kind kind = Kind::Step;
   std::vector<size_t> members;  // indices into the step list, ascending
   Operand a, b, c, d, e, out;   // external operands, role by kind (see fusion.cpp)
+  // ConvChain that also delivers the ReduceMean over the spatial dims of its result (the ReduceMean is the last
+  // member, `out` the tensor it reads, which is written too)
+  Operand out2;
+  bool has_out2 = false;
   double s0 = 0, s1 = 0, s2 = 0;
   int64_t axis = 0;
   std::vector<int64_t> perm;

@@ -396,6 +396,12 @@ int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const 
  * none) multiplies the input, each product rounded as the separate kernel rounds it; one image only.  `addend`
  * (NULL: none) has the shape and strides of `out`.  Anything else: FL_ERR_UNSUPPORTED, nothing launched. */
 int fluidml_hip_conv_chain_scale_add(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, const fl_ew_program *chain, const fl_tensor *channel_scale, const fl_tensor *addend, uint32_t flags, void *stream);
+/* Conv{With,Without}PaddingKernel -> elementwise chain -> ReduceMeanKernel over the spatial dims (keepdims) as ONE call
+ * with two results (reference conv.cpp:27-280, reduce_mean.cpp: the depthwise convolution of an inverted-residual
+ * block and the squeeze of its squeeze-and-excitation gate): `out` as for fluidml_hip_conv_chain, `mean_out`
+ * [N, F, 1, ..] its mean over the spatial dims.  One launch for a depthwise 3x3 or 5x5 convolution with stride 1 or 2
+ * whose padded input plane fits LDS (a workgroup per plane); otherwise the convolution, then the reduction. */
+int fluidml_hip_conv_chain_mean(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, const fl_ew_program *chain, const fl_tensor *mean_out, uint32_t flags, void *stream);
 /* SoftmaxKernel over K <= 16 logits [B, K, 1] -> MatMulKernel [B, M, K] x [B, K, 1] as ONE launch:
  * out[b, m, 0] = sum_k a[b, m, k] * softmax_k(logits[b, :, 0]) (reference softmax.cpp, matmul.cpp:28-59; the
  * per-position kernel of a span-based dynamic convolution).  `out` is [B, M, 1] with the element strides

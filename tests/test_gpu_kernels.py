@@ -1398,6 +1398,55 @@ def test_conv_scale_add(device):
                                                      cabi.i64_array([1, 1]), 1, ctypes.byref(none), sc.ref(), None, 0, None) == cabi.FL_ERR_UNSUPPORTED
 
 
+def test_conv_chain_mean(device):
+    """Convolution -> swish chain -> ReduceMean over the spatial dims with both results from one call: depthwise 3x3 and
+    5x5, strides 1 and 2 (one workgroup per plane), a channels-last input, and the shapes that take the two-launch
+    route (few planes, a dense convolution)."""
+    cabi = _cabi()
+    rng = np.random.default_rng(57)
+    swish = cabi.make_chain([(cabi.EW_DIV_C, 2.0), (cabi.EW_TANH, 0), (cabi.EW_ADD_C, 1.0), (cabi.EW_MUL_C, 0.5), (cabi.EW_MUL_X, 0)])
+    none = cabi.make_chain([])
+
+    def swish_ref(t):
+        u0, u1, u2, u3, u4 = (ok.View.empty(t.shape) for _ in range(5))
+        ok.unary_f32(ok.OP_DIV_C, t, u0, 2.0)
+        ok.unary_f32(ok.OP_TANH, u0, u1)
+        ok.unary_f32(ok.OP_ADD_C, u1, u2, 1.0)
+        ok.unary_f32(ok.OP_MUL_C, u2, u3, 0.5)
+        ok.binary_f32(ok.BOP_MUL, u3, t, u4)
+        return u4
+
+    cases = [((1, 144, 56, 56), 3, 1, 144, True, None),
+             ((1, 96, 57, 57), 3, 2, 96, True, None),
+             ((2, 120, 28, 28), 5, 1, 120, True, [0, 2, 3, 1]),
+             ((1, 240, 29, 31), 5, 2, 240, False, None),
+             ((1, 32, 20, 20), 3, 1, 32, True, None),    # few planes: convolution, then reduction
+             ((2, 8, 12, 12), 3, 1, 1, True, None)]      # dense convolution: the same
+    for xshape, k, st, group, with_chain, li in cases:
+        filters = xshape[1] if group != 1 else 16
+        wshape = (filters, 1 if group != 1 else xshape[1], k, k)
+        pads = [k // 2] * 4
+        od = tuple((xshape[2 + d] + 2 * (k // 2) - k) // st + 1 for d in range(2))
+        oshape = (xshape[0], filters) + od
+        x, w, bias = rand(rng, xshape, -1, 1), rand(rng, wshape, -0.3, 0.3), rand(rng, (filters,), -1, 1)
+        announce("conv_chain_mean", xshape, wshape, st, li)
+        hx = ok.View.empty(xshape, np.float32, li)
+        hx.logical()[...] = x
+        t = ok.View.empty(oshape)
+        ok.conv(hx, ok.View(w), ok.View(bias), t, pads, [st, st], [1, 1], group, 0)
+        want = swish_ref(t) if with_chain else t
+        want_mean = ok.View.empty((xshape[0], filters, 1, 1))
+        ok.reduce_mean(want, want_mean, [2, 3])
+        dx, dw, db = DeviceView(hx, device), DeviceView(ok.View(w), device), DeviceView(ok.View(bias), device)
+        do = DeviceView(ok.View.empty(oshape, fill=7), device)
+        dm = DeviceView(ok.View.empty((xshape[0], filters, 1, 1), fill=7), device)
+        cabi.call("conv_chain_mean", dx.ref(), dw.ref(), db.ref(), do.ref(), cabi.i64_array(pads), cabi.i64_array([st, st]),
+                  cabi.i64_array([1, 1]), ctypes.c_int64(group), ctypes.byref(swish if with_chain else none), dm.ref(),
+                  ctypes.c_uint32(0), None)
+        assert_close(do.logical(), want.logical(), what="conv_chain_mean: result")
+        assert_close(dm.logical(), want_mean.logical(), what="conv_chain_mean: mean")
+
+
 def test_argument_errors(device):
     """Rejected arguments return negative codes and launch nothing."""
     cabi = _cabi()

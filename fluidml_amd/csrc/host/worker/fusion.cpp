@@ -1312,7 +1312,7 @@ class Scheduler {
       return SameTensor(x.a, y.a) && x.a.layout == y.a.layout && batch == 1 && shape == hy.out.meta.GetShape() &&
              x.b.space == Operand::Space::Constant && y.b.space == Operand::Space::Constant &&
              x.b.meta.GetShape() == y.b.meta.GetShape() && x.b.layout == y.b.layout && x.has_c == y.has_c &&
-             InnerCompatible(x, y, shape.back()) && x.view_strides.empty() == y.view_strides.empty() && x.chain.n == y.chain.n &&
+             InnerCompatible(x, y, shape.back()) && x.chain.n == y.chain.n &&
              std::equal(x.chain.op, x.chain.op + x.chain.n, y.chain.op) &&
              std::equal(x.chain.c, x.chain.c + x.chain.n, y.chain.c);
     };
@@ -1361,7 +1361,7 @@ class Scheduler {
         Launch &added = g.group.back();
         if (added.n_inner == 0 && inner != 0) {
           added.n_inner = inner;
-          added.stride_outer = inner * added.view_strides.back();
+          added.stride_outer = inner * (added.view_strides.empty() ? LogicalStrides(added.out).back() : added.view_strides.back());
         }
       }
       std::sort(g.members.begin(), g.members.end());
@@ -1380,7 +1380,7 @@ class Scheduler {
     if (x.n_inner == y.n_inner) return true;
     if (x.n_inner != 0 && y.n_inner != 0) return false;
     const int64_t inner = x.n_inner != 0 ? x.n_inner : y.n_inner;
-    return !x.view_strides.empty() && !y.view_strides.empty() && columns % inner == 0;
+    return columns % inner == 0;  // (a member without folded views writes its own output: one run per row as well)
   }
 
   // Can every launch of `set` be issued at step position `position` (the last member of one of them)?

@@ -313,6 +313,22 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
     bias_col[j] = bias_by_col && n < p.N ? bias[n * p.sDn] : 0.0f;
   }
 
+  // So are the tensors added after the chain, where a lane finishes few enough values (the quartered tail: the
+  // four it will store).  Only the consumer waves of the last K split use them; the others' loads are dropped.
+  constexpr bool PRE_ADD = EXTRA != 0 && QUARTER;
+  float pre_add[PRE_ADD ? EV : 1], pre_add2[PRE_ADD ? EV : 1];
+  if constexpr (PRE_ADD) {
+    const int n = n0 + lrow;
+#pragma unroll
+    for (int e = 0; e < EV; ++e) {
+      const int m = m0 + ks * 8 + half * 4 + e;
+      const bool inside = !producer && m < p.M && n < p.N;
+      const int64_t at = boff[0] + static_cast<int64_t>(m) * sCm + static_cast<int64_t>(n) * sCn;
+      pre_add[e] = p.addend != nullptr && inside ? p.addend[at] : 0.0f;
+      pre_add2[e] = p.addend2 != nullptr && inside ? p.addend2[at] : 0.0f;
+    }
+  }
+
   // DEPTH chunks are in flight in registers: the loads of chunk c+DEPTH are issued while chunk c is
   // consumed, so a workgroup keeps DEPTH * (A tile + B tile) bytes outstanding instead of one chunk --
   // with only a few workgroups per CU that is what hides the L2/HBM latency.
@@ -678,10 +694,15 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
           float add[EV], add2[EV];
 #pragma unroll
           for (int e = 0; e < EV; ++e) {
-            const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
-            const bool inside = m < p.M && n < p.N;
-            add[e] = inside ? Eb[static_cast<int64_t>(m) * sCm + col] : 0.0f;
-            add2[e] = Eb2 != nullptr && inside ? Eb2[static_cast<int64_t>(m) * sCm + col] : 0.0f;
+            if constexpr (PRE_ADD) {
+              add[e] = pre_add[e];
+              add2[e] = pre_add2[e];
+            } else {
+              const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
+              const bool inside = m < p.M && n < p.N;
+              add[e] = inside ? Eb[static_cast<int64_t>(m) * sCm + col] : 0.0f;
+              add2[e] = Eb2 != nullptr && inside ? Eb2[static_cast<int64_t>(m) * sCm + col] : 0.0f;
+            }
           }
 #pragma unroll
           for (int e = 0; e < EV; ++e) vals[e] += add[e];

@@ -553,6 +553,41 @@ __global__ __launch_bounds__(kPairBlock) void ConvPairKernel(ConvPairArgs p, flo
   out[static_cast<int64_t>(image) * p.out_n + static_cast<int64_t>(f) * p.out_f] = acc;
 }
 
+// One of the two convolutions above on its own, for the case where the weights are too many for one or two compute
+// units to pull in reasonable time (1152 channels x 48 hidden values: 440 KB, 15 us in the kernel above): LANES lanes
+// (64 or 16) share an output, walk its weight row 128 bits at a time and add their sums with shuffles, so that the rows
+// spread over hundreds of waves; the hidden vector then travels through the stream's workspace between two launches.
+template <int LANES>
+__global__ __launch_bounds__(kBlock) void PointwiseOnePixelKernel(int32_t channels, int32_t outputs, int32_t in_n, int32_t in_c,
+                                                                  int32_t out_n, int32_t out_f, int32_t w_f, int32_t w_c,
+                                                                  int32_t b_stride, int32_t vec, fl_ew_program chain,
+                                                                  float *__restrict__ out, const float *__restrict__ in,
+                                                                  const float *__restrict__ w, const float *__restrict__ b) {
+  constexpr int kRows = kBlock / LANES;
+  const int image = blockIdx.y;
+  const int f = blockIdx.x * kRows + threadIdx.x / LANES, lane = threadIdx.x % LANES;
+  const bool live = f < outputs;
+  const float *row = w + static_cast<int64_t>(live ? f : 0) * w_f;
+  const float *x = in + static_cast<int64_t>(image) * in_n;
+  float acc = 0.0f;
+  if (vec) {
+    for (int q = lane; q < channels / 4; q += LANES) {
+      const PairQuad wv = reinterpret_cast<const PairQuad *>(row)[q], xv = reinterpret_cast<const PairQuad *>(x)[q];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc += wv.v[e] * xv.v[e];
+    }
+  } else {
+    for (int c = lane; c < channels; c += LANES) acc += row[c * w_c] * x[c * in_c];
+  }
+#pragma unroll
+  for (int off = LANES / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+  if (live && lane == 0) {
+    if (b != nullptr) acc += b[f * b_stride];
+    if (chain.n != 0) acc = RunChain(chain, acc);
+    out[static_cast<int64_t>(image) * out_n + static_cast<int64_t>(f) * out_f] = acc;
+  }
+}
+
 // [N, C, 1...] tensors: every dim from the third on has extent 1
 inline bool OnePixel(const fl_tensor *t) {
   if (t->rank < 2) return false;
@@ -603,6 +638,26 @@ int ConvPair(const fl_tensor *in, const fl_tensor *w1, const fl_tensor *b1, cons
   if (p.chain1.n > FL_EW_MAX_STEPS || p.chain2.n > FL_EW_MAX_STEPS) return FL_ERR_ATTR;
   p.vec1 = c % 4 == 0 && p.w1_c == 1 && p.w1_s % 4 == 0 && IsAligned(w1->base, 16) ? 1 : 0;
   p.vec2 = s % 4 == 0 && p.w2_s == 1 && p.w2_f % 4 == 0 && IsAligned(w2->base, 16) ? 1 : 0;
+  // Many weights: two launches over many waves each, the hidden vector in the stream's workspace in between
+  // (EfficientNet-B0's last blocks, 1152 x 48: 15 us in one launch).
+  if ((c * s + s * f) * 4 >= (256 << 10) && n * s <= static_cast<int64_t>(kWorkspaceTiles * kWorkspaceTileFloats)) {
+    if (StreamWorkspace *ws = GetStreamWorkspace(AsStream(stream))) {
+      float *hidden = ws->partials;
+      const int32_t hn = static_cast<int32_t>(s);
+      const bool x_vec = p.vec1 && p.in_c == 1 && p.in_n % 4 == 0 && IsAligned(in->base, 16);
+      const bool h_vec = p.vec2 && s % 4 == 0;
+      const fl_ew_program none{};
+      FL_LAUNCH(PointwiseOnePixelKernel<64>, dim3(static_cast<uint32_t>((s + 3) / 4), static_cast<uint32_t>(n)), dim3(kBlock), 0,
+                AsStream(stream), p.channels, p.hidden, p.in_n, p.in_c, hn, 1, p.w1_s, p.w1_c, p.b1_stride, x_vec ? 1 : 0,
+                chain1 ? *chain1 : none, hidden, static_cast<const float *>(in->base), static_cast<const float *>(w1->base),
+                b1 ? static_cast<const float *>(b1->base) : nullptr);
+      FL_LAUNCH(PointwiseOnePixelKernel<16>, dim3(static_cast<uint32_t>((f + 15) / 16), static_cast<uint32_t>(n)), dim3(kBlock), 0,
+                AsStream(stream), p.hidden, p.outputs, hn, 1, p.out_n, p.out_f, p.w2_f, p.w2_s, p.b2_stride, h_vec ? 1 : 0,
+                chain2 ? *chain2 : none, static_cast<float *>(out->base), hidden, static_cast<const float *>(w2->base),
+                b2 ? static_cast<const float *>(b2->base) : nullptr);
+      return LaunchStatus();
+    }
+  }
   const dim3 grid(static_cast<uint32_t>((f + kPairBlock - 1) / kPairBlock), static_cast<uint32_t>(n));
 #define FL_CONV_PAIR(QUADS, ROWS)                                                                                  \
   FL_LAUNCH((ConvPairKernel<QUADS, ROWS>), grid, dim3(kPairBlock), 0, AsStream(stream), p, static_cast<float *>(out->base), \

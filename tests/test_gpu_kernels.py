@@ -882,7 +882,8 @@ def test_fused_pointwise_conv_pair(device):
         return cur
 
     for n, c, hidden, f, with_bias in [(1, 96, 4, 96, True), (2, 1152, 48, 1152, True), (3, 40, 10, 300, False),
-                                          (1, 2600, 6, 1030, True), (2, 37, 5, 9, True)]:
+                                          (1, 2600, 6, 1030, True), (2, 37, 5, 9, True),
+                                          (1, 1154, 50, 1201, True)]:  # many weights, rows not 16-byte aligned: two launches
         announce("pointwise_conv_pair", n, c, hidden, f, with_bias)
         x = rand(rng, (n, c, 1, 1))
         w1, w2 = rand(rng, (hidden, c, 1, 1), -0.2, 0.2), rand(rng, (f, hidden, 1, 1), -0.5, 0.5)

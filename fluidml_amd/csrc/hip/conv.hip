@@ -640,7 +640,11 @@ int ConvPair(const fl_tensor *in, const fl_tensor *w1, const fl_tensor *b1, cons
   p.vec2 = s % 4 == 0 && p.w2_s == 1 && p.w2_f % 4 == 0 && IsAligned(w2->base, 16) ? 1 : 0;
   // Many weights: two launches over many waves each, the hidden vector in the stream's workspace in between
   // (EfficientNet-B0's last blocks, 1152 x 48: 15 us in one launch).
-  if ((c * s + s * f) * 4 >= (256 << 10) && n * s <= static_cast<int64_t>(kWorkspaceTiles * kWorkspaceTileFloats)) {
+  static const int64_t split_bytes = [] {
+    const char *v = std::getenv("FLUIDML_PAIR_SPLIT_KB");
+    return (v != nullptr ? std::strtol(v, nullptr, 10) : 64) * int64_t{1024};
+  }();
+  if ((c * s + s * f) * 4 >= split_bytes && n * s <= static_cast<int64_t>(kWorkspaceTiles * kWorkspaceTileFloats)) {
     if (StreamWorkspace *ws = GetStreamWorkspace(AsStream(stream))) {
       float *hidden = ws->partials;
       const int32_t hn = static_cast<int32_t>(s);

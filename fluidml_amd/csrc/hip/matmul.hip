@@ -218,14 +218,17 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   constexpr int LDS_ELEMS = STAGE_ELEMS > RED_ELEMS ? STAGE_ELEMS : RED_ELEMS;
   __shared__ __attribute__((aligned(16))) float lds[LDS_ELEMS];
 
-  constexpr int VB = CONV == 2 ? 4 : CONV == 1 ? 1 : VEC;
+  // VEC: floats per global load of both operands' tiles; 41 = four for A and one for B (rows of B that do not keep
+  // 16-byte alignment, a 7x7 image's 49 pixels, under weights that do)
+  constexpr int VA = VEC == 41 ? 4 : VEC;
+  constexpr int VB = CONV == 2 ? 4 : CONV == 1 || VEC == 41 ? 1 : VEC;
   static_assert(!CONV || (LB == 0 && NT % (BN / VB) == 0), "the gather keeps one output pixel (group) per thread");
   static_assert(!SPEC || !CONV, "the gather of the convolution runs in the consumer waves");
   // EXTRA: 0 = none, 1 = addends in the epilogue, 2 = addends and a scale per row of B
   static_assert(EXTRA == 0 || (LB == 0 && CONV == 0), "the extra operands exist for plain contractions with B kept [k][n]");
   const bool producer = SPEC && threadIdx.x >= NT;
   const int ltid = producer ? static_cast<int>(threadIdx.x) - NT : static_cast<int>(threadIdx.x);
-  using LoaderA = typename std::conditional<LA == 0, TileLoader<BM, BK, VEC, NT>, TileLoader<BK, BM, VEC, NT>>::type;
+  using LoaderA = typename std::conditional<LA == 0, TileLoader<BM, BK, VA, NT>, TileLoader<BK, BM, VA, NT>>::type;
   using LoaderB = typename std::conditional<LB == 0, TileLoader<BK, BN, VB, NT>, TileLoader<BN, BK, VB, NT>>::type;
 
   // Request every argument the kernel is going to read in one batch and wait for them once: left to itself the
@@ -333,7 +336,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   // consumed, so a workgroup keeps DEPTH * (A tile + B tile) bytes outstanding instead of one chunk --
   // with only a few workgroups per CU that is what hides the L2/HBM latency.
   static_assert(DEPTH % 2 == 0, "the LDS buffer index must be a compile-time function of the stage");
-  VecF<VEC> ra[DEPTH][LoaderA::kPerThread];
+  VecF<VA> ra[DEPTH][LoaderA::kPerThread];
   VecF<VB> rb[DEPTH][LoaderB::kPerThread];
   float rs[DEPTH][LoaderB::kPerThread];  // EXTRA == 2: the scale of the row each item of the B tile belongs to
   const int rows_m = p.M - m0, cols_n = p.N - n0;
@@ -353,7 +356,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
     g_base = static_cast<int32_t>(img) * p.conv.sXn;
   }
 
-  auto load_chunk = [&](int c, VecF<VEC>(&qa)[LoaderA::kPerThread], VecF<VB>(&qb)[LoaderB::kPerThread],
+  auto load_chunk = [&](int c, VecF<VA>(&qa)[LoaderA::kPerThread], VecF<VB>(&qb)[LoaderB::kPerThread],
                         float(&qs)[LoaderB::kPerThread]) {
     const int k0 = c * BK, k_valid = p.K - k0;
     if constexpr (EXTRA == 2) {
@@ -412,7 +415,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
       LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBn, p.sBk, cols_n, k_valid, qb, ltid);
     }
   };
-  auto store_chunk = [&](int buf, const VecF<VEC>(&qa)[LoaderA::kPerThread], const VecF<VB>(&qb)[LoaderB::kPerThread],
+  auto store_chunk = [&](int buf, const VecF<VA>(&qa)[LoaderA::kPerThread], const VecF<VB>(&qb)[LoaderB::kPerThread],
                          const float(&qs)[LoaderB::kPerThread]) {
     float *as = lds + buf * (A_ELEMS + B_ELEMS);
     float *bs = as + A_ELEMS;
@@ -967,11 +970,16 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
     // partial tiles costs more than the extra workgroups bring.  One workspace slot per wave and split.
     const int64_t tiles = static_cast<int64_t>(q.tiles_m) * q.tiles_n * n_batch;
     const int64_t n_chunks = (p.K + BK - 1) / BK;
-    const int64_t min_chunks = 384 / BK;  // at least 384 values of k per split
+    // At most 40 tiles (pointwise convolutions over 7x7 and 14x14 images: 12 .. 28 tiles, K = 480 .. 1152): every
+    // chunk of 128 to a workgroup of its own, up to 16 per tile -- the launch is a chain of round trips to memory and
+    // each chunk a workgroup runs after its first two adds one (EfficientNet-B0 +2.3 %; limits of 8 and 32 and bounds
+    // of 28 and 56 tiles within 0.3 % of that).
+    const bool few = tiles <= 40 && WM * WN == 1;
+    const int64_t min_chunks = few ? std::max(1, 128 / BK) : 384 / BK;  // at least 384 values of k per split otherwise
     int64_t want = std::min<int64_t>(n_chunks / min_chunks, static_cast<int64_t>(kWorkspaceTiles) / (tiles * WM * WN));
     // (64x64 tile, 3x3 convolutions on 14x14 and 28x28 images at batch 1, K = 4608: 8 -> 12 splits 36 -> 33.5 us and
     // 66 -> 61 us)
-    want = std::min<int64_t>(want, SplitKLimit(WM * WN == 1 ? 4 : 16));
+    want = std::min<int64_t>(want, SplitKLimit(few ? 16 : WM * WN == 1 ? 4 : 16));
     if (tiles > 256) want = 1;
     if (want >= 2) {
       if (WorkspaceOverride *fixed = t_workspace_override) {
@@ -1158,14 +1166,18 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   // 16-byte alignment.
   const int la = (p.sAk <= p.sAm || p.M == 1) ? 0 : 1;
   const int lb = (p.sBn <= p.sBk || p.K == 1) ? 0 : 1;
-  bool vec = IsAligned(A, 16) && IsAligned(B, 16) && siblings_aligned;
-  if (la == 0) vec = vec && (p.sAk == 1 || p.K == 1) && p.K % 4 == 0 && p.sAm % 4 == 0;
-  else vec = vec && p.sAm == 1 && p.M % 4 == 0 && p.sAk % 4 == 0;
-  if (lb == 0) vec = vec && (p.sBn == 1 || p.N == 1) && p.N % 4 == 0 && p.sBk % 4 == 0;
-  else vec = vec && p.sBk == 1 && p.K % 4 == 0 && p.sBn % 4 == 0;
-  for (int i = 0; i < nest.rank && vec; ++i) {
-    if (nest.strides[1][i] % 4 != 0 || nest.strides[2][i] % 4 != 0) vec = false;
+  bool vec_a = IsAligned(A, 16), vec_b = IsAligned(B, 16) && siblings_aligned;
+  if (la == 0) vec_a = vec_a && (p.sAk == 1 || p.K == 1) && p.K % 4 == 0 && p.sAm % 4 == 0;
+  else vec_a = vec_a && p.sAm == 1 && p.M % 4 == 0 && p.sAk % 4 == 0;
+  if (lb == 0) vec_b = vec_b && (p.sBn == 1 || p.N == 1) && p.N % 4 == 0 && p.sBk % 4 == 0;
+  else vec_b = vec_b && p.sBk == 1 && p.K % 4 == 0 && p.sBn % 4 == 0;
+  for (int i = 0; i < nest.rank; ++i) {
+    if (nest.strides[1][i] % 4 != 0) vec_a = false;
+    if (nest.strides[2][i] % 4 != 0) vec_b = false;
   }
+  const bool vec = vec_a && vec_b;
+  // k-contiguous weights over an operand whose rows lose the alignment (49 pixels): wide loads for the weights alone
+  const bool vec_a_only = vec_a && !vec_b && la == 0 && lb == 0 && !bf16;
   // a second addend with the strides of C / a scale per row of B: the tiled kernel's own instantiations (fp32)
   const bool extra = addend != nullptr || k_scale != nullptr;
   if (extra) {
@@ -1185,6 +1197,7 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
 #define FL_MM_EXTRA(E_)                                                     \
   do {                                                                      \
     if (la == 0 && vec) LaunchBySize<0, 0, 4, 0, false, E_>(p, nb, C, A, B, s);  \
+    else if (vec_a_only) LaunchBySize<0, 0, 41, 0, false, E_>(p, nb, C, A, B, s); \
     else if (la == 0) LaunchBySize<0, 0, 1, 0, false, E_>(p, nb, C, A, B, s);    \
     else if (vec) LaunchBySize<1, 0, 4, 0, false, E_>(p, nb, C, A, B, s);        \
     else LaunchBySize<1, 0, 1, 0, false, E_>(p, nb, C, A, B, s);                 \
@@ -1204,6 +1217,10 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
     } else {                                                      \
       LaunchBySize<LA_, LB_, 1, 0>(p, nb, C, A, B, s);        \
     }                                                             \
+  }
+  if (vec_a_only) {
+    LaunchBySize<0, 0, 41, 0>(p, nb, C, A, B, s);
+    return LaunchStatus();
   }
   FL_MM_DISPATCH(0, 0)
   FL_MM_DISPATCH(0, 1)

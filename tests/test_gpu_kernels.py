@@ -583,6 +583,9 @@ MATMUL_CASES = [
     ((5, 7), (7, 3)),
     ((1, 130, 70), (70, 258)),  # tile edges
     ((64, 6), (6, 64)),  # K not a multiple of 4
+    ((192, 1152), (1152, 49)),  # wide loads for the left operand only, K split over workgroups
+    ((900, 64), (64, 1001)),  # the same on the 64x64 tile
+    ((64, 1000), (1000, 40)),  # four tiles, a workgroup per chunk of K, the last chunk ragged
 ]
 
 
@@ -765,7 +768,8 @@ def test_matmul_chain_add(device):
     for ashape, bshape, lo, two, with_chain in [((1, 256, 512), (512, 512), None, True, False),
                                                 ((1, 128, 768), (768, 768), None, False, False),
                                                 ((2, 3, 70, 40), (40, 96), None, True, True),
-                                                ((1, 300, 256), (256, 1024), [0, 2, 1], True, False)]:
+                                                ((1, 300, 256), (256, 1024), [0, 2, 1], True, False),
+                                                ((1, 80, 256), (256, 49), None, True, False)]:  # rows of B unaligned
         a, b = rand(rng, ashape, -1, 1), rand(rng, bshape, -0.05, 0.05)
         oshape = ashape[:-1] + (bshape[-1],)
         bias, r1, r2 = rand(rng, (bshape[-1],), -0.5, 0.5), rand(rng, oshape, -1, 1), rand(rng, oshape, -1, 1)
@@ -1361,7 +1365,8 @@ def test_conv_scale_add(device):
     cases = [((1, 96, 28, 28), 40, 1, True, True, False, None),      # small tile, gate and skip connection
              ((1, 240, 56, 56), 80, 1, True, False, True, None),     # 64x64 tile, gate, ReLU
              ((1, 37, 9, 11), 50, 1, True, True, False, None),       # ragged extents, scalar loads
-             ((2, 64, 20, 20), 64, 1, False, True, True, None)]      # two images, skip connection
+             ((2, 64, 20, 20), 64, 1, False, True, True, None),      # two images, skip connection
+             ((1, 1152, 7, 7), 192, 1, True, True, False, None)]     # 49 pixels: wide loads for the weights alone
     for xshape, filters, k, gate, skip, with_chain, lo in cases:
         pads = [k // 2] * 4
         wshape = (filters, xshape[1], k, k)

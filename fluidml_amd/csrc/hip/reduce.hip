@@ -645,6 +645,9 @@ struct SoftmaxMatVecArgs {
   FastDiv div_rows;
   int32_t k;
   int32_t a_b, a_m, a_k, v_b, v_k, out_b, out_m;  // element strides
+  // the output's batch dim in two parts: batch b lies at (b / inner) * out_outer + (b % inner) * out_b
+  FastDiv div_inner;
+  int32_t out_outer;
 };
 
 __global__ __launch_bounds__(kBlock) void SoftmaxMatVecKernel(SoftmaxMatVecArgs p, float *__restrict__ out,
@@ -672,7 +675,9 @@ __global__ __launch_bounds__(kBlock) void SoftmaxMatVecKernel(SoftmaxMatVecArgs 
   float acc = 0.0f;
 #pragma unroll
   for (int t = 0; t < kMatVecMaxK; ++t) acc += w[t] * (x[t] / sum);
-  out[static_cast<int64_t>(b) * p.out_b + static_cast<int64_t>(m) * p.out_m] = acc;
+  uint32_t b_outer, b_inner;
+  p.div_inner.DivMod(b, b_outer, b_inner);
+  out[static_cast<int64_t>(b_outer) * p.out_outer + static_cast<int64_t>(b_inner) * p.out_b + static_cast<int64_t>(m) * p.out_m] = acc;
 }
 
 }  // namespace
@@ -959,10 +964,12 @@ int fluidml_hip_softmax_matvec(const fl_tensor *a, const fl_tensor *logits, cons
   FL_CHECK(CheckView(logits));
   FL_CHECK(CheckView(out));
   if (a->dtype != FL_FLOAT32 || logits->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
-  if (a->rank != 3 || logits->rank != 3 || out->rank != 3) return FL_ERR_RANK;
+  if (a->rank != 3 || logits->rank != 3 || (out->rank != 3 && out->rank != 4)) return FL_ERR_RANK;
   const int64_t batch = a->shape[0], rows = a->shape[1], k = a->shape[2];
-  if (logits->shape[0] != batch || logits->shape[1] != k || logits->shape[2] != 1 || out->shape[0] != batch ||
-      out->shape[1] != rows || out->shape[2] != 1) {
+  const int split = out->rank - 3;  // 1: out is [outer, inner, rows, 1] with outer * inner batches
+  const int64_t out_batch = split ? out->shape[0] * out->shape[1] : out->shape[0];
+  if (logits->shape[0] != batch || logits->shape[1] != k || logits->shape[2] != 1 || out_batch != batch ||
+      out->shape[split + 1] != rows || out->shape[split + 2] != 1 || (split && out->shape[1] < 1)) {
     return FL_ERR_SHAPE;
   }
   if (k > kMatVecMaxK) return FL_ERR_UNSUPPORTED;
@@ -976,8 +983,10 @@ int fluidml_hip_softmax_matvec(const fl_tensor *a, const fl_tensor *logits, cons
   p.a_k = static_cast<int32_t>(a->strides[2]);
   p.v_b = static_cast<int32_t>(logits->strides[0]);
   p.v_k = static_cast<int32_t>(logits->strides[1]);
-  p.out_b = static_cast<int32_t>(out->strides[0]);
-  p.out_m = static_cast<int32_t>(out->strides[1]);
+  p.out_b = static_cast<int32_t>(out->strides[split]);
+  p.out_m = static_cast<int32_t>(out->strides[split + 1]);
+  p.div_inner = FastDiv(static_cast<uint32_t>(split ? out->shape[1] : batch > 0 ? batch : 1));
+  p.out_outer = split ? static_cast<int32_t>(out->strides[0]) : 0;
   FL_LAUNCH(SoftmaxMatVecKernel, dim3((p.n_items + kBlock - 1) / kBlock), dim3(kBlock), 0, AsStream(stream), p,
             static_cast<float *>(out->base), static_cast<const float *>(a->base), static_cast<const float *>(logits->base));
   return LaunchStatus();

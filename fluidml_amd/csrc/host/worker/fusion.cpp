@@ -129,12 +129,13 @@ class ViewTracker {
 
   struct View {
     std::vector<int64_t> strides;  // per source dim
-    int64_t n_inner = 0, stride_outer = 0;  // split of the last source dim, if any
+    int64_t n_inner = 0, stride_outer = 0;  // split of the one source dim that may be split, if any
   };
 
   // Strides of the source dims inside a tensor of the current shape stored with `strides`.  Every source dim
-  // must come out as one stride, except the last one which may be two (outer, inner).
-  std::optional<View> Resolve(const std::vector<int64_t> &strides) const {
+  // must come out as one stride, except one (`split_dim`; negative: the last) which may be two (outer, inner).
+  std::optional<View> Resolve(const std::vector<int64_t> &strides, int split_dim = -1) const {
+    const size_t may_split = split_dim < 0 ? n_source_dims_ - 1 : static_cast<size_t>(split_dim);
     if (strides.size() != dims_.size()) return std::nullopt;
     std::vector<int64_t> atom_stride(atoms_.size(), 0);
     for (size_t d = 0; d < dims_.size(); ++d) {
@@ -164,7 +165,7 @@ class ViewTracker {
       if (parts.empty()) continue;
       if (parts.size() == 1) {
         v.strides[d] = parts[0].second;
-      } else if (parts.size() == 2 && d + 1 == n_source_dims_) {
+      } else if (parts.size() == 2 && d == may_split) {
         v.stride_outer = parts[0].second;
         v.n_inner = parts[1].first;
         v.strides[d] = parts[1].second;
@@ -275,6 +276,7 @@ class Scheduler {
     }
     if (fuse) ElideViews(&fused);
     if (fuse) RetryAttention(&fused);
+    if (fuse) RetrySoftmaxMatVec(&fused);
     if (fuse) PlaceConcatInputs(&fused);
     // a chain is issued where its last member stood; everything else keeps its place
     std::vector<const Launch *> at(steps_.size(), nullptr);
@@ -642,7 +644,8 @@ class Scheduler {
   // The launch that produces an input of a Concat2 can write it straight into its part of the Concat2's output
   // (every kernel takes output strides), provided nobody else reads the input, and the output's bytes -- which
   // the memory plan reserves only from the Concat2 on -- are touched by nothing else between that launch and the
-  // Concat2.  With both inputs in place the Concat2 does not run; with one, it copies the other.
+  // Concat2.  With both inputs in place the Concat2 does not run; with one, it copies the other.  A launch that
+  // already writes through folded Reshape / Transpose steps has its strides worked out again for the part.
 
   // part `side` (0: first input, 1: second) of Concat2 step c's output, as an operand
   Operand ConcatPart(size_t c, int side) const {
@@ -662,6 +665,47 @@ class Scheduler {
     return part;
   }
 
+  // A launch that writes its logical output through folded Reshape / Transpose steps (`view_strides`), asked to
+  // write into a tensor of the final shape stored with `final_strides` instead: the strides to use then.
+  std::optional<ViewTracker::View> ViewInto(const Launch &l, const std::vector<int64_t> &final_strides) const {
+    size_t head = l.members[0];
+    int split_dim = -1;
+    if (l.kind == Launch::Kind::SoftmaxMatVec) {
+      head = l.owner;
+      split_dim = 0;  // the kernel takes its batch dim in two parts
+    } else if (l.kind == Launch::Kind::Attention) {
+      for (size_t m : l.members) {
+        if (Kind(m) == OpKind::MatMul) head = m;
+      }
+    } else if (l.kind != Launch::Kind::MatMulChain) {
+      return std::nullopt;
+    }
+    ViewTracker tracker(steps_[head].out.meta.GetShape());
+    for (size_t m : l.members) {
+      if (m <= head) continue;
+      bool ok = true;
+      switch (Kind(m)) {
+        case OpKind::Reshape:
+        case OpKind::Flatten:
+        case OpKind::Squeeze:
+        case OpKind::Unsqueeze: ok = tracker.Reshape(steps_[m].out.meta.GetShape()); break;
+        case OpKind::Transpose: {
+          std::vector<int64_t> perm = Attrs(m).perm;
+          if (perm.empty()) {
+            for (int64_t d = static_cast<int64_t>(steps_[m].out.meta.GetShape().size()); d-- > 0;) perm.push_back(d);
+          }
+          ok = tracker.Transpose(perm);
+          break;
+        }
+        default: break;  // elementwise members keep the shape
+      }
+      if (!ok) return std::nullopt;
+    }
+    auto v = tracker.Resolve(final_strides, split_dim);
+    if (v && l.kind == Launch::Kind::Attention && v->n_inner != 0) return std::nullopt;
+    return v;
+  }
+
   void PlaceConcatInputs(std::vector<Launch> *fused) {
     std::vector<size_t> issued(steps_.size());
     std::vector<Launch *> owner(steps_.size(), nullptr);
@@ -673,6 +717,12 @@ class Scheduler {
         owner[m] = &l;
       }
     }
+    MarkSilent(*fused);
+    auto really_read = [&](const Operand &op) {
+      if (op.viewed) return true;
+      auto it = producer_.find(op.name);
+      return it == producer_.end() || !silent_[it->second];
+    };
     for (size_t c = 0; c < steps_.size(); ++c) {
       if (taken_[c] || Kind(c) != OpKind::Concat2) continue;
       const Step &cat = steps_[c];
@@ -694,12 +744,13 @@ class Scheduler {
         if (!producer) continue;
         Launch *l = owner[*producer];
         if (l != nullptr) {
-          const bool plain_out = l->group.empty() && l->view_strides.empty() && SameTensor(l->out, x) && !l->out.viewed && !l->has_out2;
+          const bool plain_out = l->group.empty() && SameTensor(l->out, x) && !l->out.viewed && !l->has_out2;
           const bool kind_ok = l->kind == Launch::Kind::MatMulChain || l->kind == Launch::Kind::GemmChain ||
                                l->kind == Launch::Kind::ConvChain || l->kind == Launch::Kind::ElementwiseChain ||
                                l->kind == Launch::Kind::DivAddSoftmax || l->kind == Launch::Kind::AddLayerNorm ||
                                l->kind == Launch::Kind::Attention || l->kind == Launch::Kind::MulAdd ||
-                               l->kind == Launch::Kind::AddAdd;
+                               l->kind == Launch::Kind::AddAdd ||
+                               (l->kind == Launch::Kind::SoftmaxMatVec && !l->view_strides.empty());
           if (!plain_out || !kind_ok) continue;
         } else if (taken_[*producer] || placed_[*producer] != 0) {
           continue;
@@ -709,6 +760,12 @@ class Scheduler {
         // nothing else may touch the output's bytes from the producer's launch up to the Concat2
         const Operand target = ConcatPart(c, side);
         bool ok = true;
+        // a launch that writes through folded views: its logical output's strides inside the part
+        std::optional<ViewTracker::View> into;
+        if (l != nullptr && !l->view_strides.empty()) {
+          into = ViewInto(*l, target.view_strides);
+          if (!into || l->has_skip) continue;
+        }
         for (size_t q = 0; q < steps_.size() && ok; ++q) {
           if (q == c || elided_[q]) continue;
           if (l != nullptr ? owner[q] == l : q == *producer) continue;
@@ -717,8 +774,10 @@ class Scheduler {
           const Step &st = steps_[q];
           // the other input's producer may already write its own part of the same output
           const bool other_part = st.out.viewed && SameTensor(st.out, cat.out) && placed_[c] != 0;
-          if (!other_part && Alias(st.out, target)) ok = false;
-          if (Alias(st.in0, target) || (st.node->IsDoubleInputs() && Alias(st.in1, target))) ok = false;
+          // (intermediates of a fused launch are neither written nor read)
+          if (!other_part && !silent_[q] && Alias(st.out, target)) ok = false;
+          if ((really_read(st.in0) && Alias(st.in0, target)) ||
+              (st.node->IsDoubleInputs() && really_read(st.in1) && Alias(st.in1, target))) ok = false;
           if (st.has_buffer && target.space == Operand::Space::Arena && st.buffer_offset < target.offset + target.Extent() &&
               target.offset < st.buffer_offset + st.buffer_bytes) {
             ok = false;
@@ -727,7 +786,10 @@ class Scheduler {
         // the producer's own inputs must not lie under the bytes it now writes
         for (size_t m : (l != nullptr ? l->members : std::vector<size_t>{*producer})) {
           const Step &st = steps_[m];
-          if (Alias(st.in0, target) || (st.node->IsDoubleInputs() && Alias(st.in1, target))) ok = false;
+          if ((really_read(st.in0) && Alias(st.in0, target)) ||
+              (st.node->IsDoubleInputs() && really_read(st.in1) && Alias(st.in1, target))) {
+            ok = false;
+          }
         }
         if (l != nullptr) {
           for (const Operand *op : {&l->a, &l->b, &l->c, &l->d, &l->e}) {
@@ -738,10 +800,16 @@ class Scheduler {
         steps_[*producer].out = target;
         if (l != nullptr) l->out = target;
         else rewired_[*producer] = true;
+        if (into) {
+          l->view_strides = into->strides;
+          l->n_inner = into->n_inner;
+          l->stride_outer = into->stride_outer;
+        }
         placed_[c] |= side == 0 ? 1 : 2;
       }
       if (placed_[c] != 0) taken_[c] = true;
     }
+    silent_.clear();
   }
 
   OpKind Kind(size_t i) const { return steps_[i].node->GetKind(); }
@@ -1741,8 +1809,47 @@ class Scheduler {
     for (const Launch &l : fused) {
       for (size_t m : l.members) silent_[m] = true;
       if (l.group.empty()) silent_[l.members.back()] = false;
+      if (l.has_out2 && l.members.size() >= 2) silent_[l.members[l.members.size() - 2]] = false;
       for (const Launch &g : l.group) silent_[g.members.back()] = false;
     }
+  }
+
+  // A Softmax over a few logits left alone in front of the matrix-vector product that reads it (the
+  // product possibly with views folded behind it): refused in the first sweep where a view step in between, elided
+  // since, had its output planned over the logits.
+  void RetrySoftmaxMatVec(std::vector<Launch> *fused) {
+    moved_.assign(steps_.size(), SIZE_MAX);
+    MarkSilent(*fused);
+    for (const Launch &l : *fused) {
+      if (l.kind != Launch::Kind::MatMulGroup) continue;
+      for (size_t m : l.members) moved_[m] = l.position;
+    }
+    for (size_t i = 0; i < steps_.size(); ++i) {
+      if (taken_[i] || elided_[i] || Kind(i) != OpKind::Softmax) continue;
+      auto it = readers_.find(steps_[i].out.name);
+      if (it == readers_.end() || it->second.size() != 1) continue;
+      const size_t j = it->second[0];
+      size_t yi = fused->size();
+      for (size_t k = 0; k < fused->size(); ++k) {
+        const Launch &y = (*fused)[k];
+        if (y.kind == Launch::Kind::MatMulChain && y.members[0] == j && y.group.empty() && !y.out.viewed) yi = k;
+      }
+      if (yi == fused->size()) continue;
+      const std::vector<size_t> old_members = (*fused)[yi].members;
+      for (size_t m : old_members) taken_[m] = false;
+      std::optional<Launch> l = MatchSoftmaxMatVec(i);
+      bool ok = l.has_value();
+      for (size_t m : old_members) {
+        ok = ok && std::find(l->members.begin(), l->members.end(), m) != l->members.end();
+      }
+      ok = ok && l->members.size() == old_members.size() + 1;
+      for (size_t m : old_members) taken_[m] = true;
+      if (!ok) continue;
+      taken_[i] = true;
+      (*fused)[yi] = std::move(*l);
+    }
+    moved_.clear();
+    silent_.clear();
   }
 
   // Attention blocks the first sweep had to leave alone because a projection of the same block stood between

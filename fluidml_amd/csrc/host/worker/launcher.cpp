@@ -320,6 +320,19 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       } else {
         kernel::TensorView dst(out.t.base, steps_[l.owner].out.meta);
         for (size_t d = 0; d < l.view_strides.size(); ++d) dst.t.strides[d] = l.view_strides[d];
+        if (l.n_inner != 0) {
+          // the batch dim in two parts (written into a part of a Concat2's output): [outer, inner, rows, 1]
+          const int64_t batch = dst.t.shape[0];
+          dst.t.rank = 4;
+          dst.t.shape[3] = dst.t.shape[2];
+          dst.t.strides[3] = dst.t.strides[2];
+          dst.t.shape[2] = dst.t.shape[1];
+          dst.t.strides[2] = dst.t.strides[1];
+          dst.t.shape[1] = l.n_inner;
+          dst.t.strides[1] = dst.t.strides[0];
+          dst.t.shape[0] = batch / l.n_inner;
+          dst.t.strides[0] = l.stride_outer;
+        }
         rc = fluidml_hip_softmax_matvec(&a.t, &b.t, &dst.t, ctx.stream);
       }
       break;

@@ -405,7 +405,9 @@ int fluidml_hip_conv_chain_mean(const fl_tensor *in, const fl_tensor *weights, c
 /* SoftmaxKernel over K <= 16 logits [B, K, 1] -> MatMulKernel [B, M, K] x [B, K, 1] as ONE launch:
  * out[b, m, 0] = sum_k a[b, m, k] * softmax_k(logits[b, :, 0]) (reference softmax.cpp, matmul.cpp:28-59; the
  * per-position kernel of a span-based dynamic convolution).  `out` is [B, M, 1] with the element strides
- * these dims have inside the final buffer (a following Reshape is free).  K > 16: FL_ERR_UNSUPPORTED. */
+ * these dims have inside the final buffer (a following Reshape is free), or [B / I, I, M, 1] where the batches lie
+ * in the final buffer as I at one stride under another (heads inside a part of a concatenated tensor).
+ * K > 16: FL_ERR_UNSUPPORTED. */
 int fluidml_hip_softmax_matvec(const fl_tensor *a, const fl_tensor *logits, const fl_tensor *out, void *stream);
 /* Two pointwise convolutions on tensors of one pixel ([N, C, 1, ..]), each followed by an elementwise chain, as
  * ONE launch: the squeeze-and-excitation pair Conv -> activation -> Conv -> activation behind a global pooling

@@ -927,6 +927,15 @@ def test_fused_softmax_matvec(device):
         do2 = DeviceView(ok.View.empty((batch, rows, 1), np.float32, [1, 0, 2]), device)
         cabi.call("softmax_matvec", da2.ref(), dv.ref(), do2.ref(), None)
         assert_close(do2.logical(), ho.logical(), what="softmax_matvec (strided)")
+        # the batches as `inner` heads of each position inside the second half of a [positions, 2 * inner, rows] buffer
+        inner = 6 if batch % 6 == 0 else 1
+        whole = DeviceView(ok.View.empty((batch // inner, 2 * inner, rows), np.float32, fill=3), device)
+        part = cabi.make_tensor(whole.storage.data_ptr() + inner * rows * 4, ok.FL_FLOAT32, (batch // inner, inner, rows, 1),
+                                (2 * inner * rows, rows, 1, 1))
+        cabi.call("softmax_matvec", da.ref(), dv.ref(), ctypes.byref(part), None)
+        got = whole.logical()
+        assert_close(got[:, inner:, :].reshape(batch, rows, 1), ho.logical(), what="softmax_matvec (split batch)")
+        assert np.all(got[:, :inner, :] == 3), "softmax_matvec wrote outside its part"
     big = DeviceView(ok.View(rand(rng, (2, 3, 17))), device)
     logits = DeviceView(ok.View(rand(rng, (2, 17, 1))), device)
     res = DeviceView(ok.View.empty((2, 3, 1), np.float32), device)

@@ -1859,19 +1859,26 @@ class Scheduler {
   void RetryAttention(std::vector<Launch> *fused) {
     moved_.assign(steps_.size(), SIZE_MAX);
     MarkSilent(*fused);
-    bool any = false;
     for (const Launch &l : *fused) {
       if (l.kind != Launch::Kind::MatMulGroup) continue;
       for (size_t m : l.members) moved_[m] = l.position;
-      any = true;
     }
-    for (size_t xi = 0; any && xi < fused->size(); ++xi) {
-      const Launch &x = (*fused)[xi];
-      if (x.kind != Launch::Kind::MatMulChain || Kind(x.members[0]) != OpKind::MatMul) continue;
-      const size_t head = x.members[0];
+    // launches an attention launch may take apart: contractions with their epilogues, and the Div -> Add -> Softmax
+    // rows between the two products
+    auto dissolvable = [](const Launch &y) {
+      return y.kind == Launch::Kind::MatMulChain || y.kind == Launch::Kind::DivAddSoftmax;
+    };
+    // candidates for the score product: the head of a contraction launch, or a MatMul left as a single step
+    for (size_t head = 0; head < steps_.size(); ++head) {
+      if (Kind(head) != OpKind::MatMul || elided_[head]) continue;
+      if (taken_[head]) {
+        bool heads_chain = false;
+        for (const Launch &x : *fused) heads_chain = heads_chain || (x.kind == Launch::Kind::MatMulChain && x.members[0] == head);
+        if (!heads_chain) continue;
+      }
       const std::vector<bool> saved = taken_;
       for (const Launch &y : *fused) {
-        if (y.kind != Launch::Kind::MatMulChain) continue;
+        if (!dissolvable(y)) continue;
         for (size_t m : y.members) taken_[m] = false;
       }
       std::optional<Launch> l = MatchAttention(head);
@@ -1886,7 +1893,7 @@ class Scheduler {
           const Launch &y = (*fused)[yi];
           if (std::find(y.members.begin(), y.members.end(), m) == y.members.end()) continue;
           found = true;
-          if (y.kind != Launch::Kind::MatMulChain) ok = false;
+          if (!dissolvable(y)) ok = false;
           if (std::find(touched.begin(), touched.end(), yi) == touched.end()) touched.push_back(yi);
         }
         if (!found) {
@@ -1911,7 +1918,7 @@ class Scheduler {
       }
       kept.push_back(std::move(*l));
       *fused = std::move(kept);
-      xi = static_cast<size_t>(-1);  // the list changed: start over
+      MarkSilent(*fused);
     }
     moved_.clear();
     silent_.clear();

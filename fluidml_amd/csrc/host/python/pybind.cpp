@@ -84,14 +84,14 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
       src["view_strides"] = l.out.view_strides;
       d["source"] = src;
     } else if (l.kind == worker::Launch::Kind::Placed) {
-      // a Concat2 whose inputs were written in place: nothing runs
+      // a Concat2 whose inputs were written in place, or a Reshape behind a Concat2 that wrote into its buffer: nothing runs
     } else if (l.group.empty()) {
       // (a launch with a second output writes the tensor its last member reads as well: the member before it)
       if (l.has_out2 && l.members.size() >= 2) written.push_back(l.members[l.members.size() - 2]);
       written.push_back(l.members.back());
     }
     // a launch that writes into a part of another tensor (an input of a Concat2 placed in its output)
-    if (l.kind != worker::Launch::Kind::View && l.out.viewed) {
+    if (l.kind != worker::Launch::Kind::View && l.kind != worker::Launch::Kind::Placed && l.out.viewed) {
       py::dict into = OperandOf(l.out);
       into["bytes"] = l.out.Extent();
       d["writes_into"] = into;

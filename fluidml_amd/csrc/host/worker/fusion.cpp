@@ -221,7 +221,7 @@ class Scheduler {
  public:
   Scheduler(const std::vector<Step> &steps)
       : steps_(steps), taken_(steps.size(), false), elided_(steps.size(), false), rewired_(steps.size(), false),
-        placed_(steps.size(), 0) {
+        placed_(steps.size(), 0), filled_(steps.size(), false) {
     BuildReaders();
   }
 
@@ -290,6 +290,13 @@ class Scheduler {
         l.kind = Launch::Kind::View;
         l.members = {i};
         l.out = steps_[i].out;  // rewritten: the source seen as this step's output
+        schedule.push_back(std::move(l));
+      } else if (filled_[i]) {
+        // a Reshape whose input was written straight into its buffer
+        Launch l;
+        l.kind = Launch::Kind::Placed;
+        l.members = {i};
+        l.out = steps_[i].out;
         schedule.push_back(std::move(l));
       } else if (placed_[i] != 0) {
         // a Concat2 with one or both inputs already in place
@@ -706,6 +713,46 @@ class Scheduler {
     return v;
   }
 
+  // A Concat2 read only by a Reshape / Flatten that keeps the bytes in order (both tensors stored row-major): the
+  // Concat2 -- and whoever writes its inputs in place -- can write into the Reshape's buffer, which the memory plan
+  // reserves from the Reshape on, and the Reshape does not run.  Nothing else may touch those bytes from the
+  // Concat2 to the Reshape, and the Concat2's inputs must not lie under them.
+  void WriteIntoReshape(size_t c, const std::vector<size_t> &issued) {
+    const Step &cat = steps_[c];
+    if (!Elidable(cat.out) || !DefaultLayout(cat.out)) return;
+    auto it = readers_.find(cat.out.name);
+    if (it == readers_.end() || it->second.size() != 1) return;
+    const size_t r = it->second[0];
+    if (r <= c || taken_[r] || elided_[r] || (Kind(r) != OpKind::Reshape && Kind(r) != OpKind::Flatten)) return;
+    const Step &tail = steps_[r];
+    if (!SameTensor(tail.in0, cat.out) || tail.in0.viewed || !Elidable(tail.out) || !DefaultLayout(tail.out) ||
+        tail.out.meta.GetType() != cat.out.meta.GetType() || tail.out.meta.GetSize() != cat.out.meta.GetSize()) {
+      return;
+    }
+    Operand whole = tail.out;
+    whole.meta = cat.out.meta;
+    whole.layout = cat.out.layout;
+    whole.viewed = true;
+    whole.view_offset = 0;
+    whole.view_strides = utils::GenStrides(cat.out.meta.GetShape(), cat.out.layout);
+    whole.source_bytes = tail.out.Extent();
+    if (Alias(cat.in0, whole) || Alias(cat.in1, whole)) return;
+    for (size_t q = 0; q < steps_.size(); ++q) {
+      if (q == c || q == r || elided_[q]) continue;
+      if (!((q > c && q < r) || (issued[q] >= c && issued[q] <= r))) continue;
+      const Step &st = steps_[q];
+      if (Alias(st.out, whole) || Alias(st.in0, whole) || (st.node->IsDoubleInputs() && Alias(st.in1, whole))) return;
+      if (st.has_buffer && whole.space == Operand::Space::Arena && st.buffer_offset < whole.offset + whole.Extent() &&
+          whole.offset < st.buffer_offset + st.buffer_bytes) {
+        return;
+      }
+    }
+    steps_[c].out = whole;
+    rewired_[c] = true;
+    taken_[r] = true;
+    filled_[r] = true;
+  }
+
   void PlaceConcatInputs(std::vector<Launch> *fused) {
     std::vector<size_t> issued(steps_.size());
     std::vector<Launch *> owner(steps_.size(), nullptr);
@@ -731,6 +778,7 @@ class Scheduler {
       if (axis < 0) axis += static_cast<int64_t>(oshape.size());
       if (axis < 0 || axis >= static_cast<int64_t>(oshape.size()) || cat.out.viewed || SameTensor(cat.in0, cat.in1)) continue;
       if (cat.in0.meta.GetShape().size() != oshape.size() || cat.in1.meta.GetShape().size() != oshape.size()) continue;
+      WriteIntoReshape(c, issued);
       for (int side = 0; side < 2; ++side) {
         const Operand &x = side == 0 ? cat.in0 : cat.in1;
         if (x.viewed || !Elidable(x) || x.meta.GetType() != cat.out.meta.GetType()) continue;
@@ -2096,6 +2144,7 @@ class Scheduler {
   std::vector<bool> silent_;   // per step: an intermediate of a fused launch, never written (filled by RetryAttention)
   std::vector<size_t> moved_;  // per step: the position its launch is issued at when a group moved it (else SIZE_MAX)
   std::vector<int> placed_;  // Concat2 steps: bit 0 / 1 = input 0 / 1 is written in place by its producer
+  std::vector<bool> filled_;  // Reshape steps whose buffer the Concat2 in front of them wrote: nothing runs
   std::unordered_map<std::string, std::vector<size_t>> readers_;
   std::unordered_map<std::string, size_t> producer_;  // tensor name -> the step that writes it
 };

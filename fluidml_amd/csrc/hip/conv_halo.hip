@@ -14,8 +14,10 @@
 //     added is free, so the two lane halves simply take channels 0-3 and 4-7;
 //   * LDS pitches (24 floats per patch row; 76 per weight row, read and written 128 bits at a time) keep the lanes of
 //     an access in different banks;
-//   * double-buffered LDS, the next chunk's global loads are in flight while the current one is multiplied, one
+//   * double-buffered LDS, the next two chunks' global loads are in flight while the current one is multiplied, one
 //     barrier per chunk; two workgroups fit a compute unit and overlap each other's barriers;
+//   * with few tiles (late layers at batch 1) the input channels of a tile are split over several workgroups, whose
+//     partial tiles meet in the stream's workspace and are added in split order by the wave that arrives last;
 //   * workgroup ids are dealt so that all filter tiles of a pixel tile run on one XCD, next to each other in time:
 //     the patch is fetched into that L2 once.
 // Bias and an elementwise chain (ReLU ...) are applied in registers before the stores, like in the other contractions.
@@ -36,6 +38,7 @@ constexpr int kWPitch = 76;               // floats per filter in LDS (72 + 4: r
                                           // of consecutive filters fall into different bank groups)
 constexpr int kWElems = kFT * kWPitch;    // 4864
 constexpr int kThreads = 256;
+constexpr int kSets = 2;                  // chunks on their way in registers (3: slower, 2905 against 2986 images/s on VGG-16 at batch 8)
 constexpr int kWVecs = kFT * (kCC * 9 / 4);             // 1152 float4 of weights per chunk
 constexpr int kWPer = (kWVecs + kThreads - 1) / kThreads;  // 5
 
@@ -48,6 +51,12 @@ struct HaloArgs {
   uint32_t tiles_h, tiles_w, tiles_f, tiles_pix;  // tiles_pix = images * tiles_h * tiles_w
   const float *bias;
   int32_t sB;
+  // the input channels split over n_splits workgroups per tile (blockIdx.y), chunks_per_split chunks each; every wave
+  // leaves its partial tiles in `partials` and the wave that arrives last at its counter adds them up in split order
+  uint32_t n_splits;
+  int32_t chunks_per_split;
+  float *partials;
+  uint32_t *counters;
   fl_ew_program chain;
 };
 
@@ -111,33 +120,37 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
     x_dst[t] = i < kXItems ? ch * kPlane + r * kPitch + s : -1;
   }
 
-  floatx4 wr[kWPer];
-  float xr[kXPer];
-  auto load_chunk = [&](int c) {
+  // kSets chunks are on their way in registers (chunk i of this workgroup in set i % kSets) while another is
+  // multiplied from LDS: a chunk's loads have kSets multiplication phases to arrive, not one
+  floatx4 wr[kSets][kWPer];
+  float xr[kSets][kXPer];
+  auto load_chunk = [&](int c, auto set_c) {
+    constexpr int S = decltype(set_c)::value;
     const int c0 = c * kCC;
 #pragma unroll
     for (int t = 0; t < kWPer; ++t) {
       if constexpr (FEW) {
         const int q4 = ((tid + t * kThreads) % 18) * 4, n_w = p.C * 9;  // position of the piece inside the filter's row
-        wr[t] = floatx4{w_ok[t] && q4 < n_w ? w_src[t][0] : 0.0f, w_ok[t] && q4 + 1 < n_w ? w_src[t][1] : 0.0f,
-                        w_ok[t] && q4 + 2 < n_w ? w_src[t][2] : 0.0f, w_ok[t] && q4 + 3 < n_w ? w_src[t][3] : 0.0f};
+        wr[S][t] = floatx4{w_ok[t] && q4 < n_w ? w_src[t][0] : 0.0f, w_ok[t] && q4 + 1 < n_w ? w_src[t][1] : 0.0f,
+                           w_ok[t] && q4 + 2 < n_w ? w_src[t][2] : 0.0f, w_ok[t] && q4 + 3 < n_w ? w_src[t][3] : 0.0f};
       } else {
-        wr[t] = w_ok[t] ? *reinterpret_cast<const floatx4 *>(w_src[t] + c0 * 9) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        wr[S][t] = w_ok[t] ? *reinterpret_cast<const floatx4 *>(w_src[t] + c0 * 9) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
       }
     }
 #pragma unroll
-    for (int t = 0; t < kXPer; ++t) xr[t] = x_ok[t] ? x_src[t][static_cast<int64_t>(c0) * p.sXc] : 0.0f;
+    for (int t = 0; t < kXPer; ++t) xr[S][t] = x_ok[t] ? x_src[t][static_cast<int64_t>(c0) * p.sXc] : 0.0f;
   };
-  auto store_chunk = [&](int buf) {
-    float *xs = lds + buf * kStage;
+  auto store_chunk = [&](auto set_c, auto buf_c) {
+    constexpr int S = decltype(set_c)::value;
+    float *xs = lds + decltype(buf_c)::value * kStage;
     float *ws = xs + kXElems;
 #pragma unroll
     for (int t = 0; t < kWPer; ++t) {
-      if (tid + t * kThreads < kWVecs) *reinterpret_cast<floatx4 *>(ws + w_dst[t]) = wr[t];
+      if (tid + t * kThreads < kWVecs) *reinterpret_cast<floatx4 *>(ws + w_dst[t]) = wr[S][t];
     }
 #pragma unroll
     for (int t = 0; t < kXPer; ++t) {
-      if (x_dst[t] >= 0) xs[x_dst[t]] = xr[t];
+      if (x_dst[t] >= 0) xs[x_dst[t]] = xr[S][t];
     }
   };
 
@@ -150,13 +163,19 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
   const int a_base = (wm * 32 + lrow) * kWPitch + half * 36;
   const int b_base = half * 4 * kPlane + py * kPitch + px;
 
-  const int n_chunks = FEW ? 1 : p.C / kCC;
-  load_chunk(0);
-  store_chunk(0);
-  __syncthreads();
-  for (int c = 0; c < n_chunks; ++c) {
-    if (c + 1 < n_chunks) load_chunk(c + 1);
-    const float *xs = lds + (c & 1) * kStage;
+  const int all_chunks = FEW ? 1 : p.C / kCC;
+  const int c_first = p.n_splits > 1 ? static_cast<int>(blockIdx.y) * p.chunks_per_split : 0;
+  const int n_chunks = p.n_splits > 1 ? min(all_chunks, c_first + p.chunks_per_split) : all_chunks;
+  // chunk c (the i-th of this workgroup), held in LDS buffer i % 2 and come through register set i % kSets: request
+  // chunk c + kSets into those registers, multiply, move chunk c + 1 (requested kSets - 1 phases ago) from its
+  // registers to the other buffer
+  auto phase = [&](int c, auto idx_c) {
+    constexpr int I = decltype(idx_c)::value;
+    using Regs = std::integral_constant<int, I % kSets>;
+    using NextRegs = std::integral_constant<int, (I + 1) % kSets>;
+    using NextBuf = std::integral_constant<int, (I + 1) % 2>;
+    if (c + kSets < n_chunks) load_chunk(c + kSets, Regs{});
+    const float *xs = lds + (I % 2) * kStage;
     const float *ws = xs + kXElems;
 #pragma unroll
     for (int g = 0; g < 9; ++g) {
@@ -172,10 +191,79 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
         }
       }
     }
-    if (c + 1 < n_chunks) store_chunk((c + 1) & 1);
-    // one barrier per chunk: the buffer written here was last read in the previous iteration, and every wave
+    if (c + 1 < n_chunks) store_chunk(NextRegs{}, NextBuf{});
+    // one barrier per chunk: the buffer written here was last read in the previous phase, and every wave
     // passed the previous barrier only after finishing that read
     __syncthreads();
+  };
+  StaticFor<kSets>([&](auto k) {
+    if (c_first + decltype(k)::value < n_chunks) load_chunk(c_first + decltype(k)::value, k);
+  });
+  store_chunk(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+  __syncthreads();
+  constexpr int kPeriod = kSets % 2 == 0 ? kSets : 2 * kSets;  // after this many phases registers and buffer repeat
+  for (int c = c_first; c < n_chunks; c += kPeriod) {
+    StaticFor<kPeriod>([&](auto k) {
+      if (c + decltype(k)::value < n_chunks) phase(c + decltype(k)::value, k);
+    });
+  }
+
+  // ---- channels split over workgroups: combine the partial tiles ----------------------------------------------
+  // Each wave runs the hand-off on its own slots and its own counter, so no workgroup barrier is involved.  The
+  // partial tiles travel through device-coherent accesses (agent-scope atomics: write-through stores, loads that
+  // miss in the per-XCD L2).  Release: the wave waits until every vector memory operation it has issued is
+  // acknowledged (s_waitcnt vmcnt(0); stores count in vmcnt on gfx9) before it counts its arrival; the "memory"
+  // clobber keeps the compiler from moving the stores below the wait or the counter update above it.  Acquire: the
+  // loads of the partial tiles follow the branch on the counter's returned value, which the wave has to wait for.
+  // The sums run in split order, so the result does not depend on which workgroup arrives last.
+  if (p.n_splits > 1) {
+    const uint32_t n_splits = p.n_splits;
+    const uint32_t wslot = blockIdx.x * 4 + wave;
+    float *mine = p.partials + (static_cast<size_t>(wslot) * n_splits + blockIdx.y) * (NV * 1024);
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        __hip_atomic_store(mine + v * 1024 + e * 64 + lane, acc[v][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    uint32_t arrived = 0;
+    if (lane == 0) arrived = __hip_atomic_fetch_add(&p.counters[wslot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    arrived = __shfl(arrived, 0);
+    if (arrived != n_splits - 1) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // compiler ordering only: no instruction on gfx9
+    if (lane == 0) __hip_atomic_store(&p.counters[wslot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float *all = p.partials + static_cast<size_t>(wslot) * n_splits * (NV * 1024);
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[v][e] = 0.0f;
+    // the loads of several splits are in flight together (one round trip for all of them); the sums still run in
+    // split order
+    constexpr uint32_t kAhead = 8 / NV;
+    for (uint32_t z0 = 0; z0 < n_splits; z0 += kAhead) {
+      float part[kAhead][NV][16];
+#pragma unroll
+      for (uint32_t u = 0; u < kAhead; ++u) {
+        const uint32_t z = z0 + u < n_splits ? z0 + u : z0;  // repeats a valid slot, ignored below
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            part[u][v][e] = __hip_atomic_load(all + static_cast<size_t>(z) * (NV * 1024) + v * 1024 + e * 64 + lane,
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < kAhead; ++u) {
+        if (z0 + u < n_splits) {
+#pragma unroll
+          for (int v = 0; v < NV; ++v)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[v][e] += part[u][v][e];
+        }
+      }
+    }
   }
 
   // ---- epilogue: bias, elementwise chain, stores -------------------------------------------------------------
@@ -256,11 +344,36 @@ int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *
   const int64_t tiles_pix = N * p.tiles_h * p.tiles_w;
   const int64_t n_tiles = tiles_pix * p.tiles_f;
   // worth it when the pixel tiles are mostly full and there are enough workgroups to fill the chip
-  // (14 x 14 images fill 77 % of their tiles: measured slower than the implicit-GEMM path, 113.7 against 107.9 us)
+  // (14 x 14 images fill 77 % of their tiles: without a split measured slower than the implicit-GEMM path, 113.7
+  // against 107.9 us)
   const double fill = static_cast<double>(OH * OW) / static_cast<double>(p.tiles_h * kTH * p.tiles_w * kTW);
   // (workgroups: 224 at batch 1 on 256 x 56 x 56 still win, 40.7 -> 30.3 us with 128 input channels and 56.7 -> 54.3
-  // with 256; 112 on 512 x 28 x 28 lose against the implicit GEMM with K split over workgroups, 60 -> 100 us)
-  if (n_tiles > 0x7fffffff || n_tiles < 192 || fill < 0.8) return FL_ERR_UNSUPPORTED;
+  // with 256; 112 unsplit on 512 x 28 x 28 lose against the implicit GEMM with K split over workgroups, 60 -> 100 us)
+  // Few tiles and many channels (late layers at batch 1): the chunks of a tile go to several workgroups, aiming at
+  // two workgroups per compute unit (a workgroup is one wave per SIMD: a second one fills its barriers and loads).
+  // Measured on VGG-16 at batch 1 (1474 -> 1671 images/s; with the second chunk in flight 1726): 512 x 14 x 14 with
+  // 32 tiles 34 -> 23 us, 512 x 28 x 28 with 112 tiles 61 -> 51 us, 256 x 56 x 56 with 224 tiles 54 -> 50 us; aiming
+  // at 256, 384, 640 or 1024 workgroups, or fewer than 4 chunks per workgroup, is slower.
+  constexpr int64_t kTargetWorkgroups = 512, kMinChunks = 8;
+  int64_t splits = 1;
+  const int64_t all_chunks = few ? 1 : C / kCC;
+  if (n_tiles > 0 && n_tiles < kTargetWorkgroups && n_tiles * 4 <= static_cast<int64_t>(kWorkspaceTiles)) {
+    // (one counter per wave of a tile, one workspace slot per wave, pixel tile and split)
+    splits = std::min<int64_t>({kTargetWorkgroups / n_tiles, all_chunks / kMinChunks,
+                                static_cast<int64_t>(kWorkspaceTiles) / (n_tiles * 4 * nv)});
+  }
+  StreamWorkspace *ws = splits >= 2 ? GetStreamWorkspace(AsStream(stream)) : nullptr;
+  if (ws == nullptr) splits = 1;
+  // (split, 14 x 14 images with 77 % of their tiles filled win against the implicit GEMM as well: 34 -> 23 us)
+  if (n_tiles > 0x7fffffff || n_tiles * splits < 192 || fill < (splits > 1 ? 0.75 : 0.8)) return FL_ERR_UNSUPPORTED;
+  if (splits > 1) {
+    p.chunks_per_split = static_cast<int32_t>((all_chunks + splits - 1) / splits);
+    p.n_splits = static_cast<uint32_t>((all_chunks + p.chunks_per_split - 1) / p.chunks_per_split);
+    p.partials = ws->partials;
+    p.counters = ws->counters;
+  } else {
+    p.n_splits = 1;
+  }
   p.tiles_pix = static_cast<uint32_t>(tiles_pix);
   if (bias != nullptr) {
     p.bias = static_cast<const float *>(bias->base);
@@ -268,7 +381,7 @@ int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *
   }
   if (chain != nullptr) p.chain = *chain;
 #define FL_HALO(NV_, FEW_)                                                                                          \
-  FL_LAUNCH((ConvHalo3x3Kernel<NV_, FEW_>), dim3(static_cast<uint32_t>(n_tiles)), dim3(kThreads), 0, AsStream(stream), \
+  FL_LAUNCH((ConvHalo3x3Kernel<NV_, FEW_>), dim3(static_cast<uint32_t>(n_tiles), p.n_splits), dim3(kThreads), 0, AsStream(stream), \
             static_cast<float *>(out->base), static_cast<const float *>(in->base),                                  \
             static_cast<const float *>(weights->base), p)
   if (few) {

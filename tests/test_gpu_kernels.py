@@ -1335,7 +1335,8 @@ def test_conv_large_tiles(device):
 def test_conv_staged_patch(device):
     """3x3 unit-stride convolutions that take the kernel with the input patch staged in LDS: one and two pixel tiles per
     wave, image extents that leave the last tiles ragged, a filter count that leaves the last filter tile half empty,
-    no padding, channels-last output, bias and a ReLU chain, fewer than eight input channels."""
+    no padding, channels-last output, bias and a ReLU chain, fewer than eight input channels, input channels split
+    over several workgroups per tile."""
     cabi = _cabi()
     rng = np.random.default_rng(83)
     relu = cabi.make_chain([(cabi.EW_RELU, 0)])
@@ -1343,7 +1344,11 @@ def test_conv_staged_patch(device):
                                                   ((3, 16, 30, 62), 160, [1, 1, 1, 1], [0, 3, 1, 2], False),  # ragged rows
                                                   ((2, 8, 66, 66), 128, [0, 0, 0, 0], None, True),     # no padding
                                                   ((4, 3, 64, 80), 64, [1, 1, 1, 1], None, True),      # three channels, two tiles per wave
-                                                  ((2, 5, 33, 70), 40, [1, 1, 1, 1], None, False)]:    # five channels, ragged
+                                                  ((2, 5, 33, 70), 40, [1, 1, 1, 1], None, False),     # five channels, ragged
+                                                  # few tiles: the input channels split over workgroups (8, 4 and 2 ways, the last uneven)
+                                                  ((1, 512, 14, 14), 512, [1, 1, 1, 1], None, True),
+                                                  ((1, 256, 28, 28), 256, [1, 1, 1, 1], None, False),
+                                                  ((2, 136, 24, 40), 192, [1, 1, 1, 1], None, True)]:
         wshape = (filters, xshape[1], 3, 3)
         x, w, bias = rand(rng, xshape, -1, 1), rand(rng, wshape, -0.1, 0.1), rand(rng, (filters,), -1, 1)
         oh, ow = xshape[2] + 2 * pads[0] - 2, xshape[3] + 2 * pads[1] - 2

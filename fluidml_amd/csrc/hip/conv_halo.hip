@@ -122,8 +122,9 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
 
   // kSets chunks are on their way in registers (chunk i of this workgroup in set i % kSets) while another is
   // multiplied from LDS: a chunk's loads have kSets multiplication phases to arrive, not one
-  floatx4 wr[kSets][kWPer];
-  float xr[kSets][kXPer];
+  constexpr int kS = FEW ? 1 : kSets;  // (a single chunk there)
+  floatx4 wr[kS][kWPer];
+  float xr[kS][kXPer];
   auto load_chunk = [&](int c, auto set_c) {
     constexpr int S = decltype(set_c)::value;
     const int c0 = c * kCC;
@@ -164,17 +165,17 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
   const int b_base = half * 4 * kPlane + py * kPitch + px;
 
   const int all_chunks = FEW ? 1 : p.C / kCC;
-  const int c_first = p.n_splits > 1 ? static_cast<int>(blockIdx.y) * p.chunks_per_split : 0;
-  const int n_chunks = p.n_splits > 1 ? min(all_chunks, c_first + p.chunks_per_split) : all_chunks;
+  const int c_first = !FEW && p.n_splits > 1 ? static_cast<int>(blockIdx.y) * p.chunks_per_split : 0;
+  const int n_chunks = !FEW && p.n_splits > 1 ? min(all_chunks, c_first + p.chunks_per_split) : all_chunks;
   // chunk c (the i-th of this workgroup), held in LDS buffer i % 2 and come through register set i % kSets: request
   // chunk c + kSets into those registers, multiply, move chunk c + 1 (requested kSets - 1 phases ago) from its
   // registers to the other buffer
   auto phase = [&](int c, auto idx_c) {
     constexpr int I = decltype(idx_c)::value;
-    using Regs = std::integral_constant<int, I % kSets>;
-    using NextRegs = std::integral_constant<int, (I + 1) % kSets>;
+    using Regs = std::integral_constant<int, I % kS>;
+    using NextRegs = std::integral_constant<int, (I + 1) % kS>;
     using NextBuf = std::integral_constant<int, (I + 1) % 2>;
-    if (c + kSets < n_chunks) load_chunk(c + kSets, Regs{});
+    if (c + kS < n_chunks) load_chunk(c + kS, Regs{});
     const float *xs = lds + (I % 2) * kStage;
     const float *ws = xs + kXElems;
 #pragma unroll
@@ -196,12 +197,12 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
     // passed the previous barrier only after finishing that read
     __syncthreads();
   };
-  StaticFor<kSets>([&](auto k) {
+  StaticFor<kS>([&](auto k) {
     if (c_first + decltype(k)::value < n_chunks) load_chunk(c_first + decltype(k)::value, k);
   });
   store_chunk(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
   __syncthreads();
-  constexpr int kPeriod = kSets % 2 == 0 ? kSets : 2 * kSets;  // after this many phases registers and buffer repeat
+  constexpr int kPeriod = kS % 2 == 0 ? kS : 2 * kS;  // after this many phases registers and buffer repeat
   for (int c = c_first; c < n_chunks; c += kPeriod) {
     StaticFor<kPeriod>([&](auto k) {
       if (c + decltype(k)::value < n_chunks) phase(c + decltype(k)::value, k);
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
   // clobber keeps the compiler from moving the stores below the wait or the counter update above it.  Acquire: the
   // loads of the partial tiles follow the branch on the counter's returned value, which the wave has to wait for.
   // The sums run in split order, so the result does not depend on which workgroup arrives last.
-  if (p.n_splits > 1) {
+  if (!FEW && p.n_splits > 1) {  // (a single chunk is never split)
     const uint32_t n_splits = p.n_splits;
     const uint32_t wslot = blockIdx.x * 4 + wave;
     float *mine = p.partials + (static_cast<size_t>(wslot) * n_splits + blockIdx.y) * (NV * 1024);
@@ -353,7 +354,9 @@ int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *
   // two workgroups per compute unit (a workgroup is one wave per SIMD: a second one fills its barriers and loads).
   // Measured on VGG-16 at batch 1 (1474 -> 1671 images/s; with the second chunk in flight 1726): 512 x 14 x 14 with
   // 32 tiles 34 -> 23 us, 512 x 28 x 28 with 112 tiles 61 -> 51 us, 256 x 56 x 56 with 224 tiles 54 -> 50 us; aiming
-  // at 256, 384, 640 or 1024 workgroups, or fewer than 4 chunks per workgroup, is slower.
+  // at 256, 384, 640 or 1024 workgroups, or fewer than 4 chunks per workgroup, is slower; with one or two pixel tiles
+  // per wave and 1, 2, 3, 4 or 6 splits forced on every layer, only 64 x 224 x 224 gains on this rule (two tiles: 50 ->
+  // 46 us).
   constexpr int64_t kTargetWorkgroups = 512, kMinChunks = 8;
   int64_t splits = 1;
   const int64_t all_chunks = few ? 1 : C / kCC;

@@ -244,10 +244,12 @@ def measure(args, config, executor, per_kernel=False, per_launch=False):
         "dtype": "f32",
         "data": "synthetic: seeded weights (N(0,0.02) transformers, He-normal conv nets), seeded inputs of the configuration's shape",
         "config": {"workload": workload, "executor": args.executor, "graph_nodes": len(net.nodes),
-                   "kernels_per_step": len(times), "launch": "captured hipGraph replay"},
+                   "kernels_per_step": len(times), "launch": "captured hipGraph replay",
+                   "side_branches": len(ex.plan()["regions"])},
         "roofline": roofline,
         "peak_hbm_bytes": {"arena": plan["arena_bytes"], "constants": plan["constant_bytes"],
-                           "interface": plan["interface_bytes"], "total": plan["peak_device_bytes"]},
+                           "interface": plan["interface_bytes"], "private": ex.plan()["private_bytes"],
+                           "total": ex.plan()["peak_device_bytes"]},
         "whole_graph": {"flops_per_step": total_flops, "algorithmic_bytes_per_step": total_bytes,
                         "tflops": total_flops / (ms_per_step * 1e-3) / 1e12,
                         "sum_of_kernel_ms": kernel_sum_ms, "invoke_with_host_copies_ms": invoke_ms,
@@ -341,6 +343,7 @@ def main():
             key = name if executor == "plain_greedy" else f"{name}:{executor}"
             result["configs"][key] = {"value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"], "steps": r["steps"],
                                       "kernels_per_step": r["config"]["kernels_per_step"],
+                                      "side_branches": r["config"]["side_branches"],
                                       "roofline": {k: r["roofline"][k] for k in ("bound", "kernel", "achieved", "peak", "unit", "frac")},
                                       "whole_graph_tflops": r["whole_graph"]["tflops"],
                                       "peak_hbm_bytes": r["peak_hbm_bytes"]}

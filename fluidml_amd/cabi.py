@@ -93,6 +93,7 @@ SIGNATURES = {
     "fluidml_hip_event_create": [_P(_vp)],
     "fluidml_hip_event_destroy": [_vp],
     "fluidml_hip_event_record": [_vp, _vp],
+    "fluidml_hip_stream_wait_event": [_vp, _vp],
     "fluidml_hip_event_elapsed_ns": [_vp, _vp, _P(_f64)],
     "fluidml_hip_graph_begin_capture": [_vp],
     "fluidml_hip_graph_end_capture": [_vp, _P(_vp)],

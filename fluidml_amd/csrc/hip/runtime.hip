@@ -232,6 +232,12 @@ int fluidml_hip_event_record(void *event, void *stream) {
   return FL_OK;
 }
 
+int fluidml_hip_stream_wait_event(void *stream, void *event) {
+  if (event == nullptr) return FL_ERR_NULL;
+  FL_HIP_CHECK(hipStreamWaitEvent(AsStream(stream), static_cast<hipEvent_t>(event), 0));
+  return FL_OK;
+}
+
 int fluidml_hip_event_elapsed_ns(void *start, void *stop, double *ns) {
   if (start == nullptr || stop == nullptr || ns == nullptr) return FL_ERR_NULL;
   FL_HIP_CHECK(hipEventSynchronize(static_cast<hipEvent_t>(stop)));

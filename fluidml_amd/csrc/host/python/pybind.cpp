@@ -67,6 +67,7 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
   out["arena_bytes"] = plan.GetArenaBytes();
   out["constant_bytes"] = plan.GetConstantBytes();
   out["interface_bytes"] = plan.GetInterfaceBytes();
+  out["private_bytes"] = plan.GetPrivateBytes();
   out["peak_device_bytes"] = plan.GetPeakDeviceBytes();
   out["steps"] = steps;
   py::list launches;
@@ -98,12 +99,43 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
     }
     for (const worker::Launch &m : l.group) written.push_back(m.members.back());
     d["written"] = written;
+    // what the launch reads and writes as it is issued (operands of a side branch point at buffers of their own)
+    py::list reads, writes;
+    if (l.kind != worker::Launch::Kind::View && l.kind != worker::Launch::Kind::Placed) {
+      auto add_reads = [&](const worker::Launch &x) {
+        for (const worker::Operand *op : {&x.a, &x.b, &x.c, &x.d, &x.e}) {
+          if (!op->name.empty() && (x.kind != worker::Launch::Kind::Step || x.rewired)) {
+            py::dict o = OperandOf(*op);
+            o["bytes"] = op->Extent();
+            reads.append(o);
+          }
+        }
+      };
+      auto add_write = [&](const worker::Operand &op) {
+        py::dict o = OperandOf(op);
+        o["bytes"] = op.Extent();
+        writes.append(o);
+      };
+      add_reads(l);
+      for (const worker::Launch &m : l.group) add_reads(m);
+      if (l.kind != worker::Launch::Kind::Step || l.rewired) {
+        if (l.group.empty()) add_write(l.out);
+        for (const worker::Launch &m : l.group) add_write(m.out);
+        if (l.has_out2) add_write(l.out2);
+      }
+    }
+    d["reads"] = reads;
+    d["writes"] = writes;
     d["position"] = l.group.empty() ? l.members.back() : l.position;
     d["bytes"] = l.bytes;
     d["flops"] = l.flops;
     launches.append(d);
   }
   out["launches"] = launches;
+  // runs of launches issued side by side: launches [a_begin, b_begin) on the plan's stream, [b_begin, end) beside them
+  py::list regions;
+  for (const worker::LaunchPlan::Region &r : plan.GetRegions()) regions.append(py::make_tuple(r.a_begin, r.b_begin, r.end));
+  out["regions"] = regions;
   py::list arguments;
   for (const worker::Argument &arg : plan.GetArguments()) {
     py::dict d;
@@ -153,6 +185,8 @@ PYBIND11_MODULE(fluidml, m) {
       .def("set_fuse", [](context::Context &c, bool fuse) { c->fuse = fuse; }, py::arg("fuse"))
       .def("set_graph_passes", [](context::Context &c, bool on) { c->graph_passes = on; }, py::arg("on"))
       .def("set_bf16", [](context::Context &c, bool on) { c->bf16 = on; }, py::arg("on"))
+      .def("set_branch_min_us", [](context::Context &c, double us) { c->branch_min_us = us; }, py::arg("us"))
+      .def("set_branch_check", [](context::Context &c, bool on) { c->branch_check = on; }, py::arg("on"))
       .def("plan_text", [](context::Context &c) { return c->GetModule().ToText(); });
 
   py::class_<flow::Flow, std::unique_ptr<flow::Flow>>(m, "Flow")

@@ -88,6 +88,12 @@ class ContextImpl {
   bool graph_passes = false;
   // MatMul nodes on the opt-in bf16 path (env FLUIDML_BF16=1)
   bool bf16 = false;
+  // two independent runs of launches go side by side on two streams when the shorter one is estimated at least
+  // this long, in microseconds (env FLUIDML_BRANCHES=0 never; negative: the launch plan's default)
+  double branch_min_us = -1.0;
+  // time the first replays with and without the side branches and keep the faster schedule (env FLUIDML_BRANCH_CHECK=0:
+  // keep every candidate region)
+  bool branch_check = true;
   // cost source of the layout DP (env FLUIDML_DP_COST=measure|constant|<path to table json>)
   CostMode cost_mode = CostMode::Measure;
   std::string cost_table_path;

@@ -153,6 +153,8 @@ class GeneralBuilderImpl : public GeneralBuilder {
     plan->SetUseGraph(context_->use_graph);
     plan->SetFuse(context_->fuse);
     plan->SetBf16(context_->bf16);
+    if (context_->branch_min_us >= 0) plan->SetBranchMinUs(context_->branch_min_us);
+    plan->SetBranchCheck(context_->branch_check);
     context_->SetModule(std::move(plan));
     context_->SetFuncAttr(std::move(func_attr));
   }

@@ -128,6 +128,8 @@ class ExecutorImpl : public Executor {
     plain->fuse = context_->fuse;
     plain->graph_passes = context_->graph_passes;
     plain->bf16 = context_->bf16;
+    plain->branch_min_us = context_->branch_min_us;
+    plain->branch_check = context_->branch_check;
     return plain;
   }
 

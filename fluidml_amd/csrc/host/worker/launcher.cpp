@@ -2,6 +2,8 @@
 
 #include <algorithm>
 #include <chrono>
+#include <cstdlib>
+#include <map>
 #include <sstream>
 #include <stdexcept>
 
@@ -36,6 +38,8 @@ LaunchPlan::LaunchPlan(std::string &&name, size_t arena_bytes) : name_(std::move
 
 LaunchPlan::~LaunchPlan() {
   if (graph_) fluidml_hip_graph_destroy(graph_);
+  for (void *e : region_events_) fluidml_hip_event_destroy(e);
+  if (side_stream_) fluidml_hip_stream_destroy(side_stream_);
   for (auto &kv : constants_) fluidml_hip_free(kv.second.device);
   for (auto &kv : privates_) fluidml_hip_free(kv.second.device);
   for (auto &kv : interfaces_) fluidml_hip_free(kv.second.device);
@@ -60,6 +64,13 @@ size_t LaunchPlan::GetConstantBytes() const {
   size_t n = 0;
   for (const auto &kv : constants_) n += kv.second.tensor.GetMeta().GetSize();
   for (const Step &s : steps_) n += s.kernel->GetConstantBytes();
+  return n;
+}
+
+size_t LaunchPlan::GetPrivateBytes() const {
+  GetSchedule();
+  size_t n = 0;
+  for (const auto &kv : privates_) n += kv.second.bytes;
   return n;
 }
 
@@ -142,7 +153,13 @@ std::string LaunchPlan::ToText() const {
 void LaunchPlan::Materialize() {
   if (arena_ != nullptr) return;
   Validate();
+  GetSchedule();  // may move tensors of a side branch into buffers of their own, allocated below
   Check(fluidml_hip_stream_create(&stream_), "creating the plan's stream");
+  if (!regions_.empty()) {
+    Check(fluidml_hip_stream_create(&side_stream_), "creating the plan's second stream");
+    region_events_.resize(2 * regions_.size(), nullptr);
+    for (void *&e : region_events_) Check(fluidml_hip_event_create(&e), "creating a fork/join event");
+  }
   for (auto &kv : constants_) {
     const std::vector<uint8_t> bytes = kv.second.tensor.Pack(kv.second.layout);
     Check(fluidml_hip_upload_constant(bytes.data(), bytes.size(), &kv.second.device), "uploading a constant region");
@@ -175,8 +192,192 @@ const std::vector<Launch> &LaunchPlan::GetSchedule() const {
   if (!schedule_built_) {
     schedule_ = BuildSchedule(steps_, fuse_ && flags_ == 0);
     schedule_built_ = true;
+    regions_.clear();
+    if (fuse_ && flags_ == 0 && !branches_off_) PlanBranches();
   }
   return schedule_;
+}
+
+namespace {
+bool Alias(const Operand &x, const Operand &y) {
+  if (x.space != y.space) return false;
+  if (x.space != Operand::Space::Arena) return x.name == y.name;
+  return x.offset < y.offset + y.Extent() && y.offset < x.offset + x.Extent();
+}
+
+// the operands a launch reads and writes (pointers into the launch, so that they can be redirected)
+struct Access {
+  std::vector<Operand *> reads, writes;
+  bool runs = true;     // false: a view or a step whose bytes are already in place
+  double cost_us = 0;
+};
+
+bool BranchesEnabled() {
+  static const bool on = [] {
+    const char *v = std::getenv("FLUIDML_BRANCHES");
+    return v == nullptr || std::strtol(v, nullptr, 10) != 0;
+  }();
+  return on;
+}
+}  // namespace
+
+// Looks for pairs of consecutive runs of launches A, B where B reads nothing A writes (attention block and MLP of a
+// parallel-residual layer, convolution branch and attention branch of a mixed-attention layer) and lets B run on a
+// second stream beside A.  The memory plan was made for the serial order, so bytes B writes may be ones A still
+// uses: every tensor B writes moves to a buffer of its own, and its readers with it.
+// (The scratch the memory plan reserves for some steps is not touched by any kernel here unless literal-reference
+// flags are set, and then no branches are planned.)
+void LaunchPlan::PlanBranches() const {
+  regions_.clear();
+  if (!BranchesEnabled()) return;
+  std::vector<Launch> &sched = schedule_;
+  const size_t n = sched.size();
+  // every single step carries its operands itself from here on, so that they can be redirected
+  for (Launch &l : sched) {
+    if (l.kind == Launch::Kind::Step && !l.rewired) {
+      const Step &st = steps_[l.members[0]];
+      l.rewired = true;
+      l.a = st.in0;
+      if (st.node->IsDoubleInputs()) l.b = st.in1;
+      l.out = st.out;
+    }
+  }
+  std::vector<Access> acc(n);
+  auto add_reads = [](Access &a, Launch &l) {
+    for (Operand *op : {&l.a, &l.b, &l.c, &l.d, &l.e}) {
+      if (!op->name.empty() && op->space != Operand::Space::Constant) a.reads.push_back(op);
+    }
+  };
+  for (size_t i = 0; i < n; ++i) {
+    Launch &l = sched[i];
+    Access &a = acc[i];
+    if (l.kind == Launch::Kind::View || l.kind == Launch::Kind::Placed) {
+      a.runs = false;
+      continue;
+    }
+    add_reads(a, l);
+    if (l.group.empty()) {
+      a.writes.push_back(&l.out);
+    } else {
+      for (Launch &g : l.group) {
+        add_reads(a, g);
+        a.writes.push_back(&g.out);
+      }
+    }
+    if (l.has_out2) a.writes.push_back(&l.out2);
+    // a launch is a few microseconds of latency plus its work at a fraction of the peaks
+    a.cost_us = 4.0 + l.flops / 6e7 + l.bytes / 3e6;
+  }
+  // writers of every arena tensor
+  std::map<std::string, std::vector<size_t>> writers;
+  for (size_t i = 0; i < n; ++i) {
+    for (const Operand *w : acc[i].writes) {
+      if (w->space == Operand::Space::Arena) writers[w->name].push_back(i);
+    }
+  }
+  // A fork and a join cost about 18 us on this runtime (measured on captured graphs: a region whose runs take 10 us
+  // each replays 6 us slower than the same launches in a row, one with 40 us runs 22 us faster), so only runs of some
+  // length are candidates; whether the candidates stay is decided by timing the schedule (DecideBranches).
+  constexpr size_t kMaxRun = 10;
+  static const double env_min_us = [] {
+    const char *v = std::getenv("FLUIDML_BRANCH_MIN_US");
+    return v != nullptr ? std::strtod(v, nullptr) : -1.0;
+  }();
+  const double min_us = env_min_us >= 0 ? env_min_us : branch_min_us_;
+  auto eligible = [&](size_t a0, size_t b0, size_t e) {
+    for (size_t y = b0; y < e; ++y) {
+      if (!acc[y].runs) continue;
+      for (const Operand *r : acc[y].reads) {
+        // what B produces itself moves out of the arena with its writers (checked below): no bytes shared with A
+        if (r->space == Operand::Space::Arena) {
+          auto it = writers.find(r->name);
+          if (it != writers.end() && !it->second.empty() && it->second.front() >= b0 && it->second.back() < e) continue;
+        }
+        for (size_t x = a0; x < b0; ++x) {
+          for (const Operand *w : acc[x].writes) {
+            if (Alias(*w, *r)) return false;
+          }
+        }
+      }
+      for (const Operand *w : acc[y].writes) {
+        if (w->space == Operand::Space::Arena) {
+          for (size_t wr : writers[w->name]) {
+            if (wr < b0 || wr >= e) return false;  // written elsewhere too: has to stay in the plan's bytes
+          }
+        } else {
+          // a graph output, or a buffer of its own already: nothing of A may touch it
+          for (size_t x = a0; x < b0; ++x) {
+            for (const Operand *o : acc[x].reads) {
+              if (Alias(*w, *o)) return false;
+            }
+            for (const Operand *o : acc[x].writes) {
+              if (Alias(*w, *o)) return false;
+            }
+          }
+        }
+      }
+    }
+    return true;
+  };
+  size_t i = 0;
+  while (i < n) {
+    if (!acc[i].runs) {
+      ++i;
+      continue;
+    }
+    double best_gain = std::max(0.0, min_us) - 1e-9;  // the shorter run's estimate has to reach this
+    size_t best_b = 0, best_e = 0;
+    double cost_a = 0;
+    size_t runs_a = 0;
+    for (size_t b0 = i + 1; b0 < n && runs_a < kMaxRun; ++b0) {
+      if (acc[b0 - 1].runs) {
+        cost_a += acc[b0 - 1].cost_us;
+        ++runs_a;
+      }
+      if (!acc[b0].runs) continue;  // B starts at a launch that runs
+      double cost_b = 0;
+      size_t runs_b = 0;
+      for (size_t e = b0 + 1; e <= n && runs_b < kMaxRun; ++e) {
+        if (!acc[e - 1].runs) continue;
+        cost_b += acc[e - 1].cost_us;
+        ++runs_b;
+        const double gain = std::min(cost_a, cost_b);
+        if (gain <= best_gain) continue;
+        if (!eligible(i, b0, e)) continue;  // (a longer B may take in the other writer of a tensor)
+        best_gain = gain;
+        best_b = b0;
+        best_e = e;
+      }
+    }
+    if (best_e == 0) {
+      ++i;
+      continue;
+    }
+    regions_.push_back({i, best_b, best_e});
+    // move what B writes out of the arena
+    std::map<std::string, size_t> moved;
+    for (size_t y = best_b; y < best_e; ++y) {
+      for (const Operand *w : acc[y].writes) {
+        if (w->space == Operand::Space::Arena) moved[w->name] = std::max(moved[w->name], w->Extent());
+      }
+    }
+    for (Launch &l : sched) {
+      auto redirect = [&](Launch &x) {
+        for (Operand *op : {&x.a, &x.b, &x.c, &x.d, &x.e, &x.out, &x.out2}) {
+          if (op->space != Operand::Space::Arena || op->name.empty()) continue;
+          auto it = moved.find(op->name);
+          if (it == moved.end()) continue;
+          it->second = std::max(it->second, op->Extent());
+          op->space = Operand::Space::Private;
+          op->offset = 0;
+        }
+      };
+      redirect(l);
+      for (Launch &g : l.group) redirect(g);
+    }
+    for (const auto &kv : moved) privates_[kv.first].bytes = std::max(privates_[kv.first].bytes, kv.second);
+    i = best_e;
+  }
 }
 
 void LaunchPlan::IssueStep(kernel::LaunchContext &ctx, const Step &s, const Operand *in0_view,
@@ -450,7 +651,36 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
 }
 
 void LaunchPlan::LaunchAll(kernel::LaunchContext &ctx) const {
-  for (const Launch &l : GetSchedule()) Issue(ctx, l);
+  const std::vector<Launch> &schedule = GetSchedule();
+  if (regions_.empty() || side_stream_ == nullptr) {
+    for (const Launch &l : schedule) Issue(ctx, l);
+    return;
+  }
+  kernel::LaunchContext side = ctx;
+  side.stream = side_stream_;
+  size_t r = 0;
+  for (size_t i = 0; i < schedule.size(); ++i) {
+    const bool inside = r < regions_.size() && i >= regions_[r].a_begin;
+    if (inside && i == regions_[r].a_begin) {
+      // fork: the second stream starts from the state the plan's stream has reached
+      Check(fluidml_hip_event_record(region_events_[2 * r], ctx.stream), "recording a fork");
+      Check(fluidml_hip_stream_wait_event(side_stream_, region_events_[2 * r]), "forking the second stream");
+    }
+    if (inside && i >= regions_[r].b_begin) {
+      Issue(side, schedule[i]);
+    } else {
+      Issue(ctx, schedule[i]);
+    }
+    if (inside && i + 1 == regions_[r].end) {
+      Check(fluidml_hip_event_record(region_events_[2 * r + 1], side_stream_), "recording a join");
+      Check(fluidml_hip_stream_wait_event(ctx.stream, region_events_[2 * r + 1]), "joining the second stream");
+      ++r;
+    }
+  }
+  if (side.status != 0 && ctx.status == 0) {
+    ctx.status = side.status;
+    ctx.failed = side.failed;
+  }
 }
 
 // One replay of the whole sequence on the plan's stream: the captured graph
@@ -488,6 +718,7 @@ size_t LaunchPlan::Run(const std::unordered_map<std::string, void *> &args, size
     }
   }
   Check(fluidml_hip_stream_synchronize(stream_), "waiting for input copies");
+  DecideBranches();
   kernel::LaunchContext ctx;
   ctx.stream = stream_;
   ctx.flags = flags_;
@@ -509,8 +740,37 @@ size_t LaunchPlan::Run(const std::unordered_map<std::string, void *> &args, size
   return static_cast<size_t>(std::chrono::duration_cast<std::chrono::nanoseconds>(t1 - t0).count()) / epoch;
 }
 
+// Which kernels gain from running beside each other is not something the estimate above can tell (GPT-NeoX: its MLP
+// beside the attention block gains nothing, the next layer's first projections beside an attention block 12 us;
+// ConvBERT loses with every region), so the schedule with its regions and the one without them are both replayed on
+// the first inputs and the faster one stays.
+void LaunchPlan::DecideBranches() {
+  if (branches_decided_) return;
+  branches_decided_ = true;
+  static const bool env_check = [] {
+    const char *v = std::getenv("FLUIDML_BRANCH_CHECK");
+    return v == nullptr || std::strtol(v, nullptr, 10) != 0;
+  }();
+  if (regions_.empty() || !branch_check_ || !env_check) return;
+  auto rebuild = [&](bool off) {
+    Check(fluidml_hip_stream_synchronize(stream_), "waiting for the timed replays");
+    if (graph_ != nullptr) {
+      fluidml_hip_graph_destroy(graph_);
+      graph_ = nullptr;
+    }
+    branches_off_ = off;
+    schedule_built_ = false;
+    GetSchedule();
+  };
+  const double with = TimeReplayNs(2, 12);
+  rebuild(true);
+  const double without = TimeReplayNs(2, 12);
+  if (with < 0.985 * without) rebuild(false);  // (the same regions and the same buffers again: planning is deterministic)
+}
+
 void LaunchPlan::ReplayResident(size_t n) {
   Materialize();
+  DecideBranches();
   kernel::LaunchContext ctx;
   ctx.stream = stream_;
   ctx.flags = flags_;
@@ -521,6 +781,7 @@ void LaunchPlan::ReplayResident(size_t n) {
 
 double LaunchPlan::TimeReplayNs(size_t warmup, size_t iters) {
   Materialize();
+  DecideBranches();
   kernel::LaunchContext ctx;
   ctx.stream = stream_;
   ctx.flags = flags_;
@@ -541,6 +802,7 @@ double LaunchPlan::TimeReplayNs(size_t warmup, size_t iters) {
 
 std::vector<double> LaunchPlan::ReplayTimesNs(size_t warmup, size_t iters) {
   Materialize();
+  DecideBranches();
   kernel::LaunchContext ctx;
   ctx.stream = stream_;
   ctx.flags = flags_;
@@ -562,6 +824,7 @@ std::vector<double> LaunchPlan::ReplayTimesNs(size_t warmup, size_t iters) {
 
 std::vector<StepTime> LaunchPlan::Profile(size_t warmup, size_t iters) {
   Materialize();
+  DecideBranches();
   kernel::LaunchContext ctx;
   ctx.stream = stream_;
   ctx.flags = flags_;

@@ -168,7 +168,8 @@ class LaunchPlan {
   size_t GetArenaBytes() const { return arena_bytes_; }
   size_t GetConstantBytes() const;   // constant regions + constants kernels own
   size_t GetInterfaceBytes() const;  // device staging of graph inputs and outputs
-  size_t GetPeakDeviceBytes() const { return arena_bytes_ + GetConstantBytes() + GetInterfaceBytes(); }
+  size_t GetPrivateBytes() const;    // tensors outside the arena: regions no Memory edge uses, outputs of side branches
+  size_t GetPeakDeviceBytes() const { return arena_bytes_ + GetConstantBytes() + GetInterfaceBytes() + GetPrivateBytes(); }
   const std::vector<Step> &GetSteps() const { return steps_; }
   // the launches actually replayed (steps grouped into chains when fusion is on)
   const std::vector<Launch> &GetSchedule() const;
@@ -210,6 +211,21 @@ class LaunchPlan {
   void *GetDeviceAddress(const std::string &name) const;
   void *GetArenaBase() const { return arena_; }
   void *GetStream() const { return stream_; }
+  // Two runs of launches that follow each other in the schedule, [a_begin, b_begin) and [b_begin, end), the second
+  // of which reads nothing the first writes: the second run is issued on a stream beside the plan's, between a fork
+  // in front of the first run and a join behind the second, and everything it writes lives in buffers of its own
+  // instead of the memory plan's bytes (which the first run may still be using).
+  struct Region {
+    size_t a_begin = 0, b_begin = 0, end = 0;
+  };
+  const std::vector<Region> &GetRegions() const {
+    GetSchedule();
+    return regions_;
+  }
+  // a region is formed when the shorter of its two runs is estimated at least this long (microseconds)
+  void SetBranchMinUs(double us) { branch_min_us_ = us; }
+  // whether the first run times the schedule with and without its regions and keeps the faster one
+  void SetBranchCheck(bool on) { branch_check_ = on; }
 
  private:
   struct ConstantSlot {
@@ -227,19 +243,29 @@ class LaunchPlan {
   void Issue(kernel::LaunchContext &ctx, const Launch &l) const;
   void LaunchAll(kernel::LaunchContext &ctx) const;
   void Replay(kernel::LaunchContext &ctx);
+  void PlanBranches() const;
+  void DecideBranches();
 
   std::string name_;
   size_t arena_bytes_;
   std::vector<Argument> arguments_;
   std::vector<Step> steps_;
   std::map<std::string, ConstantSlot> constants_;
-  std::map<std::string, RawSlot> privates_, interfaces_;
+  mutable std::map<std::string, RawSlot> privates_;
+  std::map<std::string, RawSlot> interfaces_;
   uint32_t flags_ = 0;
   bool use_graph_ = true;
   bool fuse_ = true;
   bool bf16_ = false;
   mutable std::vector<Launch> schedule_;
   mutable bool schedule_built_ = false;
+  mutable std::vector<Region> regions_;
+  double branch_min_us_ = 12.0;
+  bool branch_check_ = true;
+  bool branches_decided_ = false;
+  mutable bool branches_off_ = false;
+  void *side_stream_ = nullptr;
+  std::vector<void *> region_events_;  // fork and join event of every region
   void *arena_ = nullptr;
   void *stream_ = nullptr;
   void *graph_ = nullptr;

@@ -175,6 +175,10 @@ int fluidml_hip_stream_synchronize(void *stream);
 int fluidml_hip_event_create(void **event);
 int fluidml_hip_event_destroy(void *event);
 int fluidml_hip_event_record(void *event, void *stream);
+/* Work issued to `stream` after this call waits for what `event` recorded (the edge between the two branches of a
+ * launch plan that runs an independent run of launches beside another; the reference runs its nodes one after the
+ * other, runner.cpp:101-109).  Also valid while `event`'s stream is being captured: `stream` then joins the capture. */
+int fluidml_hip_stream_wait_event(void *stream, void *event);
 int fluidml_hip_event_elapsed_ns(void *start, void *stop, double *ns);
 /* Kernel-exact timing for the calling thread: until cleared with (NULL, NULL),
  * every kernel an entry point below launches stamps `start`/`stop` with the

@@ -167,7 +167,7 @@ def test_profile_and_accounting(device, tiny_bert):
     ex = fluidml.Executor.make_plain_greedy("tiny_prof")
     ex.compile(path)
     plan = ex.plan()
-    assert plan["peak_device_bytes"] == plan["arena_bytes"] + plan["constant_bytes"] + plan["interface_bytes"]
+    assert plan["peak_device_bytes"] == plan["arena_bytes"] + plan["constant_bytes"] + plan["interface_bytes"] + plan["private_bytes"]
     _invoke(ex, net, feeds)
     times = ex.profile(2, 5)
     run = [l for l in plan["launches"] if l["kind"] != "View"]  # a view step is not run: its readers use strides

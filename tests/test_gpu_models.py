@@ -50,3 +50,36 @@ def test_config_matches_oracle(device, config, flavour, tmp_path, monkeypatch):
         assert ex.invoke(args) > 0
         for name, ref in want.items():
             assert_close(outs[name], ref, what=f"{config} {flavour} {name}")
+
+
+@pytest.mark.parametrize("use_graph", [True, False], ids=["captured", "eager"])
+@pytest.mark.parametrize("config", ["convbert", "gpt_neox", "efficientnet_b0"])
+def test_side_branches_match_oracle(device, config, use_graph, tmp_path):
+    """Independent runs of launches issued on two streams (fork, two branches, join), forced on the small graphs by
+    a zero threshold: same results as the oracle, replay after replay, in a captured graph and launch by launch; what
+    the side branch writes lives in buffers of its own."""
+    from fluidml_amd import fluidml
+
+    make_net, make_feeds = _cases()[config]
+    net, feeds = make_net(), make_feeds()
+    want = graph_runner.run_graph(net, feeds)
+    path = net.save(str(tmp_path / f"{config}.onnx"))
+    ex = fluidml.Executor.make_plain_greedy(config, 2)
+    ex.context().set_branch_min_us(0.0)
+    ex.context().set_branch_check(False)  # keep every region, faster or not
+    ex.context().set_use_graph(use_graph)
+    ex.compile(path)
+    plan = ex.plan()
+    print("[case]", config, "regions", plan["regions"], flush=True)
+    if config != "efficientnet_b0":  # (a chain of blocks: nothing runs side by side there)
+        assert len(plan["regions"]) >= 2
+    for a, b, e in plan["regions"]:
+        for l in plan["launches"][b:e]:
+            assert all(w["space"] in ("private", "interface") for w in l["writes"])
+    args = {k: np.ascontiguousarray(v) for k, v in feeds.items()}
+    outs = {v.name: np.full(v.shape, np.nan, dtype=v.dtype) for v in net.outputs}
+    args.update(outs)
+    for _ in range(3):
+        assert ex.invoke(args) > 0
+        for name, ref in want.items():
+            assert_close(outs[name], ref, what=f"{config} side branches {name}")

@@ -552,6 +552,67 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     assert len(ex.plan()["launches"]) == len(ex.plan()["steps"])
 
 
+BRANCH_NETS = {
+    "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), 0.0, 2),
+    "convbert": (lambda m: m.convbert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32), 0.0, 2),
+    "bert": (lambda m: m.bert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32, seed=5), 0.0, 0),
+    # full size with the default threshold: the attention block of a layer beside its MLP
+    "gpt_neox_full": (lambda m: m.gpt_neox(), None, 3),
+    "convbert_full_forced": (lambda m: m.convbert_base(), 0.0, 6),
+}
+
+
+@pytest.mark.parametrize("which", list(BRANCH_NETS))
+def test_side_branches_are_independent(mods, which, tmp_path):
+    """Two runs of launches issued side by side on two streams: the second (B) must read nothing the first (A)
+    writes, and since the memory plan was made for the serial order, everything B writes has to live outside the
+    arena, in buffers nobody else writes and nobody reads before B."""
+    fluidml, models, _ = mods
+    make, min_us, at_least = BRANCH_NETS[which]
+    path = make(models).save(str(tmp_path / "net.onnx"))
+    ex = fluidml.Executor.make_plain_greedy("branches")
+    if min_us is not None:
+        ex.context().set_branch_min_us(min_us)
+    ex.compile(path)
+    plan = ex.plan()
+    launches, regions = plan["launches"], plan["regions"]
+    assert len(regions) >= at_least
+    runs = lambda l: l["kind"] not in ("View", "Placed")
+    last = 0
+    for a, b, e in regions:
+        assert last <= a < b < e <= len(launches)
+        last = e
+        assert runs(launches[a]) and runs(launches[b]) and runs(launches[e - 1])
+        first, second = [l for l in launches[a:b] if runs(l)], [l for l in launches[b:e] if runs(l)]
+        own = set()
+        for y in second:
+            for w in y["writes"]:
+                assert w["space"] in ("private", "interface"), "a side branch writes into the arena"
+                if w["space"] == "private":
+                    own.add(w["name"])
+            for r in y["reads"]:
+                for x in first:
+                    assert not any(_overlap(w, r) for w in x["writes"]), "a side branch reads what the other run writes"
+        for x in first:
+            for op in x["reads"] + x["writes"]:
+                assert not (op["space"] in ("private", "interface") and any(
+                    _overlap(op, w) for y in second for w in y["writes"])), "the first run touches what the side branch writes"
+        # the side branch's buffers: written only there, read only there or after the join
+        for k, l in enumerate(launches):
+            if not runs(l):
+                continue
+            outside = k < b or k >= e
+            if outside:
+                assert not any(w["space"] == "private" and w["name"] in own for w in l["writes"])
+            if k < b:
+                assert not any(r["space"] == "private" and r["name"] in own for r in l["reads"])
+    # without regions nothing is moved out of the arena
+    ex = fluidml.Executor.make_plain_greedy("no_branches")
+    ex.context().set_branch_min_us(1e9)
+    ex.compile(path)
+    assert ex.plan()["regions"] == []
+
+
 # ------------------------------------------------------------------ layout DP
 
 def test_dp_constant_cost_closed_form(mods, tiny):

@@ -372,6 +372,8 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     an elided tensor has no reader outside its chain, and moving a chain's reads to its last member's
     position crosses no write to the bytes it reads (arena intervals of the memory plan)."""
     fluidml, models, _ = mods
+    if which.endswith("_full") and flavour == "make_plain_linear":
+        pytest.skip("the linear plan reuses no bytes: the small graphs cover it, the full-size ones are here for their reuse")
     make, expected_kinds = SCHEDULE_NETS[which][:2]
     if flavour != "make_dp_greedy" and len(SCHEDULE_NETS[which]) > 2:
         expected_kinds = expected_kinds | SCHEDULE_NETS[which][2]

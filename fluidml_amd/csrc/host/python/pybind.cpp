@@ -39,6 +39,7 @@ py::dict OperandOf(const worker::Operand &op) {
   d["name"] = op.name;
   d["space"] = kSpaces[static_cast<int>(op.space)];
   d["offset"] = op.offset;
+  d["pool"] = op.pool;
   d["bytes"] = op.meta.GetSize();
   d["shape"] = op.meta.GetShape();
   d["layout"] = op.layout;

@@ -176,7 +176,7 @@ void *LaunchPlan::Resolve(const Operand &op) const {
     case Operand::Space::Arena: return static_cast<char *>(arena_) + op.offset;
     case Operand::Space::Interface: return interfaces_.at(op.name).device;
     case Operand::Space::Constant: return constants_.at(op.name).device;
-    default: return privates_.at(op.name).device;
+    default: return static_cast<char *>(privates_.at(op.pool.empty() ? op.name : op.pool).device) + op.offset;
   }
 }
 
@@ -201,8 +201,9 @@ const std::vector<Launch> &LaunchPlan::GetSchedule() const {
 namespace {
 bool Alias(const Operand &x, const Operand &y) {
   if (x.space != y.space) return false;
-  if (x.space != Operand::Space::Arena) return x.name == y.name;
-  return x.offset < y.offset + y.Extent() && y.offset < x.offset + x.Extent();
+  if (x.space == Operand::Space::Interface || x.space == Operand::Space::Constant) return x.name == y.name;
+  if (x.space == Operand::Space::Private && (x.pool.empty() ? x.name : x.pool) != (y.pool.empty() ? y.name : y.pool)) return false;
+  return x.offset < y.offset + y.Extent() && y.offset < x.offset + x.Extent();  // bytes of the arena / of one buffer
 }
 
 // the operands a launch reads and writes (pointers into the launch, so that they can be redirected)
@@ -319,6 +320,7 @@ void LaunchPlan::PlanBranches() const {
     }
     return true;
   };
+  std::vector<size_t> side_free_from;  // per shared buffer: first launch index from which nobody uses its contents
   size_t i = 0;
   while (i < n) {
     if (!acc[i].runs) {
@@ -354,28 +356,57 @@ void LaunchPlan::PlanBranches() const {
       continue;
     }
     regions_.push_back({i, best_b, best_e});
-    // move what B writes out of the arena
-    std::map<std::string, size_t> moved;
+    // Move what B writes out of the arena, into a buffer the side branches share: a region takes the first of the
+    // buffers whose previous tenants nobody touches from this region's fork on (B starts right behind the fork).
+    struct Moved {
+      size_t bytes = 0, offset = 0, last_use = 0;
+    };
+    std::map<std::string, Moved> moved;
     for (size_t y = best_b; y < best_e; ++y) {
       for (const Operand *w : acc[y].writes) {
-        if (w->space == Operand::Space::Arena) moved[w->name] = std::max(moved[w->name], w->Extent());
+        if (w->space == Operand::Space::Arena) moved[w->name].bytes = std::max(moved[w->name].bytes, w->Extent());
       }
     }
+    size_t last_use = best_e;
+    for (size_t k = 0; k < n; ++k) {
+      Launch &l = sched[k];
+      auto touch = [&](Launch &x) {
+        for (Operand *op : {&x.a, &x.b, &x.c, &x.d, &x.e, &x.out, &x.out2}) {
+          if (op->space != Operand::Space::Arena || op->name.empty()) continue;
+          auto it = moved.find(op->name);
+          if (it == moved.end()) continue;
+          it->second.bytes = std::max(it->second.bytes, op->Extent());
+          last_use = std::max(last_use, k);
+        }
+      };
+      touch(l);
+      for (Launch &g : l.group) touch(g);
+    }
+    size_t total = 0;
+    for (auto &kv : moved) {
+      kv.second.offset = total;
+      total += (kv.second.bytes + 255) / 256 * 256;
+    }
+    size_t slot = 0;
+    while (slot < side_free_from.size() && side_free_from[slot] > i) ++slot;
+    if (slot == side_free_from.size()) side_free_from.push_back(0);
+    side_free_from[slot] = last_use + 1;
+    const std::string buffer = "side:" + std::to_string(slot);
+    privates_[buffer].bytes = std::max(privates_[buffer].bytes, total);
     for (Launch &l : sched) {
       auto redirect = [&](Launch &x) {
         for (Operand *op : {&x.a, &x.b, &x.c, &x.d, &x.e, &x.out, &x.out2}) {
           if (op->space != Operand::Space::Arena || op->name.empty()) continue;
           auto it = moved.find(op->name);
           if (it == moved.end()) continue;
-          it->second = std::max(it->second, op->Extent());
           op->space = Operand::Space::Private;
-          op->offset = 0;
+          op->pool = buffer;
+          op->offset = it->second.offset;
         }
       };
       redirect(l);
       for (Launch &g : l.group) redirect(g);
     }
-    for (const auto &kv : moved) privates_[kv.first].bytes = std::max(privates_[kv.first].bytes, kv.second);
     i = best_e;
   }
 }

@@ -29,7 +29,8 @@ struct Operand {
   };
   Space space = Space::Arena;
   std::string name;
-  size_t offset = 0;  // Arena only
+  size_t offset = 0;  // Arena; Private inside a shared buffer
+  std::string pool;   // Private only: the shared buffer the tensor lives in at `offset` (empty: an allocation of its own)
   Meta meta{Type::kUnknown, std::vector<int64_t>{}};
   std::vector<size_t> layout;
   // A tensor that is not materialised but read through the bytes of another one (the output of an elided

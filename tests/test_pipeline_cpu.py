@@ -580,34 +580,50 @@ def test_side_branches_are_independent(mods, which, tmp_path):
     launches, regions = plan["launches"], plan["regions"]
     assert len(regions) >= at_least
     runs = lambda l: l["kind"] not in ("View", "Placed")
+
+    def touches(x, y):  # bytes of the arena, or of one buffer outside it
+        if x["space"] != y["space"]:
+            return False
+        if x["space"] in ("interface", "constant"):
+            return x["name"] == y["name"]
+        if x["space"] == "private" and (x["pool"] or x["name"]) != (y["pool"] or y["name"]):
+            return False
+        return x["offset"] < y["offset"] + y["bytes"] and y["offset"] < x["offset"] + x["bytes"]
+
     last = 0
     for a, b, e in regions:
         assert last <= a < b < e <= len(launches)
         last = e
         assert runs(launches[a]) and runs(launches[b]) and runs(launches[e - 1])
         first, second = [l for l in launches[a:b] if runs(l)], [l for l in launches[b:e] if runs(l)]
-        own = set()
+        own = []
         for y in second:
             for w in y["writes"]:
                 assert w["space"] in ("private", "interface"), "a side branch writes into the arena"
-                if w["space"] == "private":
-                    own.add(w["name"])
+                own.append(w)
             for r in y["reads"]:
                 for x in first:
-                    assert not any(_overlap(w, r) for w in x["writes"]), "a side branch reads what the other run writes"
-        for x in first:
-            for op in x["reads"] + x["writes"]:
-                assert not (op["space"] in ("private", "interface") and any(
-                    _overlap(op, w) for y in second for w in y["writes"])), "the first run touches what the side branch writes"
-        # the side branch's buffers: written only there, read only there or after the join
+                    assert not any(touches(w, r) for w in x["writes"]), "a side branch reads what the other run writes"
+        # The side branch's bytes (buffers the regions share, one after the other): it starts right behind the fork
+        # in front of the first run, so whoever else touches them has to come before that fork or behind the join.
         for k, l in enumerate(launches):
-            if not runs(l):
+            if not runs(l) or b <= k < e:
                 continue
-            outside = k < b or k >= e
-            if outside:
-                assert not any(w["space"] == "private" and w["name"] in own for w in l["writes"])
-            if k < b:
-                assert not any(r["space"] == "private" and r["name"] in own for r in l["reads"])
+            for op in l["reads"] + l["writes"]:
+                if any(touches(op, w) for w in own):
+                    assert k < a or k >= e, "the first run touches what the side branch writes"
+        # ... and a tensor of this branch is read for the last time before the fork of whichever later branch moves
+        # into its bytes
+        names = {w["name"] for w in own if w["space"] == "private"}
+        for k in range(b, len(launches)):
+            if not runs(launches[k]):
+                continue
+            for r in launches[k]["reads"]:
+                if r["space"] == "private" and r["name"] in names:
+                    for a2, b2, e2 in regions:
+                        if a2 >= e and a2 <= k:
+                            assert not any(touches(r, w2) for l2 in launches[b2:e2] if runs(l2) for w2 in l2["writes"]), \
+                                "a side branch overwrites bytes an earlier one's reader still needs"
     # without regions nothing is moved out of the arena
     ex = fluidml.Executor.make_plain_greedy("no_branches")
     ex.context().set_branch_min_us(1e9)

@@ -105,6 +105,7 @@ SIGNATURES = {
     "fluidml_hip_mul_add": [_T, _T, _T, _T, _vp],
     "fluidml_hip_add_add": [_T, _T, _T, _T, _vp],
     "fluidml_hip_rotary": [_T, _T, _T, _T, _i64, _vp],
+    "fluidml_hip_rotary_pair": [_T, _T, _T, _T, _T, _T, _i64, _vp],
     "fluidml_hip_sub_constant_lhs": [_T, _T, _f64, _vp],
     "fluidml_hip_sub_common": [_T, _T, _T, _vp],
     "fluidml_hip_mul_constant": [_T, _T, _f64, _vp],

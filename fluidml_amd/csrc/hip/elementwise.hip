@@ -572,9 +572,9 @@ struct RotaryArgs {
   int32_t x_half;      // half * (stride of x along the axis)
 };
 
-__global__ __launch_bounds__(256) void RotaryKernel(RotaryArgs p, float *__restrict__ out, const float *__restrict__ x,
-                                                    const float *__restrict__ cos_t, const float *__restrict__ sin_t) {
-  const uint32_t item = blockIdx.x * 256 + threadIdx.x;
+__device__ __forceinline__ void RotaryItem(const RotaryArgs &p, uint32_t item, float *__restrict__ out,
+                                           const float *__restrict__ x, const float *__restrict__ cos_t,
+                                           const float *__restrict__ sin_t) {
   if (item >= p.n) return;
   uint32_t rem = item, d = 0;
   int32_t off[4] = {0, 0, 0, 0};
@@ -598,8 +598,26 @@ __global__ __launch_bounds__(256) void RotaryKernel(RotaryArgs p, float *__restr
   out[off[0]] = v;
 }
 
-int LaunchRotary(const fl_tensor *x, const fl_tensor *cos_t, const fl_tensor *sin_t, const fl_tensor *out,
-                 int64_t rotary_dims, hipStream_t stream) {
+__global__ __launch_bounds__(256) void RotaryKernel(RotaryArgs p, float *__restrict__ out, const float *__restrict__ x,
+                                                    const float *__restrict__ cos_t, const float *__restrict__ sin_t) {
+  RotaryItem(p, blockIdx.x * 256 + threadIdx.x, out, x, cos_t, sin_t);
+}
+
+// Two tensors against the same tables in one launch (the queries and the keys of a layer): blockIdx.y picks the problem.
+__global__ __launch_bounds__(256) void RotaryPairKernel(RotaryArgs p0, RotaryArgs p1, float *__restrict__ out0,
+                                                        const float *__restrict__ x0, float *__restrict__ out1,
+                                                        const float *__restrict__ x1, const float *__restrict__ cos_t,
+                                                        const float *__restrict__ sin_t) {
+  const uint32_t item = blockIdx.x * 256 + threadIdx.x;
+  if (blockIdx.y == 0) RotaryItem(p0, item, out0, x0, cos_t, sin_t);
+  else RotaryItem(p1, item, out1, x1, cos_t, sin_t);
+}
+
+// validates one problem and fills its arguments (n = 0: nothing to do)
+int MakeRotaryArgs(const fl_tensor *x, const fl_tensor *cos_t, const fl_tensor *sin_t, const fl_tensor *out,
+                   int64_t rotary_dims, RotaryArgs *args) {
+  RotaryArgs &p = *args;
+  std::memset(&p, 0, sizeof(p));
   FL_CHECK(CheckView(x));
   FL_CHECK(CheckView(cos_t));
   FL_CHECK(CheckView(sin_t));
@@ -636,16 +654,35 @@ int LaunchRotary(const fl_tensor *x, const fl_tensor *cos_t, const fl_tensor *si
   }
   if (total == 0) return FL_OK;
   if (total > 0x7fffffff) return FL_ERR_TOO_LARGE;
-  RotaryArgs p;
-  std::memset(&p, 0, sizeof(p));
   p.nest = MakeNestArgs<4>(nest);
   p.n = static_cast<uint32_t>(total);
   p.rot = static_cast<uint32_t>(rotary_dims);
   p.half = static_cast<uint32_t>(rotary_dims / 2);
   p.x_half = static_cast<int32_t>((rotary_dims / 2) * x->strides[rank - 1]);
+  return FL_OK;
+}
+
+int LaunchRotary(const fl_tensor *x, const fl_tensor *cos_t, const fl_tensor *sin_t, const fl_tensor *out,
+                 int64_t rotary_dims, hipStream_t stream) {
+  RotaryArgs p;
+  FL_CHECK(MakeRotaryArgs(x, cos_t, sin_t, out, rotary_dims, &p));
+  if (p.n == 0) return FL_OK;
   FL_LAUNCH(RotaryKernel, dim3((p.n + 255) / 256), dim3(256), 0, stream, p, static_cast<float *>(out->base),
             static_cast<const float *>(x->base), static_cast<const float *>(cos_t->base),
             static_cast<const float *>(sin_t->base));
+  return LaunchStatus();
+}
+
+int LaunchRotaryPair(const fl_tensor *x0, const fl_tensor *out0, const fl_tensor *x1, const fl_tensor *out1,
+                     const fl_tensor *cos_t, const fl_tensor *sin_t, int64_t rotary_dims, hipStream_t stream) {
+  RotaryArgs p0, p1;
+  FL_CHECK(MakeRotaryArgs(x0, cos_t, sin_t, out0, rotary_dims, &p0));
+  FL_CHECK(MakeRotaryArgs(x1, cos_t, sin_t, out1, rotary_dims, &p1));
+  const uint32_t n = std::max(p0.n, p1.n);
+  if (n == 0) return FL_OK;
+  FL_LAUNCH(RotaryPairKernel, dim3((n + 255) / 256, 2), dim3(256), 0, stream, p0, p1, static_cast<float *>(out0->base),
+            static_cast<const float *>(x0->base), static_cast<float *>(out1->base), static_cast<const float *>(x1->base),
+            static_cast<const float *>(cos_t->base), static_cast<const float *>(sin_t->base));
   return LaunchStatus();
 }
 
@@ -696,6 +733,12 @@ int fluidml_hip_rotary(const fl_tensor *x, const fl_tensor *cos_table, const fl_
                        int64_t rotary_dims, void *stream) {
   if (!x || !cos_table || !sin_table || !out) return FL_ERR_NULL;
   return LaunchRotary(x, cos_table, sin_table, out, rotary_dims, AsStream(stream));
+}
+
+int fluidml_hip_rotary_pair(const fl_tensor *x0, const fl_tensor *out0, const fl_tensor *x1, const fl_tensor *out1,
+                            const fl_tensor *cos_table, const fl_tensor *sin_table, int64_t rotary_dims, void *stream) {
+  if (!x0 || !out0 || !x1 || !out1 || !cos_table || !sin_table) return FL_ERR_NULL;
+  return LaunchRotaryPair(x0, out0, x1, out1, cos_table, sin_table, rotary_dims, AsStream(stream));
 }
 
 int fluidml_hip_sub_constant_lhs(const fl_tensor *in, const fl_tensor *out, double value, void *stream) {

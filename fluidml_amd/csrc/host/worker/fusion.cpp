@@ -32,6 +32,7 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::AddAdd: return "AddAdd";
     case Launch::Kind::GatherAdd: return "GatherAdd";
     case Launch::Kind::Rotary: return "Rotary";
+    case Launch::Kind::RotaryPair: return "RotaryPair";
     case Launch::Kind::DivAddSoftmax: return "DivAddSoftmax";
     case Launch::Kind::Attention: return "Attention";
     case Launch::Kind::AddLayerNorm: return "AddLayerNormalization";
@@ -277,6 +278,11 @@ class Scheduler {
     if (fuse) ElideViews(&fused);
     if (fuse) RetryAttention(&fused);
     if (fuse) RetrySoftmaxMatVec(&fused);
+    if (fuse) {
+      MarkSilent(fused);
+      PairRotary(&fused);
+      silent_.clear();
+    }
     if (fuse) PlaceConcatInputs(&fused);
     // a chain is issued where its last member stood; everything else keeps its place
     std::vector<const Launch *> at(steps_.size(), nullptr);
@@ -1413,6 +1419,74 @@ class Scheduler {
     l->n_inner = best_view.n_inner;
     l->stride_outer = best_view.stride_outer;
     return best;
+  }
+
+  // Two Rotary launches with the same tables and extents, the second of which follows the first with nothing of
+  // consequence in between (the queries and the keys of a layer), become one launch at the position of the second:
+  // the first one's reads move there (nothing in between may write what it reads), its output appears later than
+  // planned (nothing in between may read it), and neither may write what the other reads.
+  void PairRotary(std::vector<Launch> *fused) const {
+    if (const char *v = std::getenv("FLUIDML_ROTARY_PAIR"); v != nullptr && std::string(v) == "0") return;
+    std::vector<bool> used(fused->size(), false);
+    std::vector<Launch> result;
+    for (size_t i = 0; i < fused->size(); ++i) {
+      if (used[i]) continue;
+      const Launch &x = (*fused)[i];
+      size_t partner = fused->size();
+      if (x.kind == Launch::Kind::Rotary) {
+        for (size_t j = 0; j < fused->size() && partner == fused->size(); ++j) {
+          const Launch &y = (*fused)[j];
+          if (j == i || used[j] || y.kind != Launch::Kind::Rotary || y.members.back() <= x.members.back()) continue;
+          if (!SameTensor(x.b, y.b) || !SameTensor(x.c, y.c) || x.b.viewed || y.b.viewed || x.c.viewed || y.c.viewed ||
+              x.axis != y.axis || x.a.meta.GetShape() != y.a.meta.GetShape()) {
+            continue;
+          }
+          std::vector<size_t> members = x.members;
+          members.insert(members.end(), y.members.begin(), y.members.end());
+          std::sort(members.begin(), members.end());
+          if (!Safe(members, {{x.members.front(), x.a}, {x.members.front(), x.b}, {x.members.front(), x.c},
+                              {y.members.front(), y.a}})) {
+            continue;
+          }
+          bool ok = !Alias(x.out, y.out) && !Alias(x.out, y.a) && !Alias(y.out, x.a);
+          // nobody reads the first result before the common position
+          auto rd = readers_.find(x.out.name);
+          if (rd != readers_.end()) {
+            for (size_t r : rd->second) ok = ok && r > y.members.back();
+          }
+          // its bytes, planned from its last member on, stay its own until then (written later than planned)
+          for (size_t s = x.members.back() + 1; s < y.members.back() && ok; ++s) {
+            if (std::find(members.begin(), members.end(), s) != members.end() || elided_[s]) continue;
+            const Step &st = steps_[s];
+            if (Alias(st.out, x.out) || Alias(st.in0, x.out) || (st.node->IsDoubleInputs() && Alias(st.in1, x.out))) ok = false;
+          }
+          if (ok) partner = j;
+        }
+      }
+      if (partner == fused->size()) {
+        result.push_back(x);
+        used[i] = true;
+        continue;
+      }
+      const Launch &y = (*fused)[partner];
+      Launch g;
+      g.kind = Launch::Kind::RotaryPair;
+      g.members = x.members;
+      g.members.insert(g.members.end(), y.members.begin(), y.members.end());
+      std::sort(g.members.begin(), g.members.end());
+      g.group = {x, y};
+      g.position = g.members.back();
+      g.a = x.a;
+      g.b = x.b;
+      g.c = x.c;
+      g.axis = x.axis;
+      g.out = y.out;
+      g.bytes = x.bytes + y.bytes;
+      g.flops = x.flops + y.flops;
+      used[i] = used[partner] = true;
+      result.push_back(std::move(g));
+    }
+    *fused = std::move(result);
   }
 
   // MatMulChains that read the same left operand with the same extents (the query / key / value projections)

@@ -612,6 +612,16 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
       rc = fluidml_hip_rotary(&a.t, &b.t, &c.t, &dst, l.axis, ctx.stream);
       break;
     }
+    case Launch::Kind::RotaryPair: {
+      const kernel::TensorView b = ViewOf(Resolve(l.b), l.b), c = ViewOf(Resolve(l.c), l.c);
+      const Launch &m0 = l.group[0], &m1 = l.group[1];
+      const kernel::TensorView x0 = ViewOf(Resolve(m0.a), m0.a), o0 = ViewOf(Resolve(m0.out), m0.out);
+      const kernel::TensorView x1 = ViewOf(Resolve(m1.a), m1.a), o1 = ViewOf(Resolve(m1.out), m1.out);
+      const fl_tensor d0 = m0.perm.empty() ? o0.t : Permuted(o0.t, m0.perm, true);
+      const fl_tensor d1 = m1.perm.empty() ? o1.t : Permuted(o1.t, m1.perm, true);
+      rc = fluidml_hip_rotary_pair(&x0.t, &d0, &x1.t, &d1, &b.t, &c.t, l.axis, ctx.stream);
+      break;
+    }
     case Launch::Kind::DivAddSoftmax: {
       const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
       rc = fluidml_hip_div_add_softmax(&a.t, l.s0, &b.t, &out.t, l.axis, ctx.stream);

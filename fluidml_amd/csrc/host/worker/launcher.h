@@ -83,6 +83,8 @@ struct Launch {
     Rotary,            // rotary position embedding (Slice, Neg, Concat2, MulCommon, AddCommon, Concat2 [, Transpose]):
                        // a = x, b = cosine table, c = sine table, axis = number of rotated values, perm = the
                        // folded Transpose (empty: none)
+    RotaryPair,        // two Rotary launches next to each other with the same tables (queries and keys of a layer) as
+                       // one launch: `group` holds the two, members = union of theirs, both outputs are written
     DivAddSoftmax,     // DivConstantRhs -> AddCommon(mask) -> Softmax
     Attention,         // MatMul -> Div|Mul constant [-> AddCommon(mask)] [-> Where(cond, x, scalar)] -> Softmax -> MatMul
     AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias

@@ -437,6 +437,9 @@ int fluidml_hip_add_add(const fl_tensor *a, const fl_tensor *b, const fl_tensor 
  * both products rounded before the sum, like the separate kernels (bit-identical to them).  cos and sin have R
  * values along the last axis; their leading dims broadcast to x's.  x and out: same shape, any strides. */
 int fluidml_hip_rotary(const fl_tensor *x, const fl_tensor *cos_table, const fl_tensor *sin_table, const fl_tensor *out, int64_t rotary_dims, void *stream);
+/* The same for two tensors against the same tables in ONE launch (the queries and the keys of an attention layer):
+ * out0 = rotary(x0), out1 = rotary(x1); each pair (x, out) has one shape, the two pairs may differ. */
+int fluidml_hip_rotary_pair(const fl_tensor *x0, const fl_tensor *out0, const fl_tensor *x1, const fl_tensor *out1, const fl_tensor *cos_table, const fl_tensor *sin_table, int64_t rotary_dims, void *stream);
 /* DivConstantRhsKernel -> AddCommonKernel(mask, broadcast) -> SoftmaxKernel:
  * out = softmax(in / div + mask, axis)
  * (reference div.cpp:24-56 + add.cpp:75-137 + softmax.cpp:22-139). */

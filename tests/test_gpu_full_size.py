@@ -59,7 +59,7 @@ def _full_configs():
 _EXPECTED_KINDS = {
     "bert_base": {"Attention", "MatMulGroup", "GatherAdd", "AddLayerNormalization"},
     "convbert_base": {"Attention", "SoftmaxMatVec"},
-    "gpt_neox": {"Attention", "Rotary"},
+    "gpt_neox": {"Attention", "RotaryPair"},
     "efficientnet_b0": {"ConvChain", "ConvPair"},
     "vgg16_b1": {"ConvChain", "GemmChain"},
     "vgg16_b8": {"ConvChain", "GemmChain"},

@@ -1006,6 +1006,15 @@ def test_fused_rotary(device):
             do = DeviceView(ok.View.empty(shape, np.float32, lo, fill=5), device)
             cabi.call("rotary", dx.ref(), dc.ref(), ds.ref(), do.ref(), ctypes.c_int64(rot), None)
             assert_close(do.logical(), want.logical(), exact=True, what="rotary")
+        # two tensors in one launch: x and 2x against the same tables, outputs in different layouts
+        announce("rotary pair", shape, rot, tshape)
+        d0, d1 = DeviceView(ok.View(x), device), DeviceView(ok.View((2 * x).astype(np.float32), list(range(rank))[::-1]), device)
+        dc, ds = DeviceView(ok.View(cos_t), device), DeviceView(ok.View(sin_t), device)
+        o0 = DeviceView(ok.View.empty(shape, np.float32, list(range(rank))[::-1], fill=5), device)
+        o1 = DeviceView(ok.View.empty(shape, np.float32, None, fill=5), device)
+        cabi.call("rotary_pair", d0.ref(), o0.ref(), d1.ref(), o1.ref(), dc.ref(), ds.ref(), ctypes.c_int64(rot), None)
+        assert_close(o0.logical(), want.logical(), exact=True, what="rotary pair, first")
+        assert_close(o1.logical(), 2 * want.logical(), exact=True, what="rotary pair, second")  # (doubling is exact)
     dx = DeviceView(ok.View.empty((2, 8)), device)
     dt = DeviceView(ok.View.empty((2, 3)), device)
     assert cabi.lib.fluidml_hip_rotary(dx.ref(), dt.ref(), dt.ref(), dx.ref(), 3, None) == -5  # FL_ERR_ATTR: odd

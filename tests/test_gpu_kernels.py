@@ -1375,6 +1375,12 @@ def test_conv_staged_patch(device):
         cabi.call("conv_chain", dx.ref(), dw.ref(), db.ref(), do.ref(), cabi.i64_array(pads), cabi.i64_array([1, 1]),
                   cabi.i64_array([1, 1]), ctypes.c_int64(1), ctypes.byref(relu if with_chain else none), ctypes.c_uint32(0), None)
         assert_close(do.logical(), want.logical(), what="conv with staged patch")
+        # (partial tiles of split channels are added in split order whichever workgroup arrives last: every run the same bits)
+        first = do.logical().copy()
+        for _ in range(3):
+            cabi.call("conv_chain", dx.ref(), dw.ref(), db.ref(), do.ref(), cabi.i64_array(pads), cabi.i64_array([1, 1]),
+                      cabi.i64_array([1, 1]), ctypes.c_int64(1), ctypes.byref(relu if with_chain else none), ctypes.c_uint32(0), None)
+            assert np.array_equal(do.logical(), first), "conv with staged patch: runs differ"
 
 
 def test_conv_scale_add(device):

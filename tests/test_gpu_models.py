@@ -22,6 +22,11 @@ def _cases():
                      lambda: models.bert_inputs(16, 100, seed=7)),
         "gpt_neox": (lambda: models.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120),
                      lambda: models.gpt_neox_inputs(24, 120, seed=8)),
+        # other extents: other memory plans under the same fusion passes
+        "convbert_wide": (lambda: models.convbert_base(seq=40, layers=3, hidden=96, heads=6, ffn=192, vocab=64, max_pos=64),
+                          lambda: models.bert_inputs(40, 64, seed=17)),
+        "gpt_neox_deep": (lambda: models.gpt_neox(seq=48, layers=3, hidden=128, heads=4, ffn=256, vocab=90),
+                          lambda: models.gpt_neox_inputs(48, 90, seed=18)),
         "efficientnet_b0": (lambda: models.efficientnet_b0(image=64, classes=10, width_div=4),
                             lambda: models.image_input((1, 3, 64, 64), seed=9)),
         "vgg16": (lambda: models.vgg16(batch=2, image=32, classes=10, width_div=8, fc=512),
@@ -30,7 +35,7 @@ def _cases():
 
 
 @pytest.mark.parametrize("flavour", ["plain_greedy", "dp_greedy"])
-@pytest.mark.parametrize("config", ["convbert", "gpt_neox", "efficientnet_b0", "vgg16"])
+@pytest.mark.parametrize("config", ["convbert", "gpt_neox", "efficientnet_b0", "vgg16", "convbert_wide", "gpt_neox_deep"])
 def test_config_matches_oracle(device, config, flavour, tmp_path, monkeypatch):
     from fluidml_amd import fluidml
 
@@ -53,7 +58,7 @@ def test_config_matches_oracle(device, config, flavour, tmp_path, monkeypatch):
 
 
 @pytest.mark.parametrize("use_graph", [True, False], ids=["captured", "eager"])
-@pytest.mark.parametrize("config", ["convbert", "gpt_neox", "efficientnet_b0"])
+@pytest.mark.parametrize("config", ["convbert", "gpt_neox", "efficientnet_b0", "convbert_wide", "gpt_neox_deep"])
 def test_side_branches_match_oracle(device, config, use_graph, tmp_path):
     """Independent runs of launches issued on two streams (fork, two branches, join), forced on the small graphs by
     a zero threshold: same results as the oracle, replay after replay, in a captured graph and launch by launch; what

@@ -360,6 +360,10 @@ SCHEDULE_NETS = {
     # without the rotary launch its steps go through the general mechanisms: views, Concat2 inputs written in place
     "gpt_neox_no_rotary": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120),
                            {"MatMulChain", "Attention", "View", "CopyInto", "MulAdd"}),
+    # other extents: other plans, other reuse of bytes under the same passes
+    "convbert_wide": (lambda m: m.convbert_base(seq=40, layers=3, hidden=96, heads=6, ffn=192, vocab=64, max_pos=64),
+                      {"MatMulChain", "AddLayerNormalization"}),
+    "gpt_neox_deep": (lambda m: m.gpt_neox(seq=48, layers=3, hidden=128, heads=4, ffn=256, vocab=90), {"MatMulChain", "Attention", "View"}),
     "efficientnet_b0": (lambda m: m.efficientnet_b0(image=64, classes=10, width_div=4), {"ConvChain", "ConvPair"}),
     "vgg16": (lambda m: m.vgg16(batch=2, image=32, classes=10, width_div=8, fc=512), {"ConvChain", "GemmChain"}),
 }
@@ -561,6 +565,8 @@ BRANCH_NETS = {
     "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), 0.0, 2),
     "convbert": (lambda m: m.convbert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32), 0.0, 2),
     "bert": (lambda m: m.bert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32, seed=5), 0.0, 0),
+    "convbert_wide": (lambda m: m.convbert_base(seq=40, layers=3, hidden=96, heads=6, ffn=192, vocab=64, max_pos=64), 0.0, 2),
+    "gpt_neox_deep": (lambda m: m.gpt_neox(seq=48, layers=3, hidden=128, heads=4, ffn=256, vocab=90), 0.0, 2),
     # full size with the default threshold: the attention block of a layer beside its MLP
     "gpt_neox_full": (lambda m: m.gpt_neox(), None, 3),
     "convbert_full_forced": (lambda m: m.convbert_base(), 0.0, 6),

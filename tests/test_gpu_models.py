@@ -88,3 +88,40 @@ def test_side_branches_match_oracle(device, config, use_graph, tmp_path):
         assert ex.invoke(args) > 0
         for name, ref in want.items():
             assert_close(outs[name], ref, what=f"{config} side branches {name}")
+
+
+OTHER_EXTENTS = [("convbert", (8, 1, 32, 2, 64)), ("convbert", (56, 2, 128, 4, 320)), ("convbert", (33, 3, 64, 4, 100)),
+                 ("bert", (24, 2, 96, 6, 128)), ("bert", (72, 1, 192, 12, 256)),
+                 ("gpt_neox", (8, 1, 64, 2, 64)), ("gpt_neox", (64, 3, 256, 4, 512)), ("gpt_neox", (25, 2, 128, 8, 128))]
+
+
+@pytest.mark.parametrize("family,dims", OTHER_EXTENTS, ids=str)
+def test_other_extents_match_oracle(device, family, dims, tmp_path):
+    """The transformer builders at a spread of extents (sequence lengths that are not multiples of the tiles, one to
+    three layers, 2 to 12 heads): every extent gives the memory plan other offsets and the fusion passes other
+    conflicts to respect.  With the schedule's default choices and with side branches forced, against the oracle."""
+    from fluidml_amd import fluidml, models
+
+    seq, layers, hidden, heads, ffn = dims
+    if family == "gpt_neox":
+        net, feeds = models.gpt_neox(seq=seq, layers=layers, hidden=hidden, heads=heads, ffn=ffn, vocab=70), models.gpt_neox_inputs(seq, 70, seed=4)
+    else:
+        make = models.convbert_base if family == "convbert" else models.bert_base
+        net = make(seq=seq, layers=layers, hidden=hidden, heads=heads, ffn=ffn, vocab=50, max_pos=128)
+        feeds = models.bert_inputs(seq, 50, seed=3)
+    want = graph_runner.run_graph(net, feeds)
+    path = net.save(str(tmp_path / "net.onnx"))
+    for forced in (False, True):
+        print("[case]", family, dims, "side branches forced" if forced else "default", flush=True)
+        ex = fluidml.Executor.make_plain_greedy("extents", 1)
+        if forced:
+            ex.context().set_branch_min_us(0.0)
+            ex.context().set_branch_check(False)
+        ex.compile(path)
+        args = {k: np.ascontiguousarray(v) for k, v in feeds.items()}
+        outs = {v.name: np.full(v.shape, np.nan, dtype=v.dtype) for v in net.outputs}
+        args.update(outs)
+        for _ in range(2):
+            assert ex.invoke(args) > 0
+            for name, ref in want.items():
+                assert_close(outs[name], ref, what=f"{family} {dims} {name}")

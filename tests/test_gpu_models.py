@@ -125,3 +125,34 @@ def test_other_extents_match_oracle(device, family, dims, tmp_path):
             assert ex.invoke(args) > 0
             for name, ref in want.items():
                 assert_close(outs[name], ref, what=f"{family} {dims} {name}")
+
+
+@pytest.mark.parametrize("family,dims", [("efficientnet_b0", (96, 2)), ("efficientnet_b0", (160, 4)), ("vgg16", (3, 48, 8)),
+                                         ("vgg16", (2, 96, 4)), ("vgg16", (8, 32, 4))], ids=str)
+@pytest.mark.parametrize("flavour", ["plain_greedy", "dp_greedy"])
+def test_conv_nets_other_extents_match_oracle(device, family, dims, flavour, tmp_path, monkeypatch):
+    """The convolutional builders at other image sizes, widths and batches (other tile counts: split and unsplit
+    staged-patch convolutions, plane kernels, one- and two-launch squeeze-and-excitation pairs), default and reversed
+    layouts, against the oracle."""
+    from fluidml_amd import fluidml, models
+
+    if family == "efficientnet_b0":
+        image, width_div = dims
+        net, feeds = models.efficientnet_b0(image=image, classes=7, width_div=width_div), models.image_input((1, 3, image, image), seed=9)
+    else:
+        batch, image, width_div = dims
+        net = models.vgg16(batch=batch, image=image, classes=10, width_div=width_div, fc=256)
+        feeds = models.image_input((batch, 3, image, image), seed=10)
+    want = graph_runner.run_graph(net, feeds)
+    path = net.save(str(tmp_path / "net.onnx"))
+    monkeypatch.setenv("FLUIDML_DP_COST", "constant")
+    print("[case]", family, dims, flavour, flush=True)
+    ex = getattr(fluidml.Executor, "make_" + flavour)("extents", 1)
+    ex.compile(path)
+    args = {k: np.ascontiguousarray(v) for k, v in feeds.items()}
+    outs = {v.name: np.full(v.shape, np.nan, dtype=v.dtype) for v in net.outputs}
+    args.update(outs)
+    for _ in range(2):
+        assert ex.invoke(args) > 0
+        for name, ref in want.items():
+            assert_close(outs[name], ref, what=f"{family} {dims} {flavour} {name}")

@@ -51,14 +51,22 @@ struct KernelTimer {
 };
 KernelTimer &ThreadKernelTimer();  // runtime.hip
 
+// First error of this thread's kernel launches since the last LaunchStatus().  The runtime's own "last error" is
+// shared with every other user of the runtime in the process (a failed probe inside another library stays there
+// until someone reads it), so FL_LAUNCH discards what it finds before the launch and keeps what the launch leaves.
+inline thread_local hipError_t t_launch_error = hipSuccess;
+
 #define FL_LAUNCH(kernel, grid, block, shmem, stream, ...)                                                       \
   do {                                                                                                           \
     const ::fl::KernelTimer &fl_timer_ = ::fl::ThreadKernelTimer();                                              \
+    (void)hipGetLastError();                                                                                     \
     if (fl_timer_.start != nullptr) {                                                                            \
       hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, fl_timer_.start, fl_timer_.stop, 0, __VA_ARGS__); \
     } else {                                                                                                     \
       hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                                       \
     }                                                                                                            \
+    const hipError_t fl_launch_err_ = hipGetLastError();                                                         \
+    if (fl_launch_err_ != hipSuccess && ::fl::t_launch_error == hipSuccess) ::fl::t_launch_error = fl_launch_err_; \
   } while (0)
 
 // Per-stream device memory for kernels that combine partial results across workgroups (split-K
@@ -175,7 +183,8 @@ inline int CheckChain(const fl_ew_program *g) {
 }
 
 inline int LaunchStatus() {
-  hipError_t err = hipGetLastError();
+  const hipError_t err = t_launch_error;
+  t_launch_error = hipSuccess;
   return err == hipSuccess ? FL_OK : static_cast<int>(err);
 }
 

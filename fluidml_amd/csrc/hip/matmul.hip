@@ -26,6 +26,7 @@
 // bf16 instruction replaces four fp32 ones.
 #include <algorithm>
 #include <cstdlib>
+#include <cstring>
 #include <mutex>
 #include <type_traits>
 
@@ -193,8 +194,22 @@ struct TileLoader {
 // while the first set only feeds the matrix cores from LDS (consumers).  With one workgroup per compute unit
 // the plain kernel leaves each SIMD idle while its single wave waits for loads, writes LDS or sits at the
 // barrier; here the two roles overlap.
+// DIRECT (> 0: the number of stages in the ring): WM x WN x KS waves with one 32x32 MFMA tile each, operands
+// k- resp. n-contiguous.  Tiles go from global memory straight into LDS (global_load_lds_dwordx4: every lane names
+// its own 16 global bytes, the wave's 64 pieces land in one contiguous KiB of LDS), no registers and no LDS stores
+// in between, so the number of bytes in flight is bounded by LDS (160 KB), not by registers.  A stage holds the
+// k range of one chunk (BK = 32 KS) as [32][32] sub-tiles: WM x KS of A ([m][k]) and KS x WN of B ([k][n]); wave
+// (wm, wn, ks) multiplies A(wm, ks) with B(ks, wn).  The 16-byte groups of a row of A are stored permuted (group q
+// of row m in place q ^ ((m + m / 8) % 8)) so that the 128-bit operand reads of lanes with consecutive m fall on
+// different banks without padding, which the contiguous landing area rules out.
+//   WM = WN = 1 (the waves only split K): a wave loads exactly the two sub-tiles it multiplies, so the K loop has no
+//   workgroup barrier at all -- the wave waits for its own oldest stage (vmcnt), runs its 16 MFMAs and requests
+//   the stage DIRECT - 1 ahead.
+//   Otherwise the loads of a stage are dealt evenly to the waves and one barrier per stage separates "my loads
+//   of stage t have landed" from "stage t is read"; the same barrier tells that stage t - 1 has been read by
+//   everyone, so its place is requested again right behind it.
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV = 0,
-          bool BF16 = false, bool SPEC = false, int EXTRA = 0>
+          bool BF16 = false, bool SPEC = false, int EXTRA = 0, int DIRECT = 0>
 __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(float *__restrict__ C_, const float *__restrict__ A,
                                                                 const float *__restrict__ B_, MatmulArgs p) {
   float *__restrict__ C = C_;
@@ -214,7 +229,14 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   constexpr bool QUARTER = KS == 4 && TM * TN == 1 && WM * WN == 1;
   constexpr int EV = QUARTER ? 4 : 16;  // values per lane in the tail
   constexpr int RED_ELEMS = KS > 1 ? (QUARTER ? KS : KS - 1) * BM * BN : 0;
-  constexpr int STAGE_ELEMS = 2 * (A_ELEMS + B_ELEMS);
+  constexpr int kSubTile = 1024;                            // floats of a [32][32] sub-tile (DIRECT)
+  constexpr int kRingStage = (WM + WN) * KS * kSubTile;     // floats per stage of the ring (DIRECT)
+  constexpr int kStageLoads = 4 * (WM + WN) * KS / (WM * WN * KS);  // load instructions per wave and stage (DIRECT)
+  static_assert(DIRECT == 0 || (TM * TN == 1 && BK == 32 * KS && LA == 0 && LB == 0 && VEC == 4 && CONV == 0 && !SPEC &&
+                                !BF16 && EXTRA != 2 && (4 * (WM + WN)) % (WM * WN) == 0 &&
+                                kStageLoads * (DIRECT - 1) < 64),
+                "the direct-to-LDS loop exists for one MFMA tile per wave of plain fp32 contractions");
+  constexpr int STAGE_ELEMS = DIRECT > 0 ? DIRECT * kRingStage : 2 * (A_ELEMS + B_ELEMS);
   constexpr int LDS_ELEMS = STAGE_ELEMS > RED_ELEMS ? STAGE_ELEMS : RED_ELEMS;
   __shared__ __attribute__((aligned(16))) float lds[LDS_ELEMS];
 
@@ -494,7 +516,93 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   // this workgroup's share of the chunks (all of them unless K is split over blockIdx.z)
   const int c_begin = p.n_splits > 1 ? static_cast<int>(blockIdx.z) * p.chunks_per_split : 0;
   const int c_end = p.n_splits > 1 ? min(n_chunks, c_begin + p.chunks_per_split) : n_chunks;
-  if constexpr (SPEC) {
+  if constexpr (DIRECT > 0) {
+    constexpr int R = DIRECT;
+    constexpr int NW = WM * WN * KS;
+    constexpr bool PRIVATE = WM * WN == 1;  // every wave loads only what it reads itself
+    const int n_st = c_end - c_begin;
+    const int lr8 = lane / 8, lg = lane % 8;
+    // This wave's loads of a stage: load i fills quarter j (rows 8j .. 8j+7) of sub-tile `sub`.  Per lane one global
+    // pointer for the first stage and one step per stage; rows of A past M repeat the last row, columns of B past N
+    // the first column group (their products are never stored).
+    const float *gp[kStageLoads];
+    int64_t step[kStageLoads];
+    int32_t dst[kStageLoads];  // float offset inside the stage
+#pragma unroll
+    for (int i = 0; i < kStageLoads; ++i) {
+      const int q = PRIVATE ? (i < 4 ? 4 * wave + i : 4 * KS + 4 * wave + (i - 4)) : wave * kStageLoads + i;
+      const int sub = q / 4, j = q % 4;
+      dst[i] = q * 256;
+      if (sub < WM * KS) {
+        const int swm = sub / KS, sks = sub % KS;
+        const int r = min(32 * swm + 8 * j + lr8, rows_m - 1);
+        gp[i] = Ab + static_cast<int64_t>(r) * p.sAm + (c_begin * BK + sks * 32 + 4 * (lg ^ ((lr8 + j) & 7)));
+        step[i] = BK;
+      } else {
+        const int sks = (sub - WM * KS) / WN, swn = (sub - WM * KS) % WN;
+        const int col = 32 * swn + 4 * lg;
+        gp[i] = Bb + static_cast<int64_t>(c_begin * BK + sks * 32 + 8 * j + lr8) * p.sBk + (col < cols_n ? col : -n0);
+        step[i] = static_cast<int64_t>(BK) * p.sBk;
+      }
+    }
+    float *ring = lds;
+    auto issue = [&](int t, int slot) {
+      float *at = ring + slot * kRingStage;
+#pragma unroll
+      for (int i = 0; i < kStageLoads; ++i) {
+        // (operands copied into locals first: with an array element written directly as an argument of this
+        // builtin the host pass silently drops the kernel's launch stub)
+        const float *from = gp[i] + t * step[i];
+        const int32_t to = dst[i];
+        __builtin_amdgcn_global_load_lds(from, at + to, 16, 0, 0);
+      }
+    };
+    // loads complete in order: "at most kStageLoads * later outstanding" means this wave's loads of stage t landed
+    auto wait_for = [&](int later) {
+      StaticFor<R>([&](auto n) {
+        if (later == decltype(n)::value) {
+          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStageLoads * decltype(n)::value) : "memory");
+        }
+      });
+    };
+    const int sw = (lrow + (lrow >> 3)) & 7;
+    const int a_sub = (wm * KS + ks) * kSubTile, b_sub = (WM * KS + ks * WN + wn) * kSubTile;
+#pragma unroll
+    for (int s = 0; s < R - 1; ++s) {
+      if (s < n_st) issue(s, s);
+    }
+    for (int t0 = 0; t0 < n_st; t0 += R) {
+#pragma unroll
+      for (int s = 0; s < R; ++s) {
+        const int t = t0 + s;
+        if (t < n_st) {  // uniform over the workgroup
+          // Place (s + R - 1) % R held stage t - 1.  PRIVATE: this wave's reads of it have returned (the MFMAs that
+          // use them are issued).  Shared: every wave passed this stage's barrier only after reading stage t - 1.
+          if constexpr (PRIVATE) {
+            if (t + R - 1 < n_st) issue(t + R - 1, (s + R - 1) % R);
+            wait_for(min(n_st - 1, t + R - 1) - t);
+          } else {
+            wait_for(min(n_st - 1, t + R - 2) - t);
+            __syncthreads();
+            if (t + R - 1 < n_st) issue(t + R - 1, (s + R - 1) % R);
+          }
+          const float *as = lds + s * kRingStage + a_sub;
+          const float *bs = lds + s * kRingStage + b_sub;
+#pragma unroll
+          for (int kk = 0; kk < 32; kk += 8) {
+            const floatx4 a4 = *reinterpret_cast<const floatx4 *>(as + lrow * 32 + 4 * ((kk / 4 + half) ^ sw));
+            float b4[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) b4[e] = bs[(kk + 4 * half + e) * 32 + lrow];
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.x, b4[0], acc[0][0], 0, 0, 0);
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.y, b4[1], acc[0][0], 0, 0, 0);
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.z, b4[2], acc[0][0], 0, 0, 0);
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, b4[3], acc[0][0], 0, 0, 0);
+          }
+        }
+      }
+    }
+  } else if constexpr (SPEC) {
     // Barrier j separates "chunk j is in LDS" from "chunk j is being consumed".  Producers store chunk j after
     // barrier j-1 (the consumers are then done with chunk j-2, the previous content of that buffer); consumers
     // compute chunk j after barrier j.  Both sides pass one barrier per chunk.
@@ -603,7 +711,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   // wave runs the protocol on its own slot, so no workgroup barrier is involved: the wave publishes its partial
   // tile, then one atomic tells it whether it arrived last; the last wave adds all partials in split order,
   // which makes the sum independent of arrival order.
-  if constexpr (TM * TN == 1 && (WM * WN == 1 || KS == 1)) {
+  if constexpr (TM * TN == 1 && (WM * WN == 1 || KS == 1 || DIRECT > 0)) {
     if (p.n_splits > 1) {
       const uint32_t n_splits = p.n_splits;
       const uint32_t tile_id = (blockIdx.y * n_tiles + blockIdx.x) * (WM * WN) + wm * WN + wn;
@@ -944,6 +1052,18 @@ __global__ __launch_bounds__(256) void ZeroWordsKernel(uint32_t *p, uint32_t n) 
   if (i < n) p[i] = 0u;
 }
 
+// What the caller fixed of a launch's configuration (fl_contract_tile, K splits; 0 = this file's rule decides).
+struct TileChoice {
+  int tile = FL_TILE_RULE;
+  int splits = 0;
+};
+inline TileChoice ChoiceOf(uint32_t contract_flags) {
+  TileChoice c;
+  c.tile = static_cast<int>((contract_flags >> FL_CONTRACT_TILE_SHIFT) & 0xfu);
+  c.splits = static_cast<int>((contract_flags >> FL_CONTRACT_SPLIT_SHIFT) & 0x3fu);
+  return c;
+}
+
 // Upper bound on the number of K splits per tile (environment FLUIDML_SPLITK; default 4 for the 32x32 tile and
 // 16 for the 64x64 tile; 1 = never split).
 inline int64_t SplitKLimit(int64_t fallback) {
@@ -956,14 +1076,15 @@ inline int64_t SplitKLimit(int64_t fallback) {
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV, bool BF16,
-          bool SPEC = false, int EXTRA = 0>
-void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
+          bool SPEC = false, int EXTRA = 0, int DIRECT = 0>
+int LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s,
+                 int forced_splits = 0) {
   MatmulArgs q = p;
   q.tiles_m = (p.M + BM - 1) / BM;
   q.tiles_n = (p.N + BN - 1) / BN;
   uint32_t splits = 1;
   constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);
-  if constexpr (TM * TN == 1 && (WM * WN == 1 || KS == 1)) {
+  if constexpr (TM * TN == 1 && (WM * WN == 1 || KS == 1 || DIRECT > 0)) {
     // Few tiles and a long K: give each tile to several workgroups.  Measured on MI355X (M = 128..256): with
     // about 100 tiles, 2 splits of 3 chunks of 128 (K = 768) and 4 splits of 4..6 chunks (K = 2048, 3072) win
     // by 8 % to 40 %; from about 400 tiles on, or with shorter runs of K per split, the exchange of the
@@ -981,6 +1102,15 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
     // 66 -> 61 us)
     want = std::min<int64_t>(want, SplitKLimit(few ? 16 : WM * WN == 1 ? 4 : 16));
     if (tiles > 256) want = 1;
+    if (forced_splits > 0) {
+      // the caller's number or nothing: a tuner must not time one configuration under two names
+      if (forced_splits > n_chunks ||
+          (forced_splits > 1 && static_cast<int64_t>(forced_splits) * tiles * WM * WN > static_cast<int64_t>(kWorkspaceTiles)) ||
+          (n_chunks + forced_splits - 1) / forced_splits * (forced_splits - 1) >= n_chunks) {
+        return FL_ERR_UNSUPPORTED;
+      }
+      want = forced_splits;
+    }
     if (want >= 2) {
       if (WorkspaceOverride *fixed = t_workspace_override) {
         // same split as with the stream's workspace, so the result is the same bit for bit; refused when
@@ -990,44 +1120,81 @@ void LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *
         const size_t waves = static_cast<size_t>(tiles) * WM * WN;  // one slot per wave and split
         if (waves * splits > fixed->slots || waves * 4 > fixed->n_counters) {
           fixed->error = FL_ERR_STATIC_SCRATCH;
-          return;
+          return FL_ERR_STATIC_SCRATCH;
         }
         q.partials = fixed->partials;
         q.counters = fixed->counters;
         const uint32_t n_zero = static_cast<uint32_t>(waves * 4);  // a wave owns up to four quarter counters
-        hipLaunchKernelGGL(ZeroWordsKernel, dim3((n_zero + 255) / 256), dim3(256), 0, s, fixed->counters, n_zero);
+        FL_LAUNCH(ZeroWordsKernel, dim3((n_zero + 255) / 256), dim3(256), 0, s, fixed->counters, n_zero);
       } else if (StreamWorkspace *ws = GetStreamWorkspace(s)) {
         q.chunks_per_split = static_cast<int32_t>((n_chunks + want - 1) / want);
         splits = static_cast<uint32_t>((n_chunks + q.chunks_per_split - 1) / q.chunks_per_split);
         q.partials = ws->partials;
         q.counters = ws->counters;
+      } else if (forced_splits > 1) {
+        return FL_ERR_UNSUPPORTED;  // no workspace (the stream is being captured before its first use)
       }
     }
+  } else if (forced_splits > 1) {
+    return FL_ERR_UNSUPPORTED;
   }
   q.n_splits = splits;
-  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV, BF16, SPEC, EXTRA>),
+  FL_LAUNCH((MatmulKernel<BM, BN, BK, WM, WN, KS, LA, LB, VEC, DEPTH, CONV, BF16, SPEC, EXTRA, DIRECT>),
             dim3(q.tiles_m * q.tiles_n, n_batch, splits), dim3(64 * WM * WN * KS * (SPEC ? 2 : 1)), 0, s, C, A, B, q);
+  return FL_OK;
 }
 
+// Picks the tile configuration (the caller's, or by the rule below) and launches it.  FL_ERR_UNSUPPORTED, with
+// nothing launched, when the caller's choice does not exist for these operands.
 template <int LA, int LB, int VEC, int CONV, bool BF16 = false, int EXTRA = 0>
-void LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s) {
-  const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
-  // (A 128x128x16 tile with two chunks in flight was measured slower than the 64x64x32 tile with four at
-  // every size tried -- 4096^3: 101 against 123 TFLOP/s, [256,512]x[512,50304]: 69 against 108, 3x3
-  // convolutions: 50 against 67..85 -- and is not built.)
-  // (Checked against the alternatives on the 19 contraction shapes of the five networks -- M = 49 .. 3136, K = 144 .. 3072,
-  // N = 24 .. 50304: either tile forced, split-K limits 1 .. 16 -- nothing beats this rule by more than the 1 % the
-  // measurement moves between runs.)
-  if (tiles_m >= 192 ||
-             (CONV && tiles_m * std::min<int64_t>({8, p.K / 384, static_cast<int64_t>(kWorkspaceTiles) / (tiles_m * 4)}) >= 192)) {
-    // also when splitting K over up to 8 workgroups per tile fills the chip (measured on 3x3 convolutions
-    // with 32..104 tiles: 1.5x to 2x over the 32x32 tile)
-    LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4, CONV, BF16, false, EXTRA>(p, n_batch, C, A, B, s);
-  } else {
-    // plain contractions run the 32x32 tile with producer and consumer waves (measured on BERT-base: 8.9 -> 8.6,
-    // 14.5 -> 13.6 and 15.9 -> 15.0 us for its three shapes); the convolution gather stays in the consumer waves
-    LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2, CONV, BF16, CONV == 0, EXTRA>(p, n_batch, C, A, B, s);
+int LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s,
+                 TileChoice choice = TileChoice()) {
+  // the direct-to-LDS loop: both operands on their 128-bit path, plain fp32 contraction
+  constexpr bool kDirect = LA == 0 && LB == 0 && VEC == 4 && CONV == 0 && !BF16 && EXTRA != 2;
+  int tile = choice.tile;
+  if (tile == FL_TILE_RULE) {
+    const int64_t tiles_m = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * n_batch;
+    // (A 128x128x16 tile with two chunks in flight was measured slower than the 64x64x32 tile with four at
+    // every size tried -- 4096^3: 101 against 123 TFLOP/s, [256,512]x[512,50304]: 69 against 108, 3x3
+    // convolutions: 50 against 67..85 -- and is not built.)
+    if (tiles_m >= 192 ||
+        (CONV && tiles_m * std::min<int64_t>({8, p.K / 384, static_cast<int64_t>(kWorkspaceTiles) / (tiles_m * 4)}) >= 192)) {
+      // also when splitting K over up to 8 workgroups per tile fills the chip (measured on 3x3 convolutions
+      // with 32..104 tiles: 1.5x to 2x over the 32x32 tile).  The direct loop on the same tile is level with it
+      // ([256,512]x[512,50304]: 133.3 against 133.0 us; 2048^3: 153.7 against 155.2; 4096^3: 1173 against 1130).
+      tile = FL_TILE_64x64_STAGED;
+    } else {
+      // the 32x32 tile whose four waves split K: direct loop where the operands allow it (BERT-base's four shapes:
+      // 7.9 -> 7.45, 13.1 -> 12.0, 13.55 -> 12.3, 14.7 -> 13.4 us), else staged through registers by producer waves
+      tile = kDirect && p.K % 128 == 0 ? FL_TILE_32x32_K4 : FL_TILE_32x32_STAGED;
+    }
   }
+  switch (tile) {
+    case FL_TILE_32x32_STAGED:
+      // plain contractions run producer and consumer waves (measured on BERT-base: 8.9 -> 8.6, 14.5 -> 13.6 and
+      // 15.9 -> 15.0 us for its three shapes); the convolution gather stays in the consumer waves
+      return LaunchConfig<32, 32, 128, 1, 1, 4, LA, LB, VEC, 2, CONV, BF16, CONV == 0, EXTRA>(p, n_batch, C, A, B, s,
+                                                                                              choice.splits);
+    case FL_TILE_64x64_STAGED:
+      return LaunchConfig<64, 64, 32, 2, 2, 1, LA, LB, VEC, 4, CONV, BF16, false, EXTRA>(p, n_batch, C, A, B, s, choice.splits);
+    default: break;
+  }
+  if constexpr (kDirect) {
+#define FL_DIRECT(TILE_, WM_, WN_, KS_, R_)                                                                          \
+  if (tile == TILE_) {                                                                                               \
+    if (p.K % (32 * KS_) != 0) return FL_ERR_UNSUPPORTED;                                                            \
+    return LaunchConfig<32 * WM_, 32 * WN_, 32 * KS_, WM_, WN_, KS_, 0, 0, 4, 2, 0, false, false, EXTRA, R_>(        \
+        p, n_batch, C, A, B, s, choice.splits);                                                                      \
+  }
+    // ring depths: the shallowest ones measured best everywhere (more workgroups fit a compute unit)
+    FL_DIRECT(FL_TILE_32x32_K4, 1, 1, 4, 2)
+    FL_DIRECT(FL_TILE_64x32_K2, 2, 1, 2, 2)
+    FL_DIRECT(FL_TILE_64x64, 2, 2, 1, 2)
+    FL_DIRECT(FL_TILE_64x64_K2, 2, 2, 2, 2)
+    FL_DIRECT(FL_TILE_128x64, 4, 2, 1, 3)
+#undef FL_DIRECT
+  }
+  return FL_ERR_UNSUPPORTED;
 }
 
 // Siblings of a grouped launch: same lhs, same extents and rhs strides, own rhs / bias / out buffers.
@@ -1043,7 +1210,7 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
              float cb, const fl_tensor *bias, void *stream, const fl_ew_program *chain = nullptr, int64_t n_inner = 0,
              int64_t stride_outer = 0, const Siblings *siblings = nullptr, bool bf16 = false,
              const float *addend = nullptr, const float *k_scale = nullptr, int64_t k_scale_stride = 0,
-             const float *addend2 = nullptr) {
+             const float *addend2 = nullptr, TileChoice choice = TileChoice()) {
   FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(lhs));
   FL_CHECK(CheckView(rhs));
@@ -1190,44 +1357,47 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
     p.k_scale = k_scale;
     p.sKs = static_cast<int32_t>(k_scale_stride);
   }
-  // at most 8 rows against k-contiguous weights: HBM-bound weight streaming, fp32 whatever `bf16` says
-  if (!extra && TrySkinnyGemm(p, n_batch, C, A, B, s)) return LaunchStatus();
+  // at most 8 rows against k-contiguous weights: HBM-bound weight streaming, fp32 whatever `bf16` says (a caller
+  // that names a tile configuration gets the tiled kernel)
+  const bool free_choice = choice.tile == FL_TILE_RULE && choice.splits == 0;
+  if (!extra && free_choice && TrySkinnyGemm(p, n_batch, C, A, B, s)) return LaunchStatus();
   const uint32_t nb = static_cast<uint32_t>(n_batch);
+  int rc = FL_ERR_UNSUPPORTED;
   if (extra) {
-#define FL_MM_EXTRA(E_)                                                     \
-  do {                                                                      \
-    if (la == 0 && vec) LaunchBySize<0, 0, 4, 0, false, E_>(p, nb, C, A, B, s);  \
-    else if (vec_a_only) LaunchBySize<0, 0, 41, 0, false, E_>(p, nb, C, A, B, s); \
-    else if (la == 0) LaunchBySize<0, 0, 1, 0, false, E_>(p, nb, C, A, B, s);    \
-    else if (vec) LaunchBySize<1, 0, 4, 0, false, E_>(p, nb, C, A, B, s);        \
-    else LaunchBySize<1, 0, 1, 0, false, E_>(p, nb, C, A, B, s);                 \
+#define FL_MM_EXTRA(E_)                                                                 \
+  do {                                                                                  \
+    if (la == 0 && vec) rc = LaunchBySize<0, 0, 4, 0, false, E_>(p, nb, C, A, B, s, choice);   \
+    else if (vec_a_only) rc = LaunchBySize<0, 0, 41, 0, false, E_>(p, nb, C, A, B, s, choice); \
+    else if (la == 0) rc = LaunchBySize<0, 0, 1, 0, false, E_>(p, nb, C, A, B, s, choice);     \
+    else if (vec) rc = LaunchBySize<1, 0, 4, 0, false, E_>(p, nb, C, A, B, s, choice);         \
+    else rc = LaunchBySize<1, 0, 1, 0, false, E_>(p, nb, C, A, B, s, choice);                  \
   } while (0)
     if (k_scale != nullptr) FL_MM_EXTRA(2);
     else FL_MM_EXTRA(1);
 #undef FL_MM_EXTRA
-    return LaunchStatus();
+    return rc != FL_OK ? rc : LaunchStatus();
   }
-#define FL_MM_DISPATCH(LA_, LB_)                              \
-  if (la == LA_ && lb == LB_) {                               \
-    if (bf16) {                                                   \
-      if (vec) LaunchBySize<LA_, LB_, 4, 0, true>(p, nb, C, A, B, s); \
-      else LaunchBySize<LA_, LB_, 1, 0, true>(p, nb, C, A, B, s);     \
-    } else if (vec) {                                             \
-      LaunchBySize<LA_, LB_, 4, 0>(p, nb, C, A, B, s);        \
-    } else {                                                      \
-      LaunchBySize<LA_, LB_, 1, 0>(p, nb, C, A, B, s);        \
-    }                                                             \
+#define FL_MM_DISPATCH(LA_, LB_)                                                  \
+  if (la == LA_ && lb == LB_) {                                                   \
+    if (bf16) {                                                                   \
+      if (vec) rc = LaunchBySize<LA_, LB_, 4, 0, true>(p, nb, C, A, B, s, choice); \
+      else rc = LaunchBySize<LA_, LB_, 1, 0, true>(p, nb, C, A, B, s, choice);     \
+    } else if (vec) {                                                             \
+      rc = LaunchBySize<LA_, LB_, 4, 0>(p, nb, C, A, B, s, choice);               \
+    } else {                                                                      \
+      rc = LaunchBySize<LA_, LB_, 1, 0>(p, nb, C, A, B, s, choice);               \
+    }                                                                             \
   }
   if (vec_a_only) {
-    LaunchBySize<0, 0, 41, 0>(p, nb, C, A, B, s);
-    return LaunchStatus();
+    rc = LaunchBySize<0, 0, 41, 0>(p, nb, C, A, B, s, choice);
+    return rc != FL_OK ? rc : LaunchStatus();
   }
   FL_MM_DISPATCH(0, 0)
   FL_MM_DISPATCH(0, 1)
   FL_MM_DISPATCH(1, 0)
   FL_MM_DISPATCH(1, 1)
 #undef FL_MM_DISPATCH
-  return LaunchStatus();
+  return rc != FL_OK ? rc : LaunchStatus();
 }
 
 }  // namespace
@@ -1356,15 +1526,16 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
   else vec = vec && p.sAm == 1 && p.M % 4 == 0 && p.sAk % 4 == 0;
   // four output pixels per gather when they sit in one input row at unit stride
   const bool quad = g.sw == 1 && g.sXw == 1 && OW % 4 == 0;
+  int rc = FL_ERR_UNSUPPORTED;
 #define FL_CONV_DISPATCH(LA_, VEC_)                                         \
   do {                                                                      \
     if (bf16) {                                                             \
-      if (quad) LaunchBySize<LA_, 0, VEC_, 2, true>(p, 1, C, A, B, s);      \
-      else LaunchBySize<LA_, 0, VEC_, 1, true>(p, 1, C, A, B, s);           \
+      if (quad) rc = LaunchBySize<LA_, 0, VEC_, 2, true>(p, 1, C, A, B, s); \
+      else rc = LaunchBySize<LA_, 0, VEC_, 1, true>(p, 1, C, A, B, s);      \
     } else if (quad) {                                                      \
-      LaunchBySize<LA_, 0, VEC_, 2>(p, 1, C, A, B, s);                      \
+      rc = LaunchBySize<LA_, 0, VEC_, 2>(p, 1, C, A, B, s);                 \
     } else {                                                                \
-      LaunchBySize<LA_, 0, VEC_, 1>(p, 1, C, A, B, s);                      \
+      rc = LaunchBySize<LA_, 0, VEC_, 1>(p, 1, C, A, B, s);                 \
     }                                                                       \
   } while (0)
   if (la == 0) {
@@ -1375,7 +1546,7 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
     else FL_CONV_DISPATCH(1, 1);
   }
 #undef FL_CONV_DISPATCH
-  return LaunchStatus();
+  return rc != FL_OK ? rc : LaunchStatus();
 }
 
 // Device address of the current device's copy of `scratch`, looked up on the first call per device.
@@ -1430,7 +1601,7 @@ int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const f
   if (!lhs || !rhs || !out) return FL_ERR_NULL;
   if (bias != nullptr && bias->rank != 1) return FL_ERR_RANK;
   return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, 0, 0, nullptr,
-                      (flags & FL_CONTRACT_BF16) != 0);
+                      (flags & FL_CONTRACT_BF16) != 0, nullptr, nullptr, 0, nullptr, fl::ChoiceOf(flags));
 }
 
 int fluidml_hip_matmul_chain_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
@@ -1451,9 +1622,9 @@ int fluidml_hip_matmul_chain_add(const fl_tensor *lhs, const fl_tensor *rhs, con
     }
     e[i] = static_cast<const float *>(t[i]->base);
   }
-  (void)flags;  // fp32 whatever the flags say: the extra operands exist in the fp32 instantiations only
+  // fp32 whatever the flags say: the extra operands exist in the fp32 instantiations only
   return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, 0, 0, nullptr, false, e[0], nullptr, 0,
-                      e[1]);
+                      e[1], fl::ChoiceOf(flags));
 }
 
 int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
@@ -1462,7 +1633,7 @@ int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, co
   if (!lhs || !rhs || !out) return FL_ERR_NULL;
   if (bias != nullptr && bias->rank != 1) return FL_ERR_RANK;
   return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, n_inner, stride_outer, nullptr,
-                      (flags & FL_CONTRACT_BF16) != 0);
+                      (flags & FL_CONTRACT_BF16) != 0, nullptr, nullptr, 0, nullptr, fl::ChoiceOf(flags));
 }
 
 int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs,
@@ -1484,7 +1655,8 @@ int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl
     }
   }
   return fl::Contract(lhs, rhs[0], out[0], false, false, 1.0f, 1.0f, bias != nullptr ? bias[0] : nullptr, stream, chain,
-                      n_inner, stride_outer != nullptr ? stride_outer[0] : 0, &sib, (flags & FL_CONTRACT_BF16) != 0);
+                      n_inner, stride_outer != nullptr ? stride_outer[0] : 0, &sib, (flags & FL_CONTRACT_BF16) != 0, nullptr,
+                      nullptr, 0, nullptr, fl::ChoiceOf(flags));
 }
 
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
@@ -1493,7 +1665,8 @@ int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_
   if (!lhs || !rhs || !bias || !out) return FL_ERR_NULL;
   if (lhs->rank != 2 || rhs->rank != 2 || out->rank != 2) return FL_ERR_RANK;
   return fl::Contract(lhs, rhs, out, trans_a != 0, trans_b != 0, static_cast<float>(alpha), static_cast<float>(beta),
-                      bias, stream, chain, 0, 0, nullptr, (flags & FL_CONTRACT_BF16) != 0);
+                      bias, stream, chain, 0, 0, nullptr, (flags & FL_CONTRACT_BF16) != 0, nullptr, nullptr, 0, nullptr,
+                      fl::ChoiceOf(flags));
 }
 
 int fluidml_hip_matmul_bf16(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, void *stream) {
@@ -1510,7 +1683,8 @@ int fluidml_hip_gemm_constant_weights_bias(const fl_tensor *lhs, const fl_tensor
   const float ca = static_cast<float>(swapped ? beta : alpha);
   const float cb = static_cast<float>(swapped ? alpha : beta);
   const bool bf16 = ((flags >> FL_CONTRACT_SHIFT) & FL_CONTRACT_BF16) != 0;
-  return fl::Contract(lhs, rhs, out, trans_a != 0, trans_b != 0, ca, cb, bias, stream, nullptr, 0, 0, nullptr, bf16);
+  return fl::Contract(lhs, rhs, out, trans_a != 0, trans_b != 0, ca, cb, bias, stream, nullptr, 0, 0, nullptr, bf16,
+                      nullptr, nullptr, 0, nullptr, fl::ChoiceOf(flags >> FL_CONTRACT_SHIFT));
 }
 
 }  // extern "C"

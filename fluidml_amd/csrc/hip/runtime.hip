@@ -66,7 +66,7 @@ KernelTimer &ThreadKernelTimer() {
 
 extern "C" {
 
-int fluidml_hip_abi_version(void) { return 2; }
+int fluidml_hip_abi_version(void) { return 3; }
 
 const char *fluidml_hip_error_string(int code) {
   switch (code) {

@@ -96,7 +96,8 @@ void Check(int rc, const char *what) {
 // Times launches of the real kernel on zero-filled device buffers.
 class MeasuredCostModel : public CostModel {
  public:
-  explicit MeasuredCostModel(uint32_t flags) : flags_(flags) {}
+  MeasuredCostModel(uint32_t flags, std::shared_ptr<kernel::ContractionTable> table)
+      : flags_(flags), table_(std::move(table)) {}
   ~MeasuredCostModel() override {
     for (auto &kv : buffers_) {
       for (void *p : {kv.second.lhs, kv.second.rhs, kv.second.out, kv.second.scratch}) fluidml_hip_free(p);
@@ -139,6 +140,9 @@ class MeasuredCostModel : public CostModel {
     }
     const bool single = g.IsSingleInput();
     const Layout &lhs_layout = key[0], &out_layout = key.back();
+    // MatMul / Gemm: the kernel yielded for these layouts carries the tile configuration tuned for them, as the
+    // reference's generators tune theirs before the evaluation times the result (eval.cpp:261-302)
+    g.SetContractionTable(table_);
     std::shared_ptr<kernel::Kernel> k = g.Yield(lhs_layout, single ? Layout{} : key[1], out_layout);
     k->Prepare();
     const kernel::TensorView lhs(b.lhs, g.GetLhsMeta(), lhs_layout), out(b.out, g.GetOutputMeta(), out_layout);
@@ -211,6 +215,7 @@ class MeasuredCostModel : public CostModel {
   };
   static constexpr double kBudgetPerKernelNs = 1.5e9;
   uint32_t flags_;
+  std::shared_ptr<kernel::ContractionTable> table_;
   void *stream_ = nullptr, *start_ = nullptr, *stop_ = nullptr;
   std::unordered_map<KernelEval *, Buffers> buffers_;
 };
@@ -218,7 +223,9 @@ class MeasuredCostModel : public CostModel {
 }  // namespace
 
 std::shared_ptr<CostModel> CostModel::MakeConstant() { return std::make_shared<ConstantCostModel>(); }
-std::shared_ptr<CostModel> CostModel::MakeMeasured(uint32_t ref_flags) { return std::make_shared<MeasuredCostModel>(ref_flags); }
+std::shared_ptr<CostModel> CostModel::MakeMeasured(uint32_t ref_flags, std::shared_ptr<kernel::ContractionTable> table) {
+  return std::make_shared<MeasuredCostModel>(ref_flags, std::move(table));
+}
 std::shared_ptr<CostModel> CostModel::MakeFromTable(const std::string &json_text) {
   return std::make_shared<TableCostModel>(json_text);
 }
@@ -233,7 +240,7 @@ std::shared_ptr<CostModel> CostModel::Make(context::Context &context) {
       ss << ifs.rdbuf();
       return MakeFromTable(ss.str());
     }
-    default: return MakeMeasured(context->ref_flags);
+    default: return MakeMeasured(context->ref_flags, context->contraction_table);
   }
 }
 

@@ -36,7 +36,8 @@ class CostModel {
   virtual size_t Cost(KernelEval &eval, const LayoutKey &key) = 0;
   static std::shared_ptr<CostModel> Make(context::Context &context);
   static std::shared_ptr<CostModel> MakeConstant();
-  static std::shared_ptr<CostModel> MakeMeasured(uint32_t ref_flags);
+  static std::shared_ptr<CostModel> MakeMeasured(uint32_t ref_flags,
+                                                 std::shared_ptr<kernel::ContractionTable> table = nullptr);
   // `json_text` is a report written by DynamicProgrammingTable::ToJson (bare or
   // wrapped as {"dp_table": ..., "plan": ...}); a lookup that misses throws
   static std::shared_ptr<CostModel> MakeFromTable(const std::string &json_text);

@@ -188,6 +188,29 @@ PYBIND11_MODULE(fluidml, m) {
       .def("set_bf16", [](context::Context &c, bool on) { c->bf16 = on; }, py::arg("on"))
       .def("set_branch_min_us", [](context::Context &c, double us) { c->branch_min_us = us; }, py::arg("us"))
       .def("set_branch_check", [](context::Context &c, bool on) { c->branch_check = on; }, py::arg("on"))
+      .def("set_branch_decision", [](context::Context &c, int keep) { c->branch_decision = keep; }, py::arg("keep"),
+           "1 / 0: keep / drop the side branches without timing them; negative: decide by timing")
+      .def("set_tune",
+           [](context::Context &c, const std::string &mode) {
+             using Mode = kernel::ContractionTable::Mode;
+             if (mode == "off") {
+               c->contraction_table->SetMode(Mode::Off);
+             } else if (mode == "measure") {
+               c->contraction_table->SetMode(Mode::Measure);
+             } else if (mode == "replay") {
+               c->contraction_table->SetMode(Mode::Replay);
+             } else {
+               c->LoadSavedDecisions(mode);
+               c->contraction_table->SetMode(Mode::Replay);
+             }
+           },
+           py::arg("mode"),
+           "tile configuration of the contractions: \"measure\" (time unknown problems at compile), \"off\" (the "
+           "library's rule), \"replay\" (only what the table holds), or the path of a JSON file an earlier compile wrote")
+      .def("load_contraction_table",
+           [](context::Context &c, const std::string &json_text) { c->contraction_table->LoadJsonText(json_text); },
+           py::arg("json_text"))
+      .def("contraction_table_json", [](context::Context &c) { return c->contraction_table->ToJson(); })
       .def("plan_text", [](context::Context &c) { return c->GetModule().ToText(); });
 
   py::class_<flow::Flow, std::unique_ptr<flow::Flow>>(m, "Flow")
@@ -318,7 +341,18 @@ PYBIND11_MODULE(fluidml, m) {
            "device nanoseconds of each of `iters` consecutive replays (events on the plan's stream)")
       .def("replay", [](worker::Executor &e, size_t n) { e.GetContext()->GetModule().ReplayResident(n); }, py::arg("n") = 1,
            "n replays of the plan on the tensors already in HBM, then a stream wait (no host copies)")
-      .def("materialize", [](worker::Executor &e) { e.GetContext()->GetModule().Materialize(); });
+      .def("materialize", [](worker::Executor &e) { e.GetContext()->GetModule().Materialize(); })
+      .def("contraction_choices",
+           [](worker::Executor &e) {
+             py::list out;
+             for (const auto &c : e.GetContext()->GetModule().GetContractionChoices()) {
+               const uint32_t tile = (c.second >> FL_CONTRACT_TILE_SHIFT) & 0xfu, splits = (c.second >> FL_CONTRACT_SPLIT_SHIFT) & 0x3fu;
+               out.append(py::make_tuple(c.first, tile, splits));
+             }
+             return out;
+           },
+           "(signature, tile, splits) of every MatMul / Gemm launch of the schedule; 0 = the library's rule")
+      .def("branch_decision", [](worker::Executor &e) { return e.GetContext()->GetModule().GetBranchDecision(); });
 
   py::class_<worker::Lower, std::unique_ptr<worker::Lower>>(m, "Lower").def("run", &worker::Lower::Run);
 
@@ -363,6 +397,36 @@ PYBIND11_MODULE(fluidml, m) {
     }
     return names;
   });
+  m.def("_contraction_candidates", &kernel::ContractionTable::Candidates, py::arg("full"));
+  m.def(
+      "_contraction_measure",
+      [](const std::vector<std::pair<int, int>> &candidates, const py::function &launch, const py::function &elapsed,
+         int rounds, double margin) {
+        const kernel::ContractPick p = kernel::ContractionTable::Measure(
+            candidates, [&](uint32_t bits) { return launch(bits).cast<int>(); }, [&]() { return elapsed().cast<double>(); },
+            rounds, margin);
+        return py::make_tuple(p.tile, p.splits, p.ns, p.rule_ns);
+      },
+      py::arg("candidates"), py::arg("launch"), py::arg("elapsed_ns"), py::arg("rounds") = 3, py::arg("margin") = 0.015,
+      "the tuner's selection rule on caller-supplied launch and timing functions");
+  m.def(
+      "_contraction_signature",
+      [](const std::string &path, const std::string &node_name, const std::vector<size_t> &lhs_layout,
+         const std::vector<size_t> &rhs_layout, const std::vector<size_t> &out_layout) {
+        std::unique_ptr<worker::Parser> parser = worker::Parser::Make();
+        std::unique_ptr<worker::Converter> converter = worker::Converter::Make();
+        graph::Graph graph = parser->Run(std::string_view(path));
+        flow::Flow flow = converter->Run(graph);
+        for (const std::shared_ptr<flow::Node> &node : flow.GetNodes()) {
+          if (node->GetName() == node_name) {
+            kernel::KernelGenerator g(*node);
+            return g.GetContractionSignature(lhs_layout, rhs_layout, out_layout);
+          }
+        }
+        throw std::out_of_range("no node named " + node_name);
+      },
+      py::arg("onnx_path"), py::arg("node"), py::arg("lhs_layout"), py::arg("rhs_layout"), py::arg("out_layout"),
+      "ContractionTable key of a MatMul / Gemm node's standalone kernel under the given layouts");
   m.def("_gen_all_orders", &utils::GenAllOrders);
   m.def("_gen_all_indices_in_order", &utils::GenAllIndicesInOrder);
   m.def("_gen_physical_shape", &utils::GenPhysicalShape);

@@ -1,7 +1,11 @@
 #include "structure/context/context.h"
 
 #include <cstdlib>
+#include <fstream>
+#include <sstream>
 #include <stdexcept>
+
+#include "utils/json.h"
 
 #include "evaluation/dp.h"
 #include "evaluation/eval.h"
@@ -31,6 +35,30 @@ ContextImpl::ContextImpl() {
       cost_mode = CostMode::Table;
       cost_table_path = mode;
     }
+  }
+  contraction_table = std::make_shared<kernel::ContractionTable>(kernel::ContractionTable::FromEnvironment());
+  // a saved compile replays everything it decided by timing: the layout costs (above), and from the same file the
+  // tile configurations and whether the side branches stayed
+  std::string saved = cost_mode == CostMode::Table ? cost_table_path : std::string();
+  if (const char *t = std::getenv("FLUIDML_TUNE")) {
+    const std::string v(t);
+    if (!v.empty() && v != "0" && v != "1") saved = v;
+  }
+  if (!saved.empty()) LoadSavedDecisions(saved);
+}
+
+void ContextImpl::LoadSavedDecisions(const std::string &path) {
+  std::ifstream ifs(path);
+  if (!ifs) return;  // the cost model reports a missing table itself
+  std::stringstream text;
+  text << ifs.rdbuf();
+  const json::Value doc = json::Parse(text.str());
+  if (doc.Has("contraction_table") && contraction_table->GetMode() != kernel::ContractionTable::Mode::Off) {
+    contraction_table->LoadJson(doc);
+    contraction_table->SetMode(kernel::ContractionTable::Mode::Replay);
+  }
+  if (doc.Has("side_branches") && doc.At("side_branches").Has("kept")) {
+    branch_decision = doc.At("side_branches").At("kept").boolean ? 1 : 0;
   }
 }
 

@@ -11,6 +11,7 @@
 #include <string>
 #include <vector>
 
+#include "structure/kernel/tuner.h"
 #include "structure/tensor/meta.h"
 
 namespace fluidml {
@@ -76,6 +77,8 @@ class ContextImpl {
   std::unique_ptr<worker::LaunchPlan> ReleaseModule();
   FuncAttr &GetFuncAttr();
   void SetFuncAttr(FuncAttr &&attr);
+  // reads "contraction_table" and "side_branches" of a JSON file an earlier Executor::Compile wrote
+  void LoadSavedDecisions(const std::string &path);
 
   // FL_REF_* literal-reference switches (env FLUIDML_REF_QUIRKS=<int>, default 0)
   uint32_t ref_flags = 0;
@@ -101,6 +104,14 @@ class ContextImpl {
   // faster (env FLUIDML_DP_CHECK=0 keeps the DP's proposal whatever it costs)
   bool dp_check_whole_plan = true;
   std::shared_ptr<evaluation::CostModel> cost_model;  // created on first use
+  // Tile configuration per contraction signature, shared by the kernel generators and the launch plan (the
+  // reference keeps the equivalent cache inside each MatMul / Gemm generator, generator/matmul.cpp:94-98).
+  // Mode from the environment (FLUIDML_TUNE: 0 = the library's rule, a file = replay that compile's table);
+  // a cost table given through FLUIDML_DP_COST that carries a "contraction_table" is replayed as well.
+  std::shared_ptr<kernel::ContractionTable> contraction_table;
+  // side branches of the launch plan: 1 / 0 = keep / drop them without timing (read back from a saved JSON),
+  // negative = let the first run decide by timing
+  int branch_decision = -1;
 
  private:
   std::unique_ptr<worker::LaunchPlan> module_;

@@ -3,6 +3,8 @@
 #include <functional>
 #include <stdexcept>
 
+#include "utils/utils.h"
+
 namespace fluidml {
 namespace kernel {
 
@@ -78,10 +80,102 @@ bool KernelGenerator::Equals(const KernelGenerator &o) const {
          same_tensor(a.t0, b.t0) && same_tensor(a.t1, b.t1) && same_tensor(a.t2, b.t2);
 }
 
-std::shared_ptr<Kernel> KernelGenerator::Yield(const std::vector<size_t> &, const std::vector<size_t> &,
-                                               const std::vector<size_t> &) {
-  if (!kernel_) kernel_ = MakeKernel(kind_, attrs_);
-  return kernel_;
+namespace {
+std::vector<size_t> LayoutOr(const std::vector<size_t> &layout, const Meta &meta) {
+  return layout.empty() ? utils::GenDefaultLayout(meta.GetShape()) : layout;
+}
+void CheckHip(int rc, const char *what) {
+  if (rc != 0) throw std::runtime_error(std::string(what) + ": " + fluidml_hip_error_string(rc));
+}
+}  // namespace
+
+std::string KernelGenerator::GetContractionSignature(const std::vector<size_t> &lhs_layout,
+                                                     const std::vector<size_t> &rhs_layout,
+                                                     const std::vector<size_t> &output_layout) const {
+  if (!IsContraction()) return std::string();
+  // views at address 0: dense and 16-byte aligned, which is how the reference's generator fills its buffers too
+  TensorView lhs(nullptr, lhs_meta_, LayoutOr(lhs_layout, lhs_meta_));
+  TensorView rhs(nullptr, *rhs_meta_, LayoutOr(rhs_layout, *rhs_meta_));
+  const TensorView out(nullptr, output_meta_, LayoutOr(output_layout, output_meta_));
+  std::string epilogue = "standalone";
+  if (kind_ == flow::OpKind::GemmConstantWeightsBias) {
+    epilogue = std::string("gemm ta") + (attrs_.trans_a ? "1" : "0") + " tb" + (attrs_.trans_b ? "1" : "0");
+  }
+  return ContractionTable::Signature(KernelNameOf(kind_), lhs.t, rhs.t, out.t, 1, epilogue);
+}
+
+ContractPick KernelGenerator::MeasureStandalone(Kernel &kernel, const std::vector<size_t> &lhs_layout,
+                                                const std::vector<size_t> &rhs_layout,
+                                                const std::vector<size_t> &output_layout) const {
+  // what the reference's generator does with FillBuffer'd host vectors and its Runner (generator/matmul.cpp:100-124)
+  void *lhs_d = nullptr, *rhs_d = nullptr, *out_d = nullptr, *stream = nullptr, *start = nullptr, *stop = nullptr;
+  ContractPick pick;
+  auto release = [&]() {
+    fluidml_hip_time_kernels(nullptr, nullptr);
+    for (void *p : {lhs_d, rhs_d, out_d}) fluidml_hip_free(p);
+    if (start) fluidml_hip_event_destroy(start);
+    if (stop) fluidml_hip_event_destroy(stop);
+    if (stream) fluidml_hip_stream_destroy(stream);
+  };
+  try {
+    CheckHip(fluidml_hip_arena_create(lhs_meta_.GetSize(), &lhs_d), "tuning buffer");
+    CheckHip(fluidml_hip_arena_create(rhs_meta_->GetSize(), &rhs_d), "tuning buffer");
+    CheckHip(fluidml_hip_arena_create(output_meta_.GetSize(), &out_d), "tuning buffer");
+    CheckHip(fluidml_hip_stream_create(&stream), "tuning stream");
+    CheckHip(fluidml_hip_event_create(&start), "tuning event");
+    CheckHip(fluidml_hip_event_create(&stop), "tuning event");
+    kernel.Prepare();
+    const TensorView lhs(lhs_d, lhs_meta_, LayoutOr(lhs_layout, lhs_meta_));
+    const TensorView rhs(rhs_d, *rhs_meta_, LayoutOr(rhs_layout, *rhs_meta_));
+    const TensorView out(out_d, output_meta_, LayoutOr(output_layout, output_meta_));
+    auto &runnable = dynamic_cast<DoubleInputsWithoutBufferKernel &>(kernel);
+    CheckHip(fluidml_hip_time_kernels(start, stop), "kernel timing on");
+    auto launch = [&](uint32_t bits) {
+      LaunchContext ctx;
+      ctx.stream = stream;
+      ctx.contract = bits;
+      runnable.Run(ctx, lhs, rhs, out);
+      return ctx.status;
+    };
+    auto elapsed = [&]() {
+      double ns = 0;
+      CheckHip(fluidml_hip_event_elapsed_ns(start, stop, &ns), "elapsed");
+      return ns;
+    };
+    pick = ContractionTable::Measure(ContractionTable::Candidates(false), launch, elapsed, 3, kTuneMargin);
+  } catch (...) {
+    release();
+    throw;
+  }
+  release();
+  return pick;
+}
+
+std::shared_ptr<Kernel> KernelGenerator::Yield(const std::vector<size_t> &lhs_layout, const std::vector<size_t> &rhs_layout,
+                                               const std::vector<size_t> &output_layout) {
+  if (!IsContraction()) {
+    if (!kernel_) kernel_ = MakeKernel(kind_, attrs_);
+    return kernel_;
+  }
+  // one kernel per layout triple, carrying the tile configuration picked for it (reference generator/matmul.cpp:94-98:
+  // `kernels_.find({lhs_layout, rhs_layout, output_layout})`)
+  const LayoutTriple key{LayoutOr(lhs_layout, lhs_meta_), LayoutOr(rhs_layout, *rhs_meta_), LayoutOr(output_layout, output_meta_)};
+  auto it = kernels_.find(key);
+  if (it != kernels_.end()) return it->second;
+  std::shared_ptr<Kernel> kernel = MakeKernel(kind_, attrs_);
+  if (table_ != nullptr && table_->GetMode() != ContractionTable::Mode::Off) {
+    const std::string signature = GetContractionSignature(lhs_layout, rhs_layout, output_layout);
+    ContractPick pick;
+    bool known = table_->Find(signature, &pick);
+    if (!known && table_->GetMode() == ContractionTable::Mode::Measure && fluidml_hip_device_count() > 0) {
+      pick = MeasureStandalone(*kernel, lhs_layout, rhs_layout, output_layout);
+      table_->Put(signature, pick);
+      known = true;
+    }
+    if (known) kernel->SetContractFlags(pick.Flags());
+  }
+  kernels_.insert({key, kernel});
+  return kernel;
 }
 
 std::shared_ptr<Kernel> KernelGenerator::YieldSingleInputKernel(const std::vector<size_t> &input_layout,

@@ -1,20 +1,28 @@
 // Per-node kernel factories (reference include/structure/kernel/generator/generator.h:11-141).
 // A generator knows a node's metas and attributes and yields the kernel for a
 // given choice of operand layouts.  On this backend a kernel reads strides
-// from its views at launch, so the yielded object does not depend on the
-// layouts; the layouts still key the cost cache of the layout DP, and two
-// generators that ShapeEquals share one cost-table entry exactly as in the
-// reference (generator.cpp:8-42: same generator type and same metas, attributes
-// ignored).
+// from its views at launch, so for most kinds the yielded object does not
+// depend on the layouts.  MatMul and Gemm are the exception, as in the
+// reference, whose generators time their kernel's variants for the layouts
+// asked for and cache the fastest per layout triple
+// (generator/matmul.cpp:88-131, gemm.cpp:106-151): here the variants are the
+// tile configurations of the contraction kernel, looked up in -- or measured
+// into -- the ContractionTable the generator was given.  The layouts also key
+// the cost cache of the layout DP, and two generators that ShapeEquals share
+// one cost-table entry exactly as in the reference (generator.cpp:8-42: same
+// generator type and same metas, attributes ignored).
 #ifndef FLUIDML_AMD_HOST_STRUCTURE_KERNEL_GENERATOR_H_
 #define FLUIDML_AMD_HOST_STRUCTURE_KERNEL_GENERATOR_H_
 
+#include <map>
 #include <memory>
 #include <string>
+#include <tuple>
 #include <vector>
 
 #include "structure/flow/flow.h"
 #include "structure/kernel/kernel.h"
+#include "structure/kernel/tuner.h"
 
 namespace fluidml {
 namespace kernel {
@@ -41,6 +49,14 @@ class KernelGenerator {
   size_t GetHashCode() const;
   bool Equals(const KernelGenerator &other) const;
 
+  // Where MatMul / Gemm generators look up (and, in its Measure mode, record) the tile configuration of the kernels
+  // they yield.  Without a table every kernel launches with the library's rule.
+  void SetContractionTable(std::shared_ptr<ContractionTable> table) { table_ = std::move(table); }
+  // The problem signature of this node's contraction under the given layouts, operands dense and aligned
+  // (the key of the ContractionTable); empty for kinds other than MatMul / Gemm.
+  std::string GetContractionSignature(const std::vector<size_t> &lhs_layout, const std::vector<size_t> &rhs_layout,
+                                      const std::vector<size_t> &output_layout) const;
+
   // The four Yield* of the reference collapse to one: the family is the node's.
   std::shared_ptr<Kernel> Yield(const std::vector<size_t> &lhs_layout, const std::vector<size_t> &rhs_layout,
                                 const std::vector<size_t> &output_layout);
@@ -58,7 +74,14 @@ class KernelGenerator {
   Meta output_meta_;
   bool has_buffer_;
   size_t buffer_size_;
-  std::shared_ptr<Kernel> kernel_;  // created once, shared by every Yield
+  using LayoutTriple = std::tuple<std::vector<size_t>, std::vector<size_t>, std::vector<size_t>>;
+  bool IsContraction() const { return kind_ == flow::OpKind::MatMul || kind_ == flow::OpKind::GemmConstantWeightsBias; }
+  // times the admissible tile configurations of the standalone kernel on zero-filled buffers of its own
+  ContractPick MeasureStandalone(Kernel &kernel, const std::vector<size_t> &lhs_layout, const std::vector<size_t> &rhs_layout,
+                                 const std::vector<size_t> &output_layout) const;
+  std::shared_ptr<Kernel> kernel_;  // kinds other than MatMul / Gemm: created once, shared by every Yield
+  std::map<LayoutTriple, std::shared_ptr<Kernel>> kernels_;  // MatMul / Gemm: one per layout triple, with its pick
+  std::shared_ptr<ContractionTable> table_;
 };
 
 }  // namespace kernel

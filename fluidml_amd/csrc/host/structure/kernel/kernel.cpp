@@ -88,8 +88,16 @@ class Base : virtual public Kernel {
     }
     return n;
   }
+  void SetContractFlags(uint32_t bits) override { contract_ = bits; }
+  uint32_t GetContractFlags() const override { return contract_; }
 
  protected:
+  // fl_contract_flags of a launch: the bf16 switch of the context plus the tile configuration (the context's, else
+  // this kernel's own)
+  uint32_t ContractBits(const LaunchContext &ctx) const {
+    return (ctx.bf16 ? static_cast<uint32_t>(FL_CONTRACT_BF16) : 0u) | (ctx.contract != 0 ? ctx.contract : contract_);
+  }
+  uint32_t contract_ = 0;
   const DeviceConstant &Const(const std::unique_ptr<DeviceConstant> &c, const char *what) const {
     if (!c) throw std::logic_error(GetKernelName() + ": missing constant " + what);
     return *c;
@@ -229,11 +237,6 @@ class SingleWithBuffer final : public SingleInputWithBufferKernel, public Base {
   }
 };
 
-// fl_contract_flags of the launch context, placed where the entry points that also take fl_ref_flags expect them
-inline uint32_t ContractBits(const LaunchContext &ctx) {
-  return ctx.bf16 ? static_cast<uint32_t>(FL_CONTRACT_BF16) << FL_CONTRACT_SHIFT : 0u;
-}
-
 class DoubleNoBuffer final : public DoubleInputsWithoutBufferKernel, public Base {
  public:
   using Base::Base;
@@ -247,18 +250,23 @@ class DoubleNoBuffer final : public DoubleInputsWithoutBufferKernel, public Base
       case OpKind::MulCommon: rc = fluidml_hip_mul_common(l, r, out, s); break;
       case OpKind::DivCommon: rc = fluidml_hip_div_common(l, r, out, s); break;
       case OpKind::Concat2: rc = fluidml_hip_concat2(l, r, out, NormAxis(attrs_.axis, out->rank), s); break;
-      case OpKind::MatMul: rc = ctx.bf16 ? fluidml_hip_matmul_bf16(l, r, out, s) : fluidml_hip_matmul(l, r, out, s); break;
+      case OpKind::MatMul: {
+        const uint32_t bits = ContractBits(ctx);
+        // (the chain entry point with neither bias nor chain is the plain product, and takes the configuration)
+        rc = bits == 0 ? fluidml_hip_matmul(l, r, out, s) : fluidml_hip_matmul_chain(l, r, nullptr, out, nullptr, bits, s);
+        break;
+      }
       case OpKind::GemmConstantWeightsBias: {
         const TensorView bias = Const(c0_, "bias").View();
         rc = fluidml_hip_gemm_constant_weights_bias(l, r, &bias.t, out, attrs_.alpha, attrs_.beta, attrs_.trans_a ? 1 : 0,
-                                                    attrs_.trans_b ? 1 : 0, ctx.flags | ContractBits(ctx), s);
+                                                    attrs_.trans_b ? 1 : 0, ctx.flags | (ContractBits(ctx) << FL_CONTRACT_SHIFT), s);
         break;
       }
       case OpKind::ConvWithoutPadding: {
         TensorView bias;
         if (c0_) bias = c0_->View();
         rc = fluidml_hip_conv_without_padding(l, r, c0_ ? &bias.t : nullptr, out, attrs_.strides.data(),
-                                              attrs_.dilations.data(), attrs_.group, ctx.flags | ContractBits(ctx), s);
+                                              attrs_.dilations.data(), attrs_.group, ctx.flags | (ContractBits(ctx) << FL_CONTRACT_SHIFT), s);
         break;
       }
       default: break;
@@ -278,7 +286,7 @@ class DoubleWithBuffer final : public DoubleInputsWithBufferKernel, public Base 
       if (c0_) bias = c0_->View();
       rc = fluidml_hip_conv_with_padding(&lhs.t, &rhs.t, c0_ ? &bias.t : nullptr, &output.t, buffer.ptr, buffer.bytes,
                                          attrs_.pads.data(), attrs_.strides.data(), attrs_.dilations.data(), attrs_.group,
-                                         ctx.flags | ContractBits(ctx), ctx.stream);
+                                         ctx.flags | (ContractBits(ctx) << FL_CONTRACT_SHIFT), ctx.stream);
     }
     ctx.Note(rc, GetKernelName());
   }

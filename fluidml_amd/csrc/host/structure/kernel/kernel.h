@@ -33,6 +33,9 @@ struct LaunchContext {
   void *stream = nullptr;  // hipStream_t
   uint32_t flags = 0;      // FL_REF_* literal-reference switches
   bool bf16 = false;       // MatMul on the opt-in bf16 path (operands rounded to bf16, fp32 accumulation)
+  // tile configuration and K splits for the contraction about to be launched (FL_CONTRACT_TILE / FL_CONTRACT_SPLITS
+  // bits); 0: the kernel object's own choice, and failing that the library's rule
+  uint32_t contract = 0;
   int status = 0;          // first non-zero return code of the C ABI
   std::string failed;      // kernel name that produced it
   void Note(int code, const std::string &kernel_name);
@@ -83,6 +86,11 @@ class Kernel {
     (void)i;
     return nullptr;
   }
+  // MatMul / Gemm: the tile configuration this kernel object launches with (FL_CONTRACT_TILE / FL_CONTRACT_SPLITS
+  // bits, 0 = the library's rule) -- what the reference's generator fixes by picking one of its loop orders
+  // (generator/matmul.cpp:88-131).  Ignored by every other kernel.
+  virtual void SetContractFlags(uint32_t bits) { (void)bits; }
+  virtual uint32_t GetContractFlags() const { return 0; }
 };
 
 class SingleInputKernel : virtual public Kernel {};

@@ -131,6 +131,7 @@ class GeneralBuilderImpl : public GeneralBuilder {
       step.node = node;
       if (from_generators_) {
         std::unique_ptr<kernel::KernelGenerator> generator = SelectKernelGenerator(node.get());
+        generator->SetContractionTable(context_->contraction_table);
         step.kernel = generator->Yield(node->GetLhs()->GetLayout(),
                                        node->IsDoubleInputs() ? node->GetRhs()->GetLayout() : std::vector<size_t>{},
                                        node->GetOutput()->GetLayout());
@@ -155,6 +156,8 @@ class GeneralBuilderImpl : public GeneralBuilder {
     plan->SetBf16(context_->bf16);
     if (context_->branch_min_us >= 0) plan->SetBranchMinUs(context_->branch_min_us);
     plan->SetBranchCheck(context_->branch_check);
+    plan->SetBranchDecision(context_->branch_decision);
+    plan->SetContractionTable(context_->contraction_table);
     context_->SetModule(std::move(plan));
     context_->SetFuncAttr(std::move(func_attr));
   }

@@ -8,6 +8,7 @@
 #include <sstream>
 #include <stdexcept>
 
+#include "fluidml_hip.h"
 #include "utils/json.h"
 
 #include "worker/builder.h"
@@ -37,6 +38,12 @@ class ExecutorImpl : public Executor {
     } else if (flavour_ == Flavour::DPGreedy && context_->cost_mode == context::CostMode::Table && context_->dp_check_whole_plan) {
       dp_json = ReplayDecision(model, std::move(dp_json));
     }
+    // Everything else that is decided by timing is decided now, so that the JSON below records it and a later
+    // compile can repeat it: the tile configuration of every contraction launch (timed inside the schedule when
+    // the plan goes onto the device) and whether the side branches of the schedule stay.  Without a device the
+    // plan stays on the host and both are settled by the first Invoke.
+    if (fluidml_hip_device_count() > 0) context_->GetModule().Settle();
+    dp_json = WithDecisions(std::move(dp_json));
     if (json) *json << dp_json;
     if (mlir) *mlir << context_;
     if (llvm) *llvm << context_;
@@ -120,9 +127,28 @@ class ExecutorImpl : public Executor {
     return Decide(keep_dp, plain, std::move(dp_json), timing);
   }
 
+  // The planner's JSON (empty for the plain planners) with the decisions this backend takes by measurement added:
+  // "contraction_table" (signature -> tile, splits, measured ns) and "side_branches" ({"kept": bool}).  The
+  // reference's two keys stay where its tools look for them.
+  std::string WithDecisions(std::string &&dp_json) {
+    std::string extra;
+    const kernel::ContractionTable &table = *context_->contraction_table;
+    if (table.GetMode() != kernel::ContractionTable::Mode::Off && table.Size() > 0) {
+      extra += "\"contraction_table\":" + table.ToJson();
+    }
+    const int kept = context_->HasModule() ? context_->GetModule().GetBranchDecision() : -1;
+    if (kept >= 0) extra += std::string(extra.empty() ? "" : ",") + "\"side_branches\":{\"kept\":" + (kept ? "true" : "false") + "}";
+    if (extra.empty()) return std::move(dp_json);
+    if (dp_json.empty() || dp_json == "null") return "{" + extra + "}";  // the plain planners have no JSON of their own
+    if (dp_json.back() != '}') throw std::logic_error("Executor: the planner's JSON is not an object");
+    return dp_json.substr(0, dp_json.size() - 1) + "," + extra + "}";
+  }
+
   // a context with this one's switches and nothing built
   context::Context PlainTwin() {
     context::Context plain;
+    plain->contraction_table = context_->contraction_table;
+    plain->branch_decision = context_->branch_decision;
     plain->ref_flags = context_->ref_flags;
     plain->use_graph = context_->use_graph;
     plain->fuse = context_->fuse;

@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <chrono>
+#include <limits>
 #include <cstdlib>
 #include <map>
 #include <sstream>
@@ -169,6 +170,7 @@ void LaunchPlan::Materialize() {
   }
   for (Step &s : steps_) s.kernel->Prepare();
   Check(fluidml_hip_arena_create(arena_bytes_, &arena_), "allocating the arena");
+  TuneContractions();
 }
 
 void *LaunchPlan::Resolve(const Operand &op) const {
@@ -412,7 +414,7 @@ void LaunchPlan::PlanBranches() const {
 }
 
 void LaunchPlan::IssueStep(kernel::LaunchContext &ctx, const Step &s, const Operand *in0_view,
-                           const Operand *in1_view, const Operand *out_view) const {
+                           const Operand *in1_view, const Operand *out_view, int *rc_out) const {
   const Operand &op0 = in0_view ? *in0_view : s.in0, &opo = out_view ? *out_view : s.out;
   const kernel::TensorView in0 = ViewOf(Resolve(op0), op0), out = ViewOf(Resolve(opo), opo);
   const kernel::Buffer buffer{s.has_buffer ? static_cast<char *>(arena_) + s.buffer_offset : nullptr, s.buffer_bytes};
@@ -425,6 +427,12 @@ void LaunchPlan::IssueStep(kernel::LaunchContext &ctx, const Step &s, const Oper
     const kernel::TensorView in1 = ViewOf(Resolve(op1), op1);
     if (s.has_buffer) dynamic_cast<kernel::DoubleInputsWithBufferKernel &>(*k).Run(ctx, in0, in1, out, buffer);
     else dynamic_cast<kernel::DoubleInputsWithoutBufferKernel &>(*k).Run(ctx, in0, in1, out);
+  }
+  if (rc_out != nullptr) {
+    *rc_out = ctx.status;
+    ctx.status = 0;
+    ctx.failed.clear();
+    return;
   }
   if (ctx.status != 0) {
     throw std::runtime_error("launching " + ctx.failed + " for node '" + s.node->GetName() + "': " +
@@ -450,15 +458,19 @@ fl_tensor Permuted(const fl_tensor &t, const std::vector<int64_t> &perm, bool in
 }
 }  // namespace
 
-void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
+void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out) const {
+  if (rc_out != nullptr) *rc_out = 0;
   if (l.kind == Launch::Kind::View || l.kind == Launch::Kind::Placed) return;  // nothing runs
   if (l.kind == Launch::Kind::Step) {
+    const uint32_t before = ctx.contract;
+    ctx.contract = l.contract;
     IssueStep(ctx, steps_[l.members[0]], l.rewired ? &l.a : nullptr, l.rewired ? &l.b : nullptr,
-              l.rewired ? &l.out : nullptr);
+              l.rewired ? &l.out : nullptr, rc_out);
+    ctx.contract = before;
     return;
   }
   const kernel::TensorView a = ViewOf(Resolve(l.a), l.a), out = ViewOf(Resolve(l.out), l.out);
-  const uint32_t contract_flags = ctx.bf16 ? FL_CONTRACT_BF16 : 0u;
+  const uint32_t contract_flags = (ctx.bf16 ? FL_CONTRACT_BF16 : 0u) | l.contract;
   int rc = FL_ERR_UNSUPPORTED;
   switch (l.kind) {
     case Launch::Kind::MatMulChain: {
@@ -684,6 +696,10 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l) const {
     }
     default: break;
   }
+  if (rc_out != nullptr) {
+    *rc_out = rc;
+    return;
+  }
   if (rc != 0) {
     ctx.Note(rc, LaunchKindName(l.kind));
     throw std::runtime_error(std::string("launching fused ") + LaunchKindName(l.kind) + " ending at node '" +
@@ -788,11 +804,10 @@ size_t LaunchPlan::Run(const std::unordered_map<std::string, void *> &args, size
 void LaunchPlan::DecideBranches() {
   if (branches_decided_) return;
   branches_decided_ = true;
-  static const bool env_check = [] {
-    const char *v = std::getenv("FLUIDML_BRANCH_CHECK");
-    return v == nullptr || std::strtol(v, nullptr, 10) != 0;
-  }();
-  if (regions_.empty() || !branch_check_ || !env_check) return;
+  had_regions_ = !regions_.empty();
+  const char *env = std::getenv("FLUIDML_BRANCH_CHECK");
+  const bool env_check = env == nullptr || std::strtol(env, nullptr, 10) != 0;
+  if (regions_.empty() || (branch_decision_ < 0 && (!branch_check_ || !env_check))) return;
   auto rebuild = [&](bool off) {
     Check(fluidml_hip_stream_synchronize(stream_), "waiting for the timed replays");
     if (graph_ != nullptr) {
@@ -802,11 +817,254 @@ void LaunchPlan::DecideBranches() {
     branches_off_ = off;
     schedule_built_ = false;
     GetSchedule();
+    ApplyContractionPicks();
   };
-  const double with = TimeReplayNs(2, 12);
-  rebuild(true);
-  const double without = TimeReplayNs(2, 12);
-  if (with < 0.985 * without) rebuild(false);  // (the same regions and the same buffers again: planning is deterministic)
+  if (branch_decision_ >= 0) {
+    // the decision of an earlier compile, read back from its JSON: nothing is timed
+    if (branch_decision_ == 0) rebuild(true);
+  } else {
+    const double with = TimeReplayNs(2, 12);
+    rebuild(true);
+    const double without = TimeReplayNs(2, 12);
+    if (with < 0.985 * without) rebuild(false);  // (the same regions and the same buffers again: planning is deterministic)
+  }
+  if (branches_off_) {
+    // nothing writes the side branches' buffers any more
+    for (auto it = privates_.begin(); it != privates_.end();) {
+      if (it->first.compare(0, 5, "side:") == 0) {
+        fluidml_hip_free(it->second.device);
+        it = privates_.erase(it);
+      } else {
+        ++it;
+      }
+    }
+  }
+}
+
+// ---- tile configurations of the contraction launches ----------------------------------------------------------
+
+namespace {
+bool IsContractionStep(const Step &s) {
+  const flow::OpKind k = s.node->GetKind();
+  return k == flow::OpKind::MatMul || k == flow::OpKind::GemmConstantWeightsBias;
+}
+
+void OperandSignature(std::ostream &os, const Operand &op) {
+  const std::vector<int64_t> &shape = op.meta.GetShape();
+  os << "[";
+  for (size_t i = 0; i < shape.size(); ++i) os << (i ? "," : "") << shape[i];
+  os << "]";
+  int64_t first_byte = 0;
+  if (op.viewed) {
+    os << "v(";
+    for (size_t i = 0; i < op.view_strides.size(); ++i) os << (i ? "," : "") << op.view_strides[i];
+    os << ")";
+    first_byte = op.view_offset * static_cast<int64_t>(GetSize(op.meta.GetType()));
+  } else {
+    os << "l(";
+    for (size_t i = 0; i < op.layout.size(); ++i) os << (i ? "," : "") << op.layout[i];
+    os << ")";
+  }
+  // arena and pooled private tensors sit at byte offsets of the memory plan inside 256-byte aligned allocations;
+  // everything else is an allocation of its own
+  if (op.space == Operand::Space::Arena || (op.space == Operand::Space::Private && !op.pool.empty())) {
+    first_byte += static_cast<int64_t>(op.offset);
+  }
+  os << (first_byte % 16 == 0 ? "a" : "u");
+}
+}  // namespace
+
+std::string LaunchPlan::ContractionSignature(size_t i) const {
+  const Launch &l = GetSchedule().at(i);
+  std::ostringstream os;
+  auto chain_tag = [&](const Launch &x) {
+    os << " b" << (x.has_c ? 1 : 0) << "c" << x.chain.n << "s" << (x.has_skip ? (x.has_skip2 ? 2 : 1) : 0);
+    if (!x.view_strides.empty()) {
+      os << " view(";
+      for (size_t d = 0; d < x.view_strides.size(); ++d) os << (d ? "," : "") << x.view_strides[d];
+      os << ")i" << x.n_inner << "o" << x.stride_outer;
+    }
+  };
+  switch (l.kind) {
+    case Launch::Kind::Step: {
+      const Step &s = steps_[l.members[0]];
+      if (!IsContractionStep(s)) return std::string();
+      os << s.kernel->GetKernelName() << " ";
+      OperandSignature(os, l.rewired ? l.a : s.in0);
+      os << "x";
+      OperandSignature(os, l.rewired ? l.b : s.in1);
+      os << "->";
+      OperandSignature(os, l.rewired ? l.out : s.out);
+      const flow::Attrs &at = s.node->GetAttrs();
+      os << " ta" << (at.trans_a ? 1 : 0) << "tb" << (at.trans_b ? 1 : 0);
+      break;
+    }
+    case Launch::Kind::MatMulChain:
+    case Launch::Kind::GemmChain: {
+      os << LaunchKindName(l.kind) << " ";
+      OperandSignature(os, l.a);
+      os << "x";
+      OperandSignature(os, l.b);
+      os << "->";
+      OperandSignature(os, l.out);
+      chain_tag(l);
+      if (l.kind == Launch::Kind::GemmChain) {
+        const flow::Attrs &at = steps_[l.owner].node->GetAttrs();
+        os << " ta" << (at.trans_a ? 1 : 0) << "tb" << (at.trans_b ? 1 : 0);
+      }
+      break;
+    }
+    case Launch::Kind::MatMulGroup: {
+      os << LaunchKindName(l.kind) << " ";
+      OperandSignature(os, l.a);
+      for (const Launch &m : l.group) {
+        os << " x";
+        OperandSignature(os, m.b);
+        os << "->";
+        OperandSignature(os, m.out);
+        chain_tag(m);
+      }
+      break;
+    }
+    default: return std::string();
+  }
+  if (bf16_) os << " bf16";
+  return os.str();
+}
+
+void LaunchPlan::ApplyContractionPicks() const {
+  const std::vector<Launch> &schedule = GetSchedule();
+  for (size_t i = 0; i < schedule.size(); ++i) {
+    schedule_[i].contract = 0;
+    if (table_ == nullptr || table_->GetMode() == kernel::ContractionTable::Mode::Off) continue;
+    const std::string signature = ContractionSignature(i);
+    kernel::ContractPick pick;
+    if (!signature.empty() && table_->Find(signature, &pick)) schedule_[i].contract = pick.Flags();
+  }
+}
+
+std::vector<std::pair<std::string, uint32_t>> LaunchPlan::GetContractionChoices() const {
+  std::vector<std::pair<std::string, uint32_t>> out;
+  const std::vector<Launch> &schedule = GetSchedule();
+  for (size_t i = 0; i < schedule.size(); ++i) {
+    const std::string signature = ContractionSignature(i);
+    if (!signature.empty()) out.push_back({signature, schedule[i].contract});
+  }
+  return out;
+}
+
+// Times the tile configurations of every contraction signature the table does not hold yet, inside this plan's
+// own schedule: for each candidate the whole schedule is issued launch by launch with that candidate on all those
+// contractions, so each one is timed with the operands, the cache state and the weights it really meets (timed
+// alone in a loop, a projection's weights stay in the last-level cache; in the schedule every launch streams its
+// own from HBM).  Durations are the dispatches' own begin/end timestamps.
+void LaunchPlan::TuneContractions() {
+  if (table_ == nullptr || table_->GetMode() == kernel::ContractionTable::Mode::Off) return;
+  const std::vector<Launch> &schedule = GetSchedule();
+  std::map<std::string, std::vector<size_t>> unknown;
+  for (size_t i = 0; i < schedule.size(); ++i) {
+    const std::string signature = ContractionSignature(i);
+    if (!signature.empty() && !table_->Find(signature, nullptr)) unknown[signature].push_back(i);
+  }
+  if (!unknown.empty() && table_->GetMode() == kernel::ContractionTable::Mode::Measure) {
+    std::vector<size_t> probes;
+    for (const auto &kv : unknown) probes.insert(probes.end(), kv.second.begin(), kv.second.end());
+    std::sort(probes.begin(), probes.end());
+    std::vector<void *> events(2 * probes.size(), nullptr);
+    for (void *&e : events) Check(fluidml_hip_event_create(&e), "event");
+    kernel::LaunchContext ctx;
+    ctx.stream = stream_;
+    ctx.flags = flags_;
+    ctx.bf16 = bf16_;
+    constexpr int kRounds = 3;
+    // durations[launch] of one candidate: the best of kRounds passes after one that warms up; false: refused
+    auto time_candidate = [&](uint32_t bits, std::vector<double> *ns, std::vector<bool> *accepted) {
+      ns->assign(probes.size(), std::numeric_limits<double>::max());
+      accepted->assign(probes.size(), true);
+      for (int round = 0; round <= kRounds; ++round) {
+        size_t p = 0;
+        for (size_t i = 0; i < schedule.size(); ++i) {
+          if (p < probes.size() && probes[p] == i) {
+            Launch probe = schedule[i];
+            probe.contract = bits;
+            int rc = 0;
+            if ((*accepted)[p]) {
+              Check(fluidml_hip_time_kernels(events[2 * p], events[2 * p + 1]), "kernel timing on");
+              Issue(ctx, probe, &rc);
+              Check(fluidml_hip_time_kernels(nullptr, nullptr), "kernel timing off");
+              if (rc == FL_ERR_UNSUPPORTED) (*accepted)[p] = false;
+              else if (rc != 0) Check(rc, "timing a contraction launch");
+            }
+            if (!(*accepted)[p]) {
+              probe.contract = 0;  // keeps the tensors behind it defined
+              Issue(ctx, probe);
+            }
+            ++p;
+          } else {
+            Issue(ctx, schedule[i]);
+          }
+        }
+        Check(fluidml_hip_stream_synchronize(stream_), "tuning sync");
+        if (round == 0) continue;
+        for (size_t q = 0; q < probes.size(); ++q) {
+          if (!(*accepted)[q]) continue;
+          double t = 0;
+          Check(fluidml_hip_event_elapsed_ns(events[2 * q], events[2 * q + 1], &t), "event elapsed");
+          (*ns)[q] = std::min((*ns)[q], t);
+        }
+      }
+    };
+    try {
+      std::map<size_t, size_t> probe_of;
+      for (size_t q = 0; q < probes.size(); ++q) probe_of[probes[q]] = q;
+      // total over a signature's launches, or a negative number if any of them refused the candidate
+      auto total = [&](const std::vector<size_t> &launches, const std::vector<double> &ns, const std::vector<bool> &ok) {
+        double sum = 0;
+        for (size_t i : launches) {
+          const size_t q = probe_of.at(i);
+          if (!ok[q]) return -1.0;
+          sum += ns[q];
+        }
+        return sum / static_cast<double>(launches.size());
+      };
+      std::vector<double> ns;
+      std::vector<bool> ok;
+      time_candidate(0, &ns, &ok);
+      std::map<std::string, kernel::ContractPick> best;
+      for (const auto &kv : unknown) {
+        kernel::ContractPick rule;
+        rule.ns = rule.rule_ns = total(kv.second, ns, ok);
+        if (rule.ns < 0) throw std::runtime_error("tuning: the library's rule refused '" + kv.first + "'");
+        best[kv.first] = rule;
+      }
+      for (const auto &c : kernel::ContractionTable::Candidates(true)) {
+        kernel::ContractPick cand;
+        cand.tile = c.first;
+        cand.splits = c.second;
+        time_candidate(cand.Flags(), &ns, &ok);
+        for (const auto &kv : unknown) {
+          kernel::ContractPick &b = best[kv.first];
+          cand.ns = total(kv.second, ns, ok);
+          cand.rule_ns = b.rule_ns;
+          if (cand.ns < 0) continue;
+          const double bar = b.IsRule() ? b.rule_ns * (1.0 - kernel::kTuneMargin) : b.ns;
+          if (cand.ns < bar) b = cand;
+        }
+      }
+      for (const auto &kv : best) table_->Put(kv.first, kv.second);
+    } catch (...) {
+      fluidml_hip_time_kernels(nullptr, nullptr);
+      for (void *e : events) fluidml_hip_event_destroy(e);
+      throw;
+    }
+    for (void *e : events) fluidml_hip_event_destroy(e);
+  }
+  ApplyContractionPicks();
+}
+
+void LaunchPlan::Settle() {
+  Materialize();
+  DecideBranches();
 }
 
 void LaunchPlan::ReplayResident(size_t n) {

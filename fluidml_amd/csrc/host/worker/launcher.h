@@ -15,6 +15,7 @@
 
 #include "structure/flow/flow.h"
 #include "structure/kernel/kernel.h"
+#include "structure/kernel/tuner.h"
 
 namespace fluidml {
 namespace worker {
@@ -135,6 +136,10 @@ struct Launch {
   size_t owner = 0;  // member whose kernel owns constants / attributes the launch needs (LayerNorm, Gemm, Conv)
   size_t owner2 = 0;  // ConvPair: the second convolution
   double bytes = 0, flops = 0;
+  // MatMulChain / MatMulGroup / GemmChain, and a Step whose node is a MatMul or Gemm: the tile configuration the
+  // launch runs with (FL_CONTRACT_TILE / FL_CONTRACT_SPLITS bits; 0 = the library's rule), set from the plan's
+  // ContractionTable once the plan is on the device
+  uint32_t contract = 0;
 };
 const char *LaunchKindName(Launch::Kind kind);
 // Groups `steps` into launches.  With `fuse` false every step is its own launch.
@@ -188,6 +193,9 @@ class LaunchPlan {
   // prepares kernels. Idempotent. Throws std::runtime_error on HIP errors.
   void Materialize();
   bool IsMaterialized() const { return arena_ != nullptr; }
+  // Materialize(), then everything the first run would decide by timing (the side branches), so that the plan
+  // replays the same schedule from its first Invoke on and the decisions can be written down at Compile.
+  void Settle();
   // H2D inputs, `epoch` replays of all steps, D2H outputs; returns mean wall
   // nanoseconds per replay of the launch-and-wait loop alone (reference
   // runner.cpp:101-119). `args` maps every argument name to a host buffer of
@@ -229,6 +237,20 @@ class LaunchPlan {
   void SetBranchMinUs(double us) { branch_min_us_ = us; }
   // whether the first run times the schedule with and without its regions and keeps the faster one
   void SetBranchCheck(bool on) { branch_check_ = on; }
+  // 1 / 0: keep / drop the side branches without timing them (a decision read back from an earlier compile's JSON);
+  // negative: decide by timing
+  void SetBranchDecision(int keep) { branch_decision_ = keep; }
+  // 1 / 0 once the first run has decided (or a decision was given), -1 before, or when there was nothing to decide
+  int GetBranchDecision() const { return branches_decided_ && had_regions_ ? (branches_off_ ? 0 : 1) : -1; }
+
+  // The table the contraction launches take their tile configuration from; in its Measure mode, signatures it does
+  // not hold yet are timed inside this plan's schedule when the plan is materialised (reference: the generators'
+  // autotune, src/structure/kernel/generator/matmul.cpp:88-131).
+  void SetContractionTable(std::shared_ptr<kernel::ContractionTable> table) { table_ = std::move(table); }
+  // signature of schedule entry `i` in the ContractionTable; empty when the launch is no MatMul / Gemm
+  std::string ContractionSignature(size_t i) const;
+  // (signature, FL_CONTRACT_* bits in use) of every contraction launch of the schedule, in schedule order
+  std::vector<std::pair<std::string, uint32_t>> GetContractionChoices() const;
 
  private:
   struct ConstantSlot {
@@ -242,8 +264,11 @@ class LaunchPlan {
   };
   void *Resolve(const Operand &op) const;
   void IssueStep(kernel::LaunchContext &ctx, const Step &s, const Operand *in0_view = nullptr,
-                 const Operand *in1_view = nullptr, const Operand *out_view = nullptr) const;
-  void Issue(kernel::LaunchContext &ctx, const Launch &l) const;
+                 const Operand *in1_view = nullptr, const Operand *out_view = nullptr, int *rc_out = nullptr) const;
+  // `rc_out` given: a refusal of the C ABI is stored there instead of being thrown (tuning probes)
+  void Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out = nullptr) const;
+  void TuneContractions();
+  void ApplyContractionPicks() const;
   void LaunchAll(kernel::LaunchContext &ctx) const;
   void Replay(kernel::LaunchContext &ctx);
   void PlanBranches() const;
@@ -267,6 +292,9 @@ class LaunchPlan {
   bool branch_check_ = true;
   bool branches_decided_ = false;
   mutable bool branches_off_ = false;
+  int branch_decision_ = -1;
+  bool had_regions_ = false;
+  std::shared_ptr<kernel::ContractionTable> table_;
   void *side_stream_ = nullptr;
   std::vector<void *> region_events_;  // fork and join event of every region
   void *arena_ = nullptr;

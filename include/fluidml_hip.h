@@ -99,8 +99,39 @@ enum fl_contract_flags {
    * (at most 8 rows against k-contiguous weights: the weights are streamed in
    * fp32; depthwise and 3-d convolutions: the direct kernel). */
   FL_CONTRACT_BF16 = 1 << 0
+  /* bits 4..7: enum fl_contract_tile; bits 8..13: number of workgroups that share
+   * the K range of a tile (FL_CONTRACT_TILE / FL_CONTRACT_SPLITS below) */
 };
 #define FL_CONTRACT_SHIFT 16
+
+/* Tile configurations of the contraction kernel (MatMul, Gemm).  The reference's
+ * generators time the six loop orders of their kernel and keep the fastest
+ * (src/structure/kernel/generator/matmul.cpp:88-131, gemm.cpp:106-151); on this
+ * backend the choice that matters is the workgroup's tile and how many
+ * workgroups share the K range of a tile.  FL_TILE_RULE / 0 splits leave either
+ * to the library's own rule.  A configuration that does not exist for the operands of
+ * a call (the direct-to-LDS ones need both operands on their 128-bit load path and K a
+ * multiple of the chunk; a split needs that many K chunks and room in the
+ * stream's workspace) makes the call return FL_ERR_UNSUPPORTED with nothing
+ * launched, so a tuner can simply try them all.  Every configuration gives the
+ * same result from run to run; different configurations add the products in
+ * different orders. */
+enum fl_contract_tile {
+  FL_TILE_RULE = 0,
+  FL_TILE_32x32_STAGED = 1, /* 32x32 tile, four waves split K, tiles staged through registers by four more waves */
+  FL_TILE_64x64_STAGED = 2, /* 64x64 tile, 2x2 waves, four K chunks in flight in registers */
+  FL_TILE_32x32_K4 = 3,     /* the following load tiles from global memory straight into LDS: */
+  FL_TILE_64x32_K2 = 4,     /*   64x32 tile, two waves side by side times two K slices */
+  FL_TILE_64x64 = 5,        /*   64x64 tile, 2x2 waves */
+  FL_TILE_64x64_K2 = 6,     /*   64x64 tile, 2x2 waves times two K slices (eight waves) */
+  FL_TILE_128x64 = 7,       /*   128x64 tile, 4x2 waves */
+  FL_TILE_COUNT = 8
+};
+#define FL_CONTRACT_TILE_SHIFT 4
+#define FL_CONTRACT_SPLIT_SHIFT 8
+#define FL_CONTRACT_MAX_SPLITS 63
+#define FL_CONTRACT_TILE(tile) ((uint32_t)(tile) << FL_CONTRACT_TILE_SHIFT)
+#define FL_CONTRACT_SPLITS(n) ((uint32_t)(n) << FL_CONTRACT_SPLIT_SHIFT)
 
 /* A short chain of elementwise operations on one float32 value, used by the
  * launch-level fusions below.  Step i replaces v (initially the chain's input
@@ -143,7 +174,8 @@ typedef struct fl_tensor {
 /* Library / device plumbing (replaces the MLIR ExecutionEngine + the per-call
  * host arena of reference src/worker/runner.cpp:56-120).                     */
 
-/* Version of this ABI; bumped on any signature change (2: `flags` of the fused Gemm and Conv entry points). */
+/* Version of this ABI; bumped on any signature change (2: `flags` of the fused Gemm and Conv entry points;
+ * 3: tile configuration and K splits in the contraction flags). */
 int fluidml_hip_abi_version(void);
 /* Human-readable text for a return code of this library (static storage). */
 const char *fluidml_hip_error_string(int code);

@@ -123,7 +123,7 @@ def test_c_abi_exports_every_declared_symbol():
     from fluidml_amd import cabi
 
     assert set(cabi.SIGNATURES) | {"fluidml_hip_error_string"} == declared
-    assert cabi.lib.fluidml_hip_abi_version() == 2
+    assert cabi.lib.fluidml_hip_abi_version() == 3
     assert cabi.error_string(-3).startswith("shapes")
 
 

@@ -798,7 +798,10 @@ class Scheduler {
         if (!producer) continue;
         Launch *l = owner[*producer];
         if (l != nullptr) {
-          const bool plain_out = l->group.empty() && SameTensor(l->out, x) && !l->out.viewed && !l->has_out2;
+          // (a launch with a residual addend or a per-channel gate reads those through the strides of its own output
+          // tensor -- the kernels take no separate strides for them -- so it cannot write into a part of a wider one)
+          const bool plain_out = l->group.empty() && SameTensor(l->out, x) && !l->out.viewed && !l->has_out2 &&
+                                 !l->has_skip && !l->has_gate;
           const bool kind_ok = l->kind == Launch::Kind::MatMulChain || l->kind == Launch::Kind::GemmChain ||
                                l->kind == Launch::Kind::ConvChain || l->kind == Launch::Kind::ElementwiseChain ||
                                l->kind == Launch::Kind::DivAddSoftmax || l->kind == Launch::Kind::AddLayerNorm ||

@@ -406,3 +406,26 @@ def vgg16(batch: int = 1, image: int = 224, classes: int = 1000, width_div: int 
 
 def image_input(shape, seed: int = 97) -> Dict[str, np.ndarray]:
     return {"input": _rng(seed).standard_normal(shape, dtype=np.float32)}
+
+
+def residual_concat_nets():
+    """Two small graphs in which a contraction that carries a residual addend feeds one half of a Concat2:
+    MatMul(relu(x), W) + relu(x) beside tanh(relu(x)) on the last axis, and a pointwise Conv with a skip connection
+    beside a second Conv on the channel axis at batch 2.  The launch that adds the residual reads it through the
+    strides of its own output tensor, so it must not be redirected into a part of the wider Concat2 output."""
+    g = Net("matmul_residual_concat", 21)
+    x = g.input("x", np.float32, (1, 16, 32))
+    r = g.relu(x)
+    y = g.add(g.matmul(r, g.normal((32, 32), 0.2)), r)
+    g.output(g.concat2(y, g.unary("Tanh", r), 2))
+    rng = _rng(22)
+    first = (g, {"x": rng.standard_normal((1, 16, 32), dtype=np.float32)})
+
+    h = Net("conv_skip_concat", 23)
+    img = h.input("input", np.float32, (2, 8, 6, 6))
+    s = h.relu(img)
+    a = h.add(h.conv(s, h.he_normal((8, 8, 1, 1), fan_in=8), h.zeros((8,)), [1, 1], [0, 0, 0, 0]), s)
+    b = h.relu(h.conv(s, h.he_normal((4, 8, 3, 3), fan_in=72), h.normal((4,), 0.1), [1, 1], [1, 1, 1, 1]))
+    h.output(h.concat2(a, b, 1))
+    second = (h, {"input": rng.standard_normal((2, 8, 6, 6), dtype=np.float32)})
+    return [first, second]

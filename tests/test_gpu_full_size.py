@@ -8,10 +8,10 @@ batch 8) is compiled from its ONNX file and run three ways on the same seeded we
 * the one-launch-per-node schedule (FLUIDML_FUSE=0) of the same plan.
 
 Both GPU schedules have to meet the oracle within the tolerance the configurations are specified with
-(rel 1e-4 / abs 1e-5, fp32), element by element.  For an element outside it the float64 evaluation of the
-network (tests/torch_reference.py, pinned against the oracle on small instances by tests/test_oracle_graphs.py)
-decides whose rounding the difference is: the element passes if the GPU value is within the same tolerance of the
-float64 value, or no farther from it than the oracle's own worst element of that output.  The oracle adds the
+(rel 1e-4 / abs 1e-5, fp32), element by element.  Only for VGG-16 (LONGEST_SUM below) an element outside it is
+referred to the float64 evaluation of the network (tests/torch_reference.py, pinned against the oracle on small
+instances by tests/test_oracle_graphs.py): it passes if the GPU value is within the same tolerance of the float64
+value, or within rel 1e-4 / abs 3e-5 of it, and at most 1 % of an output may pass that way.  The oracle adds the
 products of each dot product one after the other in fp32 like the reference's loop nests, and over the 4,608 to
 25,088 terms of VGG-16's late layers that rounding alone exceeds the tolerance on a few logits whose terms cancel
 (the test prints the counts: about 10 of 1000 oracle logits are outside the tolerance of the float64 value, with
@@ -29,6 +29,11 @@ from oracle import graph_runner
 from tests.util import assert_close, assert_close_or_exact
 
 pytestmark = pytest.mark.gpu
+
+# Terms of the longest fp32 sum behind an element of the configuration's output.  Only VGG-16's logits (25,088 products
+# in its first Gemm, 4,096 in the next two) are long enough for sequential fp32 summation to miss the tolerance by
+# itself; every other configuration is held to the plain rule (no entry = no escape).
+LONGEST_SUM = {"vgg16_b1": 25088, "vgg16_b8": 25088}
 
 
 def _run(fluidml, net, feeds, path, name, flavour="plain_greedy"):
@@ -139,8 +144,8 @@ def test_full_size_matches_oracle(device, config, tmp_path, monkeypatch, progres
     for name, (rows, ref) in want.items():
         assert np.isfinite(ref).all()
         for what, got in (("per-node launches", plain), ("fused launches", fused)):
-            assert_close_or_exact(got[name][rows], ref, lambda: exact_rows(rows), what=f"{config} {what} vs oracle, {name}",
-                                  report=progress)
+            assert_close_or_exact(got[name][rows], ref, lambda: exact_rows(rows), LONGEST_SUM.get(config),
+                                  what=f"{config} {what} vs oracle, {name}", report=progress)
     for name, ref in plain.items():  # every row, also those the oracle did not compute
         assert np.isfinite(ref).all()
         assert_close(fused[name], ref, what=f"{config} fused vs per-node {name}")
@@ -165,3 +170,25 @@ def test_bert_base_dp_layouts_match_oracle(device, tmp_path, monkeypatch, progre
         assert sum(l != sorted(l) for l in layouts) > len(layouts) // 2, "the DP plan should hold non-identity layouts"
         for name, ref in want.items():
             assert_close(outs[name], ref, what=f"bert_base (4 layers) dp_greedy fuse={fuse} {name}")
+
+
+def test_vgg16_dp_layouts_match_oracle(device, tmp_path, monkeypatch, progress):
+    """A convolutional network under the DP executor at full size (VGG-16, batch 1): with constant costs every
+    internal tensor and every weight is stored with its dimensions reversed, so the convolutions, pools and Gemm
+    layers run on non-default strides at their real extents (the direct and implicit-GEMM convolution paths that the
+    default layouts never reach at these sizes)."""
+    from fluidml_amd import fluidml, models
+
+    net = models.vgg16(batch=1)
+    feeds = {"input": _vgg_images()[:1].copy()}
+    path = net.save(str(tmp_path / "vgg16.onnx"))
+    progress("[case] vgg16_b1, dp_greedy with constant costs: oracle (cached if the full-size case ran)")
+    ref = _vgg_oracle(0)
+    monkeypatch.setenv("FLUIDML_DP_COST", "constant")
+    progress("[case] vgg16_b1, dp_greedy with constant costs: compile + invoke")
+    outs, plan = _run(fluidml, net, feeds, path, "vgg16_dp", flavour="dp_greedy")
+    layouts = [list(s["output_layout"]) for s in plan["steps"]]
+    assert sum(l != sorted(l) for l in layouts) > len(layouts) // 2, "the DP plan should hold non-identity layouts"
+    (name,) = [v.name for v in net.outputs]
+    assert_close_or_exact(outs[name][[0]], ref, lambda: _exact("vgg16_b1", net, feeds, [0]), LONGEST_SUM["vgg16_b1"],
+                          what=f"vgg16_b1 dp_greedy (constant costs) {name}", report=progress)

@@ -156,3 +156,25 @@ def test_conv_nets_other_extents_match_oracle(device, family, dims, flavour, tmp
         assert ex.invoke(args) > 0
         for name, ref in want.items():
             assert_close(outs[name], ref, what=f"{family} {dims} {flavour} {name}")
+
+
+@pytest.mark.parametrize("which", [0, 1], ids=["matmul_residual", "conv_skip"])
+def test_residual_launch_beside_a_concat_matches_oracle(device, which, tmp_path):
+    """MatMul + residual and Conv + skip connection whose result is one input of a Concat2 (last axis, and channel
+    axis at batch 2): the launch keeps its own output tensor and the graph runs and matches the oracle."""
+    from fluidml_amd import fluidml, models
+
+    net, feeds = models.residual_concat_nets()[which]
+    want = graph_runner.run_graph(net, feeds)
+    path = net.save(str(tmp_path / (net.name + ".onnx")))
+    for fuse in (True, False):
+        ex = fluidml.Executor.make_plain_greedy(net.name)
+        ex.context().set_fuse(fuse)
+        print("[case]", net.name, "fuse", fuse, flush=True)
+        ex.compile(path)
+        args = {k: np.ascontiguousarray(v) for k, v in feeds.items()}
+        outs = {v.name: np.full(v.shape, np.nan, dtype=v.dtype) for v in net.outputs}
+        args.update(outs)
+        assert ex.invoke(args) > 0
+        for name, ref in want.items():
+            assert_close(outs[name], ref, what=f"{net.name} fuse={fuse} {name}")

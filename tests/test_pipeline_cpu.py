@@ -804,3 +804,21 @@ def test_compiler_cli(mods, tmp_path, capsys, monkeypatch):
         compiler.main(["-n", "x", "-i", path, "-m", "fastest"])
     with pytest.raises(SystemExit):
         compiler.main(["-i", path])  # --name is required, as in the reference
+
+
+def test_launch_with_a_residual_is_not_placed_into_a_concat(mods, tmp_path):
+    """A MatMul or Conv launch that adds a residual (or scales by a gate) keeps its own output tensor when that tensor
+    is an input of a Concat2: the kernels read the addend through the output's strides, and a part of the wider
+    Concat2 output has other strides (such a launch used to be redirected and was then refused at its first Invoke)."""
+    fluidml, models, _ = mods
+    for net, _ in models.residual_concat_nets():
+        path = net.save(str(tmp_path / (net.name + ".onnx")))
+        ex = fluidml.Executor.make_plain_greedy("rc")
+        ex.compile(path)
+        launches = ex.plan()["launches"]
+        carriers = [l for l in launches if l["kind"] in ("MatMulChain", "ConvChain") and len(l["reads"]) >= 3]
+        assert carriers, [l["kind"] for l in launches]
+        for l in carriers:
+            assert "writes_into" not in l, l
+        # the Concat2 still runs (at most its other input was written in place)
+        assert any(l["kind"] in ("Step", "CopyInto") and len(l["members"]) == 1 for l in launches)

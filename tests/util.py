@@ -85,17 +85,25 @@ def assert_close(got, want, exact=False, what=""):
         )
 
 
-def assert_close_or_exact(got, ref, exact_fn, what="", report=None):
-    """`got` has to be within rel RTOL / abs ATOL of the oracle's result `ref`, element by element.  Where it
-    is not, the float64 evaluation of the same network (`exact_fn()`) decides whose rounding the difference is:
-    the element passes if `got` is within the same tolerance of the float64 value, or at least no farther from
-    it than the oracle's own worst element on this output is.  The oracle adds the products of a dot product
-    one after the other in fp32 like the reference's loop nests, and over the 4,608 to 25,088 terms of the late
-    VGG-16 layers that alone moves logits whose terms cancel by more than the tolerance; a result that is closer
-    to the exact value than the reference's own arithmetic gets is not in error."""
+# the shortest fp32 sum for which assert_close_or_exact consults the float64 evaluation at all
+LONG_SUM = 4096
+
+
+def assert_close_or_exact(got, ref, exact_fn, reduction_length, what="", report=None):
+    """`got` has to be within rel RTOL / abs ATOL of the oracle's result `ref`, element by element.  Only for an
+    output whose elements are fp32 sums of at least LONG_SUM products (`reduction_length`: VGG-16's 25,088- and
+    4,096-term layers; everything else is held to the plain rule), the few elements outside are referred to the
+    float64 evaluation of the same network (`exact_fn()`): the oracle adds the products one after the other in fp32
+    like the reference's loop nests, which alone moves logits whose terms cancel by more than the tolerance.  Such
+    an element passes if `got` is within rel RTOL / abs ATOL of the float64 value, or within rel RTOL / abs 3 ATOL of
+    it -- an explicit cap, whatever the oracle's own distance is -- and at most 1 % of the output may pass that way.
+    The three counts are reported."""
     got = np.asarray(got)
     ref = np.asarray(ref)
     assert got.shape == ref.shape, f"{what}: shape {got.shape} vs {ref.shape}"
+    if reduction_length is None or reduction_length < LONG_SUM:
+        assert_close(got, ref, what=what)
+        return
     err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
     bad = err > ATOL + RTOL * np.abs(ref.astype(np.float64))
     if not bad.any():
@@ -103,15 +111,21 @@ def assert_close_or_exact(got, ref, exact_fn, what="", report=None):
     exact = np.asarray(exact_fn(), np.float64)
     assert exact.shape == got.shape
     bound = ATOL + RTOL * np.abs(exact)
+    cap = 3 * ATOL + RTOL * np.abs(exact)
     err_got = np.abs(got.astype(np.float64) - exact)
     err_ref = np.abs(ref.astype(np.float64) - exact)
+    by_exact = bad & (err_got <= bound)
+    by_cap = bad & ~by_exact & (err_got <= cap)
+    still = bad & ~by_exact & ~by_cap
     if report is not None:
         report(f"[tolerance] {what}: {np.count_nonzero(bad)} of {bad.size} elements differ from the oracle by more than rel {RTOL} / "
-               f"abs {ATOL} (max {err.max():.3e}); distance to the float64 evaluation: oracle max {err_ref.max():.3e} "
-               f"({np.count_nonzero(err_ref > bound)} outside), this result max {err_got.max():.3e} ({np.count_nonzero(err_got > bound)} outside)")
-    still = bad & (err_got > np.maximum(bound, err_ref.max()))
+               f"abs {ATOL} (max {err.max():.3e}); of these {np.count_nonzero(by_exact)} are within that tolerance of the float64 "
+               f"evaluation, {np.count_nonzero(by_cap)} within rel {RTOL} / abs {3 * ATOL:g} of it, {np.count_nonzero(still)} neither "
+               f"(oracle to float64: max {err_ref.max():.3e}, {np.count_nonzero(err_ref > bound)} outside; this result: max {err_got.max():.3e})")
     assert not still.any(), (
-        f"{what}: {np.count_nonzero(still)} of {bad.size} elements are outside rel {RTOL}/abs {ATOL} of the oracle and farther from the "
-        f"float64 evaluation than the oracle ever is; max distance to the oracle {err.max():.3e}, to float64 {err_got.max():.3e} "
-        f"(oracle to float64 {err_ref.max():.3e})"
+        f"{what}: {np.count_nonzero(still)} of {bad.size} elements are outside rel {RTOL}/abs {ATOL} of the oracle and outside rel {RTOL}/"
+        f"abs {3 * ATOL:g} of the float64 evaluation; max distance to the oracle {err.max():.3e}, to float64 {err_got.max():.3e}"
+    )
+    assert np.count_nonzero(bad) <= 0.01 * bad.size, (
+        f"{what}: {np.count_nonzero(bad)} of {bad.size} elements pass only through the float64 evaluation (more than 1 %)"
     )

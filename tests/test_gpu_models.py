@@ -178,3 +178,43 @@ def test_residual_launch_beside_a_concat_matches_oracle(device, which, tmp_path)
         assert ex.invoke(args) > 0
         for name, ref in want.items():
             assert_close(outs[name], ref, what=f"{net.name} fuse={fuse} {name}")
+
+
+def test_side_branch_decision_is_written_and_replayed(device, tmp_path):
+    """Whether the side branches of a schedule stay is decided by timing at Compile, written into the executor's
+    JSON ("side_branches": {"kept": ...}) and repeated, without timing, by a compile that is given that file --
+    also when the file says the opposite of what this machine would measure."""
+    import json
+
+    from fluidml_amd import fluidml
+
+    make_net, make_feeds = _cases()["gpt_neox"]
+    net, feeds = make_net(), make_feeds()
+    want = graph_runner.run_graph(net, feeds)
+    path = net.save(str(tmp_path / "neox.onnx"))
+
+    def compile_with(saved, name):
+        ex = fluidml.Executor.make_plain_greedy(name)
+        ex.context().set_branch_min_us(0.0)  # regions exist even on this small graph
+        if saved is not None:
+            ex.context().set_tune(saved)
+        out = str(tmp_path / (name + ".json"))
+        print("[case] compile", name, "saved decisions:", saved, flush=True)
+        ex.compile(path, json=out)
+        args = {k: np.ascontiguousarray(v) for k, v in feeds.items()}
+        outs = {v.name: np.full(v.shape, np.nan, dtype=v.dtype) for v in net.outputs}
+        args.update(outs)
+        assert ex.invoke(args) > 0
+        for k, ref in want.items():
+            assert_close(outs[k], ref, what=f"{name} {k}")
+        return ex, json.load(open(out))
+
+    first, doc = compile_with(None, "timed")
+    assert first.branch_decision() in (0, 1)
+    assert doc["side_branches"]["kept"] == bool(first.branch_decision())
+    for kept in (True, False):
+        saved = str(tmp_path / f"kept_{kept}.json")
+        json.dump({"side_branches": {"kept": kept}, "contraction_table": doc.get("contraction_table", {})}, open(saved, "w"))
+        ex, again = compile_with(saved, f"replayed_{kept}")
+        assert ex.branch_decision() == int(kept) and again["side_branches"]["kept"] == kept
+        assert (len(ex.plan()["regions"]) > 0) == kept

@@ -159,6 +159,7 @@ SIGNATURES = {
     "fluidml_hip_matmul_chain_add": [_T, _T, _T, _T, _vp, _T, _T, _u32, _vp],
     "fluidml_hip_matmul_chain_view": [_T, _T, _T, _T, _i64, _i64, _vp, _u32, _vp],
     "fluidml_hip_matmul_chain_group": [_i32, _T, _vp, _vp, _vp, _i64, _i64p, _vp, _u32, _vp],
+    "fluidml_hip_matmul_chain_group_norm": [_i32, _T, _vp, _vp, _vp, _vp, _i64, _i64p, _vp, _T, _vp, _u32, _vp],
     "fluidml_hip_gemm_chain": [_T, _T, _T, _T, _f64, _f64, _i32, _i32, _vp, _u32, _vp],
     "fluidml_hip_conv_chain": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _u32, _vp],
     "fluidml_hip_conv_chain_scale_add": [_T, _T, _T, _T, _i64p, _i64p, _i64p, _i64, _vp, _T, _T, _u32, _vp],
@@ -188,6 +189,16 @@ lib.fluidml_hip_error_string.restype = ctypes.c_char_p
 class FlEwProgram(ctypes.Structure):
     """fl_ew_program of include/fluidml_hip.h"""
     _fields_ = [("n", ctypes.c_int32), ("op", ctypes.c_int32 * 8), ("c", ctypes.c_float * 8)]
+
+
+class FlNormFusion(ctypes.Structure):
+    """fl_norm_fusion of include/fluidml_hip.h"""
+    _fields_ = [("deferred", ctypes.c_int32), ("width", ctypes.c_int32), ("epsilon", ctypes.c_double),
+                ("stats", ctypes.c_void_p), ("scale", ctypes.POINTER(FlTensor)), ("shift", ctypes.POINTER(FlTensor)),
+                ("stats_out", ctypes.c_void_p)]
+
+
+FL_NORM_NONE, FL_NORM_LHS, FL_NORM_ADDEND = 0, 1, 2
 
 
 def make_chain(steps) -> FlEwProgram:

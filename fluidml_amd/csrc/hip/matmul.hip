@@ -105,6 +105,18 @@ struct MatmulArgs {
   // a separate Mul kernel's
   const float *k_scale;
   int32_t sKs;
+  // EXTRA == 1 instantiations only, one batch element: a LayerNormalization kept out of memory (fl_norm_fusion).
+  // ln_mode 1: A holds the un-normalised tensor, the epilogue turns acc into rstd * (acc - mean * c1[n]) + bias[n];
+  // ln_mode 2: the addend does, and enters as (t - mean) * rstd * scale[n] + shift[n].  Row statistics come as
+  // ln_parts (mean, M2) pairs per row, each over 32 consecutive columns of the ln_width wide tensor.
+  int32_t ln_mode, ln_parts, ln_width;
+  float ln_eps;
+  const float *ln_stats;
+  const float *ln_c1;                 // mode 1, member 0 (members g > 0: g_ln_c1[g - 1])
+  const float *ln_scale, *ln_shift;   // mode 2
+  int32_t ln_s_scale, ln_s_shift, ln_s_c1;  // element strides of the three vectors
+  float *ln_stats_out;                // non-null: (mean, M2) of every 32-column run of C's rows, ceil(N / 32) per row
+  const float *g_ln_c1[3];
   const float *gB[3];
   float *gC[3];
   const float *gbias[3];
@@ -351,6 +363,43 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
       const int64_t at = boff[0] + static_cast<int64_t>(m) * sCm + static_cast<int64_t>(n) * sCn;
       pre_add[e] = p.addend != nullptr && inside ? p.addend[at] : 0.0f;
       pre_add2[e] = p.addend2 != nullptr && inside ? p.addend2[at] : 0.0f;
+    }
+  }
+
+  // Deferred LayerNormalization: the partial statistics of this workgroup's rows are requested now (NT / BM lanes
+  // per row, each a few of the row's partials) and merged after the K loop, when they have long arrived.
+  constexpr bool NORM = EXTRA == 1;
+  constexpr int kNormLanes = NORM ? (NT / BM > 32 ? 32 : NT / BM) : 1;  // lanes per row, a power of two
+  static_assert((kNormLanes & (kNormLanes - 1)) == 0, "the merge across a row's lanes is a butterfly");
+  __shared__ float ln_rows[NORM ? 2 * BM : 1];  // mean, then 1 / sqrt(var + eps), per row of the tile
+  constexpr int kNormPer = 8;  // partials per lane: rows of up to 32 * kNormPer * kNormLanes elements
+  float ln_part_mean[NORM ? kNormPer : 1], ln_part_m2[NORM ? kNormPer : 1];
+  if constexpr (NORM) {
+    if (p.ln_mode != 0 && !producer && ltid < BM * kNormLanes) {
+      const int row = ltid / kNormLanes, sub = ltid % kNormLanes;
+      const int m = min(m0 + row, p.M - 1);
+#pragma unroll
+      for (int u = 0; u < kNormPer; ++u) {
+        const int q = sub + u * kNormLanes;
+        const float *e = p.ln_stats + (static_cast<int64_t>(m) * p.ln_parts + min(q, p.ln_parts - 1)) * 2;
+        ln_part_mean[u] = e[0];
+        ln_part_m2[u] = e[1];
+      }
+    }
+  }
+  float ln_col[TN], ln_col2[TN];  // mode 1: c1 of the lane's columns; mode 2: scale and shift
+  if constexpr (NORM) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + (wn * TN + j) * 32 + lrow;
+      ln_col[j] = ln_col2[j] = 0.0f;
+      if (p.ln_mode == 1 && n < p.N) {
+        const float *c1 = blockIdx.y > 0 && p.n_groups > 1 ? p.g_ln_c1[blockIdx.y - 1] : p.ln_c1;
+        ln_col[j] = c1[n * p.ln_s_c1];
+      } else if (p.ln_mode == 2 && n < p.N) {
+        ln_col[j] = p.ln_scale[n * p.ln_s_scale];
+        ln_col2[j] = p.ln_shift[n * p.ln_s_shift];
+      }
     }
   }
 
@@ -654,6 +703,38 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
       }
     }
   }
+  if constexpr (NORM) {
+    // merge the row's partial statistics (Chan's update: counts, means and sums of squared deviations combine
+    // exactly, no difference of large squares) and leave mean and 1 / sqrt(var + eps) where the epilogue finds them
+    if (p.ln_mode != 0 && !producer && ltid < BM * kNormLanes) {
+      const int row = ltid / kNormLanes, sub = ltid % kNormLanes;
+      float cnt = 0.0f, mean = 0.0f, m2 = 0.0f;
+      auto merge = [&](float oc, float om, float oq) {
+        const float n = cnt + oc;
+        if (oc > 0.0f) {  // (an absent partial carries the values of a clamped load)
+          const float d = om - mean;
+          mean += d * (oc / n);
+          m2 += oq + d * d * (cnt * oc / n);
+          cnt = n;
+        }
+      };
+#pragma unroll
+      for (int u = 0; u < kNormPer; ++u) {
+        const int q = sub + u * kNormLanes;
+        const float c = q < p.ln_parts ? static_cast<float>(min(32, p.ln_width - 32 * q)) : 0.0f;
+        merge(c, ln_part_mean[u], ln_part_m2[u]);
+      }
+#pragma unroll
+      for (int off = 1; off < kNormLanes; off <<= 1) {
+        const float oc = __shfl_xor(cnt, off), om = __shfl_xor(mean, off), oq = __shfl_xor(m2, off);
+        merge(oc, om, oq);
+      }
+      if (sub == 0) {
+        ln_rows[row] = mean;
+        ln_rows[BM + row] = 1.0f / sqrtf(m2 / static_cast<float>(p.ln_width) + p.ln_eps);
+      }
+    }
+  }
   __syncthreads();  // staging area is reused below
 
   // ---- combine the K slices of a workgroup through LDS ------------------------
@@ -790,6 +871,13 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
       for (int e = 0; e < EV; ++e) {
         const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
         float v = acc[i][j][e];
+        if constexpr (NORM) {
+          if (p.ln_mode == 1) {
+            // A was the un-normalised tensor: LayerNorm(t) . B = rstd * (t . (scale B) - mean * colsum(scale B)) + shift . B
+            const int r = (wm * TM + i) * 32 + tile_row(e);
+            v = ln_rows[BM + r] * (v - ln_rows[r] * ln_col[j]);
+          }
+        }
         if (bias_by_col) {
           v = p.ca * v + p.cb * bias_col[j];
         } else if (bias != nullptr && m < p.M && n < p.N) {
@@ -815,6 +903,16 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
               add2[e] = Eb2 != nullptr && inside ? Eb2[static_cast<int64_t>(m) * sCm + col] : 0.0f;
             }
           }
+          if constexpr (NORM) {
+            if (p.ln_mode == 2) {
+              // the addend is the un-normalised tensor of a LayerNormalization: normalise it on the way in
+#pragma unroll
+              for (int e = 0; e < EV; ++e) {
+                const int r = (wm * TM + i) * 32 + tile_row(e);
+                add[e] = (add[e] - ln_rows[r]) * ln_rows[BM + r] * ln_col[j] + ln_col2[j];
+              }
+            }
+          }
 #pragma unroll
           for (int e = 0; e < EV; ++e) vals[e] += add[e];
           if (Eb2 != nullptr) {
@@ -827,6 +925,32 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
       for (int e = 0; e < EV; ++e) {
         const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
         if (m < p.M && n < p.N) Cb[static_cast<int64_t>(m) * sCm + col] = vals[e];
+      }
+      if constexpr (NORM) {
+        if (p.ln_stats_out != nullptr) {
+          // statistics of this 32-column run of every row the lane's half-wave holds: mean, then the sum of squared
+          // deviations from it (two butterflies over the 32 lanes of the half; columns past N count as absent)
+          const int first = n0 + (wn * TN + j) * 32;
+          const float cols = static_cast<float>(min(32, p.N - first));
+          const int parts = (p.N + 31) / 32;
+#pragma unroll
+          for (int e = 0; e < EV; ++e) {
+            float sum = n < p.N ? vals[e] : 0.0f;
+#pragma unroll
+            for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+            const float mean = sum / cols;
+            const float d = n < p.N ? vals[e] - mean : 0.0f;
+            float sq = d * d;
+#pragma unroll
+            for (int off = 16; off > 0; off >>= 1) sq += __shfl_xor(sq, off);
+            const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
+            if (lrow == 0 && m < p.M && first < p.N) {
+              float *at = p.ln_stats_out + (static_cast<int64_t>(m) * parts + first / 32) * 2;
+              at[0] = mean;
+              at[1] = sq;
+            }
+          }
+        }
       }
   });
 }
@@ -1210,7 +1334,8 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
              float cb, const fl_tensor *bias, void *stream, const fl_ew_program *chain = nullptr, int64_t n_inner = 0,
              int64_t stride_outer = 0, const Siblings *siblings = nullptr, bool bf16 = false,
              const float *addend = nullptr, const float *k_scale = nullptr, int64_t k_scale_stride = 0,
-             const float *addend2 = nullptr, TileChoice choice = TileChoice()) {
+             const float *addend2 = nullptr, TileChoice choice = TileChoice(), const fl_norm_fusion *norm = nullptr,
+             const fl_tensor *const *col_sum = nullptr) {
   FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(lhs));
   FL_CHECK(CheckView(rhs));
@@ -1346,11 +1471,57 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
   // k-contiguous weights over an operand whose rows lose the alignment (49 pixels): wide loads for the weights alone
   const bool vec_a_only = vec_a && !vec_b && la == 0 && lb == 0 && !bf16;
   // a second addend with the strides of C / a scale per row of B: the tiled kernel's own instantiations (fp32)
-  const bool extra = addend != nullptr || k_scale != nullptr;
+  const bool extra = addend != nullptr || k_scale != nullptr || norm != nullptr;
   if (extra) {
-    if (lb != 0 || p.n_groups > 1 || p.n_inner != 0 || (addend2 != nullptr && addend == nullptr)) return FL_ERR_UNSUPPORTED;
+    // (grouped members and split output columns have their own strides of C: the addends are read through the
+    // plain ones)
+    if (lb != 0 || (addend2 != nullptr && addend == nullptr)) return FL_ERR_UNSUPPORTED;
+    if (addend != nullptr && (p.n_groups > 1 || p.n_inner != 0)) return FL_ERR_UNSUPPORTED;
     p.addend = addend;
     p.addend2 = addend2;
+  }
+  if (norm != nullptr) {
+    // a LayerNormalization folded into this launch: one batch element, fp32, rows short enough for the lanes that
+    // merge a row's partial statistics (64x64 tile: 4 lanes x 8 partials x 32 columns)
+    const int64_t real_batch = siblings != nullptr && siblings->count > 0 ? 1 : n_batch;
+    if (real_batch != 1 || bf16 || k_scale != nullptr || addend2 != nullptr) return FL_ERR_UNSUPPORTED;
+    if (norm->deferred != FL_NORM_NONE) {
+      if (norm->stats == nullptr || norm->width <= 0 || norm->width > 1024) return FL_ERR_UNSUPPORTED;
+      p.ln_mode = norm->deferred;
+      p.ln_width = norm->width;
+      p.ln_parts = (norm->width + 31) / 32;
+      p.ln_eps = static_cast<float>(norm->epsilon);
+      p.ln_stats = norm->stats;
+    }
+    auto vector_of = [&](const fl_tensor *t, int64_t extent, const float **base, int32_t *stride) -> int {
+      if (t == nullptr) return FL_ERR_NULL;
+      FL_CHECK(CheckView(t));
+      if (t->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+      if (t->rank != 1 || t->shape[0] != extent) return FL_ERR_SHAPE;
+      *base = static_cast<const float *>(t->base);
+      *stride = static_cast<int32_t>(t->strides[0]);
+      return FL_OK;
+    };
+    if (norm->deferred == FL_NORM_LHS) {
+      // the row statistics belong to A's rows: the normalised axis is K; c1 per member, the bias carries shift . B
+      if (norm->width != p.K || col_sum == nullptr || bias == nullptr || p.sDm != 0 || addend != nullptr) return FL_ERR_UNSUPPORTED;
+      if (p.ca != 1.0f || p.cb != 1.0f) return FL_ERR_UNSUPPORTED;
+      FL_CHECK(vector_of(col_sum[0], p.N, &p.ln_c1, &p.ln_s_c1));
+      for (int g = 1; g < p.n_groups; ++g) {
+        int32_t stride = 0;
+        FL_CHECK(vector_of(col_sum[g], p.N, &p.g_ln_c1[g - 1], &stride));
+        if (stride != p.ln_s_c1) return FL_ERR_SHAPE;
+      }
+    } else if (norm->deferred == FL_NORM_ADDEND) {
+      // the addend has C's shape: the normalised axis is N
+      if (norm->width != p.N || addend == nullptr) return FL_ERR_UNSUPPORTED;
+      FL_CHECK(vector_of(norm->scale, p.N, &p.ln_scale, &p.ln_s_scale));
+      FL_CHECK(vector_of(norm->shift, p.N, &p.ln_shift, &p.ln_s_shift));
+    } else if (norm->deferred != FL_NORM_NONE) {
+      return FL_ERR_ATTR;
+    }
+    if (norm->stats_out != nullptr && (p.n_groups > 1 || p.n_inner != 0)) return FL_ERR_UNSUPPORTED;
+    p.ln_stats_out = norm->stats_out;
   }
   if (k_scale != nullptr) {
     if (n_batch != 1 || k_scale_stride > INT32_MAX || k_scale_stride < 0) return FL_ERR_UNSUPPORTED;
@@ -1657,6 +1828,42 @@ int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl
   return fl::Contract(lhs, rhs[0], out[0], false, false, 1.0f, 1.0f, bias != nullptr ? bias[0] : nullptr, stream, chain,
                       n_inner, stride_outer != nullptr ? stride_outer[0] : 0, &sib, (flags & FL_CONTRACT_BF16) != 0, nullptr,
                       nullptr, 0, nullptr, fl::ChoiceOf(flags));
+}
+
+int fluidml_hip_matmul_chain_group_norm(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs,
+                                        const fl_tensor *const *bias, const fl_tensor *const *col_sum,
+                                        const fl_tensor *const *out, int64_t n_inner, const int64_t *stride_outer,
+                                        const fl_ew_program *chain, const fl_tensor *addend, const fl_norm_fusion *norm,
+                                        uint32_t flags, void *stream) {
+  if (!lhs || !rhs || !out || !norm) return FL_ERR_NULL;
+  if (count < 1 || count > 4) return FL_ERR_ATTR;
+  fl::Siblings sib;
+  sib.count = count - 1;
+  for (int g = 0; g < count; ++g) {
+    if (!rhs[g] || !out[g]) return FL_ERR_NULL;
+    if (bias != nullptr && bias[g] != nullptr && bias[g]->rank != 1) return FL_ERR_RANK;
+    if (g > 0) {
+      sib.rhs[g - 1] = rhs[g];
+      sib.out[g - 1] = out[g];
+      sib.bias[g - 1] = bias != nullptr ? bias[g] : nullptr;
+      sib.stride_outer[g - 1] = stride_outer != nullptr ? stride_outer[g] : 0;
+    }
+  }
+  const float *extra = nullptr;
+  if (addend != nullptr) {
+    if (count != 1 || n_inner != 0) return FL_ERR_UNSUPPORTED;
+    FL_CHECK(fl::CheckView(addend));
+    if (addend->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+    if (addend->rank != out[0]->rank) return FL_ERR_SHAPE;
+    for (int d = 0; d < out[0]->rank; ++d) {
+      if (addend->shape[d] != out[0]->shape[d]) return FL_ERR_SHAPE;
+      if (out[0]->shape[d] > 1 && addend->strides[d] != out[0]->strides[d]) return FL_ERR_UNSUPPORTED;
+    }
+    extra = static_cast<const float *>(addend->base);
+  }
+  return fl::Contract(lhs, rhs[0], out[0], false, false, 1.0f, 1.0f, bias != nullptr ? bias[0] : nullptr, stream, chain,
+                      n_inner, stride_outer != nullptr ? stride_outer[0] : 0, count > 1 ? &sib : nullptr, false, extra, nullptr,
+                      0, nullptr, fl::ChoiceOf(flags), norm, col_sum);
 }
 
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,

@@ -419,6 +419,35 @@ int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, co
  * projections of an attention block): rhs[i], bias[i] (all NULL or none),
  * out[i] and stride_outer[i] belong to member i.  No batch dims. */
 int fluidml_hip_matmul_chain_group(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs, const fl_tensor *const *bias, const fl_tensor *const *out, int64_t n_inner, const int64_t *stride_outer, const fl_ew_program *chain, uint32_t flags, void *stream);
+/* A LayerNormalization over the last axis that is kept out of memory between the contraction that produces its
+ * input and the contractions that consume its output (reference layer_normalization.cpp:33-220 between
+ * matmul.cpp:28-59 launches, e.g. the two post-attention / post-FFN normalisations of a transformer layer).  The
+ * tensor t that would be normalised is stored as it is, together with partial row statistics: for row r and every
+ * run j of 32 consecutive columns, stats[(r * parts + j) * 2 + 0] = mean and [.. + 1] = sum of squared deviations
+ * of that run (parts = ceil(width / 32); Chan's pairwise update combines them without cancellation).  A consumer
+ * then works on LayerNorm(t) = (t - mean_r) * rstd_r * scale + shift without it ever being written:
+ *   deferred == FL_NORM_LHS: `lhs` of the call is t.  Because the normalisation is affine per row, the product is
+ *     rstd_r * (t . (diag(scale) rhs) - mean_r * col_sum) + (shift . rhs + bias): the caller passes diag(scale) rhs
+ *     as `rhs`, col_sum[n] = sum_k scale[k] rhs[k][n] per member as `col_sum[i]`, and shift . rhs + bias as `bias[i]`.
+ *   deferred == FL_NORM_ADDEND: `addend` of the call is t; (t - mean_r) * rstd_r * scale[n] + shift[n] is added
+ *     after the chain, where a plain addend would be.
+ * `stats_out` (may be given with or without a deferred operand): the call leaves the partial statistics of its own
+ * output rows there, ceil(N / 32) pairs per row, for the next consumer.  Single batch element only. */
+enum fl_norm_deferred { FL_NORM_NONE = 0, FL_NORM_LHS = 1, FL_NORM_ADDEND = 2 };
+typedef struct fl_norm_fusion {
+  int32_t deferred;       /* enum fl_norm_deferred */
+  int32_t width;          /* extent of the normalised axis of t */
+  double epsilon;
+  const float *stats;     /* partial statistics of t's rows (device memory), NULL if deferred == FL_NORM_NONE */
+  const fl_tensor *scale; /* FL_NORM_ADDEND: rank-1 [N] */
+  const fl_tensor *shift; /* FL_NORM_ADDEND: rank-1 [N] */
+  float *stats_out;       /* NULL: none */
+} fl_norm_fusion;
+/* fluidml_hip_matmul_chain_group (count 1..4; count == 1 is a single chain) with such a normalisation folded in.
+ * `col_sum[i]`: rank-1 [N] per member, FL_NORM_LHS only (else NULL).  `addend`: a tensor with the strides of out[0]
+ * added after the chain (plain, or t of FL_NORM_ADDEND); count == 1 and n_inner == 0 only.  fp32 whatever `flags`
+ * say about bf16; the tile configuration bits of `flags` apply. */
+int fluidml_hip_matmul_chain_group_norm(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs, const fl_tensor *const *bias, const fl_tensor *const *col_sum, const fl_tensor *const *out, int64_t n_inner, const int64_t *stride_outer, const fl_ew_program *chain, const fl_tensor *addend, const fl_norm_fusion *norm, uint32_t flags, void *stream);
 /* GemmConstantWeightsBiasKernel -> elementwise chain (reference gemm.cpp:39-182); `flags` = fl_contract_flags. */
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double alpha, double beta, int32_t trans_a, int32_t trans_b, const fl_ew_program *chain, uint32_t flags, void *stream);
 /* Conv{With,Without}PaddingKernel -> elementwise chain (reference conv.cpp:27-280);

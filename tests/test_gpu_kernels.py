@@ -1272,6 +1272,126 @@ def test_fused_add_layer_norm(device):
             assert_close(do.logical(), ho.logical(), what="add_layer_normalization")
 
 
+@pytest.mark.parametrize("M,H,K0,N1", [(128, 256, 128, 384), (100, 200, 96, 72), (33, 768, 256, 768)], ids=str)
+def test_matmul_with_deferred_layer_norm(device, M, H, K0, N1):
+    """A LayerNormalization that never reaches memory (fluidml_hip_matmul_chain_group_norm) against the oracle's
+    MatMul -> Add -> Add -> LayerNormalization -> MatMul chain.  Three calls: (1) the contraction that produces the
+    residual sum s leaves the partial row statistics of s beside it; (2) a grouped pair of projections reads s as if
+    it were LayerNorm(s) (scale folded into the weights, per-row mean and rstd applied in the epilogue); (3) a
+    contraction adds LayerNorm(s) as its residual and leaves the statistics of its own result.  Widths with a
+    ragged last run of 32 columns, rows that do not fill the tiles, and every tile configuration the flags name."""
+    import torch
+
+    cabi = _cabi()
+    rng = np.random.default_rng(M + H)
+    eps = 1e-5
+    a0, w0, b0 = rand(rng, (1, M, K0), -1, 1), rand(rng, (K0, H), -0.3, 0.3), rand(rng, (H,), -0.5, 0.5)
+    x = rand(rng, (1, M, H), -2, 2) + 0.75  # rows with a mean well away from zero
+    gamma, beta = rand(rng, (H,), 0.5, 1.5), rand(rng, (H,), -0.5, 0.5)
+    w1 = [rand(rng, (H, N1), -0.2, 0.2) for _ in range(2)]
+    b1 = [rand(rng, (N1,), -0.5, 0.5) for _ in range(2)]
+    a2, w2, b2 = rand(rng, (1, M, K0), -1, 1), rand(rng, (K0, H), -0.3, 0.3), rand(rng, (H,), -0.5, 0.5)
+
+    # the oracle's unfused chain
+    def V(shape):
+        return ok.View.empty(shape)
+
+    t, t1, s_ref, h_ref = V((1, M, H)), V((1, M, H)), V((1, M, H)), V((1, M, H))
+    ok.matmul(ok.View(a0), ok.View(w0), t)
+    ok.binary_f32(ok.BOP_ADD, ok.View(b0), t, t1)
+    ok.binary_f32(ok.BOP_ADD, t1, ok.View(x), s_ref)
+    ok.layer_norm(s_ref, ok.View(gamma), ok.View(beta), h_ref, 2, eps)
+    z_ref = []
+    for w, b in zip(w1, b1):
+        z0, z = V((1, M, N1)), V((1, M, N1))
+        ok.matmul(h_ref, ok.View(w), z0)
+        ok.binary_f32(ok.BOP_ADD, ok.View(b), z0, z)
+        z_ref.append(z.logical())
+    u0, u1, u_ref = V((1, M, H)), V((1, M, H)), V((1, M, H))
+    ok.matmul(ok.View(a2), ok.View(w2), u0)
+    ok.binary_f32(ok.BOP_ADD, ok.View(b2), u0, u1)
+    ok.binary_f32(ok.BOP_ADD, u1, h_ref, u_ref)
+
+    parts = (H + 31) // 32
+    ptr = ctypes.POINTER(cabi.FlTensor)
+
+    def dev(arr):
+        return DeviceView(ok.View(np.ascontiguousarray(arr, dtype=np.float32)), device)
+
+    def one(v):
+        return (ptr * 1)(ctypes.pointer(v.tensor))
+
+    def partial_stats(rows):
+        want = np.zeros((rows.shape[0], parts, 2))
+        for j in range(parts):
+            run = rows[:, 32 * j:32 * j + 32].astype(np.float64)
+            want[:, j, 0] = run.mean(axis=1)
+            want[:, j, 1] = ((run - run.mean(axis=1, keepdims=True)) ** 2).sum(axis=1)
+        return want
+
+    da0, dw0, db0, dx = dev(a0), dev(w0), dev(b0), dev(x)
+    dgamma, dbeta = dev(gamma), dev(beta)
+    # what a caller folds at compile time: scale into the weights, their column sums, shift . W + bias
+    dw1 = [dev(gamma[:, None] * w) for w in w1]
+    dc1 = [dev((gamma[:, None].astype(np.float64) * w).sum(axis=0)) for w in w1]
+    dc2 = [dev(beta.astype(np.float64) @ w.astype(np.float64) + b) for w, b in zip(w1, b1)]
+    da2, dw2, db2 = dev(a2), dev(w2), dev(b2)
+    for tile in range(0, 8):
+        flags = ctypes.c_uint32(tile << 4)
+        ds = DeviceView(ok.View.empty((1, M, H), np.float32, None, fill=3), device)
+        stats = torch.full((M, parts, 2), 7.0, device=device)
+        norm = cabi.FlNormFusion()
+        norm.deferred, norm.stats_out = cabi.FL_NORM_NONE, stats.data_ptr()
+        announce("deferred layer norm: producer", (M, H, K0), "tile", tile)
+        rc = cabi.lib.fluidml_hip_matmul_chain_group_norm(1, da0.ref(), one(dw0), one(db0), None, one(ds), 0, None, None, dx.ref(),
+                                                          ctypes.byref(norm), flags, None)
+        if rc == -8:
+            assert tile >= 3  # the rule and the register-staged tiles take every operand
+            continue
+        assert rc == 0, cabi.error_string(rc)
+        s_got = ds.logical()
+        assert_close(s_got, s_ref.logical(), what=f"residual sum, tile {tile}")
+        got_stats = stats.cpu().numpy().astype(np.float64)
+        want_stats = partial_stats(s_got[0])
+        assert np.allclose(got_stats[..., 0], want_stats[..., 0], rtol=1e-5, atol=1e-6), "partial means"
+        assert np.allclose(got_stats[..., 1], want_stats[..., 1], rtol=1e-4, atol=1e-5), "partial sums of squared deviations"
+
+        douts = [DeviceView(ok.View.empty((1, M, N1), np.float32, None, fill=3), device) for _ in range(2)]
+        norm = cabi.FlNormFusion()
+        norm.deferred, norm.width, norm.epsilon, norm.stats = cabi.FL_NORM_LHS, H, eps, stats.data_ptr()
+        rhs = (ptr * 2)(*[ctypes.pointer(d.tensor) for d in dw1])
+        bias = (ptr * 2)(*[ctypes.pointer(d.tensor) for d in dc2])
+        csum = (ptr * 2)(*[ctypes.pointer(d.tensor) for d in dc1])
+        outs = (ptr * 2)(*[ctypes.pointer(d.tensor) for d in douts])
+        announce("deferred layer norm: normalised left operand, two projections", (M, H, N1), "tile", tile)
+        rc = cabi.lib.fluidml_hip_matmul_chain_group_norm(2, ds.ref(), rhs, bias, csum, outs, 0, None, None, None,
+                                                          ctypes.byref(norm), flags, None)
+        if rc == -8:
+            assert tile >= 3
+        else:
+            assert rc == 0, cabi.error_string(rc)
+            for d, want in zip(douts, z_ref):
+                assert_close(d.logical(), want, what=f"projection of the deferred LayerNorm, tile {tile}")
+
+        du = DeviceView(ok.View.empty((1, M, H), np.float32, None, fill=3), device)
+        stats2 = torch.full((M, parts, 2), 7.0, device=device)
+        norm = cabi.FlNormFusion()
+        norm.deferred, norm.width, norm.epsilon, norm.stats = cabi.FL_NORM_ADDEND, H, eps, stats.data_ptr()
+        norm.scale, norm.shift = ctypes.pointer(dgamma.tensor), ctypes.pointer(dbeta.tensor)
+        norm.stats_out = stats2.data_ptr()
+        announce("deferred layer norm: normalised residual", (M, K0, H), "tile", tile)
+        rc = cabi.lib.fluidml_hip_matmul_chain_group_norm(1, da2.ref(), one(dw2), one(db2), None, one(du), 0, None, None, ds.ref(),
+                                                          ctypes.byref(norm), flags, None)
+        if rc == -8:
+            assert tile >= 3
+            continue
+        assert rc == 0, cabi.error_string(rc)
+        assert_close(du.logical(), u_ref.logical(), what=f"contraction + deferred LayerNorm residual, tile {tile}")
+        want2 = partial_stats(du.logical()[0])
+        got2 = stats2.cpu().numpy().astype(np.float64)
+        assert np.allclose(got2[..., 0], want2[..., 0], rtol=1e-5, atol=1e-6) and np.allclose(got2[..., 1], want2[..., 1], rtol=1e-4, atol=1e-5)
+
+
 CONV_CASES = [
     # x shape, w shape, pads, strides, dilations, group, bias
     ((1, 768, 128), (768, 1, 9), [4, 4], [1], [1], 768, False),  # reference conv0.py (depthwise 1-d, pad 4)

@@ -469,6 +469,29 @@ inline NestArgs<NOPS> MakeNestArgs(const LoopNest &nest) {
 // ---- device-side reductions -------------------------------------------------
 
 #if defined(__HIPCC__)
+// The value of another lane through the data-parallel-primitive path of the vector ALU (a few cycles, against the
+// round trip through the LDS crossbar that a shuffle by lane index costs).  `CTRL`: 0xB1 / 0x4E swap neighbours /
+// pairs inside every four lanes, 0x141 / 0x140 mirror every 8 / 16 lanes.
+template <int CTRL>
+__device__ __forceinline__ float DppMove(float v) {
+  const int bits = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(bits, bits, CTRL, 0xf, 0xf, false));
+}
+
+// Sum over every aligned group of W consecutive lanes (W a power of two), delivered to all lanes of the group.
+// Every lane of the wave has to be active.
+template <int W>
+__device__ __forceinline__ float GroupSum(float v) {
+  static_assert(W >= 1 && W <= kWave && (W & (W - 1)) == 0, "groups are powers of two");
+  if constexpr (W >= 2) v += DppMove<0xB1>(v);
+  if constexpr (W >= 4) v += DppMove<0x4E>(v);
+  if constexpr (W >= 8) v += DppMove<0x141>(v);
+  if constexpr (W >= 16) v += DppMove<0x140>(v);
+  if constexpr (W >= 32) v += __shfl_xor(v, 16, kWave);
+  if constexpr (W >= 64) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
 template <typename T, typename F>
 __device__ __forceinline__ T WaveReduce(T v, F f) {
 #pragma unroll

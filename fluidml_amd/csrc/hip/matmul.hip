@@ -25,6 +25,7 @@
 // assignment is the one the fp32 path already uses (lane half h holds k = 4h..4h+3 of a group of 8), so one
 // bf16 instruction replaces four fp32 ones.
 #include <algorithm>
+#include <cstddef>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -70,7 +71,8 @@ struct BatchArgs {
 
 // Kernel arguments.  Every workgroup needs the first block before it can issue its first load, and a cold
 // 64-byte line of kernel arguments costs a few hundred nanoseconds: what every launch reads comes first and
-// is packed, what only some launches read (chain, siblings, convolution geometry) follows.
+// is packed (two lines), what the EXTRA instantiations read follows (the next line and a half), and what only some
+// launches read (batch dims, chain, siblings, convolution geometry) comes last.
 struct MatmulArgs {
   int32_t M, N, K;
   int32_t sAm, sAk, sBk, sBn, sCm, sCn;
@@ -91,10 +93,16 @@ struct MatmulArgs {
   float ca, cb;
   float *partials;
   uint32_t *counters;
-  BatchArgs batch;
-  FastDiv div_inner;
-  // optional elementwise chain applied after the bias (chain.n == 0: none)
-  fl_ew_program chain;
+  // copies of batch.rank and chain.n (set at launch), so that a launch without batch dims or chain never touches
+  // the lines those live in
+  int32_t batch_rank, chain_n;
+  // EXTRA == 1 instantiations only, one batch element: a LayerNormalization kept out of memory (fl_norm_fusion).
+  // ln_mode 1: A holds the un-normalised tensor, the epilogue turns acc into rstd * (acc - mean * c1[n]) + bias[n];
+  // ln_mode 2: the addend does, and enters as (t - mean) * rstd * scale[n] + shift[n].  Row statistics come as
+  // ln_parts (mean, M2) pairs per row, each over 32 consecutive columns of the ln_width wide tensor.
+  int32_t ln_mode, ln_parts, ln_width;
+  float ln_eps;
+  // ---- byte 128 ----
   // EXTRA instantiations only (plain contraction, B kept [k][n]), all optional:
   // a tensor with the strides of C, added to the value after the chain (read at the element offset the value is
   // stored at);
@@ -105,24 +113,26 @@ struct MatmulArgs {
   // a separate Mul kernel's
   const float *k_scale;
   int32_t sKs;
-  // EXTRA == 1 instantiations only, one batch element: a LayerNormalization kept out of memory (fl_norm_fusion).
-  // ln_mode 1: A holds the un-normalised tensor, the epilogue turns acc into rstd * (acc - mean * c1[n]) + bias[n];
-  // ln_mode 2: the addend does, and enters as (t - mean) * rstd * scale[n] + shift[n].  Row statistics come as
-  // ln_parts (mean, M2) pairs per row, each over 32 consecutive columns of the ln_width wide tensor.
-  int32_t ln_mode, ln_parts, ln_width;
-  float ln_eps;
+  float ln_inv_width;  // (1 / ln_width, rounded once on the host)
   const float *ln_stats;
   const float *ln_c1;                 // mode 1, member 0 (members g > 0: g_ln_c1[g - 1])
   const float *ln_scale, *ln_shift;   // mode 2
-  int32_t ln_s_scale, ln_s_shift, ln_s_c1;  // element strides of the three vectors
+  // ---- byte 192 ----
   float *ln_stats_out;                // non-null: (mean, M2) of every 32-column run of C's rows, ceil(N / 32) per row
+  int32_t ln_s_scale, ln_s_shift, ln_s_c1;  // element strides of the three vectors
+  FastDiv div_inner;
   const float *g_ln_c1[3];
   const float *gB[3];
   float *gC[3];
   const float *gbias[3];
   int32_t g_sCm[3], g_sCn[3], g_sCn_outer[3];
+  BatchArgs batch;
+  // optional elementwise chain applied after the bias (chain.n == 0: none)
+  fl_ew_program chain;
   ConvGeom conv;  // read by the CONV instantiations only
 };
+static_assert(offsetof(MatmulArgs, addend) == 128 && offsetof(MatmulArgs, ln_stats_out) == 192,
+              "the packing of the kernel arguments into lines is deliberate");
 
 inline int MakeBatchArgs(const LoopNest &nest, int64_t n_batch, BatchArgs *b) {
   std::memset(b, 0, sizeof(*b));
@@ -250,7 +260,9 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
                 "the direct-to-LDS loop exists for one MFMA tile per wave of plain fp32 contractions");
   constexpr int STAGE_ELEMS = DIRECT > 0 ? DIRECT * kRingStage : 2 * (A_ELEMS + B_ELEMS);
   constexpr int LDS_ELEMS = STAGE_ELEMS > RED_ELEMS ? STAGE_ELEMS : RED_ELEMS;
-  __shared__ __attribute__((aligned(16))) float lds[LDS_ELEMS];
+  // (one LDS object per kernel: the row statistics of a deferred LayerNormalization live behind the tiles)
+  constexpr int LN_ELEMS = EXTRA == 1 ? 2 * BM : 0;
+  __shared__ __attribute__((aligned(16))) float lds[LDS_ELEMS + LN_ELEMS];
 
   // VEC: floats per global load of both operands' tiles; 41 = four for A and one for B (rows of B that do not keep
   // 16-byte alignment, a 7x7 image's 49 pixels, under weights that do)
@@ -271,7 +283,12 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   asm volatile("" ::"s"(p.M), "s"(p.N), "s"(p.K), "s"(p.sAm), "s"(p.sAk), "s"(p.sBk), "s"(p.sBn), "s"(p.sCm), "s"(p.sCn),
                "s"(p.tiles_m), "s"(p.tiles_n), "s"(p.n_splits), "s"(p.chunks_per_split), "s"(p.n_groups), "s"(p.n_inner),
                "s"(p.sCn_outer), "s"(p.bias), "s"(p.sDm), "s"(p.sDn), "s"(p.ca), "s"(p.cb), "s"(p.partials),
-               "s"(p.counters), "s"(p.batch.rank), "s"(p.chain.n));
+               "s"(p.counters), "s"(p.batch_rank), "s"(p.chain_n));
+  if constexpr (EXTRA != 0) asm volatile("" ::"s"(p.addend), "s"(p.addend2), "s"(p.k_scale), "s"(p.sKs));
+  if constexpr (EXTRA == 1) {
+    asm volatile("" ::"s"(p.ln_mode), "s"(p.ln_parts), "s"(p.ln_width), "s"(p.ln_eps), "s"(p.ln_inv_width), "s"(p.ln_stats), "s"(p.ln_c1),
+                 "s"(p.ln_scale), "s"(p.ln_shift), "s"(p.ln_s_scale), "s"(p.ln_s_shift), "s"(p.ln_s_c1), "s"(p.ln_stats_out));
+  }
   if constexpr (CONV != 0) {
     asm volatile("" ::"s"(p.conv.H), "s"(p.conv.W), "s"(p.conv.sh), "s"(p.conv.sw), "s"(p.conv.dh), "s"(p.conv.dw),
                  "s"(p.conv.ph), "s"(p.conv.pw), "s"(p.conv.sXn), "s"(p.conv.sXc), "s"(p.conv.sXh), "s"(p.conv.sXw),
@@ -309,7 +326,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
     batch_id = 0;
   }
   int32_t boff[3] = {0, 0, 0};
-  if (p.batch.rank > 0) {
+  if (p.batch_rank > 0) {
     uint32_t rem = batch_id;
 #pragma unroll
     for (int d = kMaxBatchDims - 1; d > 0; --d) {
@@ -331,6 +348,68 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   const int wave = ltid / 64, lane = threadIdx.x % 64;
   const int ks = wave % KS, wn = (wave / KS) % WN, wm = wave / (KS * WN);
   const int lrow = lane % 32, half = lane / 32;
+  const int rows_m = p.M - m0, cols_n = p.N - n0;
+  const int n_chunks = (p.K + BK - 1) / BK;
+  // this workgroup's share of the chunks (all of them unless K is split over blockIdx.z)
+  const int c_begin = p.n_splits > 1 ? static_cast<int>(blockIdx.z) * p.chunks_per_split : 0;
+  const int c_end = p.n_splits > 1 ? min(n_chunks, c_begin + p.chunks_per_split) : n_chunks;
+
+  // ---- direct loop: the first tile loads leave before anything else is asked of memory -------------------
+  // (bias, addends, row statistics: a few hundred instructions of set-up that would otherwise stand between the
+  // start of the wave and its first tile load)
+  constexpr int R = DIRECT > 0 ? DIRECT : 1;
+  constexpr bool PRIVATE = WM * WN == 1;  // every wave loads only what it reads itself
+  const int n_st = c_end - c_begin;
+  const int lr8 = lane / 8, lg = lane % 8;
+  // This wave's loads of a stage: load i fills quarter j (rows 8j .. 8j+7) of sub-tile `sub`.  Per lane one global
+  // pointer for the first stage and one step per stage; rows of A past M repeat the last row, columns of B past N
+  // the first column group (their products are never stored).
+  const float *gp[kStageLoads];
+  int64_t step[kStageLoads];
+  int32_t dst[kStageLoads];  // float offset inside the stage
+#pragma unroll
+  for (int i = 0; i < (DIRECT > 0 ? kStageLoads : 0); ++i) {
+    const int q = PRIVATE ? (i < 4 ? 4 * wave + i : 4 * KS + 4 * wave + (i - 4)) : wave * kStageLoads + i;
+    const int sub = q / 4, j = q % 4;
+    dst[i] = q * 256;
+    if (sub < WM * KS) {
+      const int swm = sub / KS, sks = sub % KS;
+      const int r = min(32 * swm + 8 * j + lr8, rows_m - 1);
+      gp[i] = Ab + static_cast<int64_t>(r) * p.sAm + (c_begin * BK + sks * 32 + 4 * (lg ^ ((lr8 + j) & 7)));
+      step[i] = BK;
+    } else {
+      const int sks = (sub - WM * KS) / WN, swn = (sub - WM * KS) % WN;
+      const int col = 32 * swn + 4 * lg;
+      gp[i] = Bb + static_cast<int64_t>(c_begin * BK + sks * 32 + 8 * j + lr8) * p.sBk + (col < cols_n ? col : -n0);
+      step[i] = static_cast<int64_t>(BK) * p.sBk;
+    }
+  }
+  float *ring = lds;
+  auto issue = [&](int t, int slot) {
+    float *at = ring + slot * kRingStage;
+#pragma unroll
+    for (int i = 0; i < kStageLoads; ++i) {
+      // (operands copied into locals first: with an array element written directly as an argument of this
+      // builtin the host pass silently drops the kernel's launch stub)
+      const float *from = gp[i] + t * step[i];
+      const int32_t to = dst[i];
+      __builtin_amdgcn_global_load_lds(from, at + to, 16, 0, 0);
+    }
+  };
+  // loads complete in order: "at most kStageLoads * later outstanding" means this wave's loads of stage t landed
+  auto wait_for = [&](int later) {
+    StaticFor<R>([&](auto n) {
+      if (later == decltype(n)::value) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStageLoads * decltype(n)::value) : "memory");
+      }
+    });
+  };
+  if constexpr (DIRECT > 0) {
+#pragma unroll
+    for (int s = 0; s < R - 1; ++s) {
+      if (s < n_st) issue(s, s);
+    }
+  }
 
   floatx16 acc[TM][TN];
 #pragma unroll
@@ -371,7 +450,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   constexpr bool NORM = EXTRA == 1;
   constexpr int kNormLanes = NORM ? (NT / BM > 32 ? 32 : NT / BM) : 1;  // lanes per row, a power of two
   static_assert((kNormLanes & (kNormLanes - 1)) == 0, "the merge across a row's lanes is a butterfly");
-  __shared__ float ln_rows[NORM ? 2 * BM : 1];  // mean, then 1 / sqrt(var + eps), per row of the tile
+  float *const ln_rows = lds + LDS_ELEMS;  // mean, then 1 / sqrt(var + eps), per row of the tile
   constexpr int kNormPer = 8;  // partials per lane: rows of up to 32 * kNormPer * kNormLanes elements
   float ln_part_mean[NORM ? kNormPer : 1], ln_part_m2[NORM ? kNormPer : 1];
   if constexpr (NORM) {
@@ -403,6 +482,40 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
     }
   }
 
+  // Called once the first tile loads are on their way: the statistics were requested before them and arrive first,
+  // so the merge runs while the tiles travel; the barrier behind the K loop publishes its result.
+  auto merge_rows = [&]() {
+    if constexpr (NORM) {
+      // Merge the row's partial statistics and leave mean and 1 / sqrt(var + eps) where the epilogue finds them.  Two
+      // short passes without a division per partial: the mean of the row is the weighted mean of the partial means,
+      // and the sum of squared deviations about it is the partials' own plus count * (partial mean - mean)^2 each --
+      // deviations throughout, never a difference of large squares.
+      if (p.ln_mode != 0 && !producer && ltid < BM * kNormLanes) {
+        const int row = ltid / kNormLanes, sub = ltid % kNormLanes;
+        float cnt[kNormPer];
+        float sum = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kNormPer; ++u) {
+          const int q = sub + u * kNormLanes;
+          cnt[u] = q < p.ln_parts ? static_cast<float>(min(32, p.ln_width - 32 * q)) : 0.0f;  // (absent: a clamped load)
+          sum += cnt[u] * ln_part_mean[u];
+        }
+        const float mean = GroupSum<kNormLanes>(sum) * p.ln_inv_width;
+        float m2 = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kNormPer; ++u) {
+          const float d = ln_part_mean[u] - mean;
+          m2 += cnt[u] > 0.0f ? ln_part_m2[u] + cnt[u] * d * d : 0.0f;
+        }
+        m2 = GroupSum<kNormLanes>(m2);
+        if (sub == 0) {
+          ln_rows[row] = mean;
+          ln_rows[BM + row] = 1.0f / sqrtf(m2 * p.ln_inv_width + p.ln_eps);
+        }
+      }
+    }
+  };
+
   // DEPTH chunks are in flight in registers: the loads of chunk c+DEPTH are issued while chunk c is
   // consumed, so a workgroup keeps DEPTH * (A tile + B tile) bytes outstanding instead of one chunk --
   // with only a few workgroups per CU that is what hides the L2/HBM latency.
@@ -410,8 +523,6 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   VecF<VA> ra[DEPTH][LoaderA::kPerThread];
   VecF<VB> rb[DEPTH][LoaderB::kPerThread];
   float rs[DEPTH][LoaderB::kPerThread];  // EXTRA == 2: the scale of the row each item of the B tile belongs to
-  const int rows_m = p.M - m0, cols_n = p.N - n0;
-  const int n_chunks = (p.K + BK - 1) / BK;
 
   // convolution: the output pixel this thread gathers for stays the same for the whole kernel
   bool g_valid = false;
@@ -562,99 +673,60 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
     }
   };
 
-  // this workgroup's share of the chunks (all of them unless K is split over blockIdx.z)
-  const int c_begin = p.n_splits > 1 ? static_cast<int>(blockIdx.z) * p.chunks_per_split : 0;
-  const int c_end = p.n_splits > 1 ? min(n_chunks, c_begin + p.chunks_per_split) : n_chunks;
   if constexpr (DIRECT > 0) {
-    constexpr int R = DIRECT;
-    constexpr int NW = WM * WN * KS;
-    constexpr bool PRIVATE = WM * WN == 1;  // every wave loads only what it reads itself
-    const int n_st = c_end - c_begin;
-    const int lr8 = lane / 8, lg = lane % 8;
-    // This wave's loads of a stage: load i fills quarter j (rows 8j .. 8j+7) of sub-tile `sub`.  Per lane one global
-    // pointer for the first stage and one step per stage; rows of A past M repeat the last row, columns of B past N
-    // the first column group (their products are never stored).
-    const float *gp[kStageLoads];
-    int64_t step[kStageLoads];
-    int32_t dst[kStageLoads];  // float offset inside the stage
-#pragma unroll
-    for (int i = 0; i < kStageLoads; ++i) {
-      const int q = PRIVATE ? (i < 4 ? 4 * wave + i : 4 * KS + 4 * wave + (i - 4)) : wave * kStageLoads + i;
-      const int sub = q / 4, j = q % 4;
-      dst[i] = q * 256;
-      if (sub < WM * KS) {
-        const int swm = sub / KS, sks = sub % KS;
-        const int r = min(32 * swm + 8 * j + lr8, rows_m - 1);
-        gp[i] = Ab + static_cast<int64_t>(r) * p.sAm + (c_begin * BK + sks * 32 + 4 * (lg ^ ((lr8 + j) & 7)));
-        step[i] = BK;
-      } else {
-        const int sks = (sub - WM * KS) / WN, swn = (sub - WM * KS) % WN;
-        const int col = 32 * swn + 4 * lg;
-        gp[i] = Bb + static_cast<int64_t>(c_begin * BK + sks * 32 + 8 * j + lr8) * p.sBk + (col < cols_n ? col : -n0);
-        step[i] = static_cast<int64_t>(BK) * p.sBk;
-      }
-    }
-    float *ring = lds;
-    auto issue = [&](int t, int slot) {
-      float *at = ring + slot * kRingStage;
-#pragma unroll
-      for (int i = 0; i < kStageLoads; ++i) {
-        // (operands copied into locals first: with an array element written directly as an argument of this
-        // builtin the host pass silently drops the kernel's launch stub)
-        const float *from = gp[i] + t * step[i];
-        const int32_t to = dst[i];
-        __builtin_amdgcn_global_load_lds(from, at + to, 16, 0, 0);
-      }
-    };
-    // loads complete in order: "at most kStageLoads * later outstanding" means this wave's loads of stage t landed
-    auto wait_for = [&](int later) {
-      StaticFor<R>([&](auto n) {
-        if (later == decltype(n)::value) {
-          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStageLoads * decltype(n)::value) : "memory");
-        }
-      });
-    };
     const int sw = (lrow + (lrow >> 3)) & 7;
     const int a_sub = (wm * KS + ks) * kSubTile, b_sub = (WM * KS + ks * WN + wn) * kSubTile;
-#pragma unroll
-    for (int s = 0; s < R - 1; ++s) {
-      if (s < n_st) issue(s, s);
-    }
-    for (int t0 = 0; t0 < n_st; t0 += R) {
-#pragma unroll
-      for (int s = 0; s < R; ++s) {
-        const int t = t0 + s;
-        if (t < n_st) {  // uniform over the workgroup
-          // Place (s + R - 1) % R held stage t - 1.  PRIVATE: this wave's reads of it have returned (the MFMAs that
-          // use them are issued).  Shared: every wave passed this stage's barrier only after reading stage t - 1.
-          if constexpr (PRIVATE) {
-            if (t + R - 1 < n_st) issue(t + R - 1, (s + R - 1) % R);
-            wait_for(min(n_st - 1, t + R - 1) - t);
-          } else {
-            wait_for(min(n_st - 1, t + R - 2) - t);
-            __syncthreads();
-            if (t + R - 1 < n_st) issue(t + R - 1, (s + R - 1) % R);
-          }
-          const float *as = lds + s * kRingStage + a_sub;
-          const float *bs = lds + s * kRingStage + b_sub;
-#pragma unroll
-          for (int kk = 0; kk < 32; kk += 8) {
-            const floatx4 a4 = *reinterpret_cast<const floatx4 *>(as + lrow * 32 + 4 * ((kk / 4 + half) ^ sw));
-            float b4[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) b4[e] = bs[(kk + 4 * half + e) * 32 + lrow];
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.x, b4[0], acc[0][0], 0, 0, 0);
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.y, b4[1], acc[0][0], 0, 0, 0);
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.z, b4[2], acc[0][0], 0, 0, 0);
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, b4[3], acc[0][0], 0, 0, 0);
-          }
-        }
+    merge_rows();
+    // Stage t, held in place `slot` (t % R, a constant so that the LDS offsets are immediates).
+    auto stage = [&](int t, auto slot_c) {
+      constexpr int slot = decltype(slot_c)::value;
+      // Place (slot + R - 1) % R held stage t - 1.  PRIVATE: this wave's reads of it have returned (the MFMAs that
+      // use them are issued).  Shared: every wave passed this stage's barrier only after reading stage t - 1.
+      if constexpr (PRIVATE) {
+        if (t + R - 1 < n_st) issue(t + R - 1, (slot + R - 1) % R);
+        wait_for(min(n_st - 1, t + R - 1) - t);
+      } else {
+        wait_for(min(n_st - 1, t + R - 2) - t);
+        // (the bare barrier: __syncthreads() adds a fence that waits for every outstanding load, the stages
+        // in flight included; all that has to be ordered here are the tile loads, waited for just above, and
+        // the LDS reads of stage t - 1, which returned before their MFMAs were issued)
+        __builtin_amdgcn_s_barrier();
+        if (t + R - 1 < n_st) issue(t + R - 1, (slot + R - 1) % R);
       }
+      const float *as = lds + slot * kRingStage + a_sub;
+      const float *bs = lds + slot * kRingStage + b_sub;
+      // all of the stage's operands are requested before the first product, so that the LDS round trips overlap
+      floatx4 a4[4];
+      float b4[4][4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        a4[q] = *reinterpret_cast<const floatx4 *>(as + lrow * 32 + 4 * ((2 * q + half) ^ sw));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) b4[q][e] = bs[(8 * q + 4 * half + e) * 32 + lrow];
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[q].x, b4[q][0], acc[0][0], 0, 0, 0);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[q].y, b4[q][1], acc[0][0], 0, 0, 0);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[q].z, b4[q][2], acc[0][0], 0, 0, 0);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[q].w, b4[q][3], acc[0][0], 0, 0, 0);
+      }
+    };
+    // Whole rounds of the ring run without a condition around the products: with one, the compiler carries the
+    // accumulator through the loop in vector registers and moves all 16 to the accumulation registers and back
+    // around every stage.  The last n_st % R stages follow.
+    int t0 = 0;
+    for (; t0 + R <= n_st; t0 += R) {
+      StaticFor<R>([&](auto slot_c) { stage(t0 + decltype(slot_c)::value, slot_c); });
     }
+    StaticFor<R - 1>([&](auto slot_c) {
+      if (t0 + decltype(slot_c)::value < n_st) stage(t0 + decltype(slot_c)::value, slot_c);  // uniform over the workgroup
+    });
   } else if constexpr (SPEC) {
     // Barrier j separates "chunk j is in LDS" from "chunk j is being consumed".  Producers store chunk j after
     // barrier j-1 (the consumers are then done with chunk j-2, the previous content of that buffer); consumers
     // compute chunk j after barrier j.  Both sides pass one barrier per chunk.
+    if (!producer) merge_rows();
     if (producer) {
 #pragma unroll
       for (int s = 0; s < DEPTH; ++s) {
@@ -688,6 +760,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
     for (int s = 0; s < DEPTH; ++s) {
       if (c_begin + s < c_end) load_chunk(c_begin + s, ra[s], rb[s], rs[s]);
     }
+    merge_rows();
     for (int c0 = c_begin; c0 < c_end; c0 += DEPTH) {
 #pragma unroll
       for (int s = 0; s < DEPTH; ++s) {
@@ -700,38 +773,6 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
           __syncthreads();
           compute_chunk(s & 1);
         }
-      }
-    }
-  }
-  if constexpr (NORM) {
-    // merge the row's partial statistics (Chan's update: counts, means and sums of squared deviations combine
-    // exactly, no difference of large squares) and leave mean and 1 / sqrt(var + eps) where the epilogue finds them
-    if (p.ln_mode != 0 && !producer && ltid < BM * kNormLanes) {
-      const int row = ltid / kNormLanes, sub = ltid % kNormLanes;
-      float cnt = 0.0f, mean = 0.0f, m2 = 0.0f;
-      auto merge = [&](float oc, float om, float oq) {
-        const float n = cnt + oc;
-        if (oc > 0.0f) {  // (an absent partial carries the values of a clamped load)
-          const float d = om - mean;
-          mean += d * (oc / n);
-          m2 += oq + d * d * (cnt * oc / n);
-          cnt = n;
-        }
-      };
-#pragma unroll
-      for (int u = 0; u < kNormPer; ++u) {
-        const int q = sub + u * kNormLanes;
-        const float c = q < p.ln_parts ? static_cast<float>(min(32, p.ln_width - 32 * q)) : 0.0f;
-        merge(c, ln_part_mean[u], ln_part_m2[u]);
-      }
-#pragma unroll
-      for (int off = 1; off < kNormLanes; off <<= 1) {
-        const float oc = __shfl_xor(cnt, off), om = __shfl_xor(mean, off), oq = __shfl_xor(m2, off);
-        merge(oc, om, oq);
-      }
-      if (sub == 0) {
-        ln_rows[row] = mean;
-        ln_rows[BM + row] = 1.0f / sqrtf(m2 / static_cast<float>(p.ln_width) + p.ln_eps);
       }
     }
   }
@@ -885,7 +926,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
         }
         vals[e] = v;
       }
-      if (p.chain.n != 0) RunChainBlock<EV>(p.chain, vals);
+      if (p.chain_n != 0) RunChainBlock<EV>(p.chain, vals);
       if constexpr (EXTRA != 0) {
         // both tensors are requested before either is added
         if (p.addend != nullptr) {
@@ -931,23 +972,17 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
           // statistics of this 32-column run of every row the lane's half-wave holds: mean, then the sum of squared
           // deviations from it (two butterflies over the 32 lanes of the half; columns past N count as absent)
           const int first = n0 + (wn * TN + j) * 32;
-          const float cols = static_cast<float>(min(32, p.N - first));
+          const float inv_cols = 1.0f / static_cast<float>(min(32, p.N - first));
           const int parts = (p.N + 31) / 32;
 #pragma unroll
           for (int e = 0; e < EV; ++e) {
-            float sum = n < p.N ? vals[e] : 0.0f;
-#pragma unroll
-            for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-            const float mean = sum / cols;
+            const float mean = GroupSum<32>(n < p.N ? vals[e] : 0.0f) * inv_cols;
             const float d = n < p.N ? vals[e] - mean : 0.0f;
-            float sq = d * d;
-#pragma unroll
-            for (int off = 16; off > 0; off >>= 1) sq += __shfl_xor(sq, off);
+            const float sq = GroupSum<32>(d * d);
             const int m = m0 + (wm * TM + i) * 32 + tile_row(e);
             if (lrow == 0 && m < p.M && first < p.N) {
               float *at = p.ln_stats_out + (static_cast<int64_t>(m) * parts + first / 32) * 2;
-              at[0] = mean;
-              at[1] = sq;
+              *reinterpret_cast<float2 *>(at) = make_float2(mean, sq);
             }
           }
         }
@@ -1204,6 +1239,8 @@ template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VE
 int LaunchConfig(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A, const float *B, hipStream_t s,
                  int forced_splits = 0) {
   MatmulArgs q = p;
+  q.batch_rank = p.batch.rank;
+  q.chain_n = p.chain.n;
   q.tiles_m = (p.M + BM - 1) / BM;
   q.tiles_n = (p.N + BN - 1) / BN;
   uint32_t splits = 1;
@@ -1491,6 +1528,7 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
       p.ln_width = norm->width;
       p.ln_parts = (norm->width + 31) / 32;
       p.ln_eps = static_cast<float>(norm->epsilon);
+      p.ln_inv_width = 1.0f / static_cast<float>(norm->width);
       p.ln_stats = norm->stats;
     }
     auto vector_of = [&](const fl_tensor *t, int64_t extent, const float **base, int32_t *stride) -> int {

@@ -127,6 +127,17 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
     }
     d["reads"] = reads;
     d["writes"] = writes;
+    // a LayerNormalization kept out of memory: 1 = the launch normalises its left operand on the fly, 2 = its addend;
+    // "norm_emits": the launch absorbed a LayerNormalization step and leaves row statistics for its readers
+    d["norm_mode"] = l.norm_mode;
+    d["norm_emits"] = !l.norm_stats_out.empty();
+    // ... and wrote its tensor into a buffer of its own because the planned bytes are still being read by this launch
+    if (l.group.empty() && !l.norm_stats_out.empty() && l.out.space == worker::Operand::Space::Private &&
+        plan.GetSteps()[l.members.back()].out.space != worker::Operand::Space::Private) {
+      py::dict o = OperandOf(l.out);
+      o["bytes"] = l.out.Extent();
+      d["moved_out"] = o;
+    }
     d["position"] = l.group.empty() ? l.members.back() : l.position;
     d["bytes"] = l.bytes;
     d["flops"] = l.flops;

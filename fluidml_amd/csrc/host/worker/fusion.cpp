@@ -283,6 +283,7 @@ class Scheduler {
       PairRotary(&fused);
       silent_.clear();
     }
+    if (fuse) DeferLayerNorms(&fused);
     if (fuse) PlaceConcatInputs(&fused);
     // a chain is issued where its last member stood; everything else keeps its place
     std::vector<const Launch *> at(steps_.size(), nullptr);
@@ -2154,6 +2155,194 @@ class Scheduler {
     if (Alias(l.out, l.a) || Alias(l.out, l.b)) return std::nullopt;
     l.bytes = Bytes({&l.a, &l.b, &l.out}) + static_cast<double>(steps_[*j].kernel->GetConstantBytes());
     return l;
+  }
+
+  // ---- LayerNormalizations that never reach memory -------------------------------------------------------
+  // AddCommon -> LayerNormalization behind a contraction (the post-attention and post-FFN normalisations of a
+  // transformer layer) costs a launch of its own that moves 1 MB and takes 4.5 us of pure latency.  Instead:
+  //   * the contraction in front absorbs the AddCommon (the residual becomes its addend) and, where the normalised
+  //     tensor h has no reader that needs it in memory, the LayerNormalization too: it stores the sum s in h's buffer
+  //     and leaves partial row statistics of s in a private buffer;
+  //   * every reader of h is then a contraction that takes h as its left operand -- it multiplies s with the scale
+  //     folded into its weights and applies mean and 1/sigma per row in its epilogue -- or the AddCommon of the next
+  //     such pair, whose contraction normalises s while adding it.
+  // Decided back to front: a LayerNormalization can only stay out of memory if the pair that reads it as a residual
+  // can absorb its AddCommon.  A pair whose residual is such a tensor but whose own result has to exist (a graph
+  // output, or a reader that is neither of the above) absorbs the AddCommon only and runs its LayerNormalization as
+  // a step.  Launch positions: the widened launch runs where its last member stood, so its late reads and the early
+  // use of h's buffer go through the same checks as every other chain.
+  void DeferLayerNorms(std::vector<Launch> *fused) {
+    if (const char *v = std::getenv("FLUIDML_DEFER_NORM"); v != nullptr && std::string(v) == "0") return;
+    std::vector<int> owner(steps_.size(), -1);
+    for (size_t k = 0; k < fused->size(); ++k) {
+      for (size_t m : (*fused)[k].members) owner[m] = static_cast<int>(k);
+    }
+    std::vector<size_t> norms;
+    for (size_t k = 0; k < fused->size(); ++k) {
+      if ((*fused)[k].kind == Launch::Kind::AddLayerNorm) norms.push_back(k);
+    }
+    std::sort(norms.begin(), norms.end(), [&](size_t x, size_t y) { return (*fused)[x].members.back() < (*fused)[y].members.back(); });
+    struct Decision {
+      int producer = -1;  // launch that computes one addend of the AddCommon and can take the other as its addend
+      Operand residual;   // that other addend
+      bool absorbable = false;  // the launch can take the AddCommon, one way or the other:
+      bool sum_in_place = false;  // ... writing the sum where the plan put it (the LayerNormalization then runs as a step)
+      bool deferrable = false;    // ... or taking the LayerNormalization too (every reader normalises on the fly)
+      bool relocate = false;      // deferrable, but the plan put the normalised tensor over bytes the launch still reads
+    };
+    std::map<size_t, Decision> decisions;
+    std::vector<bool> produces(fused->size(), false);  // launches an (already decided, later) pair would widen
+    auto one_row_block = [](const std::vector<int64_t> &shape) {
+      int64_t batch = 1;
+      for (size_t d = 0; d + 2 < shape.size(); ++d) batch *= shape[d];
+      return shape.size() >= 2 && batch == 1;
+    };
+    // `m` (a MatMulChain, alone or inside a group) multiplies h from the left by a constant matrix only it reads
+    auto takes_as_lhs = [&](const Launch &m, size_t reader, const Operand &h, int64_t width) {
+      if (m.kind != Launch::Kind::MatMulChain || m.members[0] != reader || Kind(reader) != OpKind::MatMul) return false;
+      if (!SameTensor(m.a, h) || m.a.viewed || !SameTensor(steps_[reader].in0, h) || m.has_skip || m.norm_mode != 0) return false;
+      const Operand &w = m.b;
+      if (w.space != Operand::Space::Constant || w.viewed || !IsFloat(w) || !DefaultLayout(w)) return false;
+      const auto &wshape = w.meta.GetShape();
+      if (wshape.size() != 2 || wshape[0] != width) return false;
+      const auto it = readers_.find(w.name);
+      if (it == readers_.end() || it->second.size() != 1) return false;  // the weights get the scale folded in
+      return !m.has_c || (m.c.space == Operand::Space::Constant && m.c.meta.GetShape().size() == 1);
+    };
+    for (auto it = norms.rbegin(); it != norms.rend(); ++it) {
+      const size_t k = *it;
+      const Launch &pair = (*fused)[k];
+      const size_t add = pair.members[0], ln = pair.members[1];
+      const auto &shape = pair.out.meta.GetShape();
+      Decision dec;
+      if (!IsFloat(pair.out) || !one_row_block(shape)) {
+        decisions[k] = dec;
+        continue;
+      }
+      for (int side = 0; side < 2 && !dec.absorbable; ++side) {
+        const Operand &y = side == 0 ? pair.a : pair.b, &x = side == 0 ? pair.b : pair.a;
+        if (y.viewed || x.viewed || !Elidable(y) || !DefaultLayout(y) || !DefaultLayout(x) || !IsFloat(x)) continue;
+        if (x.space == Operand::Space::Constant || x.meta.GetShape() != shape || y.meta.GetShape() != shape) continue;
+        const auto made = producer_.find(y.name);
+        if (made == producer_.end() || owner[made->second] < 0) continue;
+        const auto yr = readers_.find(y.name);
+        if (yr == readers_.end() || yr->second.size() != 1 || yr->second[0] != add) continue;
+        const Launch &p = (*fused)[static_cast<size_t>(owner[made->second])];
+        if (p.kind != Launch::Kind::MatMulChain || p.has_skip || !p.view_strides.empty() || p.n_inner != 0 || p.norm_mode != 0 ||
+            !SameTensor(p.out, y) || p.out.viewed || p.members.back() != made->second) {
+          continue;
+        }
+        if (!IsFloat(p.b) || p.b.viewed || !DefaultLayout(p.b) || p.b.meta.GetShape().size() != 2) continue;
+        std::vector<size_t> members = p.members;
+        members.push_back(add);
+        const std::vector<std::pair<size_t, Operand>> external = {{p.members[0], p.a}, {p.members[0], p.b}, {add, x}};
+        const Operand &sum = steps_[add].out;
+        if (!Safe(members, external)) continue;
+        dec.producer = owner[made->second];
+        dec.residual = x;
+        dec.sum_in_place = OutputDisjoint(sum, {&p.a, &p.b}) && !Alias(sum, x);
+        dec.absorbable = true;  // (unless neither form works out below)
+      }
+      if (dec.absorbable) {
+        const Launch &p = (*fused)[static_cast<size_t>(dec.producer)];
+        const int64_t rank = static_cast<int64_t>(shape.size());
+        const int64_t axis = pair.axis < 0 ? pair.axis + rank : pair.axis;
+        const kernel::Kernel &norm = *steps_[ln].kernel;
+        bool ok = axis == rank - 1 && shape.back() <= 1024 && Elidable(pair.out) && !pair.out.viewed && DefaultLayout(pair.out) &&
+                  norm.GetConstant(0) != nullptr && norm.GetConstant(1) != nullptr && Attrs(ln).t0 && Attrs(ln).t1;
+        std::vector<size_t> members = p.members;
+        members.push_back(add);
+        members.push_back(ln);
+        ok = ok && Safe(members, {{p.members[0], p.a}, {p.members[0], p.b}, {add, dec.residual}});
+        // The plan often reuses the bytes of the contraction's left operand for what comes behind it.  The launch
+        // reads while it writes, so the tensor then goes into a buffer of its own, outside the arena, like what a
+        // side branch writes: the plan's offsets stay as they are, the bytes are reported as private.
+        dec.relocate = !(OutputDisjoint(pair.out, {&p.a, &p.b}) && !Alias(pair.out, dec.residual));
+        const auto hr = readers_.find(pair.out.name);
+        ok = ok && hr != readers_.end() && !hr->second.empty();
+        for (size_t r : (ok ? hr->second : std::vector<size_t>{})) {
+          if (owner[r] < 0) {
+            ok = false;
+            break;
+          }
+          const size_t c = static_cast<size_t>(owner[r]);
+          const Launch &reader = (*fused)[c];
+          bool fine = false;
+          if (reader.kind == Launch::Kind::AddLayerNorm) {
+            const auto d = decisions.find(c);
+            fine = reader.members[0] == r && d != decisions.end() && d->second.absorbable && SameTensor(d->second.residual, pair.out);
+          } else if (reader.kind == Launch::Kind::MatMulChain) {
+            // (a launch takes one deferred operand: not the left one if it may get a deferred residual later)
+            fine = !produces[c] && takes_as_lhs(reader, r, pair.out, shape.back());
+          } else if (reader.kind == Launch::Kind::MatMulGroup) {
+            for (const Launch &m : reader.group) fine = fine || takes_as_lhs(m, r, pair.out, shape.back());
+          }
+          ok = ok && fine;
+        }
+        dec.deferrable = ok;
+        dec.absorbable = dec.deferrable || dec.sum_in_place;
+        if (dec.absorbable) produces[static_cast<size_t>(dec.producer)] = true;
+      }
+      decisions[k] = dec;
+    }
+    std::map<std::string, size_t> deferred;  // normalised tensors that stay out of memory -> their LayerNormalization step
+    std::map<std::string, Operand> moved;    // ... and where they live, if not where the plan put them
+    std::vector<bool> drop(fused->size(), false);
+    for (size_t k : norms) {
+      const Decision &dec = decisions[k];
+      if (!dec.absorbable) continue;
+      const Launch pair = (*fused)[k];
+      const size_t add = pair.members[0], ln = pair.members[1];
+      const auto from = deferred.find(dec.residual.name);
+      const bool residual_deferred = from != deferred.end() && dec.residual.space != Operand::Space::Constant;
+      if (!dec.deferrable && !residual_deferred) continue;  // the pair stays one AddLayerNorm launch
+      Launch wide = (*fused)[static_cast<size_t>(dec.producer)];
+      wide.members.push_back(add);
+      const auto at = moved.find(dec.residual.name);
+      wide.d = residual_deferred && at != moved.end() ? at->second : dec.residual;
+      wide.has_skip = true;
+      wide.bytes += static_cast<double>(dec.residual.meta.GetSize());
+      if (residual_deferred) {
+        wide.norm_mode = 2;
+        wide.norm_owner = from->second;
+        wide.norm_stats = "norm:" + dec.residual.name;
+      }
+      if (dec.deferrable) {
+        wide.members.push_back(ln);
+        wide.out = pair.out;
+        if (dec.relocate) {
+          wide.out.space = Operand::Space::Private;
+          wide.out.offset = 0;
+          wide.out.pool.clear();
+          moved[pair.out.name] = wide.out;
+        }
+        wide.norm_stats_out = "norm:" + pair.out.name;
+        deferred[pair.out.name] = ln;
+      } else {
+        wide.out = steps_[add].out;
+        taken_[ln] = false;  // the LayerNormalization runs as a step of its own, on the sum the launch wrote
+      }
+      wide.flops = Flops(wide.members);
+      (*fused)[k] = wide;
+      drop[static_cast<size_t>(dec.producer)] = true;
+      if (!dec.deferrable) continue;
+      for (size_t r : readers_.at(pair.out.name)) {
+        Launch &reader = (*fused)[static_cast<size_t>(owner[r])];
+        if (reader.kind == Launch::Kind::AddLayerNorm) continue;  // widened when its turn comes
+        reader.norm_mode = 1;
+        reader.norm_owner = ln;
+        reader.norm_stats = "norm:" + pair.out.name;
+        if (dec.relocate) {
+          reader.a = wide.out;
+          for (Launch &m : reader.group) m.a = wide.out;
+        }
+      }
+    }
+    std::vector<Launch> kept;
+    for (size_t k = 0; k < fused->size(); ++k) {
+      if (!drop[k]) kept.push_back(std::move((*fused)[k]));
+    }
+    *fused = std::move(kept);
   }
 
   // Pad (constant zero) whose result only goes through steps that re-address it -- Gather with sliding-window

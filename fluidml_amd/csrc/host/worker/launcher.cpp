@@ -155,6 +155,7 @@ void LaunchPlan::Materialize() {
   if (arena_ != nullptr) return;
   Validate();
   GetSchedule();  // may move tensors of a side branch into buffers of their own, allocated below
+  FoldNorms();
   Check(fluidml_hip_stream_create(&stream_), "creating the plan's stream");
   if (!regions_.empty()) {
     Check(fluidml_hip_stream_create(&side_stream_), "creating the plan's second stream");
@@ -196,8 +197,66 @@ const std::vector<Launch> &LaunchPlan::GetSchedule() const {
     schedule_built_ = true;
     regions_.clear();
     if (fuse_ && flags_ == 0 && !branches_off_) PlanBranches();
+    PlanNormBuffers();
   }
   return schedule_;
+}
+
+void LaunchPlan::PlanNormBuffers() const {
+  for (const Launch &l : schedule_) {
+    if (l.norm_stats_out.empty()) continue;
+    const std::vector<int64_t> &shape = l.out.meta.GetShape();
+    size_t rows = 1;
+    for (size_t d = 0; d + 1 < shape.size(); ++d) rows *= static_cast<size_t>(shape[d]);
+    const size_t parts = (static_cast<size_t>(shape.back()) + 31) / 32;
+    privates_[l.norm_stats_out].bytes = rows * parts * 2 * sizeof(float);  // (mean, M2) per run of 32 columns
+    // the tensor itself, where the plan's bytes for it are still being read by the launch that writes it
+    if (l.out.space == Operand::Space::Private && l.out.pool.empty()) privates_[l.out.name].bytes = l.out.meta.GetSize();
+  }
+}
+
+void LaunchPlan::FoldNorms() {
+  auto fold = [&](const Launch &m, size_t owner) {
+    const std::string &wname = m.b.name;
+    auto done = folded_.find(wname);
+    if (done != folded_.end()) {
+      if (done->second != owner) throw std::logic_error("plan: weights " + wname + " serve two LayerNormalizations");
+      return;
+    }
+    ConstantSlot &w = constants_.at(wname);
+    const flow::Attrs &at = steps_[owner].node->GetAttrs();
+    if (!at.t0 || !at.t1) throw std::logic_error("plan: the deferred LayerNormalization holds no scale / shift");
+    const std::vector<float64_t> &scale = at.t0->Get(), &shift = at.t1->Get(), &old = w.tensor.Get();
+    const std::vector<int64_t> &shape = w.tensor.GetShape();
+    const size_t K = static_cast<size_t>(shape[0]), N = static_cast<size_t>(shape[1]);
+    if (scale.size() != K || shift.size() != K) throw std::logic_error("plan: LayerNormalization width and weight rows differ");
+    std::vector<float64_t> scaled(old.size()), c1(N, 0.0), c2(N, 0.0);
+    for (size_t k = 0; k < K; ++k) {
+      for (size_t n = 0; n < N; ++n) {
+        // the product is what the device multiplies with, so the column sums use its fp32 value
+        const float64_t v = static_cast<float64_t>(static_cast<float>(scale[k] * old[k * N + n]));
+        scaled[k * N + n] = v;
+        c1[n] += v;
+        c2[n] += shift[k] * old[k * N + n];
+      }
+    }
+    if (m.has_c) {
+      const std::vector<float64_t> &bias = constants_.at(m.c.name).tensor.Get();
+      for (size_t n = 0; n < N; ++n) c2[n] += bias[n];
+    }
+    w.tensor = Tensor(Type::kFloat32, std::vector<int64_t>(shape), std::move(scaled));
+    constants_.insert({"norm_c1:" + wname, ConstantSlot{Tensor(Type::kFloat32, {static_cast<int64_t>(N)}, std::move(c1)), {0}, nullptr}});
+    constants_.insert({"norm_c2:" + wname, ConstantSlot{Tensor(Type::kFloat32, {static_cast<int64_t>(N)}, std::move(c2)), {0}, nullptr}});
+    folded_[wname] = owner;
+  };
+  for (const Launch &l : GetSchedule()) {
+    if (l.norm_mode != 1) continue;
+    if (l.kind == Launch::Kind::MatMulGroup) {
+      for (const Launch &m : l.group) fold(m, l.norm_owner);
+    } else {
+      fold(l, l.norm_owner);
+    }
+  }
 }
 
 namespace {
@@ -477,6 +536,44 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out)
       const kernel::TensorView b = ViewOf(Resolve(l.b), l.b);
       kernel::TensorView c;
       if (l.has_c) c = ViewOf(Resolve(l.c), l.c);
+      if (l.norm_mode != 0 || !l.norm_stats_out.empty()) {
+        // a LayerNormalization folded into the launch: see DeferLayerNorms in fusion.cpp
+        kernel::TensorView d, c1, c2, dst = out;
+        if (l.has_skip) d = ViewOf(Resolve(l.d), l.d);
+        if (!l.view_strides.empty()) {
+          dst = kernel::TensorView(out.t.base, steps_[l.members[0]].out.meta);
+          for (size_t k = 0; k < l.view_strides.size(); ++k) dst.t.strides[k] = l.view_strides[k];
+        }
+        fl_norm_fusion norm{};
+        kernel::TensorView scale, shift;
+        const fl_tensor *bias = l.has_c ? &c.t : nullptr, *col_sum = nullptr;
+        if (l.norm_mode != 0) {
+          const Step &owner = steps_[l.norm_owner];
+          norm.deferred = l.norm_mode;
+          norm.epsilon = owner.node->GetAttrs().epsilon;
+          norm.stats = static_cast<const float *>(privates_.at(l.norm_stats).device);
+          if (l.norm_mode == FL_NORM_LHS) {
+            norm.width = static_cast<int32_t>(l.a.meta.GetShape().back());
+            const ConstantSlot &s1 = constants_.at("norm_c1:" + l.b.name), &s2 = constants_.at("norm_c2:" + l.b.name);
+            c1 = kernel::TensorView(s1.device, s1.tensor.GetMeta());
+            c2 = kernel::TensorView(s2.device, s2.tensor.GetMeta());
+            col_sum = &c1.t;
+            bias = &c2.t;
+          } else {
+            norm.width = static_cast<int32_t>(l.d.meta.GetShape().back());
+            scale = owner.kernel->GetConstant(0)->View();
+            shift = owner.kernel->GetConstant(1)->View();
+            norm.scale = &scale.t;
+            norm.shift = &shift.t;
+          }
+        }
+        if (!l.norm_stats_out.empty()) norm.stats_out = static_cast<float *>(privates_.at(l.norm_stats_out).device);
+        const fl_tensor *rhs_p = &b.t, *dst_p = &dst.t;
+        rc = fluidml_hip_matmul_chain_group_norm(1, &a.t, &rhs_p, &bias, col_sum != nullptr ? &col_sum : nullptr, &dst_p, l.n_inner,
+                                                 &l.stride_outer, &l.chain, l.has_skip ? &d.t : nullptr, &norm, contract_flags,
+                                                 ctx.stream);
+        break;
+      }
       if (l.has_skip) {
         const kernel::TensorView d = ViewOf(Resolve(l.d), l.d);
         kernel::TensorView e;
@@ -513,6 +610,27 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out)
         bias_p[g] = m.has_c ? &bias[g].t : nullptr;
         dst_p[g] = &dst[g].t;
         outer[g] = m.stride_outer;
+      }
+      if (l.norm_mode == FL_NORM_LHS) {
+        // the shared left operand is the un-normalised input of a LayerNormalization that is not run
+        std::vector<kernel::TensorView> c1(n), c2(n);
+        std::vector<const fl_tensor *> c1_p(n), c2_p(n);
+        for (size_t g = 0; g < n; ++g) {
+          const ConstantSlot &s1 = constants_.at("norm_c1:" + l.group[g].b.name), &s2 = constants_.at("norm_c2:" + l.group[g].b.name);
+          c1[g] = kernel::TensorView(s1.device, s1.tensor.GetMeta());
+          c2[g] = kernel::TensorView(s2.device, s2.tensor.GetMeta());
+          c1_p[g] = &c1[g].t;
+          c2_p[g] = &c2[g].t;
+        }
+        fl_norm_fusion norm{};
+        norm.deferred = FL_NORM_LHS;
+        norm.width = static_cast<int32_t>(l.a.meta.GetShape().back());
+        norm.epsilon = steps_[l.norm_owner].node->GetAttrs().epsilon;
+        norm.stats = static_cast<const float *>(privates_.at(l.norm_stats).device);
+        rc = fluidml_hip_matmul_chain_group_norm(static_cast<int32_t>(n), &a.t, rhs_p.data(), c2_p.data(), c1_p.data(), dst_p.data(),
+                                                 l.group[0].n_inner, outer.data(), &l.group[0].chain, nullptr, &norm,
+                                                 contract_flags, ctx.stream);
+        break;
       }
       rc = fluidml_hip_matmul_chain_group(static_cast<int32_t>(n), &a.t, rhs_p.data(), bias_p.data(), dst_p.data(),
                                           l.group[0].n_inner, outer.data(), &l.group[0].chain, contract_flags,
@@ -879,6 +997,7 @@ std::string LaunchPlan::ContractionSignature(size_t i) const {
   std::ostringstream os;
   auto chain_tag = [&](const Launch &x) {
     os << " b" << (x.has_c ? 1 : 0) << "c" << x.chain.n << "s" << (x.has_skip ? (x.has_skip2 ? 2 : 1) : 0);
+    if (x.norm_mode != 0 || !x.norm_stats_out.empty()) os << " norm" << x.norm_mode << (x.norm_stats_out.empty() ? "" : "e");
     if (!x.view_strides.empty()) {
       os << " view(";
       for (size_t d = 0; d < x.view_strides.size(); ++d) os << (d ? "," : "") << x.view_strides[d];
@@ -917,6 +1036,7 @@ std::string LaunchPlan::ContractionSignature(size_t i) const {
     case Launch::Kind::MatMulGroup: {
       os << LaunchKindName(l.kind) << " ";
       OperandSignature(os, l.a);
+      if (l.norm_mode != 0) os << " norm" << l.norm_mode;
       for (const Launch &m : l.group) {
         os << " x";
         OperandSignature(os, m.b);

@@ -136,6 +136,17 @@ struct Launch {
   size_t owner = 0;  // member whose kernel owns constants / attributes the launch needs (LayerNorm, Gemm, Conv)
   size_t owner2 = 0;  // ConvPair: the second convolution
   double bytes = 0, flops = 0;
+  // A LayerNormalization that is not run: the contraction in front of it stores the tensor it would have normalised
+  // (in the LayerNormalization's output buffer) together with partial row statistics, and its readers normalise on
+  // the fly (fluidml_hip_matmul_chain_group_norm).  MatMulChain / MatMulGroup:
+  //   norm_mode 1: `a` is such a tensor (the launch multiplies LayerNorm(a)); 2: the addend `d` is.  `norm_owner` is
+  //   the LayerNormalization step whose scale, shift and epsilon apply, `norm_stats` the private buffer with the row
+  //   statistics of the deferred operand.
+  //   norm_stats_out (non-empty): the launch absorbed the LayerNormalization step behind it and leaves the partial
+  //   row statistics of its result in that private buffer; `out` is the LayerNormalization's output tensor.
+  int norm_mode = 0;
+  size_t norm_owner = 0;
+  std::string norm_stats, norm_stats_out;
   // MatMulChain / MatMulGroup / GemmChain, and a Step whose node is a MatMul or Gemm: the tile configuration the
   // launch runs with (FL_CONTRACT_TILE / FL_CONTRACT_SPLITS bits; 0 = the library's rule), set from the plan's
   // ContractionTable once the plan is on the device
@@ -269,6 +280,11 @@ class LaunchPlan {
   void Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out = nullptr) const;
   void TuneContractions();
   void ApplyContractionPicks() const;
+  // LayerNormalizations the schedule keeps out of memory: private buffers for their row statistics (host side) ...
+  void PlanNormBuffers() const;
+  // ... and, once per plan, the scale folded into the weights of the contractions that read them, with the two
+  // per-column vectors their epilogue needs (new constants "norm_c1:<weights>" and "norm_c2:<weights>")
+  void FoldNorms();
   void LaunchAll(kernel::LaunchContext &ctx) const;
   void Replay(kernel::LaunchContext &ctx);
   void PlanBranches() const;
@@ -295,6 +311,7 @@ class LaunchPlan {
   int branch_decision_ = -1;
   bool had_regions_ = false;
   std::shared_ptr<kernel::ContractionTable> table_;
+  std::map<std::string, size_t> folded_;  // weight constants that carry a LayerNormalization's scale -> that step
   void *side_stream_ = nullptr;
   std::vector<void *> region_events_;  // fork and join event of every region
   void *arena_ = nullptr;

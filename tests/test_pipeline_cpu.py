@@ -393,6 +393,21 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     assert [l["position"] for l in launches] == sorted(l["position"] for l in launches)
     kinds = {l["kind"] for l in launches}
     assert expected_kinds <= kinds
+    # A launch that took a LayerNormalization may write its tensor into a buffer of its own ("moved_out") when the
+    # planned bytes are ones it still reads.  Everything below is checked against where the tensor really is, after
+    # making sure that every launch reading it was pointed there.
+    for l in launches:
+        if "moved_out" not in l:
+            continue
+        to = l["moved_out"]
+        assert to["space"] == "private" and l["norm_emits"] and steps[l["members"][-1]]["out"]["name"] == to["name"]
+        assert [w["space"] for w in l["writes"]] == ["private"]
+        for other in launches:
+            assert all(r["space"] == "private" for r in other["reads"] if r["name"] == to["name"])
+        for s in steps:
+            for op in s["inputs"] + [s["out"]]:
+                if op["name"] == to["name"]:
+                    op.update(space="private", offset=0, pool="")
     readers = {}
     for i, s in enumerate(steps):
         for op in s["inputs"]:
@@ -822,3 +837,50 @@ def test_launch_with_a_residual_is_not_placed_into_a_concat(mods, tmp_path):
             assert "writes_into" not in l, l
         # the Concat2 still runs (at most its other input was written in place)
         assert any(l["kind"] in ("Step", "CopyInto") and len(l["members"]) == 1 for l in launches)
+
+
+@pytest.mark.parametrize("which", ["bert_base_full", "bert"])
+def test_layer_norms_are_deferred_into_contractions(mods, which, tmp_path, monkeypatch):
+    """Add + LayerNormalization behind a contraction: the contraction takes the Add and writes the un-normalised sum
+    plus partial row statistics; every reader of the normalised tensor normalises on the fly (left operand: folded
+    into the epilogue; residual: on the way into the next Add).  The plan has to be consistent -- a tensor is kept
+    un-normalised exactly when all of its readers know -- and BERT-base comes out at 66 launches or fewer."""
+    fluidml, models, _ = mods
+    path = SCHEDULE_NETS[which][0](models).save(str(tmp_path / "net.onnx"))
+
+    def plan_of(defer):
+        monkeypatch.setenv("FLUIDML_DEFER_NORM", defer)
+        ex = fluidml.Executor.make_plain_greedy("defer" + defer)
+        ex.compile(path)
+        return ex.plan()
+
+    off, on = plan_of("0"), plan_of("1")
+    assert all(l["norm_mode"] == 0 and not l["norm_emits"] for l in off["launches"])
+    steps, launches = on["steps"], on["launches"]
+    assert len(launches) < len(off["launches"])
+    if which == "bert_base_full":
+        assert len([l for l in launches if l["kind"] not in ("View", "Placed")]) <= 66
+    producer = {}
+    for l in launches:
+        for m in l["written"]:
+            producer[steps[m]["out"]["name"]] = l
+    emitted = {steps[l["members"][-1]]["out"]["name"] for l in launches if l["norm_emits"]}
+    assert emitted, "no LayerNormalization was deferred"
+    for name in emitted:
+        (ln,) = [i for i, s in enumerate(steps) if s["out"]["name"] == name]
+        assert steps[ln]["kernel"] == "LayerNormalizationConstantScaleBiasKernel"
+        assert producer[name]["kind"] in ("MatMulChain", "GemmChain") and producer[name]["members"][-1] == ln
+    # every reader of a tensor kept un-normalised normalises it, and nobody normalises anything else
+    for l in launches:
+        if l["kind"] in ("View", "Placed"):
+            continue
+        read = {op["name"] for m in l["members"] for op in steps[m]["inputs"]} - {steps[m]["out"]["name"] for m in l["members"]}
+        deferred_inputs = read & emitted
+        assert bool(deferred_inputs) == (l["norm_mode"] != 0), (l["kind"], l["members"], deferred_inputs)
+        assert len(deferred_inputs) <= 1
+        if l["norm_mode"] == 1:  # as the left operand of its contraction(s)
+            assert l["kind"] in ("MatMulChain", "MatMulGroup")
+        if l["norm_mode"] == 2:  # as the residual of an Add the launch absorbed
+            assert l["kind"] == "MatMulChain"
+    # the statistics and the tensors moved out of the arena are accounted for as private bytes
+    assert on["private_bytes"] > off["private_bytes"]

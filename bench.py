@@ -145,7 +145,9 @@ def measure(args, config, executor, per_kernel=False, per_launch=False):
         path = net.save(os.path.join(tmp, args.config + ".onnx"))
         ex = getattr(fluidml.Executor, "make_" + args.executor)(args.config, 1)
         t0 = time.perf_counter()
-        ex.compile(path)
+        # (--plan-json: the JSON the compile writes -- the DP's tables, the tile configuration picked per contraction
+        # and the side-branch decision; FLUIDML_TUNE=<that file> makes a later compile repeat the picks without timing)
+        ex.compile(path, json=getattr(args, "plan_json", None))
         compile_s = time.perf_counter() - t0
     plan = ex.plan()
 
@@ -288,6 +290,8 @@ def main():
     ap.add_argument("--no-configs", action="store_true",
                     help="default workload only: skip the `configs` key (the other configurations and the DP executor)")
     ap.add_argument("--cpu-sample-layers", type=int, default=3)
+    ap.add_argument("--plan-json", default=None, metavar="PATH",
+                    help="write the JSON of the benchmark configuration's compile there (decisions taken by timing included)")
     ap.add_argument("--per-kernel", action="store_true", help="also print a per-kernel table to stderr")
     ap.add_argument("--per-launch", action="store_true", help="also print every launch of one step, in order, to stderr")
     ap.add_argument("--bf16", action="store_true",
@@ -347,7 +351,8 @@ def main():
         # the other configurations and the DP executor, GPU legs only (no CPU baseline), fewer steps
         import types
 
-        short = types.SimpleNamespace(**{**vars(args), "steps": max(20, args.steps // 4), "warmup": max(5, args.warmup // 4)})
+        short = types.SimpleNamespace(**{**vars(args), "steps": max(20, args.steps // 4), "warmup": max(5, args.warmup // 4),
+                                         "plan_json": None})
         result["configs"] = {}
         del ex
         for name, executor in [("bert_base", "dp_greedy"), ("convbert_base", "plain_greedy"), ("gpt_neox", "plain_greedy"),

@@ -131,12 +131,25 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
     // "norm_emits": the launch absorbed a LayerNormalization step and leaves row statistics for its readers
     d["norm_mode"] = l.norm_mode;
     d["norm_emits"] = !l.norm_stats_out.empty();
-    // ... and wrote its tensor into a buffer of its own because the planned bytes are still being read by this launch
-    if (l.group.empty() && !l.norm_stats_out.empty() && l.out.space == worker::Operand::Space::Private &&
-        plan.GetSteps()[l.members.back()].out.space != worker::Operand::Space::Private) {
-      py::dict o = OperandOf(l.out);
-      o["bytes"] = l.out.Extent();
-      d["moved_out"] = o;
+    // tensors this launch writes into buffers of their own although the memory plan holds bytes for them (the
+    // planned bytes are in use when the fused launch writes or reads them)
+    {
+      py::list moved;
+      auto note = [&](const worker::Operand &out, size_t step) {
+        if (out.space == worker::Operand::Space::Private && out.pool.empty() &&
+            plan.GetSteps()[step].out.space != worker::Operand::Space::Private) {
+          py::dict o = OperandOf(out);
+          o["bytes"] = out.Extent();
+          moved.append(o);
+        }
+      };
+      if (l.kind != worker::Launch::Kind::View && l.kind != worker::Launch::Kind::Placed &&
+          (l.kind != worker::Launch::Kind::Step || l.rewired)) {
+        if (l.group.empty() && !l.members.empty()) note(l.out, l.members.back());
+        if (l.has_out2 && l.members.size() >= 2) note(l.out2, l.members[l.members.size() - 2]);
+        for (const worker::Launch &m : l.group) note(m.out, m.members.back());
+      }
+      d["moved_out"] = moved;
     }
     d["position"] = l.group.empty() ? l.members.back() : l.position;
     d["bytes"] = l.bytes;

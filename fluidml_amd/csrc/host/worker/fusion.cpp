@@ -349,6 +349,44 @@ class Scheduler {
     }
   }
 
+  // ---- tensors moved out of the arena ------------------------------------------------------------------
+  // The memory plan gives every tensor its bytes for the span between its producer and its last reader in the
+  // serial order, and reuses them outside it.  A fusion that makes a tensor appear earlier or be read later than
+  // planned can therefore find other tenants on its bytes.  Such a tensor gets a buffer of its own outside the
+  // arena instead (reported with the private bytes): the plan's offsets stay exactly the reference's, and the
+  // fusion goes ahead.  Every operand copy that names the tensor is rewritten: the plan's steps (marked rewired,
+  // so that single-step launches carry the operands too) and the operands held by the launches built so far.
+  static bool MoveOperand(Operand *op, const std::string &name) {
+    if (op->name != name || op->space != Operand::Space::Arena) return false;
+    op->space = Operand::Space::Private;
+    op->offset = 0;
+    op->pool.clear();
+    return true;
+  }
+  bool Movable(const Operand &op) const {
+    if (op.space != Operand::Space::Arena || op.viewed || std::getenv("FLUIDML_MOVE_OUT_OFF") != nullptr) return false;
+    const auto p = producer_.find(op.name);
+    return p != producer_.end() && SameTensor(steps_[p->second].out, op);
+  }
+  void MoveOut(const std::string &name, std::initializer_list<std::vector<Launch> *> lists) {
+    for (size_t i = 0; i < steps_.size(); ++i) {
+      Step &st = steps_[i];
+      bool changed = MoveOperand(&st.in0, name);
+      if (st.node->IsDoubleInputs()) changed = MoveOperand(&st.in1, name) || changed;
+      changed = MoveOperand(&st.out, name) || changed;
+      if (changed) rewired_[i] = true;
+    }
+    auto in_launch = [&](Launch &l) {
+      for (Operand *op : {&l.a, &l.b, &l.c, &l.d, &l.e, &l.out, &l.out2}) MoveOperand(op, name);
+    };
+    for (std::vector<Launch> *list : lists) {
+      for (Launch &l : *list) {
+        in_launch(l);
+        for (Launch &g : l.group) in_launch(g);
+      }
+    }
+  }
+
   // ---- view elision -----------------------------------------------------------------------------------
   // A Slice, Transpose, Squeeze, Unsqueeze, a Gather whose constant indices form an arithmetic pattern (sliding
   // windows), or (where the result is still one strided pattern) a Reshape / Flatten that no fusion has absorbed
@@ -525,15 +563,19 @@ class Scheduler {
       size_t step;           // the single step
     };
     std::vector<Write> writes;
-    for (size_t q = 0; q < steps_.size(); ++q) {
-      if (owner[q] == nullptr) writes.push_back({q, steps_[q].out, nullptr, q});
-    }
-    for (const Launch &l : *fused) {
-      const size_t pos = l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back();
-      if (l.group.empty()) writes.push_back({pos, l.out, &l, 0});
-      if (l.has_out2) writes.push_back({pos, l.out2, &l, 0});
-      for (const Launch &g : l.group) writes.push_back({pos, g.out, &l, 0});
-    }
+    auto list_writes = [&]() {
+      writes.clear();
+      for (size_t q = 0; q < steps_.size(); ++q) {
+        if (owner[q] == nullptr) writes.push_back({q, steps_[q].out, nullptr, q});
+      }
+      for (const Launch &l : *fused) {
+        const size_t pos = l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back();
+        if (l.group.empty()) writes.push_back({pos, l.out, &l, 0});
+        if (l.has_out2) writes.push_back({pos, l.out2, &l, 0});
+        for (const Launch &g : l.group) writes.push_back({pos, g.out, &l, 0});
+      }
+    };
+    list_writes();
     std::vector<const Launch *> dissolved;  // copy launches both of whose steps became views
     auto is_dissolved = [&](const Launch *l) { return std::find(dissolved.begin(), dissolved.end(), l) != dissolved.end(); };
 
@@ -625,7 +667,16 @@ class Scheduler {
         seen.source_bytes = seen_first.source_bytes;
         const Operand produced = steps_[j].out;
         if (!readers_can_see(i, produced, seen, l)) {
+          // the source's bytes are reused before the last reader runs: with the source in a buffer of its own
+          // (if that is all that stands in the way) the readers can look through after all
+          Operand apart = seen;
+          apart.space = Operand::Space::Private;
+          const Operand source = steps_[i].in0;
           steps_[j].in0 = saved;
+          if (!Movable(source) || !readers_can_see(i, produced, apart, l)) continue;
+          MoveOut(source.name, {fused});
+          list_writes();
+          --i;  // once more, from the top, with the source where nothing else lives
           continue;
         }
         rewire(produced, seen);
@@ -644,7 +695,16 @@ class Scheduler {
       if (!view) continue;
       const Operand seen = seen_through(i, *view);
       const Operand produced = steps_[i].out;
-      if (!readers_can_see(i, produced, seen, nullptr)) continue;
+      if (!readers_can_see(i, produced, seen, nullptr)) {
+        Operand apart = seen;
+        apart.space = Operand::Space::Private;
+        const Operand source = steps_[i].in0;
+        if (!Movable(source) || !readers_can_see(i, produced, apart, nullptr)) continue;
+        MoveOut(source.name, {fused});
+        list_writes();
+        --i;
+        continue;
+      }
       rewire(produced, seen);
       steps_[i].out = seen;
       elided_[i] = true;
@@ -1496,7 +1556,7 @@ class Scheduler {
   // MatMulChains that read the same left operand with the same extents (the query / key / value projections)
   // become one launch at the position of the last of them, provided that moving the earlier ones there
   // crosses no reader of their outputs and no write to what they read.
-  void GroupSiblings(std::vector<Launch> *fused) const {
+  void GroupSiblings(std::vector<Launch> *fused) {
     auto compatible = [&](const Launch &x, const Launch &y) {
       if (x.kind != Launch::Kind::MatMulChain || y.kind != Launch::Kind::MatMulChain || x.has_skip || y.has_skip) return false;
       const Step &hx = steps_[x.members[0]], &hy = steps_[y.members[0]];
@@ -1525,10 +1585,12 @@ class Scheduler {
       }
       // the largest prefix of the candidates that can meet at the position of one of them
       size_t position = 0;
+      std::vector<std::string> moves;  // outputs of hoisted members that need a buffer outside the arena
       while (set.size() >= 2) {
         bool found = false;
         for (size_t k : set) {
-          if (CanGroupAt(*fused, set, (*fused)[k].members.back())) {
+          moves.clear();
+          if (CanGroupAt(*fused, set, (*fused)[k].members.back(), &moves)) {
             position = (*fused)[k].members.back();
             found = true;
             break;
@@ -1536,6 +1598,9 @@ class Scheduler {
         }
         if (found) break;
         set.pop_back();
+      }
+      if (set.size() >= 2) {
+        for (const std::string &name : moves) MoveOut(name, {fused, &result});
       }
       if (set.size() < 2) {
         result.push_back((*fused)[i]);
@@ -1578,7 +1643,11 @@ class Scheduler {
   }
 
   // Can every launch of `set` be issued at step position `position` (the last member of one of them)?
-  bool CanGroupAt(const std::vector<Launch> &fused, const std::vector<size_t> &set, size_t position) const {
+  // `moves` collects the outputs of hoisted members whose planned bytes are in use at the earlier position: the
+  // caller moves those tensors out of the arena.
+  bool CanGroupAt(const std::vector<Launch> &fused, const std::vector<size_t> &set, size_t position,
+                  std::vector<std::string> *moves) const {
+    auto moved = [&](const Operand &op) { return std::find(moves->begin(), moves->end(), op.name) != moves->end(); };
 
     std::vector<size_t> members;
     for (size_t k : set) members.insert(members.end(), fused[k].members.begin(), fused[k].members.end());
@@ -1623,29 +1692,37 @@ class Scheduler {
           const auto it = producer_.find(op.name);
           return it == producer_.end() || !silent_[it->second];
         };
-        for (size_t s = position; s <= own; ++s) {
+        bool in_use = false;
+        for (size_t s = position; s <= own && !in_use; ++s) {
           if (is_member(s)) continue;
           const Step &st = steps_[s];
           const bool unwritten = !silent_.empty() && silent_[s];
-          if (!unwritten && Alias(st.out, l.out)) return false;
-          if (exists(st.in0) && Alias(st.in0, l.out)) return false;
-          if (st.node->IsDoubleInputs() && exists(st.in1) && Alias(st.in1, l.out)) return false;
+          if (!unwritten && Alias(st.out, l.out)) in_use = true;
+          if (exists(st.in0) && Alias(st.in0, l.out)) in_use = true;
+          if (st.node->IsDoubleInputs() && exists(st.in1) && Alias(st.in1, l.out)) in_use = true;
           if (st.has_buffer && !unwritten && l.out.space == Operand::Space::Arena && st.buffer_offset < l.out.offset + l.out.meta.GetSize() &&
               l.out.offset < st.buffer_offset + st.buffer_bytes) {
-            return false;  // scratch of a step in between (untouched by these kernels, but reserved)
+            in_use = true;  // scratch of a step in between (untouched by these kernels, but reserved)
           }
+        }
+        if (in_use) {
+          if (!Movable(l.out)) return false;
+          moves->push_back(l.out.name);
         }
       }
       // the output must not overlap what a member reads at the common position
       for (size_t other : set) {
-        if (Alias(l.out, fused[other].a)) return false;
+        if (Alias(l.out, fused[other].a) && !moved(l.out)) {
+          if (own <= position || !Movable(l.out)) return false;
+          moves->push_back(l.out.name);
+        }
       }
     }
     // outputs of different members are live together from the later one's planned position on, but a hoisted
     // output and a not-yet-dead neighbour could still collide: all outputs pairwise disjoint
     for (size_t x : set) {
       for (size_t y : set) {
-        if (x < y && Alias(fused[x].out, fused[y].out)) return false;
+        if (x < y && Alias(fused[x].out, fused[y].out) && !moved(fused[x].out) && !moved(fused[y].out)) return false;
       }
     }
     return true;

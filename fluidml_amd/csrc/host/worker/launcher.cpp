@@ -179,7 +179,11 @@ void *LaunchPlan::Resolve(const Operand &op) const {
     case Operand::Space::Arena: return static_cast<char *>(arena_) + op.offset;
     case Operand::Space::Interface: return interfaces_.at(op.name).device;
     case Operand::Space::Constant: return constants_.at(op.name).device;
-    default: return static_cast<char *>(privates_.at(op.pool.empty() ? op.name : op.pool).device) + op.offset;
+    default: {
+      const auto it = privates_.find(op.pool.empty() ? op.name : op.pool);
+      if (it == privates_.end()) throw std::logic_error("plan: no buffer outside the arena for " + op.name);
+      return static_cast<char *>(it->second.device) + op.offset;
+    }
   }
 }
 
@@ -203,15 +207,26 @@ const std::vector<Launch> &LaunchPlan::GetSchedule() const {
 }
 
 void LaunchPlan::PlanNormBuffers() const {
+  // tensors the schedule moved out of the arena (the plan's bytes for them are in use when the fused launch writes
+  // or reads them): a buffer each, named like the tensor
+  auto moved_out = [&](const Operand &out) {
+    // (a launch that writes a part of the tensor -- an input of a Concat2 placed in its output -- names the whole)
+    if (out.space != Operand::Space::Private || !out.pool.empty() || out.name.empty()) return;
+    size_t &bytes = privates_[out.name].bytes;
+    bytes = std::max(bytes, out.viewed ? out.source_bytes : out.meta.GetSize());
+  };
   for (const Launch &l : schedule_) {
+    if (l.kind != Launch::Kind::View && l.kind != Launch::Kind::Placed && (l.kind != Launch::Kind::Step || l.rewired)) {
+      if (l.group.empty()) moved_out(l.out);
+      if (l.has_out2) moved_out(l.out2);
+      for (const Launch &m : l.group) moved_out(m.out);
+    }
     if (l.norm_stats_out.empty()) continue;
     const std::vector<int64_t> &shape = l.out.meta.GetShape();
     size_t rows = 1;
     for (size_t d = 0; d + 1 < shape.size(); ++d) rows *= static_cast<size_t>(shape[d]);
     const size_t parts = (static_cast<size_t>(shape.back()) + 31) / 32;
     privates_[l.norm_stats_out].bytes = rows * parts * 2 * sizeof(float);  // (mean, M2) per run of 32 columns
-    // the tensor itself, where the plan's bytes for it are still being read by the launch that writes it
-    if (l.out.space == Operand::Space::Private && l.out.pool.empty()) privates_[l.out.name].bytes = l.out.meta.GetSize();
   }
 }
 

@@ -28,7 +28,9 @@ FL_REF_GEMM_SWAPPED_SCALARS = 1 << 3
 FL_REF_GATHER_RAW_AXIS = 1 << 4
 FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
 FL_CONTRACT_BF16 = 1 << 0
+FL_CONTRACT_ADDEND_IS_FACTOR = 1 << 1
 FL_CONTRACT_SHIFT = 16
+FL_ERR_NULL = -1
 FL_ERR_UNSUPPORTED = -8
 FL_ERR_STATIC_SCRATCH = -9
 FL_NO_ALLOC_SCRATCH_BYTES = 2 << 20

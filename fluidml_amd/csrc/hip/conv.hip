@@ -730,6 +730,8 @@ int fluidml_hip_conv_chain_scale_add(const fl_tensor *in, const fl_tensor *weigh
   fl::ConvExtras extras;
   extras.channel_scale = channel_scale;
   extras.addend = addend;
+  extras.addend_is_factor = (flags & FL_CONTRACT_ADDEND_IS_FACTOR) != 0;
+  if (extras.addend_is_factor && addend == nullptr) return FL_ERR_NULL;
   return fl::Conv(in, weights, bias, out, pads, strides, dilations, group, (flags & FL_CONTRACT_BF16) << FL_CONTRACT_SHIFT, stream,
                   chain, &extras);
 }

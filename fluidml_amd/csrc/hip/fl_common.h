@@ -93,6 +93,8 @@ struct ConvExtras {
   const fl_tensor *channel_scale = nullptr;
   // tensor of the output's shape and strides, added after the elementwise chain (a residual AddCommon behind it)
   const fl_tensor *addend = nullptr;
+  // ... or multiplied with the value instead (a MulCommon behind the convolution)
+  bool addend_is_factor = false;
   // second output: the mean of the result over its spatial dims, [N, F, 1, ..] (a ReduceMean behind the convolution)
   const fl_tensor *mean_out = nullptr;
 };

@@ -120,6 +120,7 @@ struct MatmulArgs {
   // ---- byte 192 ----
   float *ln_stats_out;                // non-null: (mean, M2) of every 32-column run of C's rows, ceil(N / 32) per row
   int32_t ln_s_scale, ln_s_shift, ln_s_c1;  // element strides of the three vectors
+  int32_t addend_is_factor;                 // EXTRA: the value is multiplied by `addend` instead
   FastDiv div_inner;
   const float *g_ln_c1[3];
   const float *gB[3];
@@ -284,7 +285,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
                "s"(p.tiles_m), "s"(p.tiles_n), "s"(p.n_splits), "s"(p.chunks_per_split), "s"(p.n_groups), "s"(p.n_inner),
                "s"(p.sCn_outer), "s"(p.bias), "s"(p.sDm), "s"(p.sDn), "s"(p.ca), "s"(p.cb), "s"(p.partials),
                "s"(p.counters), "s"(p.batch_rank), "s"(p.chain_n));
-  if constexpr (EXTRA != 0) asm volatile("" ::"s"(p.addend), "s"(p.addend2), "s"(p.k_scale), "s"(p.sKs));
+  if constexpr (EXTRA != 0) asm volatile("" ::"s"(p.addend), "s"(p.addend2), "s"(p.k_scale), "s"(p.sKs), "s"(p.addend_is_factor));
   if constexpr (EXTRA == 1) {
     asm volatile("" ::"s"(p.ln_mode), "s"(p.ln_parts), "s"(p.ln_width), "s"(p.ln_eps), "s"(p.ln_inv_width), "s"(p.ln_stats), "s"(p.ln_c1),
                  "s"(p.ln_scale), "s"(p.ln_shift), "s"(p.ln_s_scale), "s"(p.ln_s_shift), "s"(p.ln_s_c1), "s"(p.ln_stats_out));
@@ -954,8 +955,13 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
               }
             }
           }
+          if (p.addend_is_factor != 0) {
 #pragma unroll
-          for (int e = 0; e < EV; ++e) vals[e] += add[e];
+            for (int e = 0; e < EV; ++e) vals[e] *= add[e];
+          } else {
+#pragma unroll
+            for (int e = 0; e < EV; ++e) vals[e] += add[e];
+          }
           if (Eb2 != nullptr) {
 #pragma unroll
             for (int e = 0; e < EV; ++e) vals[e] += add2[e];
@@ -1372,7 +1378,7 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
              int64_t stride_outer = 0, const Siblings *siblings = nullptr, bool bf16 = false,
              const float *addend = nullptr, const float *k_scale = nullptr, int64_t k_scale_stride = 0,
              const float *addend2 = nullptr, TileChoice choice = TileChoice(), const fl_norm_fusion *norm = nullptr,
-             const fl_tensor *const *col_sum = nullptr) {
+             const fl_tensor *const *col_sum = nullptr, bool addend_is_factor = false) {
   FL_CHECK(CheckChain(chain));
   FL_CHECK(CheckView(lhs));
   FL_CHECK(CheckView(rhs));
@@ -1514,8 +1520,12 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
     // plain ones)
     if (lb != 0 || (addend2 != nullptr && addend == nullptr)) return FL_ERR_UNSUPPORTED;
     if (addend != nullptr && (p.n_groups > 1 || p.n_inner != 0)) return FL_ERR_UNSUPPORTED;
+    if (addend_is_factor && (addend == nullptr || addend2 != nullptr || norm != nullptr)) return FL_ERR_UNSUPPORTED;
     p.addend = addend;
     p.addend2 = addend2;
+    p.addend_is_factor = addend_is_factor ? 1 : 0;
+  } else if (addend_is_factor) {
+    return FL_ERR_UNSUPPORTED;
   }
   if (norm != nullptr) {
     // a LayerNormalization folded into this launch: one batch element, fp32, rows short enough for the lanes that
@@ -1680,7 +1690,8 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
       }
       return Contract(&a, &b, &c, false, false, 1.0f, 1.0f, bias != nullptr ? &d : nullptr, stream, chain, 0, 0, nullptr,
                       bf16, addend, scale != nullptr ? static_cast<const float *>(scale->base) : nullptr,
-                      scale != nullptr ? scale->strides[1] : 0);
+                      scale != nullptr ? scale->strides[1] : 0, nullptr, TileChoice(), nullptr, nullptr,
+                      extras != nullptr && extras->addend_is_factor);
     }
   }
   if (scale != nullptr || addend != nullptr) return FL_ERR_UNSUPPORTED;  // only the pointwise form carries them

@@ -93,7 +93,10 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
       written.push_back(l.members.back());
     }
     // a launch that writes into a part of another tensor (an input of a Concat2 placed in its output)
-    if (l.kind != worker::Launch::Kind::View && l.kind != worker::Launch::Kind::Placed && l.out.viewed) {
+    // (a launch that writes its own result through other strides -- a Transpose it absorbed -- is not meant)
+    if (l.kind != worker::Launch::Kind::View && l.kind != worker::Launch::Kind::Placed && l.out.viewed &&
+        (l.members.empty() || l.kind == worker::Launch::Kind::CopyInto ||
+         l.out.name != plan.GetSteps()[l.members.back()].out.name)) {
       py::dict into = OperandOf(l.out);
       into["bytes"] = l.out.Extent();
       d["writes_into"] = into;

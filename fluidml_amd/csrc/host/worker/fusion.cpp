@@ -270,6 +270,8 @@ class Scheduler {
         }
       }
     }
+    for (const std::string &name : pending_moves_) MoveOut(name, {&fused});
+    pending_moves_.clear();
     if (fuse) {
       MarkSilent(fused);
       GroupSiblings(&fused);
@@ -1320,6 +1322,45 @@ class Scheduler {
         skip = *other;
       }
     }
+    // ... or a MulCommon with a tensor of the result's shape behind it, directly or behind a Transpose that swaps the
+    // channel and pixel dims of a 1-d convolution (ConvBERT's span-based kernel: the convolved keys times the
+    // queries): the launch multiplies in its epilogue and writes the product, through transposed strides where
+    // the Transpose stood
+    bool factor = false, transposed = false;
+    std::optional<size_t> between;  // the Transpose
+    if (!add) {
+      size_t value = plain.members.back();
+      std::optional<size_t> j = SoleReader(value);
+      if (j && Kind(*j) == OpKind::Transpose && in_shape.size() == 3 && Attrs(*j).perm == std::vector<int64_t>{0, 2, 1} &&
+          DefaultLayout(steps_[*j].out) && IsFloat(steps_[*j].out)) {
+        between = *j;
+        value = *j;
+        j = SoleReader(value);
+      }
+      if (j && Kind(*j) == OpKind::MulCommon) {
+        const Operand &v = steps_[value].out;
+        const auto other = Other(*j, v);
+        if (other && IsFloat(*other) && !other->viewed && DefaultLayout(*other) && other->meta.GetShape() == v.meta.GetShape() &&
+            steps_[*j].out.meta.GetShape() == v.meta.GetShape() && DefaultLayout(steps_[*j].out) && IsFloat(steps_[*j].out) &&
+            other->space != Operand::Space::Constant) {
+          add = *j;
+          skip = *other;
+          factor = true;
+          transposed = between.has_value();
+        }
+      }
+    }
+    // `op` (default layout, the shape behind the Transpose) addressed with the dims of the convolution's own result
+    auto swapped = [&](const Operand &op) {
+      Operand seen = op;
+      seen.meta = conv.out.meta;
+      const std::vector<int64_t> st = LogicalStrides(op);
+      seen.viewed = true;
+      seen.view_offset = 0;
+      seen.view_strides = {st[0], st[2], st[1]};
+      seen.source_bytes = op.Extent();
+      return seen;
+    };
     // the widest variant whose late reads are safe
     for (int variant = 0; variant < 3; ++variant) {
       const bool with_gate = variant != 2, with_skip = variant != 1;
@@ -1337,14 +1378,23 @@ class Scheduler {
         external.push_back({i, l.a});
       }
       if (with_skip) {
+        if (between) l.members.push_back(*between);
         l.members.push_back(*add);
-        l.d = skip;
+        l.d = transposed ? swapped(skip) : skip;
         l.has_skip = true;
+        l.skip_is_factor = factor;
         external.push_back({*add, skip});
       }
       l.out = steps_[l.members.back()].out;
-      if (!Safe(l.members, external) || !OutputDisjoint(l.out, {&l.a, &l.b})) continue;
-      if ((with_gate && Alias(l.out, l.c)) || (with_skip && Alias(l.out, l.d))) continue;
+      const Operand planned_out = l.out;
+      if (with_skip && transposed) l.out = swapped(l.out);
+      if (!Safe(l.members, external)) continue;
+      if (!OutputDisjoint(l.out, {&l.a, &l.b}) || (with_gate && Alias(l.out, l.c)) || (with_skip && Alias(l.out, l.d))) {
+        // the plan reuses bytes of an operand for the result (dead by then in the serial order, still read by this
+        // launch): the result moves to a buffer of its own once the sweep is over
+        if (!Movable(planned_out)) continue;
+        pending_moves_.push_back(planned_out.name);
+      }
       l.bytes = Bytes({&l.a, &l.b, &l.out}) + static_cast<double>(steps_[i].kernel->GetConstantBytes());
       if (with_gate) l.bytes += static_cast<double>(l.c.meta.GetSize());
       if (with_skip) l.bytes += static_cast<double>(l.d.meta.GetSize());
@@ -2484,6 +2534,7 @@ class Scheduler {
 
   std::vector<Step> steps_;  // own copy: view elision rewrites the inputs of the readers
   std::vector<bool> taken_, elided_, rewired_;
+  std::vector<std::string> pending_moves_;  // results to move out of the arena when the matching sweeps are over
   std::vector<bool> silent_;   // per step: an intermediate of a fused launch, never written (filled by RetryAttention)
   std::vector<size_t> moved_;  // per step: the position its launch is issued at when a group moved it (else SIZE_MAX)
   std::vector<int> placed_;  // Concat2 steps: bit 0 / 1 = input 0 / 1 is written in place by its producer

@@ -682,8 +682,8 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out)
         if (l.has_skip) skip = ViewOf(Resolve(l.d), l.d);
         rc = fluidml_hip_conv_chain_scale_add(&a.t, &b.t, bias ? &c.t : nullptr, &out.t, padded ? at.pads.data() : nullptr,
                                               at.strides.data(), at.dilations.data(), at.group, &l.chain,
-                                              l.has_gate ? &gate.t : nullptr, l.has_skip ? &skip.t : nullptr, contract_flags,
-                                              ctx.stream);
+                                              l.has_gate ? &gate.t : nullptr, l.has_skip ? &skip.t : nullptr,
+                                              contract_flags | (l.skip_is_factor ? FL_CONTRACT_ADDEND_IS_FACTOR : 0u), ctx.stream);
         break;
       }
       rc = fluidml_hip_conv_chain(&a.t, &b.t, bias ? &c.t : nullptr, &out.t, padded ? at.pads.data() : nullptr,

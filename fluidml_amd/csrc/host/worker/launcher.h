@@ -116,6 +116,8 @@ struct Launch {
   // MatMulChain: d [and e] = tensors of the output's shape added after the chain, in this order (the AddCommon
   // steps are members): has_skip [and has_skip2]
   bool has_gate = false, has_skip = false, has_skip2 = false;
+  // ConvChain: the tensor in `d` multiplies the value instead of being added to it (a MulCommon behind the convolution)
+  bool skip_is_factor = false;
   // Attention: a = queries, b = keys (transposed), c = values, d = additive mask (has_mask), the Where step
   // `owner` holds the condition (has_cond) and s1 its fill value; s0 scales the scores, dividing if `divisor`
   bool has_mask = false, has_cond = false, divisor = false;

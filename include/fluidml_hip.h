@@ -98,7 +98,10 @@ enum fl_contract_flags {
    * by bench.py.  Launches that do not run on the matrix cores ignore it
    * (at most 8 rows against k-contiguous weights: the weights are streamed in
    * fp32; depthwise and 3-d convolutions: the direct kernel). */
-  FL_CONTRACT_BF16 = 1 << 0
+  FL_CONTRACT_BF16 = 1 << 0,
+  /* fluidml_hip_conv_chain_scale_add only: `addend` multiplies the value instead of being added to it (a MulCommon
+   * behind the convolution, reference mul.cpp) */
+  FL_CONTRACT_ADDEND_IS_FACTOR = 1 << 1
   /* bits 4..7: enum fl_contract_tile; bits 8..13: number of workgroups that share
    * the K range of a tile (FL_CONTRACT_TILE / FL_CONTRACT_SPLITS below) */
 };
@@ -459,7 +462,10 @@ int fluidml_hip_conv_chain(const fl_tensor *in, const fl_tensor *weights, const 
  * Only for a 1x1 convolution with unit stride, no padding and group 1 whose pixels are one strided run in `in`
  * and `out` (it runs as a plain contraction; fp32 whatever `flags` say).  `channel_scale` ([1, C, 1, ..], NULL:
  * none) multiplies the input, each product rounded as the separate kernel rounds it; one image only.  `addend`
- * (NULL: none) has the shape and strides of `out`.  Anything else: FL_ERR_UNSUPPORTED, nothing launched. */
+ * (NULL: none) has the shape and strides of `out`; with FL_CONTRACT_ADDEND_IS_FACTOR in `flags` the value is
+ * multiplied by it instead (MulCommonKernel behind the convolution; `out` and `addend` may then both be a
+ * transposed view, which is how a Transpose between the two is absorbed).  Anything else: FL_ERR_UNSUPPORTED,
+ * nothing launched. */
 int fluidml_hip_conv_chain_scale_add(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out, const int64_t *pads, const int64_t *strides, const int64_t *dilations, int64_t group, const fl_ew_program *chain, const fl_tensor *channel_scale, const fl_tensor *addend, uint32_t flags, void *stream);
 /* Conv{With,Without}PaddingKernel -> elementwise chain -> ReduceMeanKernel over the spatial dims (keepdims) as ONE call
  * with two results (reference conv.cpp:27-280, reduce_mean.cpp: the depthwise convolution of an inverted-residual

@@ -1553,6 +1553,36 @@ def test_conv_scale_add(device):
                                                      cabi.i64_array([1, 1]), 1, ctypes.byref(none), sc.ref(), None, 0, None) == cabi.FL_ERR_UNSUPPORTED
 
 
+def test_conv_times_tensor_through_transpose(device):
+    """Pointwise 1-d convolution -> [Transpose (0, 2, 1)] -> MulCommon with a tensor of the result's shape as one call:
+    FL_CONTRACT_ADDEND_IS_FACTOR makes the entry point multiply by its `addend`, and the Transpose is expressed by
+    handing over `out` and `addend` stored with their last two dims swapped (ConvBERT's convolved keys times queries).
+    Against the oracle's conv and mul, for the 32x32 and 64x64 tiles and ragged extents."""
+    cabi = _cabi()
+    rng = np.random.default_rng(91)
+    none = cabi.make_chain([])
+    for C, F, S, lo in [(768, 384, 128, [0, 2, 1]), (64, 32, 16, [0, 2, 1]), (96, 50, 37, [0, 2, 1]), (512, 1024, 256, [0, 2, 1]),
+                        (128, 64, 40, None)]:
+        announce("conv x tensor", C, F, S, lo)
+        x, w, bias = rand(rng, (1, C, S), -1, 1), rand(rng, (F, C, 1), -0.2, 0.2), rand(rng, (F,), -1, 1)
+        q = rand(rng, (1, F, S), -1, 1)
+        conv = ok.View.empty((1, F, S))
+        ok.conv(ok.View(x), ok.View(w), ok.View(bias), conv, None, [1], [1], 1, 0)
+        hq = ok.View.empty((1, F, S), np.float32, lo)
+        hq.logical()[...] = q
+        want = ok.View.empty((1, F, S), np.float32, lo)
+        ok.binary_f32(ok.BOP_MUL, conv, hq, want)
+        dx, dw, db = (DeviceView(ok.View(t), device) for t in (x, w, bias))
+        dq = DeviceView(hq, device)
+        do = DeviceView(ok.View.empty((1, F, S), np.float32, lo, fill=7), device)
+        cabi.call("conv_chain_scale_add", dx.ref(), dw.ref(), db.ref(), do.ref(), None, cabi.i64_array([1]), cabi.i64_array([1]),
+                  ctypes.c_int64(1), ctypes.byref(none), None, dq.ref(), ctypes.c_uint32(cabi.FL_CONTRACT_ADDEND_IS_FACTOR), None)
+        assert_close(do.logical(), want.logical(), what="pointwise conv times a tensor")
+    # the factor flag without a tensor is refused
+    assert cabi.lib.fluidml_hip_conv_chain_scale_add(dx.ref(), dw.ref(), db.ref(), do.ref(), None, cabi.i64_array([1]), cabi.i64_array([1]), 1,
+                                                     ctypes.byref(none), None, None, cabi.FL_CONTRACT_ADDEND_IS_FACTOR, None) == cabi.FL_ERR_NULL
+
+
 def test_conv_chain_mean(device):
     """Convolution -> swish chain -> ReduceMean over the spatial dims with both results from one call: depthwise 3x3 and
     5x5, strides 1 and 2 (one workgroup per plane), a channels-last input, and the shapes that take the two-launch

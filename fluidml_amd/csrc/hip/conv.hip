@@ -182,10 +182,9 @@ __global__ __launch_bounds__(kBlock) void ConvDepthwisePlaneKernel(PlaneArgs p, 
 int ConvDepthwisePlane(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
                        const int64_t *pads, const int64_t *strides, const int64_t *dilations, const fl_ew_program *chain,
                        const fl_tensor *mean_out, void *stream) {
-  static const bool on = [] {
-    const char *v = std::getenv("FLUIDML_CONV_PLANE");
-    return v == nullptr || std::strtol(v, nullptr, 10) != 0;
-  }();
+  // (read at every call: a test can switch the path inside one process)
+  const char *plane_switch = std::getenv("FLUIDML_CONV_PLANE");
+  const bool on = plane_switch == nullptr || std::strtol(plane_switch, nullptr, 10) != 0;
   if (!on || out->rank != 4) return FL_ERR_UNSUPPORTED;
   const int64_t N = in->shape[0], C = in->shape[1], H = in->shape[2], W = in->shape[3];
   const int64_t OH = out->shape[2], OW = out->shape[3], K = weights->shape[2];
@@ -640,10 +639,8 @@ int ConvPair(const fl_tensor *in, const fl_tensor *w1, const fl_tensor *b1, cons
   p.vec2 = s % 4 == 0 && p.w2_s == 1 && p.w2_f % 4 == 0 && IsAligned(w2->base, 16) ? 1 : 0;
   // Many weights: two launches over many waves each, the hidden vector in the stream's workspace in between
   // (EfficientNet-B0's last blocks, 1152 x 48: 15 us in one launch).
-  static const int64_t split_bytes = [] {
-    const char *v = std::getenv("FLUIDML_PAIR_SPLIT_KB");
-    return (v != nullptr ? std::strtol(v, nullptr, 10) : 64) * int64_t{1024};
-  }();
+  const char *split_switch = std::getenv("FLUIDML_PAIR_SPLIT_KB");
+  const int64_t split_bytes = (split_switch != nullptr ? std::strtol(split_switch, nullptr, 10) : 64) * int64_t{1024};
   if ((c * s + s * f) * 4 >= split_bytes && n * s <= static_cast<int64_t>(kWorkspaceTiles * kWorkspaceTileFloats)) {
     if (StreamWorkspace *ws = GetStreamWorkspace(AsStream(stream))) {
       float *hidden = ws->partials;

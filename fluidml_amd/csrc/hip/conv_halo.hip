@@ -294,11 +294,8 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
 
 // Environment FLUIDML_CONV_HALO=0 keeps every convolution on the implicit-GEMM path.
 bool HaloEnabled() {
-  static const bool on = [] {
-    const char *v = std::getenv("FLUIDML_CONV_HALO");
-    return v == nullptr || std::strtol(v, nullptr, 10) != 0;
-  }();
-  return on;
+  const char *v = std::getenv("FLUIDML_CONV_HALO");  // (read at every call)
+  return v == nullptr || std::strtol(v, nullptr, 10) != 0;
 }
 
 }  // namespace

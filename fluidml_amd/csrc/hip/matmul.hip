@@ -1232,12 +1232,9 @@ inline TileChoice ChoiceOf(uint32_t contract_flags) {
 // Upper bound on the number of K splits per tile (environment FLUIDML_SPLITK; default 4 for the 32x32 tile and
 // 16 for the 64x64 tile; 1 = never split).
 inline int64_t SplitKLimit(int64_t fallback) {
-  static const int64_t limit = [] {
-    const char *v = std::getenv("FLUIDML_SPLITK");
-    const long n = v != nullptr ? std::strtol(v, nullptr, 10) : 0;
-    return static_cast<int64_t>(n < 0 ? 0 : n);
-  }();
-  return limit > 0 ? limit : fallback;
+  const char *v = std::getenv("FLUIDML_SPLITK");  // (read at every call)
+  const long n = v != nullptr ? std::strtol(v, nullptr, 10) : 0;
+  return n > 0 ? static_cast<int64_t>(n) : fallback;
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int KS, int LA, int LB, int VEC, int DEPTH, int CONV, bool BF16,

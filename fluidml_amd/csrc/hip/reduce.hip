@@ -586,6 +586,20 @@ __global__ __launch_bounds__(kBlock) void ReduceMeanRun(ReduceArgs a, float *__r
     const uint32_t n4 = (a.n_red - head) / 4;
     const float *body = src + head;
     uint32_t j = t;
+    // (eight loads in flight per lane while the run is long enough, then four, then one)
+    for (; j + 7 * nt < n4; j += 8 * nt) {
+      float4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4 *>(body + 4 * (j + u * nt));
+      s0 += (v[0].x + v[0].y) + (v[0].z + v[0].w);
+      s1 += (v[1].x + v[1].y) + (v[1].z + v[1].w);
+      s2 += (v[2].x + v[2].y) + (v[2].z + v[2].w);
+      s3 += (v[3].x + v[3].y) + (v[3].z + v[3].w);
+      s0 += (v[4].x + v[4].y) + (v[4].z + v[4].w);
+      s1 += (v[5].x + v[5].y) + (v[5].z + v[5].w);
+      s2 += (v[6].x + v[6].y) + (v[6].z + v[6].w);
+      s3 += (v[7].x + v[7].y) + (v[7].z + v[7].w);
+    }
     for (; j + 3 * nt < n4; j += 4 * nt) {
       const float4 v0 = *reinterpret_cast<const float4 *>(body + 4 * j);
       const float4 v1 = *reinterpret_cast<const float4 *>(body + 4 * (j + nt));

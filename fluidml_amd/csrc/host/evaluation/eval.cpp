@@ -74,7 +74,9 @@ class TableCostModel : public CostModel {
           shapes = {ints(row.At("lhs_shape")), ints(row.At("rhs_shape")), ints(row.At("output_shape"))};
           layouts = {layout(row.At("lhs_layout")), layout(row.At("rhs_layout")), layout(row.At("output_layout"))};
         }
-        costs_[RowKey(kernel.first, shapes, layouts)] = static_cast<size_t>(row.At("time_cost").number);
+        // (a table written by this backend carries the DP's own figure beside the measurement where they differ)
+        costs_[RowKey(kernel.first, shapes, layouts)] =
+            static_cast<size_t>(row.Has("dp_cost") ? row.At("dp_cost").number : row.At("time_cost").number);
       }
     }
   }
@@ -107,6 +109,7 @@ class MeasuredCostModel : public CostModel {
     fluidml_hip_stream_destroy(stream_);
   }
 
+  bool IsMeasuring() const override { return true; }
   size_t Cost(KernelEval &eval, const LayoutKey &key) override {
     kernel::KernelGenerator &g = eval.GetKernelGenerator();
     if (stream_ == nullptr) {
@@ -135,6 +138,7 @@ class MeasuredCostModel : public CostModel {
     };
     bool all_natural = true;
     for (const Layout &l : key) all_natural = all_natural && natural(l);
+    last_measured_ns_ = 0;
     if (!all_natural && b.spent_ns > kBudgetPerKernelNs) {
       return std::max<size_t>(1, static_cast<size_t>((b.default_ns > 0 ? b.default_ns : 1e8) * 8.0));
     }
@@ -203,6 +207,7 @@ class MeasuredCostModel : public CostModel {
       for (size_t i = 0; i < l.size(); ++i) all_default = all_default && l[i] == i;
     }
     if (all_default) b.default_ns = best;
+    last_measured_ns_ = best;
     if (!all_default) best = best * 1.02 + 200.0;
     return std::max<size_t>(1, static_cast<size_t>(best));
   }
@@ -251,6 +256,7 @@ size_t KernelEval::Lookup(LayoutKey &&key) {
   auto it = time_costs_.find(key);
   if (it != time_costs_.end()) return it->second;
   const size_t cost = model_->Cost(*this, key);
+  measured_ns_[key] = model_->LastMeasuredNs();
   time_costs_.insert({std::move(key), cost});
   return cost;
 }
@@ -296,7 +302,15 @@ std::string KernelEval::ToJson() const {
            ",\"output_shape\":" + JoinInts(g.GetOutputMeta().GetShape()) + ",\"lhs_layout\":" + JoinLayout(kv.first[0]) +
            ",\"rhs_layout\":" + JoinLayout(kv.first[1]) + ",\"output_layout\":" + JoinLayout(kv.first[2]);
     }
-    s += ",\"time_cost\":" + std::to_string(kv.second) + "}";
+    const auto raw = measured_ns_.find(kv.first);
+    const size_t measured = raw != measured_ns_.end() && raw->second > 0 ? std::max<size_t>(1, static_cast<size_t>(raw->second)) : 0;
+    if (measured != 0 && measured != kv.second) {
+      s += ",\"time_cost\":" + std::to_string(measured) + ",\"dp_cost\":" + std::to_string(kv.second) + "}";
+    } else if (measured == 0 && raw != measured_ns_.end() && model_->IsMeasuring()) {
+      s += ",\"time_cost\":" + std::to_string(kv.second) + ",\"measured\":false}";
+    } else {
+      s += ",\"time_cost\":" + std::to_string(kv.second) + "}";
+    }
   }
   return s + "]";
 }

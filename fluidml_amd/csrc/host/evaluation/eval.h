@@ -34,6 +34,15 @@ class CostModel {
   virtual ~CostModel() = default;
   // nanoseconds (or the constant 1) for `eval`'s kernel under `key`
   virtual size_t Cost(KernelEval &eval, const LayoutKey &key) = 0;
+  // What the last Cost() call measured, in nanoseconds, before any margin the model adds for the DP's comparison;
+  // 0 when that cost was not a measurement (a constant, an estimate for a candidate left untimed).
+  double LastMeasuredNs() const { return last_measured_ns_; }
+  virtual bool IsMeasuring() const { return false; }  // true: costs come from timing kernels on the device
+
+ protected:
+  double last_measured_ns_ = 0;
+
+ public:
   static std::shared_ptr<CostModel> Make(context::Context &context);
   static std::shared_ptr<CostModel> MakeConstant();
   static std::shared_ptr<CostModel> MakeMeasured(uint32_t ref_flags,
@@ -53,7 +62,10 @@ class KernelEval {
   size_t GetTimeCost(const Layout &input_layout, const Layout &output_layout);
   size_t GetTimeCost(const Layout &lhs_layout, const Layout &rhs_layout, const Layout &output_layout);
   size_t GetShortestTimeCost();  // minimum over every layout tuple
-  // [{"input_shape"|"lhs_shape"+"rhs_shape", "output_shape", "*_layout"..., "time_cost"}, ...]
+  // [{"input_shape"|"lhs_shape"+"rhs_shape", "output_shape", "*_layout"..., "time_cost"[, "dp_cost", "measured"]}, ...]
+  // "time_cost" is the measured kernel time wherever there is one (what the reference's table and its analyzer
+  // mean by it); "dp_cost", present where it differs, is what the DP compared (the measurement plus the margin
+  // for non-default layouts, or the estimate of a candidate that was not timed: "measured": false).
   std::string ToJson() const;
   const std::map<LayoutKey, size_t> &GetTimeCosts() const { return time_costs_; }
 
@@ -62,6 +74,7 @@ class KernelEval {
   std::shared_ptr<kernel::KernelGenerator> generator_;
   std::shared_ptr<CostModel> model_;
   std::map<LayoutKey, size_t> time_costs_;
+  std::map<LayoutKey, double> measured_ns_;  // per tuple: the raw measurement behind the cost (0: none)
 };
 
 }  // namespace evaluation

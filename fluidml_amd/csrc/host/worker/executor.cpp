@@ -103,7 +103,10 @@ class ExecutorImpl : public Executor {
     double plain_ns = plain->GetModule().TimeReplayNs(kWarmup, kIters);
     dp_ns = std::min(dp_ns, context_->GetModule().TimeReplayNs(1, kIters));  // best of two rounds each
     plain_ns = std::min(plain_ns, plain->GetModule().TimeReplayNs(1, kIters));
-    const bool keep_dp = dp_ns <= plain_ns;
+    // (the DP's proposal has to win by more than the noise of the timing: otherwise the default layouts stay, and the
+    // choice -- with it the launch count and the private bytes -- does not flip from one compile to the next)
+    constexpr double kMargin = 0.015;
+    const bool keep_dp = dp_ns < plain_ns * (1.0 - kMargin);
     const std::string timing = "\"whole_graph_ns\":{\"dp\":" + std::to_string(static_cast<long long>(dp_ns)) +
                                ",\"default_layouts\":" + std::to_string(static_cast<long long>(plain_ns)) + ",\"kept\":\"" +
                                (keep_dp ? "dp" : "default_layouts") + "\"}";

@@ -290,11 +290,8 @@ struct Access {
 };
 
 bool BranchesEnabled() {
-  static const bool on = [] {
-    const char *v = std::getenv("FLUIDML_BRANCHES");
-    return v == nullptr || std::strtol(v, nullptr, 10) != 0;
-  }();
-  return on;
+  const char *v = std::getenv("FLUIDML_BRANCHES");  // (read at every compile)
+  return v == nullptr || std::strtol(v, nullptr, 10) != 0;
 }
 }  // namespace
 
@@ -356,10 +353,8 @@ void LaunchPlan::PlanBranches() const {
   // each replays 6 us slower than the same launches in a row, one with 40 us runs 22 us faster), so only runs of some
   // length are candidates; whether the candidates stay is decided by timing the schedule (DecideBranches).
   constexpr size_t kMaxRun = 10;
-  static const double env_min_us = [] {
-    const char *v = std::getenv("FLUIDML_BRANCH_MIN_US");
-    return v != nullptr ? std::strtod(v, nullptr) : -1.0;
-  }();
+  const char *min_us_switch = std::getenv("FLUIDML_BRANCH_MIN_US");
+  const double env_min_us = min_us_switch != nullptr ? std::strtod(min_us_switch, nullptr) : -1.0;
   const double min_us = env_min_us >= 0 ? env_min_us : branch_min_us_;
   auto eligible = [&](size_t a0, size_t b0, size_t e) {
     for (size_t y = b0; y < e; ++y) {

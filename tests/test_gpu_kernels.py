@@ -1503,6 +1503,39 @@ def test_conv_staged_patch(device):
             assert np.array_equal(do.logical(), first), "conv with staged patch: runs differ"
 
 
+def test_conv_paths_against_their_fallbacks(device, monkeypatch):
+    """The specialised convolution kernels against the kernels behind them, on the same inputs: the 3x3 kernel with the
+    input patch staged in LDS against the implicit GEMM (FLUIDML_CONV_HALO=0), and the depthwise kernel that owns a
+    channel plane per workgroup against the direct kernel (FLUIDML_CONV_PLANE=0).  The switches are read at every call,
+    so both sides run inside this process; each side has to meet the oracle, and the two sides each other."""
+    cabi = _cabi()
+    rng = np.random.default_rng(97)
+    none = cabi.make_chain([])
+    cases = [("FLUIDML_CONV_HALO", (2, 64, 28, 28), 96, 1, 3), ("FLUIDML_CONV_HALO", (1, 128, 14, 14), 128, 1, 3),
+             ("FLUIDML_CONV_PLANE", (1, 96, 28, 28), 96, 96, 3), ("FLUIDML_CONV_PLANE", (2, 40, 31, 29), 40, 40, 5)]
+    for switch, xshape, filters, group, k in cases:
+        wshape = (filters, xshape[1] // group, k, k)
+        pads = [k // 2] * 4
+        x, w, bias = rand(rng, xshape, -1, 1), rand(rng, wshape, -0.1, 0.1), rand(rng, (filters,), -1, 1)
+        oshape = (xshape[0], filters, xshape[2], xshape[3])
+        hx, hw, hb, ho = ok.View(x), ok.View(w), ok.View(bias), ok.View.empty(oshape)
+        ok.conv(hx, hw, hb, ho, pads, [1, 1], [1, 1], group, 0)
+        dx, dw, db = DeviceView(hx, device), DeviceView(hw, device), DeviceView(hb, device)
+        got = {}
+        for value in ("1", "0"):
+            announce("conv path", switch, value, xshape, wshape)
+            monkeypatch.setenv(switch, value)
+            do = DeviceView(ok.View.empty(oshape, np.float32, None, fill=7), device)
+            cabi.call("conv_chain", dx.ref(), dw.ref(), db.ref(), do.ref(), cabi.i64_array(pads), cabi.i64_array([1, 1]),
+                      cabi.i64_array([1, 1]), ctypes.c_int64(group), ctypes.byref(none), ctypes.c_uint32(0), None)
+            got[value] = do.logical().copy()
+            assert_close(got[value], ho.logical(), what=f"conv with {switch}={value}")
+        monkeypatch.delenv(switch)
+        assert_close(got["1"], got["0"], what=f"conv, {switch} on against off")
+        if group > 1:  # the plane kernel folds the window in the direct kernel's order: the same bits
+            assert np.array_equal(got["1"], got["0"]) or np.allclose(got["1"], got["0"], rtol=1e-6, atol=1e-7)
+
+
 def test_conv_scale_add(device):
     """MulCommon (one factor per channel) -> Conv -> chain -> AddCommon (tensor of the output's shape) as one launch, against
     the oracle's four kernels: pointwise convolutions on both tile sizes with the gate, the skip connection or both,

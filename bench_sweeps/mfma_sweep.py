@@ -9,6 +9,7 @@ import ctypes
 import json
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 matrix peak; the opt-in bf16 rows are priced against it
 
 
 def run(repeats: int = 20, out=None) -> dict:
@@ -43,13 +44,20 @@ def run(repeats: int = 20, out=None) -> dict:
 
     rows = []
 
-    def report(name, fn, flops):
+    def report(name, fn, flops, bf16=False):
         ns = median_ns(fn)
-        row = {"case": name, "us": ns / 1e3, "flops": float(flops), "TFLOP/s": flops / ns / 1e3,
-               "frac_of_fp32_mfma_peak": flops / ns / 1e3 / FP32_MFMA_PEAK_TFLOPS}
+        row = {"case": name, "us": ns / 1e3, "flops": float(flops), "TFLOP/s": flops / ns / 1e3}
+        if bf16:
+            # operands in memory stay fp32 (rounded to bf16 on their way into LDS), so the delivery of the operands,
+            # not the bf16 matrix rate, is what this path can reach; both fractions are given
+            row["frac_of_bf16_mfma_peak"] = flops / ns / 1e3 / BF16_MFMA_PEAK_TFLOPS
+            row["speedup_over_fp32"] = rows[-1]["us"] / row["us"]
+            tail = f"{100 * row['frac_of_bf16_mfma_peak']:5.1f} % of 2500, {row['speedup_over_fp32']:.2f}x the fp32 row above"
+        else:
+            row["frac_of_fp32_mfma_peak"] = flops / ns / 1e3 / FP32_MFMA_PEAK_TFLOPS
+            tail = f"{100 * row['frac_of_fp32_mfma_peak']:5.1f} % of 157.3"
         rows.append(row)
-        print(f"{name:52s} {row['us']:9.1f} us {row['TFLOP/s']:7.1f} TFLOP/s  {100 * row['frac_of_fp32_mfma_peak']:5.1f} % of 157.3",
-              file=out, flush=True)
+        print(f"{name:58s} {row['us']:9.1f} us {row['TFLOP/s']:7.1f} TFLOP/s  {tail}", file=out, flush=True)
 
     for m, k, n in [(128, 768, 768), (128, 768, 3072), (128, 3072, 768), (256, 512, 50304), (1024, 1024, 1024),
                     (2048, 2048, 2048), (4096, 4096, 4096), (8192, 4096, 8192)]:
@@ -58,6 +66,9 @@ def run(repeats: int = 20, out=None) -> dict:
         c = torch.empty(m, n, device=dev)
         va, vb, vc = view(a), view(b), view(c)
         report(f"MatMul [{m},{k}] x [{k},{n}]", lambda: cabi.call("matmul", ref(va), ref(vb), ref(vc), None), 2.0 * m * n * k)
+        if m >= 256:
+            report(f"  bf16 operands: MatMul [{m},{k}] x [{k},{n}]", lambda: cabi.call("matmul_bf16", ref(va), ref(vb), ref(vc), None),
+                   2.0 * m * n * k, bf16=True)
         del a, b, c
     one, pad = cabi.i64_array([1, 1]), cabi.i64_array([1, 1, 1, 1])
     for images, channels, size, filters in [(8, 64, 224, 64), (8, 128, 112, 128), (8, 256, 56, 256), (8, 512, 28, 512),
@@ -71,6 +82,12 @@ def run(repeats: int = 20, out=None) -> dict:
                lambda: cabi.call("conv_with_padding", ref(vx), ref(vw), ref(vbias), ref(vy), None, 0, pad, one, one,
                                  ctypes.c_int64(1), ctypes.c_uint32(0), None),
                2.0 * images * filters * size * size * channels * 9)
+        if images >= 8:
+            bits = ctypes.c_uint32(cabi.FL_CONTRACT_BF16 << cabi.FL_CONTRACT_SHIFT)
+            report(f"  bf16 operands: Conv 3x3 [{images},{channels},{size},{size}] -> {filters}",
+                   lambda: cabi.call("conv_with_padding", ref(vx), ref(vw), ref(vbias), ref(vy), None, 0, pad, one, one,
+                                     ctypes.c_int64(1), bits, None),
+                   2.0 * images * filters * size * size * channels * 9, bf16=True)
         del x, w, y
     return {"metric": "achieved fp32 MFMA throughput of the contraction kernel", "unit": "TFLOP/s",
             "peak": FP32_MFMA_PEAK_TFLOPS, "repeats": repeats, "cases": rows}

@@ -20,10 +20,13 @@
 //   * workgroup ids are folded so that consecutive tiles land on one XCD and
 //     share its L2.
 //
-// A second, opt-in path (BF16 instantiations) rounds both operands to bf16 (round to nearest even) as they
-// leave LDS and multiplies them with v_mfma_f32_32x32x8_bf16_1k; accumulation stays fp32.  The k-to-lane
-// assignment is the one the fp32 path already uses (lane half h holds k = 4h..4h+3 of a group of 8), so one
-// bf16 instruction replaces four fp32 ones.
+// A second, opt-in path (BF16 instantiations) rounds both operands to bf16 (round to nearest even) once, on their
+// way from registers into LDS, keeps the staged tiles as bf16 (half the LDS traffic) and multiplies them with
+// v_mfma_f32_32x32x16_bf16; accumulation stays fp32.  A lane feeds the instruction 8 consecutive k of its row of A and
+// of its column of B (lane half h holds k = 8h..8h+7 of a group of 16): one 128-bit LDS read where the tile is kept
+// k-contiguous ([m][k], [n][k]), eight 16-bit reads where it is kept the other way ([k][m], [k][n]: the operand's
+// fast dimension in memory is not k, and transposing 2-byte elements on the way into LDS would cost 8-way bank
+// conflicts).  One bf16 instruction replaces eight fp32 ones at half their duration.
 #include <algorithm>
 #include <cstddef>
 #include <cstdlib>
@@ -39,13 +42,16 @@ namespace {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef short bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// float -> bf16 bits, round to nearest even (NaN stays NaN)
-__device__ __forceinline__ short ToBf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<short>((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<short>(u >> 16);
+// float -> bf16 bits, round to nearest even (NaN stays NaN): the hardware conversion (v_cvt_pk_bf16_f32, two values
+// per instruction)
+__device__ __forceinline__ short ToBf16(float f) { return __builtin_bit_cast(short, static_cast<__bf16>(f)); }
+__device__ __forceinline__ uint32_t PackBf16(float lo, float hi) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, bf16x2{static_cast<__bf16>(lo), static_cast<__bf16>(hi)});
 }
 
 // Geometry of a convolution run as an implicit GEMM: M = output channels, N = images x output pixels,
@@ -208,6 +214,34 @@ struct TileLoader {
   }
 };
 
+// The same tile as bf16: VEC consecutive values of a row become VEC consecutive 16-bit words (`ld` in 16-bit words, a
+// multiple of 4).
+template <typename Loader, int VEC>
+__device__ __forceinline__ void StoreTileBf16(uint16_t *lds, int ld, const VecF<VEC> (&regs)[Loader::kPerThread], int tid,
+                                              int nt) {
+#pragma unroll
+  for (int j = 0; j < Loader::kPerThread; ++j) {
+    const int item = tid + j * nt;
+    const int row = item / Loader::kVecsPerRow, col = (item % Loader::kVecsPerRow) * VEC;
+    if (item < Loader::kItems) {
+      if constexpr (VEC == 4) {
+        *reinterpret_cast<u32x2 *>(lds + row * ld + col) =
+            u32x2{PackBf16(regs[j].v[0], regs[j].v[1]), PackBf16(regs[j].v[2], regs[j].v[3])};
+      } else {
+        lds[row * ld + col] = static_cast<uint16_t>(ToBf16(regs[j].v[0]));
+      }
+    }
+  }
+}
+
+// Eight 16-bit words `stride` words apart, packed as the matrix instruction wants its 8 values of k.
+__device__ __forceinline__ u32x4 Gather8(const uint16_t *at, int stride) {
+  uint32_t h[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) h[e] = at[e * stride];
+  return u32x4{h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16};
+}
+
 // LA: 0 = A tile kept [m][k] (A is k-contiguous), 1 = kept [k][m].
 // LB: 0 = B tile kept [k][n] (B is n-contiguous), 1 = kept [n][k].
 // CONV: 0 = plain contraction; 1 = B is the input of a convolution addressed through p.conv (LB must be 0), one
@@ -240,7 +274,10 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   constexpr int NT = 64 * WM * WN * KS;
   constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);
   constexpr int KW = BK / KS;  // k extent one wave covers per chunk
-  static_assert(KW % 8 == 0, "a wave consumes k in groups of 8");
+  static_assert(KW % (BF16 ? 16 : 8) == 0, "a wave consumes k in groups of 8 (bf16: 16)");
+  // bf16 tiles: row pitches in 16-bit words (the regions keep the fp32 tiles' sizes: half of each stays unused)
+  constexpr int LDAH = (LA == 0 ? BK : BM) + 8, LDBH = (LB == 0 ? BN : BK) + 8;
+
   constexpr int LDA = LA == 0 ? BK + 4 : BM;
   constexpr int LDB = LB == 0 ? BN : BK + 4;
   constexpr int A_ELEMS = LA == 0 ? BM * LDA : BK * LDA;
@@ -269,6 +306,24 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   // 16-byte alignment, a 7x7 image's 49 pixels, under weights that do)
   constexpr int VA = VEC == 41 ? 4 : VEC;
   constexpr int VB = CONV == 2 ? 4 : CONV == 1 || VEC == 41 ? 1 : VEC;
+  // bf16: a B tile that arrives n-contiguous in 128-bit pieces is kept as [k / 2][n][2]: a thread stages the rows 2r
+  // and 2r + 1 of its four columns, which are 16 consecutive bytes there, and the 8 values of k a lane feeds the
+  // matrix instruction are four 32-bit words one pair-row apart (`LDPB` 16-bit words) -- no 16-bit accesses, no packing.
+  constexpr bool PAIRED_B = BF16 && LB == 0 && VB == 4 && (BK * BN / 4 / NT) % 2 == 0 && BK * BN / 4 >= 2 * NT;
+  constexpr int LDPB = 2 * BN + 16;
+  // row of the B tile that item j of a thread stages, and the item's index among the tile's column groups
+  auto b_item = [&](int j, int tid, int &row, int &colgroup) {
+    constexpr int kGroups = BN / VB;
+    if constexpr (PAIRED_B) {
+      const int it = tid + (j / 2) * NT;
+      row = 2 * (it / kGroups) + (j % 2);
+      colgroup = it % kGroups;
+    } else {
+      const int it = tid + j * NT;
+      row = it / kGroups;
+      colgroup = it % kGroups;
+    }
+  };
   static_assert(!CONV || (LB == 0 && NT % (BN / VB) == 0), "the gather keeps one output pixel (group) per thread");
   static_assert(!SPEC || !CONV, "the gather of the convolution runs in the consumer waves");
   // EXTRA: 0 = none, 1 = addends in the epilogue, 2 = addends and a scale per row of B
@@ -560,7 +615,9 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
       // same item -> (k row, n column) mapping as TileLoader<BK, BN, VB, NT>: column group = thread % (BN / VB)
 #pragma unroll
       for (int j = 0; j < LoaderB::kPerThread; ++j) {
-        const int k = k0 + static_cast<int>(threadIdx.x / (BN / VB)) + j * (NT / (BN / VB));
+        int b_row, b_group;
+        b_item(j, static_cast<int>(threadIdx.x), b_row, b_group);  // (the column group is this thread's for every j)
+        const int k = k0 + b_row;
 #pragma unroll
         for (int e = 0; e < VB; ++e) qb[j].v[e] = 0.0f;
         if (g_valid && k < p.K) {
@@ -592,6 +649,19 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
           }
         }
       }
+    } else if constexpr (PAIRED_B) {
+#pragma unroll
+      for (int j = 0; j < LoaderB::kPerThread; ++j) {
+        int row, group;
+        b_item(j, ltid, row, group);
+        const int col = group * VB;
+        if (row < k_valid && col < cols_n) {
+          qb[j] = LoadVec<VB>(Bb + static_cast<int64_t>(k0 + row) * p.sBk + static_cast<int64_t>(col) * p.sBn);
+        } else {
+#pragma unroll
+          for (int e = 0; e < VB; ++e) qb[j].v[e] = 0.0f;
+        }
+      }
     } else if constexpr (LB == 0) {
       LoaderB::Load(Bb + static_cast<int64_t>(k0) * p.sBk, p.sBk, p.sBn, k_valid, cols_n, qb, ltid);
     } else {
@@ -602,6 +672,23 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
                          const float(&qs)[LoaderB::kPerThread]) {
     float *as = lds + buf * (A_ELEMS + B_ELEMS);
     float *bs = as + A_ELEMS;
+    if constexpr (BF16) {
+      StoreTileBf16<LoaderA, VA>(reinterpret_cast<uint16_t *>(as), LDAH, qa, ltid, NT);
+      if constexpr (PAIRED_B) {
+        uint16_t *bh = reinterpret_cast<uint16_t *>(bs);
+#pragma unroll
+        for (int j = 0; j < LoaderB::kPerThread; j += 2) {
+          int row, group;
+          b_item(j, ltid, row, group);
+          *reinterpret_cast<u32x4 *>(bh + (row / 2) * LDPB + group * 8) =
+              u32x4{PackBf16(qb[j].v[0], qb[j + 1].v[0]), PackBf16(qb[j].v[1], qb[j + 1].v[1]),
+                    PackBf16(qb[j].v[2], qb[j + 1].v[2]), PackBf16(qb[j].v[3], qb[j + 1].v[3])};
+        }
+      } else {
+        StoreTileBf16<LoaderB, VB>(reinterpret_cast<uint16_t *>(bs), LDBH, qb, ltid, NT);
+      }
+      return;
+    }
     LoaderA::Store(as, LDA, qa, ltid);
     if constexpr (EXTRA == 2) {
       if (p.k_scale != nullptr) {
@@ -619,6 +706,39 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
   auto compute_chunk = [&](int buf) {
     const float *as = lds + buf * (A_ELEMS + B_ELEMS);
     const float *bs = as + A_ELEMS;
+    if constexpr (BF16) {
+      const uint16_t *ah = reinterpret_cast<const uint16_t *>(as), *bh = reinterpret_cast<const uint16_t *>(bs);
+#pragma unroll
+      for (int kk = 0; kk < KW; kk += 16) {
+        const int k8 = ks * KW + kk + 8 * half;
+        u32x4 a8[TM], b8[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int m = (wm * TM + i) * 32 + lrow;
+          if constexpr (LA == 0) a8[i] = *reinterpret_cast<const u32x4 *>(ah + m * LDAH + k8);
+          else a8[i] = Gather8(ah + k8 * LDAH + m, LDAH);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int n = (wn * TN + j) * 32 + lrow;
+          if constexpr (PAIRED_B) {
+            const uint32_t *w = reinterpret_cast<const uint32_t *>(bh + (k8 / 2) * LDPB) + n;
+            b8[j] = u32x4{w[0], w[LDPB / 2], w[2 * (LDPB / 2)], w[3 * (LDPB / 2)]};
+          } else if constexpr (LB == 0) {
+            b8[j] = Gather8(bh + k8 * LDBH + n, LDBH);
+          } else {
+            b8[j] = *reinterpret_cast<const u32x4 *>(bh + n * LDBH + k8);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a8[i]), __builtin_bit_cast(bf16x8, b8[j]),
+                                                                acc[i][j], 0, 0, 0);
+      }
+      return;
+    }
 #pragma unroll
     for (int kk = 0; kk < KW; kk += 8) {
       const int kbase = ks * KW + kk + 4 * half;
@@ -651,18 +771,7 @@ __global__ __launch_bounds__(64 * WM *WN *KS *(SPEC ? 2 : 1)) void MatmulKernel(
           b[j][3] = t.w;
         }
       }
-      if constexpr (BF16) {
-        bf16x4 ah[TM], bh[TN];
-#pragma unroll
-        for (int i = 0; i < TM; ++i) ah[i] = bf16x4{ToBf16(a[i][0]), ToBf16(a[i][1]), ToBf16(a[i][2]), ToBf16(a[i][3])};
-#pragma unroll
-        for (int j = 0; j < TN; ++j) bh[j] = bf16x4{ToBf16(b[j][0]), ToBf16(b[j][1]), ToBf16(b[j][2]), ToBf16(b[j][3])};
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(ah[i], bh[j], acc[i][j], 0, 0, 0);
-      } else {
+      {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
 #pragma unroll
@@ -1331,6 +1440,14 @@ int LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A
       // the 32x32 tile whose four waves split K: direct loop where the operands allow it (BERT-base's four shapes:
       // 7.9 -> 7.45, 13.1 -> 12.0, 13.55 -> 12.3, 14.7 -> 13.4 us), else staged through registers by producer waves
       tile = kDirect && p.K % 128 == 0 ? FL_TILE_32x32_K4 : FL_TILE_32x32_STAGED;
+    }
+  }
+  if constexpr (BF16) {
+    // bf16 needs a quarter of the matrix-pipe time per tile, so what bounds it is the delivery of the fp32 operands:
+    // where there are enough of them, 128x128 tiles (2x2 waves with 2x2 accumulators each) halve that traffic
+    const int64_t big_tiles = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * n_batch;
+    if (choice.tile == FL_TILE_RULE && choice.splits == 0 && big_tiles >= 256) {
+      return LaunchConfig<128, 128, 32, 2, 2, 1, LA, LB, VEC, 2, CONV, true, false, EXTRA>(p, n_batch, C, A, B, s, 0);
     }
   }
   switch (tile) {

@@ -657,8 +657,9 @@ def test_matmul_bf16(device):
     against the oracle run on the rounded operands; the distance to the unrounded fp32 result is printed."""
     cabi = _cabi()
     rng = np.random.default_rng(81)
+    # (the last two reach the 128x128 tile; the last one with ragged extents and K not a multiple of the chunk)
     for ashape, bshape in [((1, 128, 768), (768, 768)), ((2, 3, 70, 40), (40, 50)), ((1024, 96), (96, 1024)),
-                           ((2048, 64), (64, 2048))]:
+                           ((2048, 64), (64, 2048)), ((2100, 72), (72, 2060))]:
         a, b = rand(rng, ashape, -1, 1), rand(rng, bshape, -0.05, 0.05)
         oshape = np.matmul(np.empty(ashape, np.int8), np.empty(bshape, np.int8)).shape
         want = ok.View.empty(oshape)
@@ -1113,7 +1114,7 @@ def test_gemm_and_conv_bf16(device):
     rng = np.random.default_rng(96)
     bits = cabi.FL_CONTRACT_BF16 << cabi.FL_CONTRACT_SHIFT
     # Gemm with more than 8 rows (matrix cores); transB, alpha = beta = 1
-    for M, K, N in [(64, 256, 96), (200, 1000, 130)]:
+    for M, K, N in [(64, 256, 96), (200, 1000, 130), (2048, 96, 2100)]:  # (the last: 128x128 tiles, both tiles kept k-contiguous)
         a, b, c = rand(rng, (M, K), -1, 1), rand(rng, (N, K), -0.05, 0.05), rand(rng, (N,), -0.2, 0.2)
         want, exact = ok.View.empty((M, N)), ok.View.empty((M, N))
         ok.gemm(ok.View(_round_bf16(a)), ok.View(_round_bf16(b)), ok.View(c), want, 1.0, 1.0, 0, 1, 0)
@@ -1135,6 +1136,7 @@ def test_gemm_and_conv_bf16(device):
     # 3x3 pad 1 (gather path, 32x32 and 64x64 tiles), 1x1 (plain batched contraction), strided 3x3; depthwise ignores the option
     for xshape, wshape, pads, strides, group in [((2, 8, 20, 20), (16, 8, 3, 3), [1, 1, 1, 1], [1, 1], 1),
                                                  ((4, 12, 64, 64), (128, 12, 3, 3), [1, 1, 1, 1], [1, 1], 1),  # 12 channels: not the staged-patch kernel
+                                                 ((8, 12, 64, 64), (256, 12, 3, 3), [1, 1, 1, 1], [1, 1], 1),  # the same on 128x128 tiles
                                                  ((2, 24, 14, 14), (40, 24, 1, 1), [0, 0, 0, 0], [1, 1], 1),
                                                  ((1, 8, 21, 21), (12, 8, 3, 3), [1, 1, 1, 1], [2, 2], 1),
                                                  ((1, 6, 15, 15), (6, 1, 5, 5), [2, 2, 2, 2], [2, 2], 6)]:

@@ -243,7 +243,7 @@ int ConvImplicitGemm(const fl_tensor *in, const fl_tensor *weights, const fl_ten
 
 int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
                 const int64_t *pads, const int64_t *strides, const int64_t *dilations, const fl_ew_program *chain,
-                void *stream);  // conv_halo.hip
+                void *stream, bool bf16);  // conv_halo.hip
 
 namespace {
 
@@ -341,10 +341,9 @@ int Conv(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, c
     return ConvImplicitGemm(in, weights, bias, out, pads, strides, dilations, chain, bf16, stream, extras);
   }
   if (!depthwise && flags == 0 && ns == 2) {
-    // 3x3, unit stride: the input patch is staged once per workgroup instead of gathered tap by tap (fp32 also
-    // where bf16 operands are allowed: it is faster than the implicit GEMM on bf16 -- VGG-16 at batch 8: 2794
-    // against 2358 images/s)
-    const int rc = ConvHalo3x3(in, weights, bias, out, pads, strides, dilations, chain, stream);
+    // 3x3, unit stride: the input patch is staged once per workgroup instead of gathered tap by tap (with bf16
+    // operands where they are allowed and the channels come in chunks of 16, else fp32)
+    const int rc = ConvHalo3x3(in, weights, bias, out, pads, strides, dilations, chain, stream, bf16);
     if (rc != FL_ERR_UNSUPPORTED) return rc;
   }
   if (!depthwise && flags == 0 && ns <= 2) {

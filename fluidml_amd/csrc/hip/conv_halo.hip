@@ -21,6 +21,13 @@
 //   * workgroup ids are dealt so that all filter tiles of a pixel tile run on one XCD, next to each other in time:
 //     the patch is fetched into that L2 once.
 // Bias and an elementwise chain (ReLU ...) are applied in registers before the stores, like in the other contractions.
+//
+// Opt-in bf16 (BF16 instantiations, FL_CONTRACT_BF16): the same workgroup tile and the same staging, 16 input channels per
+// chunk, both operands rounded to bf16 (nearest even, hardware conversion) on their way into LDS and multiplied with
+// v_mfma_f32_32x32x16_bf16, fp32 accumulation.  The 144 products of a chunk are split between the lane halves by channel
+// (half h takes channels 8h .. 8h+7) and each half walks its 72 (channel, tap) pairs in the weights' own order: a lane's
+// A operand of step s is 8 consecutive bf16 of its filter's row (one 128-bit LDS read), its B operand the 8 patch
+// values at the matching (channel, kh, kw) offsets -- compile-time offsets from a per-lane base, eight 16-bit reads.
 #include "fl_common.h"
 
 namespace fl {
@@ -28,6 +35,15 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t Pack2(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, bf16x2{static_cast<__bf16>(lo), static_cast<__bf16>(hi)});
+}
+__device__ __forceinline__ uint16_t ToHalfWord(float f) { return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f)); }
 
 constexpr int kTW = 16;                   // output columns per workgroup (rows: 4 per pixel tile of a wave, NV tiles)
 constexpr int kFT = 64;                   // filters per workgroup
@@ -292,6 +308,200 @@ __global__ __launch_bounds__(kThreads) void ConvHalo3x3Kernel(float *__restrict_
   }
 }
 
+// ---- bf16 operands -----------------------------------------------------------------------------------------------
+constexpr int kCC16 = 16;                        // input channels per chunk
+constexpr int kWPitch16 = 152;                   // 16-bit words per filter in LDS: 144 + 8 (76 32-bit words, as above)
+constexpr int kWElems16 = kFT * kWPitch16;
+constexpr int kWVecs16 = kFT * (kCC16 * 9 / 4);  // 2304 float4 of weights per chunk
+constexpr int kWPer16 = kWVecs16 / kThreads;     // 9
+
+template <int NV>
+__global__ __launch_bounds__(kThreads) void ConvHalo3x3Bf16Kernel(float *__restrict__ out, const float *__restrict__ in,
+                                                                  const float *__restrict__ weights, HaloArgs p) {
+  constexpr int kTH = 4 * NV;
+  constexpr int kPRows = kTH + 2;
+  constexpr int kPlane = kPRows * kPitch + 8;   // 16-bit words per channel: the two lane halves (8 channels apart) land
+                                                // in different halves of the banks
+  constexpr int kXElems = kCC16 * kPlane;
+  constexpr int kStage = kXElems + kWElems16;   // 16-bit words per buffer (12,160 / 13,696)
+  constexpr int kXItems = kCC16 * kPRows * kPCols;
+  constexpr int kXPer = (kXItems + kThreads - 1) / kThreads;  // 7 / 12
+  __shared__ __attribute__((aligned(16))) uint16_t lds[2 * kStage];
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int lrow = lane % 32, half = lane / 32;
+  const int wm = wave / 2, wn = wave % 2;
+
+  uint32_t bid = blockIdx.x;
+  const uint32_t n_tiles = p.tiles_pix * p.tiles_f;
+  if (n_tiles % 8 == 0) bid = (bid % 8) * (n_tiles / 8) + bid / 8;
+  const uint32_t f_tile = bid % p.tiles_f;
+  uint32_t pix = bid / p.tiles_f;
+  const uint32_t tw = pix % p.tiles_w;
+  pix /= p.tiles_w;
+  const uint32_t th = pix % p.tiles_h;
+  const uint32_t img = pix / p.tiles_h;
+  const int f0 = static_cast<int>(f_tile) * kFT, oh0 = static_cast<int>(th) * kTH, ow0 = static_cast<int>(tw) * kTW;
+
+  const float *w_src[kWPer16];
+  int w_dst[kWPer16];
+  bool w_ok[kWPer16];
+#pragma unroll
+  for (int t = 0; t < kWPer16; ++t) {
+    const int i = tid + t * kThreads;
+    const int f = i / 36, q = i % 36;
+    w_ok[t] = f0 + f < p.F;
+    w_src[t] = weights + static_cast<int64_t>(min(f0 + f, p.F - 1)) * p.sWf + q * 4;
+    w_dst[t] = f * kWPitch16 + q * 4;
+  }
+  const float *x_src[kXPer];
+  int x_dst[kXPer];
+  bool x_ok[kXPer];
+  const float *image = in + static_cast<int64_t>(img) * p.sXn;
+#pragma unroll
+  for (int t = 0; t < kXPer; ++t) {
+    const int i = tid + t * kThreads;
+    const int ch = i / (kPRows * kPCols), rem = i % (kPRows * kPCols);
+    const int r = rem / kPCols, s = rem % kPCols;
+    const int ih = oh0 - p.ph + r, iw = ow0 - p.pw + s;
+    x_ok[t] = i < kXItems && static_cast<uint32_t>(ih) < static_cast<uint32_t>(p.H) &&
+              static_cast<uint32_t>(iw) < static_cast<uint32_t>(p.W);
+    x_src[t] = image + (x_ok[t] ? static_cast<int64_t>(ch) * p.sXc + ih * p.sXh + iw * p.sXw : 0);
+    x_dst[t] = i < kXItems ? ch * kPlane + r * kPitch + s : -1;
+  }
+
+  floatx4 wr[kSets][kWPer16];
+  float xr[kSets][kXPer];
+  auto load_chunk = [&](int c, auto set_c) {
+    constexpr int S = decltype(set_c)::value;
+    const int c0 = c * kCC16;
+#pragma unroll
+    for (int t = 0; t < kWPer16; ++t) {
+      wr[S][t] = w_ok[t] ? *reinterpret_cast<const floatx4 *>(w_src[t] + c0 * 9) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+#pragma unroll
+    for (int t = 0; t < kXPer; ++t) xr[S][t] = x_ok[t] ? x_src[t][static_cast<int64_t>(c0) * p.sXc] : 0.0f;
+  };
+  auto store_chunk = [&](auto set_c, auto buf_c) {
+    constexpr int S = decltype(set_c)::value;
+    uint16_t *xs = lds + decltype(buf_c)::value * kStage;
+    uint16_t *ws = xs + kXElems;
+#pragma unroll
+    for (int t = 0; t < kWPer16; ++t) {
+      *reinterpret_cast<u32x2 *>(ws + w_dst[t]) = u32x2{Pack2(wr[S][t].x, wr[S][t].y), Pack2(wr[S][t].z, wr[S][t].w)};
+    }
+#pragma unroll
+    for (int t = 0; t < kXPer; ++t) {
+      if (x_dst[t] >= 0) xs[x_dst[t]] = ToHalfWord(xr[S][t]);
+    }
+  };
+
+  floatx16 acc[NV];
+#pragma unroll
+  for (int v = 0; v < NV; ++v)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[v][e] = 0.0f;
+  const int py = lrow / 8, px = lrow % 8 + 8 * wn;
+  const int a_base = (wm * 32 + lrow) * kWPitch16 + half * 72;
+  const int b_base = half * 8 * kPlane + py * kPitch + px;
+
+  const int all_chunks = p.C / kCC16;
+  const int c_first = p.n_splits > 1 ? static_cast<int>(blockIdx.y) * p.chunks_per_split : 0;
+  const int n_chunks = p.n_splits > 1 ? min(all_chunks, c_first + p.chunks_per_split) : all_chunks;
+  auto phase = [&](int c, auto idx_c) {
+    constexpr int I = decltype(idx_c)::value;
+    using Regs = std::integral_constant<int, I % kSets>;
+    using NextRegs = std::integral_constant<int, (I + 1) % kSets>;
+    using NextBuf = std::integral_constant<int, (I + 1) % 2>;
+    if (c + kSets < n_chunks) load_chunk(c + kSets, Regs{});
+    const uint16_t *xs = lds + (I % 2) * kStage;
+    const uint16_t *ws = xs + kXElems;
+#pragma unroll
+    for (int g = 0; g < 9; ++g) {
+      const u32x4 a8 = *reinterpret_cast<const u32x4 *>(ws + a_base + 8 * g);
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        uint32_t h[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int j = 8 * g + e, c8 = j / 9, kh = (j % 9) / 3, kw = j % 3;
+          h[e] = xs[b_base + c8 * kPlane + (kh + 4 * v) * kPitch + kw];
+        }
+        const u32x4 b8 = {h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16};
+        acc[v] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a8), __builtin_bit_cast(bf16x8, b8), acc[v], 0, 0, 0);
+      }
+    }
+    if (c + 1 < n_chunks) store_chunk(NextRegs{}, NextBuf{});
+    __syncthreads();
+  };
+  StaticFor<kSets>([&](auto k) {
+    if (c_first + decltype(k)::value < n_chunks) load_chunk(c_first + decltype(k)::value, k);
+  });
+  store_chunk(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+  __syncthreads();
+  for (int c = c_first; c < n_chunks; c += kSets) {
+    StaticFor<kSets>([&](auto k) {
+      if (c + decltype(k)::value < n_chunks) phase(c + decltype(k)::value, k);
+    });
+  }
+
+  // ---- channels split over workgroups: the hand-off of the fp32 kernel above -------------------------------------
+  if (p.n_splits > 1) {
+    const uint32_t n_splits = p.n_splits;
+    const uint32_t wslot = blockIdx.x * 4 + wave;
+    float *mine = p.partials + (static_cast<size_t>(wslot) * n_splits + blockIdx.y) * (NV * 1024);
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        __hip_atomic_store(mine + v * 1024 + e * 64 + lane, acc[v][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    uint32_t arrived = 0;
+    if (lane == 0) arrived = __hip_atomic_fetch_add(&p.counters[wslot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    arrived = __shfl(arrived, 0);
+    if (arrived != n_splits - 1) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // compiler ordering only
+    if (lane == 0) __hip_atomic_store(&p.counters[wslot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float *all = p.partials + static_cast<size_t>(wslot) * n_splits * (NV * 1024);
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[v][e] = 0.0f;
+    for (uint32_t z = 0; z < n_splits; ++z) {  // in split order
+#pragma unroll
+      for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          acc[v][e] += __hip_atomic_load(all + static_cast<size_t>(z) * (NV * 1024) + v * 1024 + e * 64 + lane, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+  }
+
+  float bias_v[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int f = f0 + wm * 32 + (e / 4) * 8 + half * 4 + (e % 4);
+    bias_v[e] = p.bias != nullptr && f < p.F ? p.bias[f * p.sB] : 0.0f;
+  }
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const int oh = oh0 + py + 4 * v, ow = ow0 + px;
+    float vals[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) vals[e] = acc[v][e] + bias_v[e];
+    if (p.chain.n != 0) RunChainBlock<16>(p.chain, vals);
+    if (oh < p.OH && ow < p.OW) {
+      float *dst = out + static_cast<int64_t>(img) * p.sOn + static_cast<int64_t>(oh) * p.sOh + static_cast<int64_t>(ow) * p.sOw;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int f = f0 + wm * 32 + (e / 4) * 8 + half * 4 + (e % 4);
+        if (f < p.F) dst[static_cast<int64_t>(f) * p.sOf] = vals[e];
+      }
+    }
+  }
+}
+
 // Environment FLUIDML_CONV_HALO=0 keeps every convolution on the implicit-GEMM path.
 bool HaloEnabled() {
   const char *v = std::getenv("FLUIDML_CONV_HALO");  // (read at every call)
@@ -304,7 +514,7 @@ bool HaloEnabled() {
 // implicit-GEMM path.  Operands were validated by the caller.
 int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *bias, const fl_tensor *out,
                 const int64_t *pads, const int64_t *strides, const int64_t *dilations, const fl_ew_program *chain,
-                void *stream) {
+                void *stream, bool bf16) {
   if (!HaloEnabled() || out->rank != 4) return FL_ERR_UNSUPPORTED;
   if (weights->shape[2] != 3 || weights->shape[3] != 3) return FL_ERR_UNSUPPORTED;
   for (int d = 0; d < 2; ++d) {
@@ -314,6 +524,9 @@ int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *
   const int64_t F = out->shape[1], OH = out->shape[2], OW = out->shape[3];
   const bool few = C < kCC;
   if ((C % kCC != 0 && !few) || F < 32) return FL_ERR_UNSUPPORTED;
+  // bf16 operands: chunks of 16 channels (other channel counts, and the first layer's few channels, stay fp32)
+  const bool half_words = bf16 && !few && C % kCC16 == 0;
+  const int64_t chunk = half_words ? kCC16 : kCC;
   // weights (c, kh, kw)-contiguous inside a filter, filters 16-byte aligned
   if (weights->strides[3] != 1 || weights->strides[2] != 3 || weights->strides[1] != 9) return FL_ERR_UNSUPPORTED;
   if (!few && (weights->strides[0] % 4 != 0 || !IsAligned(weights->base, 16))) return FL_ERR_UNSUPPORTED;
@@ -356,7 +569,7 @@ int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *
   // 46 us).
   constexpr int64_t kTargetWorkgroups = 512, kMinChunks = 8;
   int64_t splits = 1;
-  const int64_t all_chunks = few ? 1 : C / kCC;
+  const int64_t all_chunks = few ? 1 : C / chunk;
   if (n_tiles > 0 && n_tiles < kTargetWorkgroups && n_tiles * 4 <= static_cast<int64_t>(kWorkspaceTiles)) {
     // (one counter per wave of a tile, one workspace slot per wave, pixel tile and split)
     splits = std::min<int64_t>({kTargetWorkgroups / n_tiles, all_chunks / kMinChunks,
@@ -384,7 +597,15 @@ int ConvHalo3x3(const fl_tensor *in, const fl_tensor *weights, const fl_tensor *
   FL_LAUNCH((ConvHalo3x3Kernel<NV_, FEW_>), dim3(static_cast<uint32_t>(n_tiles), p.n_splits), dim3(kThreads), 0, AsStream(stream), \
             static_cast<float *>(out->base), static_cast<const float *>(in->base),                                  \
             static_cast<const float *>(weights->base), p)
-  if (few) {
+  if (half_words) {
+    if (nv == 2) {
+      FL_LAUNCH((ConvHalo3x3Bf16Kernel<2>), dim3(static_cast<uint32_t>(n_tiles), p.n_splits), dim3(kThreads), 0, AsStream(stream),
+                static_cast<float *>(out->base), static_cast<const float *>(in->base), static_cast<const float *>(weights->base), p);
+    } else {
+      FL_LAUNCH((ConvHalo3x3Bf16Kernel<1>), dim3(static_cast<uint32_t>(n_tiles), p.n_splits), dim3(kThreads), 0, AsStream(stream),
+                static_cast<float *>(out->base), static_cast<const float *>(in->base), static_cast<const float *>(weights->base), p);
+    }
+  } else if (few) {
     if (nv == 2) FL_HALO(2, true);
     else FL_HALO(1, true);
   } else if (nv == 2) {

@@ -128,7 +128,8 @@ enum fl_contract_tile {
   FL_TILE_64x64 = 5,        /*   64x64 tile, 2x2 waves */
   FL_TILE_64x64_K2 = 6,     /*   64x64 tile, 2x2 waves times two K slices (eight waves) */
   FL_TILE_128x64 = 7,       /*   128x64 tile, 4x2 waves */
-  FL_TILE_COUNT = 8
+  FL_TILE_128x128_STAGED = 8, /* bf16 operands only: 128x128 tile, 2x2 waves with 2x2 accumulators each, four K chunks in flight */
+  FL_TILE_COUNT = 9
 };
 #define FL_CONTRACT_TILE_SHIFT 4
 #define FL_CONTRACT_SPLIT_SHIFT 8

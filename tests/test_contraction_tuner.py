@@ -46,11 +46,11 @@ def _fake_device(times, refused=()):
 
 def test_candidates_cover_every_tile_and_the_usual_splits():
     full = _fluidml()._contraction_candidates(True)
-    assert len(full) == len(set(full)) == 7 * 9
-    assert {t for t, _ in full} == set(range(1, 8))
+    assert len(full) == len(set(full)) == 8 * 9
+    assert {t for t, _ in full} == set(range(1, 9))
     assert {s for _, s in full} == {0, 1, 2, 3, 4, 6, 8, 12, 16}
     short = _fluidml()._contraction_candidates(False)
-    assert (0, 0) not in short and set(short) == {(t, 0) for t in range(1, 8)} | {(0, s) for s in (1, 2, 4, 8)}
+    assert (0, 0) not in short and set(short) == {(t, 0) for t in range(1, 9)} | {(0, s) for s in (1, 2, 4, 8)}
 
 
 def test_selection_takes_the_fastest_admissible_configuration():
@@ -163,7 +163,7 @@ def test_every_tile_configuration_matches_the_oracle(device, shape):
     ok.binary_f32(ok.BOP_ADD, ok.View(b), t0, want)
     da, dw, db = DeviceView(ok.View(a), device, misalign), DeviceView(ok.View(w), device), DeviceView(ok.View(b), device)
     ran, refused = [], []
-    for tile in range(0, 8):
+    for tile in range(0, 9):  # (8: bf16 operands only, refused here like every configuration that does not fit)
         for splits in (0, 1, 2, 3, 4, 8):
             flags = (tile << 4) | (splits << 8)
             outs = []

@@ -1345,7 +1345,7 @@ def test_matmul_with_deferred_layer_norm(device, M, H, K0, N1):
     dc1 = [dev((gamma[:, None].astype(np.float64) * w).sum(axis=0)) for w in w1]
     dc2 = [dev(beta.astype(np.float64) @ w.astype(np.float64) + b) for w, b in zip(w1, b1)]
     da2, dw2, db2 = dev(a2), dev(w2), dev(b2)
-    for tile in range(0, 8):
+    for tile in range(0, 9):
         flags = ctypes.c_uint32(tile << 4)
         ds = DeviceView(ok.View.empty((1, M, H), np.float32, None, fill=3), device)
         stats = torch.full((M, parts, 2), 7.0, device=device)

@@ -197,7 +197,7 @@ class FlNormFusion(ctypes.Structure):
     """fl_norm_fusion of include/fluidml_hip.h"""
     _fields_ = [("deferred", ctypes.c_int32), ("width", ctypes.c_int32), ("epsilon", ctypes.c_double),
                 ("stats", ctypes.c_void_p), ("scale", ctypes.POINTER(FlTensor)), ("shift", ctypes.POINTER(FlTensor)),
-                ("stats_out", ctypes.c_void_p)]
+                ("stats_out", ctypes.c_void_p), ("addend2", ctypes.POINTER(FlTensor))]
 
 
 FL_NORM_NONE, FL_NORM_LHS, FL_NORM_ADDEND = 0, 1, 2

@@ -1648,7 +1648,7 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
     // a LayerNormalization folded into this launch: one batch element, fp32, rows short enough for the lanes that
     // merge a row's partial statistics (64x64 tile: 4 lanes x 8 partials x 32 columns)
     const int64_t real_batch = siblings != nullptr && siblings->count > 0 ? 1 : n_batch;
-    if (real_batch != 1 || bf16 || k_scale != nullptr || addend2 != nullptr) return FL_ERR_UNSUPPORTED;
+    if (real_batch != 1 || bf16 || k_scale != nullptr) return FL_ERR_UNSUPPORTED;
     if (norm->deferred != FL_NORM_NONE) {
       if (norm->stats == nullptr || norm->width <= 0 || norm->width > 1024) return FL_ERR_UNSUPPORTED;
       p.ln_mode = norm->deferred;
@@ -2027,9 +2027,22 @@ int fluidml_hip_matmul_chain_group_norm(int32_t count, const fl_tensor *lhs, con
     }
     extra = static_cast<const float *>(addend->base);
   }
+  const float *extra2 = nullptr;
+  if (norm->addend2 != nullptr) {
+    const fl_tensor *second = norm->addend2;
+    if (addend == nullptr) return FL_ERR_UNSUPPORTED;
+    FL_CHECK(fl::CheckView(second));
+    if (second->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+    if (second->rank != out[0]->rank) return FL_ERR_SHAPE;
+    for (int d = 0; d < out[0]->rank; ++d) {
+      if (second->shape[d] != out[0]->shape[d]) return FL_ERR_SHAPE;
+      if (out[0]->shape[d] > 1 && second->strides[d] != out[0]->strides[d]) return FL_ERR_UNSUPPORTED;
+    }
+    extra2 = static_cast<const float *>(second->base);
+  }
   return fl::Contract(lhs, rhs[0], out[0], false, false, 1.0f, 1.0f, bias != nullptr ? bias[0] : nullptr, stream, chain,
                       n_inner, stride_outer != nullptr ? stride_outer[0] : 0, count > 1 ? &sib : nullptr, false, extra, nullptr,
-                      0, nullptr, fl::ChoiceOf(flags), norm, col_sum);
+                      0, extra2, fl::ChoiceOf(flags), norm, col_sum);
 }
 
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,

@@ -2364,6 +2364,7 @@ class Scheduler {
         members.push_back(add);
         const std::vector<std::pair<size_t, Operand>> external = {{p.members[0], p.a}, {p.members[0], p.b}, {add, x}};
         const Operand &sum = steps_[add].out;
+        if (!DefaultLayout(sum) || sum.viewed) continue;  // (the addend is read with the strides of what the launch writes)
         if (!Safe(members, external)) continue;
         dec.producer = owner[made->second];
         dec.residual = x;
@@ -2470,6 +2471,125 @@ class Scheduler {
       if (!drop[k]) kept.push_back(std::move((*fused)[k]));
     }
     *fused = std::move(kept);
+    DeferLoneLayerNorms(fused);
+  }
+
+  // The pre-norm form (GPT-style blocks): x, written by a contraction launch (the residual sum of the block in front),
+  // goes through a LayerNormalization of its own whose result only feeds contractions as their left operand.  The
+  // launch that writes x also leaves its partial row statistics, the LayerNormalization does not run, and its readers
+  // take x itself and normalise on the fly (the FL_NORM_LHS form above; several LayerNormalizations of one x -- the two
+  // of a parallel-residual block -- each fold their own scale and shift into their readers' weights).  For the
+  // schedule the step becomes a view of x, with everything that guards a view: x's bytes must stay untouched until
+  // the last of these readers has run, else x moves to a buffer of its own.
+  void DeferLoneLayerNorms(std::vector<Launch> *fused) {
+    for (size_t i = 0; i < steps_.size(); ++i) {
+      if (Kind(i) != OpKind::LayerNormalizationConstantScaleBias || taken_[i] || elided_[i]) continue;
+      std::vector<int> owner(steps_.size(), -1);  // (rebuilt per step: the list does not change here, but stays cheap)
+      for (size_t k = 0; k < fused->size(); ++k) {
+        for (size_t m : (*fused)[k].members) owner[m] = static_cast<int>(k);
+      }
+      const Step &ln = steps_[i];
+      const Operand x = ln.in0, h = ln.out;
+      const auto &shape = h.meta.GetShape();
+      const int64_t rank = static_cast<int64_t>(shape.size());
+      int64_t batch = 1;
+      for (size_t d = 0; d + 2 < shape.size(); ++d) batch *= shape[d];
+      const int64_t axis = Attrs(i).axis < 0 ? Attrs(i).axis + rank : Attrs(i).axis;
+      if (rank < 2 || batch != 1 || axis != rank - 1 || shape.back() > 1024 || !IsFloat(h) || !IsFloat(x)) continue;
+      if (x.viewed || h.viewed || !Elidable(h) || !DefaultLayout(h) || !DefaultLayout(x) || x.meta.GetShape() != shape) continue;
+      if (ln.kernel->GetConstant(0) == nullptr || ln.kernel->GetConstant(1) == nullptr || !Attrs(i).t0 || !Attrs(i).t1) continue;
+      // who writes x
+      const auto made = producer_.find(x.name);
+      if (made == producer_.end() || owner[made->second] < 0) continue;
+      Launch &p = (*fused)[static_cast<size_t>(owner[made->second])];
+      if (p.kind != Launch::Kind::MatMulChain || !p.group.empty() || !SameTensor(p.out, x) || p.out.viewed ||
+          !p.view_strides.empty() || p.n_inner != 0 || p.members.back() != made->second) {
+        continue;
+      }
+      if (!IsFloat(p.b) || p.b.viewed || !DefaultLayout(p.b) || p.b.meta.GetShape().size() != 2) continue;
+      const std::string stats = "norm:" + x.name;
+      if (!p.norm_stats_out.empty() && p.norm_stats_out != stats) continue;
+      // who reads the normalised tensor
+      const auto hr = readers_.find(h.name);
+      if (hr == readers_.end() || hr->second.empty()) continue;
+      bool ok = true;
+      std::vector<size_t> reader_launches;
+      size_t last_position = i;
+      for (size_t r : hr->second) {
+        if (owner[r] < 0) {
+          ok = false;
+          break;
+        }
+        const size_t c = static_cast<size_t>(owner[r]);
+        const Launch &reader = (*fused)[c];
+        bool fine = false;
+        auto lhs_of = [&](const Launch &m) {
+          if (m.kind != Launch::Kind::MatMulChain || m.members[0] != r || Kind(r) != OpKind::MatMul) return false;
+          if (!SameTensor(m.a, h) || m.a.viewed || !SameTensor(steps_[r].in0, h) || m.norm_mode != 0) return false;
+          const Operand &w = m.b;
+          if (w.space != Operand::Space::Constant || w.viewed || !IsFloat(w) || !DefaultLayout(w)) return false;
+          const auto &wshape = w.meta.GetShape();
+          if (wshape.size() != 2 || wshape[0] != shape.back()) return false;
+          const auto wr = readers_.find(w.name);
+          if (wr == readers_.end() || wr->second.size() != 1) return false;  // the weights get the scale folded in
+          return !m.has_c || (m.c.space == Operand::Space::Constant && m.c.meta.GetShape().size() == 1);
+        };
+        if (reader.kind == Launch::Kind::MatMulChain) {
+          fine = !reader.has_skip && lhs_of(reader);  // (with an addend the launch may still get a deferred residual)
+        } else if (reader.kind == Launch::Kind::MatMulGroup) {
+          for (const Launch &m : reader.group) fine = fine || lhs_of(m);
+        }
+        ok = ok && fine && !Alias(reader.out, x);
+        for (const Launch &m : reader.group) ok = ok && !Alias(m.out, x);
+        const size_t pos = reader.kind == Launch::Kind::MatMulGroup ? reader.position : reader.members.back();
+        ok = ok && pos > i;
+        last_position = std::max(last_position, pos);
+        if (std::find(reader_launches.begin(), reader_launches.end(), c) == reader_launches.end()) reader_launches.push_back(c);
+      }
+      if (!ok) continue;
+      // x's bytes between the LayerNormalization and the last of its readers: anything issued in between that
+      // writes them (outputs of single steps at their own place, of launches at the place they are issued)
+      bool untouched = true;
+      for (size_t s = i + 1; s < last_position && untouched; ++s) {
+        if (owner[s] < 0 && !elided_[s] && Alias(steps_[s].out, x)) untouched = false;
+      }
+      for (const Launch &l : *fused) {
+        const size_t pos = l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back();
+        if (pos <= i || pos >= last_position) continue;
+        if (l.group.empty() && Alias(l.out, x)) untouched = false;
+        if (l.has_out2 && Alias(l.out2, x)) untouched = false;
+        for (const Launch &m : l.group) untouched = untouched && !Alias(m.out, x);
+      }
+      if (!untouched) {
+        if (!Movable(x)) continue;
+        MoveOut(x.name, {fused});
+      }
+      const Operand source = steps_[i].in0;  // (x, where it lives now)
+      p.norm_stats_out = stats;
+      for (size_t c : reader_launches) {
+        Launch &reader = (*fused)[c];
+        reader.norm_mode = 1;
+        reader.norm_owner = i;
+        reader.norm_stats = stats;
+        if (SameTensor(reader.a, h)) reader.a = source;
+        for (Launch &m : reader.group) {
+          if (SameTensor(m.a, h)) m.a = source;
+        }
+      }
+      for (size_t r : hr->second) {
+        steps_[r].in0 = source;
+        rewired_[r] = true;
+      }
+      steps_[i].out = source;  // the step is a view of x now: nothing runs, nothing is written
+      steps_[i].out.meta = h.meta;
+      steps_[i].out.viewed = true;
+      steps_[i].out.view_offset = 0;
+      steps_[i].out.view_strides = LogicalStrides(source);
+      steps_[i].out.source_bytes = source.Extent();
+      elided_[i] = true;
+      taken_[i] = true;
+      BuildReaders();
+    }
   }
 
   // Pad (constant zero) whose result only goes through steps that re-address it -- Gather with sliding-window

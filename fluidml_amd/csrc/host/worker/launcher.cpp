@@ -548,8 +548,9 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out)
       if (l.has_c) c = ViewOf(Resolve(l.c), l.c);
       if (l.norm_mode != 0 || !l.norm_stats_out.empty()) {
         // a LayerNormalization folded into the launch: see DeferLayerNorms in fusion.cpp
-        kernel::TensorView d, c1, c2, dst = out;
+        kernel::TensorView d, e, c1, c2, dst = out;
         if (l.has_skip) d = ViewOf(Resolve(l.d), l.d);
+        if (l.has_skip2) e = ViewOf(Resolve(l.e), l.e);
         if (!l.view_strides.empty()) {
           dst = kernel::TensorView(out.t.base, steps_[l.members[0]].out.meta);
           for (size_t k = 0; k < l.view_strides.size(); ++k) dst.t.strides[k] = l.view_strides[k];
@@ -578,6 +579,7 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out)
           }
         }
         if (!l.norm_stats_out.empty()) norm.stats_out = static_cast<float *>(privates_.at(l.norm_stats_out).device);
+        if (l.has_skip2) norm.addend2 = &e.t;
         const fl_tensor *rhs_p = &b.t, *dst_p = &dst.t;
         rc = fluidml_hip_matmul_chain_group_norm(1, &a.t, &rhs_p, &bias, col_sum != nullptr ? &col_sum : nullptr, &dst_p, l.n_inner,
                                                  &l.stride_outer, &l.chain, l.has_skip ? &d.t : nullptr, &norm, contract_flags,
@@ -830,8 +832,11 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out)
   }
   if (rc != 0) {
     ctx.Note(rc, LaunchKindName(l.kind));
-    throw std::runtime_error(std::string("launching fused ") + LaunchKindName(l.kind) + " ending at node '" +
-                             steps_[l.members.back()].node->GetName() + "': " + fluidml_hip_error_string(rc));
+    std::string what = std::string("launching fused ") + LaunchKindName(l.kind) + " of " + std::to_string(l.members.size()) +
+                       " steps ending at node '" + steps_[l.members.back()].node->GetName() + "'";
+    if (l.norm_mode != 0) what += " (deferred LayerNormalization, form " + std::to_string(l.norm_mode) + ")";
+    if (!l.norm_stats_out.empty()) what += " (writes row statistics)";
+    throw std::runtime_error(what + ": " + fluidml_hip_error_string(rc));
   }
 }
 

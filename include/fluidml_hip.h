@@ -446,6 +446,7 @@ typedef struct fl_norm_fusion {
   const fl_tensor *scale; /* FL_NORM_ADDEND: rank-1 [N] */
   const fl_tensor *shift; /* FL_NORM_ADDEND: rank-1 [N] */
   float *stats_out;       /* NULL: none */
+  const fl_tensor *addend2; /* NULL: none; a second tensor with the strides of out[0], added (plain) after `addend` */
 } fl_norm_fusion;
 /* fluidml_hip_matmul_chain_group (count 1..4; count == 1 is a single chain) with such a normalisation folded in.
  * `col_sum[i]`: rank-1 [N] per member, FL_NORM_LHS only (else NULL).  `addend`: a tensor with the strides of out[0]

@@ -1310,6 +1310,9 @@ def test_matmul_with_deferred_layer_norm(device, M, H, K0, N1):
     ok.binary_f32(ok.BOP_ADD, ok.View(b0), t, t1)
     ok.binary_f32(ok.BOP_ADD, t1, ok.View(x), s_ref)
     ok.layer_norm(s_ref, ok.View(gamma), ok.View(beta), h_ref, 2, eps)
+    x2 = rand(rng, (1, M, H), -1, 1)
+    s3_ref = V((1, M, H))
+    ok.binary_f32(ok.BOP_ADD, s_ref, ok.View(x2), s3_ref)
     z_ref = []
     for w, b in zip(w1, b1):
         z0, z = V((1, M, N1)), V((1, M, N1))
@@ -1338,7 +1341,7 @@ def test_matmul_with_deferred_layer_norm(device, M, H, K0, N1):
             want[:, j, 1] = ((run - run.mean(axis=1, keepdims=True)) ** 2).sum(axis=1)
         return want
 
-    da0, dw0, db0, dx = dev(a0), dev(w0), dev(b0), dev(x)
+    da0, dw0, db0, dx, dx2 = dev(a0), dev(w0), dev(b0), dev(x), dev(x2)
     dgamma, dbeta = dev(gamma), dev(beta)
     # what a caller folds at compile time: scale into the weights, their column sums, shift . W + bias
     dw1 = [dev(gamma[:, None] * w) for w in w1]
@@ -1364,6 +1367,20 @@ def test_matmul_with_deferred_layer_norm(device, M, H, K0, N1):
         want_stats = partial_stats(s_got[0])
         assert np.allclose(got_stats[..., 0], want_stats[..., 0], rtol=1e-5, atol=1e-6), "partial means"
         assert np.allclose(got_stats[..., 1], want_stats[..., 1], rtol=1e-4, atol=1e-5), "partial sums of squared deviations"
+
+        # the same producer with a second plain addend (a parallel residual: x + attention + mlp)
+        ds3 = DeviceView(ok.View.empty((1, M, H), np.float32, None, fill=3), device)
+        stats3 = torch.full((M, parts, 2), 7.0, device=device)
+        norm = cabi.FlNormFusion()
+        norm.deferred, norm.stats_out, norm.addend2 = cabi.FL_NORM_NONE, stats3.data_ptr(), ctypes.pointer(dx2.tensor)
+        announce("deferred layer norm: producer with two addends", (M, H, K0), "tile", tile)
+        rc = cabi.lib.fluidml_hip_matmul_chain_group_norm(1, da0.ref(), one(dw0), one(db0), None, one(ds3), 0, None, None, dx.ref(),
+                                                          ctypes.byref(norm), flags, None)
+        assert rc == 0, cabi.error_string(rc)
+        assert_close(ds3.logical(), s3_ref.logical(), what=f"residual sum of two addends, tile {tile}")
+        want3 = partial_stats(ds3.logical()[0])
+        got3 = stats3.cpu().numpy().astype(np.float64)
+        assert np.allclose(got3[..., 0], want3[..., 0], rtol=1e-5, atol=1e-6) and np.allclose(got3[..., 1], want3[..., 1], rtol=1e-4, atol=1e-5)
 
         douts = [DeviceView(ok.View.empty((1, M, N1), np.float32, None, fill=3), device) for _ in range(2)]
         norm = cabi.FlNormFusion()

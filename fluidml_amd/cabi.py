@@ -27,6 +27,7 @@ FL_REF_LN_STALE_SCRATCH = 1 << 2
 FL_REF_GEMM_SWAPPED_SCALARS = 1 << 3
 FL_REF_GATHER_RAW_AXIS = 1 << 4
 FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
+FL_REF_CONSTANT_GATHERED = 1 << 6
 FL_CONTRACT_BF16 = 1 << 0
 FL_CONTRACT_ADDEND_IS_FACTOR = 1 << 1
 FL_CONTRACT_SHIFT = 16

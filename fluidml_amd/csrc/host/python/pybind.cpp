@@ -454,6 +454,15 @@ PYBIND11_MODULE(fluidml, m) {
       },
       py::arg("onnx_path"), py::arg("node"), py::arg("lhs_layout"), py::arg("rhs_layout"), py::arg("out_layout"),
       "ContractionTable key of a MatMul / Gemm node's standalone kernel under the given layouts");
+  m.def(
+      "_pack_constant_f32",
+      [](std::vector<float64_t> values, std::vector<int64_t> shape, const std::vector<size_t> &layout, bool gathered) {
+        const Tensor t(Type::kFloat32, std::move(shape), std::move(values));
+        const std::vector<uint8_t> bytes = t.Pack(layout, gathered);
+        return py::bytes(reinterpret_cast<const char *>(bytes.data()), bytes.size());
+      },
+      py::arg("values"), py::arg("shape"), py::arg("layout"), py::arg("gathered") = false,
+      "the bytes uploaded for a float32 constant stored with `layout` (gathered: FL_REF_CONSTANT_GATHERED)");
   m.def("_gen_all_orders", &utils::GenAllOrders);
   m.def("_gen_all_indices_in_order", &utils::GenAllIndicesInOrder);
   m.def("_gen_physical_shape", &utils::GenPhysicalShape);

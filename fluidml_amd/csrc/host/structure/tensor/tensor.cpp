@@ -59,13 +59,17 @@ bool operator!=(const Tensor &lhs, const Tensor &rhs) { return !(lhs == rhs); }
 namespace {
 template <typename T>
 void PackAs(const std::vector<float64_t> &values, const std::vector<int64_t> &shape,
-            const std::vector<int64_t> &strides, uint8_t *dst) {
+            const std::vector<int64_t> &strides, bool gathered, uint8_t *dst) {
   T *out = reinterpret_cast<T *>(dst);
   const size_t rank = shape.size();
   std::vector<int64_t> index(rank, 0);
   int64_t offset = 0;
   for (size_t n = 0; n < values.size(); ++n) {
-    out[offset] = static_cast<T>(values[n]);
+    if (gathered) {
+      out[n] = static_cast<T>(values[static_cast<size_t>(offset)]);
+    } else {
+      out[offset] = static_cast<T>(values[n]);
+    }
     for (size_t d = rank; d-- > 0;) {
       offset += strides[d];
       if (++index[d] < shape[d]) break;
@@ -76,16 +80,16 @@ void PackAs(const std::vector<float64_t> &values, const std::vector<int64_t> &sh
 }
 }  // namespace
 
-std::vector<uint8_t> Tensor::Pack(const std::vector<size_t> &layout) const {
+std::vector<uint8_t> Tensor::Pack(const std::vector<size_t> &layout, bool gathered) const {
   const std::vector<int64_t> &shape = meta_.GetShape();
   const std::vector<int64_t> strides = utils::GenStrides(shape, layout);
   std::vector<uint8_t> bytes(meta_.GetSize());
   switch (meta_.GetType()) {
-    case Type::kBool: PackAs<uint8_t>(*data_, shape, strides, bytes.data()); break;
-    case Type::kInt32: PackAs<int32_t>(*data_, shape, strides, bytes.data()); break;
-    case Type::kInt64: PackAs<int64_t>(*data_, shape, strides, bytes.data()); break;
-    case Type::kFloat32: PackAs<float32_t>(*data_, shape, strides, bytes.data()); break;
-    case Type::kFloat64: PackAs<float64_t>(*data_, shape, strides, bytes.data()); break;
+    case Type::kBool: PackAs<uint8_t>(*data_, shape, strides, gathered, bytes.data()); break;
+    case Type::kInt32: PackAs<int32_t>(*data_, shape, strides, gathered, bytes.data()); break;
+    case Type::kInt64: PackAs<int64_t>(*data_, shape, strides, gathered, bytes.data()); break;
+    case Type::kFloat32: PackAs<float32_t>(*data_, shape, strides, gathered, bytes.data()); break;
+    case Type::kFloat64: PackAs<float64_t>(*data_, shape, strides, gathered, bytes.data()); break;
     default: throw std::invalid_argument("Tensor::Pack: unsupported element type");
   }
   return bytes;

@@ -31,8 +31,12 @@ class Tensor {
 
   // Dense bytes of the tensor in its element type, with `layout` applied:
   // element (i0,..) of the logical tensor lands at utils::GenStrides(shape,
-  // layout). This is what gets uploaded to HBM for a constant.
-  std::vector<uint8_t> Pack(const std::vector<size_t> &layout) const;
+  // layout). This is what gets uploaded to HBM for a constant.  `gathered`
+  // (FL_REF_CONSTANT_GATHERED): the reference's form instead -- byte n in
+  // row-major order takes the value found at the strided position of element
+  // n (reference src/worker/builder.cpp:290-297), the same only for layouts
+  // whose strided numbering is its own inverse.
+  std::vector<uint8_t> Pack(const std::vector<size_t> &layout, bool gathered = false) const;
 
  private:
   size_t Linear(const std::vector<size_t> &indices) const;

@@ -163,7 +163,7 @@ void LaunchPlan::Materialize() {
     for (void *&e : region_events_) Check(fluidml_hip_event_create(&e), "creating a fork/join event");
   }
   for (auto &kv : constants_) {
-    const std::vector<uint8_t> bytes = kv.second.tensor.Pack(kv.second.layout);
+    const std::vector<uint8_t> bytes = kv.second.tensor.Pack(kv.second.layout, (flags_ & FL_REF_CONSTANT_GATHERED) != 0);
     Check(fluidml_hip_upload_constant(bytes.data(), bytes.size(), &kv.second.device), "uploading a constant region");
   }
   for (auto *slots : {&privates_, &interfaces_}) {

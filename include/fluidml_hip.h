@@ -86,7 +86,11 @@ enum fl_ref_flags {
   /* Pad copies the input into the interior and never writes the border, which
    * keeps whatever the arena held (reference pad.cpp:33-51 writes through a
    * subview only); without the flag the border is written as zero. */
-  FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5
+  FL_REF_PAD_BORDER_UNWRITTEN = 1 << 5,
+  /* Host side only (no kernel reads it): a constant tensor whose layout is not the default one is written as
+   * data[row-major position of i] = values[strided position of i] and then read through those same strides (reference
+   * src/worker/builder.cpp:290-297, :311-318); without the flag the element lands at its strided position. */
+  FL_REF_CONSTANT_GATHERED = 1 << 6
 };
 
 /* Options of the contraction entry points (MatMul, Gemm, Conv with group 1).  The fused

@@ -64,6 +64,20 @@ def layout_strides(shape, layout):
     return [phys[j] for j in layout]
 
 
+def reference_constant(logical: np.ndarray, layout):
+    """A constant tensor as the reference stores it and as its kernels then read it, for a layout other than the
+    default one (reference src/worker/builder.cpp:279-297 for float32, :306-318 for int64): the global's dense data
+    is written in row-major order of the logical indices, entry n taking buffer[GenIndex(indices_n, strides)], and the
+    kernels address the global through those same strides.  Returns (data as stored, tensor as read)."""
+    logical = np.asarray(logical)
+    shape = list(logical.shape)
+    strides = np.asarray(layout_strides(shape, layout), dtype=np.int64)
+    indices = np.indices(shape).reshape(len(shape), -1)  # column n = the n-th index tuple in row-major order
+    strided = (indices * strides[:, None]).sum(axis=0)
+    stored = logical.reshape(-1)[strided]
+    return stored, stored[strided].reshape(shape)
+
+
 class View:
     """A logical tensor stored in host memory with a layout permutation
     (layout[i] = physical position of logical dim i)."""

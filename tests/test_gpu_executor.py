@@ -195,3 +195,43 @@ def test_compiler_cli_invoke(device, tiny_bert, tmp_path, capsys):
     assert summary["mode"] == "dp_greedy" and len(summary["invoke_ns"]) == 3
     assert all(ns > 0 for ns in summary["invoke_ns"])
     assert (tmp_path / "dp.json").stat().st_size > 0
+
+
+def test_reference_constant_relayout_switch(device, tmp_path, monkeypatch):
+    """FL_REF_CONSTANT_GATHERED (bit 6 of FLUIDML_REF_QUIRKS): under the DP executor a constant stored with a layout
+    other than the default is written the reference's way (src/worker/builder.cpp:290-297) and so reads back permuted
+    unless the layout's numbering is its own inverse.  The graph's MatMul weight [6, 10] ends up stored transposed
+    under constant costs: with the switch the result is the oracle's on the permuted weight, without it the oracle's
+    on the weight itself."""
+    from oracle import kernels as ok
+
+    fluidml, models = _mods()
+    rng = np.random.default_rng(31)
+    weight = rng.uniform(-1, 1, size=(6, 10)).astype(np.float32)
+    feeds = {"x": rng.uniform(-1, 1, size=(1, 4, 6)).astype(np.float32)}
+
+    def net_with(w):
+        g = models.Net("constant_relayout", 1)
+        x = g.input("x", np.float32, (1, 4, 6))
+        g.output(g.unary("Tanh", g.matmul(g.relu(x), g.const(w))))
+        return g
+
+    net = net_with(weight)
+    path = net.save(str(tmp_path / "net.onnx"))
+    monkeypatch.setenv("FLUIDML_DP_COST", "constant")
+    results = {}
+    for quirks in ("0", "64"):
+        monkeypatch.setenv("FLUIDML_REF_QUIRKS", quirks)
+        announce("constant re-layout, FLUIDML_REF_QUIRKS =", quirks)
+        ex = fluidml.Executor.make_dp_greedy("relayout" + quirks)
+        ex.compile(path)
+        layouts = [op["layout"] for s in ex.plan()["steps"] for op in s["inputs"] if op["space"] == "constant" and list(op["shape"]) == [6, 10]]
+        assert layouts == [[1, 0]], layouts
+        (results[quirks],) = _invoke(ex, net, feeds).values()
+    (name,) = [v.name for v in net.outputs]
+    assert_close(results["0"], graph_runner.run_graph(net, feeds)[name], what="constant stored with a layout, ONNX semantics")
+    permuted = ok.reference_constant(weight, [1, 0])[1]
+    assert not np.array_equal(permuted, weight)
+    want = graph_runner.run_graph(net_with(permuted), feeds)[name]
+    assert_close(results["64"], want, what="constant stored the reference's way")
+    assert not np.allclose(results["64"], results["0"], rtol=1e-3, atol=1e-4)

@@ -56,6 +56,24 @@ def test_gen_strides(fluidml):
         assert seen == set(range(int(np.prod(phys))))
 
 
+def test_constant_bytes_for_a_layout(fluidml):
+    """Tensor::Pack, the bytes uploaded for a constant: element i at its strided position; with
+    FL_REF_CONSTANT_GATHERED the reference's form (builder.cpp:290-297), against the oracle's restatement."""
+    import numpy as np
+
+    from oracle import kernels as ok
+
+    rng = np.random.default_rng(12)
+    for shape in [(3, 5), (2, 3, 4), (7,)]:
+        logical = rng.uniform(-1, 1, size=shape).astype(np.float32)
+        for layout in itertools.permutations(range(len(shape))):
+            plain = np.frombuffer(fluidml._pack_constant_f32(logical.reshape(-1).tolist(), list(shape), list(layout)), dtype=np.float32)
+            view = ok.View(logical, list(layout))
+            assert np.array_equal(plain, view.physical.reshape(-1)), (shape, layout)
+            got = np.frombuffer(fluidml._pack_constant_f32(logical.reshape(-1).tolist(), list(shape), list(layout), True), dtype=np.float32)
+            assert np.array_equal(got, ok.reference_constant(logical, list(layout))[0]), (shape, layout)
+
+
 def test_broadcast_shapes(fluidml):
     assert fluidml._broadcast_shape([1, 1, 3], [2, 3]) == [1, 2, 3]  # meta_test.cpp:6-15
     assert fluidml._broadcast_matmul_shape([2, 1, 3], [3, 2]) == [2, 1, 2]  # meta_test.cpp:17-26

@@ -344,3 +344,31 @@ def test_conv(case):
         ok.conv(ok.View(x), ok.View(w), ok.View(bias) if with_bias else None, ho, pads, strides, dilations, group, flags)
         lit = want_unit[crop] + (bias[1] if with_bias else 0.0)
         close(ho.logical(), lit, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("shape", [(3, 5), (4, 4), (2, 3, 4), (3, 3, 3)], ids=str)
+def test_reference_constant_relayout(shape):
+    """The reference's re-layout of constants (builder.cpp:279-297), pinned by the loop the cited lines spell out,
+    written index by index, and by what the numbering implies: the default layout and every layout whose strided
+    numbering is its own inverse (a square matrix stored transposed) read back unchanged; a non-square matrix stored
+    transposed does not."""
+    import itertools
+
+    rng = rng_for("reference constant", shape)
+    logical = rand(rng, shape)
+    for layout in all_layouts(len(shape)):
+        strides = ok.layout_strides(list(shape), layout)
+        stored, as_read = ok.reference_constant(logical, layout)
+        buffer = logical.reshape(-1)
+        data = []
+        for indices in itertools.product(*[range(n) for n in shape]):  # GenAllIndicesInOrder
+            data.append(buffer[sum(i * s for i, s in zip(indices, strides))])  # data.push_back(buffer[GenIndex(..)])
+        assert np.array_equal(stored, np.asarray(data, dtype=np.float32))
+        for indices in itertools.product(*[range(n) for n in shape]):
+            assert as_read[indices] == data[sum(i * s for i, s in zip(indices, strides))]
+        if list(layout) == sorted(layout):
+            assert np.array_equal(as_read, logical)
+    if shape == (4, 4):
+        assert np.array_equal(ok.reference_constant(logical, [1, 0])[1], logical)
+    if shape == (3, 5):
+        assert not np.array_equal(ok.reference_constant(logical, [1, 0])[1], logical)

@@ -357,6 +357,9 @@ SCHEDULE_NETS = {
     "convbert_base_full": (lambda m: m.convbert_base(), {"MatMulChain", "AddLayerNormalization"},
                            {"SoftmaxMatVec", "Attention", "PadViewCopy", "Placed", "MatMulGroup"}),
     "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), {"MatMulChain", "Attention", "View", "RotaryPair"}),
+    # full size (vocabulary cut: the projection's weights play no part in the plan): the parallel-residual blocks with
+    # both LayerNormalizations of a layer deferred into their readers, side by side with the plan's real reuse of bytes
+    "gpt_neox_full": (lambda m: m.gpt_neox(vocab=1024), {"MatMulChain", "Attention", "View", "RotaryPair"}),
     # without the rotary launch its steps go through the general mechanisms: views, Concat2 inputs written in place
     "gpt_neox_no_rotary": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120),
                            {"MatMulChain", "Attention", "View", "CopyInto", "MulAdd"}),

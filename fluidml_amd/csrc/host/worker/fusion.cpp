@@ -1157,7 +1157,11 @@ class Scheduler {
     for (int attempt = 0; attempt < 2; ++attempt) {
       if (l.members.size() < 2) return std::nullopt;  // nothing fused
       l.out = steps_[l.members.back()].out;
-      if (Safe(l.members, {{i, l.a}, {i, l.b}}) && OutputDisjoint(l.out, {&l.a, &l.b})) {
+      // (a result the plan put over bytes of an operand -- dead by then in the serial order, still read by this
+      // launch -- moves to a buffer of its own once the sweep is over)
+      const bool disjoint = OutputDisjoint(l.out, {&l.a, &l.b});
+      if (Safe(l.members, {{i, l.a}, {i, l.b}}) && (disjoint || Movable(l.out))) {
+        if (!disjoint) pending_moves_.push_back(l.out.name);
         l.bytes = l.has_c ? Bytes({&l.a, &l.b, &l.c, &l.out}) : Bytes({&l.a, &l.b, &l.out});
         l.bytes += static_cast<double>(steps_[i].kernel->GetConstantBytes());
         l.flops = Flops(l.members);

@@ -370,6 +370,13 @@ class Scheduler {
     const auto p = producer_.find(op.name);
     return p != producer_.end() && SameTensor(steps_[p->second].out, op);
   }
+  // the tensor whose bytes `op` addresses: itself, or what the elided view(s) it is seen through look into
+  std::optional<Operand> Underlying(const Operand &op) const {
+    if (!op.viewed) return op;
+    const auto p = producer_.find(op.name);
+    if (p == producer_.end() || steps_[p->second].out.viewed || steps_[p->second].out.space != op.space) return std::nullopt;
+    return steps_[p->second].out;
+  }
   void MoveOut(const std::string &name, std::initializer_list<std::vector<Launch> *> lists) {
     for (size_t i = 0; i < steps_.size(); ++i) {
       Step &st = steps_[i];
@@ -675,8 +682,9 @@ class Scheduler {
           apart.space = Operand::Space::Private;
           const Operand source = steps_[i].in0;
           steps_[j].in0 = saved;
-          if (!Movable(source) || !readers_can_see(i, produced, apart, l)) continue;
-          MoveOut(source.name, {fused});
+          const auto root = Underlying(source);
+          if (!root || !Movable(*root) || !readers_can_see(i, produced, apart, l)) continue;
+          MoveOut(root->name, {fused});
           list_writes();
           --i;  // once more, from the top, with the source where nothing else lives
           continue;
@@ -701,8 +709,10 @@ class Scheduler {
         Operand apart = seen;
         apart.space = Operand::Space::Private;
         const Operand source = steps_[i].in0;
-        if (!Movable(source) || !readers_can_see(i, produced, apart, nullptr)) continue;
-        MoveOut(source.name, {fused});
+        // (the source may itself be seen through an elided view: what moves is the tensor underneath)
+        const auto root = Underlying(source);
+        if (!root || !Movable(*root) || !readers_can_see(i, produced, apart, nullptr)) continue;
+        MoveOut(root->name, {fused});
         list_writes();
         --i;
         continue;
@@ -877,46 +887,59 @@ class Scheduler {
         }
         const size_t from = issued[*producer];
         if (from >= c) continue;
-        // nothing else may touch the output's bytes from the producer's launch up to the Concat2
-        const Operand target = ConcatPart(c, side);
-        bool ok = true;
+        Operand target = ConcatPart(c, side);
         // a launch that writes through folded views: its logical output's strides inside the part
         std::optional<ViewTracker::View> into;
         if (l != nullptr && !l->view_strides.empty()) {
           into = ViewInto(*l, target.view_strides);
           if (!into || l->has_skip) continue;
         }
-        for (size_t q = 0; q < steps_.size() && ok; ++q) {
-          if (q == c || elided_[q]) continue;
-          if (l != nullptr ? owner[q] == l : q == *producer) continue;
-          const bool in_range = (q >= from && q <= c) || (issued[q] >= from && issued[q] <= c);
-          if (!in_range) continue;
-          const Step &st = steps_[q];
-          // the other input's producer may already write its own part of the same output
-          const bool other_part = st.out.viewed && SameTensor(st.out, cat.out) && placed_[c] != 0;
-          // (intermediates of a fused launch are neither written nor read)
-          if (!other_part && !silent_[q] && Alias(st.out, target)) ok = false;
-          if ((really_read(st.in0) && Alias(st.in0, target)) ||
-              (st.node->IsDoubleInputs() && really_read(st.in1) && Alias(st.in1, target))) ok = false;
-          if (st.has_buffer && target.space == Operand::Space::Arena && st.buffer_offset < target.offset + target.Extent() &&
-              target.offset < st.buffer_offset + st.buffer_bytes) {
-            ok = false;
+        auto clear_for = [&](const Operand &target) {
+          bool ok = true;
+          for (size_t q = 0; q < steps_.size() && ok; ++q) {
+            if (q == c || elided_[q]) continue;
+            if (l != nullptr ? owner[q] == l : q == *producer) continue;
+            const bool in_range = (q >= from && q <= c) || (issued[q] >= from && issued[q] <= c);
+            if (!in_range) continue;
+            const Step &st = steps_[q];
+            // the other input's producer may already write its own part of the same output
+            const bool other_part = st.out.viewed && SameTensor(st.out, cat.out) && placed_[c] != 0;
+            // (intermediates of a fused launch are neither written nor read)
+            if (!other_part && !silent_[q] && Alias(st.out, target)) ok = false;
+            if ((really_read(st.in0) && Alias(st.in0, target)) ||
+                (st.node->IsDoubleInputs() && really_read(st.in1) && Alias(st.in1, target))) ok = false;
+            if (st.has_buffer && target.space == Operand::Space::Arena && st.buffer_offset < target.offset + target.Extent() &&
+                target.offset < st.buffer_offset + st.buffer_bytes) {
+              ok = false;
+            }
           }
-        }
-        // the producer's own inputs must not lie under the bytes it now writes
-        for (size_t m : (l != nullptr ? l->members : std::vector<size_t>{*producer})) {
-          const Step &st = steps_[m];
-          if ((really_read(st.in0) && Alias(st.in0, target)) ||
-              (st.node->IsDoubleInputs() && really_read(st.in1) && Alias(st.in1, target))) {
-            ok = false;
+          // the producer's own inputs must not lie under the bytes it now writes
+          for (size_t m : (l != nullptr ? l->members : std::vector<size_t>{*producer})) {
+            const Step &st = steps_[m];
+            if ((really_read(st.in0) && Alias(st.in0, target)) ||
+                (st.node->IsDoubleInputs() && really_read(st.in1) && Alias(st.in1, target))) {
+              ok = false;
+            }
           }
-        }
-        if (l != nullptr) {
-          for (const Operand *op : {&l->a, &l->b, &l->c, &l->d, &l->e}) {
-            if (!op->name.empty() && Alias(*op, target)) ok = false;
+          if (l != nullptr) {
+            for (const Operand *op : {&l->a, &l->b, &l->c, &l->d, &l->e}) {
+              if (!op->name.empty() && Alias(*op, target)) ok = false;
+            }
           }
+          return ok;
+        };
+        // nothing else may touch the output's bytes from the producer's launch up to the Concat2; where the plan has
+        // other tenants there, the Concat2's output gets a buffer of its own outside the arena (a part already
+        // written in place moves with it: its checks held for the planned bytes and hold for bytes nobody shares)
+        if (!clear_for(target)) {
+          Operand apart = target;
+          apart.space = Operand::Space::Private;
+          apart.offset = 0;
+          apart.pool.clear();
+          if (!Movable(cat.out) || !clear_for(apart)) continue;
+          MoveOut(cat.out.name, {fused});
+          target = ConcatPart(c, side);
         }
-        if (!ok) continue;
         steps_[*producer].out = target;
         if (l != nullptr) l->out = target;
         else rewired_[*producer] = true;
@@ -973,6 +996,21 @@ class Scheduler {
     }
     // the chain's own output must not overwrite an external input another member still needs: the fused kernel
     // reads and writes concurrently, the unfused sequence only tolerates that element for element
+    return true;
+  }
+
+  // Safe, or made safe by giving the operands whose bytes get other tenants in the window a buffer of their own
+  // outside the arena (`moves`: their names, to be moved once the caller has decided for the launch).
+  bool SafeWithMoves(const std::vector<size_t> &members, const std::vector<std::pair<size_t, Operand>> &external,
+                     std::vector<std::string> *moves) const {
+    std::vector<std::string> wanted;
+    for (const auto &e : external) {
+      if (Safe(members, {e})) continue;
+      const auto root = Underlying(e.second);
+      if (!root || !Movable(*root)) return false;
+      wanted.push_back(root->name);
+    }
+    moves->insert(moves->end(), wanted.begin(), wanted.end());
     return true;
   }
 
@@ -1160,8 +1198,10 @@ class Scheduler {
       // (a result the plan put over bytes of an operand -- dead by then in the serial order, still read by this
       // launch -- moves to a buffer of its own once the sweep is over)
       const bool disjoint = OutputDisjoint(l.out, {&l.a, &l.b});
-      if (Safe(l.members, {{i, l.a}, {i, l.b}}) && (disjoint || Movable(l.out))) {
-        if (!disjoint) pending_moves_.push_back(l.out.name);
+      std::vector<std::string> moves;
+      if ((disjoint || Movable(l.out)) && SafeWithMoves(l.members, {{i, l.a}, {i, l.b}}, &moves)) {
+        if (!disjoint) moves.push_back(l.out.name);
+        pending_moves_.insert(pending_moves_.end(), moves.begin(), moves.end());
         l.bytes = l.has_c ? Bytes({&l.a, &l.b, &l.c, &l.out}) : Bytes({&l.a, &l.b, &l.out});
         l.bytes += static_cast<double>(steps_[i].kernel->GetConstantBytes());
         l.flops = Flops(l.members);
@@ -1206,8 +1246,16 @@ class Scheduler {
         external.push_back({adds[k], tensors[k]});
       }
       l.out = steps_[l.members.back()].out;
-      for (size_t k = 0; k < n; ++k) ok = ok && tensors[k].layout == l.out.layout && !Alias(l.out, tensors[k]);
-      if (!ok || !Safe(l.members, external) || !OutputDisjoint(l.out, {&l.a, &l.b})) continue;
+      bool clash = !OutputDisjoint(l.out, {&l.a, &l.b});
+      for (size_t k = 0; k < n; ++k) {
+        ok = ok && tensors[k].layout == l.out.layout;
+        clash = clash || Alias(l.out, tensors[k]);
+      }
+      std::vector<std::string> moves;
+      if (!ok || (clash && !Movable(l.out)) || !SafeWithMoves(l.members, external, &moves)) continue;
+      // (the plan put the sum over bytes of an operand the launch still reads: the sum moves out of the arena)
+      if (clash) moves.push_back(l.out.name);
+      pending_moves_.insert(pending_moves_.end(), moves.begin(), moves.end());
       l.d = tensors[0];
       l.has_skip = true;
       if (n == 2) {
@@ -1392,13 +1440,14 @@ class Scheduler {
       l.out = steps_[l.members.back()].out;
       const Operand planned_out = l.out;
       if (with_skip && transposed) l.out = swapped(l.out);
-      if (!Safe(l.members, external)) continue;
-      if (!OutputDisjoint(l.out, {&l.a, &l.b}) || (with_gate && Alias(l.out, l.c)) || (with_skip && Alias(l.out, l.d))) {
-        // the plan reuses bytes of an operand for the result (dead by then in the serial order, still read by this
-        // launch): the result moves to a buffer of its own once the sweep is over
-        if (!Movable(planned_out)) continue;
-        pending_moves_.push_back(planned_out.name);
-      }
+      std::vector<std::string> moves;
+      const bool clash = !OutputDisjoint(l.out, {&l.a, &l.b}) || (with_gate && Alias(l.out, l.c)) || (with_skip && Alias(l.out, l.d));
+      // the plan reuses bytes of an operand for the result (dead by then in the serial order, still read by this
+      // launch): the result moves to a buffer of its own once the sweep is over; so does an operand whose bytes get
+      // another tenant before the launch, which now reads it later than planned, has run
+      if ((clash && !Movable(planned_out)) || !SafeWithMoves(l.members, external, &moves)) continue;
+      if (clash) moves.push_back(planned_out.name);
+      pending_moves_.insert(pending_moves_.end(), moves.begin(), moves.end());
       l.bytes = Bytes({&l.a, &l.b, &l.out}) + static_cast<double>(steps_[i].kernel->GetConstantBytes());
       if (with_gate) l.bytes += static_cast<double>(l.c.meta.GetSize());
       if (with_skip) l.bytes += static_cast<double>(l.d.meta.GetSize());

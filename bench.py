@@ -396,8 +396,8 @@ def main():
                           "mean_abs_err_vs_fp32": float(err.mean()),
                           "note": "operands of the MatMul, Gemm and non-depthwise Conv launches that run on the matrix cores "
                                   "(3x3 Conv on the staged-patch kernel included) rounded to bf16 (nearest even), fp32 accumulation; "
-                                  "the weight-streaming Gemm kernels, depthwise Conv and the launches that carry a "
-                                  "deferred LayerNormalization stay fp32"}
+                                  "the weight-streaming Gemm kernels, depthwise Conv and pointwise Conv with a gate or skip "
+                                  "operand stay fp32"}
     if not args.no_cpu_baseline:
         if args.config == "bert_base":
             result["cpu_baseline"] = cpu_baseline(args.layers, min(args.cpu_sample_layers, args.layers), args.seq)

@@ -1447,9 +1447,11 @@ int LaunchBySize(const MatmulArgs &p, uint32_t n_batch, float *C, const float *A
     // where there are enough of them, 128x128 tiles (2x2 waves with 2x2 accumulators each) halve that traffic, and four
     // chunks on their way in registers keep it coming (two: 4096^3 310 TFLOP/s, four: 445; [256,512]x[512,50304] 89 -> 57 us)
     const int64_t big_tiles = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + 127) / 128) * n_batch;
-    if (choice.tile == FL_TILE_RULE && big_tiles >= 256) tile = FL_TILE_128x128_STAGED;
+    // (two lanes merge the statistics of one of its 128 rows: deferred LayerNormalizations up to 512 wide)
+    const bool rows_fit = EXTRA != 1 || p.ln_mode == 0 || p.ln_width <= 512;
+    if (choice.tile == FL_TILE_RULE && big_tiles >= 256 && rows_fit) tile = FL_TILE_128x128_STAGED;
     if (tile == FL_TILE_128x128_STAGED) {
-      if (choice.splits > 1) return FL_ERR_UNSUPPORTED;
+      if (choice.splits > 1 || !rows_fit) return FL_ERR_UNSUPPORTED;
       return LaunchConfig<128, 128, 32, 2, 2, 1, LA, LB, VEC, 4, CONV, true, false, EXTRA>(p, n_batch, C, A, B, s, 0);
     }
   }
@@ -1645,10 +1647,10 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
     return FL_ERR_UNSUPPORTED;
   }
   if (norm != nullptr) {
-    // a LayerNormalization folded into this launch: one batch element, fp32, rows short enough for the lanes that
+    // a LayerNormalization folded into this launch: one batch element, rows short enough for the lanes that
     // merge a row's partial statistics (64x64 tile: 4 lanes x 8 partials x 32 columns)
     const int64_t real_batch = siblings != nullptr && siblings->count > 0 ? 1 : n_batch;
-    if (real_batch != 1 || bf16 || k_scale != nullptr) return FL_ERR_UNSUPPORTED;
+    if (real_batch != 1 || k_scale != nullptr) return FL_ERR_UNSUPPORTED;
     if (norm->deferred != FL_NORM_NONE) {
       if (norm->stats == nullptr || norm->width <= 0 || norm->width > 1024) return FL_ERR_UNSUPPORTED;
       p.ln_mode = norm->deferred;
@@ -1708,7 +1710,9 @@ int Contract(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *out, b
     else if (vec) rc = LaunchBySize<1, 0, 4, 0, false, E_>(p, nb, C, A, B, s, choice);         \
     else rc = LaunchBySize<1, 0, 1, 0, false, E_>(p, nb, C, A, B, s, choice);                  \
   } while (0)
+    // (bf16 operands with the epilogue operands: the common case of dense row-major operands only)
     if (k_scale != nullptr) FL_MM_EXTRA(2);
+    else if (bf16 && la == 0 && vec) rc = LaunchBySize<0, 0, 4, 0, true, 1>(p, nb, C, A, B, s, choice);
     else FL_MM_EXTRA(1);
 #undef FL_MM_EXTRA
     return rc != FL_OK ? rc : LaunchStatus();
@@ -1960,8 +1964,8 @@ int fluidml_hip_matmul_chain_add(const fl_tensor *lhs, const fl_tensor *rhs, con
     e[i] = static_cast<const float *>(t[i]->base);
   }
   // fp32 whatever the flags say: the extra operands exist in the fp32 instantiations only
-  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, 0, 0, nullptr, false, e[0], nullptr, 0,
-                      e[1], fl::ChoiceOf(flags));
+  return fl::Contract(lhs, rhs, out, false, false, 1.0f, 1.0f, bias, stream, chain, 0, 0, nullptr,
+                      (flags & FL_CONTRACT_BF16) != 0, e[0], nullptr, 0, e[1], fl::ChoiceOf(flags));
 }
 
 int fluidml_hip_matmul_chain_view(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out,
@@ -2041,7 +2045,8 @@ int fluidml_hip_matmul_chain_group_norm(int32_t count, const fl_tensor *lhs, con
     extra2 = static_cast<const float *>(second->base);
   }
   return fl::Contract(lhs, rhs[0], out[0], false, false, 1.0f, 1.0f, bias != nullptr ? bias[0] : nullptr, stream, chain,
-                      n_inner, stride_outer != nullptr ? stride_outer[0] : 0, count > 1 ? &sib : nullptr, false, extra, nullptr,
+                      n_inner, stride_outer != nullptr ? stride_outer[0] : 0, count > 1 ? &sib : nullptr,
+                      (flags & FL_CONTRACT_BF16) != 0, extra, nullptr,
                       0, extra2, fl::ChoiceOf(flags), norm, col_sum);
 }
 

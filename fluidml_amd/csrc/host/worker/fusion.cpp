@@ -2006,8 +2006,13 @@ class Scheduler {
           transposed = true;
         }
         auto finish = [&](Launch *x, size_t x_from) {
-          if (!Safe(x->members, {{x_from, x->a}, {m1, x->b}, {m2, x->c}})) return false;
-          if (!OutputDisjoint(x->out, {&x->a, &x->b, &x->c})) return false;
+          // (operands or a result the plan has other tenants for in the launch's window move out of the arena)
+          std::vector<std::string> moves;
+          const bool clash = !OutputDisjoint(x->out, {&x->a, &x->b, &x->c});
+          if (clash && !Movable(x->out)) return false;
+          if (!SafeWithMoves(x->members, {{x_from, x->a}, {m1, x->b}, {m2, x->c}}, &moves)) return false;
+          if (clash) moves.push_back(x->out.name);
+          pending_moves_.insert(pending_moves_.end(), moves.begin(), moves.end());
           x->bytes = Bytes({&x->a, &x->b, &x->c, &x->out});
           x->flops = 0;
           return true;

@@ -412,7 +412,8 @@ int fluidml_hip_matmul_chain(const fl_tensor *lhs, const fl_tensor *rhs, const f
 /* The same followed by one or two AddCommonKernel with tensors of the output's shape and strides (a residual
  * connection, or GPT-NeoX's parallel residual x + attention + mlp): out = (chain(lhs . rhs + bias) + addend) + addend2,
  * each sum rounded like the separate kernels' (reference matmul.cpp:28-59, add.cpp:75-137).  `addend2` may be NULL.
- * `rhs` must be unit-stride along its last dim; fp32 whatever `flags` say.  Otherwise FL_ERR_UNSUPPORTED. */
+ * `rhs` must be unit-stride along its last dim, otherwise FL_ERR_UNSUPPORTED.  FL_CONTRACT_BF16 is honoured for dense
+ * row-major operands with 16-byte aligned rows; other operands keep the launch in fp32. */
 int fluidml_hip_matmul_chain_add(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, const fl_ew_program *chain, const fl_tensor *addend, const fl_tensor *addend2, uint32_t flags, void *stream);
 /* The same, followed by Reshape / Transpose steps that only re-address the
  * result (reference reshape.cpp:18-64, transpose.cpp:19-48): `out` carries the
@@ -454,8 +455,10 @@ typedef struct fl_norm_fusion {
 } fl_norm_fusion;
 /* fluidml_hip_matmul_chain_group (count 1..4; count == 1 is a single chain) with such a normalisation folded in.
  * `col_sum[i]`: rank-1 [N] per member, FL_NORM_LHS only (else NULL).  `addend`: a tensor with the strides of out[0]
- * added after the chain (plain, or t of FL_NORM_ADDEND); count == 1 and n_inner == 0 only.  fp32 whatever `flags`
- * say about bf16; the tile configuration bits of `flags` apply. */
+ * added after the chain (plain, or t of FL_NORM_ADDEND); count == 1 and n_inner == 0 only.  FL_CONTRACT_BF16 rounds
+ * the two operands of the contraction (with FL_NORM_LHS: the un-normalised left operand and the pre-scaled weights);
+ * statistics, the epilogue's correction and the addends stay fp32.  The tile configuration bits of `flags` apply
+ * (FL_TILE_128x128_STAGED: deferred rows of at most 512 elements). */
 int fluidml_hip_matmul_chain_group_norm(int32_t count, const fl_tensor *lhs, const fl_tensor *const *rhs, const fl_tensor *const *bias, const fl_tensor *const *col_sum, const fl_tensor *const *out, int64_t n_inner, const int64_t *stride_outer, const fl_ew_program *chain, const fl_tensor *addend, const fl_norm_fusion *norm, uint32_t flags, void *stream);
 /* GemmConstantWeightsBiasKernel -> elementwise chain (reference gemm.cpp:39-182); `flags` = fl_contract_flags. */
 int fluidml_hip_gemm_chain(const fl_tensor *lhs, const fl_tensor *rhs, const fl_tensor *bias, const fl_tensor *out, double alpha, double beta, int32_t trans_a, int32_t trans_b, const fl_ew_program *chain, uint32_t flags, void *stream);

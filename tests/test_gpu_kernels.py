@@ -774,29 +774,33 @@ def test_matmul_chain_add(device):
         a, b = rand(rng, ashape, -1, 1), rand(rng, bshape, -0.05, 0.05)
         oshape = ashape[:-1] + (bshape[-1],)
         bias, r1, r2 = rand(rng, (bshape[-1],), -0.5, 0.5), rand(rng, oshape, -1, 1), rand(rng, oshape, -1, 1)
-        announce("matmul_chain_add", ashape, bshape, lo, two, with_chain)
-        t0, t1 = ok.View.empty(oshape), ok.View.empty(oshape)
-        ok.matmul(ok.View(a), ok.View(b), t0)
-        ok.binary_f32(ok.BOP_ADD, ok.View(bias), t0, t1)
-        if with_chain:
-            t = ok.View.empty(oshape)
-            ok.unary_f32(ok.OP_RELU, t1, t)
-            t1 = t
-        want = ok.View.empty(oshape)
-        ok.binary_f32(ok.BOP_ADD, ok.View(r1), t1, want)
-        if two:
-            t = ok.View.empty(oshape)
-            ok.binary_f32(ok.BOP_ADD, want, ok.View(r2), t)
-            want = t
-        h1, h2 = ok.View.empty(oshape, np.float32, lo), ok.View.empty(oshape, np.float32, lo)
-        h1.logical()[...] = r1
-        h2.logical()[...] = r2
-        da, db, dbias = DeviceView(ok.View(a), device), DeviceView(ok.View(b), device), DeviceView(ok.View(bias), device)
-        d1, d2 = DeviceView(h1, device), DeviceView(h2, device)
-        do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
-        cabi.call("matmul_chain_add", da.ref(), db.ref(), dbias.ref(), do.ref(), ctypes.byref(relu if with_chain else none),
-                  d1.ref(), d2.ref() if two else None, ctypes.c_uint32(0), None)
-        assert_close(do.logical(), want.logical(), what="matmul_chain_add")
+        # (second pass: the opt-in bf16 operands, against the oracle on the rounded operands)
+        # (rows of B that are not 16-byte aligned keep the launch in fp32 whatever the flag says)
+        rounds = bshape[-1] % 4 == 0
+        for flags, opa, opb in ((0, a, b), (cabi.FL_CONTRACT_BF16, _round_bf16(a) if rounds else a, _round_bf16(b) if rounds else b)):
+            announce("matmul_chain_add", ashape, bshape, lo, two, with_chain, "flags", flags)
+            t0, t1 = ok.View.empty(oshape), ok.View.empty(oshape)
+            ok.matmul(ok.View(opa), ok.View(opb), t0)
+            ok.binary_f32(ok.BOP_ADD, ok.View(bias), t0, t1)
+            if with_chain:
+                t = ok.View.empty(oshape)
+                ok.unary_f32(ok.OP_RELU, t1, t)
+                t1 = t
+            want = ok.View.empty(oshape)
+            ok.binary_f32(ok.BOP_ADD, ok.View(r1), t1, want)
+            if two:
+                t = ok.View.empty(oshape)
+                ok.binary_f32(ok.BOP_ADD, want, ok.View(r2), t)
+                want = t
+            h1, h2 = ok.View.empty(oshape, np.float32, lo), ok.View.empty(oshape, np.float32, lo)
+            h1.logical()[...] = r1
+            h2.logical()[...] = r2
+            da, db, dbias = DeviceView(ok.View(a), device), DeviceView(ok.View(b), device), DeviceView(ok.View(bias), device)
+            d1, d2 = DeviceView(h1, device), DeviceView(h2, device)
+            do = DeviceView(ok.View.empty(oshape, np.float32, lo, fill=7), device)
+            cabi.call("matmul_chain_add", da.ref(), db.ref(), dbias.ref(), do.ref(), ctypes.byref(relu if with_chain else none),
+                      d1.ref(), d2.ref() if two else None, ctypes.c_uint32(flags), None)
+            assert_close(do.logical(), want.logical(), what=f"matmul_chain_add, flags {flags}")
     # a right operand stored k-fastest is refused
     bt = DeviceView(ok.View(rand(rng, (40, 96)), [1, 0]), device)
     a = DeviceView(ok.View(rand(rng, (70, 40))), device)
@@ -1416,6 +1420,86 @@ def test_matmul_with_deferred_layer_norm(device, M, H, K0, N1):
         want2 = partial_stats(du.logical()[0])
         got2 = stats2.cpu().numpy().astype(np.float64)
         assert np.allclose(got2[..., 0], want2[..., 0], rtol=1e-5, atol=1e-6) and np.allclose(got2[..., 1], want2[..., 1], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("M,H,K0,N1", [(128, 256, 128, 384), (33, 768, 256, 768), (300, 512, 128, 4096)], ids=str)
+def test_matmul_with_deferred_layer_norm_bf16(device, M, H, K0, N1):
+    """The three forms of fluidml_hip_matmul_chain_group_norm with FL_CONTRACT_BF16: both operands of the contraction
+    are rounded to bf16 on their way into LDS (the un-normalised sum and the pre-scaled weights where the left operand
+    carries the deferred LayerNormalization), everything else -- accumulation, row statistics, the epilogue's
+    correction, the residual's normalisation -- stays fp32.  Expected values: the same formulas in float64 on the
+    rounded operands.  The rule's tile, the 64x64 tile and, where the rows fit its two lanes per row, the 128x128 one."""
+    import torch
+
+    cabi = _cabi()
+    rng = np.random.default_rng(M + H + 1)
+    eps = 1e-5
+    a0, w0, b0 = rand(rng, (1, M, K0), -1, 1), rand(rng, (K0, H), -0.3, 0.3), rand(rng, (H,), -0.5, 0.5)
+    x = rand(rng, (1, M, H), -2, 2) + 0.75
+    gamma, beta = rand(rng, (H,), 0.5, 1.5), rand(rng, (H,), -0.5, 0.5)
+    w1, b1 = rand(rng, (H, N1), -0.2, 0.2), rand(rng, (N1,), -0.5, 0.5)
+    a2, w2, b2 = rand(rng, (1, M, K0), -1, 1), rand(rng, (K0, H), -0.3, 0.3), rand(rng, (H,), -0.5, 0.5)
+    parts = (H + 31) // 32
+    ptr = ctypes.POINTER(cabi.FlTensor)
+    f64 = np.float64
+
+    def dev(arr):
+        return DeviceView(ok.View(np.ascontiguousarray(arr, dtype=np.float32)), device)
+
+    def one(v):
+        return (ptr * 1)(ctypes.pointer(v.tensor))
+
+    r = _round_bf16
+    s_want = (r(a0[0]).astype(f64) @ r(w0).astype(f64) + b0 + x[0]).astype(np.float32)
+    da0, dw0, db0, dx = dev(a0), dev(w0), dev(b0), dev(x)
+    gw = (gamma[:, None] * w1).astype(np.float32)
+    dw1, dc1 = dev(gw), dev(gw.astype(f64).sum(axis=0))
+    dc2 = dev(beta.astype(f64) @ w1.astype(f64) + b1)
+    dgamma, dbeta, da2, dw2, db2 = dev(gamma), dev(beta), dev(a2), dev(w2), dev(b2)
+    for tile in (0, 2, 8):
+        flags = ctypes.c_uint32(cabi.FL_CONTRACT_BF16 | tile << 4)
+        ds = DeviceView(ok.View.empty((1, M, H), np.float32, None, fill=3), device)
+        stats = torch.full((M, parts, 2), 7.0, device=device)
+        norm = cabi.FlNormFusion()
+        norm.deferred, norm.stats_out = cabi.FL_NORM_NONE, stats.data_ptr()
+        announce("deferred layer norm, bf16 operands: producer", (M, H, K0), "tile", tile)
+        rc = cabi.lib.fluidml_hip_matmul_chain_group_norm(1, da0.ref(), one(dw0), one(db0), None, one(ds), 0, None, None, dx.ref(),
+                                                          ctypes.byref(norm), flags, None)
+        assert rc == 0, cabi.error_string(rc)
+        s_got = ds.logical()[0]
+        assert_close(s_got, s_want, what=f"bf16 residual sum, tile {tile}")
+        # row statistics of what was written
+        mean = s_got.astype(f64).mean(axis=1, keepdims=True)
+        rstd = 1.0 / np.sqrt(((s_got.astype(f64) - mean) ** 2).mean(axis=1, keepdims=True) + eps)
+
+        dz = DeviceView(ok.View.empty((1, M, N1), np.float32, None, fill=3), device)
+        norm = cabi.FlNormFusion()
+        norm.deferred, norm.width, norm.epsilon, norm.stats = cabi.FL_NORM_LHS, H, eps, stats.data_ptr()
+        announce("deferred layer norm, bf16 operands: normalised left operand", (M, H, N1), "tile", tile)
+        rc = cabi.lib.fluidml_hip_matmul_chain_group_norm(1, ds.ref(), one(dw1), one(dc2), one(dc1), one(dz), 0, None, None, None,
+                                                          ctypes.byref(norm), flags, None)
+        if tile == 8 and H > 512:
+            assert rc == cabi.FL_ERR_UNSUPPORTED  # two lanes per row merge at most 16 partials
+        else:
+            assert rc == 0, cabi.error_string(rc)
+            acc = r(s_got).astype(f64) @ r(gw).astype(f64)
+            z_want = rstd * (acc - mean * dc1.logical().astype(f64)) + dc2.logical().astype(f64)
+            np.testing.assert_allclose(dz.logical()[0], z_want, rtol=2e-4, atol=2e-4, err_msg=f"bf16 projection of the deferred LayerNorm, tile {tile}")
+
+        du = DeviceView(ok.View.empty((1, M, H), np.float32, None, fill=3), device)
+        norm = cabi.FlNormFusion()
+        norm.deferred, norm.width, norm.epsilon, norm.stats = cabi.FL_NORM_ADDEND, H, eps, stats.data_ptr()
+        norm.scale, norm.shift = ctypes.pointer(dgamma.tensor), ctypes.pointer(dbeta.tensor)
+        announce("deferred layer norm, bf16 operands: normalised residual", (M, K0, H), "tile", tile)
+        rc = cabi.lib.fluidml_hip_matmul_chain_group_norm(1, da2.ref(), one(dw2), one(db2), None, one(du), 0, None, None, ds.ref(),
+                                                          ctypes.byref(norm), flags, None)
+        if tile == 8 and H > 512:
+            assert rc == cabi.FL_ERR_UNSUPPORTED
+            continue
+        assert rc == 0, cabi.error_string(rc)
+        h = (s_got.astype(f64) - mean) * rstd * gamma + beta
+        u_want = r(a2[0]).astype(f64) @ r(w2).astype(f64) + b2 + h
+        np.testing.assert_allclose(du.logical()[0], u_want, rtol=1e-4, atol=1e-4, err_msg=f"bf16 contraction + deferred LayerNorm residual, tile {tile}")
 
 
 CONV_CASES = [

@@ -89,8 +89,22 @@ def run(repeats: int = 20, out=None) -> dict:
                                      ctypes.c_int64(1), bits, None),
                    2.0 * images * filters * size * size * channels * 9, bf16=True)
         del x, w, y
+    # what the matrix pipes deliver when a wave does nothing but issue dependent fp32 MFMAs, at the clock the
+    # device actually runs at: the ceiling of any contraction kernel here
+    loop = {}
+    for waves in (1, 2):
+        ns, ticks = ctypes.c_double(), ctypes.c_double()
+        count = 2048
+        cabi.call("mfma_rate", waves, count, ref(ns), ref(ticks))
+        simds = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
+        tflops = 4096.0 * count * waves * simds / (ns.value * 1e-9) / 1e12
+        loop[f"{waves}_per_simd"] = {"us": ns.value / 1e3, "shader_clock_ghz": ticks.value / ns.value,
+                                     "ticks_per_mfma": ticks.value / (count * waves), "TFLOP/s": tflops}
+        print(f"{waves} wave(s) per SIMD, {count} dependent v_mfma_f32_32x32x2_f32 each: {ns.value / 1e3:8.1f} us, shader clock "
+              f"{ticks.value / ns.value:.2f} GHz, {tflops:6.1f} TFLOP/s = {100 * tflops / FP32_MFMA_PEAK_TFLOPS:.1f} % of the published peak",
+              file=out, flush=True)
     return {"metric": "achieved fp32 MFMA throughput of the contraction kernel", "unit": "TFLOP/s",
-            "peak": FP32_MFMA_PEAK_TFLOPS, "repeats": repeats, "cases": rows}
+            "peak": FP32_MFMA_PEAK_TFLOPS, "repeats": repeats, "cases": rows, "mfma_only_loop": loop}
 
 
 if __name__ == "__main__":

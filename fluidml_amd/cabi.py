@@ -90,6 +90,7 @@ SIGNATURES = {
     "fluidml_hip_memcpy_d2h": [_vp, _vp, _sz, _vp],
     "fluidml_hip_memcpy_d2d": [_vp, _vp, _sz, _vp],
     "fluidml_hip_time_kernels": [_vp, _vp],
+    "fluidml_hip_mfma_rate": [ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)],
     "fluidml_hip_stream_create": [_P(_vp)],
     "fluidml_hip_stream_destroy": [_vp],
     "fluidml_hip_stream_synchronize": [_vp],

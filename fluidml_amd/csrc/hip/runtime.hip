@@ -5,6 +5,9 @@
 #include <mutex>
 #include <unordered_map>
 
+#include <algorithm>
+#include <vector>
+
 #include "fl_common.h"
 
 using namespace fl;
@@ -61,6 +64,25 @@ void DropStreamWorkspace(hipStream_t stream) {
 KernelTimer &ThreadKernelTimer() {
   static thread_local KernelTimer timer;
   return timer;
+}
+
+// What the matrix pipes deliver when nothing else is asked of them: every wave issues `count` dependent
+// v_mfma_f32_32x32x2_f32 (4096 flops each) and stamps the 100 MHz wall clock and the shader clock around them.
+typedef float RateAcc __attribute__((ext_vector_type(16)));
+__global__ __launch_bounds__(256) void MfmaRateKernel(int count, uint64_t *out) {
+  RateAcc acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+  const float a = static_cast<float>(threadIdx.x) * 0.001f, b = 1.0f;
+  const uint64_t w0 = wall_clock64(), c0 = clock64();
+  for (int i = 0; i < count; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+  asm volatile("" ::"v"(acc[0]));
+  const uint64_t w1 = wall_clock64(), c1 = clock64();
+  if (threadIdx.x % 64 == 0) {
+    const uint32_t w = blockIdx.x * 4 + threadIdx.x / 64;
+    out[2 * w] = w1 - w0;
+    out[2 * w + 1] = c1 - c0;
+  }
 }
 }  // namespace fl
 
@@ -252,6 +274,37 @@ int fluidml_hip_time_kernels(void *start, void *stop) {
   fl::KernelTimer &t = fl::ThreadKernelTimer();
   t.start = static_cast<hipEvent_t>(start);
   t.stop = static_cast<hipEvent_t>(stop);
+  return FL_OK;
+}
+
+int fluidml_hip_mfma_rate(int32_t waves_per_simd, int32_t count, double *ns, double *shader_ticks) {
+  if (ns == nullptr || shader_ticks == nullptr) return FL_ERR_NULL;
+  if (waves_per_simd < 1 || waves_per_simd > 2 || count < 1 || count > (1 << 20)) return FL_ERR_ATTR;
+  int dev = 0;
+  FL_HIP_CHECK(hipGetDevice(&dev));
+  hipDeviceProp_t prop;
+  FL_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+  const int groups = prop.multiProcessorCount * waves_per_simd;  // four waves each: one per SIMD of a compute unit
+  uint64_t *out = nullptr;
+  FL_HIP_CHECK(hipMalloc(&out, static_cast<size_t>(groups) * 4 * 2 * sizeof(uint64_t)));
+  std::vector<uint64_t> host(static_cast<size_t>(groups) * 8);
+  hipError_t err = hipSuccess;
+  for (int round = 0; round < 3 && err == hipSuccess; ++round) {  // (the last of three: clocks and caches settled)
+    hipLaunchKernelGGL(fl::MfmaRateKernel, dim3(groups), dim3(256), 0, nullptr, count, out);
+    err = hipDeviceSynchronize();
+  }
+  if (err == hipSuccess) err = hipMemcpy(host.data(), out, host.size() * sizeof(uint64_t), hipMemcpyDeviceToHost);
+  (void)hipFree(out);
+  if (err != hipSuccess) return static_cast<int>(err);
+  std::vector<uint64_t> wall, ticks;
+  for (size_t w = 0; w < host.size() / 2; ++w) {
+    wall.push_back(host[2 * w]);
+    ticks.push_back(host[2 * w + 1]);
+  }
+  std::nth_element(wall.begin(), wall.begin() + wall.size() / 2, wall.end());
+  std::nth_element(ticks.begin(), ticks.begin() + ticks.size() / 2, ticks.end());
+  *ns = static_cast<double>(wall[wall.size() / 2]) * 10.0;
+  *shader_ticks = static_cast<double>(ticks[ticks.size() / 2]);
   return FL_OK;
 }
 

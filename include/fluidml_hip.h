@@ -227,6 +227,12 @@ int fluidml_hip_event_elapsed_ns(void *start, void *stop, double *ns);
  * launches several kernels the events describe the last one.  Not for use
  * during launch-plan capture. */
 int fluidml_hip_time_kernels(void *start, void *stop);
+/* Measurement helper without a counterpart in the reference: `waves_per_simd` (1 or 2) waves on every SIMD of the
+ * current device each issue `count` dependent v_mfma_f32_32x32x2_f32 and nothing else.  `ns`: the median wave's
+ * duration on the 100 MHz wall clock; `shader_ticks`: the same interval in shader clock ticks (one such instruction
+ * occupies a SIMD's matrix pipe for 64 of them).  What a contraction kernel can reach at best on this device at the
+ * clock it actually runs at: 4096 * count flops per wave in `ns`.  Allocates and frees a small device buffer. */
+int fluidml_hip_mfma_rate(int32_t waves_per_simd, int32_t count, double *ns, double *shader_ticks);
 /* Launch-plan capture: the node sequence of one Invoke recorded once and
  * replayed (the counterpart of re-running `_mlir_ciface_<name>`,
  * reference runner.cpp:101-109). */

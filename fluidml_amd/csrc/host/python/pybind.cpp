@@ -94,12 +94,42 @@ py::dict StepsOf(worker::LaunchPlan &plan) {
     }
     // a launch that writes into a part of another tensor (an input of a Concat2 placed in its output)
     // (a launch that writes its own result through other strides -- a Transpose it absorbed -- is not meant)
-    if (l.kind != worker::Launch::Kind::View && l.kind != worker::Launch::Kind::Placed && l.out.viewed &&
+    auto padded = [&](const std::string &name) {  // the output of a Pad step (written in place by its input's producer)?
+      for (const worker::Step &st : plan.GetSteps()) {
+        if (st.out.name == name && !st.out.viewed) return st.node->GetKind() == flow::OpKind::Pad;
+      }
+      return false;
+    };
+    if (l.kind != worker::Launch::Kind::View && l.kind != worker::Launch::Kind::Placed && l.out.viewed && l.group.empty() &&
+        !padded(l.out.name) &&
         (l.members.empty() || l.kind == worker::Launch::Kind::CopyInto ||
          l.out.name != plan.GetSteps()[l.members.back()].out.name)) {
       py::dict into = OperandOf(l.out);
       into["bytes"] = l.out.Extent();
       d["writes_into"] = into;
+    }
+    // results written into the interior of another tensor's buffer (a zero Pad that does not run: the padded tensor
+    // lives outside the arena, its border is never written), per member of a group as well
+    {
+      py::list inside;
+      auto note = [&](const worker::Operand &out, size_t step) {
+        const worker::Step &producer = plan.GetSteps()[step];
+        if (!out.viewed || !padded(out.name) || l.kind == worker::Launch::Kind::CopyInto) return;
+        (void)producer;
+        py::dict w;
+        w["step"] = step;
+        py::dict into = OperandOf(out);
+        into["bytes"] = out.Extent();
+        into["view_offset"] = out.view_offset;
+        into["view_strides"] = out.view_strides;
+        w["into"] = into;
+        inside.append(w);
+      };
+      if (l.kind != worker::Launch::Kind::View && l.kind != worker::Launch::Kind::Placed) {
+        if (l.group.empty() && !l.members.empty()) note(l.out, l.members.back());
+        for (const worker::Launch &m : l.group) note(m.out, m.members.back());
+      }
+      d["writes_inside"] = inside;
     }
     for (const worker::Launch &m : l.group) written.push_back(m.members.back());
     d["written"] = written;

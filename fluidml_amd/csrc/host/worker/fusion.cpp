@@ -277,6 +277,7 @@ class Scheduler {
       GroupSiblings(&fused);
       silent_.clear();
     }
+    if (fuse) PlacePadInputs(&fused);
     if (fuse) ElideViews(&fused);
     if (fuse) RetryAttention(&fused);
     if (fuse) RetrySoftmaxMatVec(&fused);
@@ -830,6 +831,77 @@ class Scheduler {
     rewired_[c] = true;
     taken_[r] = true;
     filled_[r] = true;
+  }
+
+  // ---- Pad inputs written in place ------------------------------------------------------------------------
+  // A zero Pad whose input comes from a contraction launch and whose result is only looked at through views (the
+  // sliding windows of a span-based convolution: Pad -> Gather -> Transpose [-> Reshape], matched as one copy above):
+  // the padded tensor gets a buffer of its own outside the arena -- zero when it is created, and nothing ever writes
+  // its border -- the contraction writes its result straight into the interior, the Pad does not run, and the view
+  // steps behind it are left to the view elision, whose readers then address the windows inside the padded buffer.
+  void PlacePadInputs(std::vector<Launch> *fused) {
+    if (std::getenv("FLUIDML_MOVE_OUT_OFF") != nullptr) return;
+    for (size_t k = 0; k < fused->size(); ++k) {
+      if ((*fused)[k].kind != Launch::Kind::PadViewCopy) continue;
+      const Launch copy = (*fused)[k];
+      const size_t pad = copy.members[0];
+      const Operand x = steps_[pad].in0, padded = steps_[pad].out;
+      const bool own_bytes = x.space == Operand::Space::Arena || (x.space == Operand::Space::Private && x.pool.empty());
+      if (x.viewed || !own_bytes || !IsFloat(x) || !DefaultLayout(x) || !Elidable(x)) continue;
+      if (padded.viewed || !DefaultLayout(padded) || !Elidable(padded) || !Movable(padded)) continue;
+      const auto xr = readers_.find(x.name);
+      if (xr == readers_.end() || xr->second.size() != 1 || xr->second[0] != pad) continue;
+      const auto &pairs = Attrs(pad).pad_pairs;
+      const auto &xshape = x.meta.GetShape();
+      const auto &pshape = padded.meta.GetShape();
+      bool ok = pairs.size() == pshape.size() && xshape.size() == pshape.size();
+      for (size_t d = 0; ok && d < pairs.size(); ++d) {
+        ok = std::get<0>(pairs[d]) >= 0 && std::get<1>(pairs[d]) >= 0 &&
+             xshape[d] + std::get<0>(pairs[d]) + std::get<1>(pairs[d]) == pshape[d];
+      }
+      if (!ok) continue;
+      // the launch (or member of a group) that writes x, as a plain MatMul chain: it takes any output strides
+      const auto made = producer_.find(x.name);
+      if (made == producer_.end()) continue;
+      Launch *member = nullptr;
+      size_t position = 0;
+      for (Launch &l : *fused) {
+        const size_t pos = l.kind == Launch::Kind::MatMulGroup ? l.position : l.members.back();
+        if (l.group.empty()) {
+          if (SameTensor(l.out, x) && !l.out.viewed && l.members.back() == made->second) member = &l, position = pos;
+        } else {
+          for (Launch &g : l.group) {
+            if (SameTensor(g.out, x) && !g.out.viewed && g.members.back() == made->second) member = &g, position = pos;
+          }
+        }
+      }
+      if (member == nullptr || member->kind != Launch::Kind::MatMulChain || !member->view_strides.empty() ||
+          member->has_skip || member->has_out2 || member->norm_mode != 0 ||
+          !member->norm_stats_out.empty() || position >= pad) {
+        continue;
+      }
+      MoveOut(padded.name, {fused});
+      const Operand whole = steps_[pad].out;  // (where it lives now)
+      const std::vector<int64_t> strides = LogicalStrides(whole);
+      Operand interior = whole;
+      interior.meta = x.meta;
+      interior.viewed = true;
+      interior.view_strides = strides;
+      interior.view_offset = 0;
+      for (size_t d = 0; d < pairs.size(); ++d) interior.view_offset += std::get<0>(pairs[d]) * strides[d];
+      interior.source_bytes = whole.Extent();
+      for (Launch &l : *fused) {
+        // (a group carries a copy of one member's output operand as its own)
+        if (!l.group.empty() && SameTensor(l.out, x) && !l.out.viewed) l.out = interior;
+      }
+      member->out = interior;
+      steps_[made->second].out = interior;
+      filled_[pad] = true;  // nothing runs at the Pad's place
+      for (size_t m = 1; m < copy.members.size(); ++m) taken_[copy.members[m]] = false;
+      fused->erase(fused->begin() + static_cast<std::ptrdiff_t>(k));
+      --k;
+      BuildReaders();
+    }
   }
 
   void PlaceConcatInputs(std::vector<Launch> *fused) {

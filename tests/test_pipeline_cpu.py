@@ -355,7 +355,7 @@ SCHEDULE_NETS = {
     # Softmax -> MatMul pairs and attention blocks matched after view elision
     # (third entry: kinds expected with the default layouts only)
     "convbert_base_full": (lambda m: m.convbert_base(), {"MatMulChain", "AddLayerNormalization"},
-                           {"SoftmaxMatVec", "Attention", "PadViewCopy", "Placed", "MatMulGroup"}),
+                           {"SoftmaxMatVec", "Attention", "Placed", "MatMulGroup"}),
     "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), {"MatMulChain", "Attention", "View", "RotaryPair"}),
     # full size (vocabulary cut: the projection's weights play no part in the plan): the parallel-residual blocks with
     # both LayerNormalizations of a layer deferred into their readers, side by side with the plan's real reuse of bytes
@@ -403,7 +403,8 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     for l in launches:
         for to in l["moved_out"]:
             assert to["space"] == "private"
-            assert to["name"] in {steps[m]["out"]["name"] for m in l["members"]} | {l.get("writes_into", {}).get("name")}
+            assert to["name"] in ({steps[m]["out"]["name"] for m in l["members"]} | {l.get("writes_into", {}).get("name")}
+                                  | {w["into"]["name"] for w in l["writes_inside"]})
             assert any(w["space"] == "private" and w["name"] == to["name"] for w in l["writes"])
             for other in launches:
                 assert all(r["space"] == "private" for r in other["reads"] if r["name"] == to["name"])
@@ -413,6 +414,14 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
                 for op in s["inputs"] + [s["out"]]:
                     if op["name"] == to["name"]:
                         op.update(space="private", offset=0, pool="")
+    # (a tensor written into the interior of a padded buffer never touches the bytes the plan holds for it)
+    for l in launches:
+        for w in l["writes_inside"]:
+            redirected = steps[w["step"]]["out"]["name"]
+            for s in steps:
+                for op in s["inputs"] + [s["out"]]:
+                    if op["name"] == redirected:
+                        op.update(space="private", offset=0, pool="")
     readers = {}
     for i, s in enumerate(steps):
         for op in s["inputs"]:
@@ -421,6 +430,37 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     for l in launches:
         for m in l["members"]:
             issued[m] = (l["position"], l)
+    # A zero Pad that does not run ("writes_inside"): the launch that produces the Pad's input writes it into the
+    # interior of the padded tensor, which lives in a buffer of its own outside the arena (zero when it is created).
+    # The border stays zero only if nothing else ever writes the buffer; the input has no other reader; the interior
+    # is where the Pad would have put the input; the launch runs before the Pad's place.
+    padded_in_place = set()
+    for l in launches:
+        for w in l["writes_inside"]:
+            into = w["into"]
+            (t,) = [i for i, st in enumerate(steps) if st["out"]["name"] == into["name"] and st["kernel"] == "PadKernel"]
+            whole, x = steps[t]["out"], steps[t]["inputs"][0]
+            assert whole["space"] == "private" and into["space"] == "private" and whole["pool"] == ""
+            assert issued[t][1]["kind"] == "Placed" and issued[t][1]["written"] == [] and l["position"] < t
+            assert w["step"] in l["members"] and w["step"] in l["written"]
+            assert readers[x["name"]] == {t}, "a Pad input written in place has another reader"
+            assert into["shape"] == x["shape"] and whole["layout"] == sorted(whole["layout"])
+            strides = [int(np.prod(whole["shape"][d + 1:])) for d in range(len(whole["shape"]))]
+            assert list(into["view_strides"]) == strides
+            lead = into["view_offset"]
+            for d, st in enumerate(strides):  # the interior starts `before` elements in along every dim and fits
+                before, lead = divmod(lead, st)
+                assert 0 <= before and before + x["shape"][d] <= whole["shape"][d]
+            assert lead == 0
+            for other in launches:
+                if other is l:
+                    assert sum(1 for ww in other["writes"] if ww["name"] == into["name"]) == 1
+                else:
+                    assert all(ww["name"] != into["name"] for ww in other["writes"]), "someone else writes a padded buffer"
+            for q, st in enumerate(steps):  # (no step other than the Pad and the redirected producer names it as output)
+                if st["out"]["name"] == into["name"]:
+                    assert q == t or q == w["step"] or q in {ll["members"][0] for ll in launches if ll["kind"] == "View"}
+            padded_in_place.add(t)
     # A step that is not run (kind "View"): its readers address `source`, the bytes of another tensor, when
     # they are issued.  Everything that writes between the view step and such a reader -- outputs of single
     # steps at their own position, outputs of fused launches at the launch's position -- must stay off those
@@ -505,7 +545,9 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
                         op = issued[made_by[0]][1]["source"]  # read through a view that is not run: its source's bytes
                     assert not _overlap(op, into), "bytes of a Concat2 output written early are in use"
     for l in launches:
-        if l["kind"] == "Placed" and steps[l["members"][0]]["kernel"] != "Concat2Kernel":
+        if l["kind"] == "Placed" and steps[l["members"][0]]["kernel"] == "PadKernel":
+            assert l["members"][0] in padded_in_place and l["written"] == []
+        elif l["kind"] == "Placed" and steps[l["members"][0]]["kernel"] != "Concat2Kernel":
             assert l["members"][0] in filled and l["written"] == []
         elif l["kind"] == "Placed":
             assert in_place.get(l["members"][0]) == 2 and l["written"] == []

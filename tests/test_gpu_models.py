@@ -57,6 +57,40 @@ def test_config_matches_oracle(device, config, flavour, tmp_path, monkeypatch):
             assert_close(outs[name], ref, what=f"{config} {flavour} {name}")
 
 
+@pytest.mark.parametrize("config", ["convbert", "gpt_neox", "convbert_wide", "efficientnet_b0"])
+def test_without_tensors_moved_out_of_the_arena(device, config, tmp_path, monkeypatch):
+    """FLUIDML_MOVE_OUT_OFF=1: every tensor stays where the memory plan put it, so the fusions that need a buffer
+    of their own do not happen and the launches they replaced run instead (the Pad -> Gather -> Transpose copy of
+    ConvBERT's convolution branch among them); fewer tensors live outside the arena, the results are the same."""
+    from fluidml_amd import fluidml
+
+    make_net, make_feeds = _cases()[config]
+    net, feeds = make_net(), make_feeds()
+    want = graph_runner.run_graph(net, feeds)
+    path = net.save(str(tmp_path / f"{config}.onnx"))
+    plans = {}
+    for off in ("", "1"):
+        if off:
+            monkeypatch.setenv("FLUIDML_MOVE_OUT_OFF", off)
+        print("[case]", config, "FLUIDML_MOVE_OUT_OFF =", off or "(unset)", flush=True)
+        ex = fluidml.Executor.make_plain_greedy(config + off, 1)
+        ex.compile(path)
+        plans[off] = ex.plan()
+        args = {k: np.ascontiguousarray(v) for k, v in feeds.items()}
+        outs = {v.name: np.full(v.shape, np.nan, dtype=v.dtype) for v in net.outputs}
+        args.update(outs)
+        assert ex.invoke(args) > 0
+        for name, ref in want.items():
+            assert_close(outs[name], ref, what=f"{config} FLUIDML_MOVE_OUT_OFF={off} {name}")
+    kept = plans["1"]
+    assert all(not l["moved_out"] and not l["writes_inside"] for l in kept["launches"])
+    runs = lambda plan: len([l for l in plan["launches"] if l["kind"] not in ("View", "Placed")])
+    assert runs(kept) >= runs(plans[""])
+    if config.startswith("convbert"):
+        assert any(l["kind"] == "PadViewCopy" for l in kept["launches"])
+        assert any(l["writes_inside"] for l in plans[""]["launches"])
+
+
 @pytest.mark.parametrize("use_graph", [True, False], ids=["captured", "eager"])
 @pytest.mark.parametrize("config", ["convbert", "gpt_neox", "efficientnet_b0", "convbert_wide", "gpt_neox_deep"])
 def test_side_branches_match_oracle(device, config, use_graph, tmp_path):

@@ -1556,7 +1556,13 @@ class Scheduler {
     l.owner = *j;
     l.b = soft.in0;
     l.members.insert(l.members.begin(), i);
-    if (!Safe(l.members, {{i, l.b}, {*j, l.a}}) || !OutputDisjoint(l.out, {&l.a, &l.b})) return std::nullopt;
+    // (operands or a result the plan has other tenants for in the launch's window move out of the arena)
+    std::vector<std::string> moves;
+    const bool clash = !OutputDisjoint(l.out, {&l.a, &l.b});
+    if (clash && !Movable(l.out)) return std::nullopt;
+    if (!SafeWithMoves(l.members, {{i, l.b}, {*j, l.a}}, &moves)) return std::nullopt;
+    if (clash) moves.push_back(l.out.name);
+    pending_moves_.insert(pending_moves_.end(), moves.begin(), moves.end());
     l.bytes = Bytes({&l.a, &l.b, &l.out});
     l.flops = Flops(l.members);
     return l;
@@ -2373,23 +2379,32 @@ class Scheduler {
     }
     external.push_back({pv, l.c});
     l.members.push_back(pv);
-    auto finish = [&](Launch *x) {
-      if (!Safe(x->members, external)) return false;
-      if (!OutputDisjoint(x->out, {&x->a, &x->b, &x->c}) || (x->has_mask && Alias(x->out, x->d))) return false;
+    // `with_moves`: operands or a result the plan has other tenants for in the launch's window may move out of the
+    // arena.  Tried only where nothing works without: a tensor in a buffer of its own costs the replayed graph a
+    // little (BERT-base: 1 % with its twelve attention outputs moved for no launch less).
+    auto finish = [&](Launch *x, bool with_moves) {
+      std::vector<std::string> moves;
+      const bool clash = !OutputDisjoint(x->out, {&x->a, &x->b, &x->c}) || (x->has_mask && Alias(x->out, x->d));
+      if (clash && (!with_moves || !Movable(x->out))) return false;
+      if (with_moves ? !SafeWithMoves(x->members, external, &moves) : !Safe(x->members, external)) return false;
+      if (clash) moves.push_back(x->out.name);
+      pending_moves_.insert(pending_moves_.end(), moves.begin(), moves.end());
       x->bytes = x->has_mask ? Bytes({&x->a, &x->b, &x->c, &x->d, &x->out}) : Bytes({&x->a, &x->b, &x->c, &x->out});
       if (x->has_cond) x->bytes += static_cast<double>(steps_[x->owner].kernel->GetConstantBytes());
       x->flops = Flops(x->members);
       return true;
     };
-    for (size_t limit = SIZE_MAX; limit > 0;) {
-      Launch with_views = l;
-      const size_t taken = AppendViews(pv, &with_views, limit);
-      if (taken == 0) break;
-      if (with_views.n_inner == 0 && finish(&with_views)) return with_views;
-      limit = taken - 1;
+    for (const bool with_moves : {false, true}) {
+      for (size_t limit = SIZE_MAX; limit > 0;) {
+        Launch with_views = l;
+        const size_t taken = AppendViews(pv, &with_views, limit);
+        if (taken == 0) break;
+        if (with_views.n_inner == 0 && finish(&with_views, with_moves)) return with_views;
+        limit = taken - 1;
+      }
     }
     l.out = steps_[pv].out;
-    if (finish(&l)) return l;
+    if (finish(&l, false) || finish(&l, true)) return l;
     return std::nullopt;
   }
 

@@ -319,6 +319,66 @@ __global__ __launch_bounds__(kBlock) void LayerNormRowBlock(RowArgs<6> a, float 
   }
 }
 
+// An embedding lookup, the embeddings added to it and the LayerNormalization behind them, one workgroup per looked-up
+// row (len <= ITEMS * kBlock, every operand dense along the row):
+//   v = (data0[idx0[row]] + second) + third,   second = data1[idx1[row]] or a tensor's row,   out = LN(v)
+// The sums round like the separate Gather / AddCommon kernels; the statistics are the two passes of LayerNormRowBlock.
+struct EmbedArgs {
+  uint32_t len;
+  int64_t rows0, rows1;          // rows of the tables (rows1 unused without idx1)
+  uint32_t second_rows, third_rows;  // a tensor addend repeats after this many rows (leading dims of extent 1)
+};
+__device__ inline int64_t TableRow(int64_t idx, int64_t rows) {
+  if (idx < 0) idx += rows;  // ONNX negative indexing
+  return idx < 0 ? 0 : (idx >= rows ? rows - 1 : idx);  // never read outside the table
+}
+template <int ITEMS>
+__global__ __launch_bounds__(kBlock) void EmbeddingLayerNormKernel(EmbedArgs a, float *__restrict__ out,
+                                                                   const int64_t *__restrict__ idx0,
+                                                                   const float *__restrict__ data0,
+                                                                   const int64_t *__restrict__ idx1,
+                                                                   const float *__restrict__ second,
+                                                                   const float *__restrict__ third,
+                                                                   const float *__restrict__ scale,
+                                                                   const float *__restrict__ bias, float eps) {
+  __shared__ float smem[kBlock / kWave];
+  const uint32_t row = blockIdx.x;
+  const float *r0 = data0 + TableRow(idx0[row], a.rows0) * a.len;
+  const float *r1 = idx1 != nullptr ? second + TableRow(idx1[row], a.rows1) * a.len
+                                    : second + static_cast<size_t>(row % a.second_rows) * a.len;
+  const float *r2 = third != nullptr ? third + static_cast<size_t>(row % a.third_rows) * a.len : nullptr;
+  const float n = static_cast<float>(a.len);
+  float x[ITEMS], gv[ITEMS], bv[ITEMS];
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = threadIdx.x + i * kBlock;
+    const bool in = j < a.len;
+    x[i] = in ? r0[j] + r1[j] : 0.0f;
+    if (r2 != nullptr && in) x[i] = x[i] + r2[j];
+    gv[i] = in ? scale[j] : 0.0f;
+    bv[i] = in ? bias[j] : 0.0f;
+    s += x[i];
+  }
+  s = BlockReduce<kBlock / kWave>(s, SumOp{}, smem);
+  const float mean = s / n;
+  float v = 0.0f;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = threadIdx.x + i * kBlock;
+    x[i] = j < a.len ? x[i] - mean : 0.0f;
+    v += x[i] * x[i];
+  }
+  v = BlockReduce<kBlock / kWave>(v, SumOp{}, smem);
+  const float inv = 1.0f / sqrtf(v / n + eps);
+  float *dst = out + static_cast<size_t>(row) * a.len;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    const uint32_t j = threadIdx.x + i * kBlock;
+    if (j < a.len) dst[j] = (x[i] * inv) * gv[i] + bv[i];
+  }
+}
+
 // One wave per row, row cached in registers: len <= 64 * ITEMS; no workgroup barrier at all.
 template <int ITEMS>
 __global__ __launch_bounds__(kBlock) void LayerNormRowWave(RowArgs<6> a, float *__restrict__ out,
@@ -909,6 +969,103 @@ int fluidml_hip_add_layer_normalization(const fl_tensor *lhs, const fl_tensor *r
                                         void *stream) {
   if (rhs == nullptr) return FL_ERR_NULL;
   return LayerNormImpl(lhs, rhs, scale, bias, out, nullptr, 0, axis, epsilon, 0, stream);
+}
+
+namespace {
+bool DenseRowMajor(const fl_tensor *t) {
+  int64_t want = 1;
+  for (int i = t->rank - 1; i >= 0; --i) {
+    if (t->shape[i] != 1 && t->strides[i] != want) return false;
+    want *= t->shape[i];
+  }
+  return true;
+}
+int64_t Elements(const fl_tensor *t) {
+  int64_t n = 1;
+  for (int i = 0; i < t->rank; ++i) n *= t->shape[i];
+  return n;
+}
+// `t` as an addend of `out` [rows..., len]: its dims, aligned at the right, equal out's, with nothing but ones in
+// front; *rows = how many rows it holds (it repeats after them)
+int AddendRows(const fl_tensor *t, const fl_tensor *out, uint32_t *rows) {
+  FL_CHECK(CheckView(t));
+  if (t->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  if (t->rank > out->rank || t->rank < 1 || !DenseRowMajor(t)) return FL_ERR_UNSUPPORTED;
+  bool ones = false;
+  for (int i = 1; i <= out->rank; ++i) {
+    const int64_t have = i <= t->rank ? t->shape[t->rank - i] : 1;
+    const int64_t want = out->shape[out->rank - i];
+    if (!ones && have == want) continue;
+    if (have != 1 || i == 1) return FL_ERR_UNSUPPORTED;  // broadcast along the row or between kept dims
+    ones = true;
+  }
+  *rows = static_cast<uint32_t>(Elements(t) / out->shape[out->rank - 1]);
+  return FL_OK;
+}
+}  // namespace
+
+int fluidml_hip_gather_add_layer_normalization(const fl_tensor *indices0, const fl_tensor *data0,
+                                               const fl_tensor *indices1, const fl_tensor *second,
+                                               const fl_tensor *third, const fl_tensor *scale, const fl_tensor *bias,
+                                               const fl_tensor *out, double epsilon, void *stream) {
+  if (!indices0 || !data0 || !second || !scale || !bias || !out) return FL_ERR_NULL;
+  for (const fl_tensor *t : {indices0, data0, second, scale, bias, out}) FL_CHECK(CheckView(t));
+  if (indices1 != nullptr) FL_CHECK(CheckView(indices1));
+  if (indices0->dtype != FL_INT64 || (indices1 != nullptr && indices1->dtype != FL_INT64)) return FL_ERR_DTYPE;
+  if (data0->dtype != FL_FLOAT32 || second->dtype != FL_FLOAT32 || scale->dtype != FL_FLOAT32 ||
+      bias->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32)
+    return FL_ERR_DTYPE;
+  if (data0->rank != 2 || out->rank != indices0->rank + 1 || out->rank < 1) return FL_ERR_RANK;
+  const int64_t len = data0->shape[1];
+  for (int i = 0; i < indices0->rank; ++i) {
+    if (out->shape[i] != indices0->shape[i]) return FL_ERR_SHAPE;
+  }
+  if (out->shape[out->rank - 1] != len || Elements(scale) != len || Elements(bias) != len) return FL_ERR_SHAPE;
+  if (!DenseRowMajor(indices0) || !DenseRowMajor(data0) || !DenseRowMajor(out) || !DenseRowMajor(scale) ||
+      !DenseRowMajor(bias))
+    return FL_ERR_UNSUPPORTED;
+  if (len < 1 || len > FL_GATHER_LAYER_NORM_MAX_LEN) return FL_ERR_UNSUPPORTED;
+  const int64_t rows = Elements(indices0);
+  if (rows > INT32_MAX) return FL_ERR_TOO_LARGE;
+  EmbedArgs a{};
+  a.len = static_cast<uint32_t>(len);
+  a.rows0 = data0->shape[0];
+  a.second_rows = a.third_rows = 1;
+  if (indices1 != nullptr) {
+    if (second->rank != 2 || second->shape[1] != len || !DenseRowMajor(second) || !DenseRowMajor(indices1))
+      return FL_ERR_UNSUPPORTED;
+    if (indices1->rank != indices0->rank) return FL_ERR_RANK;
+    for (int i = 0; i < indices0->rank; ++i) {
+      if (indices1->shape[i] != indices0->shape[i]) return FL_ERR_SHAPE;
+    }
+    a.rows1 = second->shape[0];
+  } else {
+    FL_CHECK(AddendRows(second, out, &a.second_rows));
+  }
+  if (third != nullptr) FL_CHECK(AddendRows(third, out, &a.third_rows));
+  if (rows == 0) return FL_OK;
+  hipStream_t s = AsStream(stream);
+  float *o = static_cast<float *>(out->base);
+  const int64_t *i0 = static_cast<const int64_t *>(indices0->base);
+  const int64_t *i1 = indices1 != nullptr ? static_cast<const int64_t *>(indices1->base) : nullptr;
+  const float *d0 = static_cast<const float *>(data0->base), *d1 = static_cast<const float *>(second->base);
+  const float *d2 = third != nullptr ? static_cast<const float *>(third->base) : nullptr;
+  const float *g = static_cast<const float *>(scale->base), *b = static_cast<const float *>(bias->base);
+  const float eps = static_cast<float>(epsilon);
+  const dim3 grid(static_cast<uint32_t>(rows));
+#define FL_EMBED(ITEMS) \
+  FL_LAUNCH(EmbeddingLayerNormKernel<ITEMS>, grid, dim3(kBlock), 0, s, a, o, i0, d0, i1, d1, d2, g, b, eps)
+  if (len <= kBlock) {
+    FL_EMBED(1);
+  } else if (len <= 2 * kBlock) {
+    FL_EMBED(2);
+  } else if (len <= 4 * kBlock) {
+    FL_EMBED(4);
+  } else {
+    FL_EMBED(8);
+  }
+#undef FL_EMBED
+  return LaunchStatus();
 }
 
 int fluidml_hip_reduce_mean(const fl_tensor *in, const fl_tensor *out, const int64_t *axes, int32_t n_axes,

@@ -36,6 +36,7 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::DivAddSoftmax: return "DivAddSoftmax";
     case Launch::Kind::Attention: return "Attention";
     case Launch::Kind::AddLayerNorm: return "AddLayerNormalization";
+    case Launch::Kind::GatherAddLayerNorm: return "GatherAddLayerNormalization";
     case Launch::Kind::ReshapeTranspose: return "ReshapeTranspose";
     case Launch::Kind::View: return "View";
     case Launch::Kind::Placed: return "Placed";
@@ -287,6 +288,7 @@ class Scheduler {
       silent_.clear();
     }
     if (fuse) DeferLayerNorms(&fused);
+    if (fuse) FuseEmbeddings(&fused);
     if (fuse) PlaceConcatInputs(&fused);
     // a chain is issued where its last member stood; everything else keeps its place
     std::vector<const Launch *> at(steps_.size(), nullptr);
@@ -2105,6 +2107,107 @@ class Scheduler {
       }
     }
     return std::nullopt;
+  }
+
+  // GatherAdd (one addend) -> AddLayerNorm over the last dim, the embedding block of a BERT-style encoder: one launch
+  // (fluidml_hip_gather_add_layer_normalization).  Where the GatherAdd's addend is itself a looked-up embedding with no
+  // other reader, that lookup joins too.  Every operand in its default layout; sums in the order of the steps.
+  void FuseEmbeddings(std::vector<Launch> *fused) {
+    if (const char *v = std::getenv("FLUIDML_EMBEDDING"); v != nullptr && std::string(v) == "0") return;
+    auto only_reader = [&](const Operand &o, size_t reader) {
+      if (!Elidable(o)) return false;
+      const auto it = readers_.find(o.name);
+      return it != readers_.end() && it->second.size() == 1 && it->second[0] == reader;
+    };
+    // `t` has the trailing dims of `out` with nothing but ones in front (it repeats along out's leading dims)
+    auto repeats = [](const std::vector<int64_t> &t, const std::vector<int64_t> &out) {
+      if (t.empty() || t.size() > out.size() || t.back() != out.back()) return false;
+      bool ones = false;
+      for (size_t i = 1; i <= out.size(); ++i) {
+        const int64_t have = i <= t.size() ? t[t.size() - i] : 1;
+        if (!ones && have == out[out.size() - i]) continue;
+        if (have != 1) return false;
+        ones = true;
+      }
+      return true;
+    };
+    for (size_t n = 0; n < fused->size(); ++n) {
+      const Launch norm = (*fused)[n];
+      if (norm.kind != Launch::Kind::AddLayerNorm || norm.norm_mode != 0 || !norm.norm_stats_out.empty()) continue;
+      const std::vector<int64_t> &shape = norm.out.meta.GetShape();
+      const int64_t rank = static_cast<int64_t>(shape.size());
+      if (rank < 2 || (norm.axis != rank - 1 && norm.axis != -1) || shape.back() > FL_GATHER_LAYER_NORM_MAX_LEN) continue;
+      size_t g = fused->size();
+      for (size_t k = 0; k < fused->size() && g == fused->size(); ++k) {
+        const Launch &cand = (*fused)[k];
+        if (cand.kind != Launch::Kind::GatherAdd || cand.has_c) continue;
+        if (!SameTensor(cand.out, norm.a) && !SameTensor(cand.out, norm.b)) continue;
+        if (only_reader(cand.out, norm.members.front())) g = k;
+      }
+      if (g == fused->size()) continue;
+      const Launch gather = (*fused)[g];
+      const Operand &third = SameTensor(gather.out, norm.a) ? norm.b : norm.a;
+      if (SameTensor(third, gather.out) || !IsFloat(third) || !DefaultLayout(third) || !DefaultLayout(norm.out) ||
+          !DefaultLayout(gather.a) || !DefaultLayout(gather.b) || gather.out.meta.GetShape() != shape ||
+          !repeats(third.meta.GetShape(), shape) || !repeats(gather.b.meta.GetShape(), shape)) {
+        continue;
+      }
+      // a table of rows: the result has one dim more than the indices
+      if (steps_[gather.owner].kernel->GetConstant(0) == nullptr ||
+          static_cast<int64_t>(gather.a.meta.GetShape().size()) != rank - 1) {
+        continue;
+      }
+      Launch l;
+      l.kind = Launch::Kind::GatherAddLayerNorm;
+      l.members = gather.members;
+      l.members.insert(l.members.end(), norm.members.begin(), norm.members.end());
+      l.a = gather.a;
+      l.b = gather.b;
+      l.c = third;
+      l.has_c = true;
+      l.out = norm.out;
+      l.owner = gather.owner;
+      l.norm_owner = norm.owner;
+      l.s0 = norm.s0;
+      std::vector<std::pair<size_t, Operand>> external = {{gather.members.front(), l.a}, {norm.members.front(), l.c}};
+      // the addend of the lookup: a second lookup that nobody else reads
+      size_t second = SIZE_MAX;
+      if (const auto p = producer_.find(gather.b.name); p != producer_.end() && !taken_[p->second] &&
+                                                        Kind(p->second) == OpKind::GatherConstantDataTensor) {
+        const Step &st = steps_[p->second];
+        if (IsFloat(st.out) && st.kernel->GetConstant(0) != nullptr && only_reader(st.out, gather.members[1]) &&
+            st.out.meta.GetShape() == shape && DefaultLayout(st.in0) &&
+            st.in0.meta.GetShape() == gather.a.meta.GetShape()) {
+          second = p->second;
+        }
+      }
+      Launch with_second = l;
+      if (second != SIZE_MAX) {
+        with_second.members.push_back(second);
+        std::sort(with_second.members.begin(), with_second.members.end());
+        with_second.b = steps_[second].in0;
+        with_second.has_gate = true;
+        with_second.owner2 = second;
+        auto ext = external;
+        ext.push_back({second, with_second.b});
+        if (Safe(with_second.members, ext) && OutputDisjoint(with_second.out, {&with_second.a, &with_second.b, &with_second.c})) {
+          l = with_second;
+        } else {
+          second = SIZE_MAX;
+        }
+      }
+      if (second == SIZE_MAX) {
+        std::sort(l.members.begin(), l.members.end());
+        external.push_back({gather.members[1], l.b});
+        if (!Safe(l.members, external) || !OutputDisjoint(l.out, {&l.a, &l.b, &l.c})) continue;
+      }
+      l.bytes = Bytes({&l.a, &l.c, &l.out}) + 2.0 * static_cast<double>(l.out.meta.GetSize()) +
+                static_cast<double>(steps_[norm.owner].kernel->GetConstantBytes());
+      if (second != SIZE_MAX) taken_[second] = true;
+      (*fused)[n] = std::move(l);
+      fused->erase(fused->begin() + static_cast<std::ptrdiff_t>(g));
+      if (g < n) --n;
+    }
   }
 
   // GatherConstantDataTensor -> AddCommon [-> AddCommon] (an embedding lookup and the embeddings added to it)

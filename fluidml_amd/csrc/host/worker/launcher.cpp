@@ -801,6 +801,24 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out)
       rc = fluidml_hip_add_layer_normalization(&a.t, &b.t, &g.t, &h.t, &out.t, l.axis, l.s0, ctx.stream);
       break;
     }
+    case Launch::Kind::GatherAddLayerNorm: {
+      const kernel::DeviceConstant *table = steps_[l.owner].kernel->GetConstant(0);
+      const kernel::DeviceConstant *table2 = l.has_gate ? steps_[l.owner2].kernel->GetConstant(0) : nullptr;
+      const kernel::Kernel &ln = *steps_[l.norm_owner].kernel;
+      const kernel::DeviceConstant *scale = ln.GetConstant(0), *bias = ln.GetConstant(1);
+      if (table == nullptr || (l.has_gate && table2 == nullptr) || scale == nullptr || bias == nullptr) {
+        throw std::logic_error("fused embedding: a node holds no table / scale / bias");
+      }
+      const kernel::TensorView data = table->View(), b = ViewOf(Resolve(l.b), l.b), c = ViewOf(Resolve(l.c), l.c);
+      const kernel::TensorView g = scale->View(), h = bias->View();
+      if (l.has_gate) {
+        const kernel::TensorView data2 = table2->View();
+        rc = fluidml_hip_gather_add_layer_normalization(&a.t, &data.t, &b.t, &data2.t, &c.t, &g.t, &h.t, &out.t, l.s0, ctx.stream);
+      } else {
+        rc = fluidml_hip_gather_add_layer_normalization(&a.t, &data.t, nullptr, &b.t, &c.t, &g.t, &h.t, &out.t, l.s0, ctx.stream);
+      }
+      break;
+    }
     case Launch::Kind::CopyInto:
       rc = fluidml_hip_reshape(&a.t, &out.t, ctx.stream);  // same shape on both sides: a strided copy
       break;

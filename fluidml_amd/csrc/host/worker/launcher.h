@@ -89,6 +89,10 @@ struct Launch {
     DivAddSoftmax,     // DivConstantRhs -> AddCommon(mask) -> Softmax
     Attention,         // MatMul -> Div|Mul constant [-> AddCommon(mask)] [-> Where(cond, x, scalar)] -> Softmax -> MatMul
     AddLayerNorm,      // AddCommon -> LayerNormalizationConstantScaleBias
+    GatherAddLayerNorm,  // [GatherConstantDataTensor ->] GatherConstantDataTensor -> AddCommon -> AddCommon ->
+                         // LayerNormalizationConstantScaleBias (last dim): a = indices into the table of `owner`,
+                         // b = the first addend, or with has_gate the indices into the table of `owner2`, c = the
+                         // second addend, `norm_owner` = the LayerNormalization step, s0 = epsilon
     ReshapeTranspose,  // Reshape -> Transpose, one strided copy
     TransposeReshape,  // Transpose -> Reshape, one strided copy
     PadViewCopy,       // Pad -> steps that only re-address its result (Gather of sliding windows, Slice, Transpose,

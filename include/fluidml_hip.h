@@ -536,6 +536,21 @@ int fluidml_hip_div_add_softmax(const fl_tensor *in, double div, const fl_tensor
  * launched).  (reference matmul.cpp:28-59, div.cpp:24-56, add.cpp:75-137,
  * where.cpp:17-150, softmax.cpp:22-139) */
 int fluidml_hip_attention(const fl_tensor *q, const fl_tensor *kt, const fl_tensor *v, const fl_tensor *out, double scale, int32_t scale_is_divisor, const fl_tensor *add_mask, const fl_tensor *keep_cond, double fill, void *stream);
+/* GatherConstantDataTensorKernel [x2] -> AddCommonKernel [-> AddCommonKernel] ->
+ * LayerNormalizationConstantScaleBiasKernel over the last dim (the embedding
+ * block of a BERT-style encoder) as one launch:
+ *   out = LayerNorm((data0[indices0] + x) + third),
+ *   x = second[indices1] when indices1 is given (`second` is then a table
+ *   [rows1, len]), otherwise the tensor `second` itself.
+ * data0 [rows0, len]; indices int64 of out's leading dims; out [..., len];
+ * `second` (as a tensor) and `third` (may be NULL) have out's trailing dims
+ * with nothing but ones in front (they repeat along the leading dims);
+ * scale and bias hold len values.  Everything dense row-major and
+ * len <= FL_GATHER_LAYER_NORM_MAX_LEN, otherwise FL_ERR_UNSUPPORTED and
+ * nothing is launched.  The sums round as the separate kernels' do.
+ * (reference gather.cpp:195-272, add.cpp:75-137, layer_normalization.cpp:33-220) */
+#define FL_GATHER_LAYER_NORM_MAX_LEN 2048
+int fluidml_hip_gather_add_layer_normalization(const fl_tensor *indices0, const fl_tensor *data0, const fl_tensor *indices1, const fl_tensor *second, const fl_tensor *third, const fl_tensor *scale, const fl_tensor *bias, const fl_tensor *out, double epsilon, void *stream);
 /* AddCommonKernel -> LayerNormalizationConstantScaleBiasKernel:
  * out = LayerNorm(lhs + rhs) (reference add.cpp:75-137 +
  * layer_normalization.cpp:33-220, ONNX semantics). */

@@ -62,7 +62,7 @@ def _full_configs():
 
 # the launch kinds each configuration is expected to exercise at full size
 _EXPECTED_KINDS = {
-    "bert_base": {"Attention", "MatMulGroup", "GatherAdd", "AddLayerNormalization"},
+    "bert_base": {"Attention", "MatMulGroup", "GatherAddLayerNormalization"},
     "convbert_base": {"Attention", "SoftmaxMatVec"},
     "gpt_neox": {"Attention", "RotaryPair"},
     "efficientnet_b0": {"ConvChain", "ConvPair"},

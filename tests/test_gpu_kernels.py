@@ -1285,6 +1285,61 @@ def test_fused_add_layer_norm(device):
             assert_close(do.logical(), ho.logical(), what="add_layer_normalization")
 
 
+def test_gather_add_layer_norm(device):
+    """The embedding block as one launch against the oracle's separate Gather, Add, Add and LayerNormalization: with
+    one table or two, a second addend or none, addends that repeat along the leading dims."""
+    cabi = _cabi()
+    rng = np.random.default_rng(211)
+    for lead, length, rows0, rows1, eps in [((1, 128), 768, 1000, 2, 1e-12), ((3, 5), 33, 17, 4, 1e-5), ((7,), 2048, 9, 3, 1e-5),
+                                             ((2, 6), 300, 50, 5, 1e-5)]:
+        shape = lead + (length,)
+        t0, t1 = rand(rng, (rows0, length), -1, 1), rand(rng, (rows1, length), -1, 1)
+        i0 = rng.integers(0, rows0, size=lead).astype(np.int64)
+        i1 = rng.integers(0, rows1, size=lead).astype(np.int64)
+        g, b = rand(rng, (length,), 0.5, 1.5), rand(rng, (length,), -0.5, 0.5)
+        full = rand(rng, shape, -1, 1)
+        repeated = rand(rng, (1,) * (len(lead) - 1) + lead[-1:] + (length,), -1, 1)  # like a position embedding
+        hi0, hi1, ht0, ht1, hg, hb = (ok.View(v) for v in (i0, i1, t0, t1, g, b))
+        di0, di1, dt0, dt1, dg, db = (DeviceView(h, device) for h in (hi0, hi1, ht0, ht1, hg, hb))
+        for two_tables in (True, False):
+            for third in (None, full, repeated):
+                announce("gather_add_layer_normalization", shape, two_tables, None if third is None else third.shape)
+                first, second = ok.View.empty(shape), ok.View.empty(shape)
+                ok.gather_data_tensor(hi0, ht0, first)
+                if two_tables:
+                    ok.gather_data_tensor(hi1, ht1, second)
+                else:
+                    second = ok.View(repeated if third is full else full)
+                summed = ok.View.empty(shape)
+                ok.binary_f32(ok.BOP_ADD, first, second, summed)
+                if third is not None:
+                    both = ok.View.empty(shape)
+                    ok.binary_f32(ok.BOP_ADD, summed, ok.View(third), both)
+                    summed = both
+                want = ok.View.empty(shape)
+                ok.layer_norm(summed, hg, hb, want, len(shape) - 1, eps)
+                dsecond = dt1 if two_tables else DeviceView(second, device)
+                dthird = None if third is None else DeviceView(ok.View(third), device)
+                do = DeviceView(ok.View.empty(shape, np.float32, None, fill=5), device)
+                cabi.call("gather_add_layer_normalization", di0.ref(), dt0.ref(), di1.ref() if two_tables else None,
+                          dsecond.ref(), dthird.ref() if dthird else None, dg.ref(), db.ref(), do.ref(),
+                          ctypes.c_double(eps), None)
+                assert_close(do.logical(), want.logical(), what="gather_add_layer_normalization")
+    # refused, nothing launched: a row longer than the kernel keeps in registers, an addend that repeats along the row
+    long_t = DeviceView(ok.View(rand(rng, (4, 4096), -1, 1)), device)
+    ids = DeviceView(ok.View(np.zeros((2,), np.int64)), device)
+    vec = DeviceView(ok.View(rand(rng, (4096,), -1, 1)), device)
+    out = DeviceView(ok.View.empty((2, 4096)), device)
+    assert cabi.lib.fluidml_hip_gather_add_layer_normalization(ids.ref(), long_t.ref(), None, out.ref(), None, vec.ref(),
+                                                               vec.ref(), out.ref(), 1e-5, None) == cabi.FL_ERR_UNSUPPORTED
+    small_t = DeviceView(ok.View(rand(rng, (4, 8), -1, 1)), device)
+    col = DeviceView(ok.View(rand(rng, (2, 1), -1, 1)), device)
+    v8 = DeviceView(ok.View(rand(rng, (8,), -1, 1)), device)
+    out8 = DeviceView(ok.View.empty((2, 8)), device)
+    assert cabi.lib.fluidml_hip_gather_add_layer_normalization(ids.ref(), small_t.ref(), None, col.ref(), None, v8.ref(),
+                                                               v8.ref(), out8.ref(), 1e-5, None) == cabi.FL_ERR_UNSUPPORTED
+
+
 @pytest.mark.parametrize("M,H,K0,N1", [(128, 256, 128, 384), (100, 200, 96, 72), (33, 768, 256, 768)], ids=str)
 def test_matmul_with_deferred_layer_norm(device, M, H, K0, N1):
     """A LayerNormalization that never reaches memory (fluidml_hip_matmul_chain_group_norm) against the oracle's

@@ -346,16 +346,18 @@ def _overlap(x, y):
 
 SCHEDULE_NETS = {
     # the full-size headline graph: its memory plan reuses bytes in ways the small ones do not
-    "bert_base_full": (lambda m: m.bert_base(), {"MatMulGroup", "AddLayerNormalization", "Attention", "GatherAdd"}),
+    # (third entry: kinds expected with the default layouts only)
+    "bert_base_full": (lambda m: m.bert_base(), {"MatMulGroup", "Attention"}, {"GatherAddLayerNormalization"}),
+    # the embedding block as the separate launches (two lookups, the second with its Add, Add + LayerNormalization)
+    "bert_base_full_separate_embedding": (lambda m: m.bert_base(), {"MatMulGroup", "AddLayerNormalization", "Attention", "GatherAdd"}),
     "bert": (lambda m: m.bert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32, seed=5),
-             {"MatMulChain", "AddLayerNormalization", "Attention", "ElementwiseChain"}),
+             {"MatMulChain", "Attention", "ElementwiseChain"}, {"GatherAddLayerNormalization"}),
     "convbert": (lambda m: m.convbert_base(seq=16, layers=2, hidden=64, heads=4, ffn=128, vocab=100, max_pos=32),
-                 {"MatMulChain", "AddLayerNormalization"}),  # whether its attention fuses depends on the plan's reuse of bytes
+                 {"MatMulChain"}, {"GatherAddLayerNormalization"}),  # whether its attention fuses depends on the plan's reuse of bytes
     # full size: the Concat2 of attention and convolution heads written in place (also into the Reshape behind it),
     # Softmax -> MatMul pairs and attention blocks matched after view elision
-    # (third entry: kinds expected with the default layouts only)
-    "convbert_base_full": (lambda m: m.convbert_base(), {"MatMulChain", "AddLayerNormalization"},
-                           {"SoftmaxMatVec", "Attention", "Placed", "MatMulGroup"}),
+    "convbert_base_full": (lambda m: m.convbert_base(), {"MatMulChain"},
+                           {"SoftmaxMatVec", "Attention", "Placed", "MatMulGroup", "GatherAddLayerNormalization"}),
     "gpt_neox": (lambda m: m.gpt_neox(seq=24, layers=2, hidden=64, heads=2, ffn=128, vocab=120), {"MatMulChain", "Attention", "View", "RotaryPair"}),
     # full size (vocabulary cut: the projection's weights play no part in the plan): the parallel-residual blocks with
     # both LayerNormalizations of a layer deferred into their readers, side by side with the plan's real reuse of bytes
@@ -365,7 +367,7 @@ SCHEDULE_NETS = {
                            {"MatMulChain", "Attention", "View", "CopyInto", "MulAdd"}),
     # other extents: other plans, other reuse of bytes under the same passes
     "convbert_wide": (lambda m: m.convbert_base(seq=40, layers=3, hidden=96, heads=6, ffn=192, vocab=64, max_pos=64),
-                      {"MatMulChain", "AddLayerNormalization"}),
+                      {"MatMulChain"}, {"GatherAddLayerNormalization"}),
     "gpt_neox_deep": (lambda m: m.gpt_neox(seq=48, layers=3, hidden=128, heads=4, ffn=256, vocab=90), {"MatMulChain", "Attention", "View"}),
     "efficientnet_b0": (lambda m: m.efficientnet_b0(image=64, classes=10, width_div=4), {"ConvChain", "ConvPair"}),
     "vgg16": (lambda m: m.vgg16(batch=2, image=32, classes=10, width_div=8, fc=512), {"ConvChain", "GemmChain"}),
@@ -379,7 +381,7 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     an elided tensor has no reader outside its chain, and moving a chain's reads to its last member's
     position crosses no write to the bytes it reads (arena intervals of the memory plan)."""
     fluidml, models, _ = mods
-    if which.endswith("_full") and flavour == "make_plain_linear":
+    if "_full" in which and flavour == "make_plain_linear":
         pytest.skip("the linear plan reuses no bytes: the small graphs cover it, the full-size ones are here for their reuse")
     make, expected_kinds = SCHEDULE_NETS[which][:2]
     if flavour != "make_dp_greedy" and len(SCHEDULE_NETS[which]) > 2:
@@ -388,6 +390,8 @@ def test_fused_schedule_is_safe(mods, which, flavour, monkeypatch, tmp_path):
     monkeypatch.setenv("FLUIDML_DP_COST", "constant")
     if which.endswith("_no_rotary"):
         monkeypatch.setenv("FLUIDML_ROTARY", "0")
+    if which.endswith("_separate_embedding"):
+        monkeypatch.setenv("FLUIDML_EMBEDDING", "0")
     ex = getattr(fluidml.Executor, flavour)("sched")
     ex.compile(path)
     plan = ex.plan()

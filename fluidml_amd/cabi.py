@@ -174,6 +174,7 @@ SIGNATURES = {
     "fluidml_hip_attention": [_T, _T, _T, _T, _f64, _i32, _T, _T, _f64, _vp],
     "fluidml_hip_div_add_softmax": [_T, _f64, _T, _T, _i64, _vp],
     "fluidml_hip_add_layer_normalization": [_T, _T, _T, _T, _T, _i64, _f64, _vp],
+    "fluidml_hip_gather_constant_data_tensor_stats": [_T, _T, _T, _vp, _vp],
     "fluidml_hip_gather_add_layer_normalization": [_T, _T, _T, _T, _T, _T, _T, _T, _f64, _vp],
     "fluidml_hip_conv_without_padding": [_T, _T, _T, _T, _i64p, _i64p, _i64, _u32, _vp],
     "fluidml_hip_conv_with_padding": [_T, _T, _T, _T, _vp, _sz, _i64p, _i64p, _i64p, _i64, _u32, _vp],

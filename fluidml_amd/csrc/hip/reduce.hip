@@ -379,6 +379,39 @@ __global__ __launch_bounds__(kBlock) void EmbeddingLayerNormKernel(EmbedArgs a, 
   }
 }
 
+// An embedding lookup that also leaves what a deferred LayerNormalization of its result needs: one workgroup per
+// looked-up row copies the table row and writes (mean, sum of squared deviations) of every run of 32 columns,
+// stats[(row * parts + run) * 2 + {0, 1}] -- the partial row statistics a contraction leaves with FL_NORM stats_out.
+__global__ __launch_bounds__(kBlock) void GatherStatsKernel(uint32_t len, int64_t table_rows, float *__restrict__ out,
+                                                            const int64_t *__restrict__ idx,
+                                                            const float *__restrict__ data, float *__restrict__ stats) {
+  const uint32_t row = blockIdx.x;
+  const float *src = data + TableRow(idx[row], table_rows) * len;
+  float *dst = out + static_cast<size_t>(row) * len;
+  const uint32_t parts = (len + 31) / 32;
+  for (uint32_t base = 0; base < len; base += kBlock) {  // (uniform trip count: the shuffles below need every lane)
+    const uint32_t j = base + threadIdx.x;
+    const bool in = j < len;
+    const float x = in ? src[j] : 0.0f;
+    if (in) dst[j] = x;
+    const uint32_t first = j & ~31u;
+    const float cols = static_cast<float>(first < len ? min(32u, len - first) : 1u);
+    float sum = x;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    const float mean = sum / cols;
+    const float d = in ? x - mean : 0.0f;
+    float sq = d * d;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+    if ((threadIdx.x & 31u) == 0 && in) {
+      float *at = stats + (static_cast<size_t>(row) * parts + j / 32) * 2;
+      at[0] = mean;
+      at[1] = sq;
+    }
+  }
+}
+
 // One wave per row, row cached in registers: len <= 64 * ITEMS; no workgroup barrier at all.
 template <int ITEMS>
 __global__ __launch_bounds__(kBlock) void LayerNormRowWave(RowArgs<6> a, float *__restrict__ out,
@@ -1065,6 +1098,26 @@ int fluidml_hip_gather_add_layer_normalization(const fl_tensor *indices0, const 
     FL_EMBED(8);
   }
 #undef FL_EMBED
+  return LaunchStatus();
+}
+
+int fluidml_hip_gather_constant_data_tensor_stats(const fl_tensor *indices, const fl_tensor *data, const fl_tensor *out,
+                                                  float *stats_out, void *stream) {
+  if (!indices || !data || !out || !stats_out) return FL_ERR_NULL;
+  for (const fl_tensor *t : {indices, data, out}) FL_CHECK(CheckView(t));
+  if (indices->dtype != FL_INT64 || data->dtype != FL_FLOAT32 || out->dtype != FL_FLOAT32) return FL_ERR_DTYPE;
+  if (data->rank != 2 || out->rank != indices->rank + 1) return FL_ERR_RANK;
+  for (int i = 0; i < indices->rank; ++i) {
+    if (out->shape[i] != indices->shape[i]) return FL_ERR_SHAPE;
+  }
+  if (out->shape[out->rank - 1] != data->shape[1]) return FL_ERR_SHAPE;
+  if (!DenseRowMajor(indices) || !DenseRowMajor(data) || !DenseRowMajor(out)) return FL_ERR_UNSUPPORTED;
+  const int64_t rows = Elements(indices);
+  if (rows > INT32_MAX || data->shape[1] > INT32_MAX) return FL_ERR_TOO_LARGE;
+  if (rows == 0 || data->shape[1] == 0) return FL_OK;
+  FL_LAUNCH(GatherStatsKernel, dim3(static_cast<uint32_t>(rows)), dim3(kBlock), 0, AsStream(stream),
+            static_cast<uint32_t>(data->shape[1]), data->shape[0], static_cast<float *>(out->base),
+            static_cast<const int64_t *>(indices->base), static_cast<const float *>(data->base), stats_out);
   return LaunchStatus();
 }
 

@@ -37,6 +37,7 @@ const char *LaunchKindName(Launch::Kind kind) {
     case Launch::Kind::Attention: return "Attention";
     case Launch::Kind::AddLayerNorm: return "AddLayerNormalization";
     case Launch::Kind::GatherAddLayerNorm: return "GatherAddLayerNormalization";
+    case Launch::Kind::GatherStats: return "GatherStatistics";
     case Launch::Kind::ReshapeTranspose: return "ReshapeTranspose";
     case Launch::Kind::View: return "View";
     case Launch::Kind::Placed: return "Placed";
@@ -2748,15 +2749,30 @@ class Scheduler {
       if (ln.kernel->GetConstant(0) == nullptr || ln.kernel->GetConstant(1) == nullptr || !Attrs(i).t0 || !Attrs(i).t1) continue;
       // who writes x
       const auto made = producer_.find(x.name);
-      if (made == producer_.end() || owner[made->second] < 0) continue;
-      Launch &p = (*fused)[static_cast<size_t>(owner[made->second])];
-      if (p.kind != Launch::Kind::MatMulChain || !p.group.empty() || !SameTensor(p.out, x) || p.out.viewed ||
-          !p.view_strides.empty() || p.n_inner != 0 || p.members.back() != made->second) {
-        continue;
-      }
-      if (!IsFloat(p.b) || p.b.viewed || !DefaultLayout(p.b) || p.b.meta.GetShape().size() != 2) continue;
+      if (made == producer_.end()) continue;
       const std::string stats = "norm:" + x.name;
-      if (!p.norm_stats_out.empty() && p.norm_stats_out != stats) continue;
+      // an embedding lookup that runs as a step of its own can leave the statistics as well (GatherStats)
+      const bool from_lookup = owner[made->second] < 0;
+      if (from_lookup) {
+        const size_t g = made->second;
+        if (Kind(g) != OpKind::GatherConstantDataTensor || taken_[g] || elided_[g] || !SameTensor(steps_[g].out, x) ||
+            steps_[g].kernel->GetConstant(0) == nullptr || steps_[g].in0.viewed || !DefaultLayout(steps_[g].in0) ||
+            static_cast<int64_t>(steps_[g].in0.meta.GetShape().size()) != rank - 1 || g >= i) {
+          continue;
+        }
+      } else {
+        const Launch &p = (*fused)[static_cast<size_t>(owner[made->second])];
+        if (p.kind == Launch::Kind::GatherStats) {
+          if (p.norm_stats_out != stats) continue;
+        } else {
+          if (p.kind != Launch::Kind::MatMulChain || !p.group.empty() || !SameTensor(p.out, x) || p.out.viewed ||
+              !p.view_strides.empty() || p.n_inner != 0 || p.members.back() != made->second) {
+            continue;
+          }
+          if (!IsFloat(p.b) || p.b.viewed || !DefaultLayout(p.b) || p.b.meta.GetShape().size() != 2) continue;
+          if (!p.norm_stats_out.empty() && p.norm_stats_out != stats) continue;
+        }
+      }
       // who reads the normalised tensor
       const auto hr = readers_.find(h.name);
       if (hr == readers_.end() || hr->second.empty()) continue;
@@ -2813,7 +2829,21 @@ class Scheduler {
         MoveOut(x.name, {fused});
       }
       const Operand source = steps_[i].in0;  // (x, where it lives now)
-      p.norm_stats_out = stats;
+      if (from_lookup) {
+        const size_t g = made->second;
+        Launch lookup;
+        lookup.kind = Launch::Kind::GatherStats;
+        lookup.members = {g};
+        lookup.a = steps_[g].in0;
+        lookup.out = steps_[g].out;
+        lookup.owner = g;
+        lookup.bytes = steps_[g].bytes;
+        lookup.norm_stats_out = stats;
+        taken_[g] = true;
+        fused->push_back(std::move(lookup));
+      } else {
+        (*fused)[static_cast<size_t>(owner[made->second])].norm_stats_out = stats;
+      }
       for (size_t c : reader_launches) {
         Launch &reader = (*fused)[c];
         reader.norm_mode = 1;

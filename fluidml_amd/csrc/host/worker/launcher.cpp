@@ -801,6 +801,15 @@ void LaunchPlan::Issue(kernel::LaunchContext &ctx, const Launch &l, int *rc_out)
       rc = fluidml_hip_add_layer_normalization(&a.t, &b.t, &g.t, &h.t, &out.t, l.axis, l.s0, ctx.stream);
       break;
     }
+    case Launch::Kind::GatherStats: {
+      const kernel::DeviceConstant *table = steps_[l.owner].kernel->GetConstant(0);
+      if (table == nullptr) throw std::logic_error("Gather with statistics: the node holds no data tensor");
+      const kernel::TensorView data = table->View();
+      rc = fluidml_hip_gather_constant_data_tensor_stats(&a.t, &data.t, &out.t,
+                                                         static_cast<float *>(privates_.at(l.norm_stats_out).device),
+                                                         ctx.stream);
+      break;
+    }
     case Launch::Kind::GatherAddLayerNorm: {
       const kernel::DeviceConstant *table = steps_[l.owner].kernel->GetConstant(0);
       const kernel::DeviceConstant *table2 = l.has_gate ? steps_[l.owner2].kernel->GetConstant(0) : nullptr;

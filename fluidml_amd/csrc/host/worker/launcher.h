@@ -93,6 +93,8 @@ struct Launch {
                          // LayerNormalizationConstantScaleBias (last dim): a = indices into the table of `owner`,
                          // b = the first addend, or with has_gate the indices into the table of `owner2`, c = the
                          // second addend, `norm_owner` = the LayerNormalization step, s0 = epsilon
+    GatherStats,       // GatherConstantDataTensor whose result feeds LayerNormalizations that are not run: a = indices
+                       // into the table of `owner`; leaves the partial row statistics in `norm_stats_out`
     ReshapeTranspose,  // Reshape -> Transpose, one strided copy
     TransposeReshape,  // Transpose -> Reshape, one strided copy
     PadViewCopy,       // Pad -> steps that only re-address its result (Gather of sliding windows, Slice, Transpose,

@@ -536,6 +536,12 @@ int fluidml_hip_div_add_softmax(const fl_tensor *in, double div, const fl_tensor
  * launched).  (reference matmul.cpp:28-59, div.cpp:24-56, add.cpp:75-137,
  * where.cpp:17-150, softmax.cpp:22-139) */
 int fluidml_hip_attention(const fl_tensor *q, const fl_tensor *kt, const fl_tensor *v, const fl_tensor *out, double scale, int32_t scale_is_divisor, const fl_tensor *add_mask, const fl_tensor *keep_cond, double fill, void *stream);
+/* GatherConstantDataTensorKernel whose result feeds a LayerNormalization that is not run (fl_norm_fusion): out =
+ * data[indices] as fluidml_hip_gather_constant_data_tensor, and stats_out (device memory, 2 * ceil(len / 32) floats
+ * per looked-up row) receives the partial row statistics of `out` in the layout of fl_norm_fusion.stats.  data
+ * [rows, len], everything dense row-major, otherwise FL_ERR_UNSUPPORTED.  (reference gather.cpp:195-272,
+ * layer_normalization.cpp:33-220) */
+int fluidml_hip_gather_constant_data_tensor_stats(const fl_tensor *indices, const fl_tensor *data, const fl_tensor *out, float *stats_out, void *stream);
 /* GatherConstantDataTensorKernel [x2] -> AddCommonKernel [-> AddCommonKernel] ->
  * LayerNormalizationConstantScaleBiasKernel over the last dim (the embedding
  * block of a BERT-style encoder) as one launch:

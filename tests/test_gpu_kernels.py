@@ -1285,6 +1285,33 @@ def test_fused_add_layer_norm(device):
             assert_close(do.logical(), ho.logical(), what="add_layer_normalization")
 
 
+def test_gather_with_row_statistics(device):
+    """The lookup that also leaves the partial row statistics of its result (mean and sum of squared deviations of
+    every run of 32 columns): rows bit-identical to the oracle's Gather, statistics against float64."""
+    import torch
+
+    cabi = _cabi()
+    rng = np.random.default_rng(223)
+    for lead, length, rows in [((1, 256), 512, 1000), ((3, 5), 33, 17), ((7,), 300, 9), ((2, 2), 1056, 6)]:
+        announce("gather_constant_data_tensor_stats", lead, length, rows)
+        table = rand(rng, (rows, length), -2, 2)
+        ids = rng.integers(0, rows, size=lead).astype(np.int64)
+        hi, ht, want = ok.View(ids), ok.View(table), ok.View.empty(lead + (length,))
+        ok.gather_data_tensor(hi, ht, want)
+        di, dt = DeviceView(hi, device), DeviceView(ht, device)
+        do = DeviceView(ok.View.empty(lead + (length,), np.float32, None, fill=5), device)
+        n_rows, parts = int(np.prod(lead)), (length + 31) // 32
+        stats = torch.full((n_rows, parts, 2), 7.0, dtype=torch.float32, device=device)
+        cabi.call("gather_constant_data_tensor_stats", di.ref(), dt.ref(), do.ref(), ctypes.c_void_p(stats.data_ptr()), None)
+        assert_close(do.logical(), want.logical(), exact=True, what="gather with statistics: rows")
+        got = stats.cpu().numpy()
+        x = want.logical().reshape(n_rows, length).astype(np.float64)
+        for j in range(parts):
+            run = x[:, 32 * j:32 * (j + 1)]
+            np.testing.assert_allclose(got[:, j, 0], run.mean(axis=1), rtol=1e-5, atol=1e-6)
+            np.testing.assert_allclose(got[:, j, 1], ((run - run.mean(axis=1, keepdims=True)) ** 2).sum(axis=1), rtol=1e-4, atol=1e-5)
+
+
 def test_gather_add_layer_norm(device):
     """The embedding block as one launch against the oracle's separate Gather, Add, Add and LayerNormalization: with
     one table or two, a second addend or none, addends that repeat along the leading dims."""

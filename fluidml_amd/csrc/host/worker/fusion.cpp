@@ -1378,7 +1378,11 @@ class Scheduler {
     l.out2 = steps_[*mean].out;
     l.has_out2 = true;
     if (!IsFloat(l.out2) || !Elidable(l.out2)) return std::nullopt;
-    if (!Safe(l.members, {{i, l.a}, {i, l.b}}) || !OutputDisjoint(l.out, {&l.a, &l.b}) || !OutputDisjoint(l.out2, {&l.a, &l.b, &l.out})) return std::nullopt;
+    // (the plan may put the result over the convolution's input, dead by then in the plan but read by this launch,
+    // which runs at the ReduceMean's place: the result then moves out of the arena)
+    const bool clash = !OutputDisjoint(l.out, {&l.a, &l.b});
+    if (!Safe(l.members, {{i, l.a}, {i, l.b}}) || (clash && !Movable(l.out)) || !OutputDisjoint(l.out2, {&l.a, &l.b, &l.out})) return std::nullopt;
+    if (clash) pending_moves_.push_back(l.out.name);
     l.bytes = Bytes({&l.a, &l.b, &l.out}) + static_cast<double>(steps_[i].kernel->GetConstantBytes()) + static_cast<double>(l.out2.meta.GetSize());
     l.flops = Flops(l.members);
     return l;
